@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the token-sampling hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload tile|cfg2|cfg3|cfg5] [--no-cpu] [--no-also]
+
+A step = one launch of the fused batched sampler (ws_sample_batch) over one batch of synthetic logits that already
+sit in HBM. The default workload is the north-star tile: 256 rows x 151,936 fp32 logits ~ N(0, sigma 2), repetition /
+presence / frequency penalties over a 2048-id history per row, temperature in [0.7, 1.0], top-p 0.9 (top-k and min-p
+off, so every row needs a full-vocabulary mass select), seeded Philox draws. One JSON line goes to stdout.
+
+roofline.achieved = algorithmic bytes per launch / average launch duration, measured with HIP events recorded on the
+stream the kernel is launched on. Algorithmic bytes = rows * vocab * sizeof(logit) + 4 bytes per history id + 8 bytes
+per bias entry + allow-mask bitmap + 16 bytes of output per row.
+cpu_baseline = the reference's own sampler (oracle/_ref, compiled from the reference sources in the build container)
+or, where that library is absent, the oracle's restatement of it, one thread, on the first rows of the same batch.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(c):
+    e = 2 if c["dtype"] == "bf16" else 4
+    b = c["rows"] * c["V"] * e + c["rows"] * 16
+    if c["hist"] is not None:
+        b += c["hist"].size * 4
+    if c["bias_ids"] is not None:
+        b += c["bias_ids"].size * 8
+    if c["allow"] is not None:
+        b += c["allow"].size * 4
+    return b
+
+
+def time_gpu(c, steps, warmup, rng_mode=1):
+    import torch
+    import gpu_cases as gc
+    d = gc.upload(c)
+    smp = gc.sampler_for(c, d, rng_mode)
+    for _ in range(warmup):
+        smp.run()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        smp.run()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    kern_ms = ev0.elapsed_time(ev1) / steps
+    return smp, wall_ms, kern_ms
+
+
+def parity_sample(c, smp, n_check, rng_mode=1):
+    import gpu_cases as gc
+    rows = list(range(0, c["rows"], max(1, c["rows"] // n_check)))[:n_check]
+    res = gc.compare_rows(c, smp, rows, rng_mode, check_kept=False)
+    import torch
+    fl = smp.flags.cpu().numpy()
+    m = gc.pkg()
+    res["device_near_flags"] = int(((fl & m.FLAG_NEAR) != 0).sum())
+    res["device_failed_rows"] = int(((fl & (m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED)) != 0).sum())
+    return res
+
+
+def cpu_baseline(c, budget_s=12.0, max_rows=64):
+    """Reference sampler on the host cores of this box: penalties pre-pass (oracle) + prepare / filter / draw of the
+    reference's own code with its splitmix uniform. One thread."""
+    import ctypes as C
+    import numpy as np
+    import gpu_cases as gc
+    import wo
+    ref = wo.load("ref")
+    lib = ref if ref is not None else wo.load("oracle")
+    port = wo.load("oracle")
+    kind = "reference" if ref is not None else "port"
+    done, t_used = 0, 0.0
+    V = c["V"]
+    for r in range(min(max_rows, c["rows"])):
+        x = gc.row_f32(c, r).copy()
+        hist = np.ascontiguousarray(c["hist"][r]) if c["hist"] is not None else np.zeros(0, np.int32)
+        bi = np.ascontiguousarray(c["bias_ids"][r]) if c["bias_ids"] is not None else np.zeros(0, np.int32)
+        bv = np.ascontiguousarray(c["bias_vals"][r]) if c["bias_vals"] is not None else np.zeros(0, np.float32)
+        allow = np.ascontiguousarray(c["allow"][r]) if c["allow"] is not None else None
+        s = wo.new_sampler(top_k=int(c["top_k"][r]), top_p=float(c["top_p"][r]), min_p=float(c["min_p"][r]), seed=int(c["seed"][r]))
+        s.inv_t = c["inv_t"][r]
+        t0 = time.perf_counter()
+        port.wo_apply_penalties(wo._ptr(x), V, wo._ptr(allow) if allow is not None else None, wo._ptr(hist), hist.size,
+                                c["rep"][r], c["pres"][r], c["freq"][r], wo._ptr(bi), wo._ptr(bv), bi.size)
+        rows, keep = wo.make_rows(x[None, :], 256, 16384)
+        lib.wo_prepare_draw(C.byref(rows), C.byref(s), 0, int(c["step"][r]))
+        t_used += time.perf_counter() - t0
+        done += 1
+        if t_used > budget_s:
+            break
+    return dict(value=done / t_used, unit="rows/s", cores=1, kind=kind,
+                sample=f"first {done} rows of the same batch, penalties + escalation 256/16384/full + filter + draw, "
+                       f"{t_used:.2f} s on one host thread")
+
+
+def run_workload(name, steps, warmup, check_rows):
+    import gpu_cases as gc
+    make = dict(tile=gc.make_tile, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=lambda: gc.make_cfg5(rows=256))[name]
+    c = make()
+    smp, wall_ms, kern_ms = time_gpu(c, steps, warmup)
+    par = parity_sample(c, smp, check_rows) if check_rows else None
+    ab = algorithmic_bytes(c)
+    return c, dict(workload=name, rows=c["rows"], vocab=c["V"], dtype=c["dtype"], ms_per_step=wall_ms, kernel_ms=kern_ms,
+                   rows_per_s=c["rows"] / (wall_ms * 1e-3), algorithmic_MB=ab / 1e6, achieved_GBs=ab / (kern_ms * 1e-3) / 1e9,
+                   frac_of_hbm_peak=ab / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, parity=par)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="tile", choices=["tile", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-also", action="store_true")
+    ap.add_argument("--check-rows", type=int, default=8)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU; rows are independent, so more GPUs mean more row shards with no "
+              "communication (--gpus 1 only)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    c, main_res = run_workload(a.workload, a.steps, a.warmup, a.check_rows)
+    also = []
+    if not a.no_also:
+        for w in ("cfg2", "cfg3"):
+            if w != a.workload:
+                _, r = run_workload(w, max(20, a.steps // 4), 5, 4)
+                also.append(r)
+    cpu = None if a.no_cpu else cpu_baseline(c)
+    ab = main_res["algorithmic_MB"] * 1e6
+    out = {
+        "metric": "sampled rows/s (fused penalties + top-p sampler, batch 256 x vocab 151936 fp32)",
+        "value": main_res["rows_per_s"], "unit": "rows/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if c["dtype"] == "f32" else "bf16->f32", "data": "synthetic",
+        "config": {"workload": a.workload, "rows": c["rows"], "vocab": c["V"], "logits": c["dtype"],
+                   "history_ids_per_row": 0 if c["hist"] is None else int(c["hist"].shape[1]),
+                   "filters": "see tests/gpu_cases.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2},
+        "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": main_res["frac_of_hbm_peak"], "traffic": None, "kernel": "ws::sample_batch_kernel",
+                     "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},
+        "cpu_baseline": cpu,
+        "parity": main_res["parity"],
+        "also": also,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,195 @@
+/* C ABI of the MI355X (gfx950) token-sampling library, libwhirl_sampling_hip.so.
+ *
+ * Plain pointers and sizes only: every pointer named "device" is a HIP device address the caller owns, every
+ * struct is read on the host at call time (by-value launch arguments, no host buffer is kept after return).
+ * Calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL = the null stream) unless stated.
+ * Return value: 0 = launched, > 0 = the hipError_t of a failed HIP call, < 0 = WS_E_* argument error detected on
+ * the host before anything was launched. No exceptions cross this boundary. Per-row run-time conditions
+ * (all-masked row, candidate overflow, draw within tolerance of a boundary) are reported in device `flags`.
+ *
+ * Two groups of entry points:
+ *  (1) one launcher per reference kernel, same argument order and output layout as the kernel the reference
+ *      resolves by name (citations at each declaration), with the launch geometry chosen here;
+ *      the gfx950 code object whirl_sampling_gfx950.co exports the same `extern "C" __global__` names for callers
+ *      that use hipModuleGetFunction (block = 1024 threads, grid = rows, no dynamic LDS);
+ *  (2) the batched fused sampler and the classic speculative verify, which the reference does not have.
+ */
+#ifndef WHIRL_SAMPLING_ABI_H
+#define WHIRL_SAMPLING_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WS_ABI_VERSION 1
+
+enum {
+    WS_OK = 0,
+    WS_E_INVALID = -1,     /* null pointer, zero / oversized dimension, unknown enum value */
+    WS_E_WORKSPACE = -2,   /* workspace missing or smaller than ws_*_workspace() reports */
+    WS_E_UNSUPPORTED = -3, /* a combination this build does not implement */
+    WS_E_NO_DEVICE = -4    /* no HIP device / the code object does not load on it */
+};
+
+/* Most rows one launch of the by-value-table kernels takes (kMaxVerifyRows, include/whirl/kernels_abi.h:359-365). */
+#define WS_MAX_TABLE_ROWS 32
+
+/* RowIdx (include/whirl/kernels_abi.h:367-369, kernels/kernel_args.h:46-48): 128 bytes, passed by value. */
+typedef struct ws_row_idx {
+    int32_t v[WS_MAX_TABLE_ROWS];
+} ws_row_idx;
+
+/* DSampArgs (include/whirl/kernels_abi.h:376-387, kernels/kernel_args.h:57-66): 1024 bytes, passed by value. */
+typedef struct ws_dsamp_args {
+    int32_t on[WS_MAX_TABLE_ROWS];
+    int32_t top_k[WS_MAX_TABLE_ROWS];
+    int32_t qoff[WS_MAX_TABLE_ROWS]; /* i32 word offset of the row's q entry in qbuf */
+    float inv_t[WS_MAX_TABLE_ROWS];
+    float top_p[WS_MAX_TABLE_ROWS];
+    float min_p[WS_MAX_TABLE_ROWS];
+    uint32_t key_lo[WS_MAX_TABLE_ROWS]; /* race key base = raceBase(seed, output index), include/whirl/spec_sample.h:58-60 */
+    uint32_t key_hi[WS_MAX_TABLE_ROWS];
+} ws_dsamp_args;
+
+/* Control area of one sequence, 64 i32 words (include/whirl/kernels_abi.h:269-276). */
+enum { WS_CTL_ROWS = 0, WS_CTL_DRAFTS = 16, WS_CTL_PROBS = 32, WS_CTL_ND = 48, WS_CTL_STOP = 49, WS_CTL_WORDS = 64 };
+/* q entry of draft_sample_rows, 72 i32 words: [0] n, [1,33) ids, [33,65) f32 probabilities (include/whirl/spec_sample.h:40-46). */
+enum { WS_Q_MAX = 32, WS_Q_WORDS = 72, WS_Q_OFF_IDS = 1, WS_Q_OFF_P = 33 };
+
+int ws_abi_version(void);
+const char* ws_error_string(int code);
+/* Loads nothing and launches nothing: 0 when a gfx950 device is present and the kernels of this library can run. */
+int ws_probe(void);
+
+/* ---- (1) reference kernels ------------------------------------------------------------------------------- */
+
+/* argmax(x, n, out, ids, pos, advance): kernels/shared/misc_kv_argmax_kv_store.h:32-42. First index of the maximum
+ * into out[0] and ids[0]; pos[0] += advance. */
+int ws_argmax(void* stream, const float* x, int n, int* out, int* ids, int* pos, int advance);
+/* argmax_rows(x, n, out): kernels/shared/sample_pick_set_tokens.h:15-21. x = [rows][n]. */
+int ws_argmax_rows(void* stream, const float* x, int n, int* out, unsigned rows);
+/* argmax_rows_to(x, n, out, dst): sample_pick_set_tokens.h:47-53. Row b goes to out[dst->v[b]]; rows <= 32. */
+int ws_argmax_rows_to(void* stream, const float* x, int n, int* out, const ws_row_idx* dst, unsigned rows);
+/* argmax_prob(x, n, out_tok, out_prob): sample_pick_set_tokens.h:96-105. out_prob[0] = 1 / sum exp(x - max). */
+int ws_argmax_prob(void* stream, const float* x, int n, int* out_tok, float* out_prob);
+/* draft_pick(x, n, tok, prob, ctl, r, n_min, p_min, map): sample_pick_set_tokens.h:60-86. tok[r] = map ? map[top] : top,
+ * prob[r] = p(top); p-min cutoff words ctl[0] (drafts kept), ctl[1] (chain stopped); r > 0 and ctl[1] != 0: no-op. */
+int ws_draft_pick(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
+                  const int* map);
+/* draft_pick_rows(x, n, ctl_all, area, r, n_min, p_min, map): sample_pick_set_tokens.h:88-92. Row b uses the control
+ * area at ctl_all + area->v[b]; rows <= 32. */
+int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min,
+                       float p_min, const int* map, unsigned rows);
+/* draft_sample_rows(x, n, ctl_all, area, r, map, a, qbuf): kernels/spec_sample.hip:34-205. Rows with a->on draw draft r
+ * from the filtered draft distribution q by the race (argmin E(v) / q(v)) into ctl[16 + r] and write q; rows <= 32. */
+int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
+                         const ws_dsamp_args* a, int* qbuf, unsigned rows);
+/* topk_rows(x, n, K, inv_t, ids, vals, stats): kernels/shared/sample_cand_topk_rows.h:11-98; launch site
+ * src/model/qwen35/server_model.cpp:101-107. stats[row] = {max, sum exp((x - max) * inv_t)}, ids / vals[row][0..K) =
+ * the K largest logits. The reference leaves their order and the choice among equal values at the cut to its
+ * atomics; here both are fixed: ties at the cut keep the lowest token ids, entries are in ascending id order.
+ * Output layout as the engine's buffers expect it (src/server/engine_sampling.cpp:37-43). */
+int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows);
+
+/* ---- (2) batched fused sampler ---------------------------------------------------------------------------- */
+
+enum { WS_DTYPE_F32 = 0, WS_DTYPE_BF16 = 1 };
+enum { WS_RNG_SPLITMIX = 0, WS_RNG_PHILOX = 1 };
+
+/* Per-row flag bits written to ws_batch.flags. */
+enum {
+    WS_FLAG_NEAR_TOP_P = 1u << 0,  /* the top-p cut was within `tol` (relative) of moving by one candidate */
+    WS_FLAG_NEAR_MIN_P = 1u << 1,  /* a candidate's probability was within `tol` (relative) of the min-p floor */
+    WS_FLAG_NEAR_DRAW = 1u << 2,   /* the uniform was within `tol` (probability units) of a CDF step */
+    WS_FLAG_ALL_MASKED = 1u << 3,  /* every logit of the row is -inf / NaN: token = -1 */
+    WS_FLAG_OVERFLOW = 1u << 4,    /* more tied / clustered candidates at a cut than the kernel resolves: token = -1 */
+    WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
+    WS_FLAG_OPEN = 1u << 6         /* no filter active: drawn in the reference's open-row order */
+};
+
+/* One batch of rows. Everything per row is a device array of `rows` entries (SoA); a NULL array means the stated
+ * default for every row. The engine fills these from what it already keeps per slot: Sampler fields
+ * (src/sampling/sampler.h:26-43, set at src/server/engine_start.cpp:47-59) and the slot's token history
+ * (src/server/engine_slot.h:38-65). Order of operations per row:
+ *   allow-mask (-inf) and NaN -> -inf; logit bias (values of one id added in listed order); repetition penalty
+ *   (x > 0 ? x / rep : x * rep) then x -= freq * count + pres for ids in the history; temperature; top-k; top-p;
+ *   min-p; renormalise; inverse-CDF draw in (logit desc, id asc) order (src/sampling/sampler.cpp:15-78, :118-131). */
+typedef struct ws_batch {
+    const void* logits;  /* device, [rows][row_stride] of dtype */
+    int32_t dtype;       /* WS_DTYPE_* */
+    uint32_t rows;
+    uint32_t vocab;      /* <= 1048575 */
+    uint64_t row_stride; /* elements between rows (>= vocab) */
+
+    const float* inv_t;     /* 1 / temperature, > 0 (Sampler::inv_t) */
+    const uint32_t* top_k;  /* 0 = off (NULL: off) */
+    const double* top_p;    /* 1 = off (NULL: off) */
+    const double* min_p;    /* 0 = off (NULL: off) */
+    const uint64_t* seed;   /* Sampler::seed */
+    const uint64_t* step;   /* output token index (Sampler::pos_idx) */
+    int32_t rng;            /* WS_RNG_SPLITMIX: the reference's uniform(seed, step) (src/sampling/sampler.h:46-52);
+                               WS_RNG_PHILOX: Philox4x32-10, ctr = (step_lo, step_hi, row, stream), key = (seed_lo, seed_hi) */
+
+    const int32_t* hist;        /* concatenated token histories, row r = hist[hist_off[r] .. hist_off[r+1]) (NULL: none) */
+    const uint32_t* hist_off;   /* rows + 1 */
+    const float* rep;           /* repetition penalty (NULL: 1) */
+    const float* pres;          /* presence penalty (NULL: 0) */
+    const float* freq;          /* frequency penalty (NULL: 0) */
+    const int32_t* bias_ids;    /* concatenated logit-bias token ids (NULL: none) */
+    const float* bias_vals;
+    const uint32_t* bias_off;   /* rows + 1 */
+    uint32_t max_hist;          /* upper bound of any row's history length */
+    uint32_t max_bias;          /* upper bound of any row's bias count */
+    const uint32_t* allow;      /* allow bitmap, bit i of allow[r * allow_stride + i / 32] set = token i allowed (NULL: all) */
+    uint64_t allow_stride;      /* 32-bit words between rows */
+
+    int32_t* token;     /* out: sampled token id, -1 on a flagged failure */
+    float* prob;        /* out (may be NULL): renormalised probability of the token on the kept set */
+    uint32_t* n_kept;   /* out (may be NULL): size of the kept set (Sampler::n) */
+    uint32_t* flags;    /* out: WS_FLAG_* */
+    float* stats;       /* out (may be NULL): [rows][2] = {max logit after penalties, (float) sum exp((x - max) * inv_t)} */
+    double* margin;     /* out (may be NULL): [rows][3] distance of the top-p cut, min-p floor and draw to flipping */
+    int32_t* kept_ids;  /* out (may be NULL): [rows][kept_cap] kept token ids in ascending id order */
+    float* kept_logits; /* out (may be NULL): penalty-applied logits of kept_ids */
+    uint32_t kept_cap;
+
+    void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes */
+    uint64_t workspace_bytes;
+    double tol;             /* flag tolerance (0: 2^-40) */
+} ws_batch;
+
+/* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
+uint64_t ws_sample_batch_workspace(const ws_batch* b);
+int ws_sample_batch(void* stream, const ws_batch* b);
+
+/* Classic speculative sampling (accept u * q < p, else resample from max(p - q, 0)); no counterpart in the
+ * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32
+ * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1]. Per sequence s: u_j from
+ * (seed[s], row = s, step = step0[s] + j, stream 0); the resample / bonus draw uses stream 1 and walks the vocabulary
+ * in id order. out_tokens[s][0 .. n_accepted[s]] = accepted drafts then the drawn token. */
+typedef struct ws_spec_verify {
+    const float* p;
+    const float* q;
+    const int32_t* draft;
+    uint32_t n_seq, n_pos, vocab;
+    const uint64_t* seed;
+    const uint64_t* step0;
+    int32_t rng;
+    int32_t* out_tokens; /* [n_seq][n_pos] */
+    int32_t* n_accepted; /* [n_seq] */
+    uint32_t* flags;     /* [n_seq] WS_FLAG_NEAR_DRAW */
+    void* workspace;
+    uint64_t workspace_bytes;
+    double tol;
+} ws_spec_verify;
+
+uint64_t ws_spec_verify_workspace(const ws_spec_verify* v);
+int ws_spec_verify_classic(void* stream, const ws_spec_verify* v);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,54 @@
+"""CPU-only: the C-ABI library is built, loads and exports every symbol include/whirl_sampling_abi.h declares; the
+argument checks that run before any launch behave as the header says. No compute call is made."""
+import ctypes as C
+import os
+import re
+
+import gpu_cases
+
+ROOT = gpu_cases.ROOT
+
+
+def test_every_declared_symbol_is_exported():
+    m = gpu_cases.pkg()
+    hdr = open(os.path.join(ROOT, "include", "whirl_sampling_abi.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(ws_[a-z_0-9]+)\s*\(", hdr))
+    assert declared == set(m.ABI), (declared ^ set(m.ABI))
+    lib = m.lib()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.ws_abi_version() == 1
+    assert lib.ws_error_string(0) == b"ok" and b"workspace" in lib.ws_error_string(-2)
+
+
+def test_code_object_exports_reference_kernel_names():
+    """The kernels an engine resolves by name (include/whirl/kernels_abi.h:118-130 of the reference) are in the gfx950
+    code object with unmangled names."""
+    m = gpu_cases.pkg()
+    blob = open(m.CO_PATH, "rb").read()
+    for k in (b"argmax", b"argmax_rows", b"argmax_rows_to", b"argmax_prob", b"draft_pick", b"draft_pick_rows",
+              b"draft_sample_rows", b"topk_rows"):
+        assert b"\x00" + k + b"\x00" in blob, k
+
+
+def test_host_side_argument_checks():
+    m = gpu_cases.pkg()
+    lib = m.lib()
+    assert lib.ws_argmax_rows(None, None, 10, None, 1) == -1
+    assert lib.ws_topk_rows(None, C.c_void_p(16), 0, 4, 1.0, C.c_void_p(16), C.c_void_p(16), C.c_void_p(16), 1) == -1
+    ri = m.RowIdx()
+    assert lib.ws_argmax_rows_to(None, C.c_void_p(16), 8, C.c_void_p(16), C.byref(ri), 33) == -1  # more than 32 table rows
+    b = m.Batch()
+    assert lib.ws_sample_batch(None, C.byref(b)) == -1 and lib.ws_sample_batch_workspace(C.byref(b)) == 0
+    one = C.c_void_p(16)
+    b.logits, b.inv_t, b.seed, b.step, b.token, b.flags = one, one, one, one, one, one
+    b.rows, b.vocab, b.row_stride = 4, 151936, 151936
+    b.hist, b.hist_off, b.max_hist = one, one, 4096
+    need = lib.ws_sample_batch_workspace(C.byref(b))
+    assert need == 4 * 4096 * 16
+    assert lib.ws_sample_batch(None, C.byref(b)) == -2  # no workspace given
+    b.max_hist = 60000
+    assert lib.ws_sample_batch(None, C.byref(b)) == -3  # rank tables would not fit the LDS
+    b.vocab = 1 << 20
+    assert lib.ws_sample_batch(None, C.byref(b)) == -1

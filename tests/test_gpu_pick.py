@@ -1,0 +1,134 @@
+"""GPU: greedy picks and top-k candidates through the C ABI against the oracle / library routines, in the idiom of
+the reference's kernel tests (tests/kernels/test_misc.cpp:153-354): planted ties (first index wins), maximum in the
+last element, control words of the draft chain, top-k value multisets equal to a partial sort."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_cases
+import wo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def first_max(x):
+    return int(np.argmax(x))
+
+
+def softmax_top(x):
+    return 1.0 / np.exp(x.astype(np.float64) - float(x.max())).sum()
+
+
+@pytest.fixture(scope="module")
+def rows5():
+    rng = np.random.default_rng(100)
+    n, rows = 248320, 5
+    x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
+    x[1, 100] = 50.0
+    x[1, 9000] = 50.0  # tie: the first index must win
+    x[2, n - 1] = 60.0  # last element
+    return x, torch.from_numpy(x).to(DEV)
+
+
+def test_argmax_family(rows5):
+    m = gpu_cases.pkg()
+    x, dx = rows5
+    rows, n = x.shape
+    want = [first_max(x[r]) for r in range(rows)]
+    ids = torch.zeros(1, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([41], dtype=torch.int32, device=DEV)
+    out = m.argmax(dx[1], ids, pos, 1)
+    assert out.item() == want[1] == 100 and ids.item() == want[1] and pos.item() == 42
+    assert m.argmax_rows(dx).cpu().tolist() == want
+    buf = torch.full((64,), -1, dtype=torch.int32, device=DEV)
+    m.argmax_rows_to(dx, buf, [10 + 3 * r for r in range(rows)])
+    got = buf.cpu().numpy()
+    assert [got[10 + 3 * r] for r in range(rows)] == want and (got != -1).sum() == rows
+    tok, prob = m.argmax_prob(dx[0])
+    assert tok.item() == want[0]
+    assert abs(prob.item() - softmax_top(x[0])) <= 1e-4 * softmax_top(x[0]) + 1e-9
+
+
+def test_argmax_odd_sizes_and_misaligned_rows():
+    m = gpu_cases.pkg()
+    rng = np.random.default_rng(101)
+    for n in (1, 3, 5, 1023, 1025, 4099, 151937):
+        x = np.round(rng.standard_normal((3, n)) * 2, 1).astype(np.float32)  # many ties; odd n misaligns rows 1, 2
+        assert m.argmax_rows(torch.from_numpy(x).to(DEV)).cpu().tolist() == [first_max(r) for r in x]
+    x = np.full((2, 777), -np.inf, np.float32)
+    x[1, 5] = np.nan
+    assert m.argmax_rows(torch.from_numpy(x).to(DEV)).cpu().tolist() == [0, 0]
+
+
+def test_draft_pick_chain_and_rows(rows5):
+    """tests/kernels/test_misc.cpp:196-270."""
+    m = gpu_cases.pkg()
+    rng = np.random.default_rng(102)
+    n = 248320
+    lg = rng.standard_normal((3, n)).astype(np.float32)
+    lg[0, 5] = 30.0   # r = 0: confident
+    lg[1, 7] = 4.0    # r = 1: unconfident -> the chain stops (n_min = 1)
+    lg[2, 9] = 30.0   # r = 2: skipped
+    dl = torch.from_numpy(lg).to(DEV)
+    tok = torch.full((16,), 0x7F7F7F7F, dtype=torch.int32, device=DEV)
+    prob = torch.zeros(16, dtype=torch.float32, device=DEV)
+    ctl = torch.zeros(2, dtype=torch.int32, device=DEV)
+    for r in range(3):
+        m.draft_pick(dl[r], tok, prob, ctl, r, 1, 0.5)
+    t, c, p = tok.cpu().numpy(), ctl.cpu().numpy(), prob.cpu().numpy()
+    assert t[0] == 5 and t[1] == first_max(lg[1]) and t[2] == 0x7F7F7F7F and c[0] == 1 and c[1] == 1
+    for r in range(2):
+        assert abs(p[r] - softmax_top(lg[r])) <= 1e-4 * softmax_top(lg[r]) + 1e-9
+    ctl_all = torch.zeros(2 * m.CTL_WORDS, dtype=torch.int32, device=DEV)
+    m.draft_pick_rows(dl[:2], ctl_all, [0, m.CTL_WORDS], 0, 1, 0.5)
+    ca = ctl_all.cpu().numpy()
+    assert ca[16] == t[0] and ca[m.CTL_WORDS + 16] == t[1] and ca[48] == 1 and ca[m.CTL_WORDS + 48] == 1
+    # vocabulary map: identity == no map, any map returns map[top]
+    ident = torch.arange(n, dtype=torch.int32, device=DEV)
+    perm = (100000 + 3 * torch.arange(n, dtype=torch.int32, device=DEV))
+    t1 = torch.zeros(16, dtype=torch.int32, device=DEV)
+    t2 = torch.zeros(16, dtype=torch.int32, device=DEV)
+    c1, c2 = torch.zeros(2, dtype=torch.int32, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV)
+    for r in range(2):
+        m.draft_pick(dl[r], t1, prob, c1, r, 0, 0.0, ident)
+        m.draft_pick(dl[r], t2, prob, c2, r, 0, 0.0, perm)
+    cm = torch.zeros(2 * m.CTL_WORDS, dtype=torch.int32, device=DEV)
+    m.draft_pick_rows(dl[:2], cm, [0, m.CTL_WORDS], 0, 0, 0.0, perm)
+    top0, top1 = 5, first_max(lg[1])
+    assert t1.cpu().tolist()[:2] == [top0, top1]
+    assert t2.cpu().tolist()[:2] == [100000 + 3 * top0, 100000 + 3 * top1]
+    assert cm.cpu()[16].item() == 100000 + 3 * top0 and cm.cpu()[m.CTL_WORDS + 16].item() == 100000 + 3 * top1
+
+
+@pytest.mark.parametrize("K", [1, 16, 40, 256, 16384])
+def test_topk_rows_against_oracle(rows5, K):
+    """Value multiset == partial sort, ids consistent with values, maximum exact, normaliser within 1e-4
+    (tests/kernels/test_misc.cpp:315-354); beyond that, the id SET equals the oracle's (value desc, id asc) top-K and
+    entries come in ascending id order."""
+    m = gpu_cases.pkg()
+    lib = wo.load("oracle")
+    x, dx = rows5
+    inv_t = np.float32(1.0 / 0.7)
+    ids, vals, stats = m.topk_rows(dx[:3], K, float(inv_t))
+    ids, vals, stats = ids.cpu().numpy(), vals.cpu().numpy(), stats.cpu().numpy()
+    for r in range(3):
+        wi, wv, ws_ = np.zeros(K, np.int32), np.zeros(K, np.float32), np.zeros(2, np.float32)
+        lib.wo_topk_row(wo._ptr(np.ascontiguousarray(x[r])), x.shape[1], K, inv_t, wo._ptr(wi), wo._ptr(wv), wo._ptr(ws_))
+        assert np.array_equal(ids[r], np.sort(wi))
+        assert vals[r].tobytes() == x[r][ids[r]].tobytes()
+        assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1]
+
+
+def test_topk_rows_ties_at_the_cut_keep_lowest_ids():
+    m = gpu_cases.pkg()
+    n, K = 5000, 7
+    x = np.zeros((2, n), np.float32)
+    x[0, [4000, 10, 300]] = [3.0, 2.0, 2.0]  # 3 distinct leaders, then 4997 zeros tie for 4 places
+    x[1, :] = -1.5
+    x[1, 4999] = np.nan
+    ids, vals, _ = m.topk_rows(torch.from_numpy(x).to(DEV), K, 1.0)
+    assert ids.cpu().tolist()[0] == [0, 1, 2, 3, 10, 300, 4000]
+    assert ids.cpu().tolist()[1] == list(range(7)) and vals.cpu().tolist()[1] == [-1.5] * 7
+    ids, vals, _ = m.topk_rows(torch.from_numpy(x[:, :5]).contiguous().to(DEV), 9, 1.0)  # K > n: n entries written
+    assert ids.cpu().tolist()[0][:5] == [0, 1, 2, 3, 4] and ids.cpu().tolist()[0][5:] == [-1] * 4

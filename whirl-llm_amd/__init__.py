@@ -1,0 +1,253 @@
+"""MI355X token-sampling library: Python view of the C ABI in include/whirl_sampling_abi.h.
+
+The work is done by hand-written HIP kernels in libwhirl_sampling_hip.so (built from csrc/ by build.py). This module
+only marshals pointers: torch supplies device memory and the current HIP stream, ctypes calls the `ws_*` entry
+points. There is no CPU path: if the library is missing or a call fails, an exception is raised.
+
+The directory name holds a hyphen, so import it through `load_package()` of the repository's __graft_entry__.py or
+`importlib` (module name `whirl_llm_amd`).
+"""
+import ctypes as C
+import os
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libwhirl_sampling_hip.so")
+CO_PATH = os.path.join(HERE, "whirl_sampling_gfx950.co")
+
+DTYPE_F32, DTYPE_BF16 = 0, 1
+RNG_SPLITMIX, RNG_PHILOX = 0, 1
+FLAG_NEAR_TOP_P, FLAG_NEAR_MIN_P, FLAG_NEAR_DRAW = 1, 2, 4
+FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN = 8, 16, 32, 64
+FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
+CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
+
+
+class WsError(RuntimeError):
+    pass
+
+
+class RowIdx(C.Structure):
+    _fields_ = [("v", C.c_int32 * 32)]
+
+
+class DSampArgs(C.Structure):
+    _fields_ = [("on", C.c_int32 * 32), ("top_k", C.c_int32 * 32), ("qoff", C.c_int32 * 32), ("inv_t", C.c_float * 32),
+                ("top_p", C.c_float * 32), ("min_p", C.c_float * 32), ("key_lo", C.c_uint32 * 32),
+                ("key_hi", C.c_uint32 * 32)]
+
+
+class Batch(C.Structure):
+    _fields_ = [("logits", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_uint32), ("vocab", C.c_uint32),
+                ("row_stride", C.c_uint64),
+                ("inv_t", C.c_void_p), ("top_k", C.c_void_p), ("top_p", C.c_void_p), ("min_p", C.c_void_p),
+                ("seed", C.c_void_p), ("step", C.c_void_p), ("rng", C.c_int32),
+                ("hist", C.c_void_p), ("hist_off", C.c_void_p), ("rep", C.c_void_p), ("pres", C.c_void_p),
+                ("freq", C.c_void_p), ("bias_ids", C.c_void_p), ("bias_vals", C.c_void_p), ("bias_off", C.c_void_p),
+                ("max_hist", C.c_uint32), ("max_bias", C.c_uint32), ("allow", C.c_void_p), ("allow_stride", C.c_uint64),
+                ("token", C.c_void_p), ("prob", C.c_void_p), ("n_kept", C.c_void_p), ("flags", C.c_void_p),
+                ("stats", C.c_void_p), ("margin", C.c_void_p), ("kept_ids", C.c_void_p), ("kept_logits", C.c_void_p),
+                ("kept_cap", C.c_uint32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double)]
+
+
+class SpecVerify(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("q", C.c_void_p), ("draft", C.c_void_p), ("n_seq", C.c_uint32), ("n_pos", C.c_uint32),
+                ("vocab", C.c_uint32), ("seed", C.c_void_p), ("step0", C.c_void_p), ("rng", C.c_int32),
+                ("out_tokens", C.c_void_p), ("n_accepted", C.c_void_p), ("flags", C.c_void_p), ("workspace", C.c_void_p),
+                ("workspace_bytes", C.c_uint64), ("tol", C.c_double)]
+
+
+# every symbol include/whirl_sampling_abi.h declares: (result type, argument types)
+ABI = {
+    "ws_abi_version": (C.c_int, []),
+    "ws_error_string": (C.c_char_p, [C.c_int]),
+    "ws_probe": (C.c_int, []),
+    "ws_argmax": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
+    "ws_argmax_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_uint]),
+    "ws_argmax_rows_to": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_uint]),
+    "ws_argmax_prob": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "ws_draft_pick": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                C.c_float, C.c_void_p]),
+    "ws_draft_pick_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_int, C.c_int,
+                                     C.c_float, C.c_void_p, C.c_uint]),
+    "ws_draft_sample_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_int, C.c_void_p,
+                                       C.POINTER(DSampArgs), C.c_void_p, C.c_uint]),
+    "ws_topk_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
+                               C.c_uint]),
+    "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
+    "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
+    "ws_spec_verify_workspace": (C.c_uint64, [C.POINTER(SpecVerify)]),
+    "ws_spec_verify_classic": (C.c_int, [C.c_void_p, C.POINTER(SpecVerify)]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library; raises when it was not built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise WsError(f"{LIB_PATH} is missing: run `python whirl-llm_amd/build.py` (or __graft_entry__.build())")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in ABI.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code, what):
+    if code != 0:
+        raise WsError(f"{what}: {lib().ws_error_string(code).decode()} ({code})")
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _dev_f32(x):
+    if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()):
+        raise WsError("expected a contiguous float32 device tensor")
+    return x
+
+
+def argmax_rows(x):
+    """x: [rows, n] float32 device -> int32 [rows] (first index of each row's maximum)."""
+    _dev_f32(x)
+    out = torch.empty(x.shape[0], dtype=torch.int32, device=x.device)
+    check(lib().ws_argmax_rows(_stream(), _p(x), x.shape[1], _p(out), x.shape[0]), "ws_argmax_rows")
+    return out
+
+
+def argmax(x, ids, pos, advance=1):
+    """x: [n] row; ids, pos: int32 [1] device (next-step token / position, updated in place) -> int32 [1]."""
+    _dev_f32(x)
+    out = torch.empty(1, dtype=torch.int32, device=x.device)
+    check(lib().ws_argmax(_stream(), _p(x), x.numel(), _p(out), _p(ids), _p(pos), advance), "ws_argmax")
+    return out
+
+
+def argmax_rows_to(x, out, dst):
+    _dev_f32(x)
+    ri = RowIdx()
+    for i, d in enumerate(dst):
+        ri.v[i] = d
+    check(lib().ws_argmax_rows_to(_stream(), _p(x), x.shape[1], _p(out), C.byref(ri), x.shape[0]), "ws_argmax_rows_to")
+    return out
+
+
+def argmax_prob(x):
+    _dev_f32(x)
+    tok = torch.empty(1, dtype=torch.int32, device=x.device)
+    prob = torch.empty(1, dtype=torch.float32, device=x.device)
+    check(lib().ws_argmax_prob(_stream(), _p(x), x.numel(), _p(tok), _p(prob)), "ws_argmax_prob")
+    return tok, prob
+
+
+def draft_pick(x, tok, prob, ctl, r, n_min, p_min, vmap=None):
+    _dev_f32(x)
+    check(lib().ws_draft_pick(_stream(), _p(x), x.numel(), _p(tok), _p(prob), _p(ctl), r, n_min, p_min, _p(vmap)),
+          "ws_draft_pick")
+
+
+def draft_pick_rows(x, ctl_all, area, r, n_min, p_min, vmap=None):
+    _dev_f32(x)
+    ri = RowIdx()
+    for i, d in enumerate(area):
+        ri.v[i] = d
+    check(lib().ws_draft_pick_rows(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, n_min, p_min, _p(vmap),
+                                   x.shape[0]), "ws_draft_pick_rows")
+
+
+def draft_sample_rows(x, ctl_all, area, r, args, qbuf, vmap=None):
+    """args: list of per-row dicts (on, top_k, qoff, inv_t, top_p, min_p, key)."""
+    _dev_f32(x)
+    ri, da = RowIdx(), DSampArgs()
+    for i, d in enumerate(area):
+        ri.v[i] = d
+    for i, a in enumerate(args):
+        da.on[i], da.top_k[i], da.qoff[i] = a.get("on", 1), a["top_k"], a["qoff"]
+        da.inv_t[i], da.top_p[i], da.min_p[i] = a["inv_t"], a["top_p"], a["min_p"]
+        da.key_lo[i], da.key_hi[i] = a["key"] & 0xFFFFFFFF, a["key"] >> 32
+    check(lib().ws_draft_sample_rows(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, _p(vmap), C.byref(da),
+                                     _p(qbuf), x.shape[0]), "ws_draft_sample_rows")
+
+
+def topk_rows(x, K, inv_t):
+    """x: [rows, n] -> ids int32 [rows, K] (ascending id), vals float32 [rows, K], stats float32 [rows, 2]."""
+    _dev_f32(x)
+    rows = x.shape[0]
+    ids = torch.full((rows, K), -1, dtype=torch.int32, device=x.device)
+    vals = torch.zeros((rows, K), dtype=torch.float32, device=x.device)
+    stats = torch.empty((rows, 2), dtype=torch.float32, device=x.device)
+    check(lib().ws_topk_rows(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows), "ws_topk_rows")
+    return ids, vals, stats
+
+
+class BatchSampler:
+    """Holds the device-side parameter arrays, outputs and workspace of one batch shape; `run` launches the fused
+    kernel on the current stream and allocates nothing."""
+
+    def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
+                 hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
+                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True):
+        if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+            raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
+        if logits.dtype not in (torch.float32, torch.bfloat16):
+            raise WsError("logits: float32 or bfloat16")
+        dev = logits.device
+        rows, V = logits.shape
+        self.keep = dict(logits=logits, inv_t=inv_t, seed=seed, step=step, top_k=top_k, top_p=top_p, min_p=min_p,
+                         hist=hist, hist_off=hist_off, rep=rep, pres=pres, freq=freq, bias_ids=bias_ids,
+                         bias_vals=bias_vals, bias_off=bias_off, allow=allow)
+        self.token = torch.empty(rows, dtype=torch.int32, device=dev)
+        self.prob = torch.empty(rows, dtype=torch.float32, device=dev)
+        self.n_kept = torch.empty(rows, dtype=torch.int32, device=dev)
+        self.flags = torch.empty(rows, dtype=torch.int32, device=dev)
+        self.stats = torch.empty((rows, 2), dtype=torch.float32, device=dev)
+        self.margin = torch.empty((rows, 3), dtype=torch.float64, device=dev) if want_margin else None
+        self.kept_ids = torch.full((rows, kept_cap), -1, dtype=torch.int32, device=dev) if kept_cap else None
+        self.kept_logits = torch.zeros((rows, kept_cap), dtype=torch.float32, device=dev) if kept_cap else None
+        b = Batch()
+        b.logits, b.dtype = _p(logits), DTYPE_F32 if logits.dtype == torch.float32 else DTYPE_BF16
+        b.rows, b.vocab, b.row_stride = rows, V, logits.stride(0)
+        b.inv_t, b.top_k, b.top_p, b.min_p = _p(inv_t), _p(top_k), _p(top_p), _p(min_p)
+        b.seed, b.step, b.rng = _p(seed), _p(step), rng
+        b.hist, b.hist_off, b.rep, b.pres, b.freq = _p(hist), _p(hist_off), _p(rep), _p(pres), _p(freq)
+        b.bias_ids, b.bias_vals, b.bias_off = _p(bias_ids), _p(bias_vals), _p(bias_off)
+        b.max_hist, b.max_bias = max_hist, max_bias
+        b.allow, b.allow_stride = _p(allow), (allow.stride(0) if allow is not None else 0)
+        b.token, b.prob, b.n_kept, b.flags = _p(self.token), _p(self.prob), _p(self.n_kept), _p(self.flags)
+        b.stats, b.margin = _p(self.stats), _p(self.margin)
+        b.kept_ids, b.kept_logits, b.kept_cap = _p(self.kept_ids), _p(self.kept_logits), kept_cap
+        b.tol = tol
+        need = lib().ws_sample_batch_workspace(C.byref(b))
+        self.workspace = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
+        b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()
+        self.desc = b
+
+    def run(self, stream=None):
+        s = _stream() if stream is None else C.c_void_p(stream)
+        check(lib().ws_sample_batch(s, C.byref(self.desc)), "ws_sample_batch")
+        return self
+
+
+def spec_verify_classic(p, q, draft, seed, step0, rng=RNG_PHILOX, tol=0.0):
+    """p, q: [n_seq, n_pos, V] float32 device; draft: [n_seq, n_pos - 1] int32; seed, step0: uint64-as-int64 [n_seq]."""
+    n_seq, n_pos, V = p.shape
+    dev = p.device
+    out = torch.full((n_seq, n_pos), -1, dtype=torch.int32, device=dev)
+    nacc = torch.empty(n_seq, dtype=torch.int32, device=dev)
+    flags = torch.empty(n_seq, dtype=torch.int32, device=dev)
+    v = SpecVerify(_p(p), _p(q), _p(draft), n_seq, n_pos, V, _p(seed), _p(step0), rng, _p(out), _p(nacc), _p(flags), None, 0,
+                   tol)
+    check(lib().ws_spec_verify_classic(_stream(), C.byref(v)), "ws_spec_verify_classic")
+    return nacc, out, flags

@@ -1,0 +1,40 @@
+"""Builds the gfx950 binaries in-tree (hipcc cross-compiles without a GPU):
+
+  libwhirl_sampling_hip.so   the C-ABI library (include/whirl_sampling_abi.h)
+  whirl_sampling_gfx950.co   the code object alone, for callers that resolve kernels by name (hipModuleGetFunction)
+
+Usage: python whirl-llm_amd/build.py
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "csrc", "ws_abi.hip")
+# packed FP32 instructions are switched off for every device compile of this repository
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "'-packed-fp32-ops' is not a recognized feature"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError("build failed: " + " ".join(cmd) + "\n" + err)
+    return err
+
+
+def build(verbose=True):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    so = os.path.join(HERE, "libwhirl_sampling_hip.so")
+    co = os.path.join(HERE, "whirl_sampling_gfx950.co")
+    run([hipcc, *FLAGS, "-fPIC", "-shared", "-o", so, SRC])
+    run([hipcc, *FLAGS, "--genco", "-o", co, SRC])
+    if verbose:
+        print("built", so, "and", co)
+    return so, co
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

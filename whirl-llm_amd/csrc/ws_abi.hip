@@ -1,0 +1,207 @@
+// C ABI of libwhirl_sampling_hip.so (include/whirl_sampling_abi.h): argument checks on the host, launch geometry,
+// by-value launch structs. No allocation, no synchronisation, no host copies of device data.
+#include "../../include/whirl_sampling_abi.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "ws_common.h"
+#include "ws_draft.h"
+#include "ws_pick.h"
+#include "ws_sample.h"
+#include "ws_spec.h"
+#include "ws_topk.h"
+
+namespace {
+
+inline hipStream_t S(void* s) { return static_cast<hipStream_t>(s); }
+inline int done() { return static_cast<int>(hipGetLastError()); }
+
+constexpr uint32_t kMaxLds = 160u * 1024u;  // LDS per workgroup on gfx950
+
+struct BatchPlan {
+    uint32_t patch_cap;
+    uint32_t lds_ab;
+    uint32_t lds_total;
+    uint64_t workspace;
+    int err;
+};
+
+BatchPlan plan_batch(const ws_batch* b) {
+    BatchPlan p{};
+    p.err = WS_E_INVALID;
+    if (!b || !b->logits || !b->inv_t || !b->seed || !b->step || !b->token || !b->flags) return p;
+    if (b->rows == 0 || b->vocab == 0 || b->vocab > 1048575u || b->row_stride < b->vocab) return p;
+    if (b->dtype != WS_DTYPE_F32 && b->dtype != WS_DTYPE_BF16) return p;
+    if (b->rng != WS_RNG_SPLITMIX && b->rng != WS_RNG_PHILOX) return p;
+    if (b->hist && !b->hist_off) return p;
+    if (b->bias_ids && (!b->bias_off || !b->bias_vals)) return p;
+    if (b->kept_ids && b->kept_cap == 0) return p;
+    const uint64_t cap = (b->hist ? uint64_t{b->max_hist} : 0) + (b->bias_ids ? uint64_t{b->max_bias} : 0);
+    const uint32_t nW = (b->vocab + 31u) / 32u;
+    const uint64_t ab = cap * 8u > 65536u ? ((cap * 8u + 15u) & ~uint64_t{15}) : 65536u;
+    const uint64_t total = ab + uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
+    p.err = WS_E_UNSUPPORTED;
+    if (cap > 65535u || total + 1024u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
+    p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
+    p.lds_ab = static_cast<uint32_t>(ab);
+    p.lds_total = static_cast<uint32_t>(total);
+    p.workspace = uint64_t{b->rows} * p.patch_cap * sizeof(float4);
+    p.err = WS_OK;
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ws_abi_version(void) { return WS_ABI_VERSION; }
+
+const char* ws_error_string(int code) {
+    switch (code) {
+    case WS_OK: return "ok";
+    case WS_E_INVALID: return "invalid argument";
+    case WS_E_WORKSPACE: return "workspace missing or too small";
+    case WS_E_UNSUPPORTED: return "unsupported combination";
+    case WS_E_NO_DEVICE: return "no usable HIP device";
+    default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
+    }
+}
+
+int ws_probe(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return WS_E_NO_DEVICE;
+    }
+    hipFuncAttributes fa;
+    if (hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(&argmax_rows)) != hipSuccess) {
+        (void)hipGetLastError();
+        return WS_E_NO_DEVICE;
+    }
+    return WS_OK;
+}
+
+int ws_argmax(void* stream, const float* x, int n, int* out, int* ids, int* pos, int advance) {
+    if (!x || !out || !ids || !pos || n <= 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(argmax, dim3(1), dim3(WS_BLOCK), 0, S(stream), x, n, out, ids, pos, advance);
+    return done();
+}
+
+int ws_argmax_rows(void* stream, const float* x, int n, int* out, unsigned rows) {
+    if (!x || !out || n <= 0 || rows == 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(argmax_rows, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, out);
+    return done();
+}
+
+int ws_argmax_rows_to(void* stream, const float* x, int n, int* out, const ws_row_idx* dst, unsigned rows) {
+    if (!x || !out || !dst || n <= 0 || rows == 0 || rows > WS_MAX_TABLE_ROWS) return WS_E_INVALID;
+    RowIdx d;
+    std::memcpy(&d, dst, sizeof d);
+    hipLaunchKernelGGL(argmax_rows_to, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, out, d);
+    return done();
+}
+
+int ws_argmax_prob(void* stream, const float* x, int n, int* out_tok, float* out_prob) {
+    if (!x || !out_tok || !out_prob || n <= 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(argmax_prob, dim3(1), dim3(WS_BLOCK), 0, S(stream), x, n, out_tok, out_prob);
+    return done();
+}
+
+int ws_draft_pick(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
+                  const int* map) {
+    if (!x || !tok || !prob || !ctl || n <= 0 || r < 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(draft_pick, dim3(1), dim3(WS_BLOCK), 0, S(stream), x, n, tok, prob, ctl, r, n_min, p_min, map);
+    return done();
+}
+
+int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min, float p_min,
+                       const int* map, unsigned rows) {
+    if (!x || !ctl_all || !area || n <= 0 || r < 0 || r >= 16 || rows == 0 || rows > WS_MAX_TABLE_ROWS) return WS_E_INVALID;
+    RowIdx a;
+    std::memcpy(&a, area, sizeof a);
+    hipLaunchKernelGGL(draft_pick_rows, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, ctl_all, a, r, n_min, p_min, map);
+    return done();
+}
+
+int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
+                         const ws_dsamp_args* a, int* qbuf, unsigned rows) {
+    if (!x || !ctl_all || !area || !a || !qbuf || n <= 0 || r < 0 || r >= 16 || rows == 0 || rows > WS_MAX_TABLE_ROWS)
+        return WS_E_INVALID;
+    RowIdx ar;
+    DSampArgs da;
+    static_assert(sizeof(DSampArgs) == sizeof(ws_dsamp_args) && sizeof(DSampArgs) == 1024, "DSampArgs layout");
+    std::memcpy(&ar, area, sizeof ar);
+    std::memcpy(&da, a, sizeof da);
+    hipLaunchKernelGGL(draft_sample_rows, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, ctl_all, ar, r, map, da, qbuf);
+    return done();
+}
+
+int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows) {
+    if (!x || !ids || !vals || !stats || n <= 0 || K <= 0 || rows == 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(topk_rows, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, K, inv_t, ids, vals, stats);
+    return done();
+}
+
+uint64_t ws_sample_batch_workspace(const ws_batch* b) {
+    const BatchPlan p = plan_batch(b);
+    return p.err == WS_OK ? p.workspace : 0;
+}
+
+int ws_sample_batch(void* stream, const ws_batch* b) {
+    const BatchPlan p = plan_batch(b);
+    if (p.err != WS_OK) return p.err;
+    if (!b->workspace || b->workspace_bytes < p.workspace) return WS_E_WORKSPACE;
+    ws::BatchArgs a{};
+    a.logits = b->logits;
+    a.dtype = b->dtype;
+    a.rows = b->rows;
+    a.vocab = b->vocab;
+    a.row_stride = b->row_stride;
+    a.inv_t = b->inv_t;
+    a.top_k = b->top_k;
+    a.top_p = b->top_p;
+    a.min_p = b->min_p;
+    a.seed = b->seed;
+    a.step = b->step;
+    a.rng = b->rng;
+    a.hist = b->hist;
+    a.hist_off = b->hist_off;
+    a.rep = b->rep;
+    a.pres = b->pres;
+    a.freq = b->freq;
+    a.bias_ids = b->bias_ids;
+    a.bias_vals = b->bias_vals;
+    a.bias_off = b->bias_off;
+    a.patch_cap = p.patch_cap;
+    a.allow = b->allow;
+    a.allow_stride = b->allow_stride;
+    a.token = b->token;
+    a.prob = b->prob;
+    a.n_kept = b->n_kept;
+    a.flags = b->flags;
+    a.stats = b->stats;
+    a.margin = b->margin;
+    a.kept_ids = b->kept_ids;
+    a.kept_logits = b->kept_logits;
+    a.kept_cap = b->kept_cap;
+    a.patch = static_cast<float4*>(b->workspace);
+    a.tol = b->tol > 0 ? b->tol : 1.0 / 1099511627776.0;
+    a.lds_ab = p.lds_ab;
+    static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
+    if (!attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
+        if (e != hipSuccess) return static_cast<int>(e);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(ws::sample_batch_kernel, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
+    return done();
+}
+
+uint64_t ws_spec_verify_workspace(const ws_spec_verify* v) { return ws::spec_workspace(v); }
+
+int ws_spec_verify_classic(void* stream, const ws_spec_verify* v) { return ws::spec_launch(S(stream), v); }
+
+}  // extern "C"

@@ -1,0 +1,191 @@
+// Device helpers shared by the gfx950 sampling kernels: wave64 / block reductions and scans, order-preserving
+// float keys, vectorised row iteration. One workgroup = WS_BLOCK threads = 16 wave64 waves.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WS_BLOCK 1024
+#define WS_WAVES (WS_BLOCK / 64)
+
+namespace ws {
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// ---- order-preserving key of a float (larger float -> larger key); -0 and +0 share a key because the host order
+// compares floats (src/sampling/sampler.cpp:18-21), NaN never reaches here (callers turn it into -inf first)
+__device__ __forceinline__ uint32_t key32(float f) {
+    uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) u = 0u;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float unkey32(uint32_t k) {
+    const uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __uint_as_float(u);
+}
+// (logit desc, id asc) as one descending 64-bit key
+__device__ __forceinline__ uint64_t key64(float f, uint32_t id) {
+    return (static_cast<uint64_t>(key32(f)) << 32) | static_cast<uint64_t>(0xffffffffu - id);
+}
+
+// ---- wave reductions (xor butterflies; every lane gets the result)
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// greedy pick: the larger value, on equal values the lower index (kernels/shared/block_argmax.h:16)
+struct Best {
+    float v;
+    int i;
+};
+__device__ __forceinline__ Best pick(Best a, Best b) { return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a; }
+__device__ __forceinline__ Best wave_best(Best a) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        Best b;
+        b.v = __shfl_xor(a.v, o);
+        b.i = __shfl_xor(a.i, o);
+        a = pick(a, b);
+    }
+    return a;
+}
+
+// ---- block reductions; `red` is caller LDS of >= WS_WAVES entries; all threads get the result. Two barriers.
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    __syncthreads();
+    if (lane_id() == 0) red[wave_id()] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < WS_WAVES; ++w) r = fmaxf(r, red[w]);
+    return r;
+}
+__device__ __forceinline__ Best block_best(Best b, float* red_v, int* red_i) {
+    b = wave_best(b);
+    __syncthreads();
+    if (lane_id() == 0) {
+        red_v[wave_id()] = b.v;
+        red_i[wave_id()] = b.i;
+    }
+    __syncthreads();
+    Best r = {red_v[0], red_i[0]};
+#pragma unroll
+    for (int w = 1; w < WS_WAVES; ++w) r = pick(r, Best{red_v[w], red_i[w]});
+    return r;
+}
+// sum in a fixed order (wave butterflies, then waves 0..15): the same bits on every run
+template <class T>
+__device__ __forceinline__ T block_sum(T v, T* red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane_id() == 0) red[wave_id()] = v;
+    __syncthreads();
+    T r = red[0];
+#pragma unroll
+    for (int w = 1; w < WS_WAVES; ++w) r += red[w];
+    return r;
+}
+
+// ---- block exclusive scan of one value per thread (thread order); returns the exclusive prefix, *total = block sum
+template <class T>
+__device__ __forceinline__ T block_excl_scan(T v, T* red, T* total) {
+    T inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const T up = __shfl_up(inc, o);
+        if (lane_id() >= o) inc += up;
+    }
+    __syncthreads();
+    if (lane_id() == 63) red[wave_id()] = inc;
+    __syncthreads();
+    T base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < WS_WAVES; ++w) {
+        const T s = red[w];
+        if (w < wave_id()) base += s;
+        tot += s;
+    }
+    *total = tot;
+    return base + inc - v;
+}
+
+// ---- bf16 -> f32 (exact widening)
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(static_cast<uint32_t>(h) << 16); }
+
+// ---- row iteration: f(i, x[i]) for every i in [0, n); each thread visits its indices in increasing order.
+// 128-bit loads on the 16-byte aligned body of the row, scalar loads on a misaligned head and the tail.
+template <class F>
+__device__ __forceinline__ void for_each_f32(const float* __restrict__ x, int n, F&& f) {
+    const int t = threadIdx.x;
+    int head = static_cast<int>(((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(x)) & 15u)) & 15u) >> 2);
+    if (head > n) head = n;
+    if (t < head) f(t, x[t]);
+    const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + head);
+    const int nv = (n - head) >> 2;
+#pragma unroll 4
+    for (int j = t; j < nv; j += WS_BLOCK) {
+        const float4 v = xv[j];
+        const int i = head + 4 * j;
+        f(i, v.x);
+        f(i + 1, v.y);
+        f(i + 2, v.z);
+        f(i + 3, v.w);
+    }
+    const int i = head + 4 * nv + t;
+    if (i < n) f(i, x[i]);
+}
+
+// ---- RNG: the reference's stateless splitmix streams (src/common/spec_sample.cpp:13-21, include/whirl/spec_sample.h:53-60)
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__device__ __forceinline__ double unit53(uint64_t z) { return static_cast<double>(z >> 11) * (1.0 / 9007199254740992.0); }
+__device__ __forceinline__ double splitmix_uniform(uint64_t seed, uint64_t pos, uint32_t stream) {
+    if (stream) seed ^= static_cast<uint64_t>(stream) * 0xD1B54A32D192ED03ull;
+    return unit53(mix64(seed + (pos + 1) * 0x9E3779B97F4A7C15ull));
+}
+// Philox4x32-10 (Salmon et al., SC'11): ctr = (step_lo, step_hi, row, stream), key = (seed_lo, seed_hi)
+__device__ __forceinline__ double philox_uniform(uint64_t seed, uint32_t row, uint64_t step, uint32_t stream) {
+    uint32_t c0 = static_cast<uint32_t>(step), c1 = static_cast<uint32_t>(step >> 32), c2 = row, c3 = stream;
+    uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t a = static_cast<uint64_t>(0xD2511F53u) * c0;
+        const uint64_t b = static_cast<uint64_t>(0xCD9E8D57u) * c2;
+        const uint32_t n0 = static_cast<uint32_t>(b >> 32) ^ c1 ^ k0;
+        const uint32_t n2 = static_cast<uint32_t>(a >> 32) ^ c3 ^ k1;
+        c1 = static_cast<uint32_t>(b);
+        c3 = static_cast<uint32_t>(a);
+        c0 = n0;
+        c2 = n2;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return unit53((static_cast<uint64_t>(c1) << 32) | c0);
+}
+__device__ __forceinline__ double batch_uniform(int rng, uint64_t seed, uint32_t row, uint64_t step, uint32_t stream) {
+    return rng == 0 ? splitmix_uniform(seed, step, stream) : philox_uniform(seed, row, step, stream);
+}
+
+}  // namespace ws

@@ -1,0 +1,107 @@
+// Greedy picks for gfx950: argmax, argmax_rows, argmax_rows_to, argmax_prob, draft_pick, draft_pick_rows.
+// Same names, argument lists and results as the reference kernels (kernels/shared/misc_kv_argmax_kv_store.h:32-42,
+// kernels/shared/sample_pick_set_tokens.h:15-21, 47-53, 60-105); one pass over the row with 128-bit loads:
+// the maximum (first index on ties, kernels/shared/block_argmax.h:16) and, where a probability is asked for,
+// sum exp(x - max) by an online rescaled sum instead of the reference's second pass
+// (kernels/shared/block_argmax_psum.h). NaN logits are never picked and add nothing to the sum.
+#pragma once
+
+#include "ws_common.h"
+
+namespace ws {
+
+struct RowTop {
+    Best best;  // maximum and its first index
+    float sum;  // sum_i exp(x_i - max) when asked for
+};
+
+template <bool WITH_SUM>
+__device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
+    __shared__ float red_v[WS_WAVES];
+    __shared__ int red_i[WS_WAVES];
+    __shared__ float red_s[WS_WAVES];
+    Best b = {-INFINITY, 0};
+    float s = 0.f;
+    for_each_f32(x, n, [&](int i, float v) {
+        if (v > b.v) {
+            if (WITH_SUM) s = s * __expf(b.v - v) + 1.f;
+            b.v = v;
+            b.i = i;
+        } else if (WITH_SUM && v > -INFINITY) {
+            s += __expf(v - b.v);
+        }
+    });
+    RowTop r;
+    r.best = block_best(b, red_v, red_i);
+    r.sum = 0.f;
+    if (WITH_SUM) {
+        const float part = b.v > -INFINITY ? s * __expf(b.v - r.best.v) : 0.f;
+        r.sum = block_sum(part, red_s);
+    }
+    return r;
+}
+
+// kernels/shared/sample_pick_set_tokens.h:60-86
+__device__ __forceinline__ void draft_pick_row(const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min,
+                                               float p_min, const int* map) {
+    if (r > 0 && ctl[1] != 0) return;  // the chain stopped at an earlier draft (uniform over the block)
+    const RowTop t = row_top<true>(x, n);
+    if (threadIdx.x == 0) {
+        const float p = 1.f / t.sum;
+        tok[r] = map ? map[t.best.i] : t.best.i;
+        prob[r] = p;
+        if (p_min > 0.f && r >= n_min && p < p_min) {
+            ctl[0] = r;
+            ctl[1] = 1;
+        } else {
+            ctl[0] = r + 1;
+            if (r == 0) ctl[1] = 0;
+        }
+    }
+}
+
+}  // namespace ws
+
+struct RowIdx {
+    int v[32];
+};
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) argmax(const float* x, int n, int* out, int* ids, int* pos, int advance) {
+    const ws::RowTop t = ws::row_top<false>(x, n);
+    if (threadIdx.x == 0) {
+        out[0] = t.best.i;
+        ids[0] = t.best.i;
+        pos[0] += advance;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) argmax_rows(const float* x, int n, int* out) {
+    const ws::RowTop t = ws::row_top<false>(x + static_cast<size_t>(blockIdx.x) * n, n);
+    if (threadIdx.x == 0) out[blockIdx.x] = t.best.i;
+}
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) argmax_rows_to(const float* x, int n, int* out, RowIdx dst) {
+    const ws::RowTop t = ws::row_top<false>(x + static_cast<size_t>(blockIdx.x) * n, n);
+    if (threadIdx.x == 0) out[dst.v[blockIdx.x]] = t.best.i;
+}
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) argmax_prob(const float* x, int n, int* out_tok, float* out_prob) {
+    const ws::RowTop t = ws::row_top<true>(x, n);
+    if (threadIdx.x == 0) {
+        out_tok[0] = t.best.i;
+        out_prob[0] = 1.f / t.sum;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_pick(const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min, const int* map) {
+    ws::draft_pick_row(x, n, tok, prob, ctl, r, n_min, p_min, map);
+}
+
+// control area of the row's sequence at ctl_all + area.v[row]: drafts at +16, probabilities at +32, (nd, stop) at +48
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_pick_rows(const float* x, int n, int* ctl_all, RowIdx area, int r, int n_min, float p_min, const int* map) {
+    int* c = ctl_all + area.v[blockIdx.x];
+    ws::draft_pick_row(x + static_cast<size_t>(blockIdx.x) * n, n, c + 16, reinterpret_cast<float*>(c + 32), c + 48, r, n_min,
+                       p_min, map);
+}

@@ -1,0 +1,189 @@
+// Classic speculative sampling for gfx950 (Leviathan et al. 2023, Chen et al. 2023): accept draft j while
+// u_j * q_j(d_j) < p_j(d_j); at the first rejection draw from max(p_j - q_j, 0), after the last draft from p.
+// The reference removed this rule (include/whirl/spec_sample.h:22-24); the result is defined by the closed form
+// in include/whirl_sampling_abi.h. One workgroup per sequence: the accept chain needs 2 gathers per draft, the
+// resample streams exactly one row pair once (per-256-element sums in id order kept in LDS, a scan over them,
+// and a re-read of the one 1 KiB step the draw lands in).
+#pragma once
+
+#include "../../include/whirl_sampling_abi.h"
+#include "ws_common.h"
+
+namespace ws {
+
+constexpr uint32_t kSpecMaxSteps = 4096;  // 256-element steps of a row: vocab <= 1048576
+constexpr uint32_t kSpecNear = 4u;  // WS_FLAG_NEAR_DRAW
+
+struct SpecArgs {
+    const float* p;
+    const float* q;
+    const int32_t* draft;
+    uint32_t n_seq, n_pos, vocab;
+    const uint64_t* seed;
+    const uint64_t* step0;
+    int rng;
+    int32_t* out_tokens;
+    int32_t* n_accepted;
+    uint32_t* flags;
+    double tol;
+};
+
+__global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
+    __shared__ double step_sum[kSpecMaxSteps];
+    __shared__ double red_d[WS_WAVES];
+    __shared__ uint32_t s_u[4];
+    __shared__ double s_d[4];
+    const uint32_t s = blockIdx.x, t = threadIdx.x, V = A.vocab, P = A.n_pos;
+    const float* p = A.p + static_cast<size_t>(s) * P * V;
+    const float* q = A.q + static_cast<size_t>(s) * P * V;
+    const int32_t* dr = A.draft + static_cast<size_t>(s) * (P - 1);
+    int32_t* out = A.out_tokens + static_cast<size_t>(s) * P;
+    const uint64_t seed = A.seed[s], step0 = A.step0[s];
+
+    if (t == 0) {  // accept chain
+        uint32_t j = 0, fl = 0;
+        for (; j + 1 < P; ++j) {
+            const int32_t d = dr[j];
+            const double pj = p[static_cast<size_t>(j) * V + d], qj = q[static_cast<size_t>(j) * V + d];
+            const double lhs = batch_uniform(A.rng, seed, s, step0 + j, 0) * qj;
+            if (fabs(lhs - pj) < A.tol * pj) fl |= kSpecNear;
+            if (!(lhs < pj)) break;
+            out[j] = d;
+        }
+        s_u[0] = j;
+        s_u[1] = fl;
+    }
+    __syncthreads();
+    const uint32_t j = s_u[0];
+    uint32_t flags = s_u[1];
+    const float* pr = p + static_cast<size_t>(j) * V;
+    const float* qr = q + static_cast<size_t>(j) * V;
+    const uint32_t n_steps = (V + 255u) >> 8;
+    const uint32_t w = wave_id(), l = lane_id();
+    bool from_p = j + 1 == P;
+    double total = 0;
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        // weights in id order: step k covers ids [256k, 256k + 256), lane l the four ids 256k + 4l ..
+        for (uint32_t k = w; k < n_steps; k += WS_WAVES) {
+            const uint32_t i = (k << 8) + 4u * l;
+            double acc = 0;
+            if (i + 3 < V && (reinterpret_cast<uintptr_t>(pr) & 15u) == 0 && (reinterpret_cast<uintptr_t>(qr) & 15u) == 0) {
+                const float4 a = *reinterpret_cast<const float4*>(pr + i);
+                float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (!from_p) b = *reinterpret_cast<const float4*>(qr + i);
+                const float r0 = a.x - b.x, r1 = a.y - b.y, r2 = a.z - b.z, r3 = a.w - b.w;
+                acc += r0 > 0.f ? static_cast<double>(r0) : 0.0;
+                acc += r1 > 0.f ? static_cast<double>(r1) : 0.0;
+                acc += r2 > 0.f ? static_cast<double>(r2) : 0.0;
+                acc += r3 > 0.f ? static_cast<double>(r3) : 0.0;
+            } else {
+                for (uint32_t e = 0; e < 4 && i + e < V; ++e) {
+                    const float r = from_p ? pr[i + e] : pr[i + e] - qr[i + e];
+                    acc += r > 0.f ? static_cast<double>(r) : 0.0;
+                }
+            }
+            acc = wave_sum(acc);
+            if (l == 0) step_sum[k] = acc;
+        }
+        __syncthreads();
+        // scan of the step sums: thread t owns steps 4t .. 4t+3
+        double loc[4], lsum = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t k = 4 * t + e;
+            loc[e] = k < n_steps ? step_sum[k] : 0.0;
+            lsum += loc[e];
+        }
+        double run = block_excl_scan(lsum, red_d, &total);
+        if (!(total > 0) && !from_p) {  // zero residual: fall back to p
+            from_p = true;
+            __syncthreads();
+            continue;
+        }
+        const double target = batch_uniform(A.rng, seed, s, step0 + j, 1) * total;
+        if (t == 0) s_u[2] = 0xffffffffu;
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const double inc = run + loc[e];
+            if (inc > target && !(run > target) && loc[e] > 0) {
+                s_u[2] = 4 * t + e;
+                s_d[0] = run;
+            }
+            run = inc;
+        }
+        __syncthreads();
+        uint32_t k = s_u[2];
+        double base = s_d[0];
+        if (k == 0xffffffffu) {  // target at the very end by rounding: the last step with weight
+            k = n_steps - 1;
+            base = total;
+            flags |= kSpecNear;
+        }
+        // the step the draw lands in, re-read by wave 0: lane prefix, then the four elements of the lane
+        if (w == 0) {
+            const uint32_t i = (k << 8) + 4u * l;
+            double wv[4], lsum2 = 0;
+            for (uint32_t e = 0; e < 4; ++e) {
+                float r = 0.f;
+                if (i + e < V) r = from_p ? pr[i + e] : pr[i + e] - qr[i + e];
+                wv[e] = r > 0.f ? static_cast<double>(r) : 0.0;
+                lsum2 += wv[e];
+            }
+            double inc = lsum2;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const double up = __shfl_up(inc, o);
+                if (l >= static_cast<uint32_t>(o)) inc += up;
+            }
+            double cum = base + inc - lsum2;
+            int32_t tok = -1;
+            double mg = 1.0;
+            for (uint32_t e = 0; e < 4; ++e) {
+                const double before = cum;
+                cum += wv[e];
+                if (tok < 0 && wv[e] > 0 && cum > target && !(before > target)) {
+                    tok = static_cast<int32_t>(i + e);
+                    mg = fmin(cum - target, before > 0 ? target - before : 1e300) / total;
+                }
+            }
+            // first lane that found it wins (lower ids first); none: the last id with weight in the step
+            const uint64_t found = __ballot(tok >= 0);
+            const uint64_t any = __ballot(lsum2 > 0);
+            if (found) {
+                const int src = __ffsll(static_cast<long long>(found)) - 1;
+                tok = __shfl(tok, src);
+                mg = __shfl(mg, src);
+            } else {
+                const int src = any ? 63 - __clzll(static_cast<long long>(any)) : 0;
+                int32_t lastw = -1;
+                for (uint32_t e = 0; e < 4; ++e)
+                    if (wv[e] > 0) lastw = static_cast<int32_t>(i + e);
+                tok = __shfl(lastw, src);
+                mg = 0.0;
+            }
+            if (l == 0) {
+                if (mg < A.tol) flags |= kSpecNear;
+                out[j] = tok;
+                A.n_accepted[s] = static_cast<int32_t>(j);
+                A.flags[s] = flags;
+            }
+        }
+        break;
+    }
+}
+
+inline uint64_t spec_workspace(const ws_spec_verify*) { return 0; }
+
+inline int spec_launch(hipStream_t stream, const ws_spec_verify* v) {
+    if (!v || !v->p || !v->q || !v->draft || !v->seed || !v->step0 || !v->out_tokens || !v->n_accepted || !v->flags)
+        return WS_E_INVALID;
+    if (v->n_seq == 0 || v->n_pos < 1 || v->vocab == 0 || v->vocab > kSpecMaxSteps * 256u) return WS_E_INVALID;
+    if (v->rng != WS_RNG_SPLITMIX && v->rng != WS_RNG_PHILOX) return WS_E_INVALID;
+    SpecArgs a{v->p, v->q, v->draft, v->n_seq, v->n_pos, v->vocab, v->seed, v->step0, v->rng, v->out_tokens, v->n_accepted,
+               v->flags, v->tol > 0 ? v->tol : 1.0 / 1099511627776.0};
+    hipLaunchKernelGGL(spec_verify_kernel, dim3(v->n_seq), dim3(WS_BLOCK), 0, stream, a);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace ws
