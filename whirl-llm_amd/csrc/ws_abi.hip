@@ -41,13 +41,13 @@ BatchPlan plan_batch(const ws_batch* b) {
     const uint64_t cap = (b->hist ? uint64_t{b->max_hist} : 0) + (b->bias_ids ? uint64_t{b->max_bias} : 0);
     const uint32_t nW = (b->vocab + 31u) / 32u;
     const uint64_t ab = cap * 8u > 65536u ? ((cap * 8u + 15u) & ~uint64_t{15}) : 65536u;
-    const uint64_t total = ab + uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
+    const uint64_t total = ab + uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15}) + cap * 4u;
     p.err = WS_E_UNSUPPORTED;
-    if (cap > 65535u || total + 1024u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
+    if (cap > 65535u || total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
-    p.workspace = uint64_t{b->rows} * p.patch_cap * sizeof(float4);
+    p.workspace = 0;  // every intermediate lives in LDS
     p.err = WS_OK;
     return p;
 }
@@ -152,7 +152,7 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b) {
 int ws_sample_batch(void* stream, const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     if (p.err != WS_OK) return p.err;
-    if (!b->workspace || b->workspace_bytes < p.workspace) return WS_E_WORKSPACE;
+    if (p.workspace && (!b->workspace || b->workspace_bytes < p.workspace)) return WS_E_WORKSPACE;
     ws::BatchArgs a{};
     a.logits = b->logits;
     a.dtype = b->dtype;
@@ -186,7 +186,6 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.kept_ids = b->kept_ids;
     a.kept_logits = b->kept_logits;
     a.kept_cap = b->kept_cap;
-    a.patch = static_cast<float4*>(b->workspace);
     a.tol = b->tol > 0 ? b->tol : 1.0 / 1099511627776.0;
     a.lds_ab = p.lds_ab;
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process

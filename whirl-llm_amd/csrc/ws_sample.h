@@ -2,10 +2,10 @@
 //
 // Per row (ws_batch in include/whirl_sampling_abi.h states the order of operations):
 //   phase 0  penalties / bias: an LDS bitmap of the token ids the history and the bias list touch, a per-word
-//            prefix popcount (rank of a touched id = perfect hash), per-rank counts by LDS atomics, and one 16-byte
-//            patch record {bias sum, frequency * count + presence, flags} per touched id in the row's workspace.
-//            Rows stream unmodified from HBM; a touched element (bit set) fetches its record and is adjusted in
-//            flight, so no penalised copy of the row is ever written.
+//            prefix popcount (rank of a touched id = perfect hash), per-rank counts by LDS atomics, then the adjusted
+//            logit of every touched token (one 4-byte gather each) into an LDS array by rank. The passes below stream
+//            the row unmodified, skip touched tokens (bit set) and replay them from that array, so no penalised copy
+//            of the row is ever written and the hot loop has no dependent loads.
 //   pass 1   maximum of the adjusted row (NaN and masked tokens count as -inf).
 //   pass 2   histogram of 4096 bins of width 1/64 in a = (max - x) * inv_t, the exponent of the softmax: one LDS
 //            64-bit atomic per element adds {count, fixed-point 1 - exp(-(a - bin edge))} (degree-4 polynomial, no
@@ -22,6 +22,7 @@
 #pragma once
 
 #include "ws_common.h"
+#include "ws_exp_table.h"
 
 namespace ws {
 
@@ -30,7 +31,9 @@ constexpr uint32_t kCap = 4096;          // candidates resolved exactly in LDS p
 constexpr int kCountShift = 44;          // histogram word: count << 44 | fixed-point sum of (1 - exp(-w))
 constexpr float kFixScale = 1073741824.f;  // 2^30
 constexpr double kFixInv = 1.0 / 1073741824.0;
-constexpr float kEdgeShift = 3.814697265625e-6f;  // 2^-18: keeps w positive against the rounding of a
+constexpr float kEdgeShift = 2.44140625e-4f;  // 2^-12 bins: keeps the in-bin offset positive against the rounding of t
+// 2^30 * (1 - exp(-w / 64)) = w * (k0 + w * (k1 + w * k2)) for the in-bin offset w in [0, 1.02] (max error 1.4e-10 * 2^30)
+constexpr float kG0 = 16777216.0f, kG1 = -131070.34375f, kG2 = 678.6015014648438f;
 
 // flag bits (WS_FLAG_* of the C ABI)
 constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u;
@@ -67,138 +70,175 @@ struct BatchArgs {
     int32_t* kept_ids;
     float* kept_logits;
     uint32_t kept_cap;
-    float4* patch;  // workspace: rows * patch_cap records
     double tol;
     uint32_t lds_ab;  // bytes of the LDS region shared by the histogram / sort keys / masses / phase-0 counters
 };
 
-// One row as the passes see it: raw logits plus what adjusts them in flight.
+// One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
+// replayed from LDS, where phase 0 left their adjusted logits by rank.
 struct RowView {
     const void* base;
     uint32_t V;
     int dtype;
-    bool vec;               // 16-byte aligned base: 128-bit loads
-    const uint32_t* allow;  // global bitmap of the row or nullptr
+    bool vec;                 // 16-byte aligned base: 128-bit loads
+    const uint32_t* allow;    // global bitmap of the row or nullptr
     const uint32_t* touched;  // LDS bitmap or nullptr
     const uint16_t* wprefix;  // LDS per-word exclusive popcount prefix
-    const float4* patch;      // global records by rank
-    float rep;
+    const float* pv;          // LDS adjusted logits of the touched tokens, by rank
 };
 
-__device__ __forceinline__ float patch_one(const RowView& rv, float x, uint32_t i, uint32_t tword) {
-    const uint32_t bit = i & 31u;
-    const uint32_t rank = rv.wprefix[i >> 5] + __popc(tword & ((1u << bit) - 1u));
-    const float4 rec = rv.patch[rank];
-    const uint32_t fl = __float_as_uint(rec.z);
-    if (fl & 2u) x = __fadd_rn(x, rec.x);
-    if (fl & 1u) {
-        x = x > 0.f ? __fdiv_rn(x, rv.rep) : __fmul_rn(x, rv.rep);
-        x = __fsub_rn(x, rec.y);
-    }
-    return x;
+constexpr int kBatch = 4;  // 128-bit loads per thread and batch; two batches are in flight (double buffering)
+
+__device__ __forceinline__ float raw_logit(const RowView& rv, uint32_t i) {
+    const float v = rv.dtype == 0 ? static_cast<const float*>(rv.base)[i] : bf16_to_f32(static_cast<const uint16_t*>(rv.base)[i]);
+    return fmaxf(v, -INFINITY);  // NaN -> -inf
+}
+__device__ __forceinline__ bool is_allowed(const RowView& rv, uint32_t i) {
+    return !rv.allow || ((rv.allow[i >> 5] >> (i & 31u)) & 1u);
+}
+__device__ __forceinline__ bool is_touched(const RowView& rv, uint32_t i) {
+    return rv.touched && ((rv.touched[i >> 5] >> (i & 31u)) & 1u);
+}
+__device__ __forceinline__ uint32_t rank_of(const RowView& rv, uint32_t i) {
+    return static_cast<uint32_t>(rv.wprefix[i >> 5]) + __popc(rv.touched[i >> 5] & ((1u << (i & 31u)) - 1u));
+}
+// adjusted logit of any token (slow path: the kept-set dump)
+__device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
+    if (is_touched(rv, i)) return rv.pv[rank_of(rv, i)];
+    return is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY;
 }
 
-// f(i, adjusted logit) for every token of the row
-template <class F>
-__device__ __forceinline__ void stream_row(const RowView& rv, F&& f) {
+// f(i, logit, slot) for every token of the row, slot = position inside the thread's current batch (a compile-time
+// constant after unrolling); end_batch(j0, i) after each batch of kBatch 128-bit loads per thread (j0 = first vector
+// index of the batch; j0 = ~0 and i = the token for the one-token batches of a scalar tail), which are all issued
+// before any is used, and the next batch is requested before this one is consumed (one workgroup keeps 128 KiB of the
+// row in flight). Tokens that are masked out or that the
+// history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bin or ignores it, so the
+// hot loop has no branch. With STASH the raw logits of touched tokens are copied to stash[rank] on the way (the row
+// is read from HBM exactly once for them too); replay_touched later feeds their adjusted values.
+template <bool STASH, bool MASKED, class F, class E>
+__device__ __forceinline__ void stream_row_impl(const RowView& rv, float* stash, F&& f, E&& end_batch) {
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
-    if (rv.dtype == 0) {
-        const float* __restrict__ x = static_cast<const float*>(rv.base);
-        const uint32_t nv = rv.vec ? (V >> 2) : 0u;
-        const float4* __restrict__ xv = reinterpret_cast<const float4*>(x);
-#pragma unroll 2
-        for (uint32_t j = t; j < nv; j += WS_BLOCK) {
-            const float4 q = xv[j];
-            const uint32_t i = 4u * j;
-            float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
-            const uint32_t sh = i & 31u;
-            const uint32_t tw = rv.touched ? rv.touched[i >> 5] : 0u;
-            const uint32_t aw = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
-            if ((((tw >> sh) & 15u) | (((~aw) >> sh) & 15u)) != 0u) {
+    const uint32_t per = rv.dtype == 0 ? 4u : 8u;  // elements per 128-bit load
+    const uint32_t nv = rv.vec ? V / per : 0u;
+    const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
+    constexpr bool masked = MASKED;
+    constexpr uint32_t kStep = kBatch * WS_BLOCK;
+    struct Batch {
+        uint4 q[kBatch];
+        uint32_t na[kBatch];  // complement of the allow words
+    };
+    auto load = [&](uint32_t j0, Batch& b) {
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t j = j0 + u * WS_BLOCK + t;
+            const uint32_t jc = j < nv ? j : nv - 1u;
+            b.q[u] = xv[jc];
+            b.na[u] = (MASKED && rv.allow) ? ~rv.allow[(jc * per) >> 5] : 0u;
+        }
+    };
+    Batch cur, nxt;
+    if (nv) load(0, cur);
+    for (uint32_t j0 = 0; j0 < nv; j0 += kStep) {
+        const bool more = j0 + kStep < nv;
+        if (more) load(j0 + kStep, nxt);  // the next batch is in flight while this one is consumed
+        uint32_t tslots = 0;              // STASH: touched tokens among this thread's (at most 32) batch slots
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t j = j0 + u * WS_BLOCK + t;
+            if (j >= nv) continue;
+            const uint32_t i = j * per;
+            const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
+            const int32_t bw = static_cast<int32_t>((cur.na[u] | tw) >> (i & 31u));
+            if (STASH) tslots |= ((tw >> (i & 31u)) & (per == 4u ? 15u : 255u)) << (u * per);
+            const uint32_t w[4] = {cur.q[u].x, cur.q[u].y, cur.q[u].z, cur.q[u].w};
+            if (rv.dtype == 0) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (!((aw >> (sh + e)) & 1u)) v[e] = -INFINITY;
-                    if ((tw >> (sh + e)) & 1u) v[e] = patch_one(rv, v[e], i + e, tw);
+                    uint32_t bits = w[e];
+                    if (masked) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);  // bit e set -> all ones = NaN
+                    f(i + e, __uint_as_float(bits), u * 4 + e);
                 }
-            }
-            f(i, v[0]);
-            f(i + 1, v[1]);
-            f(i + 2, v[2]);
-            f(i + 3, v[3]);
-        }
-        for (uint32_t i = 4u * nv + t; i < V; i += WS_BLOCK) {
-            float v = fmaxf(x[i], -INFINITY);
-            const uint32_t tw = rv.touched ? rv.touched[i >> 5] : 0u;
-            if (rv.allow && !((rv.allow[i >> 5] >> (i & 31u)) & 1u)) v = -INFINITY;
-            if ((tw >> (i & 31u)) & 1u) v = patch_one(rv, v, i, tw);
-            f(i, v);
-        }
-    } else {
-        const uint16_t* __restrict__ x = static_cast<const uint16_t*>(rv.base);
-        const uint32_t nv = rv.vec ? (V >> 3) : 0u;
-        const uint4* __restrict__ xv = reinterpret_cast<const uint4*>(x);
-#pragma unroll 2
-        for (uint32_t j = t; j < nv; j += WS_BLOCK) {
-            const uint4 q = xv[j];
-            const uint32_t i = 8u * j;
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-            float v[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[2 * e] = fmaxf(__uint_as_float(w[e] << 16), -INFINITY);
-                v[2 * e + 1] = fmaxf(__uint_as_float(w[e] & 0xffff0000u), -INFINITY);
-            }
-            const uint32_t sh = i & 31u;
-            const uint32_t tw = rv.touched ? rv.touched[i >> 5] : 0u;
-            const uint32_t aw = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
-            if ((((tw >> sh) & 255u) | (((~aw) >> sh) & 255u)) != 0u) {
+            } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    if (!((aw >> (sh + e)) & 1u)) v[e] = -INFINITY;
-                    if ((tw >> (sh + e)) & 1u) v[e] = patch_one(rv, v[e], i + e, tw);
+                    uint32_t bits = (e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16);
+                    if (masked) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
+                    f(i + e, __uint_as_float(bits), u * 8 + e);
                 }
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f(i + e, v[e]);
         }
-        for (uint32_t i = 8u * nv + t; i < V; i += WS_BLOCK) {
-            float v = fmaxf(bf16_to_f32(x[i]), -INFINITY);
-            const uint32_t tw = rv.touched ? rv.touched[i >> 5] : 0u;
-            if (rv.allow && !((rv.allow[i >> 5] >> (i & 31u)) & 1u)) v = -INFINITY;
-            if ((tw >> (i & 31u)) & 1u) v = patch_one(rv, v, i, tw);
-            f(i, v);
+        if (STASH) {
+            while (tslots) {  // about one token in a hundred: re-read from the lines the batch has just pulled in
+                const uint32_t slot = static_cast<uint32_t>(__ffs(tslots)) - 1u;
+                tslots &= tslots - 1u;
+                const uint32_t i = (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
+                stash[rank_of(rv, i)] = is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY;
+            }
+        }
+        end_batch(j0, 0u);
+        if (more) cur = nxt;
+    }
+    for (uint32_t i = nv * per + t; i < V; i += WS_BLOCK) {  // unaligned row or the last few tokens: one-token batches
+        const bool tch = is_touched(rv, i), ok = is_allowed(rv, i);
+        const float x = raw_logit(rv, i);
+        if (STASH && tch) stash[rank_of(rv, i)] = ok ? x : -INFINITY;
+        f(i, (tch || !ok) ? __uint_as_float(0xffffffffu) : x, 0);
+        end_batch(0xffffffffu, i);
+    }
+}
+
+template <bool STASH, class F, class E>
+__device__ __forceinline__ void stream_row(const RowView& rv, float* stash, F&& f, E&& end_batch) {
+    if (rv.allow || rv.touched) stream_row_impl<STASH, true>(rv, stash, f, end_batch);
+    else stream_row_impl<STASH, false>(rv, stash, f, end_batch);
+}
+
+// f(i, adjusted logit) for the touched tokens: thread t walks the set bits of its chunk of bitmap words
+template <class F>
+__device__ __forceinline__ void replay_touched(const RowView& rv, F&& f) {
+    if (!rv.touched) return;
+    const uint32_t nW = (rv.V + 31u) >> 5;
+    const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
+    const uint32_t w0 = threadIdx.x * chunk, w1 = min(w0 + chunk, nW);
+    for (uint32_t w = w0; w < w1; ++w) {
+        uint32_t bits = rv.touched[w];
+        uint32_t r = rv.wprefix[w];
+        while (bits) {
+            const uint32_t b = __ffs(bits) - 1u;
+            bits &= bits - 1u;
+            f((w << 5) + b, rv.pv[r++]);
         }
     }
 }
 
-// bin of an adjusted logit; also the pieces the histogram pass needs
+// Bin of a logit: t = fl((m - x) * c64), c64 = 64 * inv_t, clamped to the tail bin 4095 (NaN, -inf and everything whose
+// mass is below e^-64 of the top token's); bin = trunc(t). tlo is the exact residual of the product, so that
+// (bin + fract(t) + tlo) / 64 equals the exponent (double)(m - x) * inv_t of the host formula to the last bit.
 struct BinPos {
-    float bf;    // bin index as float, 4095 for the tail
-    float a;     // fl((m - x) * inv_t)
-    float alo;   // exact residual of that product
-    bool tail;
+    float tc;   // clamped t
+    float tlo;  // exact residual of (m - x) * c64 (garbage for the tail)
 };
-__device__ __forceinline__ BinPos bin_of(float m, float inv_t, float x) {
+__device__ __forceinline__ BinPos bin_pos(float m, float c64, float x) {
     BinPos r;
     const float d = __fsub_rn(m, x);
-    r.a = __fmul_rn(d, inv_t);
-    r.alo = __fmaf_rn(d, inv_t, -r.a);
-    const float t = r.a * 64.f;
-    r.tail = !(t < 4095.f);
-    r.bf = r.tail ? 4095.f : floorf(t);
+    const float t = __fmul_rn(d, c64);
+    r.tlo = __fmaf_rn(d, c64, -t);
+    r.tc = t < 4095.f ? t : 4095.f;
     return r;
 }
+__device__ __forceinline__ uint32_t bin_of(float m, float c64, float x) { return static_cast<uint32_t>(bin_pos(m, c64, x).tc); }
 
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
 // every element with key32 >= the result lies in a bin < bcut. 0xffffffff when no finite logit does.
-__device__ __forceinline__ uint32_t first_key_before_bin(float m, float inv_t, int bcut) {
+__device__ __forceinline__ uint32_t first_key_before_bin(float m, float c64, int bcut) {
     uint32_t lo = key32(-INFINITY), hi = key32(m);  // bin(lo) = tail, bin(hi) = 0
-    const float fc = static_cast<float>(bcut);
-    if (!(bin_of(m, inv_t, m).bf < fc)) return 0xffffffffu;
+    if (bcut <= 0) return 0xffffffffu;
+    const uint32_t bc = static_cast<uint32_t>(bcut);
     while (lo + 1u < hi) {  // invariant: bin(lo) >= bcut, bin(hi) < bcut
         const uint32_t mid = lo + ((hi - lo) >> 1);
-        if (bin_of(m, inv_t, unkey32(mid)).bf < fc) hi = mid;
+        if (bin_of(m, c64, unkey32(mid)) < bc) hi = mid;
         else lo = mid;
     }
     return hi;
@@ -233,7 +273,27 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
     }
 }
 
+// Debug builds (-DWS_PHASE_TIMERS) store the shader-clock time of each phase of every row into kept_logits.
+#ifdef WS_PHASE_TIMERS
+#define WS_MARK(k)                                                                                                   \
+    do {                                                                                                               \
+        __syncthreads();                                                                                               \
+        if (threadIdx.x == 0 && A.kept_logits) {                                                                       \
+            const long long now = clock64();                                                                           \
+            A.kept_logits[static_cast<size_t>(blockIdx.x) * A.kept_cap + (k)] = static_cast<float>(now - ws_t0);      \
+            ws_t0 = now;                                                                                               \
+        }                                                                                                              \
+    } while (0)
+#else
+#define WS_MARK(k) \
+    do {           \
+    } while (0)
+#endif
+
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
+#ifdef WS_PHASE_TIMERS
+    long long ws_t0 = clock64();
+#endif
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ float red_f[WS_WAVES];
     __shared__ uint32_t red_u[WS_WAVES];
@@ -255,6 +315,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     double* emass = reinterpret_cast<double*>(lds + 32768);
     uint32_t* touched = reinterpret_cast<uint32_t*>(lds + A.lds_ab);
     uint16_t* wprefix = reinterpret_cast<uint16_t*>(lds + A.lds_ab + nW * 4u);
+    float* pv = reinterpret_cast<float*>(lds + A.lds_ab + nW * 4u + ((nW * 2u + 15u) & ~15u));
 
     const float inv_t = A.inv_t[row];
     const uint32_t top_k = A.top_k ? A.top_k[row] : 0u;
@@ -272,12 +333,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     rv.allow = A.allow ? A.allow + static_cast<size_t>(row) * A.allow_stride : nullptr;
     rv.touched = nullptr;
     rv.wprefix = wprefix;
-    rv.patch = A.patch + static_cast<size_t>(row) * A.patch_cap;
-    rv.rep = A.rep ? A.rep[row] : 1.f;
+    rv.pv = pv;
 
     // ------------------------------------------------------------------ phase 0: penalties and bias
     const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? A.hist_off[row + 1] - h0 : 0u;
     const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
+    uint32_t n_touched = 0;  // tokens the streaming loop sends to the tail bin as NaN and replay_touched adds back
     if (!(inv_t > 0.f) || nh + nb > A.patch_cap) flags |= kBadParam;
     if (!(flags & kBadParam) && nh + nb > 0) {
         const int32_t* hist_ids = A.hist + h0;
@@ -310,52 +371,65 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) {
             cnt[r] = 0u;
             first[r] = 0xffffffffu;
+            pv[r] = 0.f;
         }
         __syncthreads();
-        auto rank_of = [&](uint32_t id) {
-            const uint32_t w = touched[id >> 5];
-            return static_cast<uint32_t>(wprefix[id >> 5]) + __popc(w & ((1u << (id & 31u)) - 1u));
-        };
+        rv.touched = touched;
         for (uint32_t j = t; j < nh; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
-            if (id < V) atomicAdd(&cnt[rank_of(id)], 1u);
+            if (id < V) atomicAdd(&cnt[rank_of(rv, id)], 1u);
         }
         for (uint32_t j = t; j < nb; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
             if (id < V) {
-                const uint32_t r = rank_of(id);
+                const uint32_t r = rank_of(rv, id);
                 atomicMin(&first[r], j);
                 atomicAdd(&cnt[r], 1u << 20);
             }
         }
         __syncthreads();
-        const float pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
-        float4* patch = A.patch + static_cast<size_t>(row) * A.patch_cap;
-        for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) {
-            const uint32_t c = cnt[r] & 0xfffffu, nbias = cnt[r] >> 20;
-            const float pen = c ? __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres) : 0.f;
-            patch[r] = make_float4(0.f, pen, __uint_as_float((c ? 1u : 0u) | (nbias ? 2u : 0u)), 0.f);
-        }
-        __syncthreads();
-        for (uint32_t j = t; j < nb; j += WS_BLOCK) {
+        for (uint32_t j = t; j < nb; j += WS_BLOCK) {  // bias sum of an id, by the thread of its first entry
             const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
             if (id >= V) continue;
-            const uint32_t r = rank_of(id);
+            const uint32_t r = rank_of(rv, id);
             if (first[r] != j) continue;
             float sum = bias_vals[j];
             if ((cnt[r] >> 20) > 1u)  // several entries for one id: add them in listed order
                 for (uint32_t j2 = j + 1; j2 < nb; ++j2)
                     if (static_cast<uint32_t>(bias_ids[j2]) == id) sum = __fadd_rn(sum, bias_vals[j2]);
-            patch[r].x = sum;
+            pv[r] = sum;
         }
         __syncthreads();
-        rv.touched = touched;
+        // per rank: bias sum -> first[r] (float bits; the first-entry bookkeeping is dead), cnt[r] stays. The raw logits
+        // of the touched tokens are stashed into pv[] by pass 1, straight from its stream.
+        for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) first[r] = __float_as_uint(pv[r]);
+        n_touched = n_uniq;
+        __syncthreads();
     }
 
+    WS_MARK(0);
     // ------------------------------------------------------------------ pass 1: maximum
     float m = -INFINITY;
     if (!(flags & kBadParam)) {
-        stream_row(rv, [&](uint32_t, float x) { m = fmaxf(m, x); });
+        stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+        if (n_touched) {
+            // adjusted logit of every touched token, once: (mask / NaN already applied) bias, repetition, frequency, presence
+            __syncthreads();
+            const uint32_t* cnt = reinterpret_cast<const uint32_t*>(lds);
+            const uint32_t* bsum = cnt + A.patch_cap;
+            const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
+            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+                const uint32_t c = cnt[r] & 0xfffffu;
+                float x = pv[r];
+                if (cnt[r] >> 20) x = __fadd_rn(x, __uint_as_float(bsum[r]));
+                if (c) {
+                    x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                    x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
+                }
+                pv[r] = x;
+                m = fmaxf(m, x);
+            }
+        }
         m = block_max(m, red_f);
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
@@ -374,18 +448,22 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         return;
     }
 
+    WS_MARK(1);
     // ------------------------------------------------------------------ pass 2: histogram of (count, mass)
     for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
     __syncthreads();
-    stream_row(rv, [&](uint32_t, float x) {
-        const BinPos p = bin_of(m, inv_t, x);
-        const float w = __fmaf_rn(p.bf, -0.015625f, p.a) + (p.alo + kEdgeShift);
-        const float g = w * (1.f - 0.5f * w * (1.f - (1.f / 3.f) * w * (1.f - 0.25f * w)));  // 1 - exp(-w), 0 <= w < 1/64
-        const uint32_t fx = p.tail ? 0u : static_cast<uint32_t>(g * kFixScale + 0.5f);
-        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<int>(p.bf)]), (1ull << kCountShift) | fx);
-    });
+    const float c64 = inv_t * 64.f;
+    auto add_to_hist = [&](uint32_t, float x, int) {
+        const BinPos p = bin_pos(m, c64, x);
+        const float w = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);  // in-bin offset, 0 < w < 1.001 (NaN: tail)
+        const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
+        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(p.tc)]), (1ull << kCountShift) | fx);
+    };
+    stream_row<false>(rv, nullptr, add_to_hist, [](uint32_t, uint32_t) {});
+    replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
     __syncthreads();
 
+    WS_MARK(2);
     // scan: thread t owns bins 4t .. 4t+3 (bin 0 = nearest the maximum)
     uint32_t c[4], cx[4];
     double ms[4], mx[4];
@@ -397,11 +475,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             const int b = 4 * t + j;
             const uint64_t h = hist[b];
             c[j] = static_cast<uint32_t>(h >> kCountShift);
+            if (b == kBins - 1) c[j] -= n_touched;  // streamed there as NaN, replayed into their own bins
             const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
-            // mass of the bin relative to the maximum: exp(-(b/64 - 2^-18)) * sum exp(-w); the tail bin carries none
-            ms[j] = (c[j] && b < kBins - 1) ? exp(-(static_cast<double>(b) * 0.015625 - static_cast<double>(kEdgeShift))) *
-                                                  (static_cast<double>(c[j]) - fix)
-                                            : 0.0;
+            // mass of the bin relative to the maximum: exp(-(b - 2^-12) / 64) * sum exp(-w / 64); the tail bin carries none
+            ms[j] = (c[j] && b < kBins - 1) ? kExpHi[b >> 6] * kExpLo[b & 63] * (static_cast<double>(c[j]) - fix) : 0.0;
             csum += c[j];
             msum += ms[j];
         }
@@ -587,24 +664,46 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         return;
     }
 
+    WS_MARK(3);
     // ------------------------------------------------------------------ pass 3: gather, sort, exact masses
     {
-        const float f0lo = static_cast<float>(r0lo), f0hi = static_cast<float>(r0hi);
-        const float f1lo = static_cast<float>(r1lo), f1hi = static_cast<float>(r1hi);
-        stream_row(rv, [&](uint32_t i, float x) {
-            const BinPos p = bin_of(m, inv_t, x);
-            if ((p.bf >= f0lo && p.bf <= f0hi) || (p.bf >= f1lo && p.bf <= f1hi)) {
-                const uint32_t slot = atomicAdd(&s_cnt, 1u);
-                if (slot < kCap) keys[slot] = key64(x, i);
-            }
+        const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = static_cast<uint32_t>(r0hi - r0lo);
+        const uint32_t u1 = static_cast<uint32_t>(r1lo), w1 = r1hi >= r1lo ? static_cast<uint32_t>(r1hi - r1lo) : 0u;
+        const bool two = r1hi >= r1lo;
+        auto push = [&](uint32_t i, float x) {
+            const uint32_t slot = atomicAdd(&s_cnt, 1u);
+            if (slot < kCap) keys[slot] = key64(x, i);
+        };
+        auto in_ranges = [&](float x) {
+            const uint32_t b = bin_of(m, c64, x);
+            return b - u0 <= w0 || (two && b - u1 <= w1);
+        };
+        // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens) are
+        // re-read after the batch, from the cache lines the batch has just pulled in
+        uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
+        const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+        stream_row<false>(
+            rv, nullptr, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
+            [&](uint32_t j0, uint32_t i_tail) {
+                while (hit) {
+                    const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
+                    hit &= hit - 1u;
+                    const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
+                    push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
+                }
+            });
+        replay_touched(rv, [&](uint32_t i, float x) {
+            if (in_ranges(x)) push(i, x);
         });
     }
     __syncthreads();
+    WS_MARK(4);
     uint32_t P = 64;
     while (P < n_list) P <<= 1;
     for (uint32_t i = n_list + t; i < P; i += WS_BLOCK) keys[i] = 0ull;
     __syncthreads();
     sort_desc(keys, P);
+    WS_MARK(5);
 
     // thread t owns sorted entries 4t .. 4t+3
     double e[4], inc[4], exc[4];
@@ -651,6 +750,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     }
 
+    WS_MARK(6);
     // ------------------------------------------------------------------ cuts
     double mg_top_p = 1.0, mg_min_p = 1.0, mg_draw = 1.0;
     // top-k: mass of the first n1 candidates (prefix mode)
@@ -739,10 +839,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         kept_key = s_key;
     } else if (has_r1 && n3 == c1base) {  // the cut falls on the upper edge of range 1: everything in earlier bins
         Zk = m1base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(m, inv_t, r1lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(m, c64, r1lo)) << 32;
     } else if (n3 == c0base && n_r0) {
         Zk = m0base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(m, inv_t, r0lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(m, c64, r0lo)) << 32;
     } else {  // no filter at all: the whole row
         Zk = Z;
         kept_key = 0ull;
@@ -791,6 +891,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (mg_min_p < tol) flags |= kNearMinP;
     if (mg_draw < tol) flags |= kNearDraw;
 
+    WS_MARK(7);
     if (t == 0) {
         A.token[row] = token;
         A.flags[row] = flags;
@@ -819,14 +920,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             float x = -INFINITY;
             uint32_t keep = 0, tl = 0;
             if (i < V) {
-                if (A.dtype == 0) x = static_cast<const float*>(rv.base)[i];
-                else x = bf16_to_f32(static_cast<const uint16_t*>(rv.base)[i]);
-                x = fmaxf(x, -INFINITY);
-                const uint32_t tw = rv.touched ? rv.touched[i >> 5] : 0u;
-                if (rv.allow && !((rv.allow[i >> 5] >> (i & 31u)) & 1u)) x = -INFINITY;
-                if ((tw >> (i & 31u)) & 1u) x = patch_one(rv, x, i, tw);
+                x = adjusted_logit(rv, i);
                 keep = key64(x, i) >= kept_key;
-                tl = tail_extra && !keep && bin_of(m, inv_t, x).tail;  // among zero-mass candidates the lowest ids
+                tl = tail_extra && !keep && bin_of(m, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
             }
             uint32_t tot;
             const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
