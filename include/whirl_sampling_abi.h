@@ -97,6 +97,17 @@ int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* i
 /* ---- (2) batched fused sampler ---------------------------------------------------------------------------- */
 
 enum { WS_DTYPE_F32 = 0, WS_DTYPE_BF16 = 1 };
+/* How ws_sample_batch sweeps a row. Both modes return the same tokens except where a decision sits within rounding of
+ * a boundary (reported in flags / margin).
+ *   EXACT: maximum first, then every probability mass from the host sampler's own formula exp((double)(x - max) * inv_t)
+ *          with the float subtraction it uses (src/sampling/sampler.cpp:31-32): three sweeps, the 2nd and 3rd from cache.
+ *   FUSED: one sweep from HBM; masses are binned against a provisional bound above the maximum, so the subtraction that
+ *          is rounded to float is (bound - x) instead of (max - x). Identical whenever those differences are exact in
+ *          float (logits that came from bf16, for instance); otherwise the prefix masses differ by ~1e-7 relative.
+ *          Needs 16-byte aligned rows of a multiple of 8 tokens, vocab <= 163840. A row whose maximum beats the bound
+ *          is redone the exact way inside the same launch.
+ *   AUTO:  FUSED where the batch qualifies, else EXACT. */
+enum { WS_MODE_AUTO = 0, WS_MODE_EXACT = 1, WS_MODE_FUSED = 2 };
 enum { WS_RNG_SPLITMIX = 0, WS_RNG_PHILOX = 1 };
 
 /* Per-row flag bits written to ws_batch.flags. */
@@ -159,6 +170,7 @@ typedef struct ws_batch {
     void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes */
     uint64_t workspace_bytes;
     double tol;             /* flag tolerance (0: 2^-40) */
+    int32_t mode;           /* WS_MODE_* */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

@@ -12,10 +12,13 @@ import gpu_cases as gc
 pytestmark = pytest.mark.gpu
 
 
-def run_case(c, rng_mode, rows=None, kept_cap=None, expect_near=0.05):
+MODES = [1, 0]  # WS_MODE_EXACT, WS_MODE_AUTO (the fused sweep wherever the batch qualifies)
+
+
+def run_case(c, rng_mode, rows=None, kept_cap=None, expect_near=0.05, mode=0):
     d = gc.upload(c)
     cap = c["V"] if kept_cap is None else kept_cap
-    smp = gc.sampler_for(c, d, rng_mode, kept_cap=cap).run()
+    smp = gc.sampler_for(c, d, rng_mode, kept_cap=cap, mode=mode).run()
     rows = range(c["rows"]) if rows is None else rows
     res = gc.compare_rows(c, smp, rows, rng_mode)
     assert res["exact"] >= (1 - expect_near) * res["rows"], res
@@ -23,13 +26,15 @@ def run_case(c, rng_mode, rows=None, kept_cap=None, expect_near=0.05):
 
 
 @pytest.mark.parametrize("rng_mode", [0, 1])
-def test_small_batch_all_features(rng_mode):
+@pytest.mark.parametrize("mode", MODES)
+def test_small_batch_all_features(rng_mode, mode):
     c = gc.make_cfg2(rows=24, V=32000, n_hist=512, n_bias=40)
-    res, _ = run_case(c, rng_mode)
+    res, _ = run_case(c, rng_mode, mode=mode)
     print(res)
 
 
-def test_small_vocab_ties_and_duplicated_bias():
+@pytest.mark.parametrize("mode", MODES)
+def test_small_vocab_ties_and_duplicated_bias(mode):
     """Logits rounded to one decimal (thousands of exact ties at every cut), bias lists with repeated ids, odd vocab
     (scalar tail after the 128-bit body)."""
     rng = np.random.default_rng(7)
@@ -38,11 +43,12 @@ def test_small_vocab_ties_and_duplicated_bias():
     c["bias_ids"][:, 1] = c["bias_ids"][:, 0]
     c["bias_ids"][:, 5] = c["bias_ids"][:, 0]
     c["top_k"] = rng.choice([0, 1, 5, 40, 700], 16).astype(np.uint32)
-    res, _ = run_case(c, 1, expect_near=0.3)
+    res, _ = run_case(c, 1, expect_near=0.3, mode=mode)
     print(res)
 
 
-def test_top_k_only_and_min_p_only_and_top_p_only():
+@pytest.mark.parametrize("mode", MODES)
+def test_top_k_only_and_min_p_only_and_top_p_only(mode):
     c = gc.make_cfg2(rows=12, V=20000, n_hist=100, n_bias=0)
     c["top_k"] = np.array([1, 2, 50, 1000] * 3, np.uint32)
     c["top_p"][:4] = 1.0
@@ -53,20 +59,22 @@ def test_top_k_only_and_min_p_only_and_top_p_only():
     c["top_k"][8:] = 0
     c["min_p"][8:] = 0.0
     c["top_p"][8:] = [0.5, 0.9, 0.99, 0.999]
-    res, _ = run_case(c, 1)
+    res, _ = run_case(c, 1, mode=mode)
     print(res)
 
 
-def test_bf16_rows():
+@pytest.mark.parametrize("mode", MODES)
+def test_bf16_rows(mode):
     c = gc.make_cfg3(rows=6, V=40000, n_hist=256)
-    res, _ = run_case(c, 1, expect_near=0.2)
+    res, _ = run_case(c, 1, expect_near=0.2, mode=mode)
     print(res)
 
 
-def test_masked_rows():
+@pytest.mark.parametrize("mode", MODES)
+def test_masked_rows(mode):
     c = gc.make_cfg5(rows=6, V=32768, n_hist=400, n_bias=30)
     c["top_k"][:] = [1000, 100, 0, 0, 5, 1]
-    res, _ = run_case(c, 1)
+    res, _ = run_case(c, 1, mode=mode)
     print(res)
 
 
@@ -107,29 +115,34 @@ def test_rows_are_independent_and_reproducible():
     assert np.array_equal(first[0::2], b.token.cpu().numpy()[0::2])
 
 
-def test_cfg1_shape():
-    res, _ = run_case(gc.make_cfg1(), 0)
+@pytest.mark.parametrize("mode", MODES)
+def test_cfg1_shape(mode):
+    res, _ = run_case(gc.make_cfg1(), 0, mode=mode)
     print(res)
 
 
-def test_cfg2_full_size():
-    res, _ = run_case(gc.make_cfg2(), 1)
+@pytest.mark.parametrize("mode", MODES)
+def test_cfg2_full_size(mode):
+    res, _ = run_case(gc.make_cfg2(), 1, mode=mode)
     print(res)
 
 
-def test_north_star_tile_full_size():
+@pytest.mark.parametrize("mode", MODES)
+def test_north_star_tile_full_size(mode):
     c = gc.make_tile()
-    res, _ = run_case(c, 1, rows=range(0, 256, 8), kept_cap=c["V"])
+    res, _ = run_case(c, 1, rows=range(0, 256, 8), kept_cap=c["V"], mode=mode)
     print(res)
 
 
-def test_cfg3_full_size():
+@pytest.mark.parametrize("mode", MODES)
+def test_cfg3_full_size(mode):
     c = gc.make_cfg3()
-    res, _ = run_case(c, 1, rows=range(0, 256, 16), expect_near=0.2)
+    res, _ = run_case(c, 1, rows=range(0, 256, 16), expect_near=0.2, mode=mode)
     print(res)
 
 
-def test_cfg5_shape_reduced_rows():
+@pytest.mark.parametrize("mode", MODES)
+def test_cfg5_shape_reduced_rows(mode):
     c = gc.make_cfg5(rows=32)
-    res, _ = run_case(c, 1, rows=range(0, 32, 4), kept_cap=2048)
+    res, _ = run_case(c, 1, rows=range(0, 32, 4), kept_cap=2048, mode=mode)
     print(res)

@@ -18,6 +18,7 @@ CO_PATH = os.path.join(HERE, "whirl_sampling_gfx950.co")
 
 DTYPE_F32, DTYPE_BF16 = 0, 1
 RNG_SPLITMIX, RNG_PHILOX = 0, 1
+MODE_AUTO, MODE_EXACT, MODE_FUSED = 0, 1, 2
 FLAG_NEAR_TOP_P, FLAG_NEAR_MIN_P, FLAG_NEAR_DRAW = 1, 2, 4
 FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN = 8, 16, 32, 64
 FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
@@ -49,7 +50,7 @@ class Batch(C.Structure):
                 ("token", C.c_void_p), ("prob", C.c_void_p), ("n_kept", C.c_void_p), ("flags", C.c_void_p),
                 ("stats", C.c_void_p), ("margin", C.c_void_p), ("kept_ids", C.c_void_p), ("kept_logits", C.c_void_p),
                 ("kept_cap", C.c_uint32),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double)]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32)]
 
 
 class SpecVerify(C.Structure):
@@ -198,7 +199,7 @@ class BatchSampler:
 
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
-                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True):
+                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -229,6 +230,7 @@ class BatchSampler:
         b.stats, b.margin = _p(self.stats), _p(self.margin)
         b.kept_ids, b.kept_logits, b.kept_cap = _p(self.kept_ids), _p(self.kept_logits), kept_cap
         b.tol = tol
+        b.mode = mode
         need = lib().ws_sample_batch_workspace(C.byref(b))
         self.workspace = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
         b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()

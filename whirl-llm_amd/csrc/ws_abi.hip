@@ -23,7 +23,9 @@ constexpr uint32_t kMaxLds = 160u * 1024u;  // LDS per workgroup on gfx950
 struct BatchPlan {
     uint32_t patch_cap;
     uint32_t lds_ab;
+    uint32_t lds_cnt;
     uint32_t lds_total;
+    bool fused;
     uint64_t workspace;
     int err;
 };
@@ -38,12 +40,31 @@ BatchPlan plan_batch(const ws_batch* b) {
     if (b->hist && !b->hist_off) return p;
     if (b->bias_ids && (!b->bias_off || !b->bias_vals)) return p;
     if (b->kept_ids && b->kept_cap == 0) return p;
+    if (b->mode != WS_MODE_AUTO && b->mode != WS_MODE_EXACT && b->mode != WS_MODE_FUSED) return p;
     const uint64_t cap = (b->hist ? uint64_t{b->max_hist} : 0) + (b->bias_ids ? uint64_t{b->max_bias} : 0);
     const uint32_t nW = (b->vocab + 31u) / 32u;
-    const uint64_t ab = cap * 8u > 65536u ? ((cap * 8u + 15u) & ~uint64_t{15}) : 65536u;
-    const uint64_t total = ab + uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15}) + cap * 4u;
+    const uint64_t maps = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15}) + ((cap * 4u + 15u) & ~uint64_t{15});
     p.err = WS_E_UNSUPPORTED;
-    if (cap > 65535u || total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
+    if (cap > 65535u) return p;
+    // fused sweep: rows of whole 128-bit vectors that fit the register cache, and LDS room for the per-rank counters
+    // next to the histogram (the exact path reuses the histogram's LDS for them)
+    const uint64_t esz = b->dtype == WS_DTYPE_F32 ? 4 : 2;
+    const bool vec_rows = b->vocab % 8u == 0 && (b->row_stride * esz) % 16u == 0 && reinterpret_cast<uintptr_t>(b->logits) % 16u == 0;
+    const uint64_t fused_total = 65536u + maps + cap * 8u;
+    const bool can_fuse = vec_rows && b->vocab <= 163840u && fused_total + 4096u <= kMaxLds;
+    if (b->mode == WS_MODE_FUSED && !can_fuse) return p;
+    p.fused = b->mode != WS_MODE_EXACT && can_fuse;
+    uint64_t ab, total;
+    if (p.fused) {
+        ab = 65536u;
+        total = fused_total;
+        p.lds_cnt = static_cast<uint32_t>(65536u + maps);
+    } else {
+        ab = cap * 8u > 65536u ? ((cap * 8u + 15u) & ~uint64_t{15}) : 65536u;
+        total = ab + maps;
+        p.lds_cnt = 0;
+    }
+    if (total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
@@ -188,14 +209,19 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.kept_cap = b->kept_cap;
     a.tol = b->tol > 0 ? b->tol : 1.0 / 1099511627776.0;
     a.lds_ab = p.lds_ab;
+    a.lds_cnt = p.lds_cnt;
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
     if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
         if (e != hipSuccess) return static_cast<int>(e);
         attr_set = true;
     }
-    hipLaunchKernelGGL(ws::sample_batch_kernel, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
+    if (p.fused) hipLaunchKernelGGL(ws::sample_batch_kernel<true>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
+    else hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
     return done();
 }
 

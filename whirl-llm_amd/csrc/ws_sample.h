@@ -71,7 +71,8 @@ struct BatchArgs {
     float* kept_logits;
     uint32_t kept_cap;
     double tol;
-    uint32_t lds_ab;  // bytes of the LDS region shared by the histogram / sort keys / masses / phase-0 counters
+    uint32_t lds_ab;   // bytes of the LDS region shared by the histogram / sort keys / masses
+    uint32_t lds_cnt;  // byte offset of the per-rank counters {history count | bias entries, bias sum}: 8 * patch_cap bytes
 };
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
@@ -230,10 +231,118 @@ __device__ __forceinline__ BinPos bin_pos(float m, float c64, float x) {
 }
 __device__ __forceinline__ uint32_t bin_of(float m, float c64, float x) { return static_cast<uint32_t>(bin_pos(m, c64, x).tc); }
 
+// ---- fused mode: one sweep over the row does the histogram against a provisional anchor, tracks the true maximum,
+// stashes the touched tokens and keeps every token's bin index in registers (two per VGPR), so that the gather of
+// the few bins the cuts land in needs no second sweep. 160 tokens per thread: rows of up to 163840 tokens.
+constexpr int kCacheRegs = 80;
+constexpr uint32_t kCacheTokens = 2u * kCacheRegs * WS_BLOCK;
+
+template <int PER, bool MASKED>
+__device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash, float anchor, float c64, uint64_t* hist,
+                                                uint32_t (&cache)[kCacheRegs], float& m) {
+    constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
+    const uint32_t t = threadIdx.x;
+    const uint32_t nv = rv.V / PER;
+    const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
+#pragma unroll
+    for (int bt = 0; bt < NB; ++bt) {
+        uint4 q[kBatch];
+        uint32_t na[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
+            const uint32_t jc = j < nv ? j : nv - 1u;
+            q[u] = xv[jc];
+            na[u] = (MASKED && rv.allow) ? ~rv.allow[(jc * PER) >> 5] : 0u;
+        }
+        uint32_t tslots = 0;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
+            constexpr int kPairs = PER / 2;
+            const int c0 = (bt * kBatch + u) * kPairs;
+            if (j < nv) {
+                const uint32_t i = j * PER;
+                const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
+                const int32_t bw = static_cast<int32_t>((na[u] | tw) >> (i & 31u));
+                tslots |= ((tw >> (i & 31u)) & (PER == 4 ? 15u : 255u)) << (u * PER);
+                const uint32_t w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+                uint32_t bins[PER];
+#pragma unroll
+                for (int e = 0; e < PER; ++e) {
+                    uint32_t bits = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
+                    const float x = __uint_as_float(bits);
+                    m = fmaxf(m, x);
+                    const BinPos p = bin_pos(anchor, c64, x);
+                    const float wf = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);
+                    const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(wf, __fmaf_rn(wf, __fmaf_rn(wf, kG2, kG1), kG0), 0.5f));
+                    bins[e] = static_cast<uint32_t>(p.tc);
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bins[e]]), (1ull << kCountShift) | fx);
+                }
+#pragma unroll
+                for (int k = 0; k < kPairs; ++k) cache[c0 + k] = bins[2 * k] | (bins[2 * k + 1] << 16);
+            } else {
+#pragma unroll
+                for (int k = 0; k < kPairs; ++k) cache[c0 + k] = 0x0fff0fffu;  // past the row: tail bin, never gathered
+            }
+        }
+        while (tslots) {  // touched tokens: raw logit to the stash, from the lines this batch has just pulled in
+            const uint32_t slot = static_cast<uint32_t>(__ffs(tslots)) - 1u;
+            tslots &= tslots - 1u;
+            const uint32_t i = ((bt * kBatch + slot / PER) * WS_BLOCK + t) * PER + (slot % PER);
+            stash[rank_of(rv, i)] = is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY;
+        }
+    }
+}
+
+__device__ __forceinline__ void fused_pass(const RowView& rv, float* stash, float anchor, float c64, uint64_t* hist,
+                                           uint32_t (&cache)[kCacheRegs], float& m) {
+    const bool masked = rv.allow || rv.touched;
+    if (rv.dtype == 0) {
+        if (masked) fused_pass_impl<4, true>(rv, stash, anchor, c64, hist, cache, m);
+        else fused_pass_impl<4, false>(rv, stash, anchor, c64, hist, cache, m);
+    } else {
+        if (masked) fused_pass_impl<8, true>(rv, stash, anchor, c64, hist, cache, m);
+        else fused_pass_impl<8, false>(rv, stash, anchor, c64, hist, cache, m);
+    }
+}
+
+// token index of half `half` of cache register k of thread t (the layout fused_pass_impl writes)
+__device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t half) {
+    const uint32_t per = dtype == 0 ? 4u : 8u, pairs = per / 2u;
+    return ((k / pairs) * WS_BLOCK + threadIdx.x) * per + 2u * (k % pairs) + half;
+}
+
+// push(i, logit) for every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1]
+template <class P>
+__device__ __forceinline__ void gather_from_cache(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0,
+                                                  uint32_t u1, uint32_t w1, P&& push) {
+    uint32_t hits[kCacheRegs / 16];
+#pragma unroll
+    for (int g = 0; g < kCacheRegs / 16; ++g) hits[g] = 0;
+#pragma unroll
+    for (int k = 0; k < kCacheRegs; ++k) {
+        const uint32_t lo = cache[k] & 0xffffu, hi = cache[k] >> 16;
+        const uint32_t h0 = (lo - u0 <= w0) | (lo - u1 <= w1), h1 = (hi - u0 <= w0) | (hi - u1 <= w1);
+        hits[k / 16] |= (h0 | (h1 << 1)) << (2 * (k % 16));
+    }
+#pragma unroll
+    for (int g = 0; g < kCacheRegs / 16; ++g) {
+        uint32_t h = hits[g];
+        while (h) {
+            const uint32_t bit = static_cast<uint32_t>(__ffs(h)) - 1u;
+            h &= h - 1u;
+            const uint32_t i = cache_token(rv.dtype, g * 16u + (bit >> 1), bit & 1u);
+            push(i, raw_logit(rv, i));  // neither masked nor touched (those sit in the tail bin): the raw logit is the logit
+        }
+    }
+}
+
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
 // every element with key32 >= the result lies in a bin < bcut. 0xffffffff when no finite logit does.
 __device__ __forceinline__ uint32_t first_key_before_bin(float m, float c64, int bcut) {
-    uint32_t lo = key32(-INFINITY), hi = key32(m);  // bin(lo) = tail, bin(hi) = 0
+    uint32_t lo = key32(-INFINITY), hi = key32(m);  // bin(lo) = tail, bin(hi) = 0 (m = the value bins are measured from)
     if (bcut <= 0) return 0xffffffffu;
     const uint32_t bc = static_cast<uint32_t>(bcut);
     while (lo + 1u < hi) {  // invariant: bin(lo) >= bcut, bin(hi) < bcut
@@ -290,6 +399,7 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
     } while (0)
 #endif
 
+template <bool FUSED>
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #ifdef WS_PHASE_TIMERS
     long long ws_t0 = clock64();
@@ -366,7 +476,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             wprefix[w] = static_cast<uint16_t>(run);
             run += __popc(touched[w]);
         }
-        uint32_t* cnt = reinterpret_cast<uint32_t*>(lds);  // low 20 bits: history count, high 12: bias entries
+        uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);  // low 20 bits: history count, high 12: bias entries
         uint32_t* first = cnt + A.patch_cap;               // index of the id's first bias entry
         for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) {
             cnt[r] = 0u;
@@ -408,28 +518,71 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     WS_MARK(0);
-    // ------------------------------------------------------------------ pass 1: maximum
-    float m = -INFINITY;
-    if (!(flags & kBadParam)) {
-        stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
-        if (n_touched) {
-            // adjusted logit of every touched token, once: (mask / NaN already applied) bias, repetition, frequency, presence
-            __syncthreads();
-            const uint32_t* cnt = reinterpret_cast<const uint32_t*>(lds);
-            const uint32_t* bsum = cnt + A.patch_cap;
-            const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
-            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
-                const uint32_t c = cnt[r] & 0xfffffu;
-                float x = pv[r];
-                if (cnt[r] >> 20) x = __fadd_rn(x, __uint_as_float(bsum[r]));
-                if (c) {
-                    x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
-                    x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
-                }
-                pv[r] = x;
-                m = fmaxf(m, x);
+    const float c64 = inv_t * 64.f;
+    auto adjust_touched = [&](float& mref) {
+        // adjusted logit of every touched token, once: (mask / NaN already applied) bias, repetition, frequency, presence
+        if (!n_touched) return;
+        __syncthreads();
+        const uint32_t* cnt = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt);
+        const uint32_t* bsum = cnt + A.patch_cap;
+        const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
+        for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+            const uint32_t c = cnt[r] & 0xfffffu;
+            float x = pv[r];
+            if (cnt[r] >> 20) x = __fadd_rn(x, __uint_as_float(bsum[r]));
+            if (c) {
+                x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
             }
+            pv[r] = x;
+            mref = fmaxf(mref, x);
         }
+    };
+    float anchor = 0.f;  // bins are measured down from here: the row maximum, or a provisional bound above it
+    auto add_to_hist = [&](uint32_t, float x, int) {
+        const BinPos p = bin_pos(anchor, c64, x);
+        const float w = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);  // in-bin offset, 0 < w < 1.001 (NaN: tail)
+        const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
+        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(p.tc)]), (1ull << kCountShift) | fx);
+    };
+    float m = -INFINITY;
+    bool cached = false;
+    uint32_t cache[kCacheRegs];  // dead code (and no registers) in the exact instantiation
+    if (FUSED && !(flags & kBadParam)) {
+        // ---------------------------------------------------------------- fused sweep: anchor, histogram, max, stash, bins
+        // anchor = the maximum of the first 4096 vectors of the row (raw logits) + 8 exponent units of headroom
+        {
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u, nv = V / per;
+            float s = -INFINITY;
+            for (uint32_t j = t; j < nv && j < kBatch * WS_BLOCK; j += WS_BLOCK) {
+                const uint4 q = static_cast<const uint4*>(rv.base)[j];
+                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (rv.dtype == 0) s = fmaxf(s, __uint_as_float(w[e]));
+                    else s = fmaxf(s, fmaxf(__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)));
+                }
+            }
+            for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+            s = block_max(s, red_f);
+            anchor = s + 8.f / inv_t;
+        }
+        if (anchor > -INFINITY && anchor < INFINITY) {
+            if constexpr (FUSED) fused_pass(rv, pv, anchor, c64, hist, cache, m);
+            adjust_touched(m);
+            m = block_max(m, red_f);
+            // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
+            cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
+        } else {
+            stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+            adjust_touched(m);
+            m = block_max(m, red_f);
+        }
+        if (!(m > -INFINITY)) flags |= kAllMasked;
+    } else if (!(flags & kBadParam)) {
+        // ---------------------------------------------------------------- pass 1: maximum (and the stash of touched tokens)
+        stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+        adjust_touched(m);
         m = block_max(m, red_f);
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
@@ -449,19 +602,21 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     WS_MARK(1);
-    // ------------------------------------------------------------------ pass 2: histogram of (count, mass)
-    for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+    if (cached) {
+        replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
+    } else {
+        // ---------------------------------------------------------------- pass 2: histogram of (count, mass) below the maximum
+        anchor = m;
+        __syncthreads();
+        for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+        __syncthreads();
+        stream_row<false>(rv, nullptr, add_to_hist, [](uint32_t, uint32_t) {});
+        replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
+    }
     __syncthreads();
-    const float c64 = inv_t * 64.f;
-    auto add_to_hist = [&](uint32_t, float x, int) {
-        const BinPos p = bin_pos(m, c64, x);
-        const float w = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);  // in-bin offset, 0 < w < 1.001 (NaN: tail)
-        const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
-        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(p.tc)]), (1ull << kCountShift) | fx);
-    };
-    stream_row<false>(rv, nullptr, add_to_hist, [](uint32_t, uint32_t) {});
-    replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
-    __syncthreads();
+    // masses are accumulated relative to the anchor; everything below works relative to the maximum
+    const double lift = (static_cast<double>(anchor) - static_cast<double>(m)) * static_cast<double>(inv_t);  // >= 0
+    const double to_max = exp(lift);
 
     WS_MARK(2);
     // scan: thread t owns bins 4t .. 4t+3 (bin 0 = nearest the maximum)
@@ -478,7 +633,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (b == kBins - 1) c[j] -= n_touched;  // streamed there as NaN, replayed into their own bins
             const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
             // mass of the bin relative to the maximum: exp(-(b - 2^-12) / 64) * sum exp(-w / 64); the tail bin carries none
-            ms[j] = (c[j] && b < kBins - 1) ? kExpHi[b >> 6] * kExpLo[b & 63] * (static_cast<double>(c[j]) - fix) : 0.0;
+            ms[j] = (c[j] && b < kBins - 1) ? kExpHi[b >> 6] * kExpLo[b & 63] * (static_cast<double>(c[j]) - fix) * to_max : 0.0;
             csum += c[j];
             msum += ms[j];
         }
@@ -579,8 +734,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         }
         if (use_min_p) {
-            const double astar = -log(min_p) * 64.0;
-            const double lo = floor(astar - 1e-3), hi = floor(astar + 1e-3);
+            const double astar = (-log(min_p) + lift) * 64.0;  // the floor in bin coordinates (bins count from the anchor)
+            const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
             lo3 = lo < 0 ? 0 : (lo > kBins - 1 ? kBins - 1 : static_cast<int>(lo));
             hi3 = hi < 0 ? 0 : (hi > kBins - 1 ? kBins - 1 : static_cast<int>(hi));
         }
@@ -674,24 +829,29 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             const uint32_t slot = atomicAdd(&s_cnt, 1u);
             if (slot < kCap) keys[slot] = key64(x, i);
         };
+        const uint32_t u1r = two ? u1 : 0xffff0000u;  // an empty second range matches no bin
         auto in_ranges = [&](float x) {
-            const uint32_t b = bin_of(m, c64, x);
-            return b - u0 <= w0 || (two && b - u1 <= w1);
+            const uint32_t b = bin_of(anchor, c64, x);
+            return b - u0 <= w0 || b - u1r <= w1;
         };
-        // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens) are
-        // re-read after the batch, from the cache lines the batch has just pulled in
-        uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
-        const uint32_t per = rv.dtype == 0 ? 4u : 8u;
-        stream_row<false>(
-            rv, nullptr, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
-            [&](uint32_t j0, uint32_t i_tail) {
-                while (hit) {
-                    const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
-                    hit &= hit - 1u;
-                    const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
-                    push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
-                }
-            });
+        if (FUSED && cached) {
+            if constexpr (FUSED) gather_from_cache(rv, cache, u0, w0, u1r, w1, push);
+        } else {
+            // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
+            // are re-read after the batch, from the cache lines the batch has just pulled in
+            uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+            stream_row<false>(
+                rv, nullptr, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
+                [&](uint32_t j0, uint32_t i_tail) {
+                    while (hit) {
+                        const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
+                        hit &= hit - 1u;
+                        const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
+                        push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
+                    }
+                });
+        }
         replay_touched(rv, [&](uint32_t i, float x) {
             if (in_ranges(x)) push(i, x);
         });
@@ -839,10 +999,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         kept_key = s_key;
     } else if (has_r1 && n3 == c1base) {  // the cut falls on the upper edge of range 1: everything in earlier bins
         Zk = m1base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(m, c64, r1lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(anchor, c64, r1lo)) << 32;
     } else if (n3 == c0base && n_r0) {
         Zk = m0base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(m, c64, r0lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(anchor, c64, r0lo)) << 32;
     } else {  // no filter at all: the whole row
         Zk = Z;
         kept_key = 0ull;
@@ -922,7 +1082,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (i < V) {
                 x = adjusted_logit(rv, i);
                 keep = key64(x, i) >= kept_key;
-                tl = tail_extra && !keep && bin_of(m, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
+                tl = tail_extra && !keep && bin_of(anchor, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
             }
             uint32_t tot;
             const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
