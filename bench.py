@@ -24,6 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+MODE = 0
 
 
 def algorithmic_bytes(c):
@@ -42,7 +43,7 @@ def time_gpu(c, steps, warmup, rng_mode=1):
     import torch
     import gpu_cases as gc
     d = gc.upload(c)
-    smp = gc.sampler_for(c, d, rng_mode)
+    smp = gc.sampler_for(c, d, rng_mode, mode=MODE)
     for _ in range(warmup):
         smp.run()
     torch.cuda.synchronize()
@@ -126,6 +127,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-also", action="store_true")
     ap.add_argument("--check-rows", type=int, default=8)
+    ap.add_argument("--mode", default="auto", choices=["auto", "exact", "fused"], help="ws_batch.mode for every workload")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run 10 device copies of 256 MiB instead (known traffic: 256 MiB read + 256 MiB written per "
+                         "copy) to scale rocprofv3's FETCH_SIZE / WRITE_SIZE")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU; rows are independent, so more GPUs mean more row shards with no "
@@ -135,6 +140,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if a.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "10 copies", "bytes_read_per_copy": 256 << 20, "bytes_written_per_copy": 256 << 20}))
+        return
+    global MODE
+    MODE = {"auto": 0, "exact": 1, "fused": 2}[a.mode]
     c, main_res = run_workload(a.workload, a.steps, a.warmup, a.check_rows)
     also = []
     if not a.no_also:
@@ -151,7 +166,8 @@ def main():
         "dtype": "f32" if c["dtype"] == "f32" else "bf16->f32", "data": "synthetic",
         "config": {"workload": a.workload, "rows": c["rows"], "vocab": c["V"], "logits": c["dtype"],
                    "history_ids_per_row": 0 if c["hist"] is None else int(c["hist"].shape[1]),
-                   "filters": "see tests/gpu_cases.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2},
+                   "filters": "see tests/gpu_cases.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
+                   "sweep_mode": a.mode},
         "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["frac_of_hbm_peak"], "traffic": None, "kernel": "ws::sample_batch_kernel",
                      "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},

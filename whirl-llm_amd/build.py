@@ -11,6 +11,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "csrc", "ws_abi.hip")
+SRC_FUSED = os.path.join(HERE, "csrc", "ws_fused.hip")
 # packed FP32 instructions are switched off for every device compile of this repository
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -28,7 +29,7 @@ def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     so = os.path.join(HERE, "libwhirl_sampling_hip.so")
     co = os.path.join(HERE, "whirl_sampling_gfx950.co")
-    run([hipcc, *FLAGS, "-fPIC", "-shared", "-o", so, SRC])
+    run([hipcc, *FLAGS, "-fPIC", "-shared", "-o", so, SRC, SRC_FUSED])
     run([hipcc, *FLAGS, "--genco", "-o", co, SRC])
     if verbose:
         print("built", so, "and", co)

@@ -13,6 +13,11 @@
 #include "ws_spec.h"
 #include "ws_topk.h"
 
+namespace ws {
+// ws_fused.hip: the fused-sweep kernel, built for 512-thread workgroups
+int launch_fused(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
+}  // namespace ws
+
 namespace {
 
 inline hipStream_t S(void* s) { return static_cast<hipStream_t>(s); }
@@ -210,18 +215,15 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.tol = b->tol > 0 ? b->tol : 1.0 / 1099511627776.0;
     a.lds_ab = p.lds_ab;
     a.lds_cnt = p.lds_cnt;
+    if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
         if (e != hipSuccess) return static_cast<int>(e);
         attr_set = true;
     }
-    if (p.fused) hipLaunchKernelGGL(ws::sample_batch_kernel<true>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
-    else hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
+    hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
     return done();
 }
 

@@ -1,11 +1,13 @@
 // Device helpers shared by the gfx950 sampling kernels: wave64 / block reductions and scans, order-preserving
-// float keys, vectorised row iteration. One workgroup = WS_BLOCK threads = 16 wave64 waves.
+// float keys, vectorised row iteration. One workgroup = WS_BLOCK threads of wave64 waves.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#define WS_BLOCK 1024
+#ifndef WS_BLOCK
+#define WS_BLOCK 1024  // threads per workgroup; the fused sweep is compiled with 512 (256 registers per thread)
+#endif
 #define WS_WAVES (WS_BLOCK / 64)
 
 namespace ws {

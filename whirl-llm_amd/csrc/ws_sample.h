@@ -28,6 +28,7 @@ namespace ws {
 
 constexpr int kBins = 4096;
 constexpr uint32_t kCap = 4096;          // candidates resolved exactly in LDS per gather
+constexpr int kPT = kBins / WS_BLOCK;    // histogram bins, and sorted candidates, owned by one thread
 constexpr int kCountShift = 44;          // histogram word: count << 44 | fixed-point sum of (1 - exp(-w))
 constexpr float kFixScale = 1073741824.f;  // 2^30
 constexpr double kFixInv = 1.0 / 1073741824.0;
@@ -233,29 +234,35 @@ __device__ __forceinline__ uint32_t bin_of(float m, float c64, float x) { return
 
 // ---- fused mode: one sweep over the row does the histogram against a provisional anchor, tracks the true maximum,
 // stashes the touched tokens and keeps every token's bin index in registers (two per VGPR), so that the gather of
-// the few bins the cuts land in needs no second sweep. 160 tokens per thread: rows of up to 163840 tokens.
-constexpr int kCacheRegs = 80;
-constexpr uint32_t kCacheTokens = 2u * kCacheRegs * WS_BLOCK;
+// the few bins the cuts land in needs no second sweep. Rows of up to 163840 tokens.
+constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 with 512
 
 template <int PER, bool MASKED>
 __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash, float anchor, float c64, uint64_t* hist,
                                                 uint32_t (&cache)[kCacheRegs], float& m) {
     constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
+    constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
     const uint32_t nv = rv.V / PER;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
-#pragma unroll
-    for (int bt = 0; bt < NB; ++bt) {
-        uint4 q[kBatch];
-        uint32_t na[kBatch];
+    uint4 q[kRing][kBatch];
+    uint32_t na[kRing][kBatch];
+    auto load = [&](int bt, int slot) {
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;
-            q[u] = xv[jc];
-            na[u] = (MASKED && rv.allow) ? ~rv.allow[(jc * PER) >> 5] : 0u;
+            q[slot][u] = xv[jc];
+            na[slot][u] = (MASKED && rv.allow) ? ~rv.allow[(jc * PER) >> 5] : 0u;
         }
-        uint32_t tslots = 0;
+    };
+    load(0, 0);
+    if (NB > 1) load(1, 1);
+#pragma unroll
+    for (int bt = 0; bt < NB; ++bt) {
+        const int slot = bt % kRing;
+        if (bt + 2 < NB) load(bt + 2, (bt + 2) % kRing);
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the work on this batch
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
@@ -264,13 +271,13 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             if (j < nv) {
                 const uint32_t i = j * PER;
                 const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
-                const int32_t bw = static_cast<int32_t>((na[u] | tw) >> (i & 31u));
-                tslots |= ((tw >> (i & 31u)) & (PER == 4 ? 15u : 255u)) << (u * PER);
-                const uint32_t w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
-                uint32_t bins[PER];
+                const int32_t bw = static_cast<int32_t>((na[slot][u] | tw) >> (i & 31u));
+                const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
+                uint32_t bins[PER], raw[PER];
 #pragma unroll
                 for (int e = 0; e < PER; ++e) {
-                    uint32_t bits = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+                    raw[e] = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
+                    uint32_t bits = raw[e];
                     if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     const float x = __uint_as_float(bits);
                     m = fmaxf(m, x);
@@ -282,16 +289,25 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
                 }
 #pragma unroll
                 for (int k = 0; k < kPairs; ++k) cache[c0 + k] = bins[2 * k] | (bins[2 * k + 1] << 16);
+                if (MASKED) {
+                    // touched tokens of this vector (one vector in twenty has one): raw logit -> stash[rank], straight
+                    // from the registers; the select chain runs for every lane, only the store is predicated
+                    uint32_t tb = (tw >> (i & 31u)) & (PER == 4 ? 15u : 255u);
+                    uint32_t r = static_cast<uint32_t>(rv.wprefix[i >> 5]) + __popc(tw & ((1u << (i & 31u)) - 1u));
+                    const uint32_t nab = na[slot][u] >> (i & 31u);
+                    while (tb) {
+                        const uint32_t e0 = static_cast<uint32_t>(__ffs(tb)) - 1u;
+                        tb &= tb - 1u;
+                        uint32_t v = raw[0];
+#pragma unroll
+                        for (int e = 1; e < PER; ++e) v = e0 == static_cast<uint32_t>(e) ? raw[e] : v;
+                        stash[r++] = ((nab >> e0) & 1u) ? -INFINITY : fmaxf(__uint_as_float(v), -INFINITY);
+                    }
+                }
             } else {
 #pragma unroll
                 for (int k = 0; k < kPairs; ++k) cache[c0 + k] = 0x0fff0fffu;  // past the row: tail bin, never gathered
             }
-        }
-        while (tslots) {  // touched tokens: raw logit to the stash, from the lines this batch has just pulled in
-            const uint32_t slot = static_cast<uint32_t>(__ffs(tslots)) - 1u;
-            tslots &= tslots - 1u;
-            const uint32_t i = ((bt * kBatch + slot / PER) * WS_BLOCK + t) * PER + (slot % PER);
-            stash[rank_of(rv, i)] = is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY;
         }
     }
 }
@@ -314,18 +330,27 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
     return ((k / pairs) * WS_BLOCK + threadIdx.x) * per + 2u * (k % pairs) + half;
 }
 
-// push(i, logit) for every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1]
-template <class P>
-__device__ __forceinline__ void gather_from_cache(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0,
-                                                  uint32_t u1, uint32_t w1, P&& push) {
+// Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range): its index goes
+// to list[] (LDS, count in *n_list; entries past cap are dropped but counted). Both 16-bit halves of a register are
+// tested at once: with bit 15 of each half forced on, (y - lo) and (y - hi - 1) differ in bit 15 exactly for
+// lo <= bin <= hi. Hits are shifted into one mask per 16 registers; tokens are pushed after the scan.
+__device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
+                                                  uint32_t w1, uint32_t* list, uint32_t* n_list, uint32_t cap) {
+    const bool two = u1 <= 0x7fffu;
+    const uint32_t L0 = u0 * 0x10001u, H0 = (u0 + w0 + 1u) * 0x10001u;
+    const uint32_t L1 = two ? u1 * 0x10001u : 0u, H1 = two ? (u1 + w1 + 1u) * 0x10001u : 0u;
     uint32_t hits[kCacheRegs / 16];
 #pragma unroll
-    for (int g = 0; g < kCacheRegs / 16; ++g) hits[g] = 0;
+    for (int g = 0; g < kCacheRegs / 16; ++g) {
+        uint32_t acc = 0;
 #pragma unroll
-    for (int k = 0; k < kCacheRegs; ++k) {
-        const uint32_t lo = cache[k] & 0xffffu, hi = cache[k] >> 16;
-        const uint32_t h0 = (lo - u0 <= w0) | (lo - u1 <= w1), h1 = (hi - u0 <= w0) | (hi - u1 <= w1);
-        hits[k / 16] |= (h0 | (h1 << 1)) << (2 * (k % 16));
+        for (int k = 0; k < 16; ++k) {
+            const uint32_t y = cache[g * 16 + k] | 0x80008000u;
+            uint32_t r = (y - L0) ^ (y - H0);
+            if (two) r |= (y - L1) ^ (y - H1);
+            acc = (acc >> 1) | (r & 0x80008000u);  // register k: low half -> bit k, high half -> bit 16 + k
+        }
+        hits[g] = acc;
     }
 #pragma unroll
     for (int g = 0; g < kCacheRegs / 16; ++g) {
@@ -333,8 +358,8 @@ __device__ __forceinline__ void gather_from_cache(const RowView& rv, const uint3
         while (h) {
             const uint32_t bit = static_cast<uint32_t>(__ffs(h)) - 1u;
             h &= h - 1u;
-            const uint32_t i = cache_token(rv.dtype, g * 16u + (bit >> 1), bit & 1u);
-            push(i, raw_logit(rv, i));  // neither masked nor touched (those sit in the tail bin): the raw logit is the logit
+            const uint32_t slot = atomicAdd(n_list, 1u);
+            if (slot < cap) list[slot] = cache_token(dtype, g * 16u + (bit & 15u), bit >> 4);
         }
     }
 }
@@ -619,15 +644,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double to_max = exp(lift);
 
     WS_MARK(2);
-    // scan: thread t owns bins 4t .. 4t+3 (bin 0 = nearest the maximum)
-    uint32_t c[4], cx[4];
-    double ms[4], mx[4];
+    // scan: thread t owns kPT consecutive bins (bin 0 = nearest the anchor)
+    uint32_t c[kPT], cx[kPT];
+    double ms[kPT], mx[kPT];
     {
         uint32_t csum = 0;
         double msum = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int b = 4 * t + j;
+        for (int j = 0; j < kPT; ++j) {
+            const int b = kPT * t + j;
             const uint64_t h = hist[b];
             c[j] = static_cast<uint32_t>(h >> kCountShift);
             if (b == kBins - 1) c[j] -= n_touched;  // streamed there as NaN, replayed into their own bins
@@ -642,7 +667,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint32_t cb = block_excl_scan(csum, red_u, &ctot);
         double mb = block_excl_scan(msum, red_d, &mtot);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kPT; ++j) {
             cx[j] = cb;
             mx[j] = mb;
             cb += c[j];
@@ -657,20 +682,20 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // lookups in the scanned histogram; every call site is reached by the whole block
     auto find_count = [&](uint32_t n, int slot) {  // bin holding the element of rank n - 1
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (cx[j] < n && cx[j] + c[j] >= n) sel[slot] = BinSel{static_cast<int>(4 * t + j), cx[j], c[j], mx[j], ms[j]};
+        for (int j = 0; j < kPT; ++j)
+            if (cx[j] < n && cx[j] + c[j] >= n) sel[slot] = BinSel{static_cast<int>(kPT * t + j), cx[j], c[j], mx[j], ms[j]};
     };
     auto find_mass = [&](double X, bool strict, int slot) {  // first bin whose inclusive mass prefix reaches X
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kPT; ++j) {
             const double inc = mx[j] + ms[j];
             const bool hit = strict ? (inc > X && !(mx[j] > X)) : (inc >= X && !(mx[j] >= X));
-            if (hit && ms[j] > 0.0) sel[slot] = BinSel{static_cast<int>(4 * t + j), cx[j], c[j], mx[j], ms[j]};
+            if (hit && ms[j] > 0.0) sel[slot] = BinSel{static_cast<int>(kPT * t + j), cx[j], c[j], mx[j], ms[j]};
         }
     };
     auto fetch_bin = [&](int b, int slot) {
-        if (b >= 0 && static_cast<uint32_t>(b >> 2) == t) {
-            const int j = b & 3;
+        if (b >= 0 && static_cast<uint32_t>(b / kPT) == t) {
+            const int j = b % kPT;
             sel[slot] = BinSel{b, cx[j], c[j], mx[j], ms[j]};
         }
     };
@@ -835,7 +860,21 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             return b - u0 <= w0 || b - u1r <= w1;
         };
         if (FUSED && cached) {
-            if constexpr (FUSED) gather_from_cache(rv, cache, u0, w0, u1r, w1, push);
+            if constexpr (FUSED) {
+                // token indices first (no loads in the scan), then one parallel round of loads for the keys
+                uint32_t* list = reinterpret_cast<uint32_t*>(emass);
+                if (t == 0) s_u[4] = 0;
+                __syncthreads();
+                gather_from_cache(rv.dtype, cache, u0, w0, u1r, w1, list, &s_u[4], kCap);
+                __syncthreads();
+                const uint32_t n_hit = min(s_u[4], kCap);
+                for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
+                    const uint32_t i = list[k];
+                    keys[k] = key64(raw_logit(rv, i), i);  // neither masked nor touched (those sit in the tail bin)
+                }
+                if (t == 0) s_cnt = s_u[4];
+                __syncthreads();
+            }
         } else {
             // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
             // are re-read after the batch, from the cache lines the batch has just pulled in
@@ -865,15 +904,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     sort_desc(keys, P);
     WS_MARK(5);
 
-    // thread t owns sorted entries 4t .. 4t+3
-    double e[4], inc[4], exc[4];
-    uint32_t pos[4];
-    bool live[4];
+    // thread t owns kPT consecutive sorted entries
+    double e[kPT], inc[kPT], exc[kPT];
+    uint32_t pos[kPT];
+    bool live[kPT];
     {
         double esum = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t i = 4 * t + j;
+        for (int j = 0; j < kPT; ++j) {
+            const uint32_t i = kPT * t + j;
             live[j] = i < n_list;
             e[j] = 0;
             if (live[j]) {
@@ -887,17 +926,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         double run = block_excl_scan(esum, red_d, &etot);
         // masses of range 1 restart at its base: subtract the running sum at the end of range 0
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kPT; ++j) {
             exc[j] = run;
             run += e[j];
             inc[j] = run;
-            if (4 * t + j + 1 == n_r0) s_d[1] = run;
+            if (kPT * t + j + 1 == n_r0) s_d[1] = run;
         }
         __syncthreads();
         const double at_r0_end = n_r0 ? s_d[1] : 0.0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t i = 4 * t + j;
+        for (int j = 0; j < kPT; ++j) {
+            const uint32_t i = kPT * t + j;
             if (i < n_r0) {
                 pos[j] = c0base + i;
                 exc[j] += m0base;
@@ -917,7 +956,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     double M1 = Z;
     if (prefix_mode) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kPT; ++j)
             if (live[j] && pos[j] == n1 - 1) s_d[2] = inc[j];
         __syncthreads();
         M1 = s_d[2];
@@ -931,7 +970,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kPT; ++j)
             if (live[j] && pos[j] < n1 && inc[j] >= X && !(exc[j] >= X) && e[j] > 0.0) {
                 s_u[0] = pos[j] + 1;
                 s_d[3] = fmin(inc[j] - X, pos[j] > 0 ? X - exc[j] : X) / X;
@@ -951,7 +990,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint32_t ok = 0;
         double near = 1.0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kPT; ++j)
             if (live[j]) {
                 ok += e[j] >= min_p;
                 near = fmin(near, fabs(e[j] - min_p) / min_p);
@@ -985,10 +1024,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (t == 0) s_u[1] = 0;
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kPT; ++j)
         if (live[j] && pos[j] == n3 - 1) {
             s_d[4] = inc[j];
-            s_key = keys[4 * t + j];
+            s_key = keys[kPT * t + j];
             s_u[1] = 1;
         }
     __syncthreads();
@@ -1017,15 +1056,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kPT; ++j) {
         if (!live[j] || pos[j] >= n3) continue;
         if (inc[j] > target && !(exc[j] > target) && e[j] > 0.0) {
-            s_u[2] = 0xffffffffu - static_cast<uint32_t>(keys[4 * t + j]);
+            s_u[2] = 0xffffffffu - static_cast<uint32_t>(keys[kPT * t + j]);
             s_d[5] = e[j];
             s_d[6] = fmin(inc[j] - target, pos[j] > 0 ? target - exc[j] : 1e300) / Zk;
         }
         if (pos[j] == n3 - 1) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
-            s_u[3] = 0xffffffffu - static_cast<uint32_t>(keys[4 * t + j]);
+            s_u[3] = 0xffffffffu - static_cast<uint32_t>(keys[kPT * t + j]);
             s_d[7] = e[j];
         }
     }
