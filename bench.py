@@ -25,6 +25,9 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 MODE = 0
+# HBM bytes per launch of ws::sample_batch_kernel on the tile workload: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
+# what the same counter reads for a 256 MiB device copy (x2.000 and x1.000); the runs are summarised under profiles/
+TRAFFIC_BYTES = {("tile", "auto"): 168.6e6, ("tile", "fused"): 168.6e6, ("tile", "exact"): 491.1e6}
 
 
 def algorithmic_bytes(c):
@@ -71,9 +74,10 @@ def parity_sample(c, smp, n_check, rng_mode=1):
     return res
 
 
-def cpu_baseline(c, budget_s=12.0, max_rows=64):
+def cpu_baseline(c, budget_s=12.0):
     """Reference sampler on the host cores of this box: penalties pre-pass (oracle) + prepare / filter / draw of the
-    reference's own code with its splitmix uniform. One thread."""
+    reference's own code with its splitmix uniform. One thread; rows of the batch in order, wrapping round with the
+    decode step advanced, until budget_s seconds of CPU work are spent."""
     import ctypes as C
     import numpy as np
     import gpu_cases as gc
@@ -84,7 +88,8 @@ def cpu_baseline(c, budget_s=12.0, max_rows=64):
     kind = "reference" if ref is not None else "port"
     done, t_used = 0, 0.0
     V = c["V"]
-    for r in range(min(max_rows, c["rows"])):
+    for k in range(1 << 20):
+        r, lap = k % c["rows"], k // c["rows"]
         x = gc.row_f32(c, r).copy()
         hist = np.ascontiguousarray(c["hist"][r]) if c["hist"] is not None else np.zeros(0, np.int32)
         bi = np.ascontiguousarray(c["bias_ids"][r]) if c["bias_ids"] is not None else np.zeros(0, np.int32)
@@ -96,14 +101,14 @@ def cpu_baseline(c, budget_s=12.0, max_rows=64):
         port.wo_apply_penalties(wo._ptr(x), V, wo._ptr(allow) if allow is not None else None, wo._ptr(hist), hist.size,
                                 c["rep"][r], c["pres"][r], c["freq"][r], wo._ptr(bi), wo._ptr(bv), bi.size)
         rows, keep = wo.make_rows(x[None, :], 256, 16384)
-        lib.wo_prepare_draw(C.byref(rows), C.byref(s), 0, int(c["step"][r]))
+        lib.wo_prepare_draw(C.byref(rows), C.byref(s), 0, int(c["step"][r]) + lap)
         t_used += time.perf_counter() - t0
         done += 1
         if t_used > budget_s:
             break
     return dict(value=done / t_used, unit="rows/s", cores=1, kind=kind,
-                sample=f"first {done} rows of the same batch, penalties + escalation 256/16384/full + filter + draw, "
-                       f"{t_used:.2f} s on one host thread")
+                sample=f"{done} rows (the rows of the same batch in order, wrapping), penalties + escalation "
+                       f"256/16384/full + filter + draw, {t_used:.2f} s on one host thread")
 
 
 def run_workload(name, steps, warmup, check_rows):
@@ -169,7 +174,7 @@ def main():
                    "filters": "see tests/gpu_cases.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
                    "sweep_mode": a.mode},
         "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": main_res["frac_of_hbm_peak"], "traffic": None, "kernel": "ws::sample_batch_kernel",
+                     "frac": main_res["frac_of_hbm_peak"], "traffic": TRAFFIC_BYTES.get((a.workload, a.mode)), "kernel": "ws::sample_batch_kernel",
                      "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},
         "cpu_baseline": cpu,
         "parity": main_res["parity"],

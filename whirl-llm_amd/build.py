@@ -13,7 +13,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "csrc", "ws_abi.hip")
 SRC_FUSED = os.path.join(HERE, "csrc", "ws_fused.hip")
 # packed FP32 instructions are switched off for every device compile of this repository
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # the fused sweep is one fully unrolled loop of ~20 batches (its bin cache must stay in registers)
+         "-mllvm", "-pragma-unroll-threshold=262144"]
 
 
 def run(cmd):

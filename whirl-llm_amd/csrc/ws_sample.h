@@ -246,7 +246,9 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
     const uint32_t nv = rv.V / PER;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     uint4 q[kRing][kBatch];
-    uint32_t na[kRing][kBatch];
+    uint32_t na[kRing][kBatch], tq[kRing][kBatch];
+    // the touched-bitmap words ride in the ring too: LDS returns in order, so a read issued between the histogram
+    // atomics would wait for every atomic queued before it
     auto load = [&](int bt, int slot) {
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -254,6 +256,7 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             const uint32_t jc = j < nv ? j : nv - 1u;
             q[slot][u] = xv[jc];
             na[slot][u] = (MASKED && rv.allow) ? ~rv.allow[(jc * PER) >> 5] : 0u;
+            tq[slot][u] = (MASKED && rv.touched) ? rv.touched[(jc * PER) >> 5] : 0u;
         }
     };
     load(0, 0);
@@ -270,14 +273,13 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             const int c0 = (bt * kBatch + u) * kPairs;
             if (j < nv) {
                 const uint32_t i = j * PER;
-                const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
+                const uint32_t tw = tq[slot][u];
                 const int32_t bw = static_cast<int32_t>((na[slot][u] | tw) >> (i & 31u));
                 const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
-                uint32_t bins[PER], raw[PER];
+                uint32_t bins[PER];
 #pragma unroll
                 for (int e = 0; e < PER; ++e) {
-                    raw[e] = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
-                    uint32_t bits = raw[e];
+                    uint32_t bits = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
                     if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     const float x = __uint_as_float(bits);
                     m = fmaxf(m, x);
@@ -293,14 +295,16 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
                     // touched tokens of this vector (one vector in twenty has one): raw logit -> stash[rank], straight
                     // from the registers; the select chain runs for every lane, only the store is predicated
                     uint32_t tb = (tw >> (i & 31u)) & (PER == 4 ? 15u : 255u);
-                    uint32_t r = static_cast<uint32_t>(rv.wprefix[i >> 5]) + __popc(tw & ((1u << (i & 31u)) - 1u));
+                    uint32_t r = tb ? static_cast<uint32_t>(rv.wprefix[i >> 5]) + __popc(tw & ((1u << (i & 31u)) - 1u)) : 0u;
                     const uint32_t nab = na[slot][u] >> (i & 31u);
                     while (tb) {
                         const uint32_t e0 = static_cast<uint32_t>(__ffs(tb)) - 1u;
                         tb &= tb - 1u;
-                        uint32_t v = raw[0];
-#pragma unroll
-                        for (int e = 1; e < PER; ++e) v = e0 == static_cast<uint32_t>(e) ? raw[e] : v;
+                        const uint32_t wi = PER == 4 ? e0 : e0 >> 1;
+                        uint32_t v = wi == 1u ? q[slot][u].y : q[slot][u].x;
+                        v = wi == 2u ? q[slot][u].z : v;
+                        v = wi == 3u ? q[slot][u].w : v;
+                        if (PER == 8) v = (e0 & 1u) ? (v & 0xffff0000u) : (v << 16);
                         stash[r++] = ((nab >> e0) & 1u) ? -INFINITY : fmaxf(__uint_as_float(v), -INFINITY);
                     }
                 }
