@@ -169,7 +169,7 @@ typedef struct ws_batch {
 
     void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes */
     uint64_t workspace_bytes;
-    double tol;             /* flag tolerance (0: 2^-40) */
+    double tol;             /* flag tolerance, relative; values below 1e-6 (and 0) mean 1e-6, the accuracy of the mass estimates */
     int32_t mode;           /* WS_MODE_* */
 } ws_batch;
 

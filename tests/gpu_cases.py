@@ -186,7 +186,7 @@ def compare_rows(c, smp, rows_to_check, rng_mode, check_kept=True, near_tol=1e-6
 
     Bars: token ids identical; kept-set ids identical (as sets, device order is ascending id) and their
     penalty-applied logits bit-identical; n_kept identical; probability of the token within 1e-6 relative;
-    max logit bit-identical, float normaliser within 1 ulp-ish (2e-7 relative)."""
+    max logit bit-identical, float normaliser within the 1e-6 relative the probabilities are held to."""
     import torch
     m = pkg()
     torch.cuda.synchronize()
@@ -217,7 +217,7 @@ def compare_rows(c, smp, rows_to_check, rng_mode, check_kept=True, near_tol=1e-6
             continue
         res["exact"] += 1
         assert st[r, 0] == o.m, f"row {r}: max {st[r, 0]} vs {o.m}"
-        assert abs(st[r, 1] - o.sum) <= 2e-7 * o.sum, f"row {r}: sum {st[r, 1]} vs {o.sum}"
+        assert abs(st[r, 1] - o.sum) <= 1e-6 * o.sum, f"row {r}: sum {st[r, 1]} vs {o.sum}"
         rel = abs(float(prob[r]) - float(o.prob)) / float(o.prob)
         res["max_prob_rel"] = max(res["max_prob_rel"], rel)
         assert rel <= 1e-6, f"row {r}: prob {prob[r]} vs {o.prob}"

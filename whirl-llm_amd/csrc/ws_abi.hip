@@ -212,7 +212,7 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.kept_ids = b->kept_ids;
     a.kept_logits = b->kept_logits;
     a.kept_cap = b->kept_cap;
-    a.tol = b->tol > 0 ? b->tol : 1.0 / 1099511627776.0;
+    a.tol = b->tol > 1e-6 ? b->tol : 1e-6;  // the histogram masses are good to ~5e-7 relative: no decision closer than that is trusted
     a.lds_ab = p.lds_ab;
     a.lds_cnt = p.lds_cnt;
     if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);

@@ -81,6 +81,17 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     for (int w = 1; w < WS_WAVES; ++w) r = fmaxf(r, red[w]);
     return r;
 }
+__device__ __forceinline__ uint32_t block_min(uint32_t v, uint32_t* red) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = min(v, static_cast<uint32_t>(__shfl_xor(v, o)));
+    __syncthreads();
+    if (lane_id() == 0) red[wave_id()] = v;
+    __syncthreads();
+    uint32_t r = red[0];
+#pragma unroll
+    for (int w = 1; w < WS_WAVES; ++w) r = min(r, red[w]);
+    return r;
+}
 __device__ __forceinline__ Best block_best(Best b, float* red_v, int* red_i) {
     b = wave_best(b);
     __syncthreads();

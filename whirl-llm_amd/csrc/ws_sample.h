@@ -3,9 +3,10 @@
 // Per row (ws_batch in include/whirl_sampling_abi.h states the order of operations):
 //   phase 0  penalties / bias: an LDS bitmap of the token ids the history and the bias list touch, a per-word
 //            prefix popcount (rank of a touched id = perfect hash), per-rank counts by LDS atomics, then the adjusted
-//            logit of every touched token (one 4-byte gather each) into an LDS array by rank. The passes below stream
-//            the row unmodified, skip touched tokens (bit set) and replay them from that array, so no penalised copy
-//            of the row is ever written and the hot loop has no dependent loads.
+//            logit of every touched token (one 4-byte gather each) into an LDS array by rank. No penalised copy of the
+//            row is ever written: the three-pass mode streams the row unmodified, skips touched tokens (bit set) and
+//            replays them from that array; the single-sweep mode bins every token as it is and afterwards moves the
+//            touched ones from the bin of their raw logit to the bin of their adjusted logit.
 //   pass 1   maximum of the adjusted row (NaN and masked tokens count as -inf).
 //   pass 2   histogram of 4096 bins of width 1/64 in a = (max - x) * inv_t, the exponent of the softmax: one LDS
 //            64-bit atomic per element adds {count, fixed-point 1 - exp(-(a - bin edge))} (degree-4 polynomial, no
@@ -32,7 +33,6 @@ constexpr int kPT = kBins / WS_BLOCK;    // histogram bins, and sorted candidate
 constexpr int kCountShift = 44;          // histogram word: count << 44 | fixed-point sum of (1 - exp(-w))
 constexpr float kFixScale = 1073741824.f;  // 2^30
 constexpr double kFixInv = 1.0 / 1073741824.0;
-constexpr float kEdgeShift = 2.44140625e-4f;  // 2^-12 bins: keeps the in-bin offset positive against the rounding of t
 // 2^30 * (1 - exp(-w / 64)) = w * (k0 + w * (k1 + w * k2)) for the in-bin offset w in [0, 1.02] (max error 1.4e-10 * 2^30)
 constexpr float kG0 = 16777216.0f, kG1 = -131070.34375f, kG2 = 678.6015014648438f;
 
@@ -89,7 +89,7 @@ struct RowView {
     const float* pv;          // LDS adjusted logits of the touched tokens, by rank
 };
 
-constexpr int kBatch = 4;  // 128-bit loads per thread and batch; two batches are in flight (double buffering)
+constexpr int kBatch = 4;  // 128-bit loads per thread and batch
 
 __device__ __forceinline__ float raw_logit(const RowView& rv, uint32_t i) {
     const float v = rv.dtype == 0 ? static_cast<const float*>(rv.base)[i] : bf16_to_f32(static_cast<const uint16_t*>(rv.base)[i]);
@@ -113,19 +113,16 @@ __device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
 // f(i, logit, slot) for every token of the row, slot = position inside the thread's current batch (a compile-time
 // constant after unrolling); end_batch(j0, i) after each batch of kBatch 128-bit loads per thread (j0 = first vector
 // index of the batch; j0 = ~0 and i = the token for the one-token batches of a scalar tail), which are all issued
-// before any is used, and the next batch is requested before this one is consumed (one workgroup keeps 128 KiB of the
-// row in flight). Tokens that are masked out or that the
-// history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bin or ignores it, so the
-// hot loop has no branch. With STASH the raw logits of touched tokens are copied to stash[rank] on the way (the row
-// is read from HBM exactly once for them too); replay_touched later feeds their adjusted values.
-template <bool STASH, bool MASKED, class F, class E>
-__device__ __forceinline__ void stream_row_impl(const RowView& rv, float* stash, F&& f, E&& end_batch) {
+// before any is used, and the next batch is requested before this one is consumed. Tokens that are masked out or that
+// the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bin or ignores it, so the
+// hot loop has no branch; the touched ones are fed afterwards, by rank, with their adjusted values.
+template <bool MASKED, class F, class E>
+__device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch) {
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
     const uint32_t per = rv.dtype == 0 ? 4u : 8u;  // elements per 128-bit load
     const uint32_t nv = rv.vec ? V / per : 0u;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
-    constexpr bool masked = MASKED;
     constexpr uint32_t kStep = kBatch * WS_BLOCK;
     struct Batch {
         uint4 q[kBatch];
@@ -145,7 +142,6 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, float* stash,
     for (uint32_t j0 = 0; j0 < nv; j0 += kStep) {
         const bool more = j0 + kStep < nv;
         if (more) load(j0 + kStep, nxt);  // the next batch is in flight while this one is consumed
-        uint32_t tslots = 0;              // STASH: touched tokens among this thread's (at most 32) batch slots
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const uint32_t j = j0 + u * WS_BLOCK + t;
@@ -153,93 +149,74 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, float* stash,
             const uint32_t i = j * per;
             const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
             const int32_t bw = static_cast<int32_t>((cur.na[u] | tw) >> (i & 31u));
-            if (STASH) tslots |= ((tw >> (i & 31u)) & (per == 4u ? 15u : 255u)) << (u * per);
             const uint32_t w[4] = {cur.q[u].x, cur.q[u].y, cur.q[u].z, cur.q[u].w};
             if (rv.dtype == 0) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     uint32_t bits = w[e];
-                    if (masked) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);  // bit e set -> all ones = NaN
+                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);  // bit e set -> all ones = NaN
                     f(i + e, __uint_as_float(bits), u * 4 + e);
                 }
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     uint32_t bits = (e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16);
-                    if (masked) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
+                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     f(i + e, __uint_as_float(bits), u * 8 + e);
                 }
-            }
-        }
-        if (STASH) {
-            while (tslots) {  // about one token in a hundred: re-read from the lines the batch has just pulled in
-                const uint32_t slot = static_cast<uint32_t>(__ffs(tslots)) - 1u;
-                tslots &= tslots - 1u;
-                const uint32_t i = (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
-                stash[rank_of(rv, i)] = is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY;
             }
         }
         end_batch(j0, 0u);
         if (more) cur = nxt;
     }
     for (uint32_t i = nv * per + t; i < V; i += WS_BLOCK) {  // unaligned row or the last few tokens: one-token batches
-        const bool tch = is_touched(rv, i), ok = is_allowed(rv, i);
-        const float x = raw_logit(rv, i);
-        if (STASH && tch) stash[rank_of(rv, i)] = ok ? x : -INFINITY;
-        f(i, (tch || !ok) ? __uint_as_float(0xffffffffu) : x, 0);
+        const bool skip = is_touched(rv, i) || !is_allowed(rv, i);
+        f(i, skip ? __uint_as_float(0xffffffffu) : raw_logit(rv, i), 0);
         end_batch(0xffffffffu, i);
     }
 }
 
-template <bool STASH, class F, class E>
-__device__ __forceinline__ void stream_row(const RowView& rv, float* stash, F&& f, E&& end_batch) {
-    if (rv.allow || rv.touched) stream_row_impl<STASH, true>(rv, stash, f, end_batch);
-    else stream_row_impl<STASH, false>(rv, stash, f, end_batch);
+template <class F, class E>
+__device__ __forceinline__ void stream_row(const RowView& rv, F&& f, E&& end_batch) {
+    if (rv.allow || rv.touched) stream_row_impl<true>(rv, f, end_batch);
+    else stream_row_impl<false>(rv, f, end_batch);
 }
 
-// f(i, adjusted logit) for the touched tokens: thread t walks the set bits of its chunk of bitmap words
-template <class F>
-__device__ __forceinline__ void replay_touched(const RowView& rv, F&& f) {
-    if (!rv.touched) return;
-    const uint32_t nW = (rv.V + 31u) >> 5;
-    const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
-    const uint32_t w0 = threadIdx.x * chunk, w1 = min(w0 + chunk, nW);
-    for (uint32_t w = w0; w < w1; ++w) {
-        uint32_t bits = rv.touched[w];
-        uint32_t r = rv.wprefix[w];
-        while (bits) {
-            const uint32_t b = __ffs(bits) - 1u;
-            bits &= bits - 1u;
-            f((w << 5) + b, rv.pv[r++]);
-        }
-    }
+// ---- bins. A token's bin coordinate is t = fma(x, -c64, aq): c64 = 64 * inv_t and aq = anchor * c64 rounded a little
+// upwards (anchor_product), so that t >= 0 for every x <= anchor; t = 64 * (aq / 64 - x * inv_t) to half an ulp of t,
+// one rounding. bin = trunc(min(t, 4095)): bin 0 is nearest the anchor, 1/64 of an exponent unit per bin, and the tail
+// bin 4095 takes NaN, -inf and everything whose mass is below e^-64 of the anchor's. The same function is used by
+// every pass, so a token's bin never depends on who computes it.
+__device__ __forceinline__ float anchor_product(float anchor, float c64) {
+    const float a = __fmul_rn(anchor, c64);
+    return __fmaf_rn(fabsf(a), 4.76837158203125e-7f, a);  // + 2^-21 |a|: above the exact product whatever the roundings
+}
+__device__ __forceinline__ float bin_coord(float aq, float c64, float x) {
+    const float t = __fmaf_rn(x, -c64, aq);
+    return t < 4095.f ? t : 4095.f;  // NaN -> tail
+}
+__device__ __forceinline__ uint32_t bin_of(float aq, float c64, float x) { return static_cast<uint32_t>(bin_coord(aq, c64, x)); }
+// histogram word of one token: count 1 and the fixed-point cubic of the in-bin offset w = fract(t)
+__device__ __forceinline__ uint64_t bin_word(float tc) {
+    const float w = __builtin_amdgcn_fractf(tc);
+    const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
+    return (1ull << kCountShift) | fx;
 }
 
-// Bin of a logit: t = fl((m - x) * c64), c64 = 64 * inv_t, clamped to the tail bin 4095 (NaN, -inf and everything whose
-// mass is below e^-64 of the top token's); bin = trunc(t). tlo is the exact residual of the product, so that
-// (bin + fract(t) + tlo) / 64 equals the exponent (double)(m - x) * inv_t of the host formula to the last bit.
-struct BinPos {
-    float tc;   // clamped t
-    float tlo;  // exact residual of (m - x) * c64 (garbage for the tail)
-};
-__device__ __forceinline__ BinPos bin_pos(float m, float c64, float x) {
-    BinPos r;
-    const float d = __fsub_rn(m, x);
-    const float t = __fmul_rn(d, c64);
-    r.tlo = __fmaf_rn(d, c64, -t);
-    r.tc = t < 4095.f ? t : 4095.f;
-    return r;
-}
-__device__ __forceinline__ uint32_t bin_of(float m, float c64, float x) { return static_cast<uint32_t>(bin_pos(m, c64, x).tc); }
-
-// ---- fused mode: one sweep over the row does the histogram against a provisional anchor, tracks the true maximum,
-// stashes the touched tokens and keeps every token's bin index in registers (two per VGPR), so that the gather of
-// the few bins the cuts land in needs no second sweep. Rows of up to 163840 tokens.
+// ---- fused mode: one sweep over the row does the histogram against a provisional anchor, tracks the maximum and
+// keeps every token's bin index in registers (two per VGPR), so that the gather of the few bins the cuts land in
+// needs no second sweep. Rows of up to 163840 tokens. Only the allow mask is applied here; touched tokens are binned
+// with their raw logit and moved afterwards. For that their raw logits are needed: a 128-bit vector that holds a
+// touched token is copied as it is to stage[rank of its first touched token] (LDS, stage_cap slots of 16 bytes), which
+// costs two instructions per token and spares one scattered 4-byte read from HBM per touched token.
 constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 with 512
 
-template <int PER, bool MASKED>
-__device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash, float anchor, float c64, uint64_t* hist,
-                                                uint32_t (&cache)[kCacheRegs], float& m) {
+// Provisional anchor: the larger of `floor` and the maximum of the thread block's first batch of loads, plus 8 exponent
+// units of headroom; the same registers then feed the sweep. Returns false (nothing binned) when that is not finite.
+template <int PER, bool MASKED, bool TOUCHED>
+__device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
+                                                uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap,
+                                                float& anchor, float& aq, float& m) {
     constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
     constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
@@ -247,7 +224,7 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     uint4 q[kRing][kBatch];
     uint32_t na[kRing][kBatch], tq[kRing][kBatch];
-    // the touched-bitmap words ride in the ring too: LDS returns in order, so a read issued between the histogram
+    // the touched-bitmap words ride in the ring too: LDS answers in order, so a read issued between the histogram
     // atomics would wait for every atomic queued before it
     auto load = [&](int bt, int slot) {
 #pragma unroll
@@ -255,12 +232,29 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;
             q[slot][u] = xv[jc];
-            na[slot][u] = (MASKED && rv.allow) ? ~rv.allow[(jc * PER) >> 5] : 0u;
-            tq[slot][u] = (MASKED && rv.touched) ? rv.touched[(jc * PER) >> 5] : 0u;
+            na[slot][u] = MASKED ? ~rv.allow[(jc * PER) >> 5] : 0u;
+            tq[slot][u] = TOUCHED ? rv.touched[(jc * PER) >> 5] : 0u;
         }
     };
     load(0, 0);
     if (NB > 1) load(1, 1);
+    for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+    {
+        float s = floor_v;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t w[4] = {q[0][u].x, q[0][u].y, q[0][u].z, q[0][u].w};  // lanes past the row hold its last vector
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (PER == 4) s = fmaxf(s, __uint_as_float(w[e]));
+                else s = fmaxf(s, fmaxf(__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)));
+            }
+        }
+        s = block_max(s, red);  // its barriers also publish the zeroed histogram
+        anchor = s + 8.f / inv_t;
+        aq = anchor_product(anchor, c64);
+        if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
+    }
 #pragma unroll
     for (int bt = 0; bt < NB; ++bt) {
         const int slot = bt % kRing;
@@ -272,9 +266,7 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             constexpr int kPairs = PER / 2;
             const int c0 = (bt * kBatch + u) * kPairs;
             if (j < nv) {
-                const uint32_t i = j * PER;
-                const uint32_t tw = tq[slot][u];
-                const int32_t bw = static_cast<int32_t>((na[slot][u] | tw) >> (i & 31u));
+                const int32_t bw = MASKED ? static_cast<int32_t>(na[slot][u] >> ((j * PER) & 31u)) : 0;
                 const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
                 uint32_t bins[PER];
 #pragma unroll
@@ -283,29 +275,17 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
                     if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     const float x = __uint_as_float(bits);
                     m = fmaxf(m, x);
-                    const BinPos p = bin_pos(anchor, c64, x);
-                    const float wf = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);
-                    const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(wf, __fmaf_rn(wf, __fmaf_rn(wf, kG2, kG1), kG0), 0.5f));
-                    bins[e] = static_cast<uint32_t>(p.tc);
-                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bins[e]]), (1ull << kCountShift) | fx);
+                    const float tc = bin_coord(aq, c64, x);
+                    bins[e] = static_cast<uint32_t>(tc);
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bins[e]]), bin_word(tc));
                 }
 #pragma unroll
                 for (int k = 0; k < kPairs; ++k) cache[c0 + k] = bins[2 * k] | (bins[2 * k + 1] << 16);
-                if (MASKED) {
-                    // touched tokens of this vector (one vector in twenty has one): raw logit -> stash[rank], straight
-                    // from the registers; the select chain runs for every lane, only the store is predicated
-                    uint32_t tb = (tw >> (i & 31u)) & (PER == 4 ? 15u : 255u);
-                    uint32_t r = tb ? static_cast<uint32_t>(rv.wprefix[i >> 5]) + __popc(tw & ((1u << (i & 31u)) - 1u)) : 0u;
-                    const uint32_t nab = na[slot][u] >> (i & 31u);
-                    while (tb) {
-                        const uint32_t e0 = static_cast<uint32_t>(__ffs(tb)) - 1u;
-                        tb &= tb - 1u;
-                        const uint32_t wi = PER == 4 ? e0 : e0 >> 1;
-                        uint32_t v = wi == 1u ? q[slot][u].y : q[slot][u].x;
-                        v = wi == 2u ? q[slot][u].z : v;
-                        v = wi == 3u ? q[slot][u].w : v;
-                        if (PER == 8) v = (e0 & 1u) ? (v & 0xffff0000u) : (v << 16);
-                        stash[r++] = ((nab >> e0) & 1u) ? -INFINITY : fmaxf(__uint_as_float(v), -INFINITY);
+                if (TOUCHED) {
+                    const uint32_t sh = (j * PER) & 31u, tw = tq[slot][u];
+                    if ((tw >> sh) & (PER == 4 ? 15u : 255u)) {
+                        const uint32_t r = static_cast<uint32_t>(rv.wprefix[(j * PER) >> 5]) + __popc(tw & ((1u << sh) - 1u));
+                        if (r < stage_cap) stage[r] = q[slot][u];
                     }
                 }
             } else {
@@ -314,18 +294,20 @@ __device__ __forceinline__ void fused_pass_impl(const RowView& rv, float* stash,
             }
         }
     }
+    return true;
 }
 
-__device__ __forceinline__ void fused_pass(const RowView& rv, float* stash, float anchor, float c64, uint64_t* hist,
-                                           uint32_t (&cache)[kCacheRegs], float& m) {
-    const bool masked = rv.allow || rv.touched;
+__device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
+                                           uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap, float& anchor,
+                                           float& aq, float& m) {
+#define WS_FUSED_CALL(PER, AL, TC) fused_pass_impl<PER, AL, TC>(rv, floor_v, inv_t, c64, hist, cache, red, stage, stage_cap, anchor, aq, m)
     if (rv.dtype == 0) {
-        if (masked) fused_pass_impl<4, true>(rv, stash, anchor, c64, hist, cache, m);
-        else fused_pass_impl<4, false>(rv, stash, anchor, c64, hist, cache, m);
-    } else {
-        if (masked) fused_pass_impl<8, true>(rv, stash, anchor, c64, hist, cache, m);
-        else fused_pass_impl<8, false>(rv, stash, anchor, c64, hist, cache, m);
+        if (rv.touched) return rv.allow ? WS_FUSED_CALL(4, true, true) : WS_FUSED_CALL(4, false, true);
+        return rv.allow ? WS_FUSED_CALL(4, true, false) : WS_FUSED_CALL(4, false, false);
     }
+    if (rv.touched) return rv.allow ? WS_FUSED_CALL(8, true, true) : WS_FUSED_CALL(8, false, true);
+    return rv.allow ? WS_FUSED_CALL(8, true, false) : WS_FUSED_CALL(8, false, false);
+#undef WS_FUSED_CALL
 }
 
 // token index of half `half` of cache register k of thread t (the layout fused_pass_impl writes)
@@ -335,15 +317,17 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
 }
 
 // Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range): its index goes
-// to list[] (LDS, count in *n_list; entries past cap are dropped but counted). Both 16-bit halves of a register are
-// tested at once: with bit 15 of each half forced on, (y - lo) and (y - hi - 1) differ in bit 15 exactly for
-// lo <= bin <= hi. Hits are shifted into one mask per 16 registers; tokens are pushed after the scan.
+// to list[] (LDS, at most cap entries; *n_list, zeroed by the caller before a barrier, counts all hits). Both 16-bit
+// halves of a register are tested at once: with bit 15 of each half forced on, (y - lo) and (y - hi - 1) differ in
+// bit 15 exactly for lo <= bin <= hi. Hits are shifted into one mask per 16 registers; then each wave reserves a
+// stretch of the list with one atomic and its lanes write their tokens.
 __device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
                                                   uint32_t w1, uint32_t* list, uint32_t* n_list, uint32_t cap) {
     const bool two = u1 <= 0x7fffu;
     const uint32_t L0 = u0 * 0x10001u, H0 = (u0 + w0 + 1u) * 0x10001u;
     const uint32_t L1 = two ? u1 * 0x10001u : 0u, H1 = two ? (u1 + w1 + 1u) * 0x10001u : 0u;
     uint32_t hits[kCacheRegs / 16];
+    uint32_t mine = 0;
 #pragma unroll
     for (int g = 0; g < kCacheRegs / 16; ++g) {
         uint32_t acc = 0;
@@ -355,28 +339,38 @@ __device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&ca
             acc = (acc >> 1) | (r & 0x80008000u);  // register k: low half -> bit k, high half -> bit 16 + k
         }
         hits[g] = acc;
+        mine += __popc(acc);
     }
+    uint32_t inc = mine;  // inclusive prefix over the wave
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o);
+        if (lane_id() >= o) inc += up;
+    }
+    uint32_t base = 0;
+    if (lane_id() == 63 && inc) base = atomicAdd(n_list, inc);
+    uint32_t slot = __shfl(base, 63) + inc - mine;
 #pragma unroll
     for (int g = 0; g < kCacheRegs / 16; ++g) {
         uint32_t h = hits[g];
         while (h) {
             const uint32_t bit = static_cast<uint32_t>(__ffs(h)) - 1u;
             h &= h - 1u;
-            const uint32_t slot = atomicAdd(n_list, 1u);
             if (slot < cap) list[slot] = cache_token(dtype, g * 16u + (bit & 15u), bit >> 4);
+            ++slot;
         }
     }
 }
 
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
 // every element with key32 >= the result lies in a bin < bcut. 0xffffffff when no finite logit does.
-__device__ __forceinline__ uint32_t first_key_before_bin(float m, float c64, int bcut) {
-    uint32_t lo = key32(-INFINITY), hi = key32(m);  // bin(lo) = tail, bin(hi) = 0 (m = the value bins are measured from)
-    if (bcut <= 0) return 0xffffffffu;
+__device__ __forceinline__ uint32_t first_key_before_bin(float aq, float c64, float top, int bcut) {
+    uint32_t lo = key32(-INFINITY), hi = key32(top);  // bin(lo) = tail; top = a value whose bin is 0 or the first non-empty one
+    if (bcut <= 0 || bin_of(aq, c64, top) >= static_cast<uint32_t>(bcut)) return 0xffffffffu;
     const uint32_t bc = static_cast<uint32_t>(bcut);
     while (lo + 1u < hi) {  // invariant: bin(lo) >= bcut, bin(hi) < bcut
         const uint32_t mid = lo + ((hi - lo) >> 1);
-        if (bin_of(m, c64, unkey32(mid)) < bc) hi = mid;
+        if (bin_of(aq, c64, unkey32(mid)) < bc) hi = mid;
         else lo = mid;
     }
     return hi;
@@ -395,15 +389,13 @@ struct BinSel {
 __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
     for (uint32_t k = 2; k <= P; k <<= 1) {
         for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-            for (uint32_t i = threadIdx.x; i < P; i += WS_BLOCK) {
-                const uint32_t l = i ^ j;
-                if (l > i) {
-                    const uint64_t a = keys[i], b = keys[l];
-                    const bool up = (i & k) == 0;  // this pair sorts descending
-                    if (up ? (a < b) : (a > b)) {
-                        keys[i] = b;
-                        keys[l] = a;
-                    }
+            for (uint32_t q = threadIdx.x; q < (P >> 1); q += WS_BLOCK) {  // pair q: elements i and i + j
+                const uint32_t i = ((q & ~(j - 1u)) << 1) | (q & (j - 1u)), l = i | j;
+                const uint64_t a = keys[i], b = keys[l];
+                const bool up = (i & k) == 0;  // this pair sorts descending
+                if (up ? (a < b) : (a > b)) {
+                    keys[i] = b;
+                    keys[l] = a;
                 }
             }
             __syncthreads();
@@ -477,7 +469,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // ------------------------------------------------------------------ phase 0: penalties and bias
     const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? A.hist_off[row + 1] - h0 : 0u;
     const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
-    uint32_t n_touched = 0;  // tokens the streaming loop sends to the tail bin as NaN and replay_touched adds back
+    uint32_t n_touched = 0;  // distinct tokens the history and the bias list touch
+    float m_adj = -INFINITY;  // largest adjusted logit among them
+    float m_rawt = -INFINITY; // largest raw logit among them
     if (!(inv_t > 0.f) || nh + nb > A.patch_cap) flags |= kBadParam;
     if (!(flags & kBadParam) && nh + nb > 0) {
         const int32_t* hist_ids = A.hist + h0;
@@ -539,80 +533,185 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             pv[r] = sum;
         }
         __syncthreads();
-        // per rank: bias sum -> first[r] (float bits; the first-entry bookkeeping is dead), cnt[r] stays. The raw logits
-        // of the touched tokens are stashed into pv[] by pass 1, straight from its stream.
+        // per rank: bias sum -> first[r] (float bits; the first-entry bookkeeping is dead), cnt[r] stays
         for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) first[r] = __float_as_uint(pv[r]);
+        __syncthreads();
         n_touched = n_uniq;
         __syncthreads();
     }
+    const float* praw = reinterpret_cast<const float*>(lds + A.lds_cnt);           // raw logits of the touched tokens, by rank
+    const uint32_t* pid = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt) + A.patch_cap;  // their token ids
+    // Raw logit of every touched token as the sweeps see it (NaN and masked-out -> -inf), one 4-byte gather per history
+    // / bias entry (entries of one id store the same value), then its adjusted logit, once: bias, repetition, then
+    // frequency and presence, each operation rounded to float. pv[r] <- adjusted, praw[r] (the dead count slot) <- raw,
+    // pid[r] (the dead bias-sum slot) <- token id. The three-pass kernel runs this before its first pass; the
+    // single-sweep kernel after the sweep, when the row has just come through the caches.
+    auto gather_and_adjust = [&](const uint4* stage, uint32_t stage_cap) {
+        if (!n_touched) return;
+        const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+        const int32_t* hist_ids = A.hist + h0;
+        const int32_t* bias_ids = A.bias_ids + b0;
+        uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
+        uint32_t* first = cnt + A.patch_cap;
+        auto fetch4 = [&](const int32_t* ids, uint32_t n) {  // four independent gathers per thread and round
+            for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
+                uint32_t id[4], bits[4], al[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t j = j0 + k * WS_BLOCK + t;
+                    id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    // slot of the token's vector = rank of the vector's first touched token
+                    const uint32_t vb = i & ~(per - 1u), tw = touched[i >> 5];
+                    const uint32_t rf = static_cast<uint32_t>(wprefix[i >> 5]) + __popc(tw & ((1u << (vb & 31u)) - 1u));
+                    if (rf < stage_cap) {
+                        const uint32_t* sv = reinterpret_cast<const uint32_t*>(stage + rf);
+                        bits[k] = rv.dtype == 0 ? sv[i & 3u] : (((i & 1u) ? sv[(i & 7u) >> 1] & 0xffff0000u : sv[(i & 7u) >> 1] << 16));
+                    } else {
+                        bits[k] = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
+                                                : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
+                    }
+                    al[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (id[k] < V)
+                        pv[rank_of(rv, id[k])] = ((al[k] >> (id[k] & 31u)) & 1u) ? fmaxf(__uint_as_float(bits[k]), -INFINITY) : -INFINITY;
+            }
+        };
+        fetch4(hist_ids, nh);
+        fetch4(bias_ids, nb);
+        __syncthreads();
+        {
+            const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
+            float ma = -INFINITY, mr = -INFINITY;
+            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+                const uint32_t cw = cnt[r], c = cw & 0xfffffu;
+                const float raw = pv[r];
+                float x = raw;
+                if (cw >> 20) x = __fadd_rn(x, __uint_as_float(first[r]));
+                if (c) {
+                    x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                    x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
+                }
+                pv[r] = x;
+                cnt[r] = __float_as_uint(raw);
+                ma = fmaxf(ma, x);
+                mr = fmaxf(mr, raw);
+            }
+            m_adj = block_max(ma, red_f);
+            m_rawt = block_max(mr, red_f);
+        }
+        if (FUSED) {
+            for (uint32_t j = t; j < nh; j += WS_BLOCK) {
+                const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
+                if (id < V) first[rank_of(rv, id)] = id;
+            }
+            for (uint32_t j = t; j < nb; j += WS_BLOCK) {
+                const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
+                if (id < V) first[rank_of(rv, id)] = id;
+            }
+        }
+        __syncthreads();
+    };
+    // f(token, adjusted logit) for every touched token. The single-sweep kernel keeps praw / pid in LDS of their own;
+    // in the three-pass kernel that LDS is the histogram's, so it walks the set bits of the bitmap instead.
+    auto replay_touched = [&](auto&& f) {
+        if (FUSED) {
+            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) f(pid[r], pv[r]);
+        } else if (n_touched) {
+            const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
+            const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
+            for (uint32_t w = w0; w < w1; ++w) {
+                uint32_t bits = touched[w];
+                uint32_t r = wprefix[w];
+                while (bits) {
+                    const uint32_t b = __ffs(bits) - 1u;
+                    bits &= bits - 1u;
+                    f((w << 5) + b, pv[r++]);
+                }
+            }
+        }
+    };
 
     WS_MARK(0);
     const float c64 = inv_t * 64.f;
-    auto adjust_touched = [&](float& mref) {
-        // adjusted logit of every touched token, once: (mask / NaN already applied) bias, repetition, frequency, presence
-        if (!n_touched) return;
-        __syncthreads();
-        const uint32_t* cnt = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt);
-        const uint32_t* bsum = cnt + A.patch_cap;
-        const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
-        for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
-            const uint32_t c = cnt[r] & 0xfffffu;
-            float x = pv[r];
-            if (cnt[r] >> 20) x = __fadd_rn(x, __uint_as_float(bsum[r]));
-            if (c) {
-                x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
-                x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
-            }
-            pv[r] = x;
-            mref = fmaxf(mref, x);
-        }
-    };
     float anchor = 0.f;  // bins are measured down from here: the row maximum, or a provisional bound above it
+    float aq = 0.f;      // anchor_product(anchor, c64)
     auto add_to_hist = [&](uint32_t, float x, int) {
-        const BinPos p = bin_pos(anchor, c64, x);
-        const float w = __builtin_amdgcn_fractf(p.tc) + (p.tlo + kEdgeShift);  // in-bin offset, 0 < w < 1.001 (NaN: tail)
-        const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
-        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(p.tc)]), (1ull << kCountShift) | fx);
+        const float tc = bin_coord(aq, c64, x);
+        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(tc)]), bin_word(tc));
     };
     float m = -INFINITY;
     bool cached = false;
     uint32_t cache[kCacheRegs];  // dead code (and no registers) in the exact instantiation
     if (FUSED && !(flags & kBadParam)) {
-        // ---------------------------------------------------------------- fused sweep: anchor, histogram, max, stash, bins
-        // anchor = the maximum of the first 4096 vectors of the row (raw logits) + 8 exponent units of headroom
-        {
-            const uint32_t per = rv.dtype == 0 ? 4u : 8u, nv = V / per;
-            float s = -INFINITY;
-            for (uint32_t j = t; j < nv && j < kBatch * WS_BLOCK; j += WS_BLOCK) {
-                const uint4 q = static_cast<const uint4*>(rv.base)[j];
-                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (rv.dtype == 0) s = fmaxf(s, __uint_as_float(w[e]));
-                    else s = fmaxf(s, fmaxf(__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)));
-                }
+        // ---------------------------------------------------------------- fused sweep: anchor, histogram, max, bins
+        bool swept = false;
+        // staging room for the vectors that hold touched tokens: the LDS of the candidate masses, idle until pass 3
+        uint4* stage = reinterpret_cast<uint4*>(emass);
+        const uint32_t stage_cap = rv.vec ? 2048u : 0u;
+        if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, cache, red_f, stage, stage_cap, anchor, aq, m);
+        __syncthreads();
+        WS_MARK(8);
+        gather_and_adjust(stage, swept ? stage_cap : 0u);
+        WS_MARK(9);
+        if (swept) {
+            m = block_max(m, red_f);  // over the raw row (allow mask applied), touched tokens included
+            // touched tokens: out of the bin of the raw logit, into the bin of the adjusted one
+            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+                const float t0 = bin_coord(aq, c64, praw[r]), t1 = bin_coord(aq, c64, pv[r]);
+                atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
+                atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
             }
-            for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
-            s = block_max(s, red_f);
-            anchor = s + 8.f / inv_t;
-        }
-        if (anchor > -INFINITY && anchor < INFINITY) {
-            if constexpr (FUSED) fused_pass(rv, pv, anchor, c64, hist, cache, m);
-            adjust_touched(m);
-            m = block_max(m, red_f);
+            bool ok = true;
+            if (n_touched && m_rawt >= m) {
+                // the largest raw logit belongs to a touched token: the largest untouched one sits in the first
+                // non-empty bin (or further down, and then an adjusted touched token of that bin is the maximum)
+                __syncthreads();
+                uint32_t fb = kBins;
+#pragma unroll
+                for (int j = kPT - 1; j >= 0; --j)
+                    if (hist[kPT * t + j] >> kCountShift) fb = kPT * t + j;
+                fb = block_min(fb, red_u);
+                float mu = -INFINITY;
+                ok = fb < kBins - 1;
+                if constexpr (FUSED) {
+                    if (ok) {
+                        uint32_t* list = reinterpret_cast<uint32_t*>(emass);  // free until pass 3
+                        if (t == 0) s_u[4] = 0;
+                        __syncthreads();
+                        gather_from_cache(rv.dtype, cache, fb, 0u, 0xffff0000u, 0u, list, &s_u[4], 2u * kCap);
+                        __syncthreads();
+                        const uint32_t n_hit = s_u[4];
+                        ok = n_hit <= 2u * kCap;
+                        if (ok)
+                            for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
+                                const uint32_t i = list[k];
+                                if (!is_touched(rv, i)) mu = fmaxf(mu, raw_logit(rv, i));
+                            }
+                    }
+                }
+                m = block_max(mu, red_f);
+            }
+            m = fmaxf(m, m_adj);
             // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
-            cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
-        } else {
-            stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
-            adjust_touched(m);
-            m = block_max(m, red_f);
+            cached = ok && m <= anchor && (anchor - m) * c64 <= 1024.f;
+        }
+        if (!cached) {
+            m = -INFINITY;
+            stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+            m = fmaxf(block_max(m, red_f), m_adj);
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     } else if (!(flags & kBadParam)) {
-        // ---------------------------------------------------------------- pass 1: maximum (and the stash of touched tokens)
-        stream_row<true>(rv, pv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
-        adjust_touched(m);
-        m = block_max(m, red_f);
+        // ---------------------------------------------------------------- pass 1: maximum
+        gather_and_adjust(nullptr, 0u);
+        stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+        m = fmaxf(block_max(m, red_f), m_adj);
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
     if (flags) {  // uniform over the block
@@ -631,20 +730,20 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     WS_MARK(1);
-    if (cached) {
-        replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
-    } else {
+    if (!cached) {
         // ---------------------------------------------------------------- pass 2: histogram of (count, mass) below the maximum
         anchor = m;
+        aq = anchor_product(anchor, c64);
         __syncthreads();
         for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
         __syncthreads();
-        stream_row<false>(rv, nullptr, add_to_hist, [](uint32_t, uint32_t) {});
-        replay_touched(rv, [&](uint32_t i, float x) { add_to_hist(i, x, 0); });
+        stream_row(rv, add_to_hist, [](uint32_t, uint32_t) {});
+        replay_touched([&](uint32_t i, float x) { add_to_hist(i, x, 0); });
     }
+    const uint32_t tail_fix = cached ? 0u : n_touched;  // pass 2 streams touched tokens into the tail bin as NaN
     __syncthreads();
     // masses are accumulated relative to the anchor; everything below works relative to the maximum
-    const double lift = (static_cast<double>(anchor) - static_cast<double>(m)) * static_cast<double>(inv_t);  // >= 0
+    const double lift = static_cast<double>(aq) * (1.0 / 64.0) - static_cast<double>(m) * static_cast<double>(inv_t);  // >= 0
     const double to_max = exp(lift);
 
     WS_MARK(2);
@@ -659,9 +758,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             const int b = kPT * t + j;
             const uint64_t h = hist[b];
             c[j] = static_cast<uint32_t>(h >> kCountShift);
-            if (b == kBins - 1) c[j] -= n_touched;  // streamed there as NaN, replayed into their own bins
+            if (b == kBins - 1) c[j] -= tail_fix;  // streamed there as NaN, replayed into their own bins
             const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
-            // mass of the bin relative to the maximum: exp(-(b - 2^-12) / 64) * sum exp(-w / 64); the tail bin carries none
+            // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail bin carries none
             ms[j] = (c[j] && b < kBins - 1) ? kExpHi[b >> 6] * kExpLo[b & 63] * (static_cast<double>(c[j]) - fix) * to_max : 0.0;
             csum += c[j];
             msum += ms[j];
@@ -860,23 +959,43 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         };
         const uint32_t u1r = two ? u1 : 0xffff0000u;  // an empty second range matches no bin
         auto in_ranges = [&](float x) {
-            const uint32_t b = bin_of(anchor, c64, x);
+            const uint32_t b = bin_of(aq, c64, x);
             return b - u0 <= w0 || b - u1r <= w1;
         };
         if (FUSED && cached) {
             if constexpr (FUSED) {
-                // token indices first (no loads in the scan), then one parallel round of loads for the keys
+                // token indices first (no loads in the scan), then rounds of independent loads for the keys; a hit
+                // that is a touched token (cached with the bin of its raw logit) is dropped here and fed below
                 uint32_t* list = reinterpret_cast<uint32_t*>(emass);
                 if (t == 0) s_u[4] = 0;
                 __syncthreads();
-                gather_from_cache(rv.dtype, cache, u0, w0, u1r, w1, list, &s_u[4], kCap);
+                gather_from_cache(rv.dtype, cache, u0, w0, u1r, w1, list, &s_u[4], 2u * kCap);
                 __syncthreads();
-                const uint32_t n_hit = min(s_u[4], kCap);
-                for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
-                    const uint32_t i = list[k];
-                    keys[k] = key64(raw_logit(rv, i), i);  // neither masked nor touched (those sit in the tail bin)
+                const uint32_t n_hit = min(s_u[4], 2u * kCap);
+                if (s_u[4] > 2u * kCap) flags |= kOverflow;
+                for (uint32_t k0 = 0; k0 < n_hit; k0 += 4u * WS_BLOCK) {
+                    uint32_t idx[4];
+                    float xs[4];
+                    bool keep[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t k = k0 + q * WS_BLOCK + t;
+                        idx[q] = k < n_hit ? list[k] : 0u;
+                        keep[q] = k < n_hit && !is_touched(rv, idx[q]);
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) xs[q] = keep[q] ? raw_logit(rv, idx[q]) : 0.f;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        // one slot reservation per wave: lanes that keep their hit take consecutive slots
+                        const uint64_t mask = __ballot(keep[q]);
+                        uint32_t base = 0;
+                        if (lane_id() == 0 && mask) base = atomicAdd(&s_cnt, static_cast<uint32_t>(__popcll(mask)));
+                        base = __shfl(base, 0);
+                        const uint32_t slot = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane_id()) - 1ull)));
+                        if (keep[q] && slot < kCap) keys[slot] = key64(xs[q], idx[q]);
+                    }
                 }
-                if (t == 0) s_cnt = s_u[4];
                 __syncthreads();
             }
         } else {
@@ -884,8 +1003,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             // are re-read after the batch, from the cache lines the batch has just pulled in
             uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
             const uint32_t per = rv.dtype == 0 ? 4u : 8u;
-            stream_row<false>(
-                rv, nullptr, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
+            stream_row(
+                rv, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
                 [&](uint32_t j0, uint32_t i_tail) {
                     while (hit) {
                         const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
@@ -895,11 +1014,25 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     }
                 });
         }
-        replay_touched(rv, [&](uint32_t i, float x) {
+        replay_touched([&](uint32_t i, float x) {
             if (in_ranges(x)) push(i, x);
         });
     }
     __syncthreads();
+    if (flags & kOverflow) {  // uniform: more cached hits than the list holds
+        if (t == 0) {
+            A.token[row] = -1;
+            A.flags[row] = flags;
+            if (A.prob) A.prob[row] = 0.f;
+            if (A.n_kept) A.n_kept[row] = 0u;
+            if (A.stats) {
+                A.stats[2 * row] = m;
+                A.stats[2 * row + 1] = static_cast<float>(Z);
+            }
+            if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
+        }
+        return;
+    }
     WS_MARK(4);
     uint32_t P = 64;
     while (P < n_list) P <<= 1;
@@ -1042,10 +1175,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         kept_key = s_key;
     } else if (has_r1 && n3 == c1base) {  // the cut falls on the upper edge of range 1: everything in earlier bins
         Zk = m1base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(anchor, c64, r1lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(aq, c64, m, r1lo)) << 32;
     } else if (n3 == c0base && n_r0) {
         Zk = m0base;
-        kept_key = static_cast<uint64_t>(first_key_before_bin(anchor, c64, r0lo)) << 32;
+        kept_key = static_cast<uint64_t>(first_key_before_bin(aq, c64, m, r0lo)) << 32;
     } else {  // no filter at all: the whole row
         Zk = Z;
         kept_key = 0ull;
@@ -1125,7 +1258,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (i < V) {
                 x = adjusted_logit(rv, i);
                 keep = key64(x, i) >= kept_key;
-                tl = tail_extra && !keep && bin_of(anchor, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
+                tl = tail_extra && !keep && bin_of(aq, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
             }
             uint32_t tot;
             const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
