@@ -116,6 +116,29 @@ def test_rows_are_independent_and_reproducible():
 
 
 @pytest.mark.parametrize("mode", MODES)
+def test_history_holds_the_top_tokens(mode):
+    """The largest logits of every row sit in its history (what repetition penalties are for), some next to each other
+    in one 128-bit vector, and a bias lifts a middling token above everything else in some rows: the row maximum after
+    penalties is then a token the plain stream never shows as the largest."""
+    rng = np.random.default_rng(11)
+    c = gc.make_cfg2(rows=16, V=151936, n_hist=512, n_bias=8)
+    x = c["logits"]
+    for r in range(16):
+        top = np.argsort(-x[r])[:40]
+        c["hist"][r, :40] = top                           # the 40 largest, penalised
+        c["hist"][r, 40:44] = (top[0] & ~3) + np.arange(4)  # and the whole vector around the largest
+        if r % 4 == 0:
+            x[r, top[0] ^ 1] = x[r, top[0]] - 0.01        # runner-up in the same vector as the largest, also touched
+        if r % 4 == 1:
+            c["bias_ids"][r, 0] = int(rng.integers(0, 151936))
+            c["bias_vals"][r, 0] = 9.0                    # a bias that beats the provisional bound some of the time
+        c["rep"][r] = 1.0 + 0.3 * (r % 3)
+    c["top_k"][:] = [0, 20, 50, 0] * 4
+    res, _ = run_case(c, 1, kept_cap=4096, mode=mode)
+    print(res)
+
+
+@pytest.mark.parametrize("mode", MODES)
 def test_cfg1_shape(mode):
     res, _ = run_case(gc.make_cfg1(), 0, mode=mode)
     print(res)

@@ -22,6 +22,8 @@
 // fixed summation order for doubles.
 #pragma once
 
+#include <type_traits>
+
 #include "ws_common.h"
 #include "ws_exp_table.h"
 
@@ -223,9 +225,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     const uint32_t nv = rv.V / PER;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     uint4 q[kRing][kBatch];
-    uint32_t na[kRing][kBatch], tq[kRing][kBatch];
-    // the touched-bitmap words ride in the ring too: LDS answers in order, so a read issued between the histogram
-    // atomics would wait for every atomic queued before it
+    uint32_t na[kRing][kBatch];
     auto load = [&](int bt, int slot) {
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -233,7 +233,6 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
             const uint32_t jc = j < nv ? j : nv - 1u;
             q[slot][u] = xv[jc];
             na[slot][u] = MASKED ? ~rv.allow[(jc * PER) >> 5] : 0u;
-            tq[slot][u] = TOUCHED ? rv.touched[(jc * PER) >> 5] : 0u;
         }
     };
     load(0, 0);
@@ -269,12 +268,13 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
                 const int32_t bw = MASKED ? static_cast<int32_t>(na[slot][u] >> ((j * PER) & 31u)) : 0;
                 const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
                 uint32_t bins[PER];
+                float vm = -INFINITY;  // maximum of this vector
 #pragma unroll
                 for (int e = 0; e < PER; ++e) {
                     uint32_t bits = PER == 4 ? w[e & 3] : ((e & 1) ? (w[e >> 1] & 0xffff0000u) : (w[e >> 1] << 16));
                     if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     const float x = __uint_as_float(bits);
-                    m = fmaxf(m, x);
+                    vm = fmaxf(vm, x);
                     const float tc = bin_coord(aq, c64, x);
                     bins[e] = static_cast<uint32_t>(tc);
                     atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bins[e]]), bin_word(tc));
@@ -282,11 +282,17 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
 #pragma unroll
                 for (int k = 0; k < kPairs; ++k) cache[c0 + k] = bins[2 * k] | (bins[2 * k + 1] << 16);
                 if (TOUCHED) {
-                    const uint32_t sh = (j * PER) & 31u, tw = tq[slot][u];
+                    // the running maximum skips vectors with touched tokens: their untouched tokens are looked at
+                    // when the touched ones are collected
+                    const uint32_t sh = (j * PER) & 31u, tw = rv.touched[(j * PER) >> 5];
                     if ((tw >> sh) & (PER == 4 ? 15u : 255u)) {
                         const uint32_t r = static_cast<uint32_t>(rv.wprefix[(j * PER) >> 5]) + __popc(tw & ((1u << sh) - 1u));
                         if (r < stage_cap) stage[r] = q[slot][u];
+                    } else {
+                        m = fmaxf(m, vm);
                     }
+                } else {
+                    m = fmaxf(m, vm);
                 }
             } else {
 #pragma unroll
@@ -318,28 +324,34 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
 
 // Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range): its index goes
 // to list[] (LDS, at most cap entries; *n_list, zeroed by the caller before a barrier, counts all hits). Both 16-bit
-// halves of a register are tested at once: with bit 15 of each half forced on, (y - lo) and (y - hi - 1) differ in
-// bit 15 exactly for lo <= bin <= hi. Hits are shifted into one mask per 16 registers; then each wave reserves a
-// stretch of the list with one atomic and its lanes write their tokens.
+// halves of a register are tested at once with packed 16-bit subtractions: (y - lo) and (y - hi - 1) differ in bit 15
+// exactly for lo <= bin <= hi (bins are below 4096, so neither difference wraps twice). Hits are shifted into one
+// mask per 16 registers; then each wave reserves a stretch of the list with one atomic and its lanes write their tokens.
 __device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
                                                   uint32_t w1, uint32_t* list, uint32_t* n_list, uint32_t cap) {
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
     const bool two = u1 <= 0x7fffu;
-    const uint32_t L0 = u0 * 0x10001u, H0 = (u0 + w0 + 1u) * 0x10001u;
-    const uint32_t L1 = two ? u1 * 0x10001u : 0u, H1 = two ? (u1 + w1 + 1u) * 0x10001u : 0u;
+    const u16x2 L0 = static_cast<unsigned short>(u0), H0 = static_cast<unsigned short>(u0 + w0 + 1u);
+    const u16x2 L1 = static_cast<unsigned short>(two ? u1 : 0u), H1 = static_cast<unsigned short>(two ? u1 + w1 + 1u : 0u);
     uint32_t hits[kCacheRegs / 16];
     uint32_t mine = 0;
-#pragma unroll
-    for (int g = 0; g < kCacheRegs / 16; ++g) {
+    auto test16 = [&](int g, u16x2 lo, u16x2 hi) {  // bit k / 16 + k: low / high half of register 16 g + k lies in [lo, hi)
         uint32_t acc = 0;
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
-            const uint32_t y = cache[g * 16 + k] | 0x80008000u;
-            uint32_t r = (y - L0) ^ (y - H0);
-            if (two) r |= (y - L1) ^ (y - H1);
-            acc = (acc >> 1) | (r & 0x80008000u);  // register k: low half -> bit k, high half -> bit 16 + k
+            const u16x2 y = __builtin_bit_cast(u16x2, cache[g * 16 + k]);
+            const uint32_t r = __builtin_bit_cast(uint32_t, static_cast<u16x2>(y - lo)) ^ __builtin_bit_cast(uint32_t, static_cast<u16x2>(y - hi));
+            acc = (acc >> 1) | (r & 0x80008000u);
         }
+        return acc;
+    };
+#pragma unroll
+    for (int g = 0; g < kCacheRegs / 16; ++g) {
+        uint32_t acc = test16(g, L0, H0);
+        if (two) acc |= test16(g, L1, H1);  // uniform branch
         hits[g] = acc;
         mine += __popc(acc);
+        __builtin_amdgcn_sched_barrier(0);  // one group at a time: a wider scheduling window costs more registers than it hides
     }
     uint32_t inc = mine;  // inclusive prefix over the wave
 #pragma unroll
@@ -471,7 +483,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
     uint32_t n_touched = 0;  // distinct tokens the history and the bias list touch
     float m_adj = -INFINITY;  // largest adjusted logit among them
-    float m_rawt = -INFINITY; // largest raw logit among them
+    float m_near = -INFINITY; // largest untouched, allowed logit among the 128-bit vectors that hold them (single-sweep mode)
     if (!(inv_t > 0.f) || nh + nb > A.patch_cap) flags |= kBadParam;
     if (!(flags & kBadParam) && nh + nb > 0) {
         const int32_t* hist_ids = A.hist + h0;
@@ -553,9 +565,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const int32_t* bias_ids = A.bias_ids + b0;
         uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
         uint32_t* first = cnt + A.patch_cap;
+        float mu = -INFINITY;  // largest untouched, allowed logit among the vectors that hold touched tokens
         auto fetch4 = [&](const int32_t* ids, uint32_t n) {  // four independent gathers per thread and round
             for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
                 uint32_t id[4], bits[4], al[4];
+                uint4 vec[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t j = j0 + k * WS_BLOCK + t;
@@ -564,22 +578,42 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
-                    // slot of the token's vector = rank of the vector's first touched token
-                    const uint32_t vb = i & ~(per - 1u), tw = touched[i >> 5];
-                    const uint32_t rf = static_cast<uint32_t>(wprefix[i >> 5]) + __popc(tw & ((1u << (vb & 31u)) - 1u));
-                    if (rf < stage_cap) {
-                        const uint32_t* sv = reinterpret_cast<const uint32_t*>(stage + rf);
-                        bits[k] = rv.dtype == 0 ? sv[i & 3u] : (((i & 1u) ? sv[(i & 7u) >> 1] & 0xffff0000u : sv[(i & 7u) >> 1] << 16));
-                    } else {
-                        bits[k] = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
-                                                : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
-                    }
                     al[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
+                    if (rv.vec && i < (V / per) * per) {
+                        // the token's whole 128-bit vector: staged by the sweep under the rank of the vector's first
+                        // touched token, else fetched
+                        const uint32_t vb = i & ~(per - 1u), tw = touched[i >> 5];
+                        const uint32_t rf = static_cast<uint32_t>(wprefix[i >> 5]) + __popc(tw & ((1u << (vb & 31u)) - 1u));
+                        vec[k] = rf < stage_cap ? stage[rf] : static_cast<const uint4*>(rv.base)[i / per];
+                    } else {
+                        const uint32_t b = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
+                                                         : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
+                        vec[k] = make_uint4(b, b, b, b);
+                    }
                 }
 #pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (id[k] < V)
-                        pv[rank_of(rv, id[k])] = ((al[k] >> (id[k] & 31u)) & 1u) ? fmaxf(__uint_as_float(bits[k]), -INFINITY) : -INFINITY;
+                for (int k = 0; k < 4; ++k) {
+                    if (id[k] >= V) continue;
+                    const uint32_t i = id[k];
+                    const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
+                    const bool whole = rv.vec && i < (V / per) * per;
+                    if (!whole) bits[k] = w[0];
+                    else bits[k] = rv.dtype == 0 ? w[i & 3u] : ((i & 1u) ? w[(i & 7u) >> 1] & 0xffff0000u : w[(i & 7u) >> 1] << 16);
+                    pv[rank_of(rv, i)] = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits[k]), -INFINITY) : -INFINITY;
+                    if (FUSED && whole) {
+                        const uint32_t vb = i & ~(per - 1u);
+                        const uint32_t free_bits = (al[k] & ~touched[i >> 5]) >> (vb & 31u);  // allowed and untouched
+                        if (rv.dtype == 0) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float(w[e]));
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float((e & 1) ? w[e >> 1] & 0xffff0000u : w[e >> 1] << 16));
+                        }
+                    }
+                }
             }
         };
         fetch4(hist_ids, nh);
@@ -587,7 +621,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         __syncthreads();
         {
             const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
-            float ma = -INFINITY, mr = -INFINITY;
+            float ma = -INFINITY;
             for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
                 const uint32_t cw = cnt[r], c = cw & 0xfffffu;
                 const float raw = pv[r];
@@ -600,10 +634,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 pv[r] = x;
                 cnt[r] = __float_as_uint(raw);
                 ma = fmaxf(ma, x);
-                mr = fmaxf(mr, raw);
             }
             m_adj = block_max(ma, red_f);
-            m_rawt = block_max(mr, red_f);
+            m_near = block_max(mu, red_f);
         }
         if (FUSED) {
             for (uint32_t j = t; j < nh; j += WS_BLOCK) {
@@ -660,46 +693,16 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         gather_and_adjust(stage, swept ? stage_cap : 0u);
         WS_MARK(9);
         if (swept) {
-            m = block_max(m, red_f);  // over the raw row (allow mask applied), touched tokens included
+            m = block_max(m, red_f);  // over the vectors of the row that hold no touched token (allow mask applied)
             // touched tokens: out of the bin of the raw logit, into the bin of the adjusted one
             for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
                 const float t0 = bin_coord(aq, c64, praw[r]), t1 = bin_coord(aq, c64, pv[r]);
                 atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
                 atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
             }
-            bool ok = true;
-            if (n_touched && m_rawt >= m) {
-                // the largest raw logit belongs to a touched token: the largest untouched one sits in the first
-                // non-empty bin (or further down, and then an adjusted touched token of that bin is the maximum)
-                __syncthreads();
-                uint32_t fb = kBins;
-#pragma unroll
-                for (int j = kPT - 1; j >= 0; --j)
-                    if (hist[kPT * t + j] >> kCountShift) fb = kPT * t + j;
-                fb = block_min(fb, red_u);
-                float mu = -INFINITY;
-                ok = fb < kBins - 1;
-                if constexpr (FUSED) {
-                    if (ok) {
-                        uint32_t* list = reinterpret_cast<uint32_t*>(emass);  // free until pass 3
-                        if (t == 0) s_u[4] = 0;
-                        __syncthreads();
-                        gather_from_cache(rv.dtype, cache, fb, 0u, 0xffff0000u, 0u, list, &s_u[4], 2u * kCap);
-                        __syncthreads();
-                        const uint32_t n_hit = s_u[4];
-                        ok = n_hit <= 2u * kCap;
-                        if (ok)
-                            for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
-                                const uint32_t i = list[k];
-                                if (!is_touched(rv, i)) mu = fmaxf(mu, raw_logit(rv, i));
-                            }
-                    }
-                }
-                m = block_max(mu, red_f);
-            }
-            m = fmaxf(m, m_adj);
+            m = fmaxf(fmaxf(m, m_near), m_adj);
             // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
-            cached = ok && m <= anchor && (anchor - m) * c64 <= 1024.f;
+            cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
         }
         if (!cached) {
             m = -INFINITY;
@@ -747,10 +750,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double to_max = exp(lift);
 
     WS_MARK(2);
-    // scan: thread t owns kPT consecutive bins (bin 0 = nearest the anchor)
-    uint32_t c[kPT], cx[kPT];
-    double ms[kPT], mx[kPT];
+    // scan: thread t owns kPT consecutive bins (bin 0 = nearest the anchor). The exclusive prefixes go back to LDS -
+    // masses pm[0..4096] over the histogram itself, counts pc[0..4096] behind them - so that the lookups below hold
+    // nothing in registers between barriers (the bin cache of the single-sweep mode needs them)
+    double* pm = reinterpret_cast<double*>(lds);                       // 4097 doubles
+    uint32_t* pc = reinterpret_cast<uint32_t*>(lds + 32768 + 16);      // 4097 counts
     {
+        uint32_t c[kPT];
+        double ms[kPT];
         uint32_t csum = 0;
         double msum = 0;
 #pragma unroll
@@ -768,39 +775,48 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint32_t ctot;
         double mtot;
         uint32_t cb = block_excl_scan(csum, red_u, &ctot);
-        double mb = block_excl_scan(msum, red_d, &mtot);
+        double mb = block_excl_scan(msum, red_d, &mtot);  // its barriers separate the reads of hist above from the writes below
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
-            cx[j] = cb;
-            mx[j] = mb;
+            pc[kPT * t + j] = cb;
+            pm[kPT * t + j] = mb;
             cb += c[j];
             mb += ms[j];
         }
-        if (t == 0) s_d[0] = mtot;
+        if (t == WS_BLOCK - 1) {
+            pc[kBins] = ctot;
+            pm[kBins] = mtot;
+        }
     }
-    __syncthreads();  // the histogram is dead from here on: its LDS becomes the key buffer
-    const double Z = s_d[0];
+    __syncthreads();  // the histogram is gone; after the lookups its LDS becomes the key buffer
+    const double Z = pm[kBins];
     const double Zf = static_cast<double>(static_cast<float>(Z));  // Sampler::sum is a float (src/sampling/sampler.h:38)
 
-    // lookups in the scanned histogram; every call site is reached by the whole block
+    // lookups in the scanned histogram; every call site is reached by the whole block. A bin's mass interval is
+    // [pm[b], pm[b + 1]), its rank interval [pc[b], pc[b + 1])
+    auto bin_sel = [&](int b) {
+        const uint32_t cx = pc[b];
+        const double mx = pm[b];
+        return BinSel{b, cx, pc[b + 1] - cx, mx, pm[b + 1] - mx};
+    };
     auto find_count = [&](uint32_t n, int slot) {  // bin holding the element of rank n - 1
 #pragma unroll
-        for (int j = 0; j < kPT; ++j)
-            if (cx[j] < n && cx[j] + c[j] >= n) sel[slot] = BinSel{static_cast<int>(kPT * t + j), cx[j], c[j], mx[j], ms[j]};
+        for (int j = 0; j < kPT; ++j) {
+            const int b = kPT * t + j;
+            if (pc[b] < n && pc[b + 1] >= n) sel[slot] = bin_sel(b);
+        }
     };
-    auto find_mass = [&](double X, bool strict, int slot) {  // first bin whose inclusive mass prefix reaches X
+    auto find_mass = [&](double X, bool strict, int slot) {  // first non-empty bin whose inclusive mass prefix reaches X
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
-            const double inc = mx[j] + ms[j];
-            const bool hit = strict ? (inc > X && !(mx[j] > X)) : (inc >= X && !(mx[j] >= X));
-            if (hit && ms[j] > 0.0) sel[slot] = BinSel{static_cast<int>(kPT * t + j), cx[j], c[j], mx[j], ms[j]};
+            const int b = kPT * t + j;
+            const double lo = pm[b], hi = pm[b + 1];
+            const bool hit = strict ? (hi > X && !(lo > X)) : (hi >= X && !(lo >= X));
+            if (hit && hi > lo && pc[b + 1] > pc[b]) sel[slot] = bin_sel(b);
         }
     };
     auto fetch_bin = [&](int b, int slot) {
-        if (b >= 0 && static_cast<uint32_t>(b / kPT) == t) {
-            const int j = b % kPT;
-            sel[slot] = BinSel{b, cx[j], c[j], mx[j], ms[j]};
-        }
+        if (b >= 0 && static_cast<uint32_t>(b / kPT) == t) sel[slot] = bin_sel(b);
     };
 
     uint32_t n1 = (top_k > 0 && top_k < V) ? top_k : V;
@@ -922,7 +938,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     fetch_bin(r0hi, 1);
     fetch_bin(r1hi >= r1lo ? r1lo : -1, 2);
     fetch_bin(r1hi >= r1lo ? r1hi : -1, 3);
-    if (t == 0) s_cnt = 0;
+    if (t == 0) s_cnt = s_u[5] = 0;
     __syncthreads();
     const uint32_t c0base = sel[0].cx, n_r0 = sel[1].cx + sel[1].c - sel[0].cx;
     const double m0base = sel[0].mx;
@@ -953,11 +969,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = static_cast<uint32_t>(r0hi - r0lo);
         const uint32_t u1 = static_cast<uint32_t>(r1lo), w1 = r1hi >= r1lo ? static_cast<uint32_t>(r1hi - r1lo) : 0u;
         const bool two = r1hi >= r1lo;
+        const uint32_t u1r = two ? u1 : 0xffff0000u;  // an empty second range matches no bin
+        // candidates of range 0 fill keys[0, n_r0), those of range 1 keys[n_r0, n_list): every key of range 0 ranks
+        // before every key of range 1, so the sort below never compares across the two
         auto push = [&](uint32_t i, float x) {
-            const uint32_t slot = atomicAdd(&s_cnt, 1u);
+            const bool in1 = bin_of(aq, c64, x) - u1r <= w1;
+            const uint32_t slot = in1 ? n_r0 + atomicAdd(&s_u[5], 1u) : atomicAdd(&s_cnt, 1u);
             if (slot < kCap) keys[slot] = key64(x, i);
         };
-        const uint32_t u1r = two ? u1 : 0xffff0000u;  // an empty second range matches no bin
         auto in_ranges = [&](float x) {
             const uint32_t b = bin_of(aq, c64, x);
             return b - u0 <= w0 || b - u1r <= w1;
@@ -971,6 +990,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 __syncthreads();
                 gather_from_cache(rv.dtype, cache, u0, w0, u1r, w1, list, &s_u[4], 2u * kCap);
                 __syncthreads();
+                WS_MARK(10);
                 const uint32_t n_hit = min(s_u[4], 2u * kCap);
                 if (s_u[4] > 2u * kCap) flags |= kOverflow;
                 for (uint32_t k0 = 0; k0 < n_hit; k0 += 4u * WS_BLOCK) {
@@ -987,12 +1007,16 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     for (int q = 0; q < 4; ++q) xs[q] = keep[q] ? raw_logit(rv, idx[q]) : 0.f;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        // one slot reservation per wave: lanes that keep their hit take consecutive slots
-                        const uint64_t mask = __ballot(keep[q]);
-                        uint32_t base = 0;
-                        if (lane_id() == 0 && mask) base = atomicAdd(&s_cnt, static_cast<uint32_t>(__popcll(mask)));
-                        base = __shfl(base, 0);
-                        const uint32_t slot = base + static_cast<uint32_t>(__popcll(mask & ((1ull << lane_id()) - 1ull)));
+                        // one slot reservation per wave and range: lanes that keep their hit take consecutive slots
+                        const bool in1 = keep[q] && bin_of(aq, c64, xs[q]) - u1r <= w1;
+                        const uint64_t m1 = __ballot(in1), m0 = __ballot(keep[q] && !in1);
+                        uint32_t b0 = 0, b1 = 0;
+                        if (lane_id() == 0 && m0) b0 = atomicAdd(&s_cnt, static_cast<uint32_t>(__popcll(m0)));
+                        if (lane_id() == 0 && m1) b1 = atomicAdd(&s_u[5], static_cast<uint32_t>(__popcll(m1)));
+                        const uint64_t below = (1ull << lane_id()) - 1ull;
+                        const uint32_t s0 = __shfl(b0, 0) + static_cast<uint32_t>(__popcll(m0 & below));  // every lane takes part
+                        const uint32_t s1 = n_r0 + __shfl(b1, 0) + static_cast<uint32_t>(__popcll(m1 & below));
+                        const uint32_t slot = in1 ? s1 : s0;
                         if (keep[q] && slot < kCap) keys[slot] = key64(xs[q], idx[q]);
                     }
                 }
@@ -1034,46 +1058,123 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         return;
     }
     WS_MARK(4);
-    uint32_t P = 64;
-    while (P < n_list) P <<= 1;
-    for (uint32_t i = n_list + t; i < P; i += WS_BLOCK) keys[i] = 0ull;
-    __syncthreads();
-    sort_desc(keys, P);
+#ifdef WS_PHASE_TIMERS
+    if (t == 0 && A.kept_logits) {
+        float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
+        dbg[11] = static_cast<float>(n_r0);
+        dbg[12] = static_cast<float>(n_r1);
+        dbg[13] = static_cast<float>(r0hi - r0lo + 1);
+        dbg[14] = static_cast<float>(r1hi >= r1lo ? r1hi - r1lo + 1 : 0);
+    }
+#endif
+    constexpr int kMergeCh = 3;  // keys per thread the merge sort takes
+    if (n_list <= kMergeCh * WS_BLOCK) {
+        // Few candidates (the usual case): one or two per thread. Each wave ranks 64 keys among themselves by counting
+        // and writes them out as a sorted run; then every key finds its rank in each other run by binary search; the
+        // sum of the ranks is its place. Three barriers instead of one per bitonic stage. Slots past n_list hold
+        // key 0, which sorts last (equal keys keep their slot order).
+        uint64_t* runs = reinterpret_cast<uint64_t*>(emass);  // idle until the masses are written below
+        const uint32_t nruns = (n_list + 63u) >> 6;
+        uint64_t key[kMergeCh];
+        uint32_t place[kMergeCh];
+#pragma unroll
+        for (int q = 0; q < kMergeCh; ++q) {
+            const uint32_t i = q * WS_BLOCK + t, run_id = i >> 6;
+            key[q] = i < n_list ? keys[i] : 0ull;
+            place[q] = 0;
+            if (run_id < nruns) {  // uniform per wave
+                const uint32_t klo = static_cast<uint32_t>(key[q]), khi = static_cast<uint32_t>(key[q] >> 32);
+#pragma unroll
+                for (int j = 0; j < 64; ++j) {
+                    const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(khi, j))) << 32) |
+                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(klo, j));
+                    place[q] += (other > key[q] || (other == key[q] && j < lane_id())) ? 1u : 0u;
+                }
+                runs[(run_id << 6) + place[q]] = key[q];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kMergeCh; ++q) {
+            const uint32_t i = q * WS_BLOCK + t, run_id = i >> 6;
+            if (run_id >= nruns) continue;
+            // only the runs that hold keys of this key's own range need a search: slots before them hold larger keys
+            const uint32_t v_a = i < n_r0 ? 0u : n_r0 >> 6;
+            const uint32_t v_b = i < n_r0 ? (n_r0 - 1u) >> 6 : nruns - 1u;
+            place[q] += v_a << 6;
+            // four runs at a time, so that four binary searches wait for LDS together (a search of the own run,
+            // or of a run past the last, is carried along and dropped)
+            for (uint32_t v0 = v_a; v0 <= v_b; v0 += 4u) {
+                uint32_t cnt[4] = {0u, 0u, 0u, 0u};
+                const uint64_t* run[4];
+                bool tie[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t v = min(v0 + r, v_b);
+                    run[r] = runs + (v << 6);  // descending
+                    tie[r] = v < run_id;       // equal keys: the earlier run goes first
+                }
+                // members of a run ranked before this key: greater, or equal in an earlier run
+#pragma unroll
+                for (uint32_t sdx = 32; sdx >= 1; sdx >>= 1) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint64_t o = run[r][cnt[r] + sdx - 1u];
+                        if (o > key[q] || (o == key[q] && tie[r])) cnt[r] += sdx;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint64_t o = run[r][cnt[r]];
+                    if (o > key[q] || (o == key[q] && tie[r])) cnt[r] += 1u;
+                    if (v0 + r <= v_b && v0 + r != run_id) place[q] += cnt[r];
+                }
+            }
+        }
+        __syncthreads();  // every read of keys[] above is done
+#pragma unroll
+        for (int q = 0; q < kMergeCh; ++q)
+            if (((q * WS_BLOCK + t) >> 6) < nruns) keys[place[q]] = key[q];
+        __syncthreads();
+    } else {
+        uint32_t P = 64;
+        while (P < n_list) P <<= 1;
+        for (uint32_t i = n_list + t; i < P; i += WS_BLOCK) keys[i] = 0ull;
+        __syncthreads();
+        sort_desc(keys, P);
+    }
     WS_MARK(5);
 
-    // thread t owns kPT consecutive sorted entries
+    // sorted entry j * WS_BLOCK + t belongs to thread t: with the usual few hundred candidates every thread has one
     double e[kPT], inc[kPT], exc[kPT];
     uint32_t pos[kPT];
     bool live[kPT];
     {
-        double esum = 0;
+        double carry = 0;
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
-            const uint32_t i = kPT * t + j;
+            const uint32_t i = j * WS_BLOCK + t;
             live[j] = i < n_list;
-            e[j] = 0;
-            if (live[j]) {
-                const float x = unkey32(static_cast<uint32_t>(keys[i] >> 32));
-                const float d = __fsub_rn(m, x);
-                e[j] = exp(-(static_cast<double>(d) * static_cast<double>(inv_t)));
+            e[j] = exc[j] = inc[j] = 0;
+            if (static_cast<uint32_t>(j) * WS_BLOCK < n_list) {  // uniform
+                if (live[j]) {
+                    const float x = unkey32(static_cast<uint32_t>(keys[i] >> 32));
+                    const float d = __fsub_rn(m, x);
+                    e[j] = exp(-(static_cast<double>(d) * static_cast<double>(inv_t)));
+                }
+                double tot;
+                exc[j] = carry + block_excl_scan(e[j], red_d, &tot);
+                inc[j] = exc[j] + e[j];
+                carry += tot;
+                if (live[j] && i + 1 == n_r0) s_d[1] = inc[j];
             }
-            esum += e[j];
-        }
-        double etot;
-        double run = block_excl_scan(esum, red_d, &etot);
-        // masses of range 1 restart at its base: subtract the running sum at the end of range 0
-#pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            exc[j] = run;
-            run += e[j];
-            inc[j] = run;
-            if (kPT * t + j + 1 == n_r0) s_d[1] = run;
         }
         __syncthreads();
+        // masses of range 1 restart at its base: subtract the running sum at the end of range 0
         const double at_r0_end = n_r0 ? s_d[1] : 0.0;
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
-            const uint32_t i = kPT * t + j;
+            const uint32_t i = j * WS_BLOCK + t;
             if (i < n_r0) {
                 pos[j] = c0base + i;
                 exc[j] += m0base;
@@ -1164,7 +1265,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     for (int j = 0; j < kPT; ++j)
         if (live[j] && pos[j] == n3 - 1) {
             s_d[4] = inc[j];
-            s_key = keys[kPT * t + j];
+            s_key = keys[j * WS_BLOCK + t];
             s_u[1] = 1;
         }
     __syncthreads();
@@ -1196,12 +1297,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     for (int j = 0; j < kPT; ++j) {
         if (!live[j] || pos[j] >= n3) continue;
         if (inc[j] > target && !(exc[j] > target) && e[j] > 0.0) {
-            s_u[2] = 0xffffffffu - static_cast<uint32_t>(keys[kPT * t + j]);
+            s_u[2] = 0xffffffffu - static_cast<uint32_t>(keys[j * WS_BLOCK + t]);
             s_d[5] = e[j];
             s_d[6] = fmin(inc[j] - target, pos[j] > 0 ? target - exc[j] : 1e300) / Zk;
         }
         if (pos[j] == n3 - 1) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
-            s_u[3] = 0xffffffffu - static_cast<uint32_t>(keys[kPT * t + j]);
+            s_u[3] = 0xffffffffu - static_cast<uint32_t>(keys[j * WS_BLOCK + t]);
             s_d[7] = e[j];
         }
     }
