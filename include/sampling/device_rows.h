@@ -1,0 +1,69 @@
+// RowSource over logits that live in MI355X memory. prepareRow runs the fused device sampler on the row (penalties,
+// bias, temperature, top-k / top-p / min-p, all in one launch) and brings back only the kept candidates, already
+// filtered: s.closed is true and the list is what filterCands would have left. Rows the device flags as unresolved
+// (more candidates tied at a cut than it handles, or no filter at all) go the reference's way instead: device top-k
+// of 256, then 16384, then the full row, each through filterCands (src/server/engine_sampling.cpp:51-84).
+//
+// Not in the reference: it plays the role of the engine's SampleBuffers (src/server/engine_sampling.h:20-73).
+#pragma once
+
+#include "sampling/sampler.h"
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace whirl::sampling {
+
+// a failed device call: op names the entry point, code is its return value (hipError_t when positive, WS_E_* when negative)
+struct DeviceError : std::runtime_error {
+    DeviceError(const char* op_, int code_, const std::string& what_) : std::runtime_error(what_), op(op_), code(code_) {}
+    const char* op;
+    int code;
+};
+
+// optional per-row penalties and bias, all host arrays (copied to the device per call)
+struct RowAdjust {
+    const std::int32_t* history = nullptr;  // token ids seen so far
+    std::uint32_t n_history = 0;
+    float repetition = 1.f, presence = 0.f, frequency = 0.f;
+    const std::int32_t* bias_ids = nullptr;
+    const float* bias_vals = nullptr;
+    std::uint32_t n_bias = 0;
+};
+
+class DeviceRows final : public RowSource {
+public:
+    // d_logits: device pointer to [rows][n_vocab] floats; stream: hipStream_t (nullptr = the null stream)
+    DeviceRows(const float* d_logits, std::uint32_t rows, std::uint32_t n_vocab, void* stream = nullptr);
+    ~DeviceRows() override;
+    DeviceRows(const DeviceRows&) = delete;
+    DeviceRows& operator=(const DeviceRows&) = delete;
+
+    void setAdjust(const RowAdjust& a) { adj_ = a; }  // applies to the rows prepared from now on
+
+    void prepareRow(Sampler& s, std::uint32_t r) override;
+    const float* loadFullRow(std::uint32_t gr) override;
+    float logitAt(std::uint32_t gr, std::uint32_t t) override;
+    std::uint32_t nVocab() const override { return vocab_; }
+    std::uint8_t* inCands() override { return marks_.data(); }
+
+    std::uint32_t lastFlags() const { return last_flags_; }  // WS_FLAG_* of the last prepared row
+
+private:
+    void escalate(Sampler& s, std::uint32_t gr);
+    struct Dev;  // device scratch
+    const float* logits_;
+    std::uint32_t rows_, vocab_;
+    void* stream_;
+    RowAdjust adj_;
+    Dev* dev_;
+    std::vector<float> row_host_;
+    std::vector<std::uint8_t> marks_;
+    std::uint32_t last_flags_ = 0;
+    static constexpr std::uint32_t kNoRow = 0xffffffffu;
+    std::uint32_t adjusted_row_ = kNoRow;  // row whose penalised copy row_host_ holds (after an escalation)
+};
+
+}  // namespace whirl::sampling

@@ -1,0 +1,49 @@
+/* C entry point of libwhirl_sampling_host.so, the C++ host layer (include/sampling/*.h, include/whirl/*.h) over the
+ * device library. No counterpart in the reference, whose host sampler is called from C++ only; it exists for language
+ * bindings and tests: one token per row the way the engine's decode loop obtains it (RowSource::prepareRow on the
+ * device-backed sampling::DeviceRows, set the output index, sampling::sampleRow).
+ */
+#ifndef WHIRL_SAMPLING_HOST_H
+#define WHIRL_SAMPLING_HOST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Everything except d_logits is host memory; per-row arrays have `rows` entries, NULL means the stated default.
+ * History and bias lists are concatenated with rows + 1 offsets, as in ws_batch. */
+typedef struct wsh_rows {
+    const float* d_logits; /* device, [rows][vocab] */
+    uint32_t rows, vocab;
+    const float* inv_t;
+    const uint32_t* top_k;  /* NULL: off */
+    const double* top_p;    /* NULL: off */
+    const double* min_p;    /* NULL: off */
+    const uint64_t* seed;
+    const uint64_t* pos_idx; /* output token index (Sampler::pos_idx, src/sampling/sampler.h:33) */
+    const int32_t* hist;     /* NULL: no penalties */
+    const uint32_t* hist_off;
+    const float* rep;
+    const float* pres;
+    const float* freq;
+    const int32_t* bias_ids; /* NULL: no bias */
+    const float* bias_vals;
+    const uint32_t* bias_off;
+    int32_t race;            /* non-zero: exponential-race draw (Sampler::race) instead of inverse CDF */
+    int32_t* token;          /* out */
+    double* prob;            /* out (may be NULL): probability of the token on the kept set */
+    uint32_t* n_kept;        /* out (may be NULL): Sampler::n */
+    uint32_t* flags;         /* out (may be NULL): WS_FLAG_* the device reported */
+    int32_t* closed;         /* out (may be NULL): Sampler::closed */
+} wsh_rows;
+
+/* 0 = ok, otherwise the code of the failing call (hipError_t > 0, WS_E_* < 0); text from wsh_last_error(). Synchronous. */
+int wsh_sample_rows(void* stream, const wsh_rows* a);
+const char* wsh_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -50,3 +50,21 @@ def test_host_side_argument_checks():
     assert lib.ws_sample_batch(None, C.byref(b)) == -3  # rank tables would not fit the LDS
     b.vocab = 1 << 20
     assert lib.ws_sample_batch(None, C.byref(b)) == -1
+
+
+def test_host_layer_exports_its_c_entry_points():
+    """libwhirl_sampling_host.so (the C++ host API) is built and exports what include/whirl_sampling_host.h declares,
+    plus the C++ symbols of the reference's host interface (whirl::sampling::filterCands and friends)."""
+    m = gpu_cases.pkg()
+    hdr = open(os.path.join(ROOT, "include", "whirl_sampling_host.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(wsh_[a-z_0-9]+)\s*\(", hdr))
+    assert declared == set(m.HOST_ABI), declared ^ set(m.HOST_ABI)
+    blob = open(m.HOST_LIB_PATH, "rb").read()
+    for name in declared:
+        assert name.encode() in blob, name
+    for mangled in (b"_ZN5whirl8sampling11filterCandsERNS0_7SamplerEmb", b"_ZN5whirl8sampling9sampleRowERNS0_9RowSourceERNS0_7SamplerESt8optionalIjEd",
+                    b"_ZN5whirl8sampling10sampleRaceERNS0_9RowSourceERNS0_7SamplerE", b"_ZN5whirl8sampling6probOfERNS0_9RowSourceERNS0_7SamplerEj",
+                    b"_ZNK5whirl8sampling8Acceptor6greedyE", b"_ZNK5whirl8sampling8Acceptor6sampleE", b"_ZN5whirl4spec9draftDistE",
+                    b"_ZN5whirl8sampling10DeviceRows10prepareRowERNS0_7SamplerEj"):
+        assert mangled in blob, mangled

@@ -1,0 +1,58 @@
+"""GPU: the C++ host layer (sampling::DeviceRows as RowSource + sampling::sampleRow) against the CPU oracle.
+The rows go through RowSource::prepareRow exactly as the engine's decode loop calls it; the oracle is the reference's
+own escalation (256 / 16384 / full row) + filterCands + inverse-CDF draw with the splitmix uniform."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_cases as gc
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(c, rows):
+    m = gc.pkg()
+    d = gc.upload(c)
+    nh = c["hist"].shape[1] if c["hist"] is not None else 0
+    nb = c["bias_ids"].shape[1] if c["bias_ids"] is not None else 0
+    R = c["rows"]
+    out = m.host_sample_rows(
+        d["logits"], c["inv_t"], c["seed"], c["step"], top_k=c["top_k"], top_p=c["top_p"], min_p=c["min_p"],
+        hist=c["hist"], hist_off=np.arange(R + 1, dtype=np.uint32) * nh if nh else None, rep=c["rep"], pres=c["pres"], freq=c["freq"],
+        bias_ids=c["bias_ids"], bias_vals=c["bias_vals"], bias_off=np.arange(R + 1, dtype=np.uint32) * nb if nb else None)
+    near = 0
+    for r in rows:
+        o, kept, _ = gc.oracle_row(c, r, 0)  # rng 0: the reference's uniform(seed, pos_idx)
+        close = min(o.margin, o.margin_top_p, o.margin_min_p) < 1e-6
+        if out["token"][r] != o.token or out["n_kept"][r] != o.n_kept:
+            assert close, (r, out["token"][r], o.token, out["n_kept"][r], o.n_kept, o.margin, o.margin_top_p, o.margin_min_p)
+            near += 1
+            continue
+        assert out["closed"][r] == o.closed, r
+        assert abs(out["prob"][r] - o.prob) <= 1e-6 * o.prob, (r, out["prob"][r], o.prob)
+    return near, out
+
+
+def test_host_rows_small_vocab_with_penalties_and_bias():
+    c = gc.make_cfg2(rows=12, V=32000, n_hist=300, n_bias=20)
+    near, _ = _run(c, range(12))
+    assert near <= 1
+
+
+def test_host_rows_full_vocab():
+    c = gc.make_cfg2(rows=6)
+    near, _ = _run(c, range(6))
+    assert near <= 1
+
+
+def test_host_rows_open_row_takes_the_reference_route():
+    """No filter at all: the device reports an open row and the host layer walks the reference's own path (top-256 in
+    sorted order, then the tail in id order), so even these tokens match."""
+    m = gc.pkg()
+    c = gc.make_cfg2(rows=4, V=20000, n_hist=0, n_bias=0)
+    c["top_k"][:] = 0
+    c["top_p"][:] = 1.0
+    c["min_p"][:] = 0.0
+    near, out = _run(c, range(4))
+    assert near == 0
+    assert all(out["flags"] & m.FLAG_OPEN) and not any(out["closed"])

@@ -9,7 +9,7 @@ import wo
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 FIX = json.load(open(os.path.join(HERE, "golden", "acceptor_cases.json")))
-LIBS = ["oracle"] + (["ref"] if wo.load("ref") is not None else [])
+LIBS = ["oracle", "host"] + (["ref"] if wo.load("ref") is not None else [])
 
 
 @pytest.mark.parametrize("which", LIBS)
@@ -52,8 +52,9 @@ def test_random_cases_fixture():
     assert accepted > 1000
 
 
-@pytest.mark.skipif(wo.load("ref") is None, reason="oracle/_ref not built (needs the reference tree)")
-def test_random_cases_live_reference():
-    ref, lib = wo.load("ref"), wo.load("oracle")
+@pytest.mark.parametrize("other", [w for w in LIBS if w != "oracle"])
+def test_random_cases_against_other_implementations(other):
+    """The oracle against the product's host API (always) and the reference's own code (where it is built)."""
+    ref, lib = wo.load(other), wo.load("oracle")
     for c in acase.random_cases(600):
         assert acase.run(lib, c) == acase.run(ref, c), c

@@ -8,7 +8,7 @@ import pytest
 
 import wo
 
-LIBS = ["oracle"] + (["ref"] if wo.load("ref") is not None else [])
+LIBS = ["oracle", "host"] + (["ref"] if wo.load("ref") is not None else [])
 
 
 def cands_of(logits):
@@ -208,11 +208,11 @@ def test_draw_is_first_crossing_and_follows_p():
     assert chi < crit
 
 
-@pytest.mark.skipif(wo.load("ref") is None, reason="oracle/_ref not built (needs the reference tree)")
-def test_prepare_and_draws_match_compiled_reference():
+@pytest.mark.parametrize("other", [w for w in LIBS if w != "oracle"])
+def test_prepare_and_draws_match_other_implementations(other):
     """Random rows through escalation (ks 4 / kb 16 and the engine's 256 / 16384), inverse CDF, race, residual draw
-    and probOf: bit-identical to the reference's own code."""
-    ref, lib = wo.load("ref"), wo.load("oracle")
+    and probOf: the oracle is bit-identical to the product's host API and, where it is built, the reference's own code."""
+    ref, lib = wo.load(other), wo.load("oracle")
     rng = np.random.default_rng(5)
     for it in range(400):
         big = it % 40 == 0

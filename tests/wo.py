@@ -101,7 +101,10 @@ _cache = {}
 
 
 def lib_path(which):
-    return os.path.join(ROOT, "oracle", "liboracle.so" if which == "oracle" else os.path.join("_ref", "libwhirl_ref.so"))
+    """oracle: the CPU restatement; ref: the reference's own sources (built only where the reference tree is mounted);
+    host: the product's C++ host API (whirl-llm_amd/host) behind the same C symbols."""
+    rel = {"oracle": "liboracle.so", "ref": os.path.join("_ref", "libwhirl_ref.so"), "host": os.path.join("_host", "libwhirl_hostapi.so")}
+    return os.path.join(ROOT, "oracle", rel[which])
 
 
 def load(which="oracle"):

@@ -253,3 +253,69 @@ def spec_verify_classic(p, q, draft, seed, step0, rng=RNG_PHILOX, tol=0.0):
                    tol)
     check(lib().ws_spec_verify_classic(_stream(), C.byref(v)), "ws_spec_verify_classic")
     return nacc, out, flags
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the C++ host layer (libwhirl_sampling_host.so) through its C entry point, include/whirl_sampling_host.h
+HOST_LIB_PATH = os.path.join(HERE, "libwhirl_sampling_host.so")
+
+
+class HostRows(C.Structure):
+    """wsh_rows of include/whirl_sampling_host.h."""
+    _fields_ = [("d_logits", C.c_void_p), ("rows", C.c_uint32), ("vocab", C.c_uint32), ("inv_t", C.c_void_p), ("top_k", C.c_void_p),
+                ("top_p", C.c_void_p), ("min_p", C.c_void_p), ("seed", C.c_void_p), ("pos_idx", C.c_void_p), ("hist", C.c_void_p),
+                ("hist_off", C.c_void_p), ("rep", C.c_void_p), ("pres", C.c_void_p), ("freq", C.c_void_p), ("bias_ids", C.c_void_p),
+                ("bias_vals", C.c_void_p), ("bias_off", C.c_void_p), ("race", C.c_int32), ("token", C.c_void_p), ("prob", C.c_void_p),
+                ("n_kept", C.c_void_p), ("flags", C.c_void_p), ("closed", C.c_void_p)]
+
+
+HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]), "wsh_last_error": (C.c_char_p, [])}
+_host_lib = None
+
+
+def host_lib():
+    """The loaded host-layer library; raises when it was not built."""
+    global _host_lib
+    if _host_lib is None:
+        lib()  # the device library first: the host layer links against it
+        if not os.path.exists(HOST_LIB_PATH):
+            raise WsError(f"{HOST_LIB_PATH} is missing: run `python whirl-llm_amd/build.py` (or __graft_entry__.build())")
+        handle = C.CDLL(HOST_LIB_PATH)
+        for name, (res, args) in HOST_ABI.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _host_lib = handle
+    return _host_lib
+
+
+def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p=None, hist=None, hist_off=None, rep=None, pres=None,
+                     freq=None, bias_ids=None, bias_vals=None, bias_off=None, race=False):
+    """One token per row through the C++ host API (sampling::DeviceRows + sampling::sampleRow). logits: [rows, vocab]
+    float32 device tensor; everything else numpy arrays on the host. Returns a dict of numpy arrays
+    (token, prob, n_kept, flags, closed)."""
+    import numpy as np
+    _dev_f32(logits)
+    rows, vocab = logits.shape
+    keep = []
+
+    def h(a, dt):
+        if a is None:
+            return None
+        a = np.ascontiguousarray(a, dtype=dt)
+        keep.append(a)
+        return a.ctypes.data_as(C.c_void_p)
+
+    out = dict(token=np.zeros(rows, np.int32), prob=np.zeros(rows, np.float64), n_kept=np.zeros(rows, np.uint32),
+               flags=np.zeros(rows, np.uint32), closed=np.zeros(rows, np.int32))
+    a = HostRows(d_logits=_p(logits), rows=rows, vocab=vocab, inv_t=h(inv_t, np.float32), top_k=h(top_k, np.uint32),
+                 top_p=h(top_p, np.float64), min_p=h(min_p, np.float64), seed=h(seed, np.uint64), pos_idx=h(pos_idx, np.uint64),
+                 hist=h(hist, np.int32), hist_off=h(hist_off, np.uint32), rep=h(rep, np.float32), pres=h(pres, np.float32),
+                 freq=h(freq, np.float32), bias_ids=h(bias_ids, np.int32), bias_vals=h(bias_vals, np.float32),
+                 bias_off=h(bias_off, np.uint32), race=int(race), token=out["token"].ctypes.data_as(C.c_void_p),
+                 prob=out["prob"].ctypes.data_as(C.c_void_p), n_kept=out["n_kept"].ctypes.data_as(C.c_void_p),
+                 flags=out["flags"].ctypes.data_as(C.c_void_p), closed=out["closed"].ctypes.data_as(C.c_void_p))
+    rc = host_lib().wsh_sample_rows(_stream(), C.byref(a))
+    if rc != 0:
+        raise WsError(f"wsh_sample_rows: {host_lib().wsh_last_error().decode()} ({rc})")
+    return out

@@ -2,6 +2,7 @@
 
   libwhirl_sampling_hip.so   the C-ABI library (include/whirl_sampling_abi.h)
   whirl_sampling_gfx950.co   the code object alone, for callers that resolve kernels by name (hipModuleGetFunction)
+  libwhirl_sampling_host.so  the C++ host API (include/sampling/*.h, include/whirl/*.h) over the C-ABI library
 
 Usage: python whirl-llm_amd/build.py
 """
@@ -27,14 +28,25 @@ def run(cmd):
     return err
 
 
+HOST_SRCS = [os.path.join(HERE, "host", f) for f in ("sampler.cpp", "acceptor.cpp", "spec_sample.cpp", "device_rows.cpp", "host_c_api.cpp")]
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+
+
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     so = os.path.join(HERE, "libwhirl_sampling_hip.so")
     co = os.path.join(HERE, "whirl_sampling_gfx950.co")
+    host = os.path.join(HERE, "libwhirl_sampling_host.so")
     run([hipcc, *FLAGS, "-fPIC", "-shared", "-o", so, SRC, SRC_FUSED])
     run([hipcc, *FLAGS, "--genco", "-o", co, SRC])
+    # host layer: plain C++20, no device code; -ffp-contract=off keeps the float arithmetic of the penalties unfused
+    run([os.environ.get("CXX", "g++"), "-std=c++20", "-O2", "-fPIC", "-shared", "-ffp-contract=off", "-Wall", "-Wextra",
+         "-D__HIP_PLATFORM_AMD__", "-I" + INCLUDE, "-I" + os.path.join(rocm, "include"), "-o", host, *HOST_SRCS,
+         "-L" + HERE, "-lwhirl_sampling_hip", "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN",
+         "-Wl,-rpath," + os.path.join(rocm, "lib")])
     if verbose:
-        print("built", so, "and", co)
+        print("built", so, "and", co, "and", host)
     return so, co
 
 

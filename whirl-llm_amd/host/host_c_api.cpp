@@ -1,0 +1,72 @@
+// A small C entry point over the C++ host API, for language bindings and tests that cannot call C++ classes:
+// sample one token per row through sampling::DeviceRows + sampling::sampleRow, the way the engine's decode loop does
+// (prepareRow, set the output index, draw).
+#include "sampling/device_rows.h"
+#include "sampling/sampler.h"
+#include "whirl_sampling_abi.h"
+#include "whirl_sampling_host.h"
+
+#include <cstdint>
+#include <cstdio>
+#include <exception>
+#include <vector>
+
+namespace ws = whirl::sampling;
+
+// 0 = ok; otherwise the failing call's code (message through wsh_last_error)
+static thread_local char g_err[256];
+
+extern "C" {
+
+const char* wsh_last_error(void) { return g_err; }
+
+int wsh_sample_rows(void* stream, const wsh_rows* a) {
+    g_err[0] = 0;
+    try {
+        ws::DeviceRows src(a->d_logits, a->rows, a->vocab, stream);
+        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+        for (uint32_t r = 0; r < a->rows; ++r) {
+            ws::Sampler s;
+            s.inv_t = a->inv_t[r];
+            s.temp = 1.0 / s.inv_t;
+            s.top_k = a->top_k ? a->top_k[r] : 0;
+            s.top_p = a->top_p ? a->top_p[r] : 1.0;
+            s.min_p = a->min_p ? a->min_p[r] : 0.0;
+            s.seed = a->seed[r];
+            s.pos_idx = a->pos_idx[r];
+            s.cands = &scratch;
+            s.race = a->race != 0;
+            ws::RowAdjust adj;
+            if (a->hist) {
+                adj.history = a->hist + a->hist_off[r];
+                adj.n_history = a->hist_off[r + 1] - a->hist_off[r];
+                adj.repetition = a->rep ? a->rep[r] : 1.f;
+                adj.presence = a->pres ? a->pres[r] : 0.f;
+                adj.frequency = a->freq ? a->freq[r] : 0.f;
+            }
+            if (a->bias_ids) {
+                adj.bias_ids = a->bias_ids + a->bias_off[r];
+                adj.bias_vals = a->bias_vals + a->bias_off[r];
+                adj.n_bias = a->bias_off[r + 1] - a->bias_off[r];
+            }
+            src.setAdjust(adj);
+            src.prepareRow(s, r);
+            s.pos_idx = a->pos_idx[r];
+            const uint32_t t = ws::sampleRow(src, s, std::nullopt, 0);
+            a->token[r] = static_cast<int32_t>(t);
+            if (a->prob) a->prob[r] = ws::probOf(src, s, t);
+            if (a->n_kept) a->n_kept[r] = static_cast<uint32_t>(s.n);
+            if (a->flags) a->flags[r] = src.lastFlags();
+            if (a->closed) a->closed[r] = s.closed;
+        }
+        return 0;
+    } catch (const ws::DeviceError& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return e.code ? e.code : -1;
+    } catch (const std::exception& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return -1;
+    }
+}
+
+}  // extern "C"
