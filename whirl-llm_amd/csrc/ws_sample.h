@@ -441,7 +441,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ float red_f[WS_WAVES];
     __shared__ uint32_t red_u[WS_WAVES];
     __shared__ double red_d[WS_WAVES];
-    __shared__ BinSel sel[6];
     __shared__ uint32_t s_cnt;
     __shared__ double s_d[8];
     __shared__ uint32_t s_u[8];
@@ -789,34 +788,39 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     }
     __syncthreads();  // the histogram is gone; after the lookups its LDS becomes the key buffer
+    WS_MARK(15);
     const double Z = pm[kBins];
     const double Zf = static_cast<double>(static_cast<float>(Z));  // Sampler::sum is a float (src/sampling/sampler.h:38)
 
-    // lookups in the scanned histogram; every call site is reached by the whole block. A bin's mass interval is
-    // [pm[b], pm[b + 1]), its rank interval [pc[b], pc[b + 1])
+    // Lookups in the scanned histogram. A bin's mass interval is [pm[b], pm[b + 1]), its rank interval
+    // [pc[b], pc[b + 1]). Every thread runs the same binary searches on these LDS arrays (broadcast reads), so the
+    // answers are in registers everywhere and the phase needs no barrier.
     auto bin_sel = [&](int b) {
+        if (b < 0) return BinSel{-1, 0u, 0u, 0.0, 0.0};
         const uint32_t cx = pc[b];
         const double mx = pm[b];
         return BinSel{b, cx, pc[b + 1] - cx, mx, pm[b + 1] - mx};
     };
-    auto find_count = [&](uint32_t n, int slot) {  // bin holding the element of rank n - 1
-#pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            const int b = kPT * t + j;
-            if (pc[b] < n && pc[b + 1] >= n) sel[slot] = bin_sel(b);
-        }
+    // smallest bin for which reached(bin) holds (monotone in the bin), kBins if none: a 64-way search by the wave,
+    // lane i probing the last bin of the i-th stretch of 64 bins, then bin i of the stretch found. Two LDS round trips.
+    auto first_bin = [&](auto&& reached) {
+        const int lane = lane_id();
+        const uint64_t coarse = __ballot(reached(64 * lane + 63));
+        if (!coarse) return static_cast<int>(kBins);
+        const int base = 64 * (__ffsll(static_cast<unsigned long long>(coarse)) - 1);
+        const uint64_t fine = __ballot(reached(base + lane));
+        return base + (__ffsll(static_cast<unsigned long long>(fine)) - 1);
     };
-    auto find_mass = [&](double X, bool strict, int slot) {  // first non-empty bin whose inclusive mass prefix reaches X
-#pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            const int b = kPT * t + j;
-            const double lo = pm[b], hi = pm[b + 1];
-            const bool hit = strict ? (hi > X && !(lo > X)) : (hi >= X && !(lo >= X));
-            if (hit && hi > lo && pc[b + 1] > pc[b]) sel[slot] = bin_sel(b);
-        }
+    auto find_count = [&](uint32_t n) {  // bin holding the element of rank n - 1, -1 if there is none
+        if (n == 0) return -1;
+        const int b = first_bin([&](int k) { return pc[k + 1] >= n; });
+        return b < kBins ? b : -1;
     };
-    auto fetch_bin = [&](int b, int slot) {
-        if (b >= 0 && static_cast<uint32_t>(b / kPT) == t) sel[slot] = bin_sel(b);
+    auto find_mass = [&](double X, bool strict) {  // first non-empty bin whose inclusive mass prefix reaches X, -1 if none
+        if (!strict && !(X > 0.0)) return -1;
+        int b = strict ? first_bin([&](int k) { return pm[k + 1] > X; }) : first_bin([&](int k) { return pm[k + 1] >= X; });
+        while (b < kBins && pc[b + 1] == pc[b]) ++b;  // an empty bin can only turn up through rounding at a scan seam
+        return b < kBins ? b : -1;
     };
 
     uint32_t n1 = (top_k > 0 && top_k < V) ? top_k : V;
@@ -829,24 +833,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
     bool minp_in_list = false, topp_in_list = false;
     double X = 0;  // top-p target in mass units (known here unless top-k closes the set)
-    if (t < 6) sel[t].b = -1;
-    __syncthreads();
     if (prefix_mode) {
-        find_count(n1, 0);
-        fetch_bin(kBins - 1, 5);
-        __syncthreads();
-        BinSel s1 = sel[0];
+        BinSel s1 = bin_sel(find_count(n1));
         if (s1.b < 0 || s1.b >= kBins - 1) {
             // top-k reaches into the tail bin (-inf and logits whose mass is below e^-64 of the top token's): those
             // candidates stay in the kept count, as in the host filter, but carry no mass; cuts and the draw see the
             // candidates ranked before the tail
-            n1 = sel[5].cx;
-            __syncthreads();
-            if (t == 0) sel[0].b = -1;
-            __syncthreads();
-            find_count(n1, 0);
-            __syncthreads();
-            s1 = sel[0];
+            n1 = pc[kBins - 1];
+            s1 = bin_sel(find_count(n1));
         }
         if (s1.b < 0 || s1.b >= kBins - 1 || s1.cx + s1.c > kCap) {
             flags |= kOverflow;
@@ -862,20 +856,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         int b2 = -1, lo3 = kBins, hi3 = -1;
         if (use_top_p) {
             X = top_p * (top_k > 0 ? Z : Zf);
-            find_mass(X, false, 0);
-            __syncthreads();
-            if (top_k == 0 && sel[0].b >= 0 && sel[0].cx >= 16384u) {
+            b2 = find_mass(X, false);
+            if (top_k == 0 && b2 >= 0 && pc[b2] >= 16384u) {
                 X = top_p * Z;
-                __syncthreads();
-                if (t == 0) sel[0].b = -1;
-                __syncthreads();
-                find_mass(X, false, 0);
-                __syncthreads();
+                b2 = find_mass(X, false);
             }
-            b2 = sel[0].b;
-            if (b2 < 0) {  // rounding pushed the target past the total: the cut is the whole row
-                b2 = kBins - 1;
-            }
+            if (b2 < 0) b2 = kBins - 1;  // rounding pushed the target past the total: the cut is the whole row
         }
         if (use_min_p) {
             const double astar = (-log(min_p) + lift) * 64.0;  // the floor in bin coordinates (bins count from the anchor)
@@ -896,25 +882,16 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             minp_in_list = topp_in_list = true;
         }
         // bounds of the kept mass -> bins the draw can land in
-        __syncthreads();
-        if (t < 6) sel[t].b = -1;
-        __syncthreads();
         const double u = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
         double zlo, zhi;
         if (r1hi >= r1lo) {
-            fetch_bin(r1lo, 1);
-            fetch_bin(r1hi, 2);
-            __syncthreads();
-            zlo = sel[1].mx;
-            zhi = sel[2].mx + sel[2].ms;
+            zlo = pm[r1lo];
+            zhi = pm[r1hi + 1];
             if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);  // the top token is always kept
         } else {
             zlo = zhi = Z;
         }
-        find_mass(u * zlo * (1.0 - 1e-9), true, 3);
-        find_mass(u * zhi * (1.0 + 1e-9), true, 4);
-        __syncthreads();
-        int b4lo = sel[3].b, b4hi = sel[4].b;
+        int b4lo = find_mass(u * zlo * (1.0 - 1e-9), true), b4hi = find_mass(u * zhi * (1.0 + 1e-9), true);
         if (b4lo < 0) b4lo = 0;
         if (b4hi < 0) b4hi = (r1hi >= r1lo) ? r1hi : kBins - 2;
         if (b4hi < b4lo) b4hi = b4lo;
@@ -931,22 +908,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     // bases of the two ranges
-    __syncthreads();
-    if (t < 6) sel[t].b = -1;
-    __syncthreads();
-    fetch_bin(r0lo, 0);
-    fetch_bin(r0hi, 1);
-    fetch_bin(r1hi >= r1lo ? r1lo : -1, 2);
-    fetch_bin(r1hi >= r1lo ? r1hi : -1, 3);
-    if (t == 0) s_cnt = s_u[5] = 0;
-    __syncthreads();
-    const uint32_t c0base = sel[0].cx, n_r0 = sel[1].cx + sel[1].c - sel[0].cx;
-    const double m0base = sel[0].mx;
     const bool has_r1 = r1hi >= r1lo;
-    const uint32_t c1base = has_r1 ? sel[2].cx : 0u, n_r1 = has_r1 ? sel[3].cx + sel[3].c - sel[2].cx : 0u;
-    const double m1base = has_r1 ? sel[2].mx : 0.0;
+    const uint32_t c0base = pc[r0lo], n_r0 = r0hi >= r0lo ? pc[r0hi + 1] - c0base : 0u;
+    const double m0base = pm[r0lo];
+    const uint32_t c1base = has_r1 ? pc[r1lo] : 0u, n_r1 = has_r1 ? pc[r1hi + 1] - c1base : 0u;
+    const double m1base = has_r1 ? pm[r1lo] : 0.0;
     const uint32_t n_list = n_r0 + n_r1;
     if (n_list > kCap || n_list == 0) flags |= kOverflow;
+    if (t == 0) s_cnt = s_u[5] = 0;
+    __syncthreads();  // the last reads of pm / pc are done: their LDS is the key buffer and the candidate list from here
 
     if (flags & kOverflow) {
         if (t == 0) {
@@ -1102,15 +1072,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             const uint32_t v_a = i < n_r0 ? 0u : n_r0 >> 6;
             const uint32_t v_b = i < n_r0 ? (n_r0 - 1u) >> 6 : nruns - 1u;
             place[q] += v_a << 6;
-            // four runs at a time, so that four binary searches wait for LDS together (a search of the own run,
+            // kIlp runs at a time, so that as many binary searches wait for LDS together (a search of the own run,
             // or of a run past the last, is carried along and dropped)
-            for (uint32_t v0 = v_a; v0 <= v_b; v0 += 4u) {
-                uint32_t cnt[4] = {0u, 0u, 0u, 0u};
-                const uint64_t* run[4];
-                bool tie[4];
+            constexpr int kIlp = 4;
+            for (uint32_t v0 = v_a; v0 <= v_b; v0 += kIlp) {
+                uint32_t cnt[kIlp];
+                const uint64_t* run[kIlp];
+                bool tie[kIlp];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < kIlp; ++r) {
                     const uint32_t v = min(v0 + r, v_b);
+                    cnt[r] = 0u;
                     run[r] = runs + (v << 6);  // descending
                     tie[r] = v < run_id;       // equal keys: the earlier run goes first
                 }
@@ -1118,13 +1090,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #pragma unroll
                 for (uint32_t sdx = 32; sdx >= 1; sdx >>= 1) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
+                    for (int r = 0; r < kIlp; ++r) {
                         const uint64_t o = run[r][cnt[r] + sdx - 1u];
                         if (o > key[q] || (o == key[q] && tie[r])) cnt[r] += sdx;
                     }
                 }
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < kIlp; ++r) {
                     const uint64_t o = run[r][cnt[r]];
                     if (o > key[q] || (o == key[q] && tie[r])) cnt[r] += 1u;
                     if (v0 + r <= v_b && v0 + r != run_id) place[q] += cnt[r];
