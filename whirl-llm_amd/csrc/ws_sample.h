@@ -9,7 +9,7 @@
 //            touched ones from the bin of their raw logit to the bin of their adjusted logit.
 //   pass 1   maximum of the adjusted row (NaN and masked tokens count as -inf).
 //   pass 2   histogram of 4096 bins of width 1/64 in a = (max - x) * inv_t, the exponent of the softmax: one LDS
-//            64-bit atomic per element adds {count, fixed-point 1 - exp(-(a - bin edge))} (degree-4 polynomial, no
+//            64-bit atomic per element adds {count, fixed-point 1 - exp(-(a - bin edge))} (a quadratic, no
 //            transcendental per element). A block scan turns it into count and mass prefixes in (logit desc) order.
 //            The normaliser sum exp((x - max) * inv_t) is the total mass.
 //   select   top-k is a count query, top-p and the draw are mass queries, min-p is a value query on these prefixes;
@@ -35,8 +35,10 @@ constexpr int kPT = kBins / WS_BLOCK;    // histogram bins, and sorted candidate
 constexpr int kCountShift = 44;          // histogram word: count << 44 | fixed-point sum of (1 - exp(-w))
 constexpr float kFixScale = 1073741824.f;  // 2^30
 constexpr double kFixInv = 1.0 / 1073741824.0;
-// 2^30 * (1 - exp(-w / 64)) = w * (k0 + w * (k1 + w * k2)) for the in-bin offset w in [0, 1.02] (max error 1.4e-10 * 2^30)
-constexpr float kG0 = 16777216.0f, kG1 = -131070.34375f, kG2 = 678.6015014648438f;
+// 2^30 * (1 - exp(-w / 64)) ~ w * (k0 + w * k1) for the in-bin offset w in [0, 1): minimax fit, off by at most 28 units,
+// 2.6e-8 of a token's mass - well inside the 1e-6 the mass estimates are trusted to, and one instruction per token less
+// than the cubic that would be exact to a unit
+constexpr float kG0 = 16776924.0f, kG1 = -130126.3125f;
 
 // flag bits (WS_FLAG_* of the C ABI)
 constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u;
@@ -198,10 +200,10 @@ __device__ __forceinline__ float bin_coord(float aq, float c64, float x) {
     return t < 4095.f ? t : 4095.f;  // NaN -> tail
 }
 __device__ __forceinline__ uint32_t bin_of(float aq, float c64, float x) { return static_cast<uint32_t>(bin_coord(aq, c64, x)); }
-// histogram word of one token: count 1 and the fixed-point cubic of the in-bin offset w = fract(t)
+// histogram word of one token: count 1 and the fixed-point quadratic of the in-bin offset w = fract(t)
 __device__ __forceinline__ uint64_t bin_word(float tc) {
     const float w = __builtin_amdgcn_fractf(tc);
-    const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, __fmaf_rn(w, kG2, kG1), kG0), 0.5f));
+    const uint32_t fx = static_cast<uint32_t>(__fmaf_rn(w, __fmaf_rn(w, kG1, kG0), 0.5f));
     return (1ull << kCountShift) | fx;
 }
 
@@ -1037,8 +1039,110 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         dbg[14] = static_cast<float>(r1hi >= r1lo ? r1hi - r1lo + 1 : 0);
     }
 #endif
+    // ---- sort keys[0, n_list) descending. First choice: a bucket sort. A candidate's bucket is its bin and the
+    // position inside the bin in S equal steps (both from the bin coordinate every pass uses, so buckets are ordered
+    // like the keys); candidates are counted per bucket, the counts scanned, the keys scattered to their bucket, and
+    // ranked inside it by comparing with the few other members. Logits that spread evenly inside a bin - any continuous
+    // distribution - give buckets of a handful of keys whatever the size of the list. A bin whose candidates all share
+    // one logit (coarse logits: bf16, rounded values) is cut into steps of the token id instead, the order of equal
+    // logits. Anything else that piles up (several heavily repeated logits in one bin) goes to the comparison sorts below.
+    constexpr uint32_t kMaxBuckets = 2048, kMaxInBucket = 96, kMaxBucketSort = 3072;
+    bool sorted = false;
+    {
+        const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+        uint32_t S = 64;
+        while (S > 1 && (nb0 + nb1) * S > kMaxBuckets) S >>= 1;
+        const uint32_t nbk = (nb0 + nb1) * S;
+        if (nbk <= kMaxBuckets && n_list <= kMaxBucketSort && n_list > 64) {
+            uint64_t* tmp = reinterpret_cast<uint64_t*>(emass);                        // 24 KiB: the scattered keys
+            uint32_t* bcnt = reinterpret_cast<uint32_t*>(emass) + 2 * kMaxBucketSort;  // 8 KiB: counts, then bucket starts
+            constexpr int kCh = kMaxBucketSort / WS_BLOCK;                             // keys per thread
+            uint64_t key[kCh];
+            uint32_t bucket[kCh], arrival[kCh];
+            // smallest and largest logit key per bin, to spot the bins whose candidates are all ties (up to kTieBins bins)
+            constexpr uint32_t kTieBins = 32;
+            __shared__ uint32_t bin_lo[kTieBins], bin_hi[kTieBins];
+            const bool spot_ties = nb0 + nb1 <= kTieBins;
+            for (uint32_t b = t; b <= nbk; b += WS_BLOCK) bcnt[b] = 0u;
+            if (t < kTieBins) {
+                bin_lo[t] = 0xffffffffu;
+                bin_hi[t] = 0u;
+            }
+            __syncthreads();
+            uint32_t rb[kCh];
+            float tcs[kCh];
+#pragma unroll
+            for (int q = 0; q < kCh; ++q) {
+                const uint32_t i = q * WS_BLOCK + t;
+                if (i < n_list) {
+                    key[q] = keys[i];
+                    const uint32_t k32 = static_cast<uint32_t>(key[q] >> 32);
+                    tcs[q] = bin_coord(aq, c64, unkey32(k32));
+                    const uint32_t bin = static_cast<uint32_t>(tcs[q]);
+                    rb[q] = (has_r1 && i >= n_r0) ? nb0 + (bin - static_cast<uint32_t>(r1lo)) : bin - static_cast<uint32_t>(r0lo);
+                    rb[q] = min(rb[q], nb0 + nb1 - 1u);
+                    if (spot_ties) {
+                        atomicMin(&bin_lo[rb[q]], k32);
+                        atomicMax(&bin_hi[rb[q]], k32);
+                    }
+                }
+            }
+            __syncthreads();
+            const float id_step = static_cast<float>(S) / static_cast<float>(V);
+#pragma unroll
+            for (int q = 0; q < kCh; ++q) {
+                const uint32_t i = q * WS_BLOCK + t;
+                if (i < n_list) {
+                    const bool all_tied = spot_ties && bin_lo[rb[q]] == bin_hi[rb[q]];
+                    const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
+                    const float pos = all_tied ? static_cast<float>(id) * id_step : __builtin_amdgcn_fractf(tcs[q]) * static_cast<float>(S);
+                    bucket[q] = rb[q] * S + min(S - 1u, static_cast<uint32_t>(pos));
+                    arrival[q] = atomicAdd(&bcnt[bucket[q]], 1u);
+                }
+            }
+            __syncthreads();
+            // exclusive scan of the counts (a few consecutive buckets per thread) and the largest bucket
+            constexpr uint32_t kPB = kMaxBuckets / WS_BLOCK;
+            uint32_t local[kPB], sum = 0, biggest = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < kPB; ++j) {
+                const uint32_t b = kPB * t + j;
+                local[j] = b < nbk ? bcnt[b] : 0u;
+                sum += local[j];
+                biggest = max(biggest, local[j]);
+            }
+            uint32_t total;
+            uint32_t run = block_excl_scan(sum, red_u, &total);
+            biggest = 0xffffffffu - block_min(0xffffffffu - biggest, red_u);
+#pragma unroll
+            for (uint32_t j = 0; j < kPB; ++j) {
+                const uint32_t b = kPB * t + j;
+                if (b < nbk) bcnt[b] = run;
+                run += local[j];
+            }
+            if (t == 0) bcnt[nbk] = total;
+            __syncthreads();
+            if (biggest <= kMaxInBucket) {  // uniform
+#pragma unroll
+                for (int q = 0; q < kCh; ++q)
+                    if (q * WS_BLOCK + t < n_list) tmp[bcnt[bucket[q]] + arrival[q]] = key[q];
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < kCh; ++q) {
+                    if (q * WS_BLOCK + t >= n_list) continue;
+                    const uint32_t b0 = bcnt[bucket[q]], b1 = bcnt[bucket[q] + 1u];
+                    uint32_t before = 0;
+                    for (uint32_t j = b0; j < b1; ++j) before += tmp[j] > key[q] ? 1u : 0u;
+                    keys[b0 + before] = key[q];  // every key was read into registers before the first barrier above
+                }
+                __syncthreads();
+                sorted = true;
+            }
+        }
+    }
     constexpr int kMergeCh = 3;  // keys per thread the merge sort takes
-    if (n_list <= kMergeCh * WS_BLOCK) {
+    if (sorted) {
+    } else if (n_list <= kMergeCh * WS_BLOCK) {
         // Few candidates (the usual case): one or two per thread. Each wave ranks 64 keys among themselves by counting
         // and writes them out as a sorted run; then every key finds its rank in each other run by binary search; the
         // sum of the ranks is its place. Three barriers instead of one per bitonic stage. Slots past n_list hold
