@@ -490,9 +490,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const int32_t* hist_ids = A.hist + h0;
         const int32_t* bias_ids = A.bias_ids + b0;
         const float* bias_vals = A.bias_vals + b0;
+        // the first kHid history ids of each thread stay in registers for both passes over the history
+        constexpr int kHid = 4;
+        uint32_t hid[kHid];
+#pragma unroll
+        for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
         for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
         __syncthreads();
-        for (uint32_t j = t; j < nh; j += WS_BLOCK) {
+#pragma unroll
+        for (int k = 0; k < kHid; ++k)
+            if (hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
+        for (uint32_t j = t + kHid * WS_BLOCK; j < nh; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
         }
@@ -521,10 +529,24 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         __syncthreads();
         rv.touched = touched;
-        for (uint32_t j = t; j < nh; j += WS_BLOCK) {
+        // without a bias list the second table is free from the start: it takes the token id of each rank right away
+        const bool ids_now = FUSED && nb == 0;
+#pragma unroll
+        for (int k = 0; k < kHid; ++k)
+            if (hid[k] < V) {
+                const uint32_t r = rank_of(rv, hid[k]);
+                atomicAdd(&cnt[r], 1u);
+                if (ids_now) first[r] = hid[k];
+            }
+        for (uint32_t j = t + kHid * WS_BLOCK; j < nh; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
-            if (id < V) atomicAdd(&cnt[rank_of(rv, id)], 1u);
+            if (id < V) {
+                const uint32_t r = rank_of(rv, id);
+                atomicAdd(&cnt[r], 1u);
+                if (ids_now) first[r] = id;
+            }
         }
+        if (nb)
         for (uint32_t j = t; j < nb; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
             if (id < V) {
@@ -534,6 +556,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         }
         __syncthreads();
+        if (nb) {  // uniform
         for (uint32_t j = t; j < nb; j += WS_BLOCK) {  // bias sum of an id, by the thread of its first entry
             const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
             if (id >= V) continue;
@@ -549,8 +572,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         // per rank: bias sum -> first[r] (float bits; the first-entry bookkeeping is dead), cnt[r] stays
         for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) first[r] = __float_as_uint(pv[r]);
         __syncthreads();
+        }
         n_touched = n_uniq;
-        __syncthreads();
     }
     const float* praw = reinterpret_cast<const float*>(lds + A.lds_cnt);           // raw logits of the touched tokens, by rank
     const uint32_t* pid = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt) + A.patch_cap;  // their token ids
@@ -639,7 +662,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             m_adj = block_max(ma, red_f);
             m_near = block_max(mu, red_f);
         }
-        if (FUSED) {
+        if (FUSED && nb) {  // with a bias list the ids could not be stored before the bias sums were consumed
             for (uint32_t j = t; j < nh; j += WS_BLOCK) {
                 const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
                 if (id < V) first[rank_of(rv, id)] = id;
