@@ -485,14 +485,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     uint32_t n_touched = 0;  // distinct tokens the history and the bias list touch
     float m_adj = -INFINITY;  // largest adjusted logit among them
     float m_near = -INFINITY; // largest untouched, allowed logit among the 128-bit vectors that hold them (single-sweep mode)
+    // the first kHid history ids of each thread stay in registers: two passes of phase 0 and the collection of the
+    // touched logits after the sweep use them
+    constexpr int kHid = 4;
+    uint32_t hid[kHid];
+#pragma unroll
+    for (int k = 0; k < kHid; ++k) hid[k] = 0xffffffffu;
     if (!(inv_t > 0.f) || nh + nb > A.patch_cap) flags |= kBadParam;
     if (!(flags & kBadParam) && nh + nb > 0) {
         const int32_t* hist_ids = A.hist + h0;
         const int32_t* bias_ids = A.bias_ids + b0;
         const float* bias_vals = A.bias_vals + b0;
-        // the first kHid history ids of each thread stay in registers for both passes over the history
-        constexpr int kHid = 4;
-        uint32_t hid[kHid];
 #pragma unroll
         for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
         for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
@@ -590,14 +593,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
         uint32_t* first = cnt + A.patch_cap;
         float mu = -INFINITY;  // largest untouched, allowed logit among the vectors that hold touched tokens
-        auto fetch4 = [&](const int32_t* ids, uint32_t n) {  // four independent gathers per thread and round
+        auto fetch4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {  // four independent gathers per thread and round
             for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
                 uint32_t id[4], bits[4], al[4];
                 uint4 vec[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t j = j0 + k * WS_BLOCK + t;
-                    id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
+                    if (in_regs && j0 == 0) id[k] = hid[k];  // kHid = 4: the first round is in registers
+                    else id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
                 }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -640,8 +644,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
             }
         };
-        fetch4(hist_ids, nh);
-        fetch4(bias_ids, nb);
+        static_assert(kHid == 4, "fetch4 takes its first round from hid");
+        fetch4(hist_ids, nh, true);
+        fetch4(bias_ids, nb, false);
         __syncthreads();
         {
             const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
