@@ -74,22 +74,16 @@ def parity_sample(c, smp, n_check, rng_mode=1):
     return res
 
 
-def cpu_baseline(c, budget_s=12.0):
-    """Reference sampler on the host cores of this box: penalties pre-pass (oracle) + prepare / filter / draw of the
-    reference's own code with its splitmix uniform. One thread; rows of the batch in order, wrapping round with the
-    decode step advanced, until budget_s seconds of CPU work are spent."""
+def _cpu_rows(c, lib, port, kind_rows, budget_s):
+    """Runs rows of the batch (an iterable of (row, lap)) through the CPU sampler until budget_s seconds of its own work
+    are spent; returns (rows done, seconds of sampler work)."""
     import ctypes as C
     import numpy as np
     import gpu_cases as gc
     import wo
-    ref = wo.load("ref")
-    lib = ref if ref is not None else wo.load("oracle")
-    port = wo.load("oracle")
-    kind = "reference" if ref is not None else "port"
     done, t_used = 0, 0.0
     V = c["V"]
-    for k in range(1 << 20):
-        r, lap = k % c["rows"], k // c["rows"]
+    for r, lap in kind_rows:
         x = gc.row_f32(c, r).copy()
         hist = np.ascontiguousarray(c["hist"][r]) if c["hist"] is not None else np.zeros(0, np.int32)
         bi = np.ascontiguousarray(c["bias_ids"][r]) if c["bias_ids"] is not None else np.zeros(0, np.int32)
@@ -106,9 +100,37 @@ def cpu_baseline(c, budget_s=12.0):
         done += 1
         if t_used > budget_s:
             break
+    return done, t_used
+
+
+def cpu_baseline(c, budget_s=9.0, budget_all_s=6.0):
+    """Reference sampler on the host cores of this box: penalties pre-pass (oracle) + prepare / filter / draw of the
+    reference's own code with its splitmix uniform. `value` is one thread (the reference engine samples on one
+    thread); rows of the batch in order, wrapping round with the decode step advanced, until budget_s seconds of CPU
+    work are spent. `all_cores` repeats it with the rows sharded over the box's cores (rows are independent)."""
+    import itertools
+    from concurrent.futures import ThreadPoolExecutor
+    import wo
+    ref = wo.load("ref")
+    lib = ref if ref is not None else wo.load("oracle")
+    port = wo.load("oracle")
+    kind = "reference" if ref is not None else "port"
+    R = c["rows"]
+    seq = ((k % R, k // R) for k in itertools.count())
+    done, t_used = _cpu_rows(c, lib, port, seq, budget_s)
+    # the library calls release the interpreter lock, so plain threads shard the rows
+    n_thr = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(n_thr) as ex:
+        parts = list(ex.map(lambda w: _cpu_rows(c, lib, port, (((w + k * n_thr) % R, (w + k * n_thr) // R) for k in itertools.count()),
+                                                budget_all_s), range(n_thr)))
+    wall = time.perf_counter() - t0
+    done_all = sum(p[0] for p in parts)
     return dict(value=done / t_used, unit="rows/s", cores=1, kind=kind,
                 sample=f"{done} rows (the rows of the same batch in order, wrapping), penalties + escalation "
-                       f"256/16384/full + filter + draw, {t_used:.2f} s on one host thread")
+                       f"256/16384/full + filter + draw, {t_used:.2f} s on one host thread",
+                all_cores=dict(value=done_all / wall, unit="rows/s", cores=n_thr,
+                               sample=f"{done_all} rows sharded over {n_thr} threads, {wall:.2f} s wall clock"))
 
 
 def run_workload(name, steps, warmup, check_rows):

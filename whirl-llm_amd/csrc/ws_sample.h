@@ -1074,7 +1074,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // distribution - give buckets of a handful of keys whatever the size of the list. A bin whose candidates all share
     // one logit (coarse logits: bf16, rounded values) is cut into steps of the token id instead, the order of equal
     // logits. Anything else that piles up (several heavily repeated logits in one bin) goes to the comparison sorts below.
-    constexpr uint32_t kMaxBuckets = 2048, kMaxInBucket = 96, kMaxBucketSort = 3072;
+    constexpr uint32_t kMaxBuckets = 2047, kMaxInBucket = 96, kMaxBucketSort = 3072;  // starts of 2047 buckets + the end: 8 KiB
     bool sorted = false;
     {
         const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
@@ -1130,7 +1130,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
             __syncthreads();
             // exclusive scan of the counts (a few consecutive buckets per thread) and the largest bucket
-            constexpr uint32_t kPB = kMaxBuckets / WS_BLOCK;
+            constexpr uint32_t kPB = (kMaxBuckets + WS_BLOCK - 1) / WS_BLOCK;
             uint32_t local[kPB], sum = 0, biggest = 0;
 #pragma unroll
             for (uint32_t j = 0; j < kPB; ++j) {
