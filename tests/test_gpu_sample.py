@@ -139,6 +139,34 @@ def test_history_holds_the_top_tokens(mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
+def test_bias_values_of_one_id_are_added_one_by_one(mode):
+    """A token listed three times with +1e8, -1e8, +1: added one by one to the logit x the result is
+    ((x + 1e8) - 1e8) + 1 with the float roundings of each step; summed first and added once it would be x + 1.
+    The oracle adds one by one (tests/test_oracle_batch.py pins that), and so must the kernel."""
+    c = gc.make_cfg2(rows=4, V=8000, n_hist=64, n_bias=6)
+    c["top_k"][:] = 0
+    c["top_p"][:] = 1.0
+    c["min_p"][:] = 0.001
+    for r in range(4):
+        star = int(np.argmax(c["logits"][r]))
+        c["bias_ids"][r, :3] = star
+        c["bias_vals"][r, :3] = [1e8, -1e8, 1.0]
+        c["hist"][r, :] = (star + 1 + np.arange(64)) % 8000   # keep the star out of the history
+    res, smp = run_case(c, 1, kept_cap=8000, mode=mode)
+    for r in range(4):
+        star = int(np.argmax(c["logits"][r]))
+        ids = smp.kept_ids[r].cpu().numpy()
+        lg = smp.kept_logits[r].cpu().numpy()
+        n = int(smp.n_kept[r].item())
+        where = np.nonzero(ids[:n] == star)[0]
+        x = np.float32(c["logits"][r, star])
+        one_by_one = np.float32(np.float32(np.float32(x + np.float32(1e8)) - np.float32(1e8)) + np.float32(1.0))
+        assert one_by_one != np.float32(x + np.float32(1.0))  # the two orders do differ for this row
+        assert where.size == 1 and lg[where[0]] == one_by_one
+    print(res)
+
+
+@pytest.mark.parametrize("mode", MODES)
 def test_cfg1_shape(mode):
     res, _ = run_case(gc.make_cfg1(), 0, mode=mode)
     print(res)

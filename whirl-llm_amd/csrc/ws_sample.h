@@ -77,7 +77,7 @@ struct BatchArgs {
     uint32_t kept_cap;
     double tol;
     uint32_t lds_ab;   // bytes of the LDS region shared by the histogram / sort keys / masses
-    uint32_t lds_cnt;  // byte offset of the per-rank counters {history count | bias entries, bias sum}: 8 * patch_cap bytes
+    uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
 };
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
@@ -559,23 +559,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         }
         __syncthreads();
-        if (nb) {  // uniform
-        for (uint32_t j = t; j < nb; j += WS_BLOCK) {  // bias sum of an id, by the thread of its first entry
-            const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
-            if (id >= V) continue;
-            const uint32_t r = rank_of(rv, id);
-            if (first[r] != j) continue;
-            float sum = bias_vals[j];
-            if ((cnt[r] >> 20) > 1u)  // several entries for one id: add them in listed order
-                for (uint32_t j2 = j + 1; j2 < nb; ++j2)
-                    if (static_cast<uint32_t>(bias_ids[j2]) == id) sum = __fadd_rn(sum, bias_vals[j2]);
-            pv[r] = sum;
-        }
-        __syncthreads();
-        // per rank: bias sum -> first[r] (float bits; the first-entry bookkeeping is dead), cnt[r] stays
-        for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) first[r] = __float_as_uint(pv[r]);
-        __syncthreads();
-        }
         n_touched = n_uniq;
     }
     const float* praw = reinterpret_cast<const float*>(lds + A.lds_cnt);           // raw logits of the touched tokens, by rank
@@ -590,6 +573,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const uint32_t per = rv.dtype == 0 ? 4u : 8u;
         const int32_t* hist_ids = A.hist + h0;
         const int32_t* bias_ids = A.bias_ids + b0;
+        const float* bias_vals = A.bias_vals + b0;
         uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
         uint32_t* first = cnt + A.patch_cap;
         float mu = -INFINITY;  // largest untouched, allowed logit among the vectors that hold touched tokens
@@ -655,7 +639,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 const uint32_t cw = cnt[r], c = cw & 0xfffffu;
                 const float raw = pv[r];
                 float x = raw;
-                if (cw >> 20) x = __fadd_rn(x, __uint_as_float(first[r]));
+                if (cw >> 20) {
+                    // the bias values of this id, added one by one in listed order, starting at its first entry
+                    uint32_t j = first[r];
+                    const int32_t id = bias_ids[j];
+                    x = __fadd_rn(x, bias_vals[j]);
+                    if ((cw >> 20) > 1u)
+                        for (++j; j < nb; ++j)
+                            if (bias_ids[j] == id) x = __fadd_rn(x, bias_vals[j]);
+                }
                 if (c) {
                     x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
                     x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
@@ -667,7 +659,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             m_adj = block_max(ma, red_f);
             m_near = block_max(mu, red_f);
         }
-        if (FUSED && nb) {  // with a bias list the ids could not be stored before the bias sums were consumed
+        if (FUSED && nb) {  // with a bias list the second table held the first-entry indices until the adjustment above
             for (uint32_t j = t; j < nh; j += WS_BLOCK) {
                 const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
                 if (id < V) first[rank_of(rv, id)] = id;
