@@ -2,7 +2,8 @@
 // bias, temperature, top-k / top-p / min-p, all in one launch) and brings back only the kept candidates, already
 // filtered: s.closed is true and the list is what filterCands would have left. Rows the device flags as unresolved
 // (more candidates tied at a cut than it handles, or no filter at all) go the reference's way instead: device top-k
-// of 256, then 16384, then the full row, each through filterCands (src/server/engine_sampling.cpp:51-84).
+// of 256, then 16384, then the full row, each through filterCands (src/server/engine_sampling.cpp:51-84), on a penalised
+// copy of the row that the device writes when penalties or a bias list are in force.
 //
 // Not in the reference: it plays the role of the engine's SampleBuffers (src/server/engine_sampling.h:20-73).
 #pragma once
@@ -63,7 +64,7 @@ private:
     std::vector<std::uint8_t> marks_;
     std::uint32_t last_flags_ = 0;
     static constexpr std::uint32_t kNoRow = 0xffffffffu;
-    std::uint32_t adjusted_row_ = kNoRow;  // row whose penalised copy row_host_ holds (after an escalation)
+    std::uint32_t adjusted_row_ = kNoRow;  // row whose penalised copy sits on the device (after an escalation)
 };
 
 }  // namespace whirl::sampling

@@ -177,6 +177,31 @@ typedef struct ws_batch {
 uint64_t ws_sample_batch_workspace(const ws_batch* b);
 int ws_sample_batch(void* stream, const ws_batch* b);
 
+/* Penalised fp32 copy of logits rows: out[row][i] = the logit ws_sample_batch samples from (allow mask and NaN -> -inf,
+ * bias, repetition, frequency / presence; same fields and meaning as in ws_batch). No counterpart in the reference, which
+ * has no penalties; it lets the reference's own route - ws_topk_rows on the row, host filter, full-row download
+ * (src/server/engine_sampling.cpp:51-84) - run on penalised logits. out: device [rows][out_stride] floats. */
+typedef struct ws_adjust {
+    const void* logits;
+    int32_t dtype;
+    uint32_t rows, vocab;
+    uint64_t row_stride;
+    const int32_t* hist;
+    const uint32_t* hist_off;
+    const float* rep;
+    const float* pres;
+    const float* freq;
+    const int32_t* bias_ids;
+    const float* bias_vals;
+    const uint32_t* bias_off;
+    const uint32_t* allow;
+    uint64_t allow_stride;
+    float* out;
+    uint64_t out_stride; /* >= vocab */
+} ws_adjust;
+
+int ws_adjust_rows(void* stream, const ws_adjust* a);
+
 /* Classic speculative sampling (accept u * q < p, else resample from max(p - q, 0)); no counterpart in the
  * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32
  * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1]. Per sequence s: u_j from

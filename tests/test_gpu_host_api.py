@@ -56,3 +56,17 @@ def test_host_rows_open_row_takes_the_reference_route():
     near, out = _run(c, range(4))
     assert near == 0
     assert all(out["flags"] & m.FLAG_OPEN) and not any(out["closed"])
+
+
+def test_host_rows_open_row_with_penalties_uses_the_penalised_copy():
+    """No filter, but a history and a bias list: the reference route then runs on the device's penalised copy of the row
+    (ws_adjust_rows -> ws_topk_rows -> filterCands -> tail walk over the downloaded penalised row)."""
+    m = gc.pkg()
+    c = gc.make_cfg2(rows=4, V=20000, n_hist=200, n_bias=12)
+    c["top_k"][:] = 0
+    c["top_p"][:] = 1.0
+    c["min_p"][:] = 0.0
+    c["inv_t"][:] = 0.4  # flat rows: the top 256 hold little mass, most draws walk the tail
+    near, out = _run(c, range(4))
+    assert near == 0
+    assert all(out["flags"] & m.FLAG_OPEN) and not any(out["closed"])

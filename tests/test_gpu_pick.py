@@ -132,3 +132,30 @@ def test_topk_rows_ties_at_the_cut_keep_lowest_ids():
     assert ids.cpu().tolist()[1] == list(range(7)) and vals.cpu().tolist()[1] == [-1.5] * 7
     ids, vals, _ = m.topk_rows(torch.from_numpy(x[:, :5]).contiguous().to(DEV), 9, 1.0)  # K > n: n entries written
     assert ids.cpu().tolist()[0][:5] == [0, 1, 2, 3, 4] and ids.cpu().tolist()[0][5:] == [-1] * 4
+
+
+def test_adjust_rows_matches_the_oracle_bit_for_bit():
+    """ws_adjust_rows: the penalised copy of a row equals the oracle's wo_apply_penalties on every token, with mask, bias
+    (repeated ids included), history counts, fp32 and bf16 input."""
+    gc = gpu_cases
+    m = gc.pkg()
+    lib = wo.load("oracle")
+    cases = [gc.make_cfg2(rows=5, V=32000, n_hist=700, n_bias=40), gc.make_cfg5(rows=3, V=16384, n_hist=300, n_bias=25),
+             gc.make_cfg3(rows=3, V=24000, n_hist=200)]
+    cases[0]["bias_ids"][:, 3] = cases[0]["bias_ids"][:, 0]
+    cases[0]["bias_ids"][:, 9] = cases[0]["bias_ids"][:, 0]
+    for c in cases:
+        d = gc.upload(c)
+        out = m.adjust_rows(d["logits"], hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
+                            bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], allow=d["allow"])
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        for r in range(c["rows"]):
+            x = gc.row_f32(c, r).copy()
+            hist = np.ascontiguousarray(c["hist"][r]) if c["hist"] is not None else np.zeros(0, np.int32)
+            bi = np.ascontiguousarray(c["bias_ids"][r]) if c["bias_ids"] is not None else np.zeros(0, np.int32)
+            bv = np.ascontiguousarray(c["bias_vals"][r]) if c["bias_vals"] is not None else np.zeros(0, np.float32)
+            allow = np.ascontiguousarray(c["allow"][r]) if c["allow"] is not None else None
+            lib.wo_apply_penalties(wo._ptr(x), c["V"], wo._ptr(allow) if allow is not None else None, wo._ptr(hist), hist.size,
+                                   c["rep"][r], c["pres"][r], c["freq"][r], wo._ptr(bi), wo._ptr(bv), bi.size)
+            assert got[r].tobytes() == x.tobytes(), (c["name"], r)

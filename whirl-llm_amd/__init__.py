@@ -60,6 +60,14 @@ class SpecVerify(C.Structure):
                 ("workspace_bytes", C.c_uint64), ("tol", C.c_double)]
 
 
+class Adjust(C.Structure):
+    """ws_adjust of include/whirl_sampling_abi.h."""
+    _fields_ = [("logits", C.c_void_p), ("dtype", C.c_int32), ("rows", C.c_uint32), ("vocab", C.c_uint32), ("row_stride", C.c_uint64),
+                ("hist", C.c_void_p), ("hist_off", C.c_void_p), ("rep", C.c_void_p), ("pres", C.c_void_p), ("freq", C.c_void_p),
+                ("bias_ids", C.c_void_p), ("bias_vals", C.c_void_p), ("bias_off", C.c_void_p), ("allow", C.c_void_p),
+                ("allow_stride", C.c_uint64), ("out", C.c_void_p), ("out_stride", C.c_uint64)]
+
+
 # every symbol include/whirl_sampling_abi.h declares: (result type, argument types)
 ABI = {
     "ws_abi_version": (C.c_int, []),
@@ -79,6 +87,7 @@ ABI = {
                                C.c_uint]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
+    "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
     "ws_spec_verify_workspace": (C.c_uint64, [C.POINTER(SpecVerify)]),
     "ws_spec_verify_classic": (C.c_int, [C.c_void_p, C.POINTER(SpecVerify)]),
 }
@@ -191,6 +200,21 @@ def topk_rows(x, K, inv_t):
     stats = torch.empty((rows, 2), dtype=torch.float32, device=x.device)
     check(lib().ws_topk_rows(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows), "ws_topk_rows")
     return ids, vals, stats
+
+
+def adjust_rows(logits, hist=None, hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
+                allow=None):
+    """Penalised float32 copy of logits rows (ws_adjust_rows): [rows, vocab] float32 / bfloat16 device tensor -> float32."""
+    if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1 or logits.dtype not in (torch.float32, torch.bfloat16):
+        raise WsError("logits: [rows, vocab] float32 / bfloat16 device tensor with unit inner stride")
+    rows, vocab = logits.shape
+    out = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
+    a = Adjust(logits=_p(logits), dtype=DTYPE_F32 if logits.dtype == torch.float32 else DTYPE_BF16, rows=rows, vocab=vocab,
+               row_stride=logits.stride(0), hist=_p(hist), hist_off=_p(hist_off), rep=_p(rep), pres=_p(pres), freq=_p(freq),
+               bias_ids=_p(bias_ids), bias_vals=_p(bias_vals), bias_off=_p(bias_off), allow=_p(allow),
+               allow_stride=allow.shape[1] if allow is not None else 0, out=_p(out), out_stride=vocab)
+    check(lib().ws_adjust_rows(_stream(), C.byref(a)), "ws_adjust_rows")
+    return out
 
 
 class BatchSampler:

@@ -6,6 +6,7 @@
 
 #include <cstring>
 
+#include "ws_adjust.h"
 #include "ws_common.h"
 #include "ws_draft.h"
 #include "ws_pick.h"
@@ -224,6 +225,32 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
         attr_set = true;
     }
     hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
+    return done();
+}
+
+int ws_adjust_rows(void* stream, const ws_adjust* b) {
+    if (!b || !b->logits || !b->out || b->rows == 0 || b->vocab == 0 || b->row_stride < b->vocab || b->out_stride < b->vocab)
+        return WS_E_INVALID;
+    if (b->dtype != WS_DTYPE_F32 && b->dtype != WS_DTYPE_BF16) return WS_E_INVALID;
+    if ((b->hist && !b->hist_off) || (b->bias_ids && (!b->bias_off || !b->bias_vals))) return WS_E_INVALID;
+    ws::AdjustArgs a{};
+    a.logits = b->logits;
+    a.dtype = b->dtype;
+    a.vocab = b->vocab;
+    a.row_stride = b->row_stride;
+    a.hist = b->hist;
+    a.hist_off = b->hist_off;
+    a.rep = b->rep;
+    a.pres = b->pres;
+    a.freq = b->freq;
+    a.bias_ids = b->bias_ids;
+    a.bias_vals = b->bias_vals;
+    a.bias_off = b->bias_off;
+    a.allow = b->allow;
+    a.allow_stride = b->allow_stride;
+    a.out = b->out;
+    a.out_stride = b->out_stride;
+    hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows), dim3(WS_BLOCK), ws::kAdjustLdsIds * sizeof(int32_t), S(stream), a);
     return done();
 }
 

@@ -55,6 +55,7 @@ struct DeviceRows::Dev {
     std::int32_t* topk_ids = nullptr;  // escalation: ids | vals | stats of one row, kBig candidates
     float* topk_vals = nullptr;
     float* topk_stats = nullptr;
+    float* adjusted = nullptr;         // escalation: penalised copy of the row (ws_adjust_rows)
     std::vector<std::int32_t> h_ids;
     std::vector<float> h_vals;
 };
@@ -75,7 +76,7 @@ DeviceRows::~DeviceRows() {
     for (void* p : {static_cast<void*>(dev_->prm), static_cast<void*>(dev_->res), static_cast<void*>(dev_->kept_ids),
                     static_cast<void*>(dev_->kept_logits), static_cast<void*>(dev_->hist), static_cast<void*>(dev_->bias_ids),
                     static_cast<void*>(dev_->bias_vals), static_cast<void*>(dev_->topk_ids), static_cast<void*>(dev_->topk_vals),
-                    static_cast<void*>(dev_->topk_stats)})
+                    static_cast<void*>(dev_->topk_stats), static_cast<void*>(dev_->adjusted)})
         if (p) (void)hipFree(p);
     delete dev_;
 }
@@ -190,66 +191,86 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     if (n > kBig) s.full_used += 1;
 }
 
-// The reference's way for a row the device did not resolve: its penalised copy on the host, the 256 best candidates
-// through filterCands, then 16384, then the whole row.
+// The reference's way for a row the device did not resolve (src/server/engine_sampling.cpp:51-84): the device's top 256
+// of the row through filterCands, then its top 16384, then the whole row. With penalties or a bias list in force the
+// device first writes a penalised copy of the row (ws_adjust_rows), and every later step reads that copy.
 void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
-    (void)loadFullRow(gr);
-    std::vector<float>& x = row_host_;  // loadFullRow filled it; penalise in place
-    if (adj_.n_bias)
-        for (std::uint32_t j = 0; j < adj_.n_bias; ++j)
-            if (static_cast<std::uint32_t>(adj_.bias_ids[j]) < vocab_) x[adj_.bias_ids[j]] += adj_.bias_vals[j];
-    if (adj_.n_history) {
-        std::vector<std::uint32_t> count(vocab_, 0);
-        for (std::uint32_t j = 0; j < adj_.n_history; ++j)
-            if (static_cast<std::uint32_t>(adj_.history[j]) < vocab_) count[adj_.history[j]] += 1;
-        for (std::uint32_t t = 0; t < vocab_; ++t) {
-            if (!count[t]) continue;
-            float v = x[t];
-            v = v > 0.f ? v / adj_.repetition : v * adj_.repetition;
-            x[t] = v - (adj_.frequency * static_cast<float>(count[t]) + adj_.presence);
+    auto stream = static_cast<hipStream_t>(stream_);
+    Dev& d = *dev_;
+    const float* src = logits_ + static_cast<std::size_t>(gr) * vocab_;
+    if (adj_.n_history || adj_.n_bias) {
+        if (!d.adjusted) checkHip(hipMalloc(reinterpret_cast<void**>(&d.adjusted), vocab_ * sizeof(float)), "hipMalloc");
+        ws_adjust a{};
+        a.logits = src;
+        a.dtype = WS_DTYPE_F32;
+        a.rows = 1;
+        a.vocab = vocab_;
+        a.row_stride = vocab_;
+        if (adj_.n_history) {  // the lists and the parameter block are still on the device from prepareRow
+            a.hist = d.hist;
+            a.hist_off = d.prm->hist_off;
+            a.rep = &d.prm->rep;
+            a.pres = &d.prm->pres;
+            a.freq = &d.prm->freq;
         }
+        if (adj_.n_bias) {
+            a.bias_ids = d.bias_ids;
+            a.bias_vals = d.bias_vals;
+            a.bias_off = d.prm->bias_off;
+        }
+        a.out = d.adjusted;
+        a.out_stride = vocab_;
+        check(ws_adjust_rows(stream_, &a), "ws_adjust_rows");
+        src = d.adjusted;
+        adjusted_row_ = gr;
     }
-    for (float& v : x)
-        if (std::isnan(v)) v = -std::numeric_limits<float>::infinity();
-    adjusted_row_ = gr;  // a tail walk of this row must see the penalised logits
-    std::vector<std::uint32_t> order(vocab_);
-    for (std::uint32_t i = 0; i < vocab_; ++i) order[i] = i;
-    const std::uint32_t ks = std::min(kSmall, vocab_), kb = std::min(kBig, vocab_);
-    std::partial_sort(order.begin(), order.begin() + kb, order.end(),
-                      [&](std::uint32_t a, std::uint32_t b) { return x[a] != x[b] ? x[a] > x[b] : a < b; });
-    s.m = x[order[0]];
-    double z = 0;
-    for (std::uint32_t i = 0; i < vocab_; ++i) z += std::exp(static_cast<double>(x[i] - s.m) * s.inv_t);
-    s.sum = static_cast<float>(z);
+    if (!d.topk_ids) {
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_ids), kBig * sizeof(std::int32_t)), "hipMalloc");
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_vals), kBig * sizeof(float)), "hipMalloc");
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_stats), 2 * sizeof(float)), "hipMalloc");
+    }
     Cand* c = s.cands->data();
-    for (std::uint32_t j = 0; j < ks; ++j) c[j] = {order[j], x[order[j]], 0.0};
-    if (filterCands(s, ks, false)) return;
-    s.big_used += 1;
-    for (std::uint32_t j = 0; j < kb; ++j) c[j] = {order[j], x[order[j]], 0.0};
-    if (filterCands(s, kb, false)) return;
+    bool first = true;
+    for (std::uint32_t k : {std::min(kSmall, vocab_), std::min(kBig, vocab_)}) {
+        check(ws_topk_rows(stream_, src, static_cast<int>(vocab_), static_cast<int>(k), s.inv_t, d.topk_ids, d.topk_vals, d.topk_stats, 1),
+              "ws_topk_rows");
+        float stats[2];
+        checkHip(hipMemcpyAsync(d.h_ids.data(), d.topk_ids, k * sizeof(std::int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+        checkHip(hipMemcpyAsync(d.h_vals.data(), d.topk_vals, k * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+        checkHip(hipMemcpyAsync(stats, d.topk_stats, sizeof stats, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+        checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+        if (first) {  // the row's maximum and normaliser, once (the second call recomputes the same values)
+            s.m = stats[0];
+            s.sum = stats[1];
+        } else {
+            s.big_used += 1;
+        }
+        first = false;
+        for (std::uint32_t j = 0; j < k; ++j) c[j] = {static_cast<std::uint32_t>(d.h_ids[j]), d.h_vals[j], 0.0};
+        if (filterCands(s, k, false)) return;
+    }
     s.full_used += 1;
+    const float* x = loadFullRow(gr);
     for (std::uint32_t j = 0; j < vocab_; ++j) c[j] = {j, x[j], 0.0};
     filterCands(s, vocab_, true);
 }
 
 const float* DeviceRows::loadFullRow(std::uint32_t gr) {
     if (gr >= rows_) throw DeviceError("loadFullRow", WS_E_INVALID, "loadFullRow: row out of range");
-    if (gr == adjusted_row_) return row_host_.data();
     row_host_.resize(vocab_);
     auto stream = static_cast<hipStream_t>(stream_);
-    checkHip(hipMemcpyAsync(row_host_.data(), logits_ + static_cast<std::size_t>(gr) * vocab_, vocab_ * sizeof(float),
-                            hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+    const float* src = gr == adjusted_row_ ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
+    checkHip(hipMemcpyAsync(row_host_.data(), src, vocab_ * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     return row_host_.data();
 }
 
 float DeviceRows::logitAt(std::uint32_t gr, std::uint32_t t) {
     if (gr >= rows_ || t >= vocab_) throw DeviceError("logitAt", WS_E_INVALID, "logitAt: out of range");
-    if (gr == adjusted_row_) return row_host_[t];
     float v = 0;
     auto stream = static_cast<hipStream_t>(stream_);
-    checkHip(hipMemcpyAsync(&v, logits_ + static_cast<std::size_t>(gr) * vocab_ + t, sizeof v, hipMemcpyDeviceToHost, stream),
-             "hipMemcpyAsync");
+    const float* src = gr == adjusted_row_ ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
+    checkHip(hipMemcpyAsync(&v, src + t, sizeof v, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     return v;
 }
