@@ -30,6 +30,7 @@ struct BatchPlan {
     uint32_t patch_cap;
     uint32_t lds_ab;
     uint32_t lds_cnt;
+    uint32_t lds_tie;
     uint32_t lds_total;
     bool fused;
     uint64_t workspace;
@@ -71,6 +72,13 @@ BatchPlan plan_batch(const ws_batch* b) {
         p.lds_cnt = 0;
     }
     if (total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
+    // spare room for the tie bitmap (vocab / 32 words + 16-bit prefixes), when there is any
+    const uint64_t tie_bytes = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
+    p.lds_tie = 0;
+    if (total + tie_bytes + 4096u <= kMaxLds) {
+        p.lds_tie = static_cast<uint32_t>((total + 15u) & ~uint64_t{15});
+        total = p.lds_tie + tie_bytes;
+    }
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
@@ -216,6 +224,7 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.tol = b->tol > 1e-6 ? b->tol : 1e-6;  // the histogram masses are good to ~5e-7 relative: no decision closer than that is trusted
     a.lds_ab = p.lds_ab;
     a.lds_cnt = p.lds_cnt;
+    a.lds_tie = p.lds_tie;
     if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
     if (!attr_set) {

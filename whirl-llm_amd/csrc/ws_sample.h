@@ -77,6 +77,8 @@ struct BatchArgs {
     uint32_t kept_cap;
     double tol;
     uint32_t lds_ab;   // bytes of the LDS region shared by the histogram / sort keys / masses
+    uint32_t lds_tie;  // byte offset of a spare id bitmap + prefix (vocab / 32 words + as many 16-bit counts) for sorting heavy
+                       // ties by id, 0 when the LDS has no room for it
     uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
 };
 
@@ -1083,11 +1085,19 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             constexpr uint32_t kTieBins = 32;
             __shared__ uint32_t bin_lo[kTieBins], bin_hi[kTieBins];
             const bool spot_ties = nb0 + nb1 <= kTieBins;
+            // (buckets of more than kMaxInBucket keys are listed further down, up to kMaxBig of them)
+            constexpr uint32_t kMaxBig = 8;
+            __shared__ uint32_t big_bucket[kMaxBig], big_lo[kMaxBig], big_hi[kMaxBig];
             for (uint32_t b = t; b <= nbk; b += WS_BLOCK) bcnt[b] = 0u;
             if (t < kTieBins) {
                 bin_lo[t] = 0xffffffffu;
                 bin_hi[t] = 0u;
             }
+            if (t < kMaxBig) {
+                big_lo[t] = 0xffffffffu;
+                big_hi[t] = 0u;
+            }
+            if (t == 0) s_u[6] = 0;
             __syncthreads();
             uint32_t rb[kCh];
             float tcs[kCh];
@@ -1123,6 +1133,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             __syncthreads();
             // exclusive scan of the counts (a few consecutive buckets per thread) and the largest bucket
             constexpr uint32_t kPB = (kMaxBuckets + WS_BLOCK - 1) / WS_BLOCK;
+            // Buckets of more than kMaxInBucket keys are listed: where all keys of such a bucket carry one logit - the
+            // heavy ties of coarse logits - they are ranked by token id through a bitmap of the ids.
             uint32_t local[kPB], sum = 0, biggest = 0;
 #pragma unroll
             for (uint32_t j = 0; j < kPB; ++j) {
@@ -1130,6 +1142,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 local[j] = b < nbk ? bcnt[b] : 0u;
                 sum += local[j];
                 biggest = max(biggest, local[j]);
+                if (local[j] > kMaxInBucket) {
+                    const uint32_t slot = atomicAdd(&s_u[6], 1u);
+                    if (slot < kMaxBig) big_bucket[slot] = b;
+                }
             }
             uint32_t total;
             uint32_t run = block_excl_scan(sum, red_u, &total);
@@ -1142,25 +1158,79 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
             if (t == 0) bcnt[nbk] = total;
             __syncthreads();
-            if (biggest <= kMaxInBucket) {  // uniform
+            const uint32_t n_big = s_u[6];
+            bool ok = biggest <= kMaxInBucket;
+            int big_of[kCh];  // index of the key's bucket in the list of big buckets, -1 for an ordinary bucket
 #pragma unroll
-                for (int q = 0; q < kCh; ++q)
-                    if (q * WS_BLOCK + t < n_list) tmp[bcnt[bucket[q]] + arrival[q]] = key[q];
-                __syncthreads();
+            for (int q = 0; q < kCh; ++q) big_of[q] = -1;
+            if (!ok && n_big <= kMaxBig && A.lds_tie) {  // uniform
+                // one logit per big bucket?
 #pragma unroll
                 for (int q = 0; q < kCh; ++q) {
                     if (q * WS_BLOCK + t >= n_list) continue;
+                    for (uint32_t k = 0; k < n_big; ++k)
+                        if (big_bucket[k] == bucket[q]) big_of[q] = static_cast<int>(k);
+                    if (big_of[q] >= 0) {
+                        atomicMin(&big_lo[big_of[q]], static_cast<uint32_t>(key[q] >> 32));
+                        atomicMax(&big_hi[big_of[q]], static_cast<uint32_t>(key[q] >> 32));
+                    }
+                }
+                __syncthreads();
+                ok = true;
+                for (uint32_t k = 0; k < n_big; ++k) ok = ok && big_lo[k] == big_hi[k];
+            }
+            if (ok) {  // uniform; keys[] has not been written so far, so the comparison sorts below can still take over
+#pragma unroll
+                for (int q = 0; q < kCh; ++q)
+                    if (q * WS_BLOCK + t < n_list && big_of[q] < 0) tmp[bcnt[bucket[q]] + arrival[q]] = key[q];
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < kCh; ++q) {
+                    if (q * WS_BLOCK + t >= n_list || big_of[q] >= 0) continue;
                     const uint32_t b0 = bcnt[bucket[q]], b1 = bcnt[bucket[q] + 1u];
                     uint32_t before = 0;
                     for (uint32_t j = b0; j < b1; ++j) before += tmp[j] > key[q] ? 1u : 0u;
                     keys[b0 + before] = key[q];  // every key was read into registers before the first barrier above
+                }
+                // a big bucket of equal logits: its keys in ascending id order = set the ids' bits, count the bits below
+                uint32_t* tie_bits = reinterpret_cast<uint32_t*>(lds + A.lds_tie);
+                uint16_t* tie_pref = reinterpret_cast<uint16_t*>(lds + A.lds_tie + nW * 4u);
+                for (uint32_t k = 0; k < (biggest > kMaxInBucket ? n_big : 0u); ++k) {
+                    __syncthreads();
+                    for (uint32_t w = t; w < nW; w += WS_BLOCK) tie_bits[w] = 0u;
+                    __syncthreads();
+#pragma unroll
+                    for (int q = 0; q < kCh; ++q)
+                        if (big_of[q] == static_cast<int>(k)) {
+                            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
+                            atomicOr(&tie_bits[id >> 5], 1u << (id & 31u));
+                        }
+                    __syncthreads();
+                    const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
+                    const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
+                    uint32_t mine = 0;
+                    for (uint32_t w = w0; w < w1; ++w) mine += __popc(tie_bits[w]);
+                    uint32_t all;
+                    uint32_t at = block_excl_scan(mine, red_u, &all);
+                    for (uint32_t w = w0; w < w1; ++w) {
+                        tie_pref[w] = static_cast<uint16_t>(at);
+                        at += __popc(tie_bits[w]);
+                    }
+                    __syncthreads();
+#pragma unroll
+                    for (int q = 0; q < kCh; ++q)
+                        if (big_of[q] == static_cast<int>(k)) {
+                            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
+                            const uint32_t rank = static_cast<uint32_t>(tie_pref[id >> 5]) + __popc(tie_bits[id >> 5] & ((1u << (id & 31u)) - 1u));
+                            keys[bcnt[bucket[q]] + rank] = key[q];
+                        }
                 }
                 __syncthreads();
                 sorted = true;
             }
         }
     }
-    constexpr int kMergeCh = 3;  // keys per thread the merge sort takes
+    constexpr int kMergeCh = 6;  // keys per thread the merge sort takes (3072 keys; beyond that the bitonic sort)
     if (sorted) {
     } else if (n_list <= kMergeCh * WS_BLOCK) {
         // Few candidates (the usual case): one or two per thread. Each wave ranks 64 keys among themselves by counting
