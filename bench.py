@@ -135,7 +135,7 @@ def cpu_baseline(c, budget_s=9.0, budget_all_s=6.0):
 
 def run_workload(name, steps, warmup, check_rows):
     import gpu_cases as gc
-    make = dict(tile=gc.make_tile, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=lambda: gc.make_cfg5(rows=256))[name]
+    make = dict(tile=gc.make_tile, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
     c = make()
     smp, wall_ms, kern_ms = time_gpu(c, steps, warmup)
     par = parity_sample(c, smp, check_rows) if check_rows else None
