@@ -262,7 +262,19 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     for (int bt = 0; bt < NB; ++bt) {
         const int slot = bt % kRing;
         if (bt + 2 < NB) load(bt + 2, (bt + 2) % kRing);
-        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the work on this batch
+        // The touched words of the whole batch are read before its first histogram update: LDS operations of a wave
+        // complete in order, so a read placed behind the updates would make the wave wait for all of them.
+        uint32_t tws[kBatch], wps[kBatch];
+        if (TOUCHED) {
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
+                const uint32_t word = ((j < nv ? j : nv - 1u) * PER) >> 5;
+                tws[u] = rv.touched[word];
+                wps[u] = rv.wprefix[word];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch and those reads above the work on this batch
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
@@ -288,9 +300,9 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
                 if (TOUCHED) {
                     // the running maximum skips vectors with touched tokens: their untouched tokens are looked at
                     // when the touched ones are collected
-                    const uint32_t sh = (j * PER) & 31u, tw = rv.touched[(j * PER) >> 5];
+                    const uint32_t sh = (j * PER) & 31u, tw = tws[u];
                     if ((tw >> sh) & (PER == 4 ? 15u : 255u)) {
-                        const uint32_t r = static_cast<uint32_t>(rv.wprefix[(j * PER) >> 5]) + __popc(tw & ((1u << sh) - 1u));
+                        const uint32_t r = wps[u] + __popc(tw & ((1u << sh) - 1u));
                         if (r < stage_cap) stage[r] = q[slot][u];
                     } else {
                         m = fmaxf(m, vm);
@@ -447,8 +459,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ double red_d[WS_WAVES];
     __shared__ uint32_t s_cnt;
     __shared__ double s_d[8];
+    __shared__ double s_exp[128];  // kExpHi, kExpLo
     __shared__ uint32_t s_u[8];
-    __shared__ uint64_t s_key;
 
     const uint32_t row = blockIdx.x;
     const uint32_t t = threadIdx.x;
@@ -468,6 +480,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double top_p = A.top_p ? A.top_p[row] : 1.0;
     const double min_p = A.min_p ? A.min_p[row] : 0.0;
     const double tol = A.tol;
+    const uint64_t seed = A.seed[row], step = A.step[row];
+    // exp(-b / 64) tables of the histogram scan: fetched now, parked in LDS before the sweep, so that the scan does not
+    // wait for global memory in the middle of the row's tail
+    const double exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);
     uint32_t flags = 0;
 
     RowView rv;
@@ -694,6 +710,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
 
     WS_MARK(0);
+    if (t < 128) s_exp[t] = exp_tab;  // read by the histogram scan, many barriers from here
     const float c64 = inv_t * 64.f;
     float anchor = 0.f;  // bins are measured down from here: the row maximum, or a provisional bound above it
     float aq = 0.f;      // anchor_product(anchor, c64)
@@ -791,14 +808,43 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (b == kBins - 1) c[j] -= tail_fix;  // streamed there as NaN, replayed into their own bins
             const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
             // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail bin carries none
-            ms[j] = (c[j] && b < kBins - 1) ? kExpHi[b >> 6] * kExpLo[b & 63] * (static_cast<double>(c[j]) - fix) * to_max : 0.0;
+            ms[j] = (c[j] && b < kBins - 1) ? s_exp[b >> 6] * s_exp[64 + (b & 63)] * (static_cast<double>(c[j]) - fix) * to_max : 0.0;
             csum += c[j];
             msum += ms[j];
         }
-        uint32_t ctot;
-        double mtot;
-        uint32_t cb = block_excl_scan(csum, red_u, &ctot);
-        double mb = block_excl_scan(msum, red_d, &mtot);  // its barriers separate the reads of hist above from the writes below
+        // exclusive scan of (count, mass) over the threads, both in one go; its barriers separate the reads of hist
+        // above from the writes below
+        uint32_t cinc = csum;
+        double minc = msum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t cu = __shfl_up(cinc, o);
+            const double mu = __shfl_up(minc, o);
+            if (lane_id() >= o) {
+                cinc += cu;
+                minc += mu;
+            }
+        }
+        __syncthreads();
+        if (lane_id() == 63) {
+            red_u[wave_id()] = cinc;
+            red_d[wave_id()] = minc;
+        }
+        __syncthreads();
+        uint32_t ctot = 0, cb = cinc - csum;
+        double mtot = 0, mbase = 0;
+#pragma unroll
+        for (int w = 0; w < WS_WAVES; ++w) {
+            const uint32_t cw = red_u[w];
+            const double mw = red_d[w];
+            if (w < wave_id()) {
+                cb += cw;
+                mbase += mw;
+            }
+            ctot += cw;
+            mtot += mw;
+        }
+        double mb = mbase + minc - msum;
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
             pc[kPT * t + j] = cb;
@@ -906,7 +952,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             minp_in_list = topp_in_list = true;
         }
         // bounds of the kept mass -> bins the draw can land in
-        const double u = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
+        const double u = batch_uniform(A.rng, seed, row, step, 0);
         double zlo, zhi;
         if (r1hi >= r1lo) {
             zlo = pm[r1lo];
@@ -1311,135 +1357,109 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
     WS_MARK(5);
 
-    // sorted entry j * WS_BLOCK + t belongs to thread t: with the usual few hundred candidates every thread has one
-    double e[kPT], inc[kPT], exc[kPT];
-    uint32_t pos[kPT];
-    bool live[kPT];
+    // Exact masses of the sorted candidates and their running sum: sorted entry j * WS_BLOCK + t belongs to thread t
+    // (with the usual few hundred candidates every thread has one), ps[i] = sum of the masses of entries 0..i. From
+    // there every wave works the cuts and the draw out by itself, reading ps[] and keys[] with 64-way searches: all
+    // waves reach the same results and no barrier is needed any more.
+    double* ps = emass;
     {
         double carry = 0;
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
             const uint32_t i = j * WS_BLOCK + t;
-            live[j] = i < n_list;
-            e[j] = exc[j] = inc[j] = 0;
             if (static_cast<uint32_t>(j) * WS_BLOCK < n_list) {  // uniform
-                if (live[j]) {
+                double ej = 0;
+                if (i < n_list) {
                     const float x = unkey32(static_cast<uint32_t>(keys[i] >> 32));
-                    const float d = __fsub_rn(m, x);
-                    e[j] = exp(-(static_cast<double>(d) * static_cast<double>(inv_t)));
+                    ej = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
                 }
                 double tot;
-                exc[j] = carry + block_excl_scan(e[j], red_d, &tot);
-                inc[j] = exc[j] + e[j];
+                const double ex = carry + block_excl_scan(ej, red_d, &tot);
+                if (i < n_list) ps[i] = ex + ej;
                 carry += tot;
-                if (live[j] && i + 1 == n_r0) s_d[1] = inc[j];
             }
         }
         __syncthreads();
-        // masses of range 1 restart at its base: subtract the running sum at the end of range 0
-        const double at_r0_end = n_r0 ? s_d[1] : 0.0;
-#pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            const uint32_t i = j * WS_BLOCK + t;
-            if (i < n_r0) {
-                pos[j] = c0base + i;
-                exc[j] += m0base;
-                inc[j] += m0base;
-            } else {
-                pos[j] = c1base + (i - n_r0);
-                exc[j] = m1base + (exc[j] - at_r0_end);
-                inc[j] = m1base + (inc[j] - at_r0_end);
-            }
-        }
     }
-
     WS_MARK(6);
+    const double at_r0_end = n_r0 ? ps[n_r0 - 1u] : 0.0;  // masses of range 1 restart at its base
+    auto pos_of = [&](uint32_t i) { return i < n_r0 ? c0base + i : c1base + (i - n_r0); };  // rank in the row of entry i
+    auto inc_of = [&](uint32_t i) { return i < n_r0 ? m0base + ps[i] : m1base + (ps[i] - at_r0_end); };  // mass up to and with entry i
+    auto exc_of = [&](uint32_t i) {  // mass ranked before entry i
+        const double before = i ? ps[i - 1u] : 0.0;
+        return i < n_r0 ? m0base + before : m1base + (before - at_r0_end);
+    };
+    auto mass_of = [&](uint32_t i) {
+        const float x = unkey32(static_cast<uint32_t>(keys[i] >> 32));
+        return exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
+    };
+    // entry that holds rank `p` of the row, or n_list when that rank was not gathered
+    auto entry_of = [&](uint32_t p) {
+        if (p >= c0base && p - c0base < n_r0) return p - c0base;
+        if (has_r1 && p >= c1base && p - c1base < n_r1) return n_r0 + (p - c1base);
+        return n_list;
+    };
+    // first entry for which `reached` holds (it holds from some entry on); n_list when for none. Two rounds of 64 probes.
+    auto first_entry = [&](auto&& reached) -> uint32_t {
+        const uint32_t lane = static_cast<uint32_t>(lane_id());
+        const uint64_t coarse = __ballot(reached(min(64u * lane + 63u, n_list - 1u)));
+        if (!coarse) return n_list;
+        const uint32_t base = 64u * static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(coarse)) - 1);
+        const uint32_t i = min(base + lane, n_list - 1u);
+        const uint64_t fine = __ballot(reached(i));
+        return base + static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(fine)) - 1);
+    };
+
     // ------------------------------------------------------------------ cuts
     double mg_top_p = 1.0, mg_min_p = 1.0, mg_draw = 1.0;
-    // top-k: mass of the first n1 candidates (prefix mode)
+    // top-k: mass of the first n1 candidates (prefix mode: one range that starts at rank 0)
     double M1 = Z;
     if (prefix_mode) {
-#pragma unroll
-        for (int j = 0; j < kPT; ++j)
-            if (live[j] && pos[j] == n1 - 1) s_d[2] = inc[j];
-        __syncthreads();
-        M1 = s_d[2];
+        M1 = inc_of(n1 - 1u);
         X = top_p * M1;
     }
     uint32_t n2 = n1;
     if (use_top_p && topp_in_list) {
-        if (t == 0) {
-            s_u[0] = 0xffffffffu;
-            s_d[3] = 1.0;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < kPT; ++j)
-            if (live[j] && pos[j] < n1 && inc[j] >= X && !(exc[j] >= X) && e[j] > 0.0) {
-                s_u[0] = pos[j] + 1;
-                s_d[3] = fmin(inc[j] - X, pos[j] > 0 ? X - exc[j] : X) / X;
+        const uint32_t i = first_entry([&](uint32_t k) { return inc_of(k) >= X; });
+        bool found = false;
+        if (i < n_list) {
+            const double in = inc_of(i), ex = exc_of(i);
+            const uint32_t p = pos_of(i);
+            if (p < n1 && !(ex >= X) && in > ex) {
+                found = true;
+                n2 = p + 1u;
+                mg_top_p = fmin(in - X, p > 0 ? X - ex : X) / X;
             }
-        __syncthreads();
-        if (s_u[0] != 0xffffffffu) {
-            n2 = s_u[0];
-            mg_top_p = s_d[3];
-        } else {  // rounding: the cut falls just past the gathered bins
+        }
+        if (!found) {  // rounding: the cut falls just past the gathered bins
             n2 = prefix_mode ? n1 : min(n1, has_r1 ? c1base + n_r1 : c0base + n_r0);
             mg_top_p = 0.0;
         }
     }
     uint32_t n3 = n2;
-    if (use_min_p) {
-        // candidates are in descending order, so those at or above the floor form a prefix: count them
-        uint32_t ok = 0;
+    if (use_min_p && minp_in_list) {
+        // candidates are in descending order, so those at or above the floor form a prefix of the gathered entries;
+        // entries ranked before the min-p bins pass by construction
+        const uint32_t passed = first_entry([&](uint32_t k) { return !(mass_of(k) >= min_p); });
         double near = 1.0;
-#pragma unroll
-        for (int j = 0; j < kPT; ++j)
-            if (live[j]) {
-                ok += e[j] >= min_p;
-                near = fmin(near, fabs(e[j] - min_p) / min_p);
-            }
-        // ranges are contiguous in rank only inside themselves: entries before the min-p bins pass by construction
-        const uint32_t passed = block_sum(ok, red_u);
-        double nr = near;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) nr = fmin(nr, __shfl_xor(nr, o));
-        __syncthreads();
-        if (lane_id() == 0) red_d[wave_id()] = nr;
-        __syncthreads();
-        nr = red_d[0];
-        for (int w = 1; w < WS_WAVES; ++w) nr = fmin(nr, red_d[w]);
-        __syncthreads();
-        if (minp_in_list) {
-            uint32_t n3p;
-            if (has_r1)
-                n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
-            else
-                n3p = c0base + passed;
-            if (passed == n_list && !prefix_mode) {
-                // every gathered candidate passes: the floor lies past the gathered bins only by rounding
-            }
-            n3 = min(n2, n3p);
-            if (n3 < 1u) n3 = 1u;
-            mg_min_p = nr;
-        }
+        if (passed > 0u) near = fmin(near, fabs(mass_of(passed - 1u) - min_p) / min_p);
+        if (passed < n_list) near = fmin(near, fabs(mass_of(passed) - min_p) / min_p);
+        uint32_t n3p;
+        if (has_r1)
+            n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
+        else
+            n3p = c0base + passed;
+        n3 = min(n2, n3p);
+        if (n3 < 1u) n3 = 1u;
+        mg_min_p = near;
     }
     // kept mass = inclusive mass at rank n3 - 1; when that rank is just before a gathered range, the range's base
-    if (t == 0) s_u[1] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < kPT; ++j)
-        if (live[j] && pos[j] == n3 - 1) {
-            s_d[4] = inc[j];
-            s_key = keys[j * WS_BLOCK + t];
-            s_u[1] = 1;
-        }
-    __syncthreads();
+    const uint32_t i_last = entry_of(n3 - 1u);
     double Zk;
     uint64_t kept_key;
-    if (s_u[1]) {
-        Zk = s_d[4];
-        kept_key = s_key;
+    if (i_last < n_list) {
+        Zk = inc_of(i_last);
+        kept_key = keys[i_last];
     } else if (has_r1 && n3 == c1base) {  // the cut falls on the upper edge of range 1: everything in earlier bins
         Zk = m1base;
         kept_key = static_cast<uint64_t>(first_key_before_bin(aq, c64, m, r1lo)) << 32;
@@ -1452,41 +1472,32 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     // ------------------------------------------------------------------ draw
-    const double u = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
+    const double u = batch_uniform(A.rng, seed, row, step, 0);
     const double target = u * Zk;
-    if (t == 0) {
-        s_u[2] = 0xffffffffu;
-        s_u[3] = 0xffffffffu;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < kPT; ++j) {
-        if (!live[j] || pos[j] >= n3) continue;
-        if (inc[j] > target && !(exc[j] > target) && e[j] > 0.0) {
-            s_u[2] = 0xffffffffu - static_cast<uint32_t>(keys[j * WS_BLOCK + t]);
-            s_d[5] = e[j];
-            s_d[6] = fmin(inc[j] - target, pos[j] > 0 ? target - exc[j] : 1e300) / Zk;
+    int32_t token = -1;
+    double ptok = 0;
+    {
+        const uint32_t i = first_entry([&](uint32_t k) { return inc_of(k) > target; });
+        bool found = false;
+        if (i < n_list) {
+            const double in = inc_of(i), ex = exc_of(i);
+            const uint32_t p = pos_of(i);
+            if (p < n3 && !(ex > target) && in > ex) {
+                found = true;
+                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(keys[i]));
+                ptok = mass_of(i) / Zk;
+                mg_draw = fmin(in - target, p > 0 ? target - ex : 1e300) / Zk;
+            }
         }
-        if (pos[j] == n3 - 1) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
-            s_u[3] = 0xffffffffu - static_cast<uint32_t>(keys[j * WS_BLOCK + t]);
-            s_d[7] = e[j];
+        if (!found) {
+            if (i_last < n_list) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
+                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(keys[i_last]));
+                ptok = mass_of(i_last) / Zk;
+                mg_draw = 0.0;
+            } else {
+                flags |= kOverflow;
+            }
         }
-    }
-    __syncthreads();
-    int32_t token;
-    double ptok;
-    if (s_u[2] != 0xffffffffu) {
-        token = static_cast<int32_t>(s_u[2]);
-        ptok = s_d[5] / Zk;
-        mg_draw = s_d[6];
-    } else if (s_u[3] != 0xffffffffu) {
-        token = static_cast<int32_t>(s_u[3]);
-        ptok = s_d[7] / Zk;
-        mg_draw = 0.0;
-    } else {
-        token = -1;
-        ptok = 0;
-        flags |= kOverflow;
     }
     // zero-mass tail candidates a top-k kept (no top-p / min-p cut them away again)
     const uint32_t tail_extra = (!use_top_p && !use_min_p && n3 == n1) ? n1_asked - n1 : 0u;
