@@ -81,6 +81,24 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     for (int w = 1; w < WS_WAVES; ++w) r = fmaxf(r, red[w]);
     return r;
 }
+// two maxima at once (a, b are replaced by the block's); red_a / red_b: WS_WAVES entries each
+__device__ __forceinline__ void block_max2(float& a, float& b, float* red_a, float* red_b) {
+    a = wave_max(a);
+    b = wave_max(b);
+    __syncthreads();
+    if (lane_id() == 0) {
+        red_a[wave_id()] = a;
+        red_b[wave_id()] = b;
+    }
+    __syncthreads();
+    a = red_a[0];
+    b = red_b[0];
+#pragma unroll
+    for (int w = 1; w < WS_WAVES; ++w) {
+        a = fmaxf(a, red_a[w]);
+        b = fmaxf(b, red_b[w]);
+    }
+}
 __device__ __forceinline__ uint32_t block_min(uint32_t v, uint32_t* red) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = min(v, static_cast<uint32_t>(__shfl_xor(v, o)));
@@ -118,15 +136,34 @@ __device__ __forceinline__ T block_sum(T v, T* red) {
     return r;
 }
 
+// ---- wave inclusive scan (sum of lanes 0..own) on the data-parallel-primitive path: four shifts inside each row of
+// 16 lanes, then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3. Lanes without a source,
+// and rows a step leaves out, add 0. Six dependent vector instructions instead of six trips through the LDS crossbar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROW_MASK, 0xf, true));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_or_zero(double v) {
+    const uint64_t b = static_cast<uint64_t>(__double_as_longlong(v));
+    const uint32_t lo = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b)), hi = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b >> 32));
+    return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
+}
+template <class T>
+__device__ __forceinline__ T wave_incl_scan(T v) {
+    v += dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // ---- block exclusive scan of one value per thread (thread order); returns the exclusive prefix, *total = block sum
 template <class T>
 __device__ __forceinline__ T block_excl_scan(T v, T* red, T* total) {
-    T inc = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const T up = __shfl_up(inc, o);
-        if (lane_id() >= o) inc += up;
-    }
+    const T inc = wave_incl_scan(v);
     __syncthreads();
     if (lane_id() == 63) red[wave_id()] = inc;
     __syncthreads();

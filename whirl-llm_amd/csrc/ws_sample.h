@@ -127,7 +127,7 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
     const uint32_t per = rv.dtype == 0 ? 4u : 8u;  // elements per 128-bit load
-    const uint32_t nv = rv.vec ? V / per : 0u;
+    const uint32_t nv = rv.vec ? V >> (rv.dtype == 0 ? 2 : 3) : 0u;  // per is 4 or 8: shifts, never a division
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     constexpr uint32_t kStep = kBatch * WS_BLOCK;
     struct Batch {
@@ -334,8 +334,8 @@ __device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, flo
 
 // token index of half `half` of cache register k of thread t (the layout fused_pass_impl writes)
 __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t half) {
-    const uint32_t per = dtype == 0 ? 4u : 8u, pairs = per / 2u;
-    return ((k / pairs) * WS_BLOCK + threadIdx.x) * per + 2u * (k % pairs) + half;
+    const uint32_t lp = dtype == 0 ? 1u : 2u;  // log2 of the registers per vector; shifts, never a division
+    return (((k >> lp) * WS_BLOCK + threadIdx.x) << (lp + 1u)) + 2u * (k & ((1u << lp) - 1u)) + half;
 }
 
 // Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range): its index goes
@@ -369,12 +369,7 @@ __device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&ca
         mine += __popc(acc);
         __builtin_amdgcn_sched_barrier(0);  // one group at a time: a wider scheduling window costs more registers than it hides
     }
-    uint32_t inc = mine;  // inclusive prefix over the wave
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const uint32_t up = __shfl_up(inc, o);
-        if (lane_id() >= o) inc += up;
-    }
+    const uint32_t inc = wave_incl_scan(mine);  // inclusive prefix over the wave
     uint32_t base = 0;
     if (lane_id() == 63 && inc) base = atomicAdd(n_list, inc);
     uint32_t slot = __shfl(base, 63) + inc - mine;
@@ -481,6 +476,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double min_p = A.min_p ? A.min_p[row] : 0.0;
     const double tol = A.tol;
     const uint64_t seed = A.seed[row], step = A.step[row];
+    const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
     // exp(-b / 64) tables of the histogram scan: fetched now, parked in LDS before the sweep, so that the scan does not
     // wait for global memory in the middle of the row's tail
     const double exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);
@@ -518,6 +514,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
         for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
         __syncthreads();
+        WS_MARK(16);
 #pragma unroll
         for (int k = 0; k < kHid; ++k)
             if (hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
@@ -530,16 +527,35 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
         }
         __syncthreads();
+        WS_MARK(17);
         // exclusive popcount prefix per bitmap word: contiguous chunk of words per thread
         const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
         const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
-        uint32_t local = 0;
-        for (uint32_t w = w0; w < w1; ++w) local += __popc(touched[w]);
+        constexpr uint32_t kChunkRegs = 10;  // rows the single-sweep kernel takes: 163840 / 32 / 512 words per thread
         uint32_t n_uniq;
-        uint32_t run = block_excl_scan(local, red_u, &n_uniq);
-        for (uint32_t w = w0; w < w1; ++w) {
-            wprefix[w] = static_cast<uint16_t>(run);
-            run += __popc(touched[w]);
+        if (FUSED && chunk <= kChunkRegs) {
+            // the thread's words in registers: independent reads, one trip to LDS instead of one per word and pass
+            uint32_t wd[kChunkRegs];
+            uint32_t local = 0;
+#pragma unroll
+            for (uint32_t k = 0; k < kChunkRegs; ++k) {
+                wd[k] = w0 + k < w1 ? touched[w0 + k] : 0u;
+                local += __popc(wd[k]);
+            }
+            uint32_t run = block_excl_scan(local, red_u, &n_uniq);
+#pragma unroll
+            for (uint32_t k = 0; k < kChunkRegs; ++k) {
+                if (w0 + k < w1) wprefix[w0 + k] = static_cast<uint16_t>(run);
+                run += __popc(wd[k]);
+            }
+        } else {
+            uint32_t local = 0;
+            for (uint32_t w = w0; w < w1; ++w) local += __popc(touched[w]);
+            uint32_t run = block_excl_scan(local, red_u, &n_uniq);
+            for (uint32_t w = w0; w < w1; ++w) {
+                wprefix[w] = static_cast<uint16_t>(run);
+                run += __popc(touched[w]);
+            }
         }
         uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);  // low 20 bits: history count, high 12: bias entries
         uint32_t* first = cnt + A.patch_cap;               // index of the id's first bias entry
@@ -549,6 +565,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             pv[r] = 0.f;
         }
         __syncthreads();
+        WS_MARK(18);
         rv.touched = touched;
         // without a bias list the second table is free from the start: it takes the token id of each rank right away
         const bool ids_now = FUSED && nb == 0;
@@ -588,7 +605,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // single-sweep kernel after the sweep, when the row has just come through the caches.
     auto gather_and_adjust = [&](const uint4* stage, uint32_t stage_cap) {
         if (!n_touched) return;
-        const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+        const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
         const int32_t* hist_ids = A.hist + h0;
         const int32_t* bias_ids = A.bias_ids + b0;
         const float* bias_vals = A.bias_vals + b0;
@@ -609,12 +626,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
                     al[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
-                    if (rv.vec && i < (V / per) * per) {
+                    if (rv.vec && i < (V & ~(per - 1u))) {
                         // the token's whole 128-bit vector: staged by the sweep under the rank of the vector's first
                         // touched token, else fetched
                         const uint32_t vb = i & ~(per - 1u), tw = touched[i >> 5];
                         const uint32_t rf = static_cast<uint32_t>(wprefix[i >> 5]) + __popc(tw & ((1u << (vb & 31u)) - 1u));
-                        vec[k] = rf < stage_cap ? stage[rf] : static_cast<const uint4*>(rv.base)[i / per];
+                        vec[k] = rf < stage_cap ? stage[rf] : static_cast<const uint4*>(rv.base)[i >> lper];
                     } else {
                         const uint32_t b = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
                                                          : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
@@ -626,7 +643,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     if (id[k] >= V) continue;
                     const uint32_t i = id[k];
                     const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
-                    const bool whole = rv.vec && i < (V / per) * per;
+                    const bool whole = rv.vec && i < (V & ~(per - 1u));
                     if (!whole) bits[k] = w[0];
                     else bits[k] = rv.dtype == 0 ? w[i & 3u] : ((i & 1u) ? w[(i & 7u) >> 1] & 0xffff0000u : w[(i & 7u) >> 1] << 16);
                     pv[rank_of(rv, i)] = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits[k]), -INFINITY) : -INFINITY;
@@ -650,8 +667,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         fetch4(hist_ids, nh, true);
         fetch4(bias_ids, nb, false);
         __syncthreads();
+        WS_MARK(19);
         {
-            const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
             float ma = -INFINITY;
             for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
                 const uint32_t cw = cnt[r], c = cw & 0xfffffu;
@@ -674,17 +691,23 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 cnt[r] = __float_as_uint(raw);
                 ma = fmaxf(ma, x);
             }
-            m_adj = block_max(ma, red_f);
-            m_near = block_max(mu, red_f);
+            WS_MARK(20);
+            block_max2(ma, mu, red_f, reinterpret_cast<float*>(red_u));  // its barriers also end the reads of first[] above
+            m_adj = ma;
+            m_near = mu;
         }
-        if (FUSED && nb) {  // with a bias list the second table held the first-entry indices until the adjustment above
-            for (uint32_t j = t; j < nh; j += WS_BLOCK) {
-                const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
-                if (id < V) first[rank_of(rv, id)] = id;
-            }
-            for (uint32_t j = t; j < nb; j += WS_BLOCK) {
-                const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
-                if (id < V) first[rank_of(rv, id)] = id;
+        if (FUSED && nb) {
+            // with a bias list the second table held the first-entry indices until the adjustment above; now it takes
+            // the token id of each rank, read off the bitmap: rank = the word's prefix + the bit's place among its set bits
+            const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
+            const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
+            for (uint32_t w = w0; w < w1; ++w) {
+                uint32_t bits = touched[w];
+                uint32_t r = wprefix[w];
+                while (bits) {
+                    first[r++] = (w << 5) + static_cast<uint32_t>(__ffs(bits)) - 1u;
+                    bits &= bits - 1u;
+                }
             }
         }
         __syncthreads();
@@ -814,17 +837,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         // exclusive scan of (count, mass) over the threads, both in one go; its barriers separate the reads of hist
         // above from the writes below
-        uint32_t cinc = csum;
-        double minc = msum;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t cu = __shfl_up(cinc, o);
-            const double mu = __shfl_up(minc, o);
-            if (lane_id() >= o) {
-                cinc += cu;
-                minc += mu;
-            }
-        }
+        const uint32_t cinc = wave_incl_scan(csum);
+        const double minc = wave_incl_scan(msum);
         __syncthreads();
         if (lane_id() == 63) {
             red_u[wave_id()] = cinc;
@@ -1066,14 +1080,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
             // are re-read after the batch, from the cache lines the batch has just pulled in
             uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
-            const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
             stream_row(
                 rv, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
                 [&](uint32_t j0, uint32_t i_tail) {
                     while (hit) {
                         const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
                         hit &= hit - 1u;
-                        const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot / per) * WS_BLOCK + t) * per + (slot % per);
+                        const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot >> lper) * WS_BLOCK + t) * per + (slot & (per - 1u));
                         push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
                     }
                 });
