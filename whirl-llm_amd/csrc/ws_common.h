@@ -31,27 +31,60 @@ __device__ __forceinline__ uint64_t key64(float f, uint32_t id) {
     return (static_cast<uint64_t>(key32(f)) << 32) | static_cast<uint64_t>(0xffffffffu - id);
 }
 
-// ---- wave reductions (xor butterflies; every lane gets the result)
+// ---- wave inclusive scan (sum of lanes 0..own) on the data-parallel-primitive path: four shifts inside each row of
+// 16 lanes, then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3. Lanes without a source,
+// and rows a step leaves out, add 0. Six dependent vector instructions instead of six trips through the LDS crossbar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROW_MASK, 0xf, true));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_or_zero(double v) {
+    const uint64_t b = static_cast<uint64_t>(__double_as_longlong(v));
+    const uint32_t lo = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b)), hi = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b >> 32));
+    return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+    return __uint_as_float(dpp_or_zero<CTRL, ROW_MASK>(__float_as_uint(v)));
+}
+template <class T>
+__device__ __forceinline__ T wave_incl_scan(T v) {
+    v += dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// the same steps with a lane's own value where there is no source: lane 63 ends with the reduction of the wave
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_self(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ uint32_t last_lane(uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63)); }
+__device__ __forceinline__ float last_lane(float v) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63)); }
+__device__ __forceinline__ double last_lane(double v) {
+    const uint64_t b = static_cast<uint64_t>(__double_as_longlong(v));
+    const uint64_t r = (static_cast<uint64_t>(last_lane(static_cast<uint32_t>(b >> 32))) << 32) | last_lane(static_cast<uint32_t>(b));
+    return __longlong_as_double(static_cast<long long>(r));
+}
+
+// ---- wave reductions (every lane gets the result)
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
+    v = fmaxf(v, dpp_or_self<0x111, 0xf>(v));
+    v = fmaxf(v, dpp_or_self<0x112, 0xf>(v));
+    v = fmaxf(v, dpp_or_self<0x114, 0xf>(v));
+    v = fmaxf(v, dpp_or_self<0x118, 0xf>(v));
+    v = fmaxf(v, dpp_or_self<0x142, 0xa>(v));
+    v = fmaxf(v, dpp_or_self<0x143, 0xc>(v));
+    return last_lane(v);
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return last_lane(wave_incl_scan(v)); }
+__device__ __forceinline__ double wave_sum(double v) { return last_lane(wave_incl_scan(v)); }
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) { return last_lane(wave_incl_scan(v)); }
 
 // greedy pick: the larger value, on equal values the lower index (kernels/shared/block_argmax.h:16)
 struct Best {
@@ -134,30 +167,6 @@ __device__ __forceinline__ T block_sum(T v, T* red) {
 #pragma unroll
     for (int w = 1; w < WS_WAVES; ++w) r += red[w];
     return r;
-}
-
-// ---- wave inclusive scan (sum of lanes 0..own) on the data-parallel-primitive path: four shifts inside each row of
-// 16 lanes, then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into rows 2 and 3. Lanes without a source,
-// and rows a step leaves out, add 0. Six dependent vector instructions instead of six trips through the LDS crossbar.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
-    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROW_MASK, 0xf, true));
-}
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ double dpp_or_zero(double v) {
-    const uint64_t b = static_cast<uint64_t>(__double_as_longlong(v));
-    const uint32_t lo = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b)), hi = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(b >> 32));
-    return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
-}
-template <class T>
-__device__ __forceinline__ T wave_incl_scan(T v) {
-    v += dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
-    v += dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
-    v += dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
-    v += dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
-    v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-    v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
 }
 
 // ---- block exclusive scan of one value per thread (thread order); returns the exclusive prefix, *total = block sum

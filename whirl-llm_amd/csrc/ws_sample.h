@@ -22,8 +22,6 @@
 // fixed summation order for doubles.
 #pragma once
 
-#include <type_traits>
-
 #include "ws_common.h"
 #include "ws_exp_table.h"
 
@@ -213,7 +211,7 @@ __device__ __forceinline__ uint64_t bin_word(float tc) {
 // keeps every token's bin index in registers (two per VGPR), so that the gather of the few bins the cuts land in
 // needs no second sweep. Rows of up to 163840 tokens. Only the allow mask is applied here; touched tokens are binned
 // with their raw logit and moved afterwards. For that their raw logits are needed: a 128-bit vector that holds a
-// touched token is copied as it is to stage[rank of its first touched token] (LDS, stage_cap slots of 16 bytes), which
+// touched token is copied as it is to stage[rank of its first touched token] (LDS, stage_cap + 1 slots of 16 bytes), which
 // costs two instructions per token and spares one scattered 4-byte read from HBM per touched token.
 constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 with 512
 
@@ -268,8 +266,9 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
         if (TOUCHED) {
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                const uint32_t j = (bt * kBatch + u) * WS_BLOCK + t;
-                const uint32_t word = ((j < nv ? j : nv - 1u) * PER) >> 5;
+                // a vector past the row reads a word past the bitmap: still inside the block's LDS (the tables behind
+                // the bitmap), and never looked at. Unclamped, the address is the thread's base plus a constant.
+                const uint32_t word = (((bt * kBatch + u) * WS_BLOCK + t) * PER) >> 5;
                 tws[u] = rv.touched[word];
                 wps[u] = rv.wprefix[word];
             }
@@ -303,7 +302,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
                     const uint32_t sh = (j * PER) & 31u, tw = tws[u];
                     if ((tw >> sh) & (PER == 4 ? 15u : 255u)) {
                         const uint32_t r = wps[u] + __popc(tw & ((1u << sh) - 1u));
-                        if (r < stage_cap) stage[r] = q[slot][u];
+                        stage[min(r, stage_cap)] = q[slot][u];  // slot stage_cap itself is a dump nobody reads
                     } else {
                         m = fmaxf(m, vm);
                     }
@@ -749,7 +748,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         bool swept = false;
         // staging room for the vectors that hold touched tokens: the LDS of the candidate masses, idle until pass 3
         uint4* stage = reinterpret_cast<uint4*>(emass);
-        const uint32_t stage_cap = rv.vec ? 2048u : 0u;
+        const uint32_t stage_cap = rv.vec ? 2047u : 0u;  // the region's last slot takes the vectors of the ranks beyond
         if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, cache, red_f, stage, stage_cap, anchor, aq, m);
         __syncthreads();
         WS_MARK(8);
