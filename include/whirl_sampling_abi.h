@@ -202,6 +202,33 @@ typedef struct ws_adjust {
 
 int ws_adjust_rows(void* stream, const ws_adjust* a);
 
+/* Draft acceptance on the device for the plain sampling rule. Stands in for the host loop Acceptor::sample
+ * (src/sampling/acceptor.cpp:63-100, rule "sample": no race, no typical acceptance), which samples output index
+ * n_gen + acc from verify row acc and accepts while the token equals the draft. Each output index draws from its own
+ * counter (src/sampling/acceptor.h:10-12), so the caller samples all verify rows of all sequences in one
+ * ws_sample_batch launch - row of position j of a sequence: step = n_gen + j, seed and filters of the sequence - and
+ * this call turns the tokens into counts, with no host round trip in between. Per sequence s, control area
+ * c = ctl_all + area[s] (layout above): nd = c[WS_CTL_ND] clamped to 0..15, drafts c[WS_CTL_DRAFTS .. + nd).
+ *   acc = number of leading positions j < nd whose token equals draft j; chosen = token of position acc;
+ *   c[WS_CTL_ROWS + j] = token of position j for j <= acc (the words the greedy path fills with row argmaxes,
+ *   src/model/qwen35/forward/mtp_verify.cpp:226); n_accepted[s] = acc; chosen[s].
+ *   status[s] = WS_ACCEPT_HOST when a position up to the stop has no usable token (token < 0, or WS_FLAG_OPEN: such a
+ *   row is drawn in another order than the reference's): the host then runs Acceptor::sample for that sequence. */
+enum { WS_ACCEPT_OK = 0, WS_ACCEPT_HOST = 1 };
+typedef struct ws_accept {
+    const int32_t* token;  /* device [rows]: ws_batch.token of the launch that sampled the verify rows */
+    const uint32_t* flags; /* device [rows]: ws_batch.flags of that launch */
+    const uint32_t* row0;  /* device [n_seq]: row of position 0 of the sequence in that launch */
+    int32_t* ctl_all;      /* device: the control areas */
+    const int32_t* area;   /* device [n_seq]: i32 word offset of the sequence's control area */
+    uint32_t n_seq;
+    int32_t* n_accepted;   /* out, device [n_seq] */
+    int32_t* chosen;       /* out, device [n_seq] */
+    uint32_t* status;      /* out, device [n_seq]: WS_ACCEPT_* */
+} ws_accept;
+
+int ws_accept_sampled(void* stream, const ws_accept* a);
+
 /* Classic speculative sampling (accept u * q < p, else resample from max(p - q, 0)); no counterpart in the
  * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32
  * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1]. Per sequence s: u_j from

@@ -68,6 +68,12 @@ class Adjust(C.Structure):
                 ("allow_stride", C.c_uint64), ("out", C.c_void_p), ("out_stride", C.c_uint64)]
 
 
+class Accept(C.Structure):
+    """ws_accept of include/whirl_sampling_abi.h."""
+    _fields_ = [("token", C.c_void_p), ("flags", C.c_void_p), ("row0", C.c_void_p), ("ctl_all", C.c_void_p), ("area", C.c_void_p),
+                ("n_seq", C.c_uint32), ("n_accepted", C.c_void_p), ("chosen", C.c_void_p), ("status", C.c_void_p)]
+
+
 # every symbol include/whirl_sampling_abi.h declares: (result type, argument types)
 ABI = {
     "ws_abi_version": (C.c_int, []),
@@ -88,6 +94,7 @@ ABI = {
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
+    "ws_accept_sampled": (C.c_int, [C.c_void_p, C.POINTER(Accept)]),
     "ws_spec_verify_workspace": (C.c_uint64, [C.POINTER(SpecVerify)]),
     "ws_spec_verify_classic": (C.c_int, [C.c_void_p, C.POINTER(SpecVerify)]),
 }
@@ -215,6 +222,23 @@ def adjust_rows(logits, hist=None, hist_off=None, rep=None, pres=None, freq=None
                allow_stride=allow.shape[1] if allow is not None else 0, out=_p(out), out_stride=vocab)
     check(lib().ws_adjust_rows(_stream(), C.byref(a)), "ws_adjust_rows")
     return out
+
+
+def accept_sampled(token, flags, row0, ctl_all, area):
+    """Accepted draft count and chosen token per sequence from the sampled tokens of its verify rows (ws_accept_sampled).
+    token int32 [rows], flags uint32-as-int32 [rows], row0 int32 [n_seq], ctl_all int32 control areas, area int32 [n_seq]
+    word offsets; all device tensors. Returns (n_accepted, chosen, status) int32 device tensors; ctl_all is updated."""
+    for name, v in (("token", token), ("flags", flags), ("row0", row0), ("ctl_all", ctl_all), ("area", area)):
+        if not v.is_cuda or v.dtype != torch.int32 or not v.is_contiguous():
+            raise WsError(f"{name}: contiguous int32 device tensor")
+    n_seq = row0.numel()
+    n_acc = torch.empty(n_seq, dtype=torch.int32, device=token.device)
+    chosen = torch.empty(n_seq, dtype=torch.int32, device=token.device)
+    status = torch.empty(n_seq, dtype=torch.int32, device=token.device)
+    a = Accept(token=_p(token), flags=_p(flags), row0=_p(row0), ctl_all=_p(ctl_all), area=_p(area), n_seq=n_seq,
+               n_accepted=_p(n_acc), chosen=_p(chosen), status=_p(status))
+    check(lib().ws_accept_sampled(_stream(), C.byref(a)), "ws_accept_sampled")
+    return n_acc, chosen, status
 
 
 class BatchSampler:

@@ -6,6 +6,7 @@
 
 #include <cstring>
 
+#include "ws_accept.h"
 #include "ws_adjust.h"
 #include "ws_common.h"
 #include "ws_draft.h"
@@ -260,6 +261,25 @@ int ws_adjust_rows(void* stream, const ws_adjust* b) {
     a.out = b->out;
     a.out_stride = b->out_stride;
     hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows), dim3(WS_BLOCK), ws::kAdjustLdsIds * sizeof(int32_t), S(stream), a);
+    return done();
+}
+
+int ws_accept_sampled(void* stream, const ws_accept* b) {
+    if (!b || !b->token || !b->flags || !b->row0 || !b->ctl_all || !b->area || !b->n_accepted || !b->chosen || !b->status)
+        return WS_E_INVALID;
+    if (b->n_seq == 0) return WS_E_INVALID;
+    ws::AcceptArgs a{};
+    a.token = b->token;
+    a.flags = b->flags;
+    a.row0 = b->row0;
+    a.ctl_all = b->ctl_all;
+    a.area = b->area;
+    a.n_seq = b->n_seq;
+    a.host_mask = WS_FLAG_ALL_MASKED | WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_OPEN;
+    a.n_accepted = b->n_accepted;
+    a.chosen = b->chosen;
+    a.status = b->status;
+    hipLaunchKernelGGL(ws::accept_sampled_kernel, dim3((b->n_seq + 63u) / 64u), dim3(64), 0, S(stream), a);
     return done();
 }
 
