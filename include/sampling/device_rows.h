@@ -42,7 +42,12 @@ public:
     DeviceRows(const DeviceRows&) = delete;
     DeviceRows& operator=(const DeviceRows&) = delete;
 
-    void setAdjust(const RowAdjust& a) { adj_ = a; }  // applies to the rows prepared from now on
+    void setAdjust(const RowAdjust& a);  // applies to the rows prepared from now on
+
+    // Filters rows s.row_base + r0 .. + n - 1 in one device launch and keeps the results on the host: the prepareRow
+    // calls that follow for these rows, with the same temperature and filters in `s`, cost no device call. The verify
+    // rows of a sequence share their sampler, so the engine calls this once before Acceptor::sample.
+    void prefetchRows(const Sampler& s, std::uint32_t r0, std::uint32_t n);
 
     void prepareRow(Sampler& s, std::uint32_t r) override;
     const float* loadFullRow(std::uint32_t gr) override;
@@ -54,7 +59,15 @@ public:
 
 private:
     void escalate(Sampler& s, std::uint32_t gr);
-    struct Dev;  // device scratch
+    void uploadInputs(const Sampler& s, std::uint32_t n);
+    void filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32_t n);
+    struct Dev;    // device scratch
+    struct Ready;  // a row filtered on the device, held for its prepareRow
+    struct ReadyKey {
+        float inv_t = 0.f;
+        std::uint32_t top_k = 0;
+        double top_p = 0.0, min_p = 0.0;
+    };
     const float* logits_;
     std::uint32_t rows_, vocab_;
     void* stream_;
@@ -63,6 +76,8 @@ private:
     std::vector<float> row_host_;
     std::vector<std::uint8_t> marks_;
     std::uint32_t last_flags_ = 0;
+    std::vector<Ready> ready_;
+    ReadyKey ready_key_;
     static constexpr std::uint32_t kNoRow = 0xffffffffu;
     std::uint32_t adjusted_row_ = kNoRow;  // row whose penalised copy sits on the device (after an escalation)
 };

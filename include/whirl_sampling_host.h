@@ -41,6 +41,27 @@ typedef struct wsh_rows {
 
 /* 0 = ok, otherwise the code of the failing call (hipError_t > 0, WS_E_* < 0); text from wsh_last_error(). Synchronous. */
 int wsh_sample_rows(void* stream, const wsh_rows* a);
+
+/* Acceptor::sample (src/sampling/acceptor.cpp:63-100) for one sequence over device logits: verify rows row0 .. row0 + nd
+ * of d_logits, drafts dr[0 .. nd), output index n_gen + accepted. With prefetch != 0 the rows are filtered by one device
+ * launch (sampling::DeviceRows::prefetchRows) before the loop, otherwise one launch per visited row. Relaxed acceptance
+ * and the repetition guard are off. */
+typedef struct wsh_accept {
+    const float* d_logits; /* device, [rows][vocab] */
+    uint32_t rows, vocab;
+    float inv_t;
+    uint32_t top_k;
+    double top_p, min_p;
+    uint64_t seed;
+    int32_t race;       /* Sampler::race: the "specsample" rule instead of "sample" */
+    const uint32_t* dr; /* drafts */
+    uint32_t nd, row0;
+    uint64_t n_gen;
+    int32_t prefetch;
+    uint32_t acc, chosen;        /* out */
+    uint32_t big_used, full_used; /* out: Sampler counters after the loop */
+} wsh_accept;
+int wsh_accept_sample(void* stream, wsh_accept* a);
 const char* wsh_last_error(void);
 
 #ifdef __cplusplus

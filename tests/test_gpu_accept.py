@@ -116,3 +116,22 @@ def test_accept_sampled_rejects_missing_arguments():
     m = gc.pkg()
     a = m.Accept()
     assert m.lib().ws_accept_sampled(None, C.byref(a)) == -1
+
+
+@pytest.mark.parametrize("prefetch", [True, False])
+def test_host_acceptor_over_device_rows_matches_the_oracle(prefetch):
+    """Acceptor::sample of the C++ host layer with sampling::DeviceRows as its RowSource (all verify rows filtered in one
+    device launch when prefetched, else one launch per visited row) against the oracle's Acceptor::sample."""
+    m = gc.pkg()
+    seqs = _sequences(10, 4242)
+    row0 = np.cumsum([0] + [q["nd"] + 1 for q in seqs])
+    x = torch.from_numpy(np.concatenate([q["x"] for q in seqs])).to("cuda:0")
+    accepted = 0
+    for s, q in enumerate(seqs):
+        p = q["prm"]
+        acc, chosen, big, full = m.host_accept_sample(x, q["dr"], q["nd"], int(row0[s]), q["n_gen"], p["temp"], p["top_k"], p["top_p"],
+                                                      p["min_p"], p["seed"], prefetch=prefetch)
+        assert (acc, chosen) == (q["acc"], q["chosen"]), (s, acc, chosen, q["acc"], q["chosen"])
+        assert big == 0 and full == 0  # top-k of at most 50: the kept sets fit the small candidate list
+        accepted += acc
+    assert accepted >= len(seqs)

@@ -317,7 +317,16 @@ class HostRows(C.Structure):
                 ("n_kept", C.c_void_p), ("flags", C.c_void_p), ("closed", C.c_void_p)]
 
 
-HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]), "wsh_last_error": (C.c_char_p, [])}
+class HostAccept(C.Structure):
+    """wsh_accept of include/whirl_sampling_host.h."""
+    _fields_ = [("d_logits", C.c_void_p), ("rows", C.c_uint32), ("vocab", C.c_uint32), ("inv_t", C.c_float), ("top_k", C.c_uint32),
+                ("top_p", C.c_double), ("min_p", C.c_double), ("seed", C.c_uint64), ("race", C.c_int32), ("dr", C.c_void_p),
+                ("nd", C.c_uint32), ("row0", C.c_uint32), ("n_gen", C.c_uint64), ("prefetch", C.c_int32), ("acc", C.c_uint32),
+                ("chosen", C.c_uint32), ("big_used", C.c_uint32), ("full_used", C.c_uint32)]
+
+
+HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]),
+            "wsh_accept_sample": (C.c_int, [C.c_void_p, C.POINTER(HostAccept)]), "wsh_last_error": (C.c_char_p, [])}
 _host_lib = None
 
 
@@ -367,3 +376,18 @@ def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p
     if rc != 0:
         raise WsError(f"wsh_sample_rows: {host_lib().wsh_last_error().decode()} ({rc})")
     return out
+
+
+def host_accept_sample(logits, dr, nd, row0, n_gen, temp, top_k, top_p, min_p, seed, race=False, prefetch=True):
+    """Acceptor::sample of the C++ host API for one sequence over device logits (wsh_accept_sample). Returns
+    (accepted, chosen, big_used, full_used)."""
+    import numpy as np
+    _dev_f32(logits)
+    dr = np.ascontiguousarray(dr, dtype=np.uint32)
+    a = HostAccept(d_logits=_p(logits), rows=logits.shape[0], vocab=logits.shape[1], inv_t=float(np.float32(1.0 / temp)), top_k=top_k,
+                   top_p=top_p, min_p=min_p, seed=seed, race=int(race), dr=dr.ctypes.data_as(C.c_void_p), nd=nd, row0=row0,
+                   n_gen=n_gen, prefetch=int(prefetch))
+    rc = host_lib().wsh_accept_sample(_stream(), C.byref(a))
+    if rc != 0:
+        raise WsError(f"wsh_accept_sample: {host_lib().wsh_last_error().decode()} ({rc})")
+    return a.acc, a.chosen, a.big_used, a.full_used

@@ -1,6 +1,7 @@
 // sampling::DeviceRows: a RowSource whose rows are sampled on the GPU through the C ABI (whirl_sampling_abi.h).
 // One prepareRow = one launch of ws_sample_batch on that row with the kept-set dump on, one small download, and a
-// sort of the kept candidates on the host. No vocabulary-sized work happens here unless the device flags the row.
+// sort of the kept candidates on the host; prefetchRows does the launch and the download for several rows at once.
+// No vocabulary-sized work happens here unless the device flags the row.
 #include "sampling/device_rows.h"
 
 #include "whirl_sampling_abi.h"
@@ -28,48 +29,89 @@ void checkHip(hipError_t e, const char* op) {
 
 }  // namespace
 
-// device scratch of one DeviceRows: parameters, outputs and side inputs of a one-row batch
+// device scratch of one DeviceRows: parameters, outputs and side inputs of a batch of rows that share one sampler
 struct DeviceRows::Dev {
-    // parameter block, uploaded per call
-    struct Params {
-        double top_p, min_p;
-        std::uint64_t seed, step;
-        float inv_t, rep, pres, freq;
-        std::uint32_t top_k, hist_off[2], bias_off[2];
+    // Parameter block for R rows, one device allocation and one upload: arrays in the order below, 8-byte types first.
+    struct ParamView {
+        double* top_p;
+        double* min_p;
+        std::uint64_t* seed;
+        std::uint64_t* step;
+        float* inv_t;
+        float* rep;
+        float* pres;
+        float* freq;
+        std::uint32_t* top_k;
+        std::uint32_t* hist_off;  // R + 1
+        std::uint32_t* bias_off;  // R + 1
     };
-    // result block, downloaded per call
-    struct Result {
-        std::int32_t token;
-        float prob;
-        std::uint32_t n_kept, flags;
-        float stats[2];
+    static std::size_t paramBytes(std::uint32_t R) { return std::size_t{R} * (4 * 8 + 5 * 4) + 2 * (std::size_t{R} + 1) * 4; }
+    static ParamView view(unsigned char* base, std::uint32_t R) {
+        ParamView v;
+        v.top_p = reinterpret_cast<double*>(base);
+        v.min_p = v.top_p + R;
+        v.seed = reinterpret_cast<std::uint64_t*>(v.min_p + R);
+        v.step = v.seed + R;
+        v.inv_t = reinterpret_cast<float*>(v.step + R);
+        v.rep = v.inv_t + R;
+        v.pres = v.rep + R;
+        v.freq = v.pres + R;
+        v.top_k = reinterpret_cast<std::uint32_t*>(v.freq + R);
+        v.hist_off = v.top_k + R;
+        v.bias_off = v.hist_off + R + 1;
+        return v;
+    }
+    // Result block for R rows, one download: token i32, prob f32, n_kept u32, flags u32, stats 2 x f32
+    struct ResultView {
+        std::int32_t* token;
+        float* prob;
+        std::uint32_t* n_kept;
+        std::uint32_t* flags;
+        float* stats;
     };
-    Params* prm = nullptr;
-    Result* res = nullptr;
-    std::int32_t* kept_ids = nullptr;
+    static std::size_t resultBytes(std::uint32_t R) { return std::size_t{R} * 24; }
+    static ResultView view_res(unsigned char* base, std::uint32_t R) {
+        ResultView v;
+        v.token = reinterpret_cast<std::int32_t*>(base);
+        v.prob = reinterpret_cast<float*>(v.token + R);
+        v.n_kept = reinterpret_cast<std::uint32_t*>(v.prob + R);
+        v.flags = v.n_kept + R;
+        v.stats = reinterpret_cast<float*>(v.flags + R);
+        return v;
+    }
+    std::uint32_t row_cap = 0;     // rows the blocks below are sized for
+    std::uint32_t rows_now = 0;    // rows of the parameter block that is on the device
+    unsigned char* prm = nullptr;
+    unsigned char* res = nullptr;
+    std::int32_t* kept_ids = nullptr;  // [row_cap][cap]
     float* kept_logits = nullptr;
-    std::int32_t* hist = nullptr;
+    std::int32_t* hist = nullptr;      // the history, once per row
     std::int32_t* bias_ids = nullptr;
     float* bias_vals = nullptr;
-    std::uint32_t hist_cap = 0, bias_cap = 0;
+    std::size_t hist_cap = 0, bias_cap = 0;
     std::int32_t* topk_ids = nullptr;  // escalation: ids | vals | stats of one row, kBig candidates
     float* topk_vals = nullptr;
     float* topk_stats = nullptr;
     float* adjusted = nullptr;         // escalation: penalised copy of the row (ws_adjust_rows)
+    std::vector<unsigned char> h_prm, h_res;
     std::vector<std::int32_t> h_ids;
     std::vector<float> h_vals;
+};
+
+// one row the device has filtered already, waiting on the host for its prepareRow
+struct DeviceRows::Ready {
+    std::uint32_t gr;
+    std::uint32_t n_kept, flags;
+    float m, sum;
+    std::vector<std::int32_t> ids;
+    std::vector<float> logits;
 };
 
 DeviceRows::DeviceRows(const float* d_logits, std::uint32_t rows, std::uint32_t n_vocab, void* stream)
     : logits_(d_logits), rows_(rows), vocab_(n_vocab), stream_(stream), dev_(new Dev), marks_(n_vocab, 0) {
     check(ws_probe(), "ws_probe");
-    const std::uint32_t cap = std::min(kKeptCap, vocab_);
-    checkHip(hipMalloc(reinterpret_cast<void**>(&dev_->prm), sizeof(Dev::Params)), "hipMalloc");
-    checkHip(hipMalloc(reinterpret_cast<void**>(&dev_->res), sizeof(Dev::Result)), "hipMalloc");
-    checkHip(hipMalloc(reinterpret_cast<void**>(&dev_->kept_ids), cap * sizeof(std::int32_t)), "hipMalloc");
-    checkHip(hipMalloc(reinterpret_cast<void**>(&dev_->kept_logits), cap * sizeof(float)), "hipMalloc");
-    dev_->h_ids.resize(std::max(cap, kBig));
-    dev_->h_vals.resize(std::max(cap, kBig));
+    dev_->h_ids.resize(kBig);
+    dev_->h_vals.resize(kBig);
 }
 
 DeviceRows::~DeviceRows() {
@@ -81,102 +123,176 @@ DeviceRows::~DeviceRows() {
     delete dev_;
 }
 
-void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
-    const std::uint32_t gr = s.row_base + r;
-    if (gr >= rows_) throw DeviceError("prepareRow", WS_E_INVALID, "prepareRow: row out of range");
-    s.row = gr;
-    adjusted_row_ = kNoRow;
+void DeviceRows::setAdjust(const RowAdjust& a) {
+    adj_ = a;
+    ready_.clear();  // rows filtered under the old penalties are of no use any more
+}
+
+// Parameters of `n` rows that share sampler `s` and the current penalties, and the penalty lists once per row, go to
+// the device (the lists are replicated because a batch addresses them through one ascending offset array).
+void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
     auto stream = static_cast<hipStream_t>(stream_);
     Dev& d = *dev_;
-    // side inputs: grow the device copies when needed, then upload
-    if (adj_.n_history > d.hist_cap) {
+    const std::uint32_t cap = std::min(kKeptCap, vocab_);
+    if (n > d.row_cap) {
+        for (void* p : {static_cast<void*>(d.prm), static_cast<void*>(d.res), static_cast<void*>(d.kept_ids), static_cast<void*>(d.kept_logits)})
+            if (p) (void)hipFree(p);
+        d.prm = d.res = nullptr;
+        d.kept_ids = nullptr;
+        d.kept_logits = nullptr;
+        d.row_cap = n;
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.prm), Dev::paramBytes(n)), "hipMalloc");
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.res), Dev::resultBytes(n)), "hipMalloc");
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.kept_ids), std::size_t{n} * cap * sizeof(std::int32_t)), "hipMalloc");
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.kept_logits), std::size_t{n} * cap * sizeof(float)), "hipMalloc");
+    }
+    const std::size_t nh = adj_.n_history, nb = adj_.n_bias;
+    if (nh * n > d.hist_cap) {
         if (d.hist) (void)hipFree(d.hist);
-        d.hist_cap = std::max(adj_.n_history, 2 * d.hist_cap);
+        d.hist = nullptr;
+        d.hist_cap = std::max(nh * n, 2 * d.hist_cap);
         checkHip(hipMalloc(reinterpret_cast<void**>(&d.hist), d.hist_cap * sizeof(std::int32_t)), "hipMalloc");
     }
-    if (adj_.n_bias > d.bias_cap) {
+    if (nb * n > d.bias_cap) {
         if (d.bias_ids) (void)hipFree(d.bias_ids);
         if (d.bias_vals) (void)hipFree(d.bias_vals);
-        d.bias_cap = std::max(adj_.n_bias, 2 * d.bias_cap);
+        d.bias_ids = nullptr;
+        d.bias_vals = nullptr;
+        d.bias_cap = std::max(nb * n, 2 * d.bias_cap);
         checkHip(hipMalloc(reinterpret_cast<void**>(&d.bias_ids), d.bias_cap * sizeof(std::int32_t)), "hipMalloc");
         checkHip(hipMalloc(reinterpret_cast<void**>(&d.bias_vals), d.bias_cap * sizeof(float)), "hipMalloc");
     }
-    if (adj_.n_history)
-        checkHip(hipMemcpyAsync(d.hist, adj_.history, adj_.n_history * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-    if (adj_.n_bias) {
-        checkHip(hipMemcpyAsync(d.bias_ids, adj_.bias_ids, adj_.n_bias * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-        checkHip(hipMemcpyAsync(d.bias_vals, adj_.bias_vals, adj_.n_bias * sizeof(float), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    for (std::uint32_t r = 0; r < n; ++r) {
+        if (nh) checkHip(hipMemcpyAsync(d.hist + r * nh, adj_.history, nh * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+        if (nb) {
+            checkHip(hipMemcpyAsync(d.bias_ids + r * nb, adj_.bias_ids, nb * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+            checkHip(hipMemcpyAsync(d.bias_vals + r * nb, adj_.bias_vals, nb * sizeof(float), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+        }
     }
-    Dev::Params p{};
-    p.top_p = s.top_p;
-    p.min_p = s.min_p;
-    p.seed = s.seed;
-    p.step = s.pos_idx;
-    p.inv_t = s.inv_t;
-    p.rep = adj_.repetition;
-    p.pres = adj_.presence;
-    p.freq = adj_.frequency;
-    p.top_k = s.top_k;
-    p.hist_off[1] = adj_.n_history;
-    p.bias_off[1] = adj_.n_bias;
-    checkHip(hipMemcpyAsync(d.prm, &p, sizeof p, hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    d.h_prm.assign(Dev::paramBytes(n), 0);
+    const Dev::ParamView h = Dev::view(d.h_prm.data(), n);
+    for (std::uint32_t r = 0; r < n; ++r) {
+        h.top_p[r] = s.top_p;
+        h.min_p[r] = s.min_p;
+        h.seed[r] = s.seed;
+        h.step[r] = s.pos_idx;  // the draw is made on the host; the device's own is not looked at
+        h.inv_t[r] = s.inv_t;
+        h.rep[r] = adj_.repetition;
+        h.pres[r] = adj_.presence;
+        h.freq[r] = adj_.frequency;
+        h.top_k[r] = s.top_k;
+    }
+    for (std::uint32_t r = 0; r <= n; ++r) {
+        h.hist_off[r] = static_cast<std::uint32_t>(r * nh);
+        h.bias_off[r] = static_cast<std::uint32_t>(r * nb);
+    }
+    // the pageable staging buffer is read before the call returns, so it may be rewritten by the next call
+    checkHip(hipMemcpyAsync(d.prm, d.h_prm.data(), d.h_prm.size(), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+    d.rows_now = n;
+}
 
+// One launch of the fused sampler over rows [gr0, gr0 + n), all with sampler `s` and the current penalties; what it
+// keeps of every row comes back to ready_.
+void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32_t n) {
+    if (n == 0 || gr0 >= rows_ || n > rows_ - gr0) throw DeviceError("prepareRow", WS_E_INVALID, "prepareRow: row out of range");
+    if (static_cast<std::uint64_t>(adj_.n_history) * n > 0xffffffffull || static_cast<std::uint64_t>(adj_.n_bias) * n > 0xffffffffull)
+        throw DeviceError("prepareRow", WS_E_INVALID, "prepareRow: history too long for this many rows");
+    auto stream = static_cast<hipStream_t>(stream_);
+    uploadInputs(s, n);
+    Dev& d = *dev_;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
+    const Dev::ParamView p = Dev::view(d.prm, n);
+    const Dev::ResultView o = Dev::view_res(d.res, n);
     ws_batch b{};
-    b.logits = logits_ + static_cast<std::size_t>(gr) * vocab_;
+    b.logits = logits_ + static_cast<std::size_t>(gr0) * vocab_;
     b.dtype = WS_DTYPE_F32;
-    b.rows = 1;
+    b.rows = n;
     b.vocab = vocab_;
     b.row_stride = vocab_;
-    b.inv_t = &d.prm->inv_t;
-    b.top_k = &d.prm->top_k;
-    b.top_p = &d.prm->top_p;
-    b.min_p = &d.prm->min_p;
-    b.seed = &d.prm->seed;
-    b.step = &d.prm->step;
+    b.inv_t = p.inv_t;
+    b.top_k = p.top_k;
+    b.top_p = p.top_p;
+    b.min_p = p.min_p;
+    b.seed = p.seed;
+    b.step = p.step;
     b.rng = WS_RNG_SPLITMIX;
     if (adj_.n_history) {
         b.hist = d.hist;
-        b.hist_off = d.prm->hist_off;
-        b.rep = &d.prm->rep;
-        b.pres = &d.prm->pres;
-        b.freq = &d.prm->freq;
+        b.hist_off = p.hist_off;
+        b.rep = p.rep;
+        b.pres = p.pres;
+        b.freq = p.freq;
         b.max_hist = adj_.n_history;
     }
     if (adj_.n_bias) {
         b.bias_ids = d.bias_ids;
         b.bias_vals = d.bias_vals;
-        b.bias_off = d.prm->bias_off;
+        b.bias_off = p.bias_off;
         b.max_bias = adj_.n_bias;
     }
-    b.token = &d.res->token;
-    b.prob = &d.res->prob;
-    b.n_kept = &d.res->n_kept;
-    b.flags = &d.res->flags;
-    b.stats = d.res->stats;
+    b.token = o.token;
+    b.prob = o.prob;
+    b.n_kept = o.n_kept;
+    b.flags = o.flags;
+    b.stats = o.stats;
     b.kept_ids = d.kept_ids;
     b.kept_logits = d.kept_logits;
     b.kept_cap = cap;
     b.mode = WS_MODE_AUTO;
     check(ws_sample_batch(stream_, &b), "ws_sample_batch");
 
-    Dev::Result res{};
-    checkHip(hipMemcpyAsync(&res, d.res, sizeof res, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+    d.h_res.resize(Dev::resultBytes(n));
+    checkHip(hipMemcpyAsync(d.h_res.data(), d.res, d.h_res.size(), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-    last_flags_ = res.flags;
-    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM;
-    if ((res.flags & unresolved) || res.n_kept > cap || (res.flags & WS_FLAG_ALL_MASKED)) {
+    const Dev::ResultView h = Dev::view_res(d.h_res.data(), n);
+    ready_.clear();
+    ready_.resize(n);
+    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
+    for (std::uint32_t r = 0; r < n; ++r) {
+        Ready& q = ready_[r];
+        q.gr = gr0 + r;
+        q.n_kept = h.n_kept[r];
+        q.flags = h.flags[r];
+        q.m = h.stats[2 * r];
+        q.sum = h.stats[2 * r + 1];
+        if ((q.flags & unresolved) || q.n_kept > cap) continue;  // such a row is escalated when it is asked for
+        q.ids.resize(q.n_kept);
+        q.logits.resize(q.n_kept);
+        checkHip(hipMemcpyAsync(q.ids.data(), d.kept_ids + std::size_t{r} * cap, q.n_kept * sizeof(std::int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+        checkHip(hipMemcpyAsync(q.logits.data(), d.kept_logits + std::size_t{r} * cap, q.n_kept * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+    }
+    checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    ready_key_ = {s.inv_t, s.top_k, s.top_p, s.min_p};
+}
+
+void DeviceRows::prefetchRows(const Sampler& s, std::uint32_t r0, std::uint32_t n) { filterOnDevice(s, s.row_base + r0, n); }
+
+void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
+    const std::uint32_t gr = s.row_base + r;
+    if (gr >= rows_) throw DeviceError("prepareRow", WS_E_INVALID, "prepareRow: row out of range");
+    s.row = gr;
+    adjusted_row_ = kNoRow;
+    const Ready* q = nullptr;
+    const bool same = ready_key_.inv_t == s.inv_t && ready_key_.top_k == s.top_k && ready_key_.top_p == s.top_p && ready_key_.min_p == s.min_p;
+    if (same)
+        for (const Ready& c : ready_)
+            if (c.gr == gr) q = &c;
+    if (!q) {
+        filterOnDevice(s, gr, 1);
+        q = &ready_[0];
+    }
+    last_flags_ = q->flags;
+    const std::uint32_t cap = std::min(kKeptCap, vocab_);
+    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
+    if ((q->flags & unresolved) || q->n_kept > cap) {
         escalate(s, gr);
         return;
     }
-    const std::uint32_t n = res.n_kept;
-    checkHip(hipMemcpyAsync(d.h_ids.data(), d.kept_ids, n * sizeof(std::int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-    checkHip(hipMemcpyAsync(d.h_vals.data(), d.kept_logits, n * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-    checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-    s.m = res.stats[0];
-    s.sum = res.stats[1];
+    const std::uint32_t n = q->n_kept;
+    s.m = q->m;
+    s.sum = q->sum;
     Cand* c = s.cands->data();
-    for (std::uint32_t i = 0; i < n; ++i) c[i] = {static_cast<std::uint32_t>(d.h_ids[i]), d.h_vals[i], 0.0};
+    for (std::uint32_t i = 0; i < n; ++i) c[i] = {static_cast<std::uint32_t>(q->ids[i]), q->logits[i], 0.0};
     std::sort(c, c + n, [](const Cand& a, const Cand& b2) { return a.logit != b2.logit ? a.logit > b2.logit : a.id < b2.id; });
     // probabilities as the host filter leaves them: exp((double)(float)(l - m) * inv_t) / sum, renormalised over the kept set
     double z = 0;
@@ -200,23 +316,25 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
     const float* src = logits_ + static_cast<std::size_t>(gr) * vocab_;
     if (adj_.n_history || adj_.n_bias) {
         if (!d.adjusted) checkHip(hipMalloc(reinterpret_cast<void**>(&d.adjusted), vocab_ * sizeof(float)), "hipMalloc");
+        uploadInputs(s, 1);  // the row may come from an earlier batch: its lists and parameters go up again
+        const Dev::ParamView p = Dev::view(d.prm, 1);
         ws_adjust a{};
         a.logits = src;
         a.dtype = WS_DTYPE_F32;
         a.rows = 1;
         a.vocab = vocab_;
         a.row_stride = vocab_;
-        if (adj_.n_history) {  // the lists and the parameter block are still on the device from prepareRow
+        if (adj_.n_history) {
             a.hist = d.hist;
-            a.hist_off = d.prm->hist_off;
-            a.rep = &d.prm->rep;
-            a.pres = &d.prm->pres;
-            a.freq = &d.prm->freq;
+            a.hist_off = p.hist_off;
+            a.rep = p.rep;
+            a.pres = p.pres;
+            a.freq = p.freq;
         }
         if (adj_.n_bias) {
             a.bias_ids = d.bias_ids;
             a.bias_vals = d.bias_vals;
-            a.bias_off = d.prm->bias_off;
+            a.bias_off = p.bias_off;
         }
         a.out = d.adjusted;
         a.out_stride = vocab_;

@@ -1,6 +1,7 @@
 // A small C entry point over the C++ host API, for language bindings and tests that cannot call C++ classes:
 // sample one token per row through sampling::DeviceRows + sampling::sampleRow, the way the engine's decode loop does
 // (prepareRow, set the output index, draw).
+#include "sampling/acceptor.h"
 #include "sampling/device_rows.h"
 #include "sampling/sampler.h"
 #include "whirl_sampling_abi.h"
@@ -9,6 +10,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <exception>
+#include <span>
 #include <vector>
 
 namespace ws = whirl::sampling;
@@ -59,6 +61,45 @@ int wsh_sample_rows(void* stream, const wsh_rows* a) {
             if (a->flags) a->flags[r] = src.lastFlags();
             if (a->closed) a->closed[r] = s.closed;
         }
+        return 0;
+    } catch (const ws::DeviceError& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return e.code ? e.code : -1;
+    } catch (const std::exception& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return -1;
+    }
+}
+
+int wsh_accept_sample(void* stream, wsh_accept* a) {
+    g_err[0] = 0;
+    try {
+        ws::DeviceRows src(a->d_logits, a->rows, a->vocab, stream);
+        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+        ws::Sampler s;
+        s.inv_t = a->inv_t;
+        s.temp = 1.0 / s.inv_t;
+        s.top_k = a->top_k;
+        s.top_p = a->top_p;
+        s.min_p = a->min_p;
+        s.seed = a->seed;
+        s.cands = &scratch;
+        s.race = a->race != 0;
+        s.row_base = a->row0;
+        if (a->prefetch) src.prefetchRows(s, 0, a->nd + 1);
+        const whirl::relax::Params no_relax{};
+        const ws::Acceptor acceptor(no_relax);
+        std::uint32_t relaxed = 0;
+        ws::Drafts drafts;
+        drafts.dr = std::span<const std::uint32_t>(a->dr, a->nd);
+        drafts.nd = a->nd;
+        drafts.row0 = a->row0;
+        const ws::Accepted r = acceptor.sample(src, s, drafts, false, static_cast<std::uint32_t>(a->n_gen),
+                                               [](std::uint32_t) { return false; }, relaxed);
+        a->acc = r.acc;
+        a->chosen = r.chosen;
+        a->big_used = s.big_used;
+        a->full_used = s.full_used;
         return 0;
     } catch (const ws::DeviceError& e) {
         snprintf(g_err, sizeof g_err, "%s", e.what());
