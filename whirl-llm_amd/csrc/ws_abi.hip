@@ -73,12 +73,15 @@ BatchPlan plan_batch(const ws_batch* b) {
         p.lds_cnt = 0;
     }
     if (total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
-    // spare room for the tie bitmap (vocab / 32 words + 16-bit prefixes), when there is any
+    // spare room, when there is any, for a second copy of the histogram during the single sweep (odd lanes add there,
+    // which halves the collisions of a wave's atomics on a crowded bin) and later for the tie bitmap of the sort
+    // (vocab / 32 words + 16-bit prefixes)
     const uint64_t tie_bytes = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
+    const uint64_t spare_bytes = tie_bytes > 32768u ? tie_bytes : 32768u;
     p.lds_tie = 0;
-    if (total + tie_bytes + 4096u <= kMaxLds) {
+    if (total + spare_bytes + 4096u <= kMaxLds) {
         p.lds_tie = static_cast<uint32_t>((total + 15u) & ~uint64_t{15});
-        total = p.lds_tie + tie_bytes;
+        total = p.lds_tie + spare_bytes;
     }
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);

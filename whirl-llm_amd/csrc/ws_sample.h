@@ -1,25 +1,28 @@
-// Fused batched sampler for gfx950 (wave64): one workgroup of 1024 threads per logits row.
+// Fused batched sampler for gfx950 (wave64): one workgroup per logits row (1024 threads in the three-pass mode, 512 in
+// the single-sweep mode, where each thread keeps the bin of every token it has seen in registers).
 //
 // Per row (ws_batch in include/whirl_sampling_abi.h states the order of operations):
 //   phase 0  penalties / bias: an LDS bitmap of the token ids the history and the bias list touch, a per-word
 //            prefix popcount (rank of a touched id = perfect hash), per-rank counts by LDS atomics, then the adjusted
-//            logit of every touched token (one 4-byte gather each) into an LDS array by rank. No penalised copy of the
-//            row is ever written: the three-pass mode streams the row unmodified, skips touched tokens (bit set) and
-//            replays them from that array; the single-sweep mode bins every token as it is and afterwards moves the
-//            touched ones from the bin of their raw logit to the bin of their adjusted logit.
+//            logit of every touched token into an LDS array by rank. No penalised copy of the row is ever written: the
+//            three-pass mode streams the row unmodified, skips touched tokens (bit set) and replays them from that
+//            array; the single-sweep mode bins every token as it is and afterwards moves the touched ones from the
+//            bin of their raw logit to the bin of their adjusted logit.
 //   pass 1   maximum of the adjusted row (NaN and masked tokens count as -inf).
 //   pass 2   histogram of 4096 bins of width 1/64 in a = (max - x) * inv_t, the exponent of the softmax: one LDS
 //            64-bit atomic per element adds {count, fixed-point 1 - exp(-(a - bin edge))} (a quadratic, no
 //            transcendental per element). A block scan turns it into count and mass prefixes in (logit desc) order.
 //            The normaliser sum exp((x - max) * inv_t) is the total mass.
+//            The single-sweep mode does passes 1 and 2 in one sweep, against a bound above the maximum taken from the
+//            first loads, and remembers every token's bin (fused_pass_impl).
 //   select   top-k is a count query, top-p and the draw are mass queries, min-p is a value query on these prefixes;
-//            each lands in one bin (or a short range of bins).
-//   pass 3   the elements of those bins (at most kCap) are gathered into LDS as 64-bit (logit desc, id asc) keys,
-//            sorted (bitonic), given their exact double-precision mass exp(-(double)(max - x) * inv_t) - the host
-//            sampler's own formula (src/sampling/sampler.cpp:31-32) - and scanned; the cut positions and the drawn
-//            token are read off that list.
-// Rows are re-read from L2 / Infinity Cache in passes 2 and 3. Everything is deterministic: integer atomics only,
-// fixed summation order for doubles.
+//            each lands in one bin (or a short range of bins), found by 64-way searches of a wave.
+//   pass 3   the elements of those bins (at most kCap) are gathered into LDS as 64-bit (logit desc, id asc) keys -
+//            by a third sweep, or from the remembered bins - sorted, given their exact double-precision mass
+//            exp(-(double)(max - x) * inv_t), the host sampler's own formula (src/sampling/sampler.cpp:31-32), and
+//            scanned; the cut positions and the drawn token are read off that list.
+// The three-pass mode re-reads the row from L2 / Infinity Cache in passes 2 and 3. Everything is deterministic: integer
+// atomics only, fixed summation order for doubles.
 #pragma once
 
 #include "ws_common.h"
@@ -75,8 +78,9 @@ struct BatchArgs {
     uint32_t kept_cap;
     double tol;
     uint32_t lds_ab;   // bytes of the LDS region shared by the histogram / sort keys / masses
-    uint32_t lds_tie;  // byte offset of a spare id bitmap + prefix (vocab / 32 words + as many 16-bit counts) for sorting heavy
-                       // ties by id, 0 when the LDS has no room for it
+    uint32_t lds_tie;  // byte offset of spare LDS, 0 when there is no room for it: at least 32 KiB and vocab / 32 words + as
+                       // many 16-bit counts. Second copy of the histogram during the single sweep, then the id bitmap +
+                       // prefix that sorts heavy ties by id
     uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
 };
 
@@ -219,8 +223,8 @@ constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 
 // units of headroom; the same registers then feed the sweep. Returns false (nothing binned) when that is not finite.
 template <int PER, bool MASKED, bool TOUCHED>
 __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
-                                                uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap,
-                                                float& anchor, float& aq, float& m) {
+                                                uint64_t* hist2, uint32_t (&cache)[kCacheRegs], float* red, uint4* stage,
+                                                uint32_t stage_cap, float& anchor, float& aq, float& m) {
     constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
     constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
@@ -240,6 +244,12 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     load(0, 0);
     if (NB > 1) load(1, 1);
     for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+    if (hist2) {
+        // a second copy for the odd lanes: the 64 atomics of a wave instruction that meet on one bin are served one
+        // after the other, and two copies halve the longest such queue; the scan adds the copies up
+        for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
+        if (t & 1u) hist = hist2;
+    }
     {
         float s = floor_v;
 #pragma unroll
@@ -318,10 +328,10 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     return true;
 }
 
-__device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
+__device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist, uint64_t* hist2,
                                            uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap, float& anchor,
                                            float& aq, float& m) {
-#define WS_FUSED_CALL(PER, AL, TC) fused_pass_impl<PER, AL, TC>(rv, floor_v, inv_t, c64, hist, cache, red, stage, stage_cap, anchor, aq, m)
+#define WS_FUSED_CALL(PER, AL, TC) fused_pass_impl<PER, AL, TC>(rv, floor_v, inv_t, c64, hist, hist2, cache, red, stage, stage_cap, anchor, aq, m)
     if (rv.dtype == 0) {
         if (rv.touched) return rv.allow ? WS_FUSED_CALL(4, true, true) : WS_FUSED_CALL(4, false, true);
         return rv.allow ? WS_FUSED_CALL(4, true, false) : WS_FUSED_CALL(4, false, false);
@@ -452,7 +462,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ uint32_t red_u[WS_WAVES];
     __shared__ double red_d[WS_WAVES];
     __shared__ uint32_t s_cnt;
-    __shared__ double s_d[8];
     __shared__ double s_exp[128];  // kExpHi, kExpLo
     __shared__ uint32_t s_u[8];
 
@@ -742,6 +751,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
     float m = -INFINITY;
     bool cached = false;
+    uint64_t* hist2 = FUSED && A.lds_tie ? reinterpret_cast<uint64_t*>(lds + A.lds_tie) : nullptr;  // second copy of the histogram
     uint32_t cache[kCacheRegs];  // dead code (and no registers) in the exact instantiation
     if (FUSED && !(flags & kBadParam)) {
         // ---------------------------------------------------------------- fused sweep: anchor, histogram, max, bins
@@ -749,7 +759,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         // staging room for the vectors that hold touched tokens: the LDS of the candidate masses, idle until pass 3
         uint4* stage = reinterpret_cast<uint4*>(emass);
         const uint32_t stage_cap = rv.vec ? 2047u : 0u;  // the region's last slot takes the vectors of the ranks beyond
-        if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, cache, red_f, stage, stage_cap, anchor, aq, m);
+        if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m);
         __syncthreads();
         WS_MARK(8);
         gather_and_adjust(stage, swept ? stage_cap : 0u);
@@ -825,7 +835,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #pragma unroll
         for (int j = 0; j < kPT; ++j) {
             const int b = kPT * t + j;
-            const uint64_t h = hist[b];
+            const uint64_t h = hist[b] + (cached && hist2 ? hist2[b] : 0ull);  // the fields add up without a carry between them
             c[j] = static_cast<uint32_t>(h >> kCountShift);
             if (b == kBins - 1) c[j] -= tail_fix;  // streamed there as NaN, replayed into their own bins
             const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
