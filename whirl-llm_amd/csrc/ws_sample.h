@@ -347,33 +347,34 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
     return (((k >> lp) * WS_BLOCK + threadIdx.x) << (lp + 1u)) + 2u * (k & ((1u << lp) - 1u)) + half;
 }
 
-// Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range): its index goes
-// to list[] (LDS, at most cap entries; *n_list, zeroed by the caller before a barrier, counts all hits). Both 16-bit
-// halves of a register are tested at once with packed 16-bit subtractions: (y - lo) and (y - hi - 1) differ in bit 15
-// exactly for lo <= bin <= hi (bins are below 4096, so neither difference wraps twice). Hits are shifted into one
-// mask per 16 registers; then each wave reserves a stretch of the list with one atomic and its lanes write their tokens.
+// Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range; else
+// u0 + w0 < u1): its index goes to list[] (LDS, at most cap entries; *n_list, zeroed by the caller before a barrier,
+// counts all hits). Both 16-bit halves of a register are tested at once with ordinary 32-bit additions: bins are
+// below 4096, so y + (0x8000 - c) in each half neither carries into the other half nor wraps, and its bit 15 says
+// bin >= c. With the bounds lo0 < hi0 <= lo1 < hi1 (hi = last bin + 1) the four answers turn true one after the other
+// as the bin grows, so the bin lies in a range exactly when an odd number of them is true: the xor of the four sums has
+// bit 15 set. Hits are shifted into one mask per 16 registers; then each wave reserves a stretch of the list with one
+// atomic and its lanes write their tokens.
 __device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
                                                   uint32_t w1, uint32_t* list, uint32_t* n_list, uint32_t cap) {
-    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
     const bool two = u1 <= 0x7fffu;
-    const u16x2 L0 = static_cast<unsigned short>(u0), H0 = static_cast<unsigned short>(u0 + w0 + 1u);
-    const u16x2 L1 = static_cast<unsigned short>(two ? u1 : 0u), H1 = static_cast<unsigned short>(two ? u1 + w1 + 1u : 0u);
+    auto at_least = [](uint32_t c) { return 0x80008000u - c * 0x10001u; };  // y + this: bit 15 of a half = (bin >= c)
+    const uint32_t L0 = at_least(u0), H0 = at_least(u0 + w0 + 1u);
+    const uint32_t L1 = at_least(two ? u1 : 0u), H1 = at_least(two ? u1 + w1 + 1u : 0u);
     uint32_t hits[kCacheRegs / 16];
     uint32_t mine = 0;
-    auto test16 = [&](int g, u16x2 lo, u16x2 hi) {  // bit k / 16 + k: low / high half of register 16 g + k lies in [lo, hi)
+    // bit k / 16 + k of the result: low / high half of register 16 g + k lies in a range
+    auto test16 = [&](int g, auto&& sign) {
         uint32_t acc = 0;
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const u16x2 y = __builtin_bit_cast(u16x2, cache[g * 16 + k]);
-            const uint32_t r = __builtin_bit_cast(uint32_t, static_cast<u16x2>(y - lo)) ^ __builtin_bit_cast(uint32_t, static_cast<u16x2>(y - hi));
-            acc = (acc >> 1) | (r & 0x80008000u);
-        }
+        for (int k = 0; k < 16; ++k) acc = (acc >> 1) | (sign(cache[g * 16 + k]) & 0x80008000u);
         return acc;
     };
 #pragma unroll
     for (int g = 0; g < kCacheRegs / 16; ++g) {
-        uint32_t acc = test16(g, L0, H0);
-        if (two) acc |= test16(g, L1, H1);  // uniform branch
+        uint32_t acc;
+        if (two) acc = test16(g, [&](uint32_t y) { return (y + L0) ^ (y + H0) ^ (y + L1) ^ (y + H1); });  // uniform branch
+        else acc = test16(g, [&](uint32_t y) { return (y + L0) ^ (y + H0); });
         hits[g] = acc;
         mine += __popc(acc);
         __builtin_amdgcn_sched_barrier(0);  // one group at a time: a wider scheduling window costs more registers than it hides
