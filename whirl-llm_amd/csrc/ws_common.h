@@ -82,6 +82,20 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_or_self<0x143, 0xc>(v));
     return last_lane(v);
 }
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_self(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    v = min(v, dpp_or_self<0x111, 0xf>(v));
+    v = min(v, dpp_or_self<0x112, 0xf>(v));
+    v = min(v, dpp_or_self<0x114, 0xf>(v));
+    v = min(v, dpp_or_self<0x118, 0xf>(v));
+    v = min(v, dpp_or_self<0x142, 0xa>(v));
+    v = min(v, dpp_or_self<0x143, 0xc>(v));
+    return last_lane(v);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) { return ~wave_min_u32(~v); }
 __device__ __forceinline__ float wave_sum(float v) { return last_lane(wave_incl_scan(v)); }
 __device__ __forceinline__ double wave_sum(double v) { return last_lane(wave_incl_scan(v)); }
 __device__ __forceinline__ uint32_t wave_sum(uint32_t v) { return last_lane(wave_incl_scan(v)); }
@@ -133,8 +147,7 @@ __device__ __forceinline__ void block_max2(float& a, float& b, float* red_a, flo
     }
 }
 __device__ __forceinline__ uint32_t block_min(uint32_t v, uint32_t* red) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = min(v, static_cast<uint32_t>(__shfl_xor(v, o)));
+    v = wave_min_u32(v);
     __syncthreads();
     if (lane_id() == 0) red[wave_id()] = v;
     __syncthreads();
@@ -184,6 +197,29 @@ __device__ __forceinline__ T block_excl_scan(T v, T* red, T* total) {
         tot += s;
     }
     *total = tot;
+    return base + inc - v;
+}
+
+// the same for uint32 counts, with the block's maximum of a second value on the same two barriers (mx is replaced by it)
+__device__ __forceinline__ uint32_t block_excl_scan_max(uint32_t v, uint32_t& mx, uint32_t* red, uint32_t* red_mx, uint32_t* total) {
+    const uint32_t inc = wave_incl_scan(v);
+    const uint32_t wmx = wave_max_u32(mx);
+    __syncthreads();
+    if (lane_id() == 63) {
+        red[wave_id()] = inc;
+        red_mx[wave_id()] = wmx;
+    }
+    __syncthreads();
+    uint32_t base = 0, tot = 0, m = 0;
+#pragma unroll
+    for (int w = 0; w < WS_WAVES; ++w) {
+        const uint32_t s = red[w];
+        if (w < wave_id()) base += s;
+        tot += s;
+        m = max(m, red_mx[w]);
+    }
+    *total = tot;
+    mx = m;
     return base + inc - v;
 }
 

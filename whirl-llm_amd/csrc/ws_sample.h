@@ -409,6 +409,19 @@ __device__ __forceinline__ uint32_t first_key_before_bin(float aq, float c64, fl
     return hi;
 }
 
+// number of keys in a[b0, b1) greater than key; four independent reads per round (the last index stands in past the end)
+__device__ __forceinline__ uint32_t ranked_before(const uint64_t* a, uint32_t b0, uint32_t b1, uint64_t key) {
+    uint32_t before = 0;
+    for (uint32_t j = b0; j < b1; j += 4u) {
+        uint64_t v[4];
+#pragma unroll
+        for (uint32_t e = 0; e < 4u; ++e) v[e] = a[min(j + e, b1 - 1u)];
+#pragma unroll
+        for (uint32_t e = 0; e < 4u; ++e) before += (j + e < b1 && v[e] > key) ? 1u : 0u;
+    }
+    return before;
+}
+
 // results of a lookup in the scanned histogram
 struct BinSel {
     int b;        // bin, -1 = none
@@ -436,16 +449,12 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
     }
 }
 
-// Debug builds (-DWS_PHASE_TIMERS) store the shader-clock time of each phase of every row into kept_logits.
+// Debug builds (-DWS_PHASE_TIMERS): thread 0 notes the shader clock at each mark in LDS (no barrier, no global store on
+// the way) and writes the times since the start of the row into kept_logits when the row is done.
 #ifdef WS_PHASE_TIMERS
-#define WS_MARK(k)                                                                                                   \
-    do {                                                                                                               \
-        __syncthreads();                                                                                               \
-        if (threadIdx.x == 0 && A.kept_logits) {                                                                       \
-            const long long now = clock64();                                                                           \
-            A.kept_logits[static_cast<size_t>(blockIdx.x) * A.kept_cap + (k)] = static_cast<float>(now - ws_t0);      \
-            ws_t0 = now;                                                                                               \
-        }                                                                                                              \
+#define WS_MARK(k)                                          \
+    do {                                                    \
+        if (threadIdx.x == 0) ws_marks[(k)] = clock64();    \
     } while (0)
 #else
 #define WS_MARK(k) \
@@ -456,7 +465,10 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
 template <bool FUSED>
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #ifdef WS_PHASE_TIMERS
-    long long ws_t0 = clock64();
+    __shared__ long long ws_marks[32];
+    const long long ws_t0 = clock64();
+    if (threadIdx.x < 32) ws_marks[threadIdx.x] = 0;
+    __syncthreads();
 #endif
     extern __shared__ __align__(16) unsigned char lds[];
     __shared__ float red_f[WS_WAVES];
@@ -464,6 +476,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ double red_d[WS_WAVES];
     __shared__ uint32_t s_cnt;
     __shared__ double s_exp[128];  // kExpHi, kExpLo
+    __shared__ double pm64[64];    // every 64th entry of the scanned histogram's mass prefixes
+    __shared__ uint32_t pc64[64];  // and of its count prefixes
+    __shared__ double tot_m[64];   // histogram scan: mass and count of each stretch of 64 bins
+    __shared__ uint32_t tot_c[64];
     __shared__ uint32_t s_u[8];
 
     const uint32_t row = blockIdx.x;
@@ -547,8 +563,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             uint32_t wd[kChunkRegs];
             uint32_t local = 0;
 #pragma unroll
+            for (uint32_t k = 0; k < kChunkRegs; ++k) wd[k] = touched[min(w0 + k, nW - 1u)];  // unconditional: the reads go out together
+#pragma unroll
             for (uint32_t k = 0; k < kChunkRegs; ++k) {
-                wd[k] = w0 + k < w1 ? touched[w0 + k] : 0u;
+                if (w0 + k >= w1) wd[k] = 0u;
                 local += __popc(wd[k]);
             }
             uint32_t run = block_excl_scan(local, red_u, &n_uniq);
@@ -622,8 +640,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint32_t* first = cnt + A.patch_cap;
         float mu = -INFINITY;  // largest untouched, allowed logit among the vectors that hold touched tokens
         auto fetch4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {  // four independent gathers per thread and round
+            const uint32_t whole_end = rv.vec ? (V & ~(per - 1u)) : 0u;  // tokens below this sit in whole 128-bit vectors
             for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
-                uint32_t id[4], bits[4], al[4];
+                // Every step for all four entries before the next step: reads that sit inside a branch are waited for
+                // one by one, reads issued side by side wait once.
+                uint32_t id[4], al[4], tw[4], wp[4], rf[4];
                 uint4 vec[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -635,12 +656,23 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
                     al[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
-                    if (rv.vec && i < (V & ~(per - 1u))) {
-                        // the token's whole 128-bit vector: staged by the sweep under the rank of the vector's first
-                        // touched token, else fetched
-                        const uint32_t vb = i & ~(per - 1u), tw = touched[i >> 5];
-                        const uint32_t rf = static_cast<uint32_t>(wprefix[i >> 5]) + __popc(tw & ((1u << (vb & 31u)) - 1u));
-                        vec[k] = rf < stage_cap ? stage[rf] : static_cast<const uint4*>(rv.base)[i >> lper];
+                    tw[k] = touched[i >> 5];
+                    wp[k] = wprefix[i >> 5];
+                }
+                // the token's whole 128-bit vector: staged by the sweep under the rank of the vector's first touched
+                // token, else fetched
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    const uint32_t vb = i & ~(per - 1u);
+                    rf[k] = wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u));
+                    if (stage_cap) vec[k] = stage[min(rf[k], stage_cap)];  // uniform; slot stage_cap is the sweep's dump
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    if (i < whole_end) {
+                        if (rf[k] >= stage_cap) vec[k] = static_cast<const uint4*>(rv.base)[i >> lper];
                     } else {
                         const uint32_t b = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
                                                          : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
@@ -652,13 +684,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     if (id[k] >= V) continue;
                     const uint32_t i = id[k];
                     const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
-                    const bool whole = rv.vec && i < (V & ~(per - 1u));
-                    if (!whole) bits[k] = w[0];
-                    else bits[k] = rv.dtype == 0 ? w[i & 3u] : ((i & 1u) ? w[(i & 7u) >> 1] & 0xffff0000u : w[(i & 7u) >> 1] << 16);
-                    pv[rank_of(rv, i)] = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits[k]), -INFINITY) : -INFINITY;
+                    const bool whole = i < whole_end;
+                    uint32_t bits;
+                    if (!whole) bits = w[0];
+                    else bits = rv.dtype == 0 ? w[i & 3u] : ((i & 1u) ? w[(i & 7u) >> 1] & 0xffff0000u : w[(i & 7u) >> 1] << 16);
+                    const uint32_t rank = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));  // rank_of(rv, i)
+                    pv[rank] = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits), -INFINITY) : -INFINITY;
                     if (FUSED && whole) {
                         const uint32_t vb = i & ~(per - 1u);
-                        const uint32_t free_bits = (al[k] & ~touched[i >> 5]) >> (vb & 31u);  // allowed and untouched
+                        const uint32_t free_bits = (al[k] & ~tw[k]) >> (vb & 31u);  // allowed and untouched
                         if (rv.dtype == 0) {
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
@@ -823,62 +857,85 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double to_max = exp(lift);
 
     WS_MARK(2);
-    // scan: thread t owns kPT consecutive bins (bin 0 = nearest the anchor). The exclusive prefixes go back to LDS -
-    // masses pm[0..4096] over the histogram itself, counts pc[0..4096] behind them - so that the lookups below hold
-    // nothing in registers between barriers (the bin cache of the single-sweep mode needs them)
+    // scan (bin 0 = nearest the anchor). The exclusive prefixes go back to LDS - masses pm[0..4096] over the histogram
+    // itself, counts pc[0..4096] behind them - so that the lookups below hold nothing in registers between barriers
+    // (the bin cache of the single-sweep mode needs them). The bins are taken in 64 stretches of 64: stretch g goes to
+    // wave g % WS_WAVES, bin by lane, so that every LDS access here has neighbouring lanes on neighbouring words, the
+    // populated stretches (a few hundred bins below the maximum) spread over all waves, and a stretch without a token
+    // costs no arithmetic. Each stretch is scanned by its wave, the 64 stretch totals by every wave again.
     double* pm = reinterpret_cast<double*>(lds);                       // 4097 doubles
     uint32_t* pc = reinterpret_cast<uint32_t*>(lds + 32768 + 16);      // 4097 counts
     {
-        uint32_t c[kPT];
-        double ms[kPT];
-        uint32_t csum = 0;
-        double msum = 0;
+        constexpr int kR = 64 / WS_WAVES;  // stretches per wave
+        const uint32_t lane = static_cast<uint32_t>(lane_id());
+        const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+        const bool two_copies = cached && hist2;
+        const uint64_t* hist_b = two_copies ? hist2 : hist;  // the same words twice when there is one copy
+        const double el = s_exp[64 + lane];                  // exp(-(b & 63) / 64)
+        uint64_t h[kR];
 #pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            const int b = kPT * t + j;
-            const uint64_t h = hist[b] + (cached && hist2 ? hist2[b] : 0ull);  // the fields add up without a carry between them
-            c[j] = static_cast<uint32_t>(h >> kCountShift);
-            if (b == kBins - 1) c[j] -= tail_fix;  // streamed there as NaN, replayed into their own bins
-            const double fix = static_cast<double>(h & ((1ull << kCountShift) - 1ull)) * kFixInv;
-            // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail bin carries none
-            ms[j] = (c[j] && b < kBins - 1) ? s_exp[b >> 6] * s_exp[64 + (b & 63)] * (static_cast<double>(c[j]) - fix) * to_max : 0.0;
-            csum += c[j];
-            msum += ms[j];
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t b = 64u * (r * WS_WAVES + wv) + lane;
+            h[r] = hist[b];
+            const uint64_t hb = hist_b[b];
+            if (two_copies) h[r] += hb;  // the fields add up without a carry between them
         }
-        // exclusive scan of (count, mass) over the threads, both in one go; its barriers separate the reads of hist
-        // above from the writes below
-        const uint32_t cinc = wave_incl_scan(csum);
-        const double minc = wave_incl_scan(msum);
-        __syncthreads();
-        if (lane_id() == 63) {
-            red_u[wave_id()] = cinc;
-            red_d[wave_id()] = minc;
-        }
-        __syncthreads();
-        uint32_t ctot = 0, cb = cinc - csum;
-        double mtot = 0, mbase = 0;
+        WS_MARK(24);
+        uint32_t c[kR], cex[kR];
+        double mex[kR];
 #pragma unroll
-        for (int w = 0; w < WS_WAVES; ++w) {
-            const uint32_t cw = red_u[w];
-            const double mw = red_d[w];
-            if (w < wave_id()) {
-                cb += cw;
-                mbase += mw;
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t g = r * WS_WAVES + wv, b = 64u * g + lane;
+            c[r] = static_cast<uint32_t>(h[r] >> kCountShift);
+            if (b == kBins - 1) c[r] -= tail_fix;  // streamed there as NaN, replayed into their own bins
+            double minc = 0.0;
+            uint32_t cinc = 0u;
+            mex[r] = 0.0;
+            cex[r] = 0u;
+            if (__ballot(c[r] != 0u)) {  // uniform: a stretch without a token needs no arithmetic at all
+                const double fix = static_cast<double>(h[r] & ((1ull << kCountShift) - 1ull)) * kFixInv;
+                // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail bin carries none
+                const double ms = (c[r] && b < kBins - 1) ? s_exp[g] * el * (static_cast<double>(c[r]) - fix) * to_max : 0.0;
+                minc = wave_incl_scan(ms);
+                cinc = wave_incl_scan(c[r]);
+                // exclusive inside the stretch = the lane below's inclusive value: no subtraction, no rounding of its own
+                const double mup = __shfl_up(minc, 1);
+                mex[r] = lane ? mup : 0.0;
+                cex[r] = cinc - c[r];
             }
-            ctot += cw;
-            mtot += mw;
+            if (lane == 63u) {
+                tot_c[g] = cinc;
+                tot_m[g] = minc;
+            }
         }
-        double mb = mbase + minc - msum;
+        WS_MARK(25);
+        __syncthreads();  // every read of the histogram is done (the prefixes go over it); the stretch totals are in place
+        WS_MARK(26);
+        const uint32_t uc = tot_c[lane];
+        const double um = tot_m[lane];
+        const uint32_t Pc = wave_incl_scan(uc);  // counts up to and with stretch `lane` = pc[64 lane + 64]
+        const double Pm = wave_incl_scan(um);
+        const double Pm_up = __shfl_up(Pm, 1);
+        const double Em = lane ? Pm_up : 0.0;    // masses before stretch `lane`: exactly the value published as pm64[lane - 1]
+        const uint32_t Ec = Pc - uc;
+        if (wv == 0u) {  // every 64th prefix once more, side by side, for the searches' first probe
+            pc64[lane] = Pc;
+            pm64[lane] = Pm;
+            if (lane == 63u) {
+                pc[kBins] = Pc;
+                pm[kBins] = Pm;
+            }
+        }
 #pragma unroll
-        for (int j = 0; j < kPT; ++j) {
-            pc[kPT * t + j] = cb;
-            pm[kPT * t + j] = mb;
-            cb += c[j];
-            mb += ms[j];
-        }
-        if (t == WS_BLOCK - 1) {
-            pc[kBins] = ctot;
-            pm[kBins] = mtot;
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t g = r * WS_WAVES + wv, b = 64u * g + lane;
+            const uint32_t bc = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(Ec), g));
+            const uint64_t em_bits = static_cast<uint64_t>(__double_as_longlong(Em));
+            const uint32_t em_lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(em_bits)), g));
+            const uint32_t em_hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(em_bits >> 32)), g));
+            const double bm = __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(em_hi) << 32) | em_lo));
+            pc[b] = bc + cex[r];
+            pm[b] = bm + mex[r];
         }
     }
     __syncthreads();  // the histogram is gone; after the lookups its LDS becomes the key buffer
@@ -897,9 +954,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
     // smallest bin for which reached(bin) holds (monotone in the bin), kBins if none: a 64-way search by the wave,
     // lane i probing the last bin of the i-th stretch of 64 bins, then bin i of the stretch found. Two LDS round trips.
-    auto first_bin = [&](auto&& reached) {
+    // reached_end(i): the predicate at the last bin of stretch i, read from the side arrays (pc64[i] = pc[64 i + 64],
+    // pm64[i] = pm[64 i + 64]: neighbouring lanes read neighbouring words instead of one LDS bank all together)
+    auto first_bin = [&](auto&& reached_end, auto&& reached) {
         const int lane = lane_id();
-        const uint64_t coarse = __ballot(reached(64 * lane + 63));
+        const uint64_t coarse = __ballot(reached_end(lane));
         if (!coarse) return static_cast<int>(kBins);
         const int base = 64 * (__ffsll(static_cast<unsigned long long>(coarse)) - 1);
         const uint64_t fine = __ballot(reached(base + lane));
@@ -907,12 +966,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
     auto find_count = [&](uint32_t n) {  // bin holding the element of rank n - 1, -1 if there is none
         if (n == 0) return -1;
-        const int b = first_bin([&](int k) { return pc[k + 1] >= n; });
+        const int b = first_bin([&](int i) { return pc64[i] >= n; }, [&](int k) { return pc[k + 1] >= n; });
         return b < kBins ? b : -1;
     };
     auto find_mass = [&](double X, bool strict) {  // first non-empty bin whose inclusive mass prefix reaches X, -1 if none
         if (!strict && !(X > 0.0)) return -1;
-        int b = strict ? first_bin([&](int k) { return pm[k + 1] > X; }) : first_bin([&](int k) { return pm[k + 1] >= X; });
+        int b = strict ? first_bin([&](int i) { return pm64[i] > X; }, [&](int k) { return pm[k + 1] > X; })
+                       : first_bin([&](int i) { return pm64[i] >= X; }, [&](int k) { return pm[k + 1] >= X; });
         while (b < kBins && pc[b + 1] == pc[b]) ++b;  // an empty bin can only turn up through rounding at a scan seam
         return b < kBins ? b : -1;
     };
@@ -1174,6 +1234,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #pragma unroll
             for (int q = 0; q < kCh; ++q) {
                 const uint32_t i = q * WS_BLOCK + t;
+                key[q] = 0ull;
+                rb[q] = 0u;
                 if (i < n_list) {
                     key[q] = keys[i];
                     const uint32_t k32 = static_cast<uint32_t>(key[q] >> 32);
@@ -1181,7 +1243,20 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     const uint32_t bin = static_cast<uint32_t>(tcs[q]);
                     rb[q] = (has_r1 && i >= n_r0) ? nb0 + (bin - static_cast<uint32_t>(r1lo)) : bin - static_cast<uint32_t>(r0lo);
                     rb[q] = min(rb[q], nb0 + nb1 - 1u);
-                    if (spot_ties) {
+                }
+                if (spot_ties && static_cast<uint32_t>(q) * WS_BLOCK < n_list) {  // uniform
+                    // candidates arrive bin after bin, so the lanes of a wave mostly share their bin: one pair of
+                    // atomics per wave then, instead of 64 that queue on one address
+                    const bool live = i < n_list;
+                    const uint32_t k32 = static_cast<uint32_t>(key[q] >> 32);
+                    const uint32_t rb0 = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(live ? rb[q] : 0xffffffffu)));
+                    if (__ballot(live && rb[q] != rb0) == 0ull && rb0 != 0xffffffffu) {
+                        const uint32_t lo = wave_min_u32(live ? k32 : 0xffffffffu), hi = wave_max_u32(live ? k32 : 0u);
+                        if (lane_id() == 0) {
+                            atomicMin(&bin_lo[rb0], lo);
+                            atomicMax(&bin_hi[rb0], hi);
+                        }
+                    } else if (live) {
                         atomicMin(&bin_lo[rb[q]], k32);
                         atomicMax(&bin_hi[rb[q]], k32);
                     }
@@ -1201,6 +1276,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
             }
             __syncthreads();
+            WS_MARK(21);
             // exclusive scan of the counts (a few consecutive buckets per thread) and the largest bucket
             constexpr uint32_t kPB = (kMaxBuckets + WS_BLOCK - 1) / WS_BLOCK;
             // Buckets of more than kMaxInBucket keys are listed: where all keys of such a bucket carry one logit - the
@@ -1218,8 +1294,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
             }
             uint32_t total;
-            uint32_t run = block_excl_scan(sum, red_u, &total);
-            biggest = 0xffffffffu - block_min(0xffffffffu - biggest, red_u);
+            uint32_t run = block_excl_scan_max(sum, biggest, red_u, reinterpret_cast<uint32_t*>(red_f), &total);
 #pragma unroll
             for (uint32_t j = 0; j < kPB; ++j) {
                 const uint32_t b = kPB * t + j;
@@ -1233,6 +1308,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             int big_of[kCh];  // index of the key's bucket in the list of big buckets, -1 for an ordinary bucket
 #pragma unroll
             for (int q = 0; q < kCh; ++q) big_of[q] = -1;
+            // Second level for the big buckets, all at once: where every key of such a bucket carries one logit, the
+            // order inside it is the order of the token ids, so the bucket is cut into kS2 steps of the id, counted,
+            // scanned and ranked like the first level. Counters: the spare LDS (n_big * kS2 + 1 words).
+            constexpr uint32_t kS2 = 256;
+            constexpr uint32_t kPB2 = (kMaxBig * kS2 + WS_BLOCK - 1) / WS_BLOCK;
+            uint32_t* c2 = reinterpret_cast<uint32_t*>(lds + A.lds_tie);
+            uint32_t sub2[kCh], arr2[kCh];
             if (!ok && n_big <= kMaxBig && A.lds_tie) {  // uniform
                 // one logit per big bucket?
 #pragma unroll
@@ -1245,10 +1327,42 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         atomicMax(&big_hi[big_of[q]], static_cast<uint32_t>(key[q] >> 32));
                     }
                 }
+                for (uint32_t b = t; b <= n_big * kS2; b += WS_BLOCK) c2[b] = 0u;
                 __syncthreads();
                 ok = true;
                 for (uint32_t k = 0; k < n_big; ++k) ok = ok && big_lo[k] == big_hi[k];
+                if (ok) {  // uniform
+                    const float step2 = static_cast<float>(kS2) / static_cast<float>(V);
+#pragma unroll
+                    for (int q = 0; q < kCh; ++q)
+                        if (big_of[q] >= 0) {
+                            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
+                            sub2[q] = static_cast<uint32_t>(big_of[q]) * kS2 + min(kS2 - 1u, static_cast<uint32_t>(static_cast<float>(id) * step2));
+                            arr2[q] = atomicAdd(&c2[sub2[q]], 1u);
+                        }
+                    __syncthreads();
+                    uint32_t local2[kPB2], sum2 = 0, biggest2 = 0;
+#pragma unroll
+                    for (uint32_t j = 0; j < kPB2; ++j) {
+                        const uint32_t b2 = kPB2 * t + j;
+                        local2[j] = b2 < n_big * kS2 ? c2[b2] : 0u;
+                        sum2 += local2[j];
+                        biggest2 = max(biggest2, local2[j]);
+                    }
+                    uint32_t total2;
+                    uint32_t run2 = block_excl_scan_max(sum2, biggest2, red_u, reinterpret_cast<uint32_t*>(red_f), &total2);
+#pragma unroll
+                    for (uint32_t j = 0; j < kPB2; ++j) {
+                        const uint32_t b2 = kPB2 * t + j;
+                        if (b2 < n_big * kS2) c2[b2] = run2;
+                        run2 += local2[j];
+                    }
+                    if (t == 0) c2[n_big * kS2] = total2;
+                    __syncthreads();
+                    ok = biggest2 <= kMaxInBucket;  // ids that crowd one step: the comparison sorts take over
+                }
             }
+            WS_MARK(22);
             if (ok) {  // uniform; keys[] has not been written so far, so the comparison sorts below can still take over
 #pragma unroll
                 for (int q = 0; q < kCh; ++q)
@@ -1258,46 +1372,26 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 for (int q = 0; q < kCh; ++q) {
                     if (q * WS_BLOCK + t >= n_list || big_of[q] >= 0) continue;
                     const uint32_t b0 = bcnt[bucket[q]], b1 = bcnt[bucket[q] + 1u];
-                    uint32_t before = 0;
-                    for (uint32_t j = b0; j < b1; ++j) before += tmp[j] > key[q] ? 1u : 0u;
-                    keys[b0 + before] = key[q];  // every key was read into registers before the first barrier above
+                    keys[b0 + ranked_before(tmp, b0, b1, key[q])] = key[q];  // every key was read into registers before the first barrier above
                 }
-                // a big bucket of equal logits: its keys in ascending id order = set the ids' bits, count the bits below
-                uint32_t* tie_bits = reinterpret_cast<uint32_t*>(lds + A.lds_tie);
-                uint16_t* tie_pref = reinterpret_cast<uint16_t*>(lds + A.lds_tie + nW * 4u);
-                for (uint32_t k = 0; k < (biggest > kMaxInBucket ? n_big : 0u); ++k) {
-                    __syncthreads();
-                    for (uint32_t w = t; w < nW; w += WS_BLOCK) tie_bits[w] = 0u;
+                if (biggest > kMaxInBucket) {  // uniform: the keys of the big buckets, through the same staging array
                     __syncthreads();
 #pragma unroll
                     for (int q = 0; q < kCh; ++q)
-                        if (big_of[q] == static_cast<int>(k)) {
-                            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
-                            atomicOr(&tie_bits[id >> 5], 1u << (id & 31u));
-                        }
+                        if (big_of[q] >= 0) tmp[c2[sub2[q]] + arr2[q]] = key[q];
                     __syncthreads();
-                    const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
-                    const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
-                    uint32_t mine = 0;
-                    for (uint32_t w = w0; w < w1; ++w) mine += __popc(tie_bits[w]);
-                    uint32_t all;
-                    uint32_t at = block_excl_scan(mine, red_u, &all);
-                    for (uint32_t w = w0; w < w1; ++w) {
-                        tie_pref[w] = static_cast<uint16_t>(at);
-                        at += __popc(tie_bits[w]);
+#pragma unroll
+                    for (int q = 0; q < kCh; ++q) {
+                        if (big_of[q] < 0) continue;
+                        const uint32_t b0 = c2[sub2[q]], b1 = c2[sub2[q] + 1u];
+                        const uint32_t before = ranked_before(tmp, b0, b1, key[q]);  // equal logits: the lower id is the larger key
+                        keys[bcnt[bucket[q]] + (b0 - c2[static_cast<uint32_t>(big_of[q]) * kS2]) + before] = key[q];
                     }
-                    __syncthreads();
-#pragma unroll
-                    for (int q = 0; q < kCh; ++q)
-                        if (big_of[q] == static_cast<int>(k)) {
-                            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key[q]);
-                            const uint32_t rank = static_cast<uint32_t>(tie_pref[id >> 5]) + __popc(tie_bits[id >> 5] & ((1u << (id & 31u)) - 1u));
-                            keys[bcnt[bucket[q]] + rank] = key[q];
-                        }
                 }
                 __syncthreads();
                 sorted = true;
             }
+            WS_MARK(23);
         }
     }
     constexpr int kMergeCh = 6;  // keys per thread the merge sort takes (3072 keys; beyond that the bitonic sort)
@@ -1530,6 +1624,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (mg_draw < tol) flags |= kNearDraw;
 
     WS_MARK(7);
+#ifdef WS_PHASE_TIMERS
+    if (t == 0 && A.kept_logits) {
+        float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
+        for (uint32_t k = 0; k < 32u && k < A.kept_cap; ++k)
+            if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
+    }
+#endif
     if (t == 0) {
         A.token[row] = token;
         A.flags[row] = flags;
