@@ -78,6 +78,24 @@ def test_masked_rows(mode):
     print(res)
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_rows_masked_by_minus_infinity_in_the_logits(mode):
+    """Constrained decoding the plain way: no allow bitmap, most of the row set to -inf (and a few NaN) in the logits
+    themselves. All those tokens land in the tail of the histogram; one row asks for more candidates than it has
+    finite logits, so its top-k reaches into the tail."""
+    c = gc.make_cfg2(rows=6, V=65536, n_hist=300, n_bias=20)
+    rng = np.random.default_rng(99)
+    for r, keep in enumerate([0.5, 0.1, 0.02, 0.002, 0.0005, 0.1]):
+        off = rng.random(c["V"]) >= keep
+        c["logits"][r, off] = -np.inf
+        c["logits"][r, rng.integers(0, c["V"], 7)] = np.nan
+    c["top_k"][:] = [0, 50, 20, 0, 50, 0]
+    c["top_p"][:] = [0.9, 0.95, 1.0, 0.9, 1.0, 0.8]
+    c["min_p"][:] = [0.0, 0.0, 0.0, 0.01, 0.0, 0.05]
+    res, _ = run_case(c, 1, mode=mode)
+    print(res)
+
+
 def test_flagged_rows():
     m = gc.pkg()
     c = gc.make_cfg5(rows=3, V=8192, n_hist=50, n_bias=5)

@@ -122,7 +122,7 @@ __device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
 // constant after unrolling); end_batch(j0, i) after each batch of kBatch 128-bit loads per thread (j0 = first vector
 // index of the batch; j0 = ~0 and i = the token for the one-token batches of a scalar tail), which are all issued
 // before any is used, and the next batch is requested before this one is consumed. Tokens that are masked out or that
-// the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bin or ignores it, so the
+// the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bins or ignores it, so the
 // hot loop has no branch; the touched ones are fed afterwards, by rank, with their adjusted values.
 template <bool MASKED, class F, class E>
 __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch) {
@@ -192,17 +192,22 @@ __device__ __forceinline__ void stream_row(const RowView& rv, F&& f, E&& end_bat
 
 // ---- bins. A token's bin coordinate is t = fma(x, -c64, aq): c64 = 64 * inv_t and aq = anchor * c64 rounded a little
 // upwards (anchor_product), so that t >= 0 for every x <= anchor; t = 64 * (aq / 64 - x * inv_t) to half an ulp of t,
-// one rounding. bin = trunc(min(t, 4095)): bin 0 is nearest the anchor, 1/64 of an exponent unit per bin, and the tail
-// bin 4095 takes NaN, -inf and everything whose mass is below e^-64 of the anchor's. The same function is used by
-// every pass, so a token's bin never depends on who computes it.
+// one rounding. bin = trunc(min(t, tail)): bin 0 is nearest the anchor, 1/64 of an exponent unit per bin. Bins kTail ..
+// 4095, the last stretch of 64, are the tail: NaN, -inf and everything whose mass is below e^-63 of the anchor's; they
+// carry no mass and are told apart by nobody. A thread that adds to the histogram clamps to a tail bin of its own
+// lane (kTail + lane): a row masked down to a fraction of its vocabulary sends tokens there by the hundred thousand, and
+// 64 lanes adding to one LDS word are served one after the other. Below the tail the same function is used by every
+// pass, so a token's bin never depends on who computes it.
 __device__ __forceinline__ float anchor_product(float anchor, float c64) {
     const float a = __fmul_rn(anchor, c64);
     return __fmaf_rn(fabsf(a), 4.76837158203125e-7f, a);  // + 2^-21 |a|: above the exact product whatever the roundings
 }
-__device__ __forceinline__ float bin_coord(float aq, float c64, float x) {
+constexpr int kTail = 4032;  // first bin of the tail
+__device__ __forceinline__ float bin_coord(float aq, float c64, float x, float tail = 4095.f) {
     const float t = __fmaf_rn(x, -c64, aq);
-    return t < 4095.f ? t : 4095.f;  // NaN -> tail
+    return __builtin_fminf(t, tail);  // minNum: NaN -> tail
 }
+__device__ __forceinline__ float own_tail() { return static_cast<float>(kTail + lane_id()); }
 __device__ __forceinline__ uint32_t bin_of(float aq, float c64, float x) { return static_cast<uint32_t>(bin_coord(aq, c64, x)); }
 // histogram word of one token: count 1 and the fixed-point quadratic of the in-bin offset w = fract(t)
 __device__ __forceinline__ uint64_t bin_word(float tc) {
@@ -229,6 +234,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
     const uint32_t nv = rv.V / PER;
+    const float tail_f = own_tail();
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     uint4 q[kRing][kBatch];
     uint32_t na[kRing][kBatch];
@@ -300,7 +306,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
                     if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
                     const float x = __uint_as_float(bits);
                     vm = fmaxf(vm, x);
-                    const float tc = bin_coord(aq, c64, x);
+                    const float tc = bin_coord(aq, c64, x, tail_f);
                     bins[e] = static_cast<uint32_t>(tc);
                     atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bins[e]]), bin_word(tc));
                 }
@@ -780,8 +786,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const float c64 = inv_t * 64.f;
     float anchor = 0.f;  // bins are measured down from here: the row maximum, or a provisional bound above it
     float aq = 0.f;      // anchor_product(anchor, c64)
+    const float tail_f = own_tail();
     auto add_to_hist = [&](uint32_t, float x, int) {
-        const float tc = bin_coord(aq, c64, x);
+        const float tc = bin_coord(aq, c64, x, tail_f);
         atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(tc)]), bin_word(tc));
     };
     float m = -INFINITY;
@@ -803,7 +810,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             m = block_max(m, red_f);  // over the vectors of the row that hold no touched token (allow mask applied)
             // touched tokens: out of the bin of the raw logit, into the bin of the adjusted one
             for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
-                const float t0 = bin_coord(aq, c64, praw[r]), t1 = bin_coord(aq, c64, pv[r]);
+                const float t0 = bin_coord(aq, c64, praw[r], tail_f), t1 = bin_coord(aq, c64, pv[r], tail_f);
                 atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
                 atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
             }
@@ -850,7 +857,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         stream_row(rv, add_to_hist, [](uint32_t, uint32_t) {});
         replay_touched([&](uint32_t i, float x) { add_to_hist(i, x, 0); });
     }
-    const uint32_t tail_fix = cached ? 0u : n_touched;  // pass 2 streams touched tokens into the tail bin as NaN
     __syncthreads();
     // masses are accumulated relative to the anchor; everything below works relative to the maximum
     const double lift = static_cast<double>(aq) * (1.0 / 64.0) - static_cast<double>(m) * static_cast<double>(inv_t);  // >= 0
@@ -887,15 +893,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         for (int r = 0; r < kR; ++r) {
             const uint32_t g = r * WS_WAVES + wv, b = 64u * g + lane;
             c[r] = static_cast<uint32_t>(h[r] >> kCountShift);
-            if (b == kBins - 1) c[r] -= tail_fix;  // streamed there as NaN, replayed into their own bins
             double minc = 0.0;
             uint32_t cinc = 0u;
             mex[r] = 0.0;
             cex[r] = 0u;
             if (__ballot(c[r] != 0u)) {  // uniform: a stretch without a token needs no arithmetic at all
                 const double fix = static_cast<double>(h[r] & ((1ull << kCountShift) - 1ull)) * kFixInv;
-                // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail bin carries none
-                const double ms = (c[r] && b < kBins - 1) ? s_exp[g] * el * (static_cast<double>(c[r]) - fix) * to_max : 0.0;
+                // mass of the bin relative to the maximum: exp(-b / 64) * sum exp(-w / 64); the tail carries none
+                const double ms = (c[r] && b < static_cast<uint32_t>(kTail)) ? s_exp[g] * el * (static_cast<double>(c[r]) - fix) * to_max : 0.0;
                 minc = wave_incl_scan(ms);
                 cinc = wave_incl_scan(c[r]);
                 // exclusive inside the stretch = the lane below's inclusive value: no subtraction, no rounding of its own
@@ -913,11 +918,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         WS_MARK(26);
         const uint32_t uc = tot_c[lane];
         const double um = tot_m[lane];
-        const uint32_t Pc = wave_incl_scan(uc);  // counts up to and with stretch `lane` = pc[64 lane + 64]
+        uint32_t Pc = wave_incl_scan(uc);  // counts up to and with stretch `lane` = pc[64 lane + 64]
         const double Pm = wave_incl_scan(um);
         const double Pm_up = __shfl_up(Pm, 1);
         const double Em = lane ? Pm_up : 0.0;    // masses before stretch `lane`: exactly the value published as pm64[lane - 1]
         const uint32_t Ec = Pc - uc;
+        // The last stretch is the tail. Its words are not looked at one by one (touched tokens were taken out of words
+        // other than the ones they went into, and the three-pass mode streams them there once too often): every token
+        // of the row is in some bin, so the tail holds what the other stretches do not.
+        if (lane == 63u) Pc = V;
         if (wv == 0u) {  // every 64th prefix once more, side by side, for the searches' first probe
             pc64[lane] = Pc;
             pm64[lane] = Pm;
@@ -989,14 +998,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     double X = 0;  // top-p target in mass units (known here unless top-k closes the set)
     if (prefix_mode) {
         BinSel s1 = bin_sel(find_count(n1));
-        if (s1.b < 0 || s1.b >= kBins - 1) {
-            // top-k reaches into the tail bin (-inf and logits whose mass is below e^-64 of the top token's): those
+        if (s1.b < 0 || s1.b >= kTail) {
+            // top-k reaches into the tail (-inf and logits whose mass is below e^-63 of the anchor's): those
             // candidates stay in the kept count, as in the host filter, but carry no mass; cuts and the draw see the
             // candidates ranked before the tail
-            n1 = pc[kBins - 1];
+            n1 = pc[kTail];
             s1 = bin_sel(find_count(n1));
         }
-        if (s1.b < 0 || s1.b >= kBins - 1 || s1.cx + s1.c > kCap) {
+        if (s1.b < 0 || s1.b >= kTail || s1.cx + s1.c > kCap) {
             flags |= kOverflow;
         } else {
             r0lo = 0;
@@ -1015,13 +1024,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 X = top_p * Z;
                 b2 = find_mass(X, false);
             }
-            if (b2 < 0) b2 = kBins - 1;  // rounding pushed the target past the total: the cut is the whole row
+            if (b2 < 0) b2 = kTail;  // rounding pushed the target past the total: the cut is the whole row
         }
         if (use_min_p) {
             const double astar = (-log(min_p) + lift) * 64.0;  // the floor in bin coordinates (bins count from the anchor)
             const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
-            lo3 = lo < 0 ? 0 : (lo > kBins - 1 ? kBins - 1 : static_cast<int>(lo));
-            hi3 = hi < 0 ? 0 : (hi > kBins - 1 ? kBins - 1 : static_cast<int>(hi));
+            lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
+            hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
         }
         if (use_top_p && (!use_min_p || b2 < lo3)) {
             r1lo = r1hi = b2;
@@ -1047,7 +1056,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         int b4lo = find_mass(u * zlo * (1.0 - 1e-9), true), b4hi = find_mass(u * zhi * (1.0 + 1e-9), true);
         if (b4lo < 0) b4lo = 0;
-        if (b4hi < 0) b4hi = (r1hi >= r1lo) ? r1hi : kBins - 2;
+        if (b4hi < 0) b4hi = (r1hi >= r1lo) ? r1hi : kTail - 1;
         if (b4hi < b4lo) b4hi = b4lo;
         if (r1hi >= r1lo && b4hi >= r1lo - 1) {  // adjacent or overlapping: one range
             r0lo = min(b4lo, r1lo);
@@ -1058,7 +1067,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             r0lo = b4lo;
             r0hi = b4hi;
         }
-        if (r0hi >= kBins - 1 || r1hi >= kBins - 1) flags |= kOverflow;  // the tail bin has no mass resolution
+        if (r0hi >= kTail || r1hi >= kTail) flags |= kOverflow;  // the tail has no mass resolution
     }
 
     // bases of the two ranges
@@ -1661,7 +1670,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (i < V) {
                 x = adjusted_logit(rv, i);
                 keep = key64(x, i) >= kept_key;
-                tl = tail_extra && !keep && bin_of(aq, c64, x) == kBins - 1;  // among zero-mass candidates the lowest ids
+                tl = tail_extra && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail);  // among zero-mass candidates the lowest ids
             }
             uint32_t tot;
             const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
