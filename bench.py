@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0
 MODE = 0
 # HBM bytes per launch of ws::sample_batch_kernel on the tile workload: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
 # what the same counter reads for a 256 MiB device copy (x2.000 and x1.000); the runs are summarised under profiles/
-TRAFFIC_BYTES = {("tile", "auto"): 168.4e6, ("tile", "fused"): 168.4e6, ("tile", "exact"): 524.7e6}
+TRAFFIC_BYTES = {("tile", "auto"): 168.0e6, ("tile", "fused"): 168.0e6, ("tile", "exact"): 524.7e6}
 
 
 def algorithmic_bytes(c):
