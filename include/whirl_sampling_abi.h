@@ -106,7 +106,9 @@ enum { WS_DTYPE_F32 = 0, WS_DTYPE_BF16 = 1 };
  *          float (logits that came from bf16, for instance); otherwise the prefix masses differ by ~1e-7 relative.
  *          Needs 16-byte aligned rows of a multiple of 8 tokens, vocab <= 163840. A row whose maximum beats the bound
  *          is redone the exact way inside the same launch.
- *   AUTO:  FUSED where the batch qualifies, else EXACT. */
+ *   AUTO:  FUSED where the batch qualifies; else two sweeps: maximum and histogram in one, against such a bound (guessed
+ *          from the head of the row and the penalised tokens), then the gather. A row the bound does not fit is done
+ *          the EXACT way inside the same launch. */
 enum { WS_MODE_AUTO = 0, WS_MODE_EXACT = 1, WS_MODE_FUSED = 2 };
 enum { WS_RNG_SPLITMIX = 0, WS_RNG_PHILOX = 1 };
 

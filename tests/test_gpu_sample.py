@@ -96,6 +96,27 @@ def test_rows_masked_by_minus_infinity_in_the_logits(mode):
     print(res)
 
 
+@pytest.mark.parametrize("V", [40000, 40004])  # 40004: not a multiple of 8, so AUTO takes the two-sweep kernel
+@pytest.mark.parametrize("mode", MODES)
+def test_maximum_far_above_the_head_of_the_row(mode, V):
+    """The one-sweep histograms measure bins down from a bound guessed from the first few thousand tokens. Rows whose
+    maximum lies far above that guess (one token at +60 near the end, or everything before it tiny) or far below it (a
+    head of large logits that are all masked out by the history penalty) must fall back to the exact route and still
+    give the oracle's token."""
+    c = gc.make_cfg2(rows=4, V=V, n_hist=64, n_bias=8)
+    c["logits"][0, V - 3] = 60.0
+    c["logits"][1, : V // 2] -= 50.0
+    c["logits"][2, V - 1] = 25.0
+    c["logits"][3, :32] = 30.0
+    c["hist"][3, :32] = np.arange(32)
+    c["rep"][3] = 8.0
+    c["freq"][3] = 2.0
+    c["top_k"][:] = [0, 50, 20, 0]
+    c["top_p"][:] = [0.9, 0.95, 1.0, 0.9]
+    res, _ = run_case(c, 1, mode=mode)
+    print(res)
+
+
 def test_flagged_rows():
     m = gc.pkg()
     c = gc.make_cfg5(rows=3, V=8192, n_hist=50, n_bias=5)
@@ -212,7 +233,7 @@ def test_cfg3_full_size(mode):
 
 def test_cfg5_full_size():
     """configs[4] at its full size: 1024 rows x 262144 fp32 logits (1 GiB), 90 % masked, 8192-id histories, 500 bias entries,
-    top-k 1000 + top-p 0.95. The vocabulary is past what the single-sweep mode caches, so this is the three-pass kernel.
+    top-k 1000 + top-p 0.95. The vocabulary is past what the single-sweep mode caches, so this is the two-sweep route.
     A sample of rows against the oracle, every row for the size-independent facts: a token that is allowed, a kept count
     within top-k, no failure flag."""
     m = gc.pkg()

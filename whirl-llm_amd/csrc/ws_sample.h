@@ -81,6 +81,7 @@ struct BatchArgs {
     uint32_t lds_tie;  // byte offset of spare LDS, 0 when there is no room for it: at least 32 KiB and vocab / 32 words + as
                        // many 16-bit counts. Second copy of the histogram during the single sweep, then the id bitmap +
                        // prefix that sorts heavy ties by id
+    int two_sweep;     // rows the single sweep cannot take: histogram against a provisional bound in the first sweep (else: exact mode)
     uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
 };
 
@@ -825,10 +826,38 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     } else if (!(flags & kBadParam)) {
-        // ---------------------------------------------------------------- pass 1: maximum
         gather_and_adjust(nullptr, 0u);
-        stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
-        m = fmaxf(block_max(m, red_f), m_adj);
+        if (A.two_sweep) {
+            // ------------------------------------------------------------ maximum and histogram in one sweep, against a
+            // bound above the maximum guessed from the adjusted tokens and the head of the row (as the single-sweep
+            // mode does); rows the guess does not fit fall through to the two passes below
+            float s = m_adj;
+            for (uint32_t i = t; i < min(V, 8u * WS_BLOCK); i += WS_BLOCK)
+                if (is_allowed(rv, i) && !is_touched(rv, i)) s = fmaxf(s, raw_logit(rv, i));
+            s = block_max(s, red_f);
+            anchor = s + 8.f / inv_t;
+            if (anchor > -INFINITY && anchor < INFINITY) {  // uniform
+                aq = anchor_product(anchor, c64);
+                for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+                __syncthreads();
+                stream_row(
+                    rv,
+                    [&](uint32_t i, float x, int slot) {
+                        m = fmaxf(m, x);
+                        add_to_hist(i, x, slot);
+                    },
+                    [](uint32_t, uint32_t) {});
+                replay_touched([&](uint32_t i, float x) { add_to_hist(i, x, 0); });
+                m = fmaxf(block_max(m, red_f), m_adj);
+                cached = m <= anchor && (anchor - m) * c64 <= 1024.f;  // here: the histogram stands
+            }
+        }
+        if (!cached) {
+            // ------------------------------------------------------------ pass 1: maximum
+            m = -INFINITY;
+            stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+            m = fmaxf(block_max(m, red_f), m_adj);
+        }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
     if (flags) {  // uniform over the block
