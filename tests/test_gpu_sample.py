@@ -254,3 +254,48 @@ def test_cfg5_shape_reduced_rows(mode):
     c = gc.make_cfg5(rows=32)
     res, _ = run_case(c, 1, rows=range(0, 32, 4), kept_cap=2048, mode=mode)
     print(res)
+
+
+def test_random_shapes_filters_and_masks_both_kernels():
+    """A seeded sweep over vocabulary sizes (fusable or not), batch sizes, history / bias lengths, dtypes, filter
+    settings, temperatures and -inf masking, every case through WS_MODE_EXACT and WS_MODE_AUTO with either RNG: every
+    row must give the oracle's token, kept set and probabilities (or be reported as a boundary case by the oracle)."""
+    rng = np.random.default_rng(20240611)
+    seed0 = gc.DATA_SEED
+    tot = dict(rows=0, exact=0)
+    try:
+        for case in range(16):
+            gc.DATA_SEED = int(rng.integers(1, 1 << 30))
+            kind = rng.choice(["cfg2", "cfg3", "cfg5", "tile"])
+            V = int(rng.choice([1000, 4096, 8008, 32000, 50257, 65536, 100003, 163840, 200000]))
+            rows = int(rng.integers(1, 6))
+            nh = int(rng.choice([0, 1, 17, 300, 2048, 5000]))
+            nb = int(rng.choice([0, 1, 30, 300]))
+            if kind == "cfg2":
+                c = gc.make_cfg2(rows=rows, V=V, n_hist=nh, n_bias=nb)
+            elif kind == "cfg3":
+                c = gc.make_cfg3(rows=rows, V=V, n_hist=nh)
+            elif kind == "cfg5":
+                V = (V + 31) // 32 * 32
+                c = gc.make_cfg5(rows=rows, V=V, n_hist=nh, n_bias=nb)
+            else:
+                c = gc.make_tile(rows=rows, V=V, n_hist=nh)
+            c["top_k"] = rng.choice([0, 1, 5, 40, 1000, 3000], rows).astype(np.uint32)
+            c["top_p"] = rng.choice([1.0, 0.999, 0.95, 0.9, 0.5, 0.1], rows).astype(np.float64)
+            c["min_p"] = rng.choice([0.0, 0.0, 0.01, 0.2], rows).astype(np.float64)
+            c["inv_t"] = (1.0 / rng.uniform(0.3, 2.0, rows)).astype(np.float32)
+            for r in range(rows):  # a row without any filter is the open case the device flags: keep one filter on
+                if c["top_k"][r] == 0 and c["top_p"][r] == 1.0 and c["min_p"][r] == 0.0:
+                    c["top_p"][r] = 0.97
+            if rng.random() < 0.3:
+                for r in range(rows):
+                    off = rng.random(V) < rng.choice([0.5, 0.9, 0.99])
+                    c["logits"][r][off] = 0xFF80 if c["dtype"] == "bf16" else -np.inf
+            for mode in MODES:
+                res, _ = run_case(c, int(rng.integers(0, 2)), kept_cap=min(V, 4096), expect_near=0.5, mode=mode)
+                tot["rows"] += res["rows"]
+                tot["exact"] += res["exact"]
+    finally:
+        gc.DATA_SEED = seed0
+    print(tot)
+    assert tot["exact"] >= 0.9 * tot["rows"], tot
