@@ -1,9 +1,14 @@
 // topk_rows for gfx950: per row the softmax normaliser {max, sum exp((x - max) * inv_t)} and the K largest logits
 // (reference: kernels/shared/sample_cand_topk_rows.h:11-98, same arguments and output layout).
-// Differences by design: the maximum and the normaliser come from one pass (online rescaled sum); the K-th largest
-// key is found by a 12 + 12 + 8 bit radix select with one LDS histogram per pass; the output is written by an
-// ordered compaction, so entries are in ascending token id and, among logits equal to the K-th largest, the lowest
-// ids are kept (the reference leaves both to the order of its atomics). NaN logits count as -inf.
+// Differences by design: the maximum and the normaliser come from one pass (online rescaled sum); the output is in
+// ascending token id and, among logits equal to the K-th largest, the lowest ids are kept (the reference leaves both
+// to the order of its atomics). NaN logits count as -inf.
+// Two routes to the K-th largest (logit, id). The usual one: the first pass also counts the tokens in 4096 bins of
+// a width fitted to the spread of the head of the row, under a bound guessed from it; the bin the K-th largest falls in is read off the scanned
+// counts; a second pass (from cache) lists that bin's few tokens and counts the tokens above it per stretch of the row;
+// the list is ranked; a third pass writes the output in order. The other, for rows that do not fit (unaligned, tiny,
+// heavy ties at the cut, logits more than 120 units apart): a 12 + 12 + 8 bit radix select on the keys and a
+// compaction tile by tile.
 #pragma once
 
 #include "ws_common.h"
@@ -87,29 +92,211 @@ __device__ __forceinline__ void select_in_id_order(const float* __restrict__ x, 
     }
 }
 
-}  // namespace ws
+// ---- the histogram route. All threads return the same answer; false = nothing was written, take the radix route.
+constexpr uint32_t kTopkCap = 2048;     // tokens of the cut's bin resolved in LDS
+constexpr int kTopkBins = 4096;
+constexpr int kTopkTail = kTopkBins - 64;  // the last 64 bins take everything else, one bin per lane (same-word atomics queue)
 
-extern "C" __global__ void __launch_bounds__(WS_BLOCK)
-    topk_rows(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
-    __shared__ uint32_t hist[4096];
-    __shared__ float red_f[WS_WAVES];
-    __shared__ uint32_t red_u[WS_WAVES];
-    __shared__ uint32_t s_sel[2];
-    const int row = blockIdx.x;
-    x += static_cast<size_t>(row) * n;
-    ids += static_cast<size_t>(row) * K;
-    vals += static_cast<size_t>(row) * K;
+struct TopkLds {
+    uint32_t* hist;   // kTopkBins
+    uint64_t* cand;   // kTopkCap
+    float* red_f;     // WS_WAVES
+    uint32_t* red_u;  // WS_WAVES
+    uint32_t* sel;    // 2
+    uint32_t* cnt;    // WS_WAVES: kept tokens per stretch of the row
+    uint32_t* n_cand; // 1
+    uint64_t* kmin;   // 1: the K-th largest (logit, id) as a key
+};
 
-    // pass 1: max and sum exp((x - max) * inv_t), rescaled online per thread
-    float m = -INFINITY, s = 0.f;
-    ws::for_each_f32(x, n, [&](int, float v) {
+// bin = (bound - v) * scale, a32 = bound * scale
+__device__ __forceinline__ uint32_t topk_bin(float v, float scale, float a32, float tail) {
+    return static_cast<uint32_t>(__builtin_fminf(__fmaf_rn(v, -scale, a32), tail));  // NaN -> tail; above the bound -> 0
+}
+
+// Pass 1 of both routes: per-thread online maximum and rescaled sum; with `hist` also the bin counts.
+template <bool COUNT>
+__device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist, float& m,
+                                                float& s) {
+    const float tail = static_cast<float>(kTopkTail + lane_id());
+    for_each_f32(x, n, [&](int, float v) {
         if (v > m) {
             s = s * __expf((m - v) * inv_t) + 1.f;
             m = v;
         } else if (v > -INFINITY) {
             s += __expf((v - m) * inv_t);
         }
+        if (COUNT) atomicAdd(&hist[topk_bin(v, scale, a32, tail)], 1u);
     });
+}
+
+// After the first pass with counts: the rest of the histogram route.
+__device__ __forceinline__ bool topk_by_counts(const float* __restrict__ x, int n, uint32_t kk, float scale, float a32, const TopkLds& L,
+                                               int* ids, float* vals) {
+    const uint32_t t = threadIdx.x, lane = static_cast<uint32_t>(lane_id());
+    const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+    // the bin the kk-th largest falls in: bins ascend as logits fall, 4 consecutive bins per thread
+    uint32_t c[4], tot = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        c[j] = L.hist[4u * t + j];
+        tot += c[j];
+    }
+    uint32_t all;
+    uint32_t above = block_excl_scan(tot, L.red_u, &all);
+    if (t == 0) {
+        L.sel[0] = 0xffffffffu;
+        L.n_cand[0] = 0u;
+    }
+    if (t < WS_WAVES) L.cnt[t] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (above < kk && above + c[j] >= kk) {
+            L.sel[0] = 4u * t + j;
+            L.sel[1] = kk - above;
+        }
+        above += c[j];
+    }
+    __syncthreads();
+    const uint32_t bcut = L.sel[0], need = L.sel[1];
+    if (bcut >= static_cast<uint32_t>(kTopkTail)) return false;  // the cut lies among -inf / NaN / far-off logits
+
+    // second pass: wave w takes the w-th stretch of the row, 64 vectors at a time in id order
+    const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
+    const uint32_t nv = static_cast<uint32_t>(n) >> 2;
+    const uint32_t R = (nv + WS_WAVES - 1u) / WS_WAVES;
+    const uint32_t j_begin = min(wv * R, nv), j_end = min(j_begin + R, nv);
+    const float tail = static_cast<float>(kTopkTail + lane);
+    uint32_t n_above = 0;
+    constexpr uint32_t kU = 4;  // vectors per lane in flight: the loads of a round go out before any is looked at
+    for (uint32_t j0 = j_begin; j0 < j_end; j0 += 64u * kU) {
+        float4 q[kU];
+#pragma unroll
+        for (uint32_t u = 0; u < kU; ++u) q[u] = x4[min(j0 + 64u * u + lane, j_end - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < kU; ++u) {
+            const uint32_t j = j0 + 64u * u + lane;
+            const bool valid = j < j_end;
+            const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t b = valid ? topk_bin(v[e], scale, a32, tail) : 0xffffffffu;  // NaN -> tail, never the cut's bin
+                n_above += b < bcut ? 1u : 0u;  // per lane; summed over the wave after the loop
+                if (b == bcut) {
+                    const uint32_t slot = atomicAdd(L.n_cand, 1u);
+                    if (slot < kTopkCap) L.cand[slot] = key64(v[e], 4u * j + e);
+                }
+            }
+        }
+    }
+    n_above = wave_sum(n_above);
+    if (lane == 0) atomicAdd(&L.cnt[wv], n_above);
+    __syncthreads();
+    const uint32_t n_cand = L.n_cand[0];
+    if (n_cand > kTopkCap) return false;  // heavy ties at the cut
+    // rank the bin's tokens by (logit desc, id asc): the first `need` of them are kept, the last of those is the cut
+    for (uint32_t i = t; i < n_cand; i += WS_BLOCK) {
+        const uint64_t mine = L.cand[i];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < n_cand; j += 4u) {
+            uint64_t o[4];
+#pragma unroll
+            for (uint32_t e = 0; e < 4u; ++e) o[e] = L.cand[min(j + e, n_cand - 1u)];
+#pragma unroll
+            for (uint32_t e = 0; e < 4u; ++e) rank += (j + e < n_cand && o[e] > mine) ? 1u : 0u;
+        }
+        if (rank < need) {
+            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(mine);
+            atomicAdd(&L.cnt[min((id >> 2) / R, static_cast<uint32_t>(WS_WAVES - 1))], 1u);
+            if (rank + 1u == need) L.kmin[0] = mine;
+        }
+    }
+    __syncthreads();
+    // at or above the cut: a larger logit, or the cut's logit (finite: its bin is not in the tail) and an id up to the cut's
+    const uint64_t kmin = L.kmin[0];
+    const float cut_v = unkey32(static_cast<uint32_t>(kmin >> 32));
+    const uint32_t cut_id = 0xffffffffu - static_cast<uint32_t>(kmin);
+    uint32_t run = 0;  // output slots before this wave's stretch
+    for (uint32_t w = 0; w < wv; ++w) run += L.cnt[w];
+    // third pass: every token at or above the cut, in id order
+    for (uint32_t j0 = j_begin; j0 < j_end; j0 += 64u * kU) {
+        float4 q[kU];
+#pragma unroll
+        for (uint32_t u = 0; u < kU; ++u) q[u] = x4[min(j0 + 64u * u + lane, j_end - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < kU; ++u) {
+            const uint32_t j = j0 + 64u * u + lane;
+            const bool valid = j < j_end;
+            const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+            bool keep[4];
+            uint32_t mine = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                keep[e] = valid && (v[e] > cut_v || (v[e] == cut_v && 4u * j + e <= cut_id));  // NaN: neither
+                mine += keep[e] ? 1u : 0u;
+            }
+            if (__ballot(mine != 0u) == 0ull) continue;  // uniform: most stretches of 256 tokens hold none of the K
+            const uint32_t inc = wave_incl_scan(mine);
+            uint32_t o = run + inc - mine;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (keep[e]) {
+                    ids[o] = static_cast<int>(4u * j + e);
+                    vals[o] = v[e];
+                    ++o;
+                }
+            run += last_lane(inc);
+        }
+    }
+    return true;
+}
+
+}  // namespace ws
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    topk_rows(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
+    __shared__ uint32_t hist[4096];
+    __shared__ uint64_t cand[ws::kTopkCap];
+    __shared__ float red_f[WS_WAVES];
+    __shared__ uint32_t red_u[WS_WAVES];
+    __shared__ uint32_t s_sel[2];
+    __shared__ uint32_t s_cnt[WS_WAVES];
+    __shared__ uint32_t s_n;
+    __shared__ uint64_t s_kmin;
+    const int row = blockIdx.x;
+    x += static_cast<size_t>(row) * n;
+    ids += static_cast<size_t>(row) * K;
+    vals += static_cast<size_t>(row) * K;
+    const uint32_t kk = static_cast<uint32_t>(K < n ? K : n);
+
+    // A bound above the maximum (+ 8 units) and the spread of the logits, both from the first 4096 of them: the bins
+    // of the histogram route hang from the bound and are as fine as 3968 of them over bound - smallest allow (fine
+    // bins: few tokens of a wave instruction meet on one counter, and few tokens share the cut's bin).
+    // Rows it cannot take - unaligned, short, a bound that is not finite - count nothing and go the radix way.
+    bool counted = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (n & 3) == 0 && n >= 4 * WS_BLOCK && kk > 0 && kk < static_cast<uint32_t>(n);
+    float scale = 0.f, a32 = 0.f, bound = 0.f;
+    if (counted) {  // uniform
+        const float4 q = reinterpret_cast<const float4*>(x)[threadIdx.x];
+        const float v[4] = {q.x, q.y, q.z, q.w};
+        float hi = -INFINITY, lo = INFINITY;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            hi = fmaxf(hi, v[e]);
+            if (v[e] > -INFINITY) lo = fminf(lo, v[e]);  // finite ones (NaN compares false)
+        }
+        bound = ws::block_max(hi, red_f) + 8.f;
+        const float low = -ws::block_max(-lo, red_f);
+        counted = bound > -INFINITY && bound < INFINITY && low < INFINITY;
+        scale = fminf(static_cast<float>(ws::kTopkTail - 64) / (bound - low), 1048576.f);
+        a32 = bound * scale;
+        for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
+        __syncthreads();
+    }
+
+    // pass 1: max and sum exp((x - max) * inv_t), rescaled online per thread (and the bin counts)
+    float m = -INFINITY, s = 0.f;
+    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, m, s);
+    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, m, s);
     const float top = ws::block_max(m, red_f);
     const float part = m > -INFINITY ? s * __expf((m - top) * inv_t) : 0.f;
     const float sum = ws::block_sum(part, red_f);
@@ -117,8 +304,14 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
         stats[2 * row] = top;
         stats[2 * row + 1] = sum;
     }
-    const uint32_t kk = static_cast<uint32_t>(K < n ? K : n);
     if (kk == 0) return;
+    __syncthreads();  // the counts are complete
+
+    if (counted && top <= bound) {  // uniform
+        const ws::TopkLds L{hist, cand, red_f, red_u, s_sel, s_cnt, &s_n, &s_kmin};
+        if (ws::topk_by_counts(x, n, kk, scale, a32, L, ids, vals)) return;
+        __syncthreads();
+    }
 
     uint32_t thr, need;
     ws::radix_kth(x, n, kk, hist, red_u, s_sel, thr, need);
