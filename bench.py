@@ -2,6 +2,7 @@
 """Benchmark of the token-sampling hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload tile|cfg2|cfg3|cfg5] [--no-cpu] [--no-also]
+    python bench.py --reference-kernels      (greedy picks and topk_rows at the engine's shapes)
 
 A step = one launch of the fused batched sampler (ws_sample_batch) over one batch of synthetic logits that already
 sit in HBM. The default workload is the north-star tile: 256 rows x 151,936 fp32 logits ~ N(0, sigma 2), repetition /
@@ -145,6 +146,48 @@ def run_workload(name, steps, warmup, check_rows):
                    frac_of_hbm_peak=ab / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, parity=par)
 
 
+def reference_kernels(steps):
+    """Launch times of the replacements of the reference's own kernels at the engine's shapes (vocab 151936): the greedy
+    picks on 1 / 32 / 256 rows, topk_rows with the engine's two list sizes on 1 / 32 rows. Synthetic N(0, sigma 2) logits."""
+    import torch
+    import gpu_cases as gc
+    m = gc.pkg()
+    L, S, P = m.lib(), m._stream, m._p
+    V = 151936
+    out = []
+
+    def timed(name, rows, fn, bytes_):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1000
+        out.append(dict(kernel=name, rows=rows, vocab=V, us_per_launch=us, algorithmic_GBs=bytes_ / (us * 1e-6) / 1e9))
+
+    for rows in (1, 32, 256):
+        x = torch.randn(rows, V, device="cuda:0") * 2
+        o = torch.empty(rows, dtype=torch.int32, device="cuda:0")
+        timed("argmax_rows", rows, lambda: L.ws_argmax_rows(S(), P(x), V, P(o), rows), rows * V * 4)
+        if rows > 32:
+            continue
+        ids = torch.empty((rows, 16384), dtype=torch.int32, device="cuda:0")
+        vals = torch.empty((rows, 16384), dtype=torch.float32, device="cuda:0")
+        st = torch.empty((rows, 2), dtype=torch.float32, device="cuda:0")
+        for K in (256, 16384):
+            timed(f"topk_rows K={K}", rows, lambda: L.ws_topk_rows(S(), P(x), V, K, 1.25, P(ids), P(vals), P(st), rows),
+                  rows * (V * 4 + K * 8 + 8))
+    x = torch.randn(1, V, device="cuda:0") * 2
+    tok = torch.empty(1, dtype=torch.int32, device="cuda:0")
+    pr = torch.empty(1, dtype=torch.float32, device="cuda:0")
+    timed("argmax_prob", 1, lambda: L.ws_argmax_prob(S(), P(x), V, P(tok), P(pr)), V * 4)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -155,6 +198,9 @@ def main():
     ap.add_argument("--no-also", action="store_true")
     ap.add_argument("--check-rows", type=int, default=8)
     ap.add_argument("--mode", default="auto", choices=["auto", "exact", "fused"], help="ws_batch.mode for every workload")
+    ap.add_argument("--reference-kernels", action="store_true",
+                    help="time the replacements of the reference's own kernels (greedy picks, topk_rows) instead and print "
+                         "their launch times as one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run 10 device copies of 256 MiB instead (known traffic: 256 MiB read + 256 MiB written per "
                          "copy) to scale rocprofv3's FETCH_SIZE / WRITE_SIZE")
@@ -174,6 +220,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "10 copies", "bytes_read_per_copy": 256 << 20, "bytes_written_per_copy": 256 << 20}))
+        return
+    if a.reference_kernels:
+        print(json.dumps({"reference_kernels": reference_kernels(max(20, a.steps // 4)), "data": "synthetic"}))
         return
     global MODE
     MODE = {"auto": 0, "exact": 1, "fused": 2}[a.mode]
