@@ -114,19 +114,119 @@ __device__ __forceinline__ uint32_t topk_bin(float v, float scale, float a32, fl
 }
 
 // Pass 1 of both routes: per-thread online maximum and rescaled sum; with `hist` also the bin counts.
+// With COUNT every token is also counted in its bin, and tokens of the bins up to `list_bin` (-1: none) are put on the
+// list as keys: when the list ends up holding at least K tokens, the K largest are among them and no further pass over
+// the row is needed.
 template <bool COUNT>
-__device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist, float& m,
-                                                float& s) {
+__device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist,
+                                                int list_bin, uint64_t* list, uint32_t* n_list, float& m, float& s) {
     const float tail = static_cast<float>(kTopkTail + lane_id());
-    for_each_f32(x, n, [&](int, float v) {
+    for_each_f32(x, n, [&](int i, float v) {
         if (v > m) {
             s = s * __expf((m - v) * inv_t) + 1.f;
             m = v;
         } else if (v > -INFINITY) {
             s += __expf((v - m) * inv_t);
         }
-        if (COUNT) atomicAdd(&hist[topk_bin(v, scale, a32, tail)], 1u);
+        if (COUNT) {
+            const uint32_t b = topk_bin(v, scale, a32, tail);
+            atomicAdd(&hist[b], 1u);
+            if (static_cast<int>(b) <= list_bin) {  // a few per thousand tokens
+                const uint32_t slot = atomicAdd(n_list, 1u);
+                if (slot < kTopkCap) list[slot] = key64(v, static_cast<uint32_t>(i));
+            }
+        }
     });
+}
+
+// The list holds every token of the row up to bin `list_bin`, the counts say in which bin the kk-th largest lies. When
+// that bin is on the list, the tokens of the bins before it are kept as they are, the cut bin's few tokens are ranked
+// among themselves, and the kk kept ones are sorted by id (bitonic, in LDS) and written out. `work`: LDS, 4096 words
+// (the counts, read first and then overwritten). Returns 0 when done; otherwise nothing was written: 1 = the list does
+// not reach the cut (the counts are still there), 2 = too many tokens tie at the cut (the counts are gone).
+__device__ __forceinline__ int topk_from_list(const float* __restrict__ x, const uint64_t* list, uint32_t n_list, int list_bin, uint32_t kk,
+                                               float scale, float a32, uint32_t* work, uint32_t* red, uint32_t* sel, int* ids,
+                                               float* vals) {
+    const uint32_t t = threadIdx.x;
+    // the bin of the kk-th largest, as in the count route
+    uint32_t c[4], tot = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        c[j] = work[4u * t + j];
+        tot += c[j];
+    }
+    uint32_t all;
+    uint32_t above = block_excl_scan(tot, red, &all);
+    if (t == 0) {
+        sel[0] = 0xffffffffu;
+        sel[2] = 0u;  // kept so far
+        sel[3] = 0u;  // tokens of the cut bin found on the list
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (above < kk && above + c[j] >= kk) {
+            sel[0] = 4u * t + j;
+            sel[1] = kk - above;
+        }
+        above += c[j];
+    }
+    __syncthreads();  // also: every read of the counts is done, `work` is free
+    const uint32_t bcut = sel[0], need = sel[1];
+    if (bcut > static_cast<uint32_t>(list_bin)) return 1;
+    uint64_t* kept = reinterpret_cast<uint64_t*>(work);          // up to 1024 entries: id << 32 | slot in the list
+    uint64_t* cut = reinterpret_cast<uint64_t*>(work) + 1024;    // up to 1024 keys of the cut bin
+    constexpr uint32_t kCutCap = 1024;
+    const float no_tail = 4095.f;  // listed tokens lie before the tail: any clamp at or past it gives their bin
+    for (uint32_t i = t; i < n_list; i += WS_BLOCK) {
+        const uint64_t k = list[i];
+        const uint32_t b = topk_bin(unkey32(static_cast<uint32_t>(k >> 32)), scale, a32, no_tail);
+        if (b < bcut) {
+            const uint32_t o = atomicAdd(&sel[2], 1u);
+            kept[o] = (static_cast<uint64_t>(0xffffffffu - static_cast<uint32_t>(k)) << 32) | i;
+        } else if (b == bcut) {
+            const uint32_t o = atomicAdd(&sel[3], 1u);
+            if (o < kCutCap) cut[o] = k;
+        }
+    }
+    __syncthreads();
+    const uint32_t n_cut = sel[3];
+    if (n_cut > kCutCap) return 2;  // heavy ties at the cut
+    for (uint32_t i = t; i < n_cut; i += WS_BLOCK) {
+        const uint64_t mine = cut[i];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < n_cut; ++j) rank += cut[j] > mine ? 1u : 0u;
+        if (rank < need) {
+            const uint32_t o = atomicAdd(&sel[2], 1u);
+            kept[o] = static_cast<uint64_t>(0xffffffffu - static_cast<uint32_t>(mine)) << 32;
+        }
+    }
+    __syncthreads();  // sel[2] == kk now
+    // ascending id: bitonic sort of the kept entries, padded with the largest key to a power of two
+    uint32_t P = 2;
+    while (P < kk) P <<= 1;
+    for (uint32_t i = kk + t; i < P; i += WS_BLOCK) kept[i] = ~0ull;
+    __syncthreads();
+    for (uint32_t k2 = 2; k2 <= P; k2 <<= 1) {
+        for (uint32_t j = k2 >> 1; j > 0; j >>= 1) {
+            for (uint32_t q = t; q < (P >> 1); q += WS_BLOCK) {
+                const uint32_t i = ((q & ~(j - 1u)) << 1) | (q & (j - 1u)), l = i | j;
+                const uint64_t u = kept[i], w = kept[l];
+                const bool up = (i & k2) == 0;  // this pair sorts ascending
+                if (up ? (u > w) : (u < w)) {
+                    kept[i] = w;
+                    kept[l] = u;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for (uint32_t i = t; i < kk; i += WS_BLOCK) {
+        const uint32_t id = static_cast<uint32_t>(kept[i] >> 32);
+        ids[i] = static_cast<int>(id);
+        vals[i] = x[id];  // the logit as it stands in the row (a key does not tell -0 from +0); never NaN here
+    }
+    return 0;
 }
 
 // After the first pass with counts: the rest of the histogram route.
@@ -275,6 +375,7 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     // Rows it cannot take - unaligned, short, a bound that is not finite - count nothing and go the radix way.
     bool counted = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (n & 3) == 0 && n >= 4 * WS_BLOCK && kk > 0 && kk < static_cast<uint32_t>(n);
     float scale = 0.f, a32 = 0.f, bound = 0.f;
+    int list_bin = -1;
     if (counted) {  // uniform
         const float4 q = reinterpret_cast<const float4*>(x)[threadIdx.x];
         const float v[4] = {q.x, q.y, q.z, q.w};
@@ -290,13 +391,43 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
         scale = fminf(static_cast<float>(ws::kTopkTail - 64) / (bound - low), 1048576.f);
         a32 = bound * scale;
         for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
+        if (threadIdx.x == 0) s_n = 0u;
         __syncthreads();
+        // For a short list (K up to a quarter of the list's room) the head of the row also says where the K-th largest
+        // will roughly be: the bin that holds the sample's (2 K / n)-quantile, and a few tokens more. The first pass
+        // lists every token up to that bin.
+        if (counted && kk <= ws::kTopkCap / 4u) {  // uniform
+            const float tail = static_cast<float>(ws::kTopkTail + ws::lane_id());
+#pragma unroll
+            for (int e = 0; e < 4; ++e) atomicAdd(&hist[ws::topk_bin(v[e], scale, a32, tail)], 1u);
+            __syncthreads();
+            const uint32_t want = min(4u * WS_BLOCK, static_cast<uint32_t>((2ull * kk * 4u * WS_BLOCK) / static_cast<uint32_t>(n)) + 8u);
+            uint32_t c[4], tot = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                c[j] = hist[4u * threadIdx.x + j];
+                tot += c[j];
+            }
+            uint32_t all;
+            uint32_t above = ws::block_excl_scan(tot, red_u, &all);
+            if (threadIdx.x == 0) s_sel[0] = 0xffffffffu;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (above < want && above + c[j] >= want) s_sel[0] = 4u * threadIdx.x + j;
+                above += c[j];
+            }
+            __syncthreads();
+            if (s_sel[0] < static_cast<uint32_t>(ws::kTopkTail)) list_bin = static_cast<int>(s_sel[0]);
+            for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
+            __syncthreads();
+        }
     }
 
-    // pass 1: max and sum exp((x - max) * inv_t), rescaled online per thread (and the bin counts)
+    // pass 1: max and sum exp((x - max) * inv_t), rescaled online per thread (and the bin counts, and the list)
     float m = -INFINITY, s = 0.f;
-    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, m, s);
-    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, m, s);
+    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, list_bin, cand, &s_n, m, s);
+    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, &s_n, m, s);
     const float top = ws::block_max(m, red_f);
     const float part = m > -INFINITY ? s * __expf((m - top) * inv_t) : 0.f;
     const float sum = ws::block_sum(part, red_f);
@@ -307,7 +438,15 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     if (kk == 0) return;
     __syncthreads();  // the counts are complete
 
-    if (counted && top <= bound) {  // uniform
+    int counts_left = counted && top <= bound;  // uniform
+    if (counts_left && list_bin >= 0 && s_n >= kk && s_n <= ws::kTopkCap) {  // the K largest may all be on the list
+        __shared__ uint32_t s_list[4];
+        const int rc = ws::topk_from_list(x, cand, s_n, list_bin, kk, scale, a32, hist, red_u, s_list, ids, vals);
+        if (rc == 0) return;
+        __syncthreads();
+        counts_left = rc == 1;
+    }
+    if (counts_left) {
         const ws::TopkLds L{hist, cand, red_f, red_u, s_sel, s_cnt, &s_n, &s_kmin};
         if (ws::topk_by_counts(x, n, kk, scale, a32, L, ids, vals)) return;
         __syncthreads();
