@@ -120,7 +120,9 @@ enum {
     WS_FLAG_ALL_MASKED = 1u << 3,  /* every logit of the row is -inf / NaN: token = -1 */
     WS_FLAG_OVERFLOW = 1u << 4,    /* more tied / clustered candidates at a cut than the kernel resolves: token = -1 */
     WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
-    WS_FLAG_OPEN = 1u << 6         /* no filter active: drawn in the reference's open-row order */
+    WS_FLAG_OPEN = 1u << 6         /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
+                                      the 256 top candidates in sorted order, then from the other tokens in id order
+                                      (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
 };
 
 /* One batch of rows. Everything per row is a device array of `rows` entries (SoA); a NULL array means the stated
@@ -214,8 +216,8 @@ int ws_adjust_rows(void* stream, const ws_adjust* a);
  *   acc = number of leading positions j < nd whose token equals draft j; chosen = token of position acc;
  *   c[WS_CTL_ROWS + j] = token of position j for j <= acc (the words the greedy path fills with row argmaxes,
  *   src/model/qwen35/forward/mtp_verify.cpp:226); n_accepted[s] = acc; chosen[s].
- *   status[s] = WS_ACCEPT_HOST when a position up to the stop has no usable token (token < 0, or WS_FLAG_OPEN: such a
- *   row is drawn in another order than the reference's): the host then runs Acceptor::sample for that sequence. */
+ *   status[s] = WS_ACCEPT_HOST when a position up to the stop has no usable token (token < 0): the host then runs
+ *   Acceptor::sample for that sequence. */
 enum { WS_ACCEPT_OK = 0, WS_ACCEPT_HOST = 1 };
 typedef struct ws_accept {
     const int32_t* token;  /* device [rows]: ws_batch.token of the launch that sampled the verify rows */

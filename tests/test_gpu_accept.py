@@ -28,7 +28,7 @@ def _oracle_accept(lib, x, prm, dr, nd, n_gen):
     return acc.value, chosen.value
 
 
-def _sequences(n_seq, seed):
+def _sequences(n_seq, seed, open_rows=False):
     rng = np.random.default_rng(seed)
     lib = wo.load("oracle")
     seqs = []
@@ -39,6 +39,8 @@ def _sequences(n_seq, seed):
             x[r, rng.integers(0, V, size=3)] += np.float32(9.0)
         prm = dict(temp=float(rng.uniform(0.6, 1.1)), top_k=int(rng.choice([20, 40, 50])), top_p=float(rng.uniform(0.85, 0.99)),
                    min_p=float(rng.choice([0.0, 0.02])), seed=int(rng.integers(0, 2**62)))
+        if open_rows:  # no filter at all: Sampler::closed stays false
+            prm.update(top_k=0, top_p=1.0, min_p=0.0)
         n_gen = int(rng.integers(0, 5000))
         dr = rng.integers(0, V, size=16).astype(np.uint32)
         for r in range(nd):  # draft r = what the oracle samples at position r given the drafts before it, most of the time
@@ -98,6 +100,22 @@ def test_accept_sampled_matches_the_oracle_acceptor():
         assert list(ctl[s, 16:31]) == list(q["dr"][:15].view(np.int32)) and ctl[s, 48] == q["nd"], s
     assert near <= 2 and exact >= len(seqs) - 2, (exact, near)
     assert accepted >= len(seqs), accepted  # the case does exercise chains of accepted drafts
+
+
+def test_accept_sampled_on_open_rows():
+    """Sequences that sample without any filter: every verify row is an open row, drawn on the device in the
+    reference's order (top candidates, then the rest of the vocabulary by id), so no sequence goes back to the host."""
+    seqs = _sequences(16, 31337, open_rows=True)
+    n_acc, chosen, status, ctl, token, flags, row0 = _device_accept(seqs)
+    assert all(flags & 64)  # WS_FLAG_OPEN
+    exact = 0
+    for s, q in enumerate(seqs):
+        assert status[s] == 0, s
+        if n_acc[s] == q["acc"] and chosen[s] == q["chosen"]:
+            exact += 1
+        else:
+            assert any(flags[row0[s] + j] & NEAR for j in range(min(int(n_acc[s]), q["acc"]) + 1)), (s, n_acc[s], q["acc"])
+    assert exact >= len(seqs) - 2, exact
 
 
 def test_accept_sampled_hands_a_failed_row_to_the_host():

@@ -63,6 +63,46 @@ def test_top_k_only_and_min_p_only_and_top_p_only(mode):
     print(res)
 
 
+def _open(c):
+    c["top_k"][:] = 0
+    c["top_p"][:] = 1.0
+    c["min_p"][:] = 0.0
+    return c
+
+
+@pytest.mark.parametrize("rng_mode", [0, 1])
+@pytest.mark.parametrize("mode", MODES)
+def test_open_rows_are_drawn_in_the_reference_order(rng_mode, mode):
+    """No filter at all: the 256 top candidates in sorted order, then the other tokens in id order
+    (src/sampling/sampler.cpp:118-146), with penalties and bias in force. Temperatures from 0.3 (nearly every draw
+    inside the list) to 2 (nearly every draw in the walk over the rest of the row)."""
+    c = _open(gc.make_cfg2(rows=48, V=32000, n_hist=512, n_bias=40))
+    c["inv_t"] = (1.0 / np.linspace(0.3, 2.0, 48)).astype(np.float32)
+    res, smp = run_case(c, rng_mode, kept_cap=512, mode=mode)
+    fl = smp.flags.cpu().numpy()
+    assert all(fl & gc.pkg().FLAG_OPEN)
+    in_list = sum(gc.oracle_row(c, r, rng_mode)[0].full_used == 0 for r in range(48))
+    assert 5 <= in_list <= 43, in_list  # the case has draws of both kinds
+    print(res, in_list)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_open_rows_odd_shapes(mode):
+    """Open rows of a vocabulary shorter than the candidate list, of an odd length, in bf16, and masked down to fewer
+    allowed tokens than the list holds."""
+    for c in (_open(gc.make_cfg2(rows=8, V=200, n_hist=10, n_bias=4)), _open(gc.make_cfg2(rows=8, V=5003, n_hist=300, n_bias=24)),
+              _open(gc.make_cfg3(rows=8, V=40000, n_hist=256)), _open(gc.make_cfg5(rows=8, V=32768, n_hist=400, n_bias=30))):
+        res, _ = run_case(c, 1, kept_cap=512, expect_near=0.2, mode=mode)
+        print(c["name"], res)
+    c = _open(gc.make_tile(rows=6, V=8192, n_hist=64))
+    for r in range(6):
+        off = np.ones(8192, bool)
+        off[np.random.default_rng(r).choice(8192, 100 + 40 * r, replace=False)] = False
+        c["logits"][r][off] = -np.inf
+    res, _ = run_case(c, 1, kept_cap=512, expect_near=0.2, mode=mode)
+    print(res)
+
+
 @pytest.mark.parametrize("mode", MODES)
 def test_bf16_rows(mode):
     c = gc.make_cfg3(rows=6, V=40000, n_hist=256)
@@ -284,9 +324,6 @@ def test_random_shapes_filters_and_masks_both_kernels():
             c["top_p"] = rng.choice([1.0, 0.999, 0.95, 0.9, 0.5, 0.1], rows).astype(np.float64)
             c["min_p"] = rng.choice([0.0, 0.0, 0.01, 0.2], rows).astype(np.float64)
             c["inv_t"] = (1.0 / rng.uniform(0.3, 2.0, rows)).astype(np.float32)
-            for r in range(rows):  # a row without any filter is the open case the device flags: keep one filter on
-                if c["top_k"][r] == 0 and c["top_p"][r] == 1.0 and c["min_p"][r] == 0.0:
-                    c["top_p"][r] = 0.97
             if rng.random() < 0.3:
                 for r in range(rows):
                     off = rng.random(V) < rng.choice([0.5, 0.9, 0.99])

@@ -279,7 +279,7 @@ int ws_accept_sampled(void* stream, const ws_accept* b) {
     a.ctl_all = b->ctl_all;
     a.area = b->area;
     a.n_seq = b->n_seq;
-    a.host_mask = WS_FLAG_ALL_MASKED | WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_OPEN;
+    a.host_mask = WS_FLAG_ALL_MASKED | WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM;
     a.n_accepted = b->n_accepted;
     a.chosen = b->chosen;
     a.status = b->status;

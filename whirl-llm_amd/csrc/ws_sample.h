@@ -42,6 +42,7 @@ constexpr double kFixInv = 1.0 / 1073741824.0;
 constexpr float kG0 = 16776924.0f, kG1 = -130126.3125f;
 
 // flag bits (WS_FLAG_* of the C ABI)
+constexpr uint32_t kOpenList = 256u;  // candidates of the engine's short list (k_small, src/server/engine_sampling.h:20)
 constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u;
 
 struct BatchArgs {
@@ -125,21 +126,21 @@ __device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
 // before any is used, and the next batch is requested before this one is consumed. Tokens that are masked out or that
 // the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bins or ignores it, so the
 // hot loop has no branch; the touched ones are fed afterwards, by rank, with their adjusted values.
-template <bool MASKED, class F, class E>
+template <bool MASKED, int KB, class F, class E>
 __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch) {
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
     const uint32_t per = rv.dtype == 0 ? 4u : 8u;  // elements per 128-bit load
     const uint32_t nv = rv.vec ? V >> (rv.dtype == 0 ? 2 : 3) : 0u;  // per is 4 or 8: shifts, never a division
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
-    constexpr uint32_t kStep = kBatch * WS_BLOCK;
+    constexpr uint32_t kStep = KB * WS_BLOCK;
     struct Batch {
-        uint4 q[kBatch];
-        uint32_t na[kBatch];  // complement of the allow words
+        uint4 q[KB];
+        uint32_t na[KB];  // complement of the allow words
     };
     auto load = [&](uint32_t j0, Batch& b) {
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < KB; ++u) {
             const uint32_t j = j0 + u * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;
             b.q[u] = xv[jc];
@@ -152,7 +153,7 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
         const bool more = j0 + kStep < nv;
         if (more) load(j0 + kStep, nxt);  // the next batch is in flight while this one is consumed
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
+        for (int u = 0; u < KB; ++u) {
             const uint32_t j = j0 + u * WS_BLOCK + t;
             if (j >= nv) continue;
             const uint32_t i = j * per;
@@ -187,8 +188,15 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
 
 template <class F, class E>
 __device__ __forceinline__ void stream_row(const RowView& rv, F&& f, E&& end_batch) {
-    if (rv.allow || rv.touched) stream_row_impl<true>(rv, f, end_batch);
-    else stream_row_impl<false>(rv, f, end_batch);
+    if (rv.allow || rv.touched) stream_row_impl<true, kBatch>(rv, f, end_batch);
+    else stream_row_impl<false, kBatch>(rv, f, end_batch);
+}
+// the same with twice the loads in flight, for passes that run when the bin cache no longer holds the registers
+constexpr int kWide = 2 * kBatch;
+template <class F, class E>
+__device__ __forceinline__ void stream_row_wide(const RowView& rv, F&& f, E&& end_batch) {
+    if (rv.allow || rv.touched) stream_row_impl<true, kWide>(rv, f, end_batch);
+    else stream_row_impl<false, kWide>(rv, f, end_batch);
 }
 
 // ---- bins. A token's bin coordinate is t = fma(x, -c64, aq): c64 = 64 * inv_t and aq = anchor * c64 rounded a little
@@ -1016,16 +1024,23 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
 
     uint32_t n1 = (top_k > 0 && top_k < V) ? top_k : V;
-    const uint32_t n1_asked = n1;
     const bool use_top_p = top_p < 1.0, use_min_p = min_p > 0.0;
     const bool prefix_mode = n1 < V;
-    if (!use_top_p && !use_min_p && !prefix_mode) flags |= kOpen;
+    // No filter at all: an open row. The reference draws it from the engine's short candidate list in sorted order
+    // first (k_small, src/server/engine_sampling.h:20), probabilities over the float normaliser, and past that list
+    // from the rest of the vocabulary in id order (src/sampling/sampler.cpp:118-146). The list is gathered like a top-k.
+    const bool open_row = !use_top_p && !use_min_p && !prefix_mode;
+    if (open_row) {
+        flags |= kOpen;
+        n1 = min(kOpenList, V);
+    }
+    const uint32_t n1_asked = n1;
 
     // ranges of bins to gather: r0 (ranked first) and r1
     int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
     bool minp_in_list = false, topp_in_list = false;
     double X = 0;  // top-p target in mass units (known here unless top-k closes the set)
-    if (prefix_mode) {
+    if (prefix_mode || open_row) {
         BinSel s1 = bin_sel(find_count(n1));
         if (s1.b < 0 || s1.b >= kTail) {
             // top-k reaches into the tail (-inf and logits whose mass is below e^-63 of the anchor's): those
@@ -1629,6 +1644,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 
     // ------------------------------------------------------------------ draw
     const double u = batch_uniform(A.rng, seed, row, step, 0);
+    if (open_row) Zk = Zf;  // an open row is not renormalised: p = mass / Sampler::sum
     const double target = u * Zk;
     int32_t token = -1;
     double ptok = 0;
@@ -1643,6 +1659,165 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(keys[i]));
                 ptok = mass_of(i) / Zk;
                 mg_draw = fmin(in - target, p > 0 ? target - ex : 1e300) / Zk;
+            }
+        }
+        if (!found && open_row) {
+            // Past the listed candidates: the sum goes on over the tokens outside the list, in id order
+            // (src/sampling/sampler.cpp:132-146). One more sweep over the row leaves the mass of every chunk of
+            // consecutive tokens (the 64 vectors one wave loads with one instruction: 256 fp32 or 512 bf16 tokens) in
+            // LDS; every wave then finds the chunk in which the sum passes the target and scans that chunk. Masses
+            // here come from the 32-bit exponential unit (1.2e-7 relative), so the running sum is good to ~1e-7 of
+            // the row's mass: inside the smallest `tol`.
+            const uint32_t lane = static_cast<uint32_t>(lane_id());
+            const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+            const uint64_t list_key = kept_key;
+            const double rest = target - inc_of(i_last);
+            // mass of a token outside the list: 2^((x - m) * inv_t * log2 e) with the product carried in two floats (the
+            // exponent to ~1e-7 absolute), 0 for listed tokens, for -inf and for NaN (masked, or touched in the sweep)
+            const double k2 = static_cast<double>(inv_t) * 1.4426950408889634;
+            const float kh = static_cast<float>(k2), kl = static_cast<float>(k2 - static_cast<double>(kh));
+            const float cut_x = unkey32(static_cast<uint32_t>(list_key >> 32));
+            const uint32_t cut_id = 0xffffffffu - static_cast<uint32_t>(list_key);
+            auto mass = [&](uint32_t i, float x) -> float {
+                const float d = __fsub_rn(x, m);
+                const float yh = __fmul_rn(d, kh);
+                const float yl = __fmaf_rn(d, kl, __fmaf_rn(d, kh, -yh));
+                const float n = rintf(yh);
+                const float e = ldexpf(__builtin_amdgcn_exp2f(__fadd_rn(__fsub_rn(yh, n), yl)), static_cast<int>(n));
+                const bool out = (yh > -140.f) & !(x > cut_x) & (!(x == cut_x) | (i > cut_id));  // no branches: bitwise
+                return out ? e : 0.f;
+            };
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u, shift = rv.dtype == 0 ? 8u : 9u;
+            const uint32_t n_vec = rv.vec ? V / per : 0u;  // tokens below n_vec * per arrive in 128-bit vectors
+            const uint32_t n_chunks = (V >> shift) + 1u;
+            double* chunk = reinterpret_cast<double*>(keys);
+            WS_MARK(27);
+            __syncthreads();  // every wave has taken what it needs from keys[] and ps[]
+            for (uint32_t c = t; c < n_chunks; c += WS_BLOCK) chunk[c] = 0.0;
+            __syncthreads();
+            if (n_vec) {
+                float acc[2 * kWide] = {};  // per group of four tokens of a load (a bf16 vector has two), slot >> 2
+                stream_row_wide(
+                    rv,
+                    [&](uint32_t i, float x, int slot) {
+                        acc[slot >> 2] += mass(i, x);  // tokens after the last whole vector land here too and are never written out
+                    },
+                    [&](uint32_t j0, uint32_t) {
+                        if (j0 == 0xffffffffu) return;  // the tokens after the last whole vector follow below
+#pragma unroll
+                        for (int u = 0; u < kWide; ++u) {
+                            const uint32_t v0 = j0 + u * WS_BLOCK + wv * 64u;  // first vector of this wave's load
+                            const float own = per == 4u ? acc[u] : __fadd_rn(acc[2 * u], acc[2 * u + 1]);
+                            const double tot = wave_sum(static_cast<double>(own));
+                            if (lane == 0 && v0 < n_vec) chunk[v0 >> 6] = tot;
+                        }
+#pragma unroll
+                        for (int k = 0; k < 2 * kWide; ++k) acc[k] = 0.f;
+                    });
+            }
+            __syncthreads();
+            WS_MARK(28);
+            // touched tokens were skipped by the sweep: their adjusted logits, by rank
+            if (n_touched) {
+                const uint32_t span = (nW + WS_BLOCK - 1) / WS_BLOCK;
+                const uint32_t w0 = t * span, w1 = min(w0 + span, nW);
+                for (uint32_t w = w0; w < w1; ++w) {
+                    uint32_t bits = touched[w];
+                    uint32_t r = wprefix[w];
+                    while (bits) {
+                        const uint32_t i = (w << 5) + (__ffs(bits) - 1u);
+                        bits &= bits - 1u;
+                        const float e = i < n_vec * per ? mass(i, pv[r]) : 0.f;
+                        ++r;
+                        if (e != 0.f) unsafeAtomicAdd(&chunk[i >> shift], static_cast<double>(e));
+                    }
+                }
+            }
+            // tokens after the last whole vector (a row that is not aligned has only such tokens): 64 per wave and round
+            for (uint32_t i0 = n_vec * per + wv * 64u; i0 < V; i0 += WS_BLOCK) {
+                const uint32_t i = i0 + lane;
+                const double tot = wave_sum(i < V ? static_cast<double>(mass(i, adjusted_logit(rv, i))) : 0.0);
+                if (lane == 0 && tot != 0.0) unsafeAtomicAdd(&chunk[i0 >> shift], tot);
+            }
+            __syncthreads();
+            WS_MARK(29);
+            // chunk in which the sum passes `rest`: lane l adds up chunks [l g, (l + 1) g), a scan over the lanes, then a
+            // walk through the group of the first lane that is past it
+            const uint32_t g = (n_chunks + 63u) >> 6;
+            double mine = 0;
+            for (uint32_t c = lane * g; c < min(n_chunks, (lane + 1u) * g); ++c) mine += chunk[c];
+            const double upto = wave_incl_scan(mine);
+            const uint64_t past = __ballot(upto > rest);
+            double before = 0;
+            uint32_t cx = n_chunks;
+            if (past) {
+                const int src = __ffsll(static_cast<unsigned long long>(past)) - 1;
+                before = __shfl(upto - mine, src);
+                for (uint32_t c = src * g; c < min(n_chunks, (src + 1u) * g); ++c) {
+                    const double tc = chunk[c];
+                    if (before + tc > rest) {
+                        cx = c;
+                        break;
+                    }
+                    before += tc;
+                }
+            }
+            if (cx < n_chunks) {
+                // every wave scans the chunk: lane l owns its l-th vector, or 4 (8) tokens of a row without vectors
+                const uint32_t lo = cx << shift;
+                float e[8], half[2] = {0.f, 0.f};  // summed as the sweep sums them: by groups of four
+#pragma unroll
+                for (uint32_t q = 0; q < 8u; ++q) {
+                    const uint32_t i = lo + per * lane + q;
+                    e[q] = (q < per && i < V) ? mass(i, adjusted_logit(rv, i)) : 0.f;
+                    half[q >> 2] += e[q];
+                }
+                const double own = static_cast<double>(__fadd_rn(half[0], half[1]));
+                const double incl = before + wave_incl_scan(own);
+                uint64_t over = __ballot(incl > rest);
+                const uint64_t any = __ballot(own > 0.0);
+                bool seam = false;
+                if (!over && any) {  // the chunk's total was added up in another order: its last token with a mass
+                    over = 1ull << (63 - __builtin_clzll(any));
+                    seam = true;
+                }
+                if (over) {
+                    const int src = __ffsll(static_cast<unsigned long long>(over)) - 1;
+                    double c = incl - own, in = 0, ex = 0, pe = 0;
+                    int32_t tk = -1;
+#pragma unroll
+                    for (uint32_t q = 0; q < 8u; ++q) {
+                        if (e[q] > 0.f && (seam || (tk < 0 && c + e[q] > rest))) {
+                            tk = static_cast<int32_t>(lo + per * lane + q);
+                            ex = c;
+                            in = c + e[q];
+                            pe = e[q];
+                        }
+                        c += e[q];
+                    }
+                    token = __shfl(tk, src);
+                    in = __shfl(in, src);
+                    ex = __shfl(ex, src);
+                    ptok = __shfl(pe, src) / Zk;
+                    mg_draw = seam ? 0.0 : fmin(in - rest, rest - ex) / Zk;
+                    found = token >= 0;
+                }
+            }
+            WS_MARK(30);
+            if (!found) {
+                // the walk ends without passing the target (the float normaliser lies above the exact sum): the
+                // reference returns the last token it walked, the highest id outside the list
+                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(list_key));  // every token is listed: the last of the list
+                for (uint32_t j = V; j-- > 0u;) {
+                    const float x = adjusted_logit(rv, j);
+                    if (!(key64(x, j) >= list_key)) {
+                        token = static_cast<int32_t>(j);
+                        break;
+                    }
+                }
+                ptok = 0;
+                mg_draw = 0.0;
+                found = true;
             }
         }
         if (!found) {
