@@ -116,7 +116,8 @@ enum { WS_RNG_SPLITMIX = 0, WS_RNG_PHILOX = 1 };
 enum {
     WS_FLAG_NEAR_TOP_P = 1u << 0,  /* the top-p cut was within `tol` (relative) of moving by one candidate */
     WS_FLAG_NEAR_MIN_P = 1u << 1,  /* a candidate's probability was within `tol` (relative) of the min-p floor */
-    WS_FLAG_NEAR_DRAW = 1u << 2,   /* the uniform was within `tol` (probability units) of a CDF step */
+    WS_FLAG_NEAR_DRAW = 1u << 2,   /* the uniform was within `tol` (probability units) of a CDF step; race draw: the two smallest
+                                      keys are within `tol` (relative) of each other */
     WS_FLAG_ALL_MASKED = 1u << 3,  /* every logit of the row is -inf / NaN: token = -1 */
     WS_FLAG_OVERFLOW = 1u << 4,    /* more tied / clustered candidates at a cut than the kernel resolves: token = -1 */
     WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
@@ -175,6 +176,10 @@ typedef struct ws_batch {
     uint64_t workspace_bytes;
     double tol;             /* flag tolerance, relative; values below 1e-6 (and 0) mean 1e-6, the accuracy of the mass estimates */
     int32_t mode;           /* WS_MODE_* */
+    const int32_t* race;    /* per row, non-zero: the exponential-race draw of the "specsample" rule (Sampler::race,
+                               src/sampling/sampler.cpp:80-106: argmin of E(token) / p(token) over the kept set, E keyed by
+                               (seed, step, token); an open row races over its 256 candidates when the uniform falls on
+                               their mass, else walks the rest of the row) instead of the inverse CDF (NULL: none) */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

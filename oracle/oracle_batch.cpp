@@ -161,7 +161,34 @@ void wo_sample_batch_row(float* x, uint32_t V, const uint32_t* allow, const int3
     double ptok = 0;
     uint32_t last = c[0].id;
     double plast = c[0].p;
-    for (size_t i = 0; i < s.n; ++i) {
+    bool race = prm->race != 0;
+    double open_margin = 1.0;
+    if (race && !s.closed) {  // sampler.cpp:84-93: an open row races only when the uniform falls on the candidates' mass
+        double mass = 0;
+        for (size_t i = 0; i < s.n; ++i) mass += c[i].p;
+        open_margin = std::fabs(u - mass);
+        if (!(u < mass)) race = false;  // the inverse-CDF walk below with the same u falls past the candidates
+    }
+    if (race) {  // sampler.cpp:94-105
+        const uint64_t base = wo_race_base(prm->seed, prm->step);
+        double best = std::numeric_limits<double>::infinity(), second = best;
+        tok = static_cast<int32_t>(c[0].id);
+        ptok = c[0].p;
+        for (size_t i = 0; i < s.n; ++i) {
+            if (!(c[i].p > 0)) continue;
+            const double key = wo_race_e(base, c[i].id) / c[i].p;
+            if (key < best) {
+                second = best;
+                best = key;
+                tok = static_cast<int32_t>(c[i].id);
+                ptok = c[i].p;
+            } else if (key < second) {
+                second = key;
+            }
+        }
+        margin = std::isinf(second) ? 1.0 : (second - best) / best;
+    }
+    for (size_t i = 0; tok < 0 && i < s.n; ++i) {
         const double before = cum;
         cum += c[i].p;
         last = c[i].id;
@@ -203,6 +230,7 @@ void wo_sample_batch_row(float* x, uint32_t V, const uint32_t* allow, const int3
             }
         }
     }
+    if (prm->race) margin = std::min(margin, open_margin);
     out->token = tok;
     out->prob = static_cast<float>(ptok);
     out->n_kept = static_cast<uint32_t>(s.n);

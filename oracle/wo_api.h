@@ -161,6 +161,7 @@ typedef struct wo_batch_row {
     uint64_t step;
     float rep, pres, freq;
     uint32_t n_hist, n_bias;
+    int32_t race; /* Sampler::race: the exponential-race draw of src/sampling/sampler.cpp:80-106 instead of the inverse CDF */
 } wo_batch_row;
 
 typedef struct wo_batch_out {
@@ -170,7 +171,8 @@ typedef struct wo_batch_out {
     int32_t closed;
     float m, sum;
     uint32_t big_used, full_used;
-    double margin;       /* distance of the draw to the nearest CDF step, in probability units of the kept set */
+    double margin;       /* distance of the draw to the nearest CDF step, in probability units of the kept set; race draw:
+                            relative gap between the two smallest keys (on an open row also |u - S| of the list-or-tail test) */
     double margin_top_p; /* distance of the cumulative sum to top_p on either side of the cut (1 when not cut) */
     double margin_min_p; /* relative distance of the nearest candidates' p to the min-p floor (1 when not cut) */
 } wo_batch_out;

@@ -128,7 +128,7 @@ def oracle_row(c, r, rng_mode, lib=None):
     allow = np.ascontiguousarray(c["allow"][r]) if c["allow"] is not None else None
     prm = wo.BatchRow(inv_t=c["inv_t"][r], top_k=int(c["top_k"][r]), top_p=float(c["top_p"][r]), min_p=float(c["min_p"][r]),
                       seed=int(c["seed"][r]), step=int(c["step"][r]), rep=c["rep"][r], pres=c["pres"][r], freq=c["freq"][r],
-                      n_hist=hist.size, n_bias=bi.size)
+                      n_hist=hist.size, n_bias=bi.size, race=int(c["race"][r]) if c.get("race") is not None else 0)
     cands = np.zeros(max(V, 16384), dtype=wo.CAND_DT)
     out = wo.BatchOut()
     hist, bi, bv = np.ascontiguousarray(hist), np.ascontiguousarray(bi), np.ascontiguousarray(bv)
@@ -169,6 +169,7 @@ def upload(c, device="cuda:0"):
         d["max_bias"] = n
     if c["allow"] is not None:
         d["allow"] = torch.from_numpy(c["allow"].view(np.int32)).to(device)
+    d["race"] = torch.from_numpy(np.ascontiguousarray(c["race"], np.int32)).to(device) if c.get("race") is not None else None
     return d
 
 
@@ -177,7 +178,7 @@ def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0):
     return m.BatchSampler(d["logits"], d["inv_t"], d["seed"], d["step"], top_k=d["top_k"], top_p=d["top_p"], min_p=d["min_p"],
                           rng=rng_mode, hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
                           bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], max_hist=d["max_hist"],
-                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode)
+                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"))
 
 
 def compare_rows(c, smp, rows_to_check, rng_mode, check_kept=True, near_tol=1e-6, verbose=False):

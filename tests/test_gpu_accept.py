@@ -16,10 +16,10 @@ V = 32000
 NEAR = 1 | 2 | 4  # WS_FLAG_NEAR_*
 
 
-def _oracle_accept(lib, x, prm, dr, nd, n_gen):
+def _oracle_accept(lib, x, prm, dr, nd, n_gen, race=False):
     rows, keep = wo.make_rows(x, 256, 16384)
     cands = np.zeros(max(V, 16384), dtype=wo.CAND_DT)
-    sm = wo.new_sampler(temp=prm["temp"], top_k=prm["top_k"], top_p=prm["top_p"], min_p=prm["min_p"], seed=prm["seed"])
+    sm = wo.new_sampler(temp=prm["temp"], top_k=prm["top_k"], top_p=prm["top_p"], min_p=prm["min_p"], seed=prm["seed"], race=race)
     rp = wo.Relax(0, 0, 0.0, 0.0, 0.0)
     hist = np.zeros(1, dtype=np.uint32)
     relaxed, acc, chosen = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
@@ -28,7 +28,7 @@ def _oracle_accept(lib, x, prm, dr, nd, n_gen):
     return acc.value, chosen.value
 
 
-def _sequences(n_seq, seed, open_rows=False):
+def _sequences(n_seq, seed, open_rows=False, race=False):
     rng = np.random.default_rng(seed)
     lib = wo.load("oracle")
     seqs = []
@@ -45,9 +45,9 @@ def _sequences(n_seq, seed, open_rows=False):
         dr = rng.integers(0, V, size=16).astype(np.uint32)
         for r in range(nd):  # draft r = what the oracle samples at position r given the drafts before it, most of the time
             if rng.random() < 0.8:
-                dr[r] = _oracle_accept(lib, x, prm, dr, r, n_gen)[1]
-        acc, chosen = _oracle_accept(lib, x, prm, dr, nd, n_gen)
-        seqs.append(dict(nd=nd, x=x, prm=prm, n_gen=n_gen, dr=dr, acc=acc, chosen=chosen))
+                dr[r] = _oracle_accept(lib, x, prm, dr, r, n_gen, race)[1]
+        acc, chosen = _oracle_accept(lib, x, prm, dr, nd, n_gen, race)
+        seqs.append(dict(nd=nd, x=x, prm=prm, n_gen=n_gen, dr=dr, acc=acc, chosen=chosen, race=race))
     return seqs
 
 
@@ -67,7 +67,8 @@ def _device_accept(seqs, spoil=None):
     seed = per(lambda q: q["prm"]["seed"], np.int64)
     step = np.concatenate([q["n_gen"] + np.arange(q["nd"] + 1, dtype=np.int64) for q in seqs])
     t = lambda a: torch.from_numpy(a).to(dev)
-    smp = m.BatchSampler(t(x), t(inv_t), t(seed), t(step), top_k=t(top_k), top_p=t(top_p), min_p=t(min_p), rng=0)
+    race = t(np.ones(rows, np.int32)) if seqs[0].get("race") else None
+    smp = m.BatchSampler(t(x), t(inv_t), t(seed), t(step), top_k=t(top_k), top_p=t(top_p), min_p=t(min_p), rng=0, race=race)
     smp.run()
     ctl = np.zeros((len(seqs), 64), dtype=np.int32)
     for s, q in enumerate(seqs):
@@ -116,6 +117,23 @@ def test_accept_sampled_on_open_rows():
         else:
             assert any(flags[row0[s] + j] & NEAR for j in range(min(int(n_acc[s]), q["acc"]) + 1)), (s, n_acc[s], q["acc"])
     assert exact >= len(seqs) - 2, exact
+
+
+@pytest.mark.parametrize("open_rows", [False, True])
+def test_accept_sampled_with_the_race_draw(open_rows):
+    """The "specsample" rule: the target draw of every verify row is the race (Sampler::race), drafts mostly the tokens
+    that race picks."""
+    seqs = _sequences(16, 2718, open_rows=open_rows, race=True)
+    n_acc, chosen, status, ctl, token, flags, row0 = _device_accept(seqs)
+    exact = 0
+    for s, q in enumerate(seqs):
+        assert status[s] == 0, s
+        if n_acc[s] == q["acc"] and chosen[s] == q["chosen"]:
+            exact += 1
+        else:
+            assert any(flags[row0[s] + j] & NEAR for j in range(min(int(n_acc[s]), q["acc"]) + 1)), (s, n_acc[s], q["acc"])
+    assert exact >= len(seqs) - 2, exact
+    assert sum(q["acc"] for q in seqs) >= len(seqs)
 
 
 def test_accept_sampled_hands_a_failed_row_to_the_host():

@@ -103,6 +103,35 @@ def test_open_rows_odd_shapes(mode):
     print(res)
 
 
+@pytest.mark.parametrize("rng_mode", [0, 1])
+@pytest.mark.parametrize("mode", MODES)
+def test_race_draw_matches_the_oracle(rng_mode, mode):
+    """Sampler::race (the "specsample" rule, src/sampling/sampler.cpp:80-106) on rows with a top-k (the kept set is the
+    sorted list), on rows cut by top-p / min-p alone (every kept token of the row is hashed) and on open rows (race
+    over the 256 candidates or the walk over the rest), penalties and bias in force; rows without the race in between."""
+    c = gc.make_cfg2(rows=48, V=32000, n_hist=512, n_bias=40)
+    c["top_k"][16:32] = 0
+    c["top_p"][16:24] = np.linspace(0.5, 0.99, 8)
+    _ = [c[k].__setitem__(slice(32, 48), v) for k, v in (("top_k", 0), ("top_p", 1.0), ("min_p", 0.0))]
+    c["inv_t"][32:48] = (1.0 / np.linspace(0.3, 1.6, 16)).astype(np.float32)
+    c["race"] = np.ones(48, np.int32)
+    c["race"][::5] = 0
+    res, smp = run_case(c, rng_mode, kept_cap=1024, mode=mode)
+    raced_open = sum(gc.oracle_row(c, r, rng_mode)[0].full_used == 0 for r in range(32, 48) if c["race"][r])
+    assert 3 <= raced_open <= 11, raced_open
+    print(res, raced_open)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_race_draw_on_the_tile_shape_rows(mode):
+    """Top-p alone on long Gaussian rows: tens of thousands of kept tokens per row, bf16 rows with heavy ties too."""
+    for c in (gc.make_tile(rows=6, V=151936, n_hist=2048), gc.make_cfg3(rows=6, V=40000, n_hist=256),
+              gc.make_cfg5(rows=6, V=32768, n_hist=400, n_bias=30), gc.make_cfg2(rows=6, V=5003, n_hist=300, n_bias=24)):
+        c["race"] = np.ones(6, np.int32)
+        res, _ = run_case(c, 1, kept_cap=64, expect_near=0.2, mode=mode)
+        print(c["name"], res)
+
+
 @pytest.mark.parametrize("mode", MODES)
 def test_bf16_rows(mode):
     c = gc.make_cfg3(rows=6, V=40000, n_hist=256)
@@ -324,6 +353,7 @@ def test_random_shapes_filters_and_masks_both_kernels():
             c["top_p"] = rng.choice([1.0, 0.999, 0.95, 0.9, 0.5, 0.1], rows).astype(np.float64)
             c["min_p"] = rng.choice([0.0, 0.0, 0.01, 0.2], rows).astype(np.float64)
             c["inv_t"] = (1.0 / rng.uniform(0.3, 2.0, rows)).astype(np.float32)
+            c["race"] = rng.integers(0, 2, rows).astype(np.int32)
             if rng.random() < 0.3:
                 for r in range(rows):
                     off = rng.random(V) < rng.choice([0.5, 0.9, 0.99])

@@ -154,6 +154,37 @@ def test_batch_row_equals_filter_on_penalised_row():
         assert out.token == kept["id"][j] and out.prob == np.float32(kept["p"][j]) and out.closed == 1
 
 
+def test_batch_row_race_equals_the_sampler_race():
+    """The batched row with the race draw = penalties, then prepare + sampleRace of the sampler module (pinned by the
+    reference's own cases) on the penalised row, for closed rows (top-k / top-p / min-p) and open ones (race on the
+    candidates or, past their mass, the walk over the rest of the row). The reference's uniform is the batch's
+    splitmix uniform of (seed, step)."""
+    rng = np.random.default_rng(14)
+    walked = raced_open = 0
+    for it in range(60):
+        V = int(rng.integers(300, 20000))
+        x = (rng.standard_normal(V) * 2).astype(np.float32)
+        hist = rng.integers(0, V, 100)
+        open_row = it % 3 == 0
+        temp = float(rng.uniform(0.3, 1.5))
+        prm = wo.BatchRow(inv_t=np.float32(1 / temp), top_k=0 if open_row else int(rng.choice([0, 20, 50])),
+                          top_p=1.0 if open_row else float(rng.uniform(0.8, 1.0)), min_p=0.0 if open_row else 0.02,
+                          seed=99 + it, step=7 * it, rep=1.1, pres=0.2, freq=0.05, race=1)
+        out, kept, y = batch_row(x, prm, hist=hist, row=it, rng_mode=0)
+        rows, keep = wo.make_rows(y.reshape(1, V), 256, 16384)
+        s = wo.new_sampler(top_k=prm.top_k, top_p=prm.top_p, min_p=prm.min_p, seed=prm.seed, race=True)
+        s.inv_t = prm.inv_t
+        c = np.zeros(max(V, 16384), dtype=wo.CAND_DT)
+        lib.wo_prepare_row(C.byref(rows), C.byref(s), wo._ptr(c), 0)
+        s.pos_idx = prm.step
+        want = lib.wo_sample_race(C.byref(rows), C.byref(s), wo._ptr(c))
+        assert out.token == want, (it, out.token, want)
+        assert out.closed == (0 if open_row else 1)
+        walked += out.full_used > 0 and open_row
+        raced_open += open_row and out.full_used == 0
+    assert walked >= 3 and raced_open >= 3, (walked, raced_open)
+
+
 def spec(p, q, draft, seed=9, row=3, step0=100, rng_mode=1):
     n_pos, V = p.shape
     out = np.full(n_pos, -1, dtype=np.int32)

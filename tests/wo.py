@@ -41,7 +41,7 @@ class QDist(C.Structure):
 class BatchRow(C.Structure):
     _fields_ = [("inv_t", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_double), ("min_p", C.c_double),
                 ("seed", C.c_uint64), ("step", C.c_uint64), ("rep", C.c_float), ("pres", C.c_float),
-                ("freq", C.c_float), ("n_hist", C.c_uint32), ("n_bias", C.c_uint32)]
+                ("freq", C.c_float), ("n_hist", C.c_uint32), ("n_bias", C.c_uint32), ("race", C.c_int32)]
 
 
 class BatchOut(C.Structure):

@@ -50,7 +50,8 @@ class Batch(C.Structure):
                 ("token", C.c_void_p), ("prob", C.c_void_p), ("n_kept", C.c_void_p), ("flags", C.c_void_p),
                 ("stats", C.c_void_p), ("margin", C.c_void_p), ("kept_ids", C.c_void_p), ("kept_logits", C.c_void_p),
                 ("kept_cap", C.c_uint32),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32)]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32),
+                ("race", C.c_void_p)]
 
 
 class SpecVerify(C.Structure):
@@ -247,7 +248,7 @@ class BatchSampler:
 
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
-                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO):
+                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -256,7 +257,7 @@ class BatchSampler:
         rows, V = logits.shape
         self.keep = dict(logits=logits, inv_t=inv_t, seed=seed, step=step, top_k=top_k, top_p=top_p, min_p=min_p,
                          hist=hist, hist_off=hist_off, rep=rep, pres=pres, freq=freq, bias_ids=bias_ids,
-                         bias_vals=bias_vals, bias_off=bias_off, allow=allow)
+                         bias_vals=bias_vals, bias_off=bias_off, allow=allow, race=race)
         self.token = torch.empty(rows, dtype=torch.int32, device=dev)
         self.prob = torch.empty(rows, dtype=torch.float32, device=dev)
         self.n_kept = torch.empty(rows, dtype=torch.int32, device=dev)
@@ -279,6 +280,7 @@ class BatchSampler:
         b.kept_ids, b.kept_logits, b.kept_cap = _p(self.kept_ids), _p(self.kept_logits), kept_cap
         b.tol = tol
         b.mode = mode
+        b.race = _p(race)
         need = lib().ws_sample_batch_workspace(C.byref(b))
         self.workspace = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
         b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()

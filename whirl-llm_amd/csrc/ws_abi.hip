@@ -230,6 +230,7 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.lds_cnt = p.lds_cnt;
     a.lds_tie = p.lds_tie;
     a.two_sweep = b->mode == WS_MODE_AUTO ? 1 : 0;
+    a.race = b->race;
     if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
     if (!attr_set) {

@@ -83,6 +83,7 @@ struct BatchArgs {
                        // many 16-bit counts. Second copy of the histogram during the single sweep, then the id bitmap +
                        // prefix that sorts heavy ties by id
     int two_sweep;     // rows the single sweep cannot take: histogram against a provisional bound in the first sweep (else: exact mode)
+    const int32_t* race;  // per row, non-zero: exponential-race draw
     uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
 };
 
@@ -489,6 +490,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ float red_f[WS_WAVES];
     __shared__ uint32_t red_u[WS_WAVES];
     __shared__ double red_d[WS_WAVES];
+    __shared__ unsigned long long red_q[WS_WAVES];
     __shared__ uint32_t s_cnt;
     __shared__ double s_exp[128];  // kExpHi, kExpLo
     __shared__ double pm64[64];    // every 64th entry of the scanned histogram's mass prefixes
@@ -1648,7 +1650,156 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double target = u * Zk;
     int32_t token = -1;
     double ptok = 0;
-    {
+    // The race draw of the "specsample" rule (src/sampling/sampler.cpp:80-106): the kept token with the smallest
+    // E(token) / p(token), E = -ln(1 - U) with U hashed from (seed, step, token) (src/common/spec_sample.cpp:83-87),
+    // the earlier candidate in sorted order on equal keys. An open row races over its listed candidates when the
+    // uniform falls on their mass and otherwise takes the walk below with the same uniform.
+    const bool race = A.race != nullptr && A.race[row] != 0;
+    bool raced = false;
+    if (race && (!open_row || target < inc_of(i_last))) {
+        raced = true;
+        const uint32_t lane = static_cast<uint32_t>(lane_id());
+        const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+        const uint64_t rbase = mix64((seed ^ 0xA0761D6478BD642Full) + (step + 1ull) * 0x9E3779B97F4A7C15ull);
+        const double inf = __longlong_as_double(0x7FF0000000000000ll);
+        auto hash_of = [&](uint32_t id) { return mix64(rbase + (static_cast<uint64_t>(id) + 1ull) * 0xE7037ED1A0B428DBull); };
+        auto key_of = [&](uint64_t cand) {  // E / p of a candidate given as (logit key, ~id); inf when it has no mass
+            const float x = unkey32(static_cast<uint32_t>(cand >> 32));
+            const double e = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
+            const double E = -log(1.0 - unit53(hash_of(0xffffffffu - static_cast<uint32_t>(cand))));
+            return e > 0.0 ? E * Zk / e : inf;
+        };
+        // smallest key of the block, the candidate that is earlier in sorted order (the larger `who`) on equal keys
+        auto block_first = [&](double& k, uint64_t& who) {
+#pragma unroll
+            for (int o = 32; o; o >>= 1) {
+                const double ko = __shfl_xor(k, o);
+                const uint64_t wo = __shfl_xor(who, o);
+                if (ko < k || (ko == k && wo > who)) {
+                    k = ko;
+                    who = wo;
+                }
+            }
+            __syncthreads();
+            if (lane == 0) {
+                red_d[wv] = k;
+                red_q[wv] = who;
+            }
+            __syncthreads();
+            k = red_d[0];
+            who = red_q[0];
+            for (uint32_t w = 1; w < WS_WAVES; ++w) {
+                const double ko = red_d[w];
+                const uint64_t wo = red_q[w];
+                if (ko < k || (ko == k && wo > who)) {
+                    k = ko;
+                    who = wo;
+                }
+            }
+        };
+        const uint64_t* cand = keys;
+        uint32_t n_cand = n3;  // top-k and open rows: the kept set is the first n3 entries of the sorted list
+        if (!prefix_mode && !open_row) {
+            // The kept set is a stretch of the row far longer than the list: every token of the row is hashed in one
+            // more sweep. The smallest key among the gathered candidates, K0, bounds the winner's; a kept token can
+            // reach it only if U <= E <= K0 p, which the upper 24 bits of the hash and the 32-bit mass decide for all
+            // but a few dozen tokens; those are collected (with room for everything within `tol` of K0, which the
+            // near-tie flag needs) and their keys worked out in double precision.
+            double k0 = inf;
+            uint64_t w0 = 0;
+            for (uint32_t i = t; i < n_list; i += WS_BLOCK)
+                if (pos_of(i) < n3) {
+                    const double k = key_of(keys[i]);
+                    if (k < k0) {
+                        k0 = k;
+                        w0 = keys[i];
+                    }
+                }
+            block_first(k0, w0);
+            const float thr = static_cast<float>(fmin(k0 / Zk * (1.0 + tol) * 1.0001, 3e38));
+            const double k2 = static_cast<double>(inv_t) * 1.4426950408889634;
+            const float kh = static_cast<float>(k2), kl = static_cast<float>(k2 - static_cast<double>(kh));
+            const float cut_x = unkey32(static_cast<uint32_t>(kept_key >> 32));
+            const uint32_t cut_id = 0xffffffffu - static_cast<uint32_t>(kept_key);
+            uint64_t* surv = keys;
+            if (t == 0) s_cnt = 0;
+            __syncthreads();  // the list has been read by everybody: its LDS takes the survivors
+            auto probe = [&](uint32_t i, float x) {
+                const float d = __fsub_rn(x, m);
+                const float yh = __fmul_rn(d, kh);
+                const float yl = __fmaf_rn(d, kl, __fmaf_rn(d, kh, -yh));
+                const float n = rintf(yh);
+                const float e = ldexpf(__builtin_amdgcn_exp2f(__fadd_rn(__fsub_rn(yh, n), yl)), static_cast<int>(n));
+                const bool in = (yh > -140.f) & ((x > cut_x) | ((x == cut_x) & (i <= cut_id)));
+                const float ul = static_cast<float>(static_cast<uint32_t>(hash_of(i) >> 40)) * 5.9604644775390625e-8f;  // <= U
+                if (in & (ul <= thr * e)) {
+                    const uint32_t slot = atomicAdd(&s_cnt, 1u);
+                    if (slot < kCap) surv[slot] = key64(x, i);
+                }
+            };
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u;
+            const uint32_t n_vec = rv.vec ? V / per : 0u;
+            if (n_vec)
+                stream_row_wide(
+                    rv,
+                    [&](uint32_t i, float x, int) {
+                        if (i < n_vec * per) probe(i, x);
+                    },
+                    [&](uint32_t, uint32_t) {});
+            if (n_touched) {
+                const uint32_t span = (nW + WS_BLOCK - 1) / WS_BLOCK;
+                const uint32_t w0 = t * span, w1 = min(w0 + span, nW);
+                for (uint32_t w = w0; w < w1; ++w) {
+                    uint32_t bits = touched[w];
+                    uint32_t r = wprefix[w];
+                    while (bits) {
+                        const uint32_t i = (w << 5) + (__ffs(bits) - 1u);
+                        bits &= bits - 1u;
+                        if (i < n_vec * per) probe(i, pv[r]);
+                        ++r;
+                    }
+                }
+            }
+            for (uint32_t i = n_vec * per + t; i < V; i += WS_BLOCK) probe(i, adjusted_logit(rv, i));
+            __syncthreads();
+            n_cand = s_cnt;
+            if (n_cand > kCap) {
+                flags |= kOverflow;
+                n_cand = 0;
+            }
+            cand = surv;
+        }
+        // the two smallest keys among the candidates
+        double k1 = inf, k2nd = inf;
+        uint64_t w1 = 0;
+        for (uint32_t i = t; i < n_cand; i += WS_BLOCK) {
+            const uint64_t c = cand[i];
+            const double k = key_of(c);
+            if (k < k1 || (k == k1 && c > w1)) {
+                k2nd = k1;
+                k1 = k;
+                w1 = c;
+            } else if (k < k2nd) {
+                k2nd = k;
+            }
+        }
+        double kb = k1;
+        uint64_t wb = w1;
+        block_first(kb, wb);
+        double ks = (w1 == wb && k1 == kb) ? k2nd : k1;
+        uint64_t ws_ = 0;
+        block_first(ks, ws_);
+        if (flags & kOverflow) {
+            token = -1;
+        } else {
+            if (!(kb < inf)) wb = cand[0];  // no candidate has a mass: the first one (src/sampling/sampler.cpp:95)
+            token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(wb));
+            const float x = unkey32(static_cast<uint32_t>(wb >> 32));
+            ptok = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t))) / Zk;
+            mg_draw = ks < inf ? (ks - kb) / kb : 1.0;
+        }
+    }
+    if (!raced) {
         const uint32_t i = first_entry([&](uint32_t k) { return inc_of(k) > target; });
         bool found = false;
         if (i < n_list) {
@@ -1830,6 +1981,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         }
     }
+    if (race && open_row) mg_draw = fmin(mg_draw, fabs(target - inc_of(i_last)) / Zk);  // the list-or-rest decision
     // zero-mass tail candidates a top-k kept (no top-p / min-p cut them away again)
     const uint32_t tail_extra = (!use_top_p && !use_min_p && n3 == n1) ? n1_asked - n1 : 0u;
     if (mg_top_p < tol) flags |= kNearTopP;
