@@ -148,7 +148,7 @@ def run_workload(name, steps, warmup, check_rows):
 
 def reference_kernels(steps):
     """Launch times of the replacements of the reference's own kernels at the engine's shapes (vocab 151936): the greedy
-    picks on 1 / 32 / 256 rows, topk_rows with the engine's two list sizes on 1 / 32 rows. Synthetic N(0, sigma 2) logits."""
+    picks on 1 / 32 / 256 rows, topk_rows with the engine's two list sizes on 1 / 32 rows, the drafter's dflash_topk. Synthetic N(0, sigma 2) logits."""
     import torch
     import gpu_cases as gc
     m = gc.pkg()
@@ -181,6 +181,10 @@ def reference_kernels(steps):
         for K in (256, 16384):
             timed(f"topk_rows K={K}", rows, lambda: L.ws_topk_rows(S(), P(x), V, K, 1.25, P(ids), P(vals), P(st), rows),
                   rows * (V * 4 + K * 8 + 8))
+    x = torch.randn(16, V, device="cuda:0") * 2  # the drafter's candidates: 16 per draft position, 16 positions
+    ids = torch.empty((16, 16), dtype=torch.int32, device="cuda:0")
+    vals = torch.empty((16, 16), dtype=torch.float32, device="cuda:0")
+    timed("dflash_topk k=16", 16, lambda: L.ws_dflash_topk(S(), P(x), V, V, 16, P(ids), P(vals), 16), 16 * (V * 4 + 16 * 8))
     x = torch.randn(1, V, device="cuda:0") * 2
     tok = torch.empty(1, dtype=torch.int32, device="cuda:0")
     pr = torch.empty(1, dtype=torch.float32, device="cuda:0")

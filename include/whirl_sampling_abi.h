@@ -93,6 +93,11 @@ int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, cons
  * atomics; here both are fixed: ties at the cut keep the lowest token ids, entries are in ascending id order.
  * Output layout as the engine's buffers expect it (src/server/engine_sampling.cpp:37-43). */
 int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows);
+/* dflash_topk(x, n, ld, k, ids, vals): kernels/dflash.hip:36-77; launch site src/model/dflash.cpp:302 (the drafter's
+ * candidates per draft position). ids / vals[row][0..k) = the k <= 64 largest logits of row `row` (rows ld floats apart)
+ * in key order: larger value first, then smaller index; NaN counts as -inf and is written out as it stands. The
+ * reference finds them in k passes over the row; here the row is read once. */
+int ws_dflash_topk(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows);
 
 /* ---- (2) batched fused sampler ---------------------------------------------------------------------------- */
 

@@ -110,6 +110,31 @@ void wo_topk_row(const float* x, int32_t n, int32_t K, float inv_t, int32_t* ids
     }
 }
 
+// kernels/dflash.hip:36-77: k rounds, round r takes the best key below round r - 1's; keys order by larger value,
+// then smaller index, NaN as -inf (:36-40); the value is written as it stands in the row
+void wo_dflash_topk_row(const float* x, int32_t n, int32_t k, int32_t* ids, float* vals) {
+    auto better = [](float va, int32_t ia, float vb, int32_t ib) {
+        if (va != va) va = kNegInf;
+        if (vb != vb) vb = kNegInf;
+        return va > vb || (va == vb && ia < ib);
+    };
+    float pv = std::numeric_limits<float>::infinity();
+    int32_t pi = -1;
+    for (int32_t r = 0; r < k; ++r) {
+        float best = kNegInf;
+        int32_t idx = 0x7fffffff;
+        for (int32_t i = 0; i < n; ++i)
+            if (better(pv, pi, x[i], i) && better(x[i], i, best, idx)) {
+                best = x[i];
+                idx = i;
+            }
+        pv = best;
+        pi = idx;
+        ids[r] = pi;
+        vals[r] = pv;
+    }
+}
+
 void wo_apply_penalties(float* x, uint32_t V, const uint32_t* allow, const int32_t* hist, uint32_t n_hist, float rep, float pres,
                         float freq, const int32_t* bias_ids, const float* bias_vals, uint32_t n_bias) {
     for (uint32_t i = 0; i < V; ++i) {

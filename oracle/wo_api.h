@@ -16,6 +16,8 @@
  *   include/whirl/relax_accept.h               relaxed acceptance
  *   tests/server/sampling_cases.h:69-90        host restatement of the 3-step candidate escalation
  *   tests/iso/fake_server_model.h:74-98        host top-k reference (value desc, id asc)
+ *   kernels/dflash.hip:36-77                   the drafter's small top-k in key order (k rounds), checked as
+ *                                              tests/kernels/test_dflash.cpp:99-131 checks it (partial sort by the same key)
  */
 #ifndef WO_API_H
 #define WO_API_H
@@ -143,6 +145,7 @@ int32_t wo_argmax(const float* x, int32_t n);
 float wo_argmax_prob(const float* x, int32_t n, int32_t* tok); /* 1 / sum exp(x - max), double accumulate */
 /* topk_rows reference (fake_server_model.h:74-98): K largest by (value desc, id asc), stats = {max, (float) sum_d}. */
 void wo_topk_row(const float* x, int32_t n, int32_t K, float inv_t, int32_t* ids, float* vals, float* stats);
+void wo_dflash_topk_row(const float* x, int32_t n, int32_t k, int32_t* ids, float* vals); /* kernels/dflash.hip:36-77 */
 
 /* Penalties, logit bias and allow-mask on one row, in place (not in the reference; closed forms):
  *   x = -inf where the allow bitmap (bit i of allow[i / 32]) is clear; NaN counts as -inf;

@@ -28,7 +28,7 @@ def test_code_object_exports_reference_kernel_names():
     m = gpu_cases.pkg()
     blob = open(m.CO_PATH, "rb").read()
     for k in (b"argmax", b"argmax_rows", b"argmax_rows_to", b"argmax_prob", b"draft_pick", b"draft_pick_rows",
-              b"draft_sample_rows", b"topk_rows"):
+              b"draft_sample_rows", b"topk_rows", b"dflash_topk"):
         assert b"\x00" + k + b"\x00" in blob, k
 
 

@@ -134,6 +134,36 @@ def test_topk_rows_ties_at_the_cut_keep_lowest_ids():
     assert ids.cpu().tolist()[0][:5] == [0, 1, 2, 3, 4] and ids.cpu().tolist()[0][5:] == [-1] * 4
 
 
+@pytest.mark.parametrize("k", [1, 16, 64])
+def test_dflash_topk_key_order(k):
+    """The cases of tests/kernels/test_dflash.cpp:99-131 (3-way tie at the top, ties straddling rank 16, NaN among equal
+    values) and a row with fewer numbers than k, at the drafter's vocabulary and on rows with a stride, against the
+    oracle's k rounds; ids and values exact, two runs identical."""
+    from test_oracle_batch import dflash_case
+    m = gpu_cases.pkg()
+    lib = wo.load("oracle")
+    for n, ld in ((248320, 248320), (50000, 50003), (20000, 20000)):
+        x = np.zeros((4, ld), np.float32)
+        x[:, :n] = dflash_case(n)
+        dx = torch.from_numpy(x).to(DEV)[:, :n]
+        ids, vals = m.dflash_topk(dx, k)
+        ids2, _ = m.dflash_topk(dx, k)
+        ids, vals = ids.cpu().numpy(), vals.cpu().numpy()
+        assert np.array_equal(ids, ids2.cpu().numpy())
+        for r in range(4):
+            wi, wv = np.zeros(k, np.int32), np.zeros(k, np.float32)
+            lib.wo_dflash_topk_row(wo._ptr(np.ascontiguousarray(x[r, :n])), n, k, wo._ptr(wi), wo._ptr(wv))
+            assert np.array_equal(ids[r], wi), (n, r, ids[r], wi)
+            assert vals[r].tobytes() == wv.tobytes(), (n, r)
+
+
+def test_dflash_topk_rejects_long_lists():
+    m = gpu_cases.pkg()
+    x = torch.zeros((1, 1000), device=DEV)
+    with pytest.raises(m.WsError):
+        m.dflash_topk(x, 65)
+
+
 def test_adjust_rows_matches_the_oracle_bit_for_bit():
     """ws_adjust_rows: the penalised copy of a row equals the oracle's wo_apply_penalties on every token, with mask, bias
     (repeated ids included), history counts, fp32 and bf16 input."""

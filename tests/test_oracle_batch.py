@@ -154,6 +154,40 @@ def test_batch_row_equals_filter_on_penalised_row():
         assert out.token == kept["id"][j] and out.prob == np.float32(kept["p"][j]) and out.closed == 1
 
 
+def dflash_case(n):
+    """The rows of tests/kernels/test_dflash.cpp:99-108: a 3-way tie at the top, ties straddling rank 16, a NaN among
+    equal values; one more with fewer numbers than k."""
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((4, n)).astype(np.float32)
+    x[0, [n - 1, 7, 1000]] = 10.0
+    x[1, np.arange(20) * 997] = 8.0
+    x[2, 5] = np.nan
+    x[2, [n - 2, 3, 40000 % n]] = 9.0
+    x[3, :] = -np.inf
+    x[3, [11, 5000, 4]] = [1.0, 1.0, np.nan]  # n > 5000
+    return x
+
+
+def dflash_want(row, k):
+    """The first k of a full stable sort by (value desc with NaN as -inf, index asc): the partial sort of the reference's test."""
+    v = np.where(np.isnan(row), -np.inf, row)
+    order = np.lexsort((np.arange(row.size), -v.astype(np.float64)))[:k]
+    return order.astype(np.int32), row[order]
+
+
+def test_dflash_topk_rounds_equal_a_sort_by_the_same_key():
+    x = dflash_case(50000)
+    for r in range(4):
+        for k in (1, 16, 64):
+            ids, vals = np.zeros(k, np.int32), np.zeros(k, np.float32)
+            lib.wo_dflash_topk_row(wo._ptr(x[r]), x.shape[1], k, wo._ptr(ids), wo._ptr(vals))
+            wi, wv = dflash_want(x[r], k)
+            assert np.array_equal(ids, wi) and vals.tobytes() == wv.tobytes(), (r, k)
+    ids, vals = np.zeros(8, np.int32), np.zeros(8, np.float32)
+    lib.wo_dflash_topk_row(wo._ptr(x[0][:5].copy()), 5, 8, wo._ptr(ids), wo._ptr(vals))  # k > n: the rounds run dry
+    assert list(ids[5:]) == [0x7fffffff] * 3 and all(np.isneginf(vals[5:]))
+
+
 def test_batch_row_race_equals_the_sampler_race():
     """The batched row with the race draw = penalties, then prepare + sampleRace of the sampler module (pinned by the
     reference's own cases) on the penalised row, for closed rows (top-k / top-p / min-p) and open ones (race on the

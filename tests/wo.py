@@ -89,6 +89,7 @@ _OWN_SIGS = {
     "wo_argmax": (C.c_int32, [C.c_void_p, C.c_int32]),
     "wo_argmax_prob": (C.c_float, [C.c_void_p, C.c_int32, C.POINTER(C.c_int32)]),
     "wo_topk_row": (None, [C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "wo_dflash_topk_row": (None, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
     "wo_apply_penalties": (None, [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_float, C.c_float,
                                   C.c_float, C.c_void_p, C.c_void_p, C.c_uint32]),
     "wo_sample_batch_row": (None, [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

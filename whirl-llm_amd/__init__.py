@@ -92,6 +92,7 @@ ABI = {
                                        C.POINTER(DSampArgs), C.c_void_p, C.c_uint]),
     "ws_topk_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_uint]),
+    "ws_dflash_topk": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
@@ -208,6 +209,17 @@ def topk_rows(x, K, inv_t):
     stats = torch.empty((rows, 2), dtype=torch.float32, device=x.device)
     check(lib().ws_topk_rows(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows), "ws_topk_rows")
     return ids, vals, stats
+
+
+def dflash_topk(x, k):
+    """x: [rows, n] float32, rows any stride -> ids int32 [rows, k], vals float32 [rows, k] in key order (value desc, id asc)."""
+    if not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32 or x.stride(1) != 1:
+        raise WsError("x: [rows, n] float32 device tensor with unit inner stride")
+    rows, n = x.shape
+    ids = torch.full((rows, k), -1, dtype=torch.int32, device=x.device)
+    vals = torch.zeros((rows, k), dtype=torch.float32, device=x.device)
+    check(lib().ws_dflash_topk(_stream(), _p(x), n, x.stride(0), k, _p(ids), _p(vals), rows), "ws_dflash_topk")
+    return ids, vals
 
 
 def adjust_rows(logits, hist=None, hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,

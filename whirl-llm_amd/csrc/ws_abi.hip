@@ -183,6 +183,12 @@ int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* i
     return done();
 }
 
+int ws_dflash_topk(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows) {
+    if (!x || !ids || !vals || n <= 0 || ld < n || k <= 0 || k > 64 || rows == 0) return WS_E_INVALID;
+    hipLaunchKernelGGL(dflash_topk, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, ld, k, ids, vals);
+    return done();
+}
+
 uint64_t ws_sample_batch_workspace(const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     return p.err == WS_OK ? p.workspace : 0;

@@ -351,10 +351,9 @@ __device__ __forceinline__ bool topk_by_counts(const float* __restrict__ x, int 
     return true;
 }
 
-}  // namespace ws
-
-extern "C" __global__ void __launch_bounds__(WS_BLOCK)
-    topk_rows(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
+// The K largest logits of one row (x, n tokens) into ids / vals in ascending id order, ties at the cut to the lowest ids;
+// stats (unless null) = {max, sum exp((x - max) * inv_t)}. Every return is taken by the whole workgroup.
+__device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
     __shared__ uint32_t hist[4096];
     __shared__ uint64_t cand[ws::kTopkCap];
     __shared__ float red_f[WS_WAVES];
@@ -363,10 +362,6 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     __shared__ uint32_t s_cnt[WS_WAVES];
     __shared__ uint32_t s_n;
     __shared__ uint64_t s_kmin;
-    const int row = blockIdx.x;
-    x += static_cast<size_t>(row) * n;
-    ids += static_cast<size_t>(row) * K;
-    vals += static_cast<size_t>(row) * K;
     const uint32_t kk = static_cast<uint32_t>(K < n ? K : n);
 
     // A bound above the maximum (+ 8 units) and the spread of the logits, both from the first 4096 of them: the bins
@@ -431,9 +426,9 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     const float top = ws::block_max(m, red_f);
     const float part = m > -INFINITY ? s * __expf((m - top) * inv_t) : 0.f;
     const float sum = ws::block_sum(part, red_f);
-    if (threadIdx.x == 0) {
-        stats[2 * row] = top;
-        stats[2 * row + 1] = sum;
+    if (threadIdx.x == 0 && stats) {
+        stats[0] = top;
+        stats[1] = sum;
     }
     if (kk == 0) return;
     __syncthreads();  // the counts are complete
@@ -459,4 +454,44 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
         ids[o] = i;
         vals[o] = v;
     });
+}
+
+}  // namespace ws
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    topk_rows(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
+    const size_t row = blockIdx.x;
+    ws::topk_one_row(x + row * n, n, K, inv_t, ids + row * K, vals + row * K, stats + 2 * row);
+}
+
+// dflash_topk(x, n, ld, k, ids, vals) of kernels/dflash.hip:36-77: the k <= 64 largest logits of each row in key order
+// (larger value first, then smaller index; NaN counts as -inf and is written out as it stands), rows ld floats apart.
+// The reference takes k passes over the row, one winner each; here the row is read once by the select above and the
+// k winners are put in order by one wave.
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) dflash_topk(const float* x, int n, int ld, int k, int* ids, float* vals) {
+    const size_t row = blockIdx.x;
+    ids += row * k;
+    vals += row * k;
+    ws::topk_one_row(x + row * ld, n, k, 1.f, ids, vals, nullptr);
+    __syncthreads();  // the winners are in ids / vals, in id order
+    const int kk = k < n ? k : n;
+    if (threadIdx.x >= 64) return;
+    const int lane = threadIdx.x;
+    const int id = lane < kk ? ids[lane] : 0x7fffffff;
+    const float raw = lane < kk ? x[row * ld + id] : -INFINITY;  // as it stands in the row: a NaN is written out as NaN
+    const float v = fmaxf(raw, -INFINITY);  // NaN -> -inf
+    int rank = 0;
+    for (int j = 0; j < kk; ++j) {
+        const float vj = __shfl(v, j);
+        const int ij = __shfl(id, j);
+        rank += (vj > v || (vj == v && ij < id)) ? 1 : 0;
+    }
+    if (lane < kk) {
+        ids[rank] = id;
+        vals[rank] = raw;
+    }
+    for (int o = kk + lane; o < k; o += 64) {  // rows shorter than k: the reference's rounds find nothing more
+        ids[o] = 0x7fffffff;
+        vals[o] = -INFINITY;
+    }
 }
