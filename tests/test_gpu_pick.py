@@ -120,6 +120,26 @@ def test_topk_rows_against_oracle(rows5, K):
         assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1]
 
 
+def test_topk_rows_cold_temperature_and_crowded_stretch(rows5):
+    """Paths beside the usual one: a temperature below 1 / 8 (the normaliser is then rescaled against the running maximum
+    instead of a fixed reference), and a row whose largest logits all sit in the 256 tokens one wave reads with one
+    instruction, which overflows that wave's stretch of the candidate list (the row is then counted in full)."""
+    m = gpu_cases.pkg()
+    lib = wo.load("oracle")
+    x, _ = rows5
+    x = x[:2].copy()
+    x[1, :200] = 20.0 + np.arange(200, dtype=np.float32) * 0.01
+    dx = torch.from_numpy(x).to(DEV)
+    for K, inv_t in ((3, 10.0), (256, 10.0), (256, 1.0), (512, 0.5)):
+        ids, vals, stats = (a.cpu().numpy() for a in m.topk_rows(dx, K, inv_t))
+        for r in range(2):
+            wi, wv, ws_ = np.zeros(K, np.int32), np.zeros(K, np.float32), np.zeros(2, np.float32)
+            lib.wo_topk_row(wo._ptr(np.ascontiguousarray(x[r])), x.shape[1], K, np.float32(inv_t), wo._ptr(wi), wo._ptr(wv), wo._ptr(ws_))
+            assert np.array_equal(ids[r], np.sort(wi)), (K, inv_t, r)
+            assert vals[r].tobytes() == x[r][ids[r]].tobytes()
+            assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1], (K, inv_t, r, stats[r], ws_)
+
+
 def test_topk_rows_ties_at_the_cut_keep_lowest_ids():
     m = gpu_cases.pkg()
     n, K = 5000, 7

@@ -94,6 +94,8 @@ __device__ __forceinline__ void select_in_id_order(const float* __restrict__ x, 
 
 // ---- the histogram route. All threads return the same answer; false = nothing was written, take the radix route.
 constexpr uint32_t kTopkCap = 2048;     // tokens of the cut's bin resolved in LDS
+constexpr uint32_t kTopkWaveCap = kTopkCap / WS_WAVES;  // the first pass lists per wave: a stretch of the list and a counter each
+                                                        // (one counter for all waves is one LDS word that every hit queues on)
 constexpr int kTopkBins = 4096;
 constexpr int kTopkTail = kTopkBins - 64;  // the last 64 bins take everything else, one bin per lane (same-word atomics queue)
 
@@ -113,38 +115,116 @@ __device__ __forceinline__ uint32_t topk_bin(float v, float scale, float a32, fl
     return static_cast<uint32_t>(__builtin_fminf(__fmaf_rn(v, -scale, a32), tail));  // NaN -> tail; above the bound -> 0
 }
 
-// Pass 1 of both routes: per-thread online maximum and rescaled sum; with `hist` also the bin counts.
-// With COUNT every token is also counted in its bin, and tokens of the bins up to `list_bin` (-1: none) are put on the
-// list as keys: when the list ends up holding at least K tokens, the K largest are among them and no further pass over
-// the row is needed.
+// Pass 1 of both routes: per-thread maximum and sum of exp((x - reference) * inv_t); with `hist` also the bin counts.
+// The reference is `ref` when that is a number (the caller knows a value a few units around the maximum: nothing needs
+// rescaling, s = sum 2^((v - ref) k2)), else the thread's running maximum (s is rescaled whenever that rises).
+// With COUNT every token is also counted in its bin. With a `list_bin` (>= 0) only the tokens of the bins up to it are
+// counted, and they are put on the list as keys (wave w: list[w * kTopkWaveCap ...], n_list[w] of them): when the list ends up holding at least K tokens, the K largest are
+// among them, the counts of those bins are complete and no further pass over the row is needed. (One LDS atomic per
+// token is what bounds a counting pass; a listing pass has a few per thousand tokens.)
 template <bool COUNT>
 __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist,
-                                                int list_bin, uint64_t* list, uint32_t* n_list, float& m, float& s) {
+                                                int list_bin, uint64_t* list, uint32_t* n_list, float ref, float& m, float& s) {
     const float tail = static_cast<float>(kTopkTail + lane_id());
-    for_each_f32(x, n, [&](int i, float v) {
-        if (v > m) {
-            s = s * __expf((m - v) * inv_t) + 1.f;
+    const float k2 = inv_t * 1.4426950408889634f;  // exp((v - m) * inv_t) = 2^((v - m) * k2)
+    const bool fixed = ref == ref;  // uniform
+    const float rk = ref * k2;
+    const bool listed = list_bin >= 0;
+    // a logit below this cannot lie in a bin up to list_bin (half a bin of slack for the roundings; the bin itself decides)
+    const float list_floor = listed ? (a32 - (static_cast<float>(list_bin) + 1.5f)) / scale : -INFINITY;
+    auto count = [&](int i, float v) {
+        const uint32_t b = topk_bin(v, scale, a32, tail);
+        if (!listed) {
+            atomicAdd(&hist[b], 1u);
+        } else if (static_cast<int>(b) <= list_bin) {  // a few per thousand tokens
+            atomicAdd(&hist[b], 1u);
+            const uint32_t slot = atomicAdd(&n_list[wave_id()], 1u);
+            if (slot < kTopkWaveCap) list[wave_id() * kTopkWaveCap + slot] = key64(v, static_cast<uint32_t>(i));
+        }
+    };
+    auto one = [&](int i, float v) {
+        if (fixed) {
+            if (v > -INFINITY) {  // not for NaN either
+                m = fmaxf(m, v);
+                s += __builtin_amdgcn_exp2f(__fmaf_rn(v, k2, -rk));
+            }
+        } else if (v > m) {
+            s = s * __builtin_amdgcn_exp2f((m - v) * k2) + 1.f;
             m = v;
         } else if (v > -INFINITY) {
-            s += __expf((v - m) * inv_t);
+            s += __builtin_amdgcn_exp2f((v - m) * k2);
         }
+        if (COUNT) count(i, v);
+    };
+    // 128-bit loads on the aligned body of the row: the running maximum is raised once per vector (a branch that is
+    // rarely taken after the first few vectors), then the four terms are added without a branch; scalar steps on a
+    // misaligned head and on the tail
+    const int t = threadIdx.x;
+    int head = static_cast<int>(((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(x)) & 15u)) & 15u) >> 2);
+    if (head > n) head = n;
+    if (t < head) one(t, x[t]);
+    const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + head);
+    const int nv = (n - head) >> 2;
+    // kU loads per thread go out together and the next kU are requested before these are looked at: the branches and
+    // LDS atomics below would otherwise keep the compiler from having more than one load of a thread in flight
+    constexpr int kU = 4;
+    float4 cur[kU], nxt[kU];
+    auto fetch = [&](int j0, float4 (&q)[kU]) {
+#pragma unroll
+        for (int u = 0; u < kU; ++u) q[u] = xv[min(j0 + u * WS_BLOCK + t, nv - 1)];
+    };
+    if (nv > 0) fetch(0, cur);
+    for (int j0 = 0; j0 < nv; j0 += kU * WS_BLOCK) {
+        const bool more = j0 + kU * WS_BLOCK < nv;
+        if (more) fetch(j0 + kU * WS_BLOCK, nxt);
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+        const int j = j0 + u * WS_BLOCK + t;
+        if (j >= nv) continue;
+        const float4 q = cur[u];
+        const int i = head + 4 * j;
+        // NaN -> -inf (fmaxf returns the operand that is a number)
+        const float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
+        const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+        float mk = rk;
+        if (fixed) {
+            m = fmaxf(m, vm);
+        } else {
+            if (vm > m) {
+                s *= __builtin_amdgcn_exp2f((m - vm) * k2);  // m = -inf: s is 0 and stays 0
+                m = vm;
+            }
+            mk = fmaxf(m, -1.0e30f) * k2;  // a row of -inf so far: every term below is 2^-inf = 0, never inf - inf
+        }
+        float add = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) add += __builtin_amdgcn_exp2f(__fmaf_rn(v[e], k2, -mk));
+        s += add;
         if (COUNT) {
-            const uint32_t b = topk_bin(v, scale, a32, tail);
-            atomicAdd(&hist[b], 1u);
-            if (static_cast<int>(b) <= list_bin) {  // a few per thousand tokens
-                const uint32_t slot = atomicAdd(n_list, 1u);
-                if (slot < kTopkCap) list[slot] = key64(v, static_cast<uint32_t>(i));
+            if (!listed) {  // uniform
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicAdd(&hist[topk_bin(v[e], scale, a32, tail)], 1u);
+            } else if (vm >= list_floor) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) count(i + e, v[e]);
             }
         }
-    });
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < kU; ++u) cur[u] = nxt[u];
+        }
+    }
+    const int i = head + 4 * nv + t;
+    if (i < n) one(i, x[i]);
 }
 
 // The list holds every token of the row up to bin `list_bin`, the counts say in which bin the kk-th largest lies. When
 // that bin is on the list, the tokens of the bins before it are kept as they are, the cut bin's few tokens are ranked
-// among themselves, and the kk kept ones are sorted by id (bitonic, in LDS) and written out. `work`: LDS, 4096 words
+// among themselves, and the kk kept ones are put in id order (each counts the kept ids below its own) and written out. `work`: LDS, 4096 words
 // (the counts, read first and then overwritten). Returns 0 when done; otherwise nothing was written: 1 = the list does
 // not reach the cut (the counts are still there), 2 = too many tokens tie at the cut (the counts are gone).
-__device__ __forceinline__ int topk_from_list(const float* __restrict__ x, const uint64_t* list, uint32_t n_list, int list_bin, uint32_t kk,
+__device__ __forceinline__ int topk_from_list(const float* __restrict__ x, const uint64_t* list, const uint32_t* n_list, int list_bin, uint32_t kk,
                                                float scale, float a32, uint32_t* work, uint32_t* red, uint32_t* sel, int* ids,
                                                float* vals) {
     const uint32_t t = threadIdx.x;
@@ -178,7 +258,8 @@ __device__ __forceinline__ int topk_from_list(const float* __restrict__ x, const
     uint64_t* cut = reinterpret_cast<uint64_t*>(work) + 1024;    // up to 1024 keys of the cut bin
     constexpr uint32_t kCutCap = 1024;
     const float no_tail = 4095.f;  // listed tokens lie before the tail: any clamp at or past it gives their bin
-    for (uint32_t i = t; i < n_list; i += WS_BLOCK) {
+    for (uint32_t i = t; i < kTopkCap; i += WS_BLOCK) {
+        if (i % kTopkWaveCap >= n_list[i / kTopkWaveCap]) continue;  // past the end of that wave's stretch
         const uint64_t k = list[i];
         const uint32_t b = topk_bin(unkey32(static_cast<uint32_t>(k >> 32)), scale, a32, no_tail);
         if (b < bcut) {
@@ -202,29 +283,26 @@ __device__ __forceinline__ int topk_from_list(const float* __restrict__ x, const
         }
     }
     __syncthreads();  // sel[2] == kk now
-    // ascending id: bitonic sort of the kept entries, padded with the largest key to a power of two
-    uint32_t P = 2;
-    while (P < kk) P <<= 1;
-    for (uint32_t i = kk + t; i < P; i += WS_BLOCK) kept[i] = ~0ull;
+    // ascending id: every kept entry counts the kept ids below its own (ids are distinct, so the counts are the places).
+    // The ids go to an array of their own (the cut's keys are done with), padded to a multiple of 16 with ids that are
+    // below nobody's; all threads read the same 128-bit words one after the other, which LDS serves as broadcasts,
+    // four words in flight per round.
+    uint32_t* kid = reinterpret_cast<uint32_t*>(cut);
+    for (uint32_t i = t; i < ((kk + 15u) & ~15u); i += WS_BLOCK) kid[i] = i < kk ? static_cast<uint32_t>(kept[i] >> 32) : 0xffffffffu;
     __syncthreads();
-    for (uint32_t k2 = 2; k2 <= P; k2 <<= 1) {
-        for (uint32_t j = k2 >> 1; j > 0; j >>= 1) {
-            for (uint32_t q = t; q < (P >> 1); q += WS_BLOCK) {
-                const uint32_t i = ((q & ~(j - 1u)) << 1) | (q & (j - 1u)), l = i | j;
-                const uint64_t u = kept[i], w = kept[l];
-                const bool up = (i & k2) == 0;  // this pair sorts ascending
-                if (up ? (u > w) : (u < w)) {
-                    kept[i] = w;
-                    kept[l] = u;
-                }
-            }
-            __syncthreads();
-        }
-    }
     for (uint32_t i = t; i < kk; i += WS_BLOCK) {
-        const uint32_t id = static_cast<uint32_t>(kept[i] >> 32);
-        ids[i] = static_cast<int>(id);
-        vals[i] = x[id];  // the logit as it stands in the row (a key does not tell -0 from +0); never NaN here
+        const uint32_t id = kid[i];
+        uint32_t place = 0;
+        for (uint32_t j = 0; j < kk; j += 16u) {
+            uint4 o[4];
+#pragma unroll
+            for (uint32_t e = 0; e < 4u; ++e) o[e] = reinterpret_cast<const uint4*>(kid + j)[e];
+#pragma unroll
+            for (uint32_t e = 0; e < 4u; ++e)
+                place += (o[e].x < id ? 1u : 0u) + (o[e].y < id ? 1u : 0u) + (o[e].z < id ? 1u : 0u) + (o[e].w < id ? 1u : 0u);
+        }
+        ids[place] = static_cast<int>(id);
+        vals[place] = x[id];  // the logit as it stands in the row (a key does not tell -0 from +0); never NaN here
     }
     return 0;
 }
@@ -354,13 +432,14 @@ __device__ __forceinline__ bool topk_by_counts(const float* __restrict__ x, int 
 // The K largest logits of one row (x, n tokens) into ids / vals in ascending id order, ties at the cut to the lowest ids;
 // stats (unless null) = {max, sum exp((x - max) * inv_t)}. Every return is taken by the whole workgroup.
 __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
-    __shared__ uint32_t hist[4096];
+    __shared__ __align__(16) uint32_t hist[4096];  // also viewed as 64- and 128-bit words
     __shared__ uint64_t cand[ws::kTopkCap];
     __shared__ float red_f[WS_WAVES];
     __shared__ uint32_t red_u[WS_WAVES];
     __shared__ uint32_t s_sel[2];
     __shared__ uint32_t s_cnt[WS_WAVES];
-    __shared__ uint32_t s_n;
+    __shared__ uint32_t s_n;            // candidates of the cut's bin (count route)
+    __shared__ uint32_t s_wn[WS_WAVES];  // tokens listed by each wave in the first pass
     __shared__ uint64_t s_kmin;
     const uint32_t kk = static_cast<uint32_t>(K < n ? K : n);
 
@@ -387,6 +466,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
         a32 = bound * scale;
         for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
         if (threadIdx.x == 0) s_n = 0u;
+        if (threadIdx.x < WS_WAVES) s_wn[threadIdx.x] = 0u;
         __syncthreads();
         // For a short list (K up to a quarter of the list's room) the head of the row also says where the K-th largest
         // will roughly be: the bin that holds the sample's (2 K / n)-quantile, and a few tokens more. The first pass
@@ -421,10 +501,20 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
 
     // pass 1: max and sum exp((x - max) * inv_t), rescaled online per thread (and the bin counts, and the list)
     float m = -INFINITY, s = 0.f;
-    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, list_bin, cand, &s_n, m, s);
-    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, &s_n, m, s);
+    // with a bound in hand the sum is taken against the largest logit of the head of the row (the bound is 8 above it,
+    // the maximum between the two: terms up to e^(8 inv_t), which a float holds for temperatures above 1 / 8)
+    const float nan = __uint_as_float(0x7fc00000u);
+    const float ref = (counted && inv_t > 0.f && inv_t <= 8.f) ? bound - 8.f : nan;
+    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s);
+    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
     const float top = ws::block_max(m, red_f);
-    const float part = m > -INFINITY ? s * __expf((m - top) * inv_t) : 0.f;
+    if (ref == ref && !(top <= bound)) {  // uniform: the maximum beats the bound - the sum may have overflowed: once more, the other way
+        m = -INFINITY;
+        s = 0.f;
+        ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
+    }
+    const float from = (ref == ref && top <= bound) ? ref : m;  // what this thread's sum is relative to
+    const float part = m > -INFINITY ? s * __expf((from - top) * inv_t) : 0.f;
     const float sum = ws::block_sum(part, red_f);
     if (threadIdx.x == 0 && stats) {
         stats[0] = top;
@@ -434,12 +524,29 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
     __syncthreads();  // the counts are complete
 
     int counts_left = counted && top <= bound;  // uniform
-    if (counts_left && list_bin >= 0 && s_n >= kk && s_n <= ws::kTopkCap) {  // the K largest may all be on the list
-        __shared__ uint32_t s_list[4];
-        const int rc = ws::topk_from_list(x, cand, s_n, list_bin, kk, scale, a32, hist, red_u, s_list, ids, vals);
-        if (rc == 0) return;
-        __syncthreads();
-        counts_left = rc == 1;
+    if (counts_left && list_bin >= 0) {
+        uint32_t listed = 0;
+        bool fits = true;
+        for (int w = 0; w < WS_WAVES; ++w) {
+            listed += s_wn[w];
+            fits = fits && s_wn[w] <= ws::kTopkWaveCap;
+        }
+        if (listed >= kk && fits) {  // the K largest are all on the list
+            __shared__ uint32_t s_list[4];
+            const int rc = ws::topk_from_list(x, cand, s_wn, list_bin, kk, scale, a32, hist, red_u, s_list, ids, vals);
+            if (rc == 0) return;
+            __syncthreads();
+            counts_left = rc == 1;
+        }
+        if (counts_left) {
+            // the list fell short of K tokens, overflowed or does not reach the cut: only its bins were counted, so the
+            // row is counted in full now (the maximum and the normaliser are already out)
+            for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
+            __syncthreads();
+            float m2 = -INFINITY, s2 = 0.f;
+            ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, bound - 8.f, m2, s2);
+            __syncthreads();
+        }
     }
     if (counts_left) {
         const ws::TopkLds L{hist, cand, red_f, red_u, s_sel, s_cnt, &s_n, &s_kmin};
