@@ -2,7 +2,7 @@
 // Same names, argument lists and results as the reference kernels (kernels/shared/misc_kv_argmax_kv_store.h:32-42,
 // kernels/shared/sample_pick_set_tokens.h:15-21, 47-53, 60-105); one pass over the row with 128-bit loads:
 // the maximum (first index on ties, kernels/shared/block_argmax.h:16) and, where a probability is asked for,
-// sum exp(x - max) by an online rescaled sum instead of the reference's second pass
+// sum exp(x - max) by an online rescaled sum (rescaled once per 128-bit vector) instead of the reference's second pass
 // (kernels/shared/block_argmax_psum.h). NaN logits are never picked and add nothing to the sum.
 #pragma once
 
@@ -22,15 +22,70 @@ __device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
     __shared__ float red_s[WS_WAVES];
     Best b = {-INFINITY, 0};
     float s = 0.f;
-    for_each_f32(x, n, [&](int i, float v) {
-        if (v > b.v) {
-            if (WITH_SUM) s = s * __expf(b.v - v) + 1.f;
-            b.v = v;
-            b.i = i;
-        } else if (WITH_SUM && v > -INFINITY) {
-            s += __expf(v - b.v);
+    if (!WITH_SUM) {
+        for_each_f32(x, n, [&](int i, float v) {
+            if (v > b.v) {
+                b.v = v;
+                b.i = i;
+            }
+        });
+    } else {
+        auto one = [&](int i, float v) {
+            if (v > b.v) {
+                s = s * __expf(b.v - v) + 1.f;
+                b.v = v;
+                b.i = i;
+            } else if (v > -INFINITY) {
+                s += __expf(v - b.v);
+            }
+        };
+        // 128-bit loads on the aligned body of the row, kU per thread in flight and the next kU requested before these
+        // are looked at; the maximum is raised once per vector (first index on ties: indices rise along a thread's
+        // walk and only a strictly larger logit takes over), the four terms are added without a branch
+        constexpr float kLog2e = 1.4426950408889634f;
+        const int t = threadIdx.x;
+        int head = static_cast<int>(((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(x)) & 15u)) & 15u) >> 2);
+        if (head > n) head = n;
+        if (t < head) one(t, x[t]);
+        const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + head);
+        const int nv = (n - head) >> 2;
+        constexpr int kU = 4;
+        float4 cur[kU], nxt[kU];
+        auto fetch = [&](int j0, float4 (&q)[kU]) {
+#pragma unroll
+            for (int u = 0; u < kU; ++u) q[u] = xv[min(j0 + u * WS_BLOCK + t, nv - 1)];
+        };
+        if (nv > 0) fetch(0, cur);
+        for (int j0 = 0; j0 < nv; j0 += kU * WS_BLOCK) {
+            const bool more = j0 + kU * WS_BLOCK < nv;
+            if (more) fetch(j0 + kU * WS_BLOCK, nxt);
+#pragma unroll
+            for (int u = 0; u < kU; ++u) {
+                const int j = j0 + u * WS_BLOCK + t;
+                if (j >= nv) continue;
+                const float4 q = cur[u];
+                // NaN -> -inf (fmaxf returns the operand that is a number)
+                const float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
+                const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+                if (vm > b.v) {
+                    s *= __builtin_amdgcn_exp2f((b.v - vm) * kLog2e);  // no maximum yet (-inf): s is 0 and stays 0
+                    b.v = vm;
+                    b.i = head + 4 * j + (v[0] == vm ? 0 : (v[1] == vm ? 1 : (v[2] == vm ? 2 : 3)));
+                }
+                const float mk = fmaxf(b.v, -1.0e30f) * kLog2e;  // a row of -inf so far: every term is 2^-inf = 0, never inf - inf
+                float add = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) add += __builtin_amdgcn_exp2f(__fmaf_rn(v[e], kLog2e, -mk));
+                s += add;
+            }
+            if (more) {
+#pragma unroll
+                for (int u = 0; u < kU; ++u) cur[u] = nxt[u];
+            }
         }
-    });
+        const int i = head + 4 * nv + t;
+        if (i < n) one(i, x[i]);
+    }
     RowTop r;
     r.best = block_best(b, red_v, red_i);
     r.sum = 0.f;
