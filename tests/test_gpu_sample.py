@@ -296,7 +296,7 @@ def test_north_star_tile_full_size(mode):
 @pytest.mark.parametrize("mode", MODES)
 def test_cfg3_full_size(mode):
     c = gc.make_cfg3()
-    res, _ = run_case(c, 1, rows=range(0, 256, 2), expect_near=0.2, mode=mode)
+    res, _ = run_case(c, 1, rows=range(256), expect_near=0.2, mode=mode)  # every row of the batch
     print(res)
 
 
@@ -307,7 +307,7 @@ def test_cfg5_full_size():
     within top-k, no failure flag."""
     m = gc.pkg()
     c = gc.make_cfg5()
-    res, smp = run_case(c, 1, rows=range(0, 1024, 64), kept_cap=1024, mode=0)
+    res, smp = run_case(c, 1, rows=range(0, 1024, 16), kept_cap=1024, mode=0)
     print(res)
     tok = smp.token.cpu().numpy()
     nk = smp.n_kept.cpu().numpy()
