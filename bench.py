@@ -149,6 +149,7 @@ def run_workload(name, steps, warmup, check_rows):
 def reference_kernels(steps):
     """Launch times of the replacements of the reference's own kernels at the engine's shapes (vocab 151936): the greedy
     picks on 1 / 32 / 256 rows, topk_rows with the engine's two list sizes on 1 / 32 rows, the drafter's dflash_topk. Synthetic N(0, sigma 2) logits."""
+    import ctypes as C
     import torch
     import gpu_cases as gc
     m = gc.pkg()
@@ -185,6 +186,19 @@ def reference_kernels(steps):
     ids = torch.empty((16, 16), dtype=torch.int32, device="cuda:0")
     vals = torch.empty((16, 16), dtype=torch.float32, device="cuda:0")
     timed("dflash_topk k=16", 16, lambda: L.ws_dflash_topk(S(), P(x), V, V, 16, P(ids), P(vals), 16), 16 * (V * 4 + 16 * 8))
+    # the drafter's sampled pick (the "specsample" rule): q over the 32 largest logits + race draw, one row per sequence
+    for rows in (1, 8):
+        x = torch.randn(rows, V, device="cuda:0") * 2
+        ctl = torch.zeros(rows * m.CTL_WORDS, dtype=torch.int32, device="cuda:0")
+        qbuf = torch.zeros(rows * 72, dtype=torch.int32, device="cuda:0")
+        ri, da = m.RowIdx(), m.DSampArgs()
+        for i in range(rows):
+            ri.v[i] = i * m.CTL_WORDS
+            da.on[i], da.top_k[i], da.qoff[i] = 1, 20, 72 * i
+            da.inv_t[i], da.top_p[i], da.min_p[i] = 1.25, 0.95, 0.02
+            da.key_lo[i], da.key_hi[i] = 12345 + i, 77
+        timed("draft_sample_rows", rows,
+              lambda: L.ws_draft_sample_rows(S(), P(x), V, P(ctl), C.byref(ri), 0, None, C.byref(da), P(qbuf), rows), rows * V * 4)
     x = torch.randn(1, V, device="cuda:0") * 2
     tok = torch.empty(1, dtype=torch.int32, device="cuda:0")
     pr = torch.empty(1, dtype=torch.float32, device="cuda:0")

@@ -1,9 +1,9 @@
 // draft_sample_rows for gfx950: the draft distribution q of a draft-head row and the race draw coupled to the
 // target sampler (reference: kernels/spec_sample.hip:34-205, same arguments, control-area and q-buffer layout;
 // host statement of q: src/common/spec_sample.cpp:34-81).
-// One pass for {max, sum exp((x - max) * inv_t)} (NaN adds nothing, kernels/spec_sample.hip:63-66), the radix select
-// of ws_topk.h for the K = min(top_k, 32) largest logits (ties at the cut: lowest ids), then the serial part on one
-// thread in the reference's arithmetic: f32 probabilities and filters, double-precision race keys.
+// One pass for {max, sum exp((x - max) * inv_t)} (NaN adds nothing, kernels/spec_sample.hip:63-66) and the
+// K = min(top_k, 32) largest logits (ties at the cut: lowest ids) - the short-list route of ws_topk.h -, then one wave
+// finishes in the reference's arithmetic: f32 probabilities and filters in the reference's order, double-precision race keys.
 #pragma once
 
 #include "ws_common.h"
@@ -24,12 +24,9 @@ struct DSampArgs {
 extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     draft_sample_rows(const float* x, int n, int* ctl_all, RowIdx area, int r, const int* map, DSampArgs a, int* qbuf) {
     constexpr int QMAX = 32;
-    __shared__ uint32_t hist[4096];
-    __shared__ float red_f[WS_WAVES];
-    __shared__ uint32_t red_u[WS_WAVES];
-    __shared__ uint32_t s_sel[2];
     __shared__ int s_id[QMAX];
     __shared__ float s_lg[QMAX];
+    __shared__ float s_stats[2];
     const int b = blockIdx.x;
     if (a.on[b] == 0) return;
     int* c = ctl_all + area.v[b];
@@ -39,44 +36,32 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     int K = (tk > 0 && tk < QMAX) ? tk : QMAX;
     if (K > n) K = n;
     const float inv_t = a.inv_t[b];
-
-    float m = -INFINITY, s = 0.f;
-    ws::for_each_f32(x, n, [&](int, float v) {
-        if (v > m) {
-            s = s * __expf((m - v) * inv_t) + 1.f;
-            m = v;
-        } else if (v > -INFINITY) {
-            s += __expf((v - m) * inv_t);
-        }
-    });
-    const float top = ws::block_max(m, red_f);
-    const float sum = ws::block_sum(m > -INFINITY ? s * __expf((m - top) * inv_t) : 0.f, red_f);
-
-    uint32_t thr, need;
-    ws::radix_kth(x, n, static_cast<uint32_t>(K), hist, red_u, s_sel, thr, need);
-    ws::select_in_id_order(x, n, thr, need, red_u, [&](uint32_t o, int i, float v) {
-        s_id[o] = i;
-        s_lg[o] = v;
-    });
+    // one pass over the row: {max, sum exp((x - max) * inv_t)} and the K largest logits in id order, ties at the cut to
+    // the lowest ids (the short-list route of topk_rows)
+    ws::topk_one_row(x, n, K, inv_t, s_id, s_lg, s_stats);
     __syncthreads();
-    if (threadIdx.x != 0) return;
-
-    int id[QMAX];
-    float lg[QMAX], p[QMAX];
-    for (int i = 0; i < K; ++i) {
-        id[i] = map ? map[s_id[i]] : s_id[i];
-        lg[i] = s_lg[i];
+    const float top = s_stats[0], sum = s_stats[1];
+    if (threadIdx.x >= 64) return;
+    // ---- the rest on one wave, lane i = candidate i (QMAX = 32 <= 64 lanes). What the reference's single thread does in
+    // a fixed order - the running float sums of the filters - is done in that order by every lane for itself, with the
+    // candidates' values read from their lanes; what is independent per candidate (its place in the order, its
+    // probability, its race key with a double-precision logarithm) is done by the candidate's lane.
+    const int lane = threadIdx.x;
+    const bool live = lane < K;
+    const int my_id = live ? (map ? map[s_id[lane]] : s_id[lane]) : 0x7fffffff;
+    const float my_lg = live ? s_lg[lane] : -INFINITY;
+    int place = 0;  // logit desc, (mapped) id asc, then the position in the list
+    for (int j = 0; j < K; ++j) {
+        const float lj = __shfl(my_lg, j);
+        const int ij = __shfl(my_id, j);
+        place += (lj > my_lg || (lj == my_lg && (ij < my_id || (ij == my_id && j < lane)))) ? 1 : 0;
     }
-    for (int i = 1; i < K; ++i)  // logit desc, (mapped) id asc
-        for (int j = i; j > 0 && (lg[j - 1] < lg[j] || (lg[j - 1] == lg[j] && id[j - 1] > id[j])); --j) {
-            const float tl = lg[j - 1];
-            lg[j - 1] = lg[j];
-            lg[j] = tl;
-            const int ti = id[j - 1];
-            id[j - 1] = id[j];
-            id[j] = ti;
-        }
-    for (int i = 0; i < K; ++i) p[i] = __fdiv_rn(expf(__fmul_rn(__fsub_rn(lg[i], top), inv_t)), sum);
+    // lane r takes the candidate of place r
+    const int dst = (live ? place : lane) << 2;
+    const int id = __builtin_amdgcn_ds_permute(dst, my_id);
+    const float lg = __int_as_float(__builtin_amdgcn_ds_permute(dst, __float_as_int(my_lg)));
+    float p = live ? __fdiv_rn(expf(__fmul_rn(__fsub_rn(lg, top), inv_t)), sum) : 0.f;
+    auto p_of = [&](int j) { return __shfl(p, j); };
     int nk = K;
     const bool closed = tk > 0 && tk <= K;
     if (closed) nk = tk;
@@ -85,11 +70,11 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
         float z = 1.f;
         if (closed) {
             z = 0.f;
-            for (int i = 0; i < nk; ++i) z = __fadd_rn(z, p[i]);
+            for (int i = 0; i < nk; ++i) z = __fadd_rn(z, p_of(i));
         }
         float cum = 0.f;
         for (int j = 0; j < nk; ++j) {
-            cum = __fadd_rn(cum, __fdiv_rn(p[j], z));
+            cum = __fadd_rn(cum, __fdiv_rn(p_of(j), z));
             if (cum >= top_p) {
                 nk = j + 1;
                 break;
@@ -98,32 +83,42 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     }
     const float min_p = a.min_p[b];
     if (min_p > 0.f && nk > 0) {
-        const float floor_p = __fmul_rn(min_p, p[0]);
+        const float floor_p = __fmul_rn(min_p, p_of(0));
         int j = 0;
-        while (j < nk && p[j] >= floor_p) ++j;
+        while (j < nk && p_of(j) >= floor_p) ++j;
         nk = j > 1 ? j : 1;
     }
     float z = 0.f;
-    for (int i = 0; i < nk; ++i) z = __fadd_rn(z, p[i]);
-    for (int i = 0; i < nk; ++i) p[i] = __fdiv_rn(p[i], z);
-    // race: argmin E(v) / q(v), E(v) = -ln(1 - U(key, v)) (src/common/spec_sample.cpp:83-101)
+    for (int i = 0; i < nk; ++i) z = __fadd_rn(z, p_of(i));
+    p = lane < nk ? __fdiv_rn(p, z) : 0.f;
+    // race: argmin E(v) / q(v), E(v) = -ln(1 - U(key, v)) (src/common/spec_sample.cpp:83-101); the earlier candidate on
+    // equal keys, candidate 0 when none has a probability
     const uint64_t rkey = (static_cast<uint64_t>(a.key_hi[b]) << 32) | a.key_lo[b];
-    int pick = 0;
-    double best = __longlong_as_double(0x7FF0000000000000ll);
-    for (int i = 0; i < nk; ++i) {
-        if (!(p[i] > 0.f)) continue;
-        const uint64_t h = ws::mix64(rkey + (static_cast<uint64_t>(static_cast<uint32_t>(id[i])) + 1ull) * 0xE7037ED1A0B428DBull);
-        const double k = -log(1.0 - ws::unit53(h)) / static_cast<double>(p[i]);
-        if (k < best) {
-            best = k;
-            pick = i;
+    const double inf = __longlong_as_double(0x7FF0000000000000ll);
+    double k = inf;
+    if (lane < nk && p > 0.f) {
+        const uint64_t h = ws::mix64(rkey + (static_cast<uint64_t>(static_cast<uint32_t>(id)) + 1ull) * 0xE7037ED1A0B428DBull);
+        k = -log(1.0 - ws::unit53(h)) / static_cast<double>(p);
+    }
+    int pick = lane;
+#pragma unroll
+    for (int o = 32; o; o >>= 1) {
+        const double ko = __shfl_xor(k, o);
+        const int po = __shfl_xor(pick, o);
+        if (ko < k || (ko == k && po < pick)) {
+            k = ko;
+            pick = po;
         }
     }
-    c[16 + r] = id[pick];
+    if (!(k < inf)) pick = 0;
+    const int picked = __shfl(id, pick);
     int* q = qbuf + a.qoff[b];
-    q[0] = nk;
-    for (int i = 0; i < nk; ++i) {
-        q[1 + i] = id[i];
-        q[1 + QMAX + i] = __float_as_int(p[i]);
+    if (lane == 0) {
+        c[16 + r] = picked;
+        q[0] = nk;
+    }
+    if (lane < nk) {
+        q[1 + lane] = id;
+        q[1 + QMAX + lane] = __float_as_int(p);
     }
 }
