@@ -206,6 +206,50 @@ def reference_kernels(steps):
     return out
 
 
+def spec_verify_workload(steps, warmup):
+    """configs[3]: classic speculative verification, 32 sequences x 9 positions x 151936 fp32 probabilities (target =
+    softmax of N(0, sigma 2) logits, draft = softmax of the same logits mixed 70 / 30 with fresh ones, draft ids drawn from
+    the draft distribution), one ws_spec_verify_classic call per step. Necessary bytes: the two gathers per tested draft
+    and, per sequence, the rejected position's p and q rows (or the last position's p row when every draft passed)."""
+    import ctypes as C
+    import torch
+    import gpu_cases as gc
+    m = gc.pkg()
+    n_seq, n_pos, V = 32, 9, 151936
+    g = torch.Generator(device="cuda:0").manual_seed(312)
+    tl = torch.randn((n_seq, n_pos, V), device="cuda:0", generator=g) * 2
+    dl = 0.7 * tl + 0.3 * torch.randn((n_seq, n_pos, V), device="cuda:0", generator=g) * 2
+    p, q = torch.softmax(tl, -1).contiguous(), torch.softmax(dl, -1).contiguous()
+    del tl, dl
+    draft = torch.multinomial(q[:, :n_pos - 1].reshape(-1, V), 1, generator=g).reshape(n_seq, n_pos - 1).to(torch.int32).contiguous()
+    seed = (99 + torch.arange(n_seq, device="cuda:0", dtype=torch.int64) * 104729).contiguous()
+    step0 = torch.arange(n_seq, device="cuda:0", dtype=torch.int64) * 7
+    out = torch.full((n_seq, n_pos), -1, dtype=torch.int32, device="cuda:0")
+    nacc = torch.empty(n_seq, dtype=torch.int32, device="cuda:0")
+    flags = torch.empty(n_seq, dtype=torch.int32, device="cuda:0")
+    P = m._p
+    v = m.SpecVerify(P(p), P(q), P(draft), n_seq, n_pos, V, P(seed), P(step0), m.RNG_PHILOX, P(out), P(nacc), P(flags), None, 0, 0.0)
+    L, S = m.lib(), m._stream
+    for _ in range(warmup):
+        m.check(L.ws_spec_verify_classic(S(), C.byref(v)), "ws_spec_verify_classic")
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        L.ws_spec_verify_classic(S(), C.byref(v))
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    na = nacc.cpu().numpy()
+    tested = int((na + (na < n_pos - 1)).sum())
+    nbytes = tested * 8 + int(((na < n_pos - 1) * 2 * V * 4 + (na == n_pos - 1) * V * 4).sum()) + n_seq * (n_pos * 4 + 8)
+    return {"workload": "cfg4", "sequences": n_seq, "positions": n_pos, "vocab": V, "dtype": "f32", "kernel": "ws::spec_verify_kernel",
+            "ms_per_step": ms, "kernel_ms": ms, "sequences_per_s": n_seq / (ms * 1e-3), "mean_accepted_drafts": float(na.mean()),
+            "algorithmic_MB": nbytes / 1e6, "achieved_GBs": nbytes / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "device_near_flags": int((flags.cpu().numpy() != 0).sum())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -251,6 +295,7 @@ def main():
             if w != a.workload:
                 _, r = run_workload(w, max(20, a.steps // 4), 5, 4)
                 also.append(r)
+        also.append(spec_verify_workload(max(20, a.steps // 4), 5))
     cpu = None if a.no_cpu else cpu_baseline(c)
     ab = main_res["algorithmic_MB"] * 1e6
     out = {

@@ -40,7 +40,31 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     int32_t* out = A.out_tokens + static_cast<size_t>(s) * P;
     const uint64_t seed = A.seed[s], step0 = A.step0[s];
 
-    if (t == 0) {  // accept chain
+    if (P - 1u <= 64u) {
+        // accept chain, every draft at once: lane j of wave 0 fetches p_j(d_j), q_j(d_j) and tests its draft (one trip to
+        // memory instead of one per draft); the chain stops at the first lane that rejects
+        if (t < 64u) {
+            const bool has = t + 1u < P;
+            int32_t d = 0;
+            bool ok = false, near = false;
+            if (has) {
+                d = dr[t];
+                const double pj = p[static_cast<size_t>(t) * V + d], qj = q[static_cast<size_t>(t) * V + d];
+                const double lhs = batch_uniform(A.rng, seed, s, step0 + t, 0) * qj;
+                near = fabs(lhs - pj) < A.tol * pj;
+                ok = lhs < pj;
+            }
+            const uint64_t rejects = __ballot(!ok);  // lanes past the last draft reject: there is always one
+            const uint32_t j = static_cast<uint32_t>(__ffsll(static_cast<long long>(rejects)) - 1);
+            const uint64_t tested = j >= 63u ? ~0ull : (2ull << j) - 1ull;  // drafts 0..j were looked at (j = P - 1: none there)
+            const uint64_t nears = __ballot(near) & tested;
+            if (t < j) out[t] = d;
+            if (t == 0) {
+                s_u[0] = j;
+                s_u[1] = nears ? kSpecNear : 0u;
+            }
+        }
+    } else if (t == 0) {  // accept chain, draft by draft
         uint32_t j = 0, fl = 0;
         for (; j + 1 < P; ++j) {
             const int32_t d = dr[j];
@@ -64,10 +88,37 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     double total = 0;
     for (int attempt = 0; attempt < 2; ++attempt) {
         // weights in id order: step k covers ids [256k, 256k + 256), lane l the four ids 256k + 4l ..
-        for (uint32_t k = w; k < n_steps; k += WS_WAVES) {
+        const bool aligned = (reinterpret_cast<uintptr_t>(pr) & 15u) == 0 && (reinterpret_cast<uintptr_t>(qr) & 15u) == 0;
+        // whole aligned steps, kS of a wave at a time: their loads go out together (one step at a time is one trip to
+        // memory per step and wave)
+        constexpr uint32_t kS = 4;
+        const uint32_t whole = aligned ? V >> 8 : 0u;  // steps of 256 ids that lie inside the row
+        uint32_t k_next = w;
+        for (; k_next + (kS - 1u) * WS_WAVES < whole; k_next += kS * WS_WAVES) {
+            float4 a[kS], b[kS];
+#pragma unroll
+            for (uint32_t u = 0; u < kS; ++u) {
+                const uint32_t i = ((k_next + u * WS_WAVES) << 8) + 4u * l;
+                a[u] = *reinterpret_cast<const float4*>(pr + i);
+                b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (!from_p) b[u] = *reinterpret_cast<const float4*>(qr + i);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kS; ++u) {
+                const float r0 = a[u].x - b[u].x, r1 = a[u].y - b[u].y, r2 = a[u].z - b[u].z, r3 = a[u].w - b[u].w;
+                double acc = 0;
+                acc += r0 > 0.f ? static_cast<double>(r0) : 0.0;
+                acc += r1 > 0.f ? static_cast<double>(r1) : 0.0;
+                acc += r2 > 0.f ? static_cast<double>(r2) : 0.0;
+                acc += r3 > 0.f ? static_cast<double>(r3) : 0.0;
+                acc = wave_sum(acc);
+                if (l == 0) step_sum[k_next + u * WS_WAVES] = acc;
+            }
+        }
+        for (uint32_t k = k_next; k < n_steps; k += WS_WAVES) {
             const uint32_t i = (k << 8) + 4u * l;
             double acc = 0;
-            if (i + 3 < V && (reinterpret_cast<uintptr_t>(pr) & 15u) == 0 && (reinterpret_cast<uintptr_t>(qr) & 15u) == 0) {
+            if (i + 3 < V && aligned) {
                 const float4 a = *reinterpret_cast<const float4*>(pr + i);
                 float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (!from_p) b = *reinterpret_cast<const float4*>(qr + i);
