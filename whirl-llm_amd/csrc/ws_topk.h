@@ -122,7 +122,8 @@ __device__ __forceinline__ uint32_t topk_bin(float v, float scale, float a32, fl
 // counted, and they are put on the list as keys (wave w: list[w * kTopkWaveCap ...], n_list[w] of them): when the list ends up holding at least K tokens, the K largest are
 // among them, the counts of those bins are complete and no further pass over the row is needed. (One LDS atomic per
 // token is what bounds a counting pass; a listing pass has a few per thousand tokens.)
-template <bool COUNT>
+// SUM false: only the maximum is tracked (a caller that wants no normaliser: the exponentials are a third of the pass).
+template <bool COUNT, bool SUM = true>
 __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist,
                                                 int list_bin, uint64_t* list, uint32_t* n_list, float ref, float& m, float& s) {
     const float tail = static_cast<float>(kTopkTail + lane_id());
@@ -143,7 +144,9 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
         }
     };
     auto one = [&](int i, float v) {
-        if (fixed) {
+        if (!SUM) {
+            if (v > m) m = v;
+        } else if (fixed) {
             if (v > -INFINITY) {  // not for NaN either
                 m = fmaxf(m, v);
                 s += __builtin_amdgcn_exp2f(__fmaf_rn(v, k2, -rk));
@@ -187,7 +190,7 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
         const float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
         const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
         float mk = rk;
-        if (fixed) {
+        if (fixed || !SUM) {
             m = fmaxf(m, vm);
         } else {
             if (vm > m) {
@@ -196,10 +199,12 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
             }
             mk = fmaxf(m, -1.0e30f) * k2;  // a row of -inf so far: every term below is 2^-inf = 0, never inf - inf
         }
-        float add = 0.f;
+        if (SUM) {
+            float add = 0.f;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) add += __builtin_amdgcn_exp2f(__fmaf_rn(v[e], k2, -mk));
-        s += add;
+            for (int e = 0; e < 4; ++e) add += __builtin_amdgcn_exp2f(__fmaf_rn(v[e], k2, -mk));
+            s += add;
+        }
         if (COUNT) {
             if (!listed) {  // uniform
 #pragma unroll
@@ -431,6 +436,7 @@ __device__ __forceinline__ bool topk_by_counts(const float* __restrict__ x, int 
 
 // The K largest logits of one row (x, n tokens) into ids / vals in ascending id order, ties at the cut to the lowest ids;
 // stats (unless null) = {max, sum exp((x - max) * inv_t)}. Every return is taken by the whole workgroup.
+template <bool SUM = true>
 __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
     __shared__ __align__(16) uint32_t hist[4096];  // also viewed as 64- and 128-bit words
     __shared__ uint64_t cand[ws::kTopkCap];
@@ -505,10 +511,10 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
     // the maximum between the two: terms up to e^(8 inv_t), which a float holds for temperatures above 1 / 8)
     const float nan = __uint_as_float(0x7fc00000u);
     const float ref = (counted && inv_t > 0.f && inv_t <= 8.f) ? bound - 8.f : nan;
-    if (counted) ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s);
-    else ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
+    if (counted) ws::topk_first_pass<true, SUM>(x, n, inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s);
+    else ws::topk_first_pass<false, SUM>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
     const float top = ws::block_max(m, red_f);
-    if (ref == ref && !(top <= bound)) {  // uniform: the maximum beats the bound - the sum may have overflowed: once more, the other way
+    if (SUM && ref == ref && !(top <= bound)) {  // uniform: the maximum beats the bound - the sum may have overflowed: once more, the other way
         m = -INFINITY;
         s = 0.f;
         ws::topk_first_pass<false>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
@@ -544,7 +550,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
             for (int b = threadIdx.x; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
             __syncthreads();
             float m2 = -INFINITY, s2 = 0.f;
-            ws::topk_first_pass<true>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, bound - 8.f, m2, s2);
+            ws::topk_first_pass<true, false>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, bound - 8.f, m2, s2);
             __syncthreads();
         }
     }
@@ -579,7 +585,7 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK) dflash_topk(const float* 
     const size_t row = blockIdx.x;
     ids += row * k;
     vals += row * k;
-    ws::topk_one_row(x + row * ld, n, k, 1.f, ids, vals, nullptr);
+    ws::topk_one_row<false>(x + row * ld, n, k, 1.f, ids, vals, nullptr);  // no normaliser asked for
     __syncthreads();  // the winners are in ids / vals, in id order
     const int kk = k < n ? k : n;
     if (threadIdx.x >= 64) return;
