@@ -56,6 +56,39 @@ def test_draft_sample_rows_support_probabilities_and_draw():
         assert hc[b * 64 + 16 + r] == lib.wo_sample_race_q(C.byref(got), keys[b])
 
 
+def test_draft_sample_rows_seeded_sweep():
+    """Random vocabulary sizes (down to fewer tokens than candidates), filters and temperatures, with logits rounded to
+    a quarter so that many tie (ties: lowest id first, src/common/spec_sample.cpp:43-50): ids and count of q exact,
+    probabilities to 1e-4, the draw equal to the host race over the written q."""
+    m = gc.pkg()
+    lib = wo.load("oracle")
+    rng = np.random.default_rng(302)
+    for case in range(10):
+        n = int(rng.choice([20, 33, 1000, 4096, 5000, 50000, 151936]))
+        rows, r = 4, int(rng.integers(0, 8))
+        x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
+        if case % 2:
+            x = np.round(x * 4) / 4
+        tks = [int(v) for v in rng.choice([0, 1, 3, 20, 32, 40], rows)]
+        tps = [float(v) for v in rng.choice([1.0, 0.95, 0.5], rows)]
+        mps = [float(v) for v in rng.choice([0.0, 0.05, 0.3], rows)]
+        its = [float(1 / rng.uniform(0.3, 1.5)) for _ in range(rows)]
+        keys = [lib.wo_race_base(int(rng.integers(1, 1 << 40)), int(rng.integers(0, 1000))) for _ in range(rows)]
+        dx = torch.from_numpy(x).to(DEV)
+        ctl = torch.zeros(rows * 64, dtype=torch.int32, device=DEV)
+        qb = torch.zeros(rows * m.Q_WORDS, dtype=torch.int32, device=DEV)
+        args = [dict(top_k=tks[b], qoff=b * m.Q_WORDS, inv_t=its[b], top_p=tps[b], min_p=mps[b], key=keys[b]) for b in range(rows)]
+        m.draft_sample_rows(dx, ctl, [64 * b for b in range(rows)], r, args, qb)
+        hc, hq = ctl.cpu().numpy(), qb.cpu().numpy()
+        for b in range(rows):
+            want = host_q(lib, x[b], np.float32(its[b]), tks[b], tps[b], mps[b])
+            got = wo.QDist()
+            lib.wo_q_from_words(wo._ptr(np.ascontiguousarray(hq[b * m.Q_WORDS:(b + 1) * m.Q_WORDS])), C.byref(got))
+            assert got.n == want.n and list(got.id[:got.n]) == list(want.id[:want.n]), (case, b, n, tks[b])
+            np.testing.assert_allclose(np.array(got.p[:got.n]), np.array(want.p[:want.n]), rtol=1e-4, atol=1e-7)
+            assert hc[b * 64 + 16 + r] == lib.wo_sample_race_q(C.byref(got), keys[b]), (case, b)
+
+
 def test_draft_sample_rows_nan_map_and_skips():
     m = gc.pkg()
     lib = wo.load("oracle")
