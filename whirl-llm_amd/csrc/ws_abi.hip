@@ -271,7 +271,15 @@ int ws_adjust_rows(void* stream, const ws_adjust* b) {
     a.allow_stride = b->allow_stride;
     a.out = b->out;
     a.out_stride = b->out_stride;
-    hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows), dim3(WS_BLOCK), ws::kAdjustLdsIds * sizeof(int32_t), S(stream), a);
+    a.lds_bytes = ws::kAdjustLds;
+    static bool adjust_attr_set = false;  // raising the dynamic LDS limit is per function, once per process
+    if (!adjust_attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::adjust_rows_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(ws::kAdjustLds));
+        if (e != hipSuccess) return static_cast<int>(e);
+        adjust_attr_set = true;
+    }
+    hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows), dim3(WS_BLOCK), ws::kAdjustLds, S(stream), a);
     return done();
 }
 

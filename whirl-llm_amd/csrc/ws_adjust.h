@@ -1,16 +1,18 @@
 // adjust_rows: a penalised fp32 copy of logits rows, for callers that want the adjusted logits themselves (a top-k of
 // them, a full-row download). Same order of operations as the batched sampler: NaN and masked-out -> -inf, bias values
 // of an id added one by one in listed order, repetition (x > 0 ? x / rep : x * rep), then x -= freq * count + pres,
-// every operation rounded to float. One workgroup per row; the row is copied once, then the touched tokens are patched
-// by the thread that holds the first list entry of their id (a quadratic scan of the two lists: they are short next to
-// the vocabulary, and this kernel is not on the sampler's hot path).
+// every operation rounded to float. One workgroup per row; the row is copied once, then the touched tokens are patched.
+// The usual way, as in the batched sampler: an LDS bitmap of the ids the lists name, a popcount prefix per word (rank of
+// an id = perfect hash), per rank the history count and the index of the first bias entry by LDS atomics, then one
+// thread per touched token. Lists too long for the rank tables (LDS left after the bitmap / 8 bytes per entry) are
+// patched by the thread that holds the first list entry of an id, which scans both lists (quadratic).
 #pragma once
 
 #include "ws_common.h"
 
 namespace ws {
 
-constexpr uint32_t kAdjustLdsIds = 15360;  // list entries staged in LDS (60 KiB)
+constexpr uint32_t kAdjustLds = 152u * 1024u;  // dynamic LDS of the kernel
 
 struct AdjustArgs {
     const void* logits;
@@ -29,6 +31,7 @@ struct AdjustArgs {
     uint64_t allow_stride;
     float* out;
     uint64_t out_stride;
+    uint32_t lds_bytes;
 };
 
 __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
@@ -50,10 +53,82 @@ __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
     const int32_t* bias_ids = A.bias_ids + b0;
     const float* bias_vals = A.bias_vals + b0;
     const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
-    // both lists side by side in LDS (bias ids first), when they fit: every thread scans them several times
-    extern __shared__ int32_t staged[];
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t red_u[WS_WAVES];
     const uint32_t n_all = nb + nh;
-    const bool in_lds = n_all <= kAdjustLdsIds;
+    if (n_all == 0) return;
+    const uint32_t nW = (V + 31u) >> 5;
+    const uint32_t tab_off = (nW * 6u + 15u) & ~15u;  // bitmap words, 16-bit prefixes, then the rank tables
+    if (tab_off < A.lds_bytes && n_all <= (A.lds_bytes - tab_off) / 8u && n_all <= 65535u) {  // uniform
+        uint32_t* touched = reinterpret_cast<uint32_t*>(lds);
+        uint16_t* wprefix = reinterpret_cast<uint16_t*>(lds + nW * 4u);
+        uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + tab_off);  // low 20 bits: history count, high 12: bias entries
+        uint32_t* first = cnt + n_all;                               // index of the id's first bias entry
+        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
+        __syncthreads();
+        for (uint32_t e = t; e < n_all; e += WS_BLOCK) {
+            const uint32_t id = static_cast<uint32_t>(e < nb ? bias_ids[e] : hist[e - nb]);
+            if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
+        }
+        __syncthreads();
+        const uint32_t chunk = (nW + WS_BLOCK - 1u) / WS_BLOCK;
+        const uint32_t w0 = min(t * chunk, nW), w1 = min(w0 + chunk, nW);
+        uint32_t local = 0;
+        for (uint32_t w = w0; w < w1; ++w) local += __popc(touched[w]);
+        uint32_t n_uniq;
+        uint32_t run = block_excl_scan(local, red_u, &n_uniq);
+        const uint32_t run0 = run;
+        for (uint32_t w = w0; w < w1; ++w) {
+            wprefix[w] = static_cast<uint16_t>(run);
+            run += __popc(touched[w]);
+        }
+        for (uint32_t r = t; r < n_uniq; r += WS_BLOCK) {
+            cnt[r] = 0u;
+            first[r] = 0xffffffffu;
+        }
+        __syncthreads();
+        auto rank_of_id = [&](uint32_t id) { return static_cast<uint32_t>(wprefix[id >> 5]) + __popc(touched[id >> 5] & ((1u << (id & 31u)) - 1u)); };
+        for (uint32_t e = t; e < n_all; e += WS_BLOCK) {
+            const uint32_t id = static_cast<uint32_t>(e < nb ? bias_ids[e] : hist[e - nb]);
+            if (id >= V) continue;
+            const uint32_t r = rank_of_id(id);
+            if (e < nb) {
+                atomicMin(&first[r], e);
+                atomicAdd(&cnt[r], 1u << 20);
+            } else {
+                atomicAdd(&cnt[r], 1u);
+            }
+        }
+        __syncthreads();
+        // every thread walks its words of the bitmap: one touched token per set bit, ranks in step
+        uint32_t r = run0;
+        for (uint32_t w = w0; w < w1; ++w) {
+            uint32_t bits = touched[w];
+            while (bits) {
+                const uint32_t id = (w << 5) + static_cast<uint32_t>(__ffs(bits)) - 1u;
+                bits &= bits - 1u;
+                const uint32_t cw = cnt[r], count = cw & 0xfffffu;
+                float x = out[id];
+                if (cw >> 20) {  // the bias values of this id, added one by one in listed order, starting at its first entry
+                    uint32_t j = first[r];
+                    x = __fadd_rn(x, bias_vals[j]);
+                    if ((cw >> 20) > 1u)
+                        for (++j; j < nb; ++j)
+                            if (static_cast<uint32_t>(bias_ids[j]) == id) x = __fadd_rn(x, bias_vals[j]);
+                }
+                if (count) {
+                    x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                    x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(count)), pres));
+                }
+                out[id] = x;
+                ++r;
+            }
+        }
+        return;
+    }
+    // both lists side by side in LDS (bias ids first), when they fit: every thread scans them several times
+    int32_t* staged = reinterpret_cast<int32_t*>(lds);
+    const bool in_lds = n_all <= A.lds_bytes / 4u;
     if (in_lds) {
         for (uint32_t e = t; e < n_all; e += WS_BLOCK) staged[e] = e < nb ? bias_ids[e] : hist[e - nb];
         __syncthreads();
