@@ -140,6 +140,39 @@ def test_topk_rows_cold_temperature_and_crowded_stretch(rows5):
             assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1], (K, inv_t, r, stats[r], ws_)
 
 
+def test_topk_rows_seeded_sweep():
+    """Random row lengths (whole vectors or not, so rows after the first are not 16-byte aligned), list sizes, temperatures
+    and contents - continuous, rounded to a quarter (ties at the cut), with -inf and NaN stretches, with an outlier far
+    above the head of the row - against a stable sort by (value desc, id asc) and a double-precision normaliser."""
+    m = gpu_cases.pkg()
+    rng = np.random.default_rng(303)
+    for case in range(24):
+        n = int(rng.choice([37, 4096, 4099, 20000, 65536, 151936, 151937]))
+        K = int(rng.choice([1, 7, 64, 256, 512, 513, 3000]))
+        inv_t = float(rng.choice([0.5, 1.0, 1.25, 3.0, 9.0]))
+        x = (rng.standard_normal((3, n)) * rng.choice([0.5, 2.0, 6.0])).astype(np.float32)
+        kind = case % 4
+        if kind == 1:
+            x = np.round(x * 4) / 4
+        elif kind == 2:
+            x[0, rng.random(n) < 0.9] = -np.inf
+            x[1, rng.random(n) < 0.3] = np.nan
+        elif kind == 3:
+            x[:, int(rng.integers(n // 2, n))] += 40.0
+        ids, vals, stats = (a.cpu().numpy() for a in m.topk_rows(torch.from_numpy(x).to(DEV), K, inv_t))
+        kk = min(K, n)
+        for r in range(3):
+            xr = np.where(np.isnan(x[r]), -np.inf, x[r]).astype(np.float32)
+            order = np.lexsort((np.arange(n), -xr.astype(np.float64)))[:kk]
+            assert np.array_equal(ids[r, :kk], np.sort(order)), (case, r, n, K, kind)
+            assert np.array_equal(vals[r, :kk], xr[ids[r, :kk]]), (case, r, n, K, kind)
+            top = xr.max()
+            assert stats[r, 0] == top, (case, r)
+            if np.isfinite(top):
+                want = np.exp((xr.astype(np.float64) - float(top)) * float(np.float32(inv_t))).sum()
+                assert abs(stats[r, 1] - want) <= 2e-6 * want, (case, r, n, K, inv_t, stats[r, 1], want)
+
+
 def test_topk_rows_ties_at_the_cut_keep_lowest_ids():
     m = gpu_cases.pkg()
     n, K = 5000, 7

@@ -30,19 +30,26 @@ __device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
             }
         });
     } else {
+        // Every term is 2^(fma(v, log2 e, -mk)) with mk the ROUNDED product maximum * log2 e: one instruction for the
+        // exponent, all terms of a thread off by one common factor 2^(maximum * log2 e - mk), which is taken out at the
+        // end (an fma gives that residue exactly); when the maximum rises, mk moves with it and s is rescaled by 2^(old - new)
+        constexpr float kLog2e = 1.4426950408889634f;
+        float mk = -1.0e30f;  // no maximum yet: every term is 2^-inf = 0, never inf - inf
+        auto raise = [&](float to, int at) {
+            const float mk_new = to * kLog2e;
+            s *= __builtin_amdgcn_exp2f(mk - mk_new);
+            b.v = to;
+            b.i = at;
+            mk = mk_new;
+        };
         auto one = [&](int i, float v) {
-            if (v > b.v) {
-                s = s * __expf(b.v - v) + 1.f;
-                b.v = v;
-                b.i = i;
-            } else if (v > -INFINITY) {
-                s += __expf(v - b.v);
-            }
+            v = fmaxf(v, -INFINITY);  // NaN -> -inf
+            if (v > b.v) raise(v, i);
+            s += __builtin_amdgcn_exp2f(__fmaf_rn(v, kLog2e, -mk));
         };
         // 128-bit loads on the aligned body of the row, kU per thread in flight and the next kU requested before these
         // are looked at; the maximum is raised once per vector (first index on ties: indices rise along a thread's
         // walk and only a strictly larger logit takes over), the four terms are added without a branch
-        constexpr float kLog2e = 1.4426950408889634f;
         const int t = threadIdx.x;
         int head = static_cast<int>(((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(x)) & 15u)) & 15u) >> 2);
         if (head > n) head = n;
@@ -67,12 +74,7 @@ __device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
                 // NaN -> -inf (fmaxf returns the operand that is a number)
                 const float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
                 const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-                if (vm > b.v) {
-                    s *= __builtin_amdgcn_exp2f((b.v - vm) * kLog2e);  // no maximum yet (-inf): s is 0 and stays 0
-                    b.v = vm;
-                    b.i = head + 4 * j + (v[0] == vm ? 0 : (v[1] == vm ? 1 : (v[2] == vm ? 2 : 3)));
-                }
-                const float mk = fmaxf(b.v, -1.0e30f) * kLog2e;  // a row of -inf so far: every term is 2^-inf = 0, never inf - inf
+                if (vm > b.v) raise(vm, head + 4 * j + (v[0] == vm ? 0 : (v[1] == vm ? 1 : (v[2] == vm ? 2 : 3))));
                 float add = 0.f;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) add += __builtin_amdgcn_exp2f(__fmaf_rn(v[e], kLog2e, -mk));
@@ -85,6 +87,7 @@ __device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
         }
         const int i = head + 4 * nv + t;
         if (i < n) one(i, x[i]);
+        if (b.v > -INFINITY) s *= __builtin_amdgcn_exp2f(-__fmaf_rn(b.v, kLog2e, -mk));  // the common factor of the thread's terms
     }
     RowTop r;
     r.best = block_best(b, red_v, red_i);

@@ -143,20 +143,21 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
             if (slot < kTopkWaveCap) list[wave_id() * kTopkWaveCap + slot] = key64(v, static_cast<uint32_t>(i));
         }
     };
+    // Every term is 2^(fma(v, k2, -mk)) with mk the ROUNDED product reference * k2: one instruction for the exponent,
+    // and all terms of a thread off by one common factor 2^(reference * k2 - mk), which is taken out again at the end
+    // (an fma gives that residue exactly). With a running maximum, mk moves with it and s is rescaled by 2^(old - new).
+    float mk = fixed ? rk : -1.0e30f * k2;  // no maximum yet: every term is 2^-inf = 0, never inf - inf
+    auto raise = [&](float to) {            // running maximum only: `to` > m
+        const float mk_new = to * k2;
+        s *= __builtin_amdgcn_exp2f(mk - mk_new);
+        m = to;
+        mk = mk_new;
+    };
     auto one = [&](int i, float v) {
-        if (!SUM) {
-            if (v > m) m = v;
-        } else if (fixed) {
-            if (v > -INFINITY) {  // not for NaN either
-                m = fmaxf(m, v);
-                s += __builtin_amdgcn_exp2f(__fmaf_rn(v, k2, -rk));
-            }
-        } else if (v > m) {
-            s = s * __builtin_amdgcn_exp2f((m - v) * k2) + 1.f;
-            m = v;
-        } else if (v > -INFINITY) {
-            s += __builtin_amdgcn_exp2f((v - m) * k2);
-        }
+        v = fmaxf(v, -INFINITY);  // NaN -> -inf
+        if (!SUM || fixed) m = fmaxf(m, v);
+        else if (v > m) raise(v);
+        if (SUM) s += __builtin_amdgcn_exp2f(__fmaf_rn(v, k2, -mk));
         if (COUNT) count(i, v);
     };
     // 128-bit loads on the aligned body of the row: the running maximum is raised once per vector (a branch that is
@@ -189,16 +190,8 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
         // NaN -> -inf (fmaxf returns the operand that is a number)
         const float v[4] = {fmaxf(q.x, -INFINITY), fmaxf(q.y, -INFINITY), fmaxf(q.z, -INFINITY), fmaxf(q.w, -INFINITY)};
         const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-        float mk = rk;
-        if (fixed || !SUM) {
-            m = fmaxf(m, vm);
-        } else {
-            if (vm > m) {
-                s *= __builtin_amdgcn_exp2f((m - vm) * k2);  // m = -inf: s is 0 and stays 0
-                m = vm;
-            }
-            mk = fmaxf(m, -1.0e30f) * k2;  // a row of -inf so far: every term below is 2^-inf = 0, never inf - inf
-        }
+        if (fixed || !SUM) m = fmaxf(m, vm);
+        else if (vm > m) raise(vm);
         if (SUM) {
             float add = 0.f;
 #pragma unroll
@@ -222,6 +215,10 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
     }
     const int i = head + 4 * nv + t;
     if (i < n) one(i, x[i]);
+    if (SUM) {  // the common factor of the thread's terms
+        const float at = fixed ? ref : m;
+        if (at > -INFINITY) s *= __builtin_amdgcn_exp2f(-__fmaf_rn(at, k2, -mk));
+    }
 }
 
 // The list holds every token of the row up to bin `list_bin`, the counts say in which bin the kk-th largest lies. When
