@@ -245,7 +245,7 @@ int ws_accept_sampled(void* stream, const ws_accept* a);
 
 /* Classic speculative sampling (accept u * q < p, else resample from max(p - q, 0)); no counterpart in the
  * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32
- * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1]. Per sequence s: u_j from
+ * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1] (may be NULL when n_pos is 1). Per sequence s: u_j from
  * (seed[s], row = s, step = step0[s] + j, stream 0); the resample / bonus draw uses stream 1 and walks the vocabulary
  * in id order. out_tokens[s][0 .. n_accepted[s]] = accepted drafts then the drawn token. */
 typedef struct ws_spec_verify {

@@ -173,6 +173,14 @@ def test_classic_verify_small(rng_mode):
         check_spec(p, q, draft, seed, step0, rng_mode)
 
 
+def test_classic_verify_draft_lengths():
+    """No draft at all (one position: the token comes from p), one draft, the reference's longest chain (15 drafts)."""
+    rng = np.random.default_rng(313)
+    for n_pos, V in ((1, 3000), (2, 257), (16, 5000)):
+        p, q, draft, seed, step0 = spec_case(rng, 5, n_pos, V)
+        check_spec(p, q, draft, seed, step0, 1)
+
+
 def test_classic_verify_special_cases():
     rng = np.random.default_rng(311)
     p, q, draft, seed, step0 = spec_case(rng, 4, 4, 2048)

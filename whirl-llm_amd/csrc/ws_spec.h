@@ -227,8 +227,8 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
 inline uint64_t spec_workspace(const ws_spec_verify*) { return 0; }
 
 inline int spec_launch(hipStream_t stream, const ws_spec_verify* v) {
-    if (!v || !v->p || !v->q || !v->draft || !v->seed || !v->step0 || !v->out_tokens || !v->n_accepted || !v->flags)
-        return WS_E_INVALID;
+    if (!v || !v->p || !v->q || !v->seed || !v->step0 || !v->out_tokens || !v->n_accepted || !v->flags) return WS_E_INVALID;
+    if (!v->draft && v->n_pos > 1) return WS_E_INVALID;  // one position: no draft to test, the token comes from p
     if (v->n_seq == 0 || v->n_pos < 1 || v->vocab == 0 || v->vocab > kSpecMaxSteps * 256u) return WS_E_INVALID;
     if (v->rng != WS_RNG_SPLITMIX && v->rng != WS_RNG_PHILOX) return WS_E_INVALID;
     SpecArgs a{v->p, v->q, v->draft, v->n_seq, v->n_pos, v->vocab, v->seed, v->step0, v->rng, v->out_tokens, v->n_accepted,
