@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the token-sampling hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload tile|cfg2|cfg3|cfg5] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload tile|cfg1|cfg2|cfg3|cfg5] [--no-cpu] [--no-also]
     python bench.py --reference-kernels      (greedy picks and topk_rows at the engine's shapes)
 
 A step = one launch of the fused batched sampler (ws_sample_batch) over one batch of synthetic logits that already
@@ -136,7 +136,7 @@ def cpu_baseline(c, budget_s=9.0, budget_all_s=6.0):
 
 def run_workload(name, steps, warmup, check_rows):
     import gpu_cases as gc
-    make = dict(tile=gc.make_tile, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
+    make = dict(tile=gc.make_tile, cfg1=gc.make_cfg1, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
     c = make()
     smp, wall_ms, kern_ms = time_gpu(c, steps, warmup)
     par = parity_sample(c, smp, check_rows) if check_rows else None
@@ -255,7 +255,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="tile", choices=["tile", "cfg2", "cfg3", "cfg5"])
+    ap.add_argument("--workload", default="tile", choices=["tile", "cfg1", "cfg2", "cfg3", "cfg5"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-also", action="store_true")
     ap.add_argument("--check-rows", type=int, default=8)
@@ -291,9 +291,9 @@ def main():
     c, main_res = run_workload(a.workload, a.steps, a.warmup, a.check_rows)
     also = []
     if not a.no_also:
-        for w in ("cfg2", "cfg3"):
+        for w in ("cfg1", "cfg2", "cfg3"):
             if w != a.workload:
-                _, r = run_workload(w, max(20, a.steps // 4), 5, 4)
+                _, r = run_workload(w, max(20, a.steps // 4), 5, 1 if w == "cfg1" else 4)
                 also.append(r)
         also.append(spec_verify_workload(max(20, a.steps // 4), 5))
     cpu = None if a.no_cpu else cpu_baseline(c)
