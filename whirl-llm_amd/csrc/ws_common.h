@@ -45,6 +45,11 @@ __device__ __forceinline__ double dpp_or_zero(double v) {
     return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
 }
 template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_or_zero(uint64_t v) {
+    const uint32_t lo = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(v)), hi = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(v >> 32));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ float dpp_or_zero(float v) {
     return __uint_as_float(dpp_or_zero<CTRL, ROW_MASK>(__float_as_uint(v)));
 }
@@ -66,6 +71,19 @@ __device__ __forceinline__ float dpp_or_self(float v) {
 }
 __device__ __forceinline__ uint32_t last_lane(uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63)); }
 __device__ __forceinline__ float last_lane(float v) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63)); }
+__device__ __forceinline__ uint64_t last_lane(uint64_t v) {
+    return (static_cast<uint64_t>(last_lane(static_cast<uint32_t>(v >> 32))) << 32) | last_lane(static_cast<uint32_t>(v));
+}
+// value of lane `l` (the same for the whole wave) in every lane
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t l) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), static_cast<int>(l)));
+}
+__device__ __forceinline__ uint64_t lane_value(uint64_t v, uint32_t l) {
+    return (static_cast<uint64_t>(lane_value(static_cast<uint32_t>(v >> 32), l)) << 32) | lane_value(static_cast<uint32_t>(v), l);
+}
+__device__ __forceinline__ double lane_value(double v, uint32_t l) {
+    return __longlong_as_double(static_cast<long long>(lane_value(static_cast<uint64_t>(__double_as_longlong(v)), l)));
+}
 __device__ __forceinline__ double last_lane(double v) {
     const uint64_t b = static_cast<uint64_t>(__double_as_longlong(v));
     const uint64_t r = (static_cast<uint64_t>(last_lane(static_cast<uint32_t>(b >> 32))) << 32) | last_lane(static_cast<uint32_t>(b));

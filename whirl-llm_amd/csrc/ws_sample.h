@@ -363,52 +363,119 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
     return (((k >> lp) * WS_BLOCK + threadIdx.x) << (lp + 1u)) + 2u * (k & ((1u << lp) - 1u)) + half;
 }
 
-// Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no second range; else
-// u0 + w0 < u1): its index goes to list[] (LDS, at most cap entries; *n_list, zeroed by the caller before a barrier,
-// counts all hits). Both 16-bit halves of a register are tested at once with ordinary 32-bit additions: bins are
-// below 4096, so y + (0x8000 - c) in each half neither carries into the other half nor wraps, and its bit 15 says
-// bin >= c. With the bounds lo0 < hi0 <= lo1 < hi1 (hi = last bin + 1) the four answers turn true one after the other
-// as the bin grows, so the bin lies in a range exactly when an odd number of them is true: the xor of the four sums has
-// bit 15 set. Hits are shifted into one mask per 16 registers; then each wave reserves a stretch of the list with one
-// atomic and its lanes write their tokens.
-__device__ __forceinline__ void gather_from_cache(int dtype, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
-                                                  uint32_t w1, uint32_t* list, uint32_t* n_list, uint32_t cap) {
-    const bool two = u1 <= 0x7fffu;
-    auto at_least = [](uint32_t c) { return 0x80008000u - c * 0x10001u; };  // y + this: bit 15 of a half = (bin >= c)
-    const uint32_t L0 = at_least(u0), H0 = at_least(u0 + w0 + 1u);
-    const uint32_t L1 = at_least(two ? u1 : 0u), H1 = at_least(two ? u1 + w1 + 1u : 0u);
-    uint32_t hits[kCacheRegs / 16];
-    uint32_t mine = 0;
-    // bit k / 16 + k of the result: low / high half of register 16 g + k lies in a range
-    auto test16 = [&](int g, auto&& sign) {
-        uint32_t acc = 0;
+// ---- scan of the bin cache. Every cached token whose bin lies in [u0, u0 + w0] or [u1, u1 + w1] (u1 > 0x7fff: no
+// second range; else u0 + w0 < u1) is a hit. A register holds two bins below 4096 in its 16-bit halves, so ordinary
+// 32-bit arithmetic tests both at once without a carry from one half into the other, the answer landing in bits 15 / 31:
+//   one range that starts at bin 0:  y + (0x8000 - end)          set where bin >= end                (a miss)
+//   a few single bins c:             (y ^ c) + 0x7fff            set where bin != c; and-ed over the bins (a miss)
+//   two ranges:                      xor of the four y + (0x8000 - bound)  set where the bin is in a range (a hit)
+// (one instruction per bin and register for the single bins: v_xad_u32). The flags of two registers are then spread
+// into whole bytes by one byte permute with the sign-replicating selectors, and one and-or per pair of registers files
+// them as bit j of the four bytes of a 32-bit word per 16 registers: bit 8 B + j of the word = register 2 j + (B >> 1)
+// of the group, half B & 1.
+// The first hit of a lane in each group of 16 registers has its logit requested right there (its token index follows
+// from the register's place), so the loads travel while the scan goes on; so has its second hit in the group (a
+// handful per row). A third one and beyond goes to list[] as (token | bit 31, 0) (LDS, at most cap entries; *n_list,
+// zeroed by the caller before a barrier, counts them) and is fetched by the caller afterwards.
+constexpr int kCacheGroups = kCacheRegs / 16;
+constexpr int kHitSlots = 2 * kCacheGroups;  // two per group of registers: slots g and kCacheGroups + g
+struct CacheHits {
+    uint32_t idx[kHitSlots];   // token index, 0xffffffff = none
+    uint32_t bits[kHitSlots];  // its logit as loaded: fp32 bits, or the 16 bits of a bf16
+};
+
+template <int MODE>  // 0: one range from bin 0; 1 / 2 / 3: so many single bins; 4: two ranges
+__device__ __forceinline__ uint32_t cache_group_flags(const uint32_t (&cache)[kCacheRegs], int g, uint32_t a0, uint32_t a1, uint32_t a2,
+                                                      uint32_t a3) {
+    uint32_t acc = 0;
 #pragma unroll
-        for (int k = 0; k < 16; ++k) acc = (acc >> 1) | (sign(cache[g * 16 + k]) & 0x80008000u);
-        return acc;
+    for (int j = 0; j < 8; ++j) {
+        uint32_t n[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t y = cache[g * 16 + 2 * j + h];
+            if (MODE == 0) n[h] = y + a0;
+            else if (MODE == 1) n[h] = (y ^ a0) + 0x7fff7fffu;
+            else if (MODE == 2) n[h] = ((y ^ a0) + 0x7fff7fffu) & ((y ^ a1) + 0x7fff7fffu);
+            else if (MODE == 3) n[h] = ((y ^ a0) + 0x7fff7fffu) & ((y ^ a1) + 0x7fff7fffu) & ((y ^ a2) + 0x7fff7fffu);
+            else n[h] = (y + a0) ^ (y + a1) ^ (y + a2) ^ (y + a3);
+        }
+        const uint32_t spread = __builtin_amdgcn_perm(n[1], n[0], 0x0B0A0908u);  // bytes: n0 bit 15, n0 bit 31, n1 bit 15, n1 bit 31
+        acc = (spread & (0x01010101u << j)) | acc;
+    }
+    return MODE == 4 ? acc : ~acc;
+}
+
+// the load of one logit as it is stored (one instruction, nothing done with the result: the caller waits for all of them at once)
+__device__ __forceinline__ uint32_t load_logit_bits(const RowView& rv, uint32_t i) {
+    return rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]);
+}
+__device__ __forceinline__ float logit_of_bits(const RowView& rv, uint32_t bits) {
+    return fmaxf(__uint_as_float(rv.dtype == 0 ? bits : bits << 16), -INFINITY);  // NaN -> -inf
+}
+
+template <int MODE, int DTYPE>  // the row's type is a template argument: a branch on it around a load makes the compiler wait for the loads before
+__device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t a0, uint32_t a1, uint32_t a2,
+                                                uint32_t a3, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
+    auto token_of = [&](int g, uint32_t bit) { return cache_token(DTYPE, g * 16u + 2u * (bit & 7u) + (bit >> 4), (bit >> 3) & 1u); };
+    auto load_bits = [&](uint32_t i) {
+        return DTYPE == 0 ? static_cast<const uint32_t*>(rv.base)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]);
     };
 #pragma unroll
-    for (int g = 0; g < kCacheRegs / 16; ++g) {
-        uint32_t acc;
-        if (two) acc = test16(g, [&](uint32_t y) { return (y + L0) ^ (y + H0) ^ (y + L1) ^ (y + H1); });  // uniform branch
-        else acc = test16(g, [&](uint32_t y) { return (y + L0) ^ (y + H0); });
-        hits[g] = acc;
-        mine += __popc(acc);
-        __builtin_amdgcn_sched_barrier(0);  // one group at a time: a wider scheduling window costs more registers than it hides
-    }
-    const uint32_t inc = wave_incl_scan(mine);  // inclusive prefix over the wave
-    uint32_t base = 0;
-    if (lane_id() == 63 && inc) base = atomicAdd(n_list, inc);
-    uint32_t slot = __shfl(base, 63) + inc - mine;
-#pragma unroll
-    for (int g = 0; g < kCacheRegs / 16; ++g) {
-        uint32_t h = hits[g];
-        while (h) {
-            const uint32_t bit = static_cast<uint32_t>(__ffs(h)) - 1u;
+    for (int g = 0; g < kCacheGroups; ++g) {
+        uint32_t h = cache_group_flags<MODE>(cache, g, a0, a1, a2, a3);
+        // every load has a register of its own that nothing else writes: a copy of a register with a load on the way
+        // would have to wait for it
+        hits.idx[g] = hits.idx[kCacheGroups + g] = 0xffffffffu;
+        hits.bits[g] = hits.bits[kCacheGroups + g] = 0u;
+        if (h) {
+            const uint32_t i = token_of(g, static_cast<uint32_t>(__ffs(h)) - 1u);
             h &= h - 1u;
-            if (slot < cap) list[slot] = cache_token(dtype, g * 16u + (bit & 15u), bit >> 4);
-            ++slot;
+            hits.idx[g] = i;
+            hits.bits[g] = load_bits(i);
+        }
+        if (h) {
+            const uint32_t i = token_of(g, static_cast<uint32_t>(__ffs(h)) - 1u);
+            h &= h - 1u;
+            hits.idx[kCacheGroups + g] = i;
+            hits.bits[kCacheGroups + g] = load_bits(i);
+        }
+        while (h) {
+            const uint32_t i = token_of(g, static_cast<uint32_t>(__ffs(h)) - 1u);
+            h &= h - 1u;
+            const uint32_t slot = atomicAdd(n_list, 1u);
+            if (slot < cap) list[slot] = make_uint2(i | 0x80000000u, 0u);
         }
     }
+}
+
+template <int DTYPE>
+__device__ __forceinline__ void scan_cache_typed(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
+                                                 uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
+    const bool two = u1 <= 0x7fffu;
+    auto at_least = [](uint32_t c) { return 0x80008000u - c * 0x10001u; };  // y + this: bit 15 of a half = (bin >= c)
+    auto both = [](uint32_t c) { return c * 0x10001u; };
+    const uint32_t n_single = (w0 + 1u) + (two ? w1 + 1u : 0u);  // bins asked for
+    if (!two && u0 == 0u) {
+        scan_cache_impl<0, DTYPE>(rv, cache, at_least(w0 + 1u), 0u, 0u, 0u, hits, list, n_list, cap);
+    } else if (n_single <= 3u) {
+        uint32_t c[3];
+        uint32_t k = 0;
+        for (uint32_t b = u0; b <= u0 + w0; ++b) c[k++] = both(b);
+        if (two)
+            for (uint32_t b = u1; b <= u1 + w1; ++b) c[k++] = both(b);
+        if (k == 1u) scan_cache_impl<1, DTYPE>(rv, cache, c[0], 0u, 0u, 0u, hits, list, n_list, cap);
+        else if (k == 2u) scan_cache_impl<2, DTYPE>(rv, cache, c[0], c[1], 0u, 0u, hits, list, n_list, cap);
+        else scan_cache_impl<3, DTYPE>(rv, cache, c[0], c[1], c[2], 0u, hits, list, n_list, cap);
+    } else {
+        scan_cache_impl<4, DTYPE>(rv, cache, at_least(u0), at_least(u0 + w0 + 1u), at_least(two ? u1 : 0u), at_least(two ? u1 + w1 + 1u : 0u),
+                                  hits, list, n_list, cap);
+    }
+}
+__device__ __forceinline__ void scan_cache(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
+                                           uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
+    if (rv.dtype == 0) scan_cache_typed<0>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap);
+    else scan_cache_typed<1>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap);
 }
 
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
@@ -481,9 +548,9 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
 template <bool FUSED>
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #ifdef WS_PHASE_TIMERS
-    __shared__ long long ws_marks[32];
+    __shared__ long long ws_marks[64];
     const long long ws_t0 = clock64();
-    if (threadIdx.x < 32) ws_marks[threadIdx.x] = 0;
+    if (threadIdx.x < 64) ws_marks[threadIdx.x] = 0;
     __syncthreads();
 #endif
     extern __shared__ __align__(16) unsigned char lds[];
@@ -493,10 +560,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ unsigned long long red_q[WS_WAVES];
     __shared__ uint32_t s_cnt;
     __shared__ double s_exp[128];  // kExpHi, kExpLo
-    __shared__ double pm64[64];    // every 64th entry of the scanned histogram's mass prefixes
-    __shared__ uint32_t pc64[64];  // and of its count prefixes
-    __shared__ double tot_m[64];   // histogram scan: mass and count of each stretch of 64 bins
-    __shared__ uint32_t tot_c[64];
+    __shared__ double s_pool[192];
+    double* pm64 = s_pool;                                         // every 64th entry of the scanned histogram's mass prefixes
+    double* tot_m = s_pool + 64;                                   // histogram scan: mass and count of each stretch of 64 bins
+    uint32_t* pc64 = reinterpret_cast<uint32_t*>(s_pool + 128);    // every 64th entry of the count prefixes
+    uint32_t* tot_c = reinterpret_cast<uint32_t*>(s_pool + 160);
     __shared__ uint32_t s_u[8];
 
     const uint32_t row = blockIdx.x;
@@ -519,6 +587,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double tol = A.tol;
     const uint64_t seed = A.seed[row], step = A.step[row];
     const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
+    const bool race = A.race != nullptr && A.race[row] != 0;
     // exp(-b / 64) tables of the histogram scan: fetched now, parked in LDS before the sweep, so that the scan does not
     // wait for global memory in the middle of the row's tail
     const double exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);
@@ -1124,7 +1193,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double m1base = has_r1 ? pm[r1lo] : 0.0;
     const uint32_t n_list = n_r0 + n_r1;
     if (n_list > kCap || n_list == 0) flags |= kOverflow;
-    if (t == 0) s_cnt = s_u[5] = 0;
+    if (t == 0) s_cnt = s_u[4] = s_u[5] = 0;
     __syncthreads();  // the last reads of pm / pc are done: their LDS is the key buffer and the candidate list from here
 
     if (flags & kOverflow) {
@@ -1143,6 +1212,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     WS_MARK(3);
+    // what the cuts and the draw leave behind: filled by the bucket finish inside pass 3 or by the sort-based one after it
+    double mg_top_p = 1.0, mg_min_p = 1.0, mg_draw = 1.0;
+    uint32_t n3 = n1;
+    int32_t token = -1;
+    double ptok = 0;
+    uint64_t kept_key = 0ull;
+    bool finished = false;
     // ------------------------------------------------------------------ pass 3: gather, sort, exact masses
     {
         const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = static_cast<uint32_t>(r0hi - r0lo);
@@ -1162,30 +1238,342 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         };
         if (FUSED && cached) {
             if constexpr (FUSED) {
-                // token indices first (no loads in the scan), then rounds of independent loads for the keys; a hit
-                // that is a touched token (cached with the bin of its raw logit) is dropped here and fed below
-                uint32_t* list = reinterpret_cast<uint32_t*>(emass);
-                if (t == 0) s_u[4] = 0;
+                // The scan requests the logit of a lane's first two hits per group of registers as it finds them; the lanes
+                // then line their hits up in list[] as (token, logit bits) pairs, a third hit and beyond as the token alone
+                // (kNeedsLoad), and the list is taken from there one entry per thread. A hit that is a touched token
+                // (cached with the bin of its raw logit) is dropped and fed by replay_touched.
+                constexpr uint32_t kNeedsLoad = 0x80000000u, kAdjusted = 0x40000000u, kIdMask = 0x3fffffffu;
+                uint2* list = reinterpret_cast<uint2*>(emass);  // kCap entries
+                // tables of the bucket finish below: per bucket a count and a fixed-point mass (the LDS of the histogram
+                // scan's side arrays, idle by now) and places for keys and their masses: 32 per bucket where the spare LDS
+                // takes the masses, else 16 with keys and masses sharing the key region (idle until then)
+                constexpr uint32_t kLeanBuckets = 128u;  // 64 per range
+                const uint32_t lean_shift = A.lds_tie ? 5u : 4u, lean_places = 1u << lean_shift;
+                const uint32_t lean_max = A.lds_tie ? 800u : 448u;  // candidates per range: a bucket must not run out of places
+                uint64_t* lb_mass = reinterpret_cast<uint64_t*>(s_pool);
+                uint32_t* lb_cnt = reinterpret_cast<uint32_t*>(s_pool + 128);
+                uint64_t* lb_key = reinterpret_cast<uint64_t*>(lds);           // [bucket][place]
+                double* lb_e = reinterpret_cast<double*>(lds + (A.lds_tie ? A.lds_tie : 16384u));  // exact mass of lb_key
+                __shared__ unsigned long long s_q[2];
+                if (t < kLeanBuckets) {
+                    lb_mass[t] = 0ull;
+                    lb_cnt[t] = 0u;
+                }
+                if (t == 0) {
+                    s_q[0] = ~0ull;
+                    s_q[1] = 0ull;
+                    s_u[6] = s_u[7] = 0u;
+                }
+                {
+                    CacheHits hits;
+                    scan_cache(rv, cache, u0, w0, u1r, w1, hits, list, &s_u[4], kCap);
+                    WS_MARK(10);
+                    // touched tokens whose adjusted logit lies in the ranges, while the last loads of the scan travel
+                    replay_touched([&](uint32_t i, float x) {
+                        if (in_ranges(x)) {
+                            const uint32_t slot = atomicAdd(&s_u[4], 1u);
+                            if (slot < kCap) list[slot] = make_uint2(i | kAdjusted, __float_as_uint(x));
+                        }
+                    });
+                    uint32_t mine = 0;
+#pragma unroll
+                    for (int g = 0; g < kHitSlots; ++g) mine += hits.idx[g] != 0xffffffffu ? 1u : 0u;
+                    const uint32_t inc = wave_incl_scan(mine);
+                    uint32_t base = 0;
+                    if (lane_id() == 63 && inc) base = atomicAdd(&s_u[4], inc);
+                    uint32_t slot = __shfl(base, 63) + inc - mine;
+#pragma unroll
+                    for (int g = 0; g < kHitSlots; ++g) {
+                        if (hits.idx[g] == 0xffffffffu) continue;
+                        if (slot < kCap) list[slot] = make_uint2(hits.idx[g], hits.bits[g]);
+                        ++slot;
+                    }
+                }
+                WS_MARK(40);
                 __syncthreads();
-                gather_from_cache(rv.dtype, cache, u0, w0, u1r, w1, list, &s_u[4], 2u * kCap);
-                __syncthreads();
-                WS_MARK(10);
-                const uint32_t n_hit = min(s_u[4], 2u * kCap);
-                if (s_u[4] > 2u * kCap) flags |= kOverflow;
+                WS_MARK(41);
+                const uint32_t n_hit = min(s_u[4], kCap);
+                if (s_u[4] > kCap) flags |= kOverflow;
+                // one entry of the list: is it kept, and its logit
+                auto entry = [&](uint2 en, bool live, uint32_t& id, float& x) {
+                    id = en.x & kIdMask;
+                    const bool adjusted = en.x & kAdjusted;
+                    const bool keep = live && (adjusted || !is_touched(rv, id));
+                    x = adjusted ? __uint_as_float(en.y) : logit_of_bits(rv, en.y);
+                    if (en.x & kNeedsLoad) x = keep ? raw_logit(rv, id) : 0.f;
+                    return keep;
+                };
+                // ---- bucket finish (closed rows, inverse-CDF draw, up to lean_max candidates per range). No sort: every
+                // candidate adds its exact mass, in fixed point, and a count to one of the 64 buckets of its range - equal
+                // steps of the bin coordinate across the range, so buckets are ordered like the keys - and leaves its key
+                // in one of the bucket's places. Each question - the candidate at a rank, the first candidate at which the
+                // running mass reaches a value - is then answered by finding its bucket in the scanned counts and masses
+                // (two buckets per lane, in registers) and ranking the few keys of that one bucket inside a wave. Integer
+                // sums: the same bits whatever the order of arrival. Wave 0 works the answers out (eight waves doing the same
+                // arithmetic side by side only slow each other down) and leaves them in LDS. A bucket with more keys than
+                // places (heavy ties) sends the row to the sort-based finish.
+                const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+                const bool lean = !race && !open_row && !(flags & kOverflow) && n_r0 <= lean_max && n_r1 <= lean_max && n_hit <= 4u * WS_BLOCK;
+                bool lean_failed = false;
+                if (lean) {
+                    // masses of a range in units of 2^-52 of the largest mass a token of the range can have
+                    auto edge_mass = [&](int b) { return s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001; };
+                    const double emax0 = edge_mass(r0lo), emax1 = has_r1 ? edge_mass(r1lo) : 1.0;
+                    const double scale0 = 4503599627370496.0 / emax0, scale1 = 4503599627370496.0 / emax1;
+                    const double inv0 = emax0 * (1.0 / 4503599627370496.0), inv1 = emax1 * (1.0 / 4503599627370496.0);
+                    const float step0 = 64.f / static_cast<float>(nb0), step1 = has_r1 ? 64.f / static_cast<float>(nb1) : 0.f;
+                    const float lo0 = static_cast<float>(r0lo), lo1 = static_cast<float>(r1lo);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (static_cast<uint32_t>(q) * WS_BLOCK >= n_hit) continue;  // uniform
+                        const uint32_t k = q * WS_BLOCK + t;
+                        const uint2 en = k < n_hit ? list[k] : make_uint2(0u, 0u);
+                        uint32_t id;
+                        float x;
+                        const bool on = entry(en, k < n_hit, id, x);
+                        const float tc = bin_coord(aq, c64, x);
+                        const bool in1 = has_r1 && static_cast<uint32_t>(tc) - static_cast<uint32_t>(r1lo) < nb1;
+                        const float rel = fmaxf(__fmul_rn(__fsub_rn(tc, in1 ? lo1 : lo0), in1 ? step1 : step0), 0.f);
+                        const uint32_t bkt = (in1 ? 64u : 0u) + min(63u, static_cast<uint32_t>(rel));
+                        const double e = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
+                        const uint64_t fix = static_cast<uint64_t>(__double2ull_rn(e * (in1 ? scale1 : scale0)));
+                        if (on) {
+                            const uint32_t place = atomicAdd(&lb_cnt[bkt], 1u);
+                            atomicAdd(reinterpret_cast<unsigned long long*>(&lb_mass[bkt]), static_cast<unsigned long long>(fix));
+                            if (place < lean_places) {
+                                lb_key[(bkt << lean_shift) + place] = key64(x, id);
+                                lb_e[(bkt << lean_shift) + place] = e;
+                            } else {
+                                s_u[7] = 1u;
+                            }
+                        }
+                        if (use_min_p && minp_in_list) {  // uniform
+                            // candidates at or above the floor form a prefix of the sorted entries: their number, the
+                            // smallest mass among them and the largest below the floor
+                            const bool pass = on && e >= min_p;
+                            const uint64_t np = __ballot(pass);
+                            if (lane_id() == 0 && np) atomicAdd(&s_u[6], static_cast<uint32_t>(__popcll(np)));
+                            if (pass) atomicMin(&s_q[0], static_cast<unsigned long long>(__double_as_longlong(e)));
+                            if (on && !pass) atomicMax(&s_q[1], static_cast<unsigned long long>(__double_as_longlong(e)));
+                        }
+                    }
+                    __syncthreads();
+                    WS_MARK(42);
+                    struct LeanResult {
+                        int32_t token;
+                        uint32_t n3, overflow, ok;
+                        double ptok, mg_top_p, mg_min_p, mg_draw;
+                        unsigned long long kept_key;
+                    };
+                    __shared__ LeanResult s_res;
+                    if (t < 64u) {  // wave 0
+                    // counts and masses of the buckets 2 lane, 2 lane + 1 and of all buckets before them (range 1 starts at lane 32)
+                    const uint32_t lane = static_cast<uint32_t>(lane_id());
+                    const uint32_t bc0 = lb_cnt[2u * lane], bc1 = lb_cnt[2u * lane + 1u];
+                    const uint64_t bf0 = lb_mass[2u * lane], bf1 = lb_mass[2u * lane + 1u];
+                    const uint32_t cbefore = wave_incl_scan(bc0 + bc1) - (bc0 + bc1);
+                    const uint64_t fbefore = wave_incl_scan(bf0 + bf1) - (bf0 + bf1);
+                    const uint32_t got0 = lane_value(cbefore, 32u), got = lane_value(cbefore + bc0 + bc1, 63u);
+                    const uint64_t fbase1 = lane_value(fbefore, 32u);
+                    if (s_u[7] || got0 != n_r0 || got != n_list) lean_failed = true;  // heavy ties, or the histogram and the gather disagree
+                    auto bucket_tab = [&](uint32_t b, uint32_t& cnt, uint32_t& cpre, uint64_t& fpre) {  // b is the same in all lanes
+                        const uint32_t src = b >> 1;
+                        const uint32_t c0 = lane_value(bc0, src), c1 = lane_value(bc1, src), cb = lane_value(cbefore, src);
+                        const uint64_t f0 = lane_value(bf0, src), fb = lane_value(fbefore, src);
+                        cnt = (b & 1u) ? c1 : c0;
+                        cpre = (b & 1u) ? cb + c0 : cb;
+                        fpre = (b & 1u) ? fb + f0 : fb;
+                    };
+                    // one candidate picked inside bucket b: by rank inside the bucket (by_rank), or the first whose running
+                    // mass reaches X (>= X, or > X when strict). Lane l holds key l of the bucket; every key counts the keys
+                    // before it and adds up the masses up to and with its own.
+                    struct Pick {
+                        bool found;
+                        uint64_t key;
+                        double in, ex, e;
+                        uint32_t pos;
+                    };
+                    auto pick_in_bucket = [&](uint32_t b, bool by_rank, uint32_t want, double Xq, bool strict) {
+                        Pick r{false, 0ull, 0.0, 0.0, 0.0, 0u};
+                        const bool r1 = b >= 64u;
+                        uint32_t cnt, cpre;
+                        uint64_t fpre;
+                        bucket_tab(b, cnt, cpre, fpre);
+                        const uint64_t key = lane < cnt ? lb_key[(b << lean_shift) + lane] : 0ull;
+                        const double e = lane < cnt ? lb_e[(b << lean_shift) + lane] : 0.0;
+                        const uint64_t fx = static_cast<uint64_t>(__double2ull_rn(e * (r1 ? scale1 : scale0)));  // as it went into the bucket's sum
+                        uint32_t rank = 0;
+                        uint64_t cum = 0;
+                        for (uint32_t j = 0; j < cnt; ++j) {
+                            const uint64_t kj = lane_value(key, j), fj = lane_value(fx, j);
+                            rank += kj > key ? 1u : 0u;
+                            cum += kj >= key ? fj : 0ull;
+                        }
+                        const uint64_t fb = fpre - (r1 ? fbase1 : 0ull);
+                        const double mb = r1 ? m1base : m0base, inv = r1 ? inv1 : inv0;
+                        const double in = mb + static_cast<double>(fb + cum) * inv, ex = mb + static_cast<double>(fb + cum - fx) * inv;
+                        uint32_t want_rank = want;
+                        if (!by_rank) {
+                            const bool sat = strict ? in > Xq : in >= Xq;
+                            want_rank = static_cast<uint32_t>(__popcll(__ballot(lane < cnt && !sat)));
+                        }
+                        const uint64_t who = __ballot(lane < cnt && rank == want_rank);
+                        if (!who) return r;
+                        const uint32_t src = static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(who)) - 1);
+                        r.found = true;
+                        r.key = lane_value(key, src);
+                        r.in = lane_value(in, src);
+                        r.ex = lane_value(ex, src);
+                        r.e = lane_value(e, src);
+                        r.pos = (r1 ? c1base : c0base) + (cpre - (r1 ? got0 : 0u)) + want_rank;
+                        return r;
+                    };
+                    // first bucket (in sorted order, empty ones left out) for which pred holds - pred(bucket, entries up to and
+                    // with it, masses up to and with it, both counted from the start of bucket 0) holds from some bucket on;
+                    // 128 when for none
+                    auto first_bucket = [&](auto&& pred) {
+                        const bool ok0 = bc0 != 0u && pred(2u * lane, cbefore + bc0, fbefore + bf0);
+                        const bool ok1 = bc1 != 0u && pred(2u * lane + 1u, cbefore + bc0 + bc1, fbefore + bf0 + bf1);
+                        const uint64_t any = __ballot(ok0 || ok1);
+                        if (!any) return kLeanBuckets;
+                        const uint32_t src = static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(any)) - 1);
+                        return 2u * src + (lane_value(static_cast<uint32_t>(ok0), src) ? 0u : 1u);
+                    };
+                    auto pick_mass = [&](double Xq, bool strict) {
+                        const uint32_t b = first_bucket([&](uint32_t bb, uint32_t, uint64_t fincl) {
+                            const bool r1 = bb >= 64u;
+                            const double v = (r1 ? m1base : m0base) + static_cast<double>(fincl - (r1 ? fbase1 : 0ull)) * (r1 ? inv1 : inv0);
+                            return strict ? v > Xq : v >= Xq;
+                        });
+                        if (b >= kLeanBuckets) return Pick{false, 0ull, 0.0, 0.0, 0.0, 0u};
+                        return pick_in_bucket(b, false, 0u, Xq, strict);
+                    };
+                    auto pick_rank = [&](uint32_t p) {  // the candidate of rank p in the row, if it was gathered
+                        uint32_t q, lo;
+                        if (p >= c0base && p - c0base < n_r0) {
+                            q = p - c0base;
+                            lo = 0u;
+                        } else if (has_r1 && p >= c1base && p - c1base < n_r1) {
+                            q = got0 + (p - c1base);
+                            lo = 64u;
+                        } else {
+                            return Pick{false, 0ull, 0.0, 0.0, 0.0, 0u};
+                        }
+                        const uint32_t b = first_bucket([&](uint32_t bb, uint32_t cincl, uint64_t) { return bb >= lo && bb < lo + 64u && cincl > q; });
+                        if (b >= kLeanBuckets) return Pick{false, 0ull, 0.0, 0.0, 0.0, 0u};
+                        uint32_t cnt, cpre;
+                        uint64_t fpre;
+                        bucket_tab(b, cnt, cpre, fpre);
+                        return pick_in_bucket(b, true, q - cpre, 0.0, false);
+                    };
+                    // ---- the cuts, as the sort-based finish makes them (src/sampling/sampler.cpp:35-74)
+                    Pick last{false, 0ull, 0.0, 0.0, 0.0, 0u};  // the last kept candidate where one of the picks below already is it
+                    if (prefix_mode && !lean_failed) {
+                        last = pick_rank(n1 - 1u);
+                        if (!last.found) lean_failed = true;
+                        X = top_p * last.in;
+                    }
+                    uint32_t n2 = n1;
+                    if (use_top_p && topp_in_list && !lean_failed) {
+                        const Pick c = pick_mass(X, false);
+                        if (c.found && c.pos < n1 && !(c.ex >= X) && c.in > c.ex) {
+                            n2 = c.pos + 1u;
+                            mg_top_p = fmin(c.in - X, c.pos > 0 ? X - c.ex : X) / X;
+                            last = c;
+                        } else {  // rounding: the cut falls just past the gathered bins
+                            n2 = prefix_mode ? n1 : min(n1, has_r1 ? c1base + n_r1 : c0base + n_r0);
+                            mg_top_p = 0.0;
+                        }
+                    }
+                    n3 = n2;
+                    if (use_min_p && minp_in_list) {
+                        const uint32_t passed = s_u[6];
+                        double near = 1.0;
+                        if (passed > 0u) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[0])) - min_p) / min_p);
+                        if (passed < n_list) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[1])) - min_p) / min_p);
+                        uint32_t n3p;
+                        if (has_r1)
+                            n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
+                        else
+                            n3p = c0base + passed;
+                        n3 = min(n2, n3p);
+                        if (n3 < 1u) n3 = 1u;
+                        mg_min_p = near;
+                    }
+                    double Zk = Z;
+                    bool have_last = false;
+                    if (!lean_failed) {
+                        if (!(last.found && last.pos == n3 - 1u)) last = pick_rank(n3 - 1u);
+                        if (last.found) {
+                            have_last = true;
+                            Zk = last.in;
+                            kept_key = last.key;
+                        } else if (has_r1 && n3 == c1base) {  // the cut falls on the upper edge of range 1: everything in earlier bins
+                            Zk = m1base;
+                            kept_key = static_cast<uint64_t>(first_key_before_bin(aq, c64, m, r1lo)) << 32;
+                        } else if (n3 == c0base && n_r0) {
+                            Zk = m0base;
+                            kept_key = static_cast<uint64_t>(first_key_before_bin(aq, c64, m, r0lo)) << 32;
+                        } else {  // no filter at all: the whole row
+                            Zk = Z;
+                            kept_key = 0ull;
+                        }
+                    }
+                    // ---- the draw (src/sampling/sampler.cpp:118-131)
+                    if (!lean_failed) {
+                        const double target = batch_uniform(A.rng, seed, row, step, 0) * Zk;
+                        const Pick d = pick_mass(target, true);
+                        if (!lean_failed) {
+                            if (d.found && d.pos < n3 && !(d.ex > target) && d.in > d.ex) {
+                                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(d.key));
+                                ptok = d.e / Zk;
+                                mg_draw = fmin(d.in - target, d.pos > 0 ? target - d.ex : 1e300) / Zk;
+                            } else if (have_last) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
+                                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(last.key));
+                                ptok = last.e / Zk;
+                                mg_draw = 0.0;
+                            } else {
+                                flags |= kOverflow;
+                            }
+                        }
+                    }
+                    if (lane == 0u) s_res = LeanResult{token, n3, flags & kOverflow, lean_failed ? 0u : 1u, ptok, mg_top_p, mg_min_p, mg_draw, kept_key};
+                    }  // wave 0
+                    __syncthreads();  // the answers are in place, and the bucket tables are done with
+                    if (s_res.ok) {
+                        token = s_res.token;
+                        n3 = s_res.n3;
+                        flags |= s_res.overflow;
+                        ptok = s_res.ptok;
+                        mg_top_p = s_res.mg_top_p;
+                        mg_min_p = s_res.mg_min_p;
+                        mg_draw = s_res.mg_draw;
+                        kept_key = s_res.kept_key;
+                        finished = true;
+                    } else {
+                        mg_top_p = mg_min_p = mg_draw = 1.0;
+                        n3 = n1;
+                        token = -1;
+                        ptok = 0;
+                        kept_key = 0ull;
+                    }
+                }
+                if (!finished) {  // uniform: the list goes to keys[] by range, as the sort-based finish expects it
                 for (uint32_t k0 = 0; k0 < n_hit; k0 += 4u * WS_BLOCK) {
-                    uint32_t idx[4];
+                    uint2 en[4];
                     float xs[4];
+                    uint32_t ids[4];
                     bool keep[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const uint32_t k = k0 + q * WS_BLOCK + t;
-                        idx[q] = k < n_hit ? list[k] : 0u;
-                        keep[q] = k < n_hit && !is_touched(rv, idx[q]);
+                        en[q] = k < n_hit ? list[k] : make_uint2(0u, 0u);
                     }
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) xs[q] = keep[q] ? raw_logit(rv, idx[q]) : 0.f;
+                    for (int q = 0; q < 4; ++q) keep[q] = entry(en[q], k0 + q * WS_BLOCK + t < n_hit, ids[q], xs[q]);
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
+                        if (static_cast<uint32_t>(q) * WS_BLOCK + k0 >= n_hit) continue;  // uniform
                         // one slot reservation per wave and range: lanes that keep their hit take consecutive slots
                         const bool in1 = keep[q] && bin_of(aq, c64, xs[q]) - u1r <= w1;
                         const uint64_t m1 = __ballot(in1), m0 = __ballot(keep[q] && !in1);
@@ -1196,10 +1584,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         const uint32_t s0 = __shfl(b0, 0) + static_cast<uint32_t>(__popcll(m0 & below));  // every lane takes part
                         const uint32_t s1 = n_r0 + __shfl(b1, 0) + static_cast<uint32_t>(__popcll(m1 & below));
                         const uint32_t slot = in1 ? s1 : s0;
-                        if (keep[q] && slot < kCap) keys[slot] = key64(xs[q], idx[q]);
+                        if (keep[q] && slot < kCap) keys[slot] = key64(xs[q], ids[q]);
                     }
                 }
-                __syncthreads();
+                }
             }
         } else {
             // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
@@ -1217,9 +1605,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     }
                 });
         }
-        replay_touched([&](uint32_t i, float x) {
-            if (in_ranges(x)) push(i, x);
-        });
+        if (!(FUSED && cached))
+            replay_touched([&](uint32_t i, float x) {
+                if (in_ranges(x)) push(i, x);
+            });
     }
     __syncthreads();
     if (flags & kOverflow) {  // uniform: more cached hits than the list holds
@@ -1237,6 +1626,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         return;
     }
     WS_MARK(4);
+    if (!finished) {  // uniform: the sort-based finish
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
         float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
@@ -1605,7 +1995,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     };
 
     // ------------------------------------------------------------------ cuts
-    double mg_top_p = 1.0, mg_min_p = 1.0, mg_draw = 1.0;
     // top-k: mass of the first n1 candidates (prefix mode: one range that starts at rank 0)
     double M1 = Z;
     if (prefix_mode) {
@@ -1630,7 +2019,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             mg_top_p = 0.0;
         }
     }
-    uint32_t n3 = n2;
+    n3 = n2;
     if (use_min_p && minp_in_list) {
         // candidates are in descending order, so those at or above the floor form a prefix of the gathered entries;
         // entries ranked before the min-p bins pass by construction
@@ -1650,7 +2039,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // kept mass = inclusive mass at rank n3 - 1; when that rank is just before a gathered range, the range's base
     const uint32_t i_last = entry_of(n3 - 1u);
     double Zk;
-    uint64_t kept_key;
     if (i_last < n_list) {
         Zk = inc_of(i_last);
         kept_key = keys[i_last];
@@ -1669,13 +2057,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double u = batch_uniform(A.rng, seed, row, step, 0);
     if (open_row) Zk = Zf;  // an open row is not renormalised: p = mass / Sampler::sum
     const double target = u * Zk;
-    int32_t token = -1;
-    double ptok = 0;
     // The race draw of the "specsample" rule (src/sampling/sampler.cpp:80-106): the kept token with the smallest
     // E(token) / p(token), E = -ln(1 - U) with U hashed from (seed, step, token) (src/common/spec_sample.cpp:83-87),
     // the earlier candidate in sorted order on equal keys. An open row races over its listed candidates when the
     // uniform falls on their mass and otherwise takes the walk below with the same uniform.
-    const bool race = A.race != nullptr && A.race[row] != 0;
     bool raced = false;
     if (race && (!open_row || target < inc_of(i_last))) {
         raced = true;
@@ -2003,6 +2388,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     }
     if (race && open_row) mg_draw = fmin(mg_draw, fabs(target - inc_of(i_last)) / Zk);  // the list-or-rest decision
+    }  // the sort-based finish
     // zero-mass tail candidates a top-k kept (no top-p / min-p cut them away again)
     const uint32_t tail_extra = (!use_top_p && !use_min_p && n3 == n1) ? n1_asked - n1 : 0u;
     if (mg_top_p < tol) flags |= kNearTopP;
@@ -2013,7 +2399,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
         float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
-        for (uint32_t k = 0; k < 32u && k < A.kept_cap; ++k)
+        for (uint32_t k = 0; k < 64u && k < A.kept_cap; ++k)
             if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
     }
 #endif
