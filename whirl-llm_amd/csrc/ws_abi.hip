@@ -59,7 +59,8 @@ BatchPlan plan_batch(const ws_batch* b) {
     const uint64_t esz = b->dtype == WS_DTYPE_F32 ? 4 : 2;
     const bool vec_rows = b->vocab % 8u == 0 && (b->row_stride * esz) % 16u == 0 && reinterpret_cast<uintptr_t>(b->logits) % 16u == 0;
     const uint64_t fused_total = 65536u + maps + cap * 8u;
-    const bool can_fuse = vec_rows && b->vocab <= 163840u && fused_total + 4096u <= kMaxLds;
+    // (a token's bias entries are counted in 11 bits of its rank word)
+    const bool can_fuse = vec_rows && b->vocab <= 163840u && fused_total + 4096u <= kMaxLds && (!b->bias_ids || b->max_bias <= 2047u);
     if (b->mode == WS_MODE_FUSED && !can_fuse) return p;
     p.fused = b->mode != WS_MODE_EXACT && can_fuse;
     uint64_t ab, total;

@@ -841,6 +841,110 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         __syncthreads();
     };
+    // The single-sweep kernel's version of the above, one pass and no barrier of its own: every history / bias entry
+    // finds its token's rank and claims it (one returning atomic on the rank's count word sets the top bit; the entry that
+    // finds it clear is the one that goes on, with the counts in its hands); the owner takes the token's raw logit from the
+    // vector the sweep staged (or from memory), adjusts it, leaves pv[rank] <- adjusted and pid[rank] <- token id, and, when
+    // the sweep's histogram stands (move), takes the token out of the bin of its raw logit and puts it into the bin of the
+    // adjusted one. ma / mu: the thread's largest adjusted logit, and its largest untouched, allowed logit among the
+    // vectors that hold touched tokens (the sweep's running maximum leaves those vectors out).
+    auto collect_fused = [&](const uint4* stage, uint32_t stage_cap, bool move, float aq_, float c64_, float& ma, float& mu) {
+        ma = mu = -INFINITY;
+        if (!n_touched) return;
+        constexpr uint32_t kClaim = 0x80000000u;
+        const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
+        const int32_t* hist_ids = A.hist + h0;
+        const int32_t* bias_ids = A.bias_ids + b0;
+        const float* bias_vals = A.bias_vals + b0;
+        uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
+        uint32_t* first = cnt + A.patch_cap;
+        const uint32_t whole_end = rv.vec ? (V & ~(per - 1u)) : 0u;  // tokens below this sit in whole 128-bit vectors
+        const float tail_own = own_tail();
+        auto take4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {  // four entries per thread and round, step by step side by side
+            for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
+                uint32_t id[4], al[4], tw[4], wp[4], rk[4], old[4];
+                uint4 vec[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t j = j0 + k * WS_BLOCK + t;
+                    if (in_regs && j0 == 0) id[k] = hid[k];  // kHid = 4: the first round is in registers
+                    else id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    al[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
+                    tw[k] = touched[i >> 5];
+                    wp[k] = wprefix[i >> 5];
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    const uint32_t vb = i & ~(per - 1u);
+                    const uint32_t rf = wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u));  // rank of the vector's first touched token
+                    rk[k] = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));                // rank_of(rv, i)
+                    old[k] = id[k] < V ? atomicOr(&cnt[rk[k]], kClaim) : kClaim;
+                    if (i < whole_end) {
+                        if (rf < stage_cap) vec[k] = stage[rf];
+                        else vec[k] = static_cast<const uint4*>(rv.base)[i >> lper];
+                    } else {
+                        const uint32_t b = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[i]
+                                                         : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]) << 16;
+                        vec[k] = make_uint4(b, b, b, b);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (old[k] & kClaim) continue;  // no such entry, or another entry of the same token got there first
+                    const uint32_t i = id[k];
+                    const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
+                    const bool whole = i < whole_end;
+                    uint32_t bits;
+                    if (!whole) bits = w[0];
+                    else bits = rv.dtype == 0 ? w[i & 3u] : ((i & 1u) ? w[(i & 7u) >> 1] & 0xffff0000u : w[(i & 7u) >> 1] << 16);
+                    const float raw = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits), -INFINITY) : -INFINITY;
+                    if (whole) {
+                        const uint32_t vb = i & ~(per - 1u);
+                        const uint32_t free_bits = (al[k] & ~tw[k]) >> (vb & 31u);  // allowed and untouched
+                        if (rv.dtype == 0) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float(w[e]));
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float((e & 1) ? w[e >> 1] & 0xffff0000u : w[e >> 1] << 16));
+                        }
+                    }
+                    const uint32_t cw = old[k], c = cw & 0xfffffu, n_bias = (cw >> 20) & 0x7ffu;
+                    float x = raw;
+                    if (n_bias) {
+                        // the bias values of this id, added one by one in listed order, starting at its first entry
+                        uint32_t j = first[rk[k]];
+                        x = __fadd_rn(x, bias_vals[j]);
+                        if (n_bias > 1u)
+                            for (++j; j < nb; ++j)
+                                if (static_cast<uint32_t>(bias_ids[j]) == i) x = __fadd_rn(x, bias_vals[j]);
+                    }
+                    if (c) {
+                        x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                        x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
+                    }
+                    pv[rk[k]] = x;
+                    first[rk[k]] = i;  // pid
+                    ma = fmaxf(ma, x);
+                    if (move) {
+                        const float t0 = bin_coord(aq_, c64_, raw, tail_own), t1 = bin_coord(aq_, c64_, x, tail_own);
+                        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
+                        atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
+                    }
+                }
+            }
+        };
+        static_assert(kHid == 4, "take4 takes its first round from hid");
+        take4(hist_ids, nh, true);
+        take4(bias_ids, nb, false);
+    };
     // f(token, adjusted logit) for every touched token. The single-sweep kernel keeps praw / pid in LDS of their own;
     // in the three-pass kernel that LDS is the histogram's, so it walks the set bits of the bitmap instead.
     auto replay_touched = [&](auto&& f) {
@@ -884,19 +988,20 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m);
         __syncthreads();
         WS_MARK(8);
-        gather_and_adjust(stage, swept ? stage_cap : 0u);
-        WS_MARK(9);
-        if (swept) {
-            m = block_max(m, red_f);  // over the vectors of the row that hold no touched token (allow mask applied)
-            // touched tokens: out of the bin of the raw logit, into the bin of the adjusted one
-            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
-                const float t0 = bin_coord(aq, c64, praw[r], tail_f), t1 = bin_coord(aq, c64, pv[r], tail_f);
-                atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
-                atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
+        {
+            float ma, mu;
+            collect_fused(stage, swept ? stage_cap : 0u, swept, aq, c64, ma, mu);
+            WS_MARK(9);
+            // m: over the vectors of the row that hold no touched token (allow mask applied); mu: the untouched tokens of
+            // the others; ma: the adjusted tokens. The barriers of the reduction also end the moves in the histogram.
+            float m_all = fmaxf(fmaxf(m, mu), ma);
+            block_max2(m_all, ma, red_f, reinterpret_cast<float*>(red_u));
+            m_adj = ma;
+            if (swept) {
+                m = m_all;
+                // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
+                cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
             }
-            m = fmaxf(fmaxf(m, m_near), m_adj);
-            // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
-            cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
         }
         if (!cached) {
             m = -INFINITY;
