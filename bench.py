@@ -22,13 +22,44 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MODE = 0
-# HBM bytes per launch of ws::sample_batch_kernel on the tile workload: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
-# what the same counter reads for a 256 MiB device copy (x2.000 and x1.000); the runs are summarised under profiles/
-TRAFFIC_BYTES = {("tile", "auto"): 168.0e6, ("tile", "fused"): 168.0e6, ("tile", "exact"): 524.7e6}
+# HBM bytes per launch of ws::sample_batch_kernel: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter
+# reads for a 256 MiB device copy; measured for one build of the kernel and only reported for that build (the digest
+# of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
+TRAFFIC = {
+    # (workload, mode): (bytes per launch, profiles/ file, sha256[:16] of whirl-llm_amd/csrc/ws_sample.h at the time)
+}
+
+
+def workloads():
+    """The package's workload generators (no CPU sampler behind them)."""
+    from __graft_entry__ import load_package
+    load_package()
+    import importlib
+    return importlib.import_module("whirl_llm_amd.workloads")
+
+
+def checker():
+    """tests/gpu_cases.py: the oracle over the same workloads. Only the CPU legs of the bench use it."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import gpu_cases
+    return gpu_cases
+
+
+def kernel_digest():
+    import hashlib
+    with open(os.path.join(ROOT, "whirl-llm_amd", "csrc", "ws_sample.h"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic_for(workload, mode):
+    t = TRAFFIC.get((workload, mode))
+    if not t or t[2] != kernel_digest():
+        return None, None
+    return t[0], "profiles/" + t[1]
 
 
 def algorithmic_bytes(c):
@@ -45,7 +76,7 @@ def algorithmic_bytes(c):
 
 def time_gpu(c, steps, warmup, rng_mode=1):
     import torch
-    import gpu_cases as gc
+    gc = workloads()
     d = gc.upload(c)
     smp = gc.sampler_for(c, d, rng_mode, mode=MODE)
     for _ in range(warmup):
@@ -63,15 +94,21 @@ def time_gpu(c, steps, warmup, rng_mode=1):
     return smp, wall_ms, kern_ms
 
 
+def device_report(smp):
+    """What the device says about its own launch: rows with a decision within tolerance of a boundary, failed rows."""
+    from __graft_entry__ import load_package
+    m = load_package()
+    fl = smp.flags.cpu().numpy()
+    return dict(device_near_flags=int(((fl & m.FLAG_NEAR) != 0).sum()),
+                device_failed_rows=int(((fl & (m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED)) != 0).sum()))
+
+
 def parity_sample(c, smp, n_check, rng_mode=1):
-    import gpu_cases as gc
+    """CPU leg: n_check rows of the launch against the oracle (token, kept count, probability, maximum, normaliser)."""
+    gc = checker()
     rows = list(range(0, c["rows"], max(1, c["rows"] // n_check)))[:n_check]
     res = gc.compare_rows(c, smp, rows, rng_mode, check_kept=False)
-    import torch
-    fl = smp.flags.cpu().numpy()
-    m = gc.pkg()
-    res["device_near_flags"] = int(((fl & m.FLAG_NEAR) != 0).sum())
-    res["device_failed_rows"] = int(((fl & (m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED)) != 0).sum())
+    res.update(device_report(smp))
     return res
 
 
@@ -80,7 +117,7 @@ def _cpu_rows(c, lib, port, kind_rows, budget_s):
     are spent; returns (rows done, seconds of sampler work)."""
     import ctypes as C
     import numpy as np
-    import gpu_cases as gc
+    gc = checker()
     import wo
     done, t_used = 0, 0.0
     V = c["V"]
@@ -111,6 +148,7 @@ def cpu_baseline(c, budget_s=9.0, budget_all_s=6.0):
     work are spent. `all_cores` repeats it with the rows sharded over the box's cores (rows are independent)."""
     import itertools
     from concurrent.futures import ThreadPoolExecutor
+    checker()
     import wo
     ref = wo.load("ref")
     lib = ref if ref is not None else wo.load("oracle")
@@ -119,27 +157,42 @@ def cpu_baseline(c, budget_s=9.0, budget_all_s=6.0):
     R = c["rows"]
     seq = ((k % R, k // R) for k in itertools.count())
     done, t_used = _cpu_rows(c, lib, port, seq, budget_s)
-    # the library calls release the interpreter lock, so plain threads shard the rows
-    n_thr = max(1, min(16, os.cpu_count() or 1))
+    # the library calls release the interpreter lock, so plain threads shard the rows; one thread per CPU this process
+    # may run on, at most 16 (a one-GPU box's share of its host, whatever the host's total)
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    n_thr = max(1, min(16, avail))
     t0 = time.perf_counter()
     with ThreadPoolExecutor(n_thr) as ex:
         parts = list(ex.map(lambda w: _cpu_rows(c, lib, port, (((w + k * n_thr) % R, (w + k * n_thr) // R) for k in itertools.count()),
                                                 budget_all_s), range(n_thr)))
     wall = time.perf_counter() - t0
     done_all = sum(p[0] for p in parts)
-    return dict(value=done / t_used, unit="rows/s", cores=1, kind=kind,
+    return dict(value=done / t_used, unit="rows/s", cores=1, kind=kind, cpu_model=cpu_model(), host_logical_cpus=os.cpu_count(),
+                cpus_available_to_this_process=avail,
                 sample=f"{done} rows (the rows of the same batch in order, wrapping), penalties + escalation "
                        f"256/16384/full + filter + draw, {t_used:.2f} s on one host thread",
                 all_cores=dict(value=done_all / wall, unit="rows/s", cores=n_thr,
                                sample=f"{done_all} rows sharded over {n_thr} threads, {wall:.2f} s wall clock"))
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
+
+
 def run_workload(name, steps, warmup, check_rows):
-    import gpu_cases as gc
+    gc = workloads()
     make = dict(tile=gc.make_tile, cfg1=gc.make_cfg1, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
     c = make()
     smp, wall_ms, kern_ms = time_gpu(c, steps, warmup)
-    par = parity_sample(c, smp, check_rows) if check_rows else None
+    par = parity_sample(c, smp, check_rows) if check_rows else device_report(smp)
     ab = algorithmic_bytes(c)
     return c, dict(workload=name, rows=c["rows"], vocab=c["V"], dtype=c["dtype"], ms_per_step=wall_ms, kernel_ms=kern_ms,
                    rows_per_s=c["rows"] / (wall_ms * 1e-3), algorithmic_MB=ab / 1e6, achieved_GBs=ab / (kern_ms * 1e-3) / 1e9,
@@ -151,8 +204,8 @@ def reference_kernels(steps):
     picks on 1 / 32 / 256 rows, topk_rows with the engine's two list sizes on 1 / 32 rows, the drafter's dflash_topk. Synthetic N(0, sigma 2) logits."""
     import ctypes as C
     import torch
-    import gpu_cases as gc
-    m = gc.pkg()
+    from __graft_entry__ import load_package
+    m = load_package()
     L, S, P = m.lib(), m._stream, m._p
     V = 151936
     out = []
@@ -213,8 +266,8 @@ def spec_verify_workload(steps, warmup):
     and, per sequence, the rejected position's p and q rows (or the last position's p row when every draft passed)."""
     import ctypes as C
     import torch
-    import gpu_cases as gc
-    m = gc.pkg()
+    from __graft_entry__ import load_package
+    m = load_package()
     n_seq, n_pos, V = 32, 9, 151936
     g = torch.Generator(device="cuda:0").manual_seed(312)
     tl = torch.randn((n_seq, n_pos, V), device="cuda:0", generator=g) * 2
@@ -256,7 +309,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="tile", choices=["tile", "cfg1", "cfg2", "cfg3", "cfg5"])
-    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="leave out the CPU legs: cpu_baseline and the oracle check of sampled rows")
     ap.add_argument("--no-also", action="store_true")
     ap.add_argument("--check-rows", type=int, default=8)
     ap.add_argument("--mode", default="auto", choices=["auto", "exact", "fused"], help="ws_batch.mode for every workload")
@@ -288,16 +341,19 @@ def main():
         return
     global MODE
     MODE = {"auto": 0, "exact": 1, "fused": 2}[a.mode]
-    c, main_res = run_workload(a.workload, a.steps, a.warmup, a.check_rows)
+    check = 0 if a.no_cpu else a.check_rows
+    c, main_res = run_workload(a.workload, a.steps, a.warmup, check)
     also = []
     if not a.no_also:
-        for w in ("cfg1", "cfg2", "cfg3"):
+        for w in ("cfg1", "cfg2", "cfg3", "cfg5"):
             if w != a.workload:
-                _, r = run_workload(w, max(20, a.steps // 4), 5, 1 if w == "cfg1" else 4)
+                n_chk = 0 if a.no_cpu else (1 if w == "cfg1" else 4)
+                _, r = run_workload(w, 20 if w == "cfg5" else max(20, a.steps // 4), 5, n_chk)
                 also.append(r)
         also.append(spec_verify_workload(max(20, a.steps // 4), 5))
     cpu = None if a.no_cpu else cpu_baseline(c)
     ab = main_res["algorithmic_MB"] * 1e6
+    traffic, traffic_source = traffic_for(a.workload, a.mode)
     out = {
         "metric": "sampled rows/s (fused penalties + top-p sampler, batch 256 x vocab 151936 fp32)",
         "value": main_res["rows_per_s"], "unit": "rows/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -305,10 +361,11 @@ def main():
         "dtype": "f32" if c["dtype"] == "f32" else "bf16->f32", "data": "synthetic",
         "config": {"workload": a.workload, "rows": c["rows"], "vocab": c["V"], "logits": c["dtype"],
                    "history_ids_per_row": 0 if c["hist"] is None else int(c["hist"].shape[1]),
-                   "filters": "see tests/gpu_cases.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
+                   "filters": "see whirl-llm_amd/workloads.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
                    "sweep_mode": a.mode},
         "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": main_res["frac_of_hbm_peak"], "traffic": TRAFFIC_BYTES.get((a.workload, a.mode)), "kernel": "ws::sample_batch_kernel",
+                     "frac": main_res["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "ws::sample_batch_kernel", "kernel_source_digest": kernel_digest(),
                      "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},
         "cpu_baseline": cpu,
         "parity": main_res["parity"],

@@ -44,9 +44,16 @@ public:
 
     void setAdjust(const RowAdjust& a);  // applies to the rows prepared from now on
 
-    // Filters rows s.row_base + r0 .. + n - 1 in one device launch and keeps the results on the host: the prepareRow
-    // calls that follow for these rows, with the same temperature and filters in `s`, cost no device call. The verify
-    // rows of a sequence share their sampler, so the engine calls this once before Acceptor::sample.
+    // The logits buffer has new contents (the model ran another step): nothing filtered before is used again. The
+    // device allocations stay. One object serves the whole life of a logits buffer; rows that prefetchRows filtered
+    // and no prepareRow asked for are dropped here.
+    void newCycle();
+
+    // Filters rows s.row_base + r0 .. + n - 1 in one device launch and keeps the results on the host: the first prepareRow
+    // that follows for each of these rows, with the same temperature and filters in `s`, costs no device call and uses
+    // the result up (a second prepareRow of the same row goes to the device again, so a rewritten logits buffer is never
+    // answered from an old launch). The verify rows of a sequence share their sampler, so the engine calls this once
+    // before Acceptor::sample.
     void prefetchRows(const Sampler& s, std::uint32_t r0, std::uint32_t n);
 
     void prepareRow(Sampler& s, std::uint32_t r) override;

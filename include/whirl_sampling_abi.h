@@ -258,7 +258,7 @@ typedef struct ws_spec_verify {
     int32_t rng;
     int32_t* out_tokens; /* [n_seq][n_pos] */
     int32_t* n_accepted; /* [n_seq] */
-    uint32_t* flags;     /* [n_seq] WS_FLAG_NEAR_DRAW */
+    uint32_t* flags;     /* [n_seq] WS_FLAG_NEAR_DRAW; WS_FLAG_BAD_PARAM: a tested draft id outside [0, vocab), which counts as rejected */
     void* workspace;
     uint64_t workspace_bytes;
     double tol;

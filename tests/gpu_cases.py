@@ -1,6 +1,6 @@
-"""Synthetic workloads of the sampling path (the configurations BASELINE.json lists), the oracle run over them and
-the comparison rules. Shared by the GPU tests, __graft_entry__.smoke() and bench.py's correctness / cpu_baseline legs.
-Test infrastructure: the oracle is only ever the checker here."""
+"""The oracle run over the synthetic workloads of the sampling path (whirl-llm_amd/workloads.py) and the comparison
+rules. Shared by the GPU tests, __graft_entry__.smoke() and bench.py's CPU legs. Test infrastructure: the oracle is
+only ever the checker here."""
 import ctypes as C
 import os
 import sys
@@ -13,108 +13,22 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 import wo  # noqa: E402
 
-DATA_SEED = 0xC0FFEE
-SAMPLE_SEED = 1234
-
 
 def pkg():
     from __graft_entry__ import load_package
     return load_package()
 
 
-def f32_to_bf16_bits(x):
-    """Round-to-nearest-even float32 -> bfloat16 bit patterns (uint16)."""
-    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
-    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+def _workloads():
+    pkg()
+    import importlib
+    return importlib.import_module("whirl_llm_amd.workloads")
 
 
-def bf16_bits_to_f32(b):
-    return (b.astype(np.uint32) << 16).view(np.float32)
-
-
-def _common(rows, rng, V, n_hist, n_bias):
-    c = dict(rows=rows, V=V)
-    c["seed"] = (np.uint64(SAMPLE_SEED) + np.arange(rows, dtype=np.uint64) * np.uint64(7919)).astype(np.uint64)
-    c["step"] = rng.integers(0, 5000, rows).astype(np.uint64)
-    c["hist"] = rng.integers(0, V, (rows, n_hist)).astype(np.int32) if n_hist else None
-    if n_bias:
-        c["bias_ids"] = np.stack([rng.choice(V, n_bias, replace=False) for _ in range(rows)]).astype(np.int32)
-        c["bias_vals"] = rng.uniform(-5, 5, (rows, n_bias)).astype(np.float32)
-    else:
-        c["bias_ids"] = c["bias_vals"] = None
-    c["allow"] = None
-    c["dtype"] = "f32"
-    return c
-
-
-def make_cfg1(V=151936):
-    """configs[0]: batch 1, N(0, sigma 2) with 5 tokens at +12, 256-id history, repetition 1.1, T 0.8, top-k 40, top-p 0.95."""
-    rng = np.random.default_rng(DATA_SEED + 1)
-    c = _common(1, rng, V, 256, 0)
-    x = (rng.standard_normal((1, V)) * 2).astype(np.float32)
-    x[0, rng.choice(V, 5, replace=False)] = 12.0
-    c.update(name="cfg1", logits=x, inv_t=np.array([1 / 0.8], np.float32), top_k=np.array([40], np.uint32),
-             top_p=np.array([0.95]), min_p=np.array([0.0]), rep=np.array([1.1], np.float32),
-             pres=np.zeros(1, np.float32), freq=np.zeros(1, np.float32))
-    return c
-
-
-def make_cfg2(rows=64, V=151936, n_hist=4096, n_bias=300):
-    """configs[1]: N(0, sigma 2) fp32, T in [0.5, 1.2], top-k in {0, 20, 50}, top-p in [0.8, 1], min-p 0.05, repetition /
-    presence / frequency penalties over a 4096-id history, 300 bias entries in [-5, 5]."""
-    rng = np.random.default_rng(DATA_SEED + 2)
-    c = _common(rows, rng, V, n_hist, n_bias)
-    c.update(name="cfg2", logits=(rng.standard_normal((rows, V)) * 2).astype(np.float32),
-             inv_t=(1.0 / rng.uniform(0.5, 1.2, rows)).astype(np.float32),
-             top_k=rng.choice([0, 20, 50], rows).astype(np.uint32), top_p=rng.uniform(0.8, 1.0, rows),
-             min_p=np.full(rows, 0.05), rep=np.full(rows, 1.1, np.float32), pres=np.full(rows, 0.3, np.float32),
-             freq=np.full(rows, 0.02, np.float32))
-    return c
-
-
-def make_cfg3(rows=256, V=151936, n_hist=2048):
-    """configs[2]: bf16 Zipfian logits -1.1 ln(rank) + N(0, 0.3) over a random permutation, top-k off, top-p 0.9,
-    penalties over a 2048-id history."""
-    rng = np.random.default_rng(DATA_SEED + 3)
-    c = _common(rows, rng, V, n_hist, 0)
-    base = (-1.1 * np.log(np.arange(1, V + 1, dtype=np.float64))).astype(np.float32)
-    x = np.empty((rows, V), np.float32)
-    for r in range(rows):
-        x[r, rng.permutation(V)] = base
-        x[r] += (rng.standard_normal(V) * 0.3).astype(np.float32)
-    c.update(name="cfg3", dtype="bf16", logits=f32_to_bf16_bits(x), inv_t=np.ones(rows, np.float32), top_k=np.zeros(rows, np.uint32),
-             top_p=np.full(rows, 0.9), min_p=np.zeros(rows), rep=np.full(rows, 1.1, np.float32),
-             pres=np.full(rows, 0.3, np.float32), freq=np.full(rows, 0.02, np.float32))
-    return c
-
-
-def make_tile(rows=256, V=151936, n_hist=2048):
-    """The north-star tile: fp32 N(0, sigma 2), repetition / presence / frequency penalties over a 2048-id history,
-    T in [0.7, 1.0], top-p 0.9, top-k and min-p off (a full-vocabulary mass select on every row)."""
-    rng = np.random.default_rng(DATA_SEED + 6)
-    c = _common(rows, rng, V, n_hist, 0)
-    c.update(name="tile", logits=(rng.standard_normal((rows, V)) * 2).astype(np.float32),
-             inv_t=(1.0 / rng.uniform(0.7, 1.0, rows)).astype(np.float32), top_k=np.zeros(rows, np.uint32),
-             top_p=np.full(rows, 0.9), min_p=np.zeros(rows), rep=np.full(rows, 1.1, np.float32),
-             pres=np.full(rows, 0.3, np.float32), freq=np.full(rows, 0.02, np.float32))
-    return c
-
-
-def make_cfg5(rows=1024, V=262144, n_hist=8192, n_bias=500):
-    """configs[4]: fp32 N(0, sigma 3), allow-mask with 90 % of the tokens at -inf, 500 bias entries, 8192-id history,
-    top-k 1000, top-p 0.95, T 1."""
-    rng = np.random.default_rng(DATA_SEED + 5)
-    c = _common(rows, rng, V, n_hist, n_bias)
-    allow = np.packbits(rng.random((rows, V)) < 0.1, axis=1, bitorder="little").view(np.uint32)
-    c.update(name="cfg5", logits=(rng.standard_normal((rows, V)) * 3).astype(np.float32), inv_t=np.ones(rows, np.float32),
-             top_k=np.full(rows, 1000, np.uint32), top_p=np.full(rows, 0.95), min_p=np.zeros(rows),
-             rep=np.full(rows, 1.1, np.float32), pres=np.full(rows, 0.3, np.float32), freq=np.full(rows, 0.02, np.float32),
-             allow=np.ascontiguousarray(allow))
-    return c
-
-
-def row_f32(c, r):
-    return bf16_bits_to_f32(c["logits"][r]) if c["dtype"] == "bf16" else c["logits"][r].astype(np.float32)
+workloads = _w = _workloads()
+f32_to_bf16_bits, bf16_bits_to_f32, row_f32 = _w.f32_to_bf16_bits, _w.bf16_bits_to_f32, _w.row_f32
+make_cfg1, make_cfg2, make_cfg3, make_tile, make_cfg5 = _w.make_cfg1, _w.make_cfg2, _w.make_cfg3, _w.make_tile, _w.make_cfg5
+upload, sampler_for = _w.upload, _w.sampler_for
 
 
 def oracle_row(c, r, rng_mode, lib=None):
@@ -137,57 +51,15 @@ def oracle_row(c, r, rng_mode, lib=None):
     return out, cands[:out.n_kept].copy(), x
 
 
-def upload(c, device="cuda:0"):
-    """numpy case -> dict of device tensors in the layouts ws_batch expects."""
-    import torch
-    d = {}
-    rows = c["rows"]
-    if c["dtype"] == "bf16":
-        d["logits"] = torch.from_numpy(c["logits"].view(np.int16)).to(device).view(torch.bfloat16)
-    else:
-        d["logits"] = torch.from_numpy(c["logits"]).to(device)
-    d["inv_t"] = torch.from_numpy(c["inv_t"]).to(device)
-    d["top_k"] = torch.from_numpy(c["top_k"].view(np.int32)).to(device)
-    d["top_p"] = torch.from_numpy(np.ascontiguousarray(c["top_p"], np.float64)).to(device)
-    d["min_p"] = torch.from_numpy(np.ascontiguousarray(c["min_p"], np.float64)).to(device)
-    d["seed"] = torch.from_numpy(c["seed"].view(np.int64)).to(device)
-    d["step"] = torch.from_numpy(c["step"].view(np.int64)).to(device)
-    for k in ("rep", "pres", "freq"):
-        d[k] = torch.from_numpy(c[k]).to(device)
-    d["max_hist"] = d["max_bias"] = 0
-    d["hist"] = d["hist_off"] = d["bias_ids"] = d["bias_vals"] = d["bias_off"] = d["allow"] = None
-    if c["hist"] is not None:
-        n = c["hist"].shape[1]
-        d["hist"] = torch.from_numpy(np.ascontiguousarray(c["hist"]).reshape(-1)).to(device)
-        d["hist_off"] = torch.arange(0, (rows + 1) * n, n, dtype=torch.int32, device=device)
-        d["max_hist"] = n
-    if c["bias_ids"] is not None:
-        n = c["bias_ids"].shape[1]
-        d["bias_ids"] = torch.from_numpy(np.ascontiguousarray(c["bias_ids"]).reshape(-1)).to(device)
-        d["bias_vals"] = torch.from_numpy(np.ascontiguousarray(c["bias_vals"]).reshape(-1)).to(device)
-        d["bias_off"] = torch.arange(0, (rows + 1) * n, n, dtype=torch.int32, device=device)
-        d["max_bias"] = n
-    if c["allow"] is not None:
-        d["allow"] = torch.from_numpy(c["allow"].view(np.int32)).to(device)
-    d["race"] = torch.from_numpy(np.ascontiguousarray(c["race"], np.int32)).to(device) if c.get("race") is not None else None
-    return d
-
-
-def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0):
-    m = pkg()
-    return m.BatchSampler(d["logits"], d["inv_t"], d["seed"], d["step"], top_k=d["top_k"], top_p=d["top_p"], min_p=d["min_p"],
-                          rng=rng_mode, hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
-                          bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], max_hist=d["max_hist"],
-                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"))
-
-
 def compare_rows(c, smp, rows_to_check, rng_mode, check_kept=True, near_tol=1e-6, verbose=False):
     """Device results of the given rows against the oracle. Returns a dict of counters; raises AssertionError on a
-    mismatch that is not explained by a decision within `near_tol` of a boundary on the oracle side.
+    mismatch the device did not report: a row whose token or kept count differs from the oracle's must carry one of
+    the device's own WS_FLAG_NEAR_* bits (a decision within 1e-6 of a boundary, which is what the flags are for).
 
     Bars: token ids identical; kept-set ids identical (as sets, device order is ascending id) and their
     penalty-applied logits bit-identical; n_kept identical; probability of the token within 1e-6 relative;
-    max logit bit-identical, float normaliser within the 1e-6 relative the probabilities are held to."""
+    max logit bit-identical, float normaliser within the 1e-6 relative the probabilities are held to (both also on
+    the rows that are reported near a boundary)."""
     import torch
     m = pkg()
     torch.cuda.synchronize()
@@ -199,26 +71,28 @@ def compare_rows(c, smp, rows_to_check, rng_mode, check_kept=True, near_tol=1e-6
     mg = smp.margin.cpu().numpy()
     kid = smp.kept_ids.cpu().numpy() if smp.kept_ids is not None else None
     klg = smp.kept_logits.cpu().numpy() if smp.kept_logits is not None else None
-    res = dict(rows=0, exact=0, near_oracle=0, near_device=0, failed_flags=0, max_prob_rel=0.0)
+    res = dict(rows=0, exact=0, differ=0, near_oracle=0, near_device=0, failed_flags=0, max_prob_rel=0.0)
     for r in rows_to_check:
         o, kept, xpen = oracle_row(c, r, rng_mode)
         res["rows"] += 1
         hard = fl[r] & (m.FLAG_ALL_MASKED | m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM)
         assert not hard, f"{c['name']} row {r}: device flags {fl[r]:#x}"
         near_o = min(o.margin, o.margin_top_p, o.margin_min_p) < near_tol
+        near_d = bool(fl[r] & m.FLAG_NEAR)
         res["near_oracle"] += bool(near_o)
-        res["near_device"] += bool(fl[r] & m.FLAG_NEAR)
+        res["near_device"] += near_d
         ok = tok[r] == o.token and nk[r] == o.n_kept
         if verbose:
             print(f"row {r}: tok {tok[r]}/{o.token} n {nk[r]}/{o.n_kept} p {prob[r]:.6g}/{o.prob:.6g} flags {fl[r]:#x} "
                   f"margins dev {mg[r]} oracle {o.margin:.3g} {o.margin_top_p:.3g} {o.margin_min_p:.3g} big {o.big_used} full {o.full_used}")
-        if not ok:
-            assert near_o, (f"{c['name']} row {r}: token {tok[r]} vs {o.token}, kept {nk[r]} vs {o.n_kept}, oracle margins "
-                            f"{o.margin:.3g} {o.margin_top_p:.3g} {o.margin_min_p:.3g}, device margins {mg[r]}")
-            continue
-        res["exact"] += 1
         assert st[r, 0] == o.m, f"row {r}: max {st[r, 0]} vs {o.m}"
         assert abs(st[r, 1] - o.sum) <= 1e-6 * o.sum, f"row {r}: sum {st[r, 1]} vs {o.sum}"
+        if not ok:
+            assert near_d, (f"{c['name']} row {r}: token {tok[r]} vs {o.token}, kept {nk[r]} vs {o.n_kept} and no WS_FLAG_NEAR_* bit "
+                            f"(flags {fl[r]:#x}); oracle margins {o.margin:.3g} {o.margin_top_p:.3g} {o.margin_min_p:.3g}, device margins {mg[r]}")
+            res["differ"] += 1
+            continue
+        res["exact"] += 1
         rel = abs(float(prob[r]) - float(o.prob)) / float(o.prob)
         res["max_prob_rel"] = max(res["max_prob_rel"], rel)
         assert rel <= 1e-6, f"row {r}: prob {prob[r]} vs {o.prob}"

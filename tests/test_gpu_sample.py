@@ -1,8 +1,9 @@
 """GPU: the fused batched sampler through the C ABI against the CPU oracle on identical seeded inputs.
 
 Bars (gpu_cases.compare_rows): token ids, kept-set sizes, kept id sets and penalty-applied logits identical; the
-token's probability within 1e-6 relative; rows whose decision sits within 1e-6 of a boundary on the oracle side
-may differ and are counted."""
+token's probability within 1e-6 relative. A row may differ from the oracle only where the device itself reports a
+decision within 1e-6 of a boundary (WS_FLAG_NEAR_*), and every test states how many such rows it allows: none, except
+the bf16 rows with ties at the cut, where it is one."""
 import numpy as np
 import pytest
 import torch
@@ -15,13 +16,13 @@ pytestmark = pytest.mark.gpu
 MODES = [1, 0]  # WS_MODE_EXACT, WS_MODE_AUTO (the fused sweep wherever the batch qualifies)
 
 
-def run_case(c, rng_mode, rows=None, kept_cap=None, expect_near=0.05, mode=0):
+def run_case(c, rng_mode, rows=None, kept_cap=None, max_differ=0, mode=0):
     d = gc.upload(c)
     cap = c["V"] if kept_cap is None else kept_cap
     smp = gc.sampler_for(c, d, rng_mode, kept_cap=cap, mode=mode).run()
     rows = range(c["rows"]) if rows is None else rows
     res = gc.compare_rows(c, smp, rows, rng_mode)
-    assert res["exact"] >= (1 - expect_near) * res["rows"], res
+    assert res["differ"] <= max_differ and res["exact"] + res["differ"] == res["rows"], res
     return res, smp
 
 
@@ -43,7 +44,7 @@ def test_small_vocab_ties_and_duplicated_bias(mode):
     c["bias_ids"][:, 1] = c["bias_ids"][:, 0]
     c["bias_ids"][:, 5] = c["bias_ids"][:, 0]
     c["top_k"] = rng.choice([0, 1, 5, 40, 700], 16).astype(np.uint32)
-    res, _ = run_case(c, 1, expect_near=0.3, mode=mode)
+    res, _ = run_case(c, 1, mode=mode)
     print(res)
 
 
@@ -92,14 +93,14 @@ def test_open_rows_odd_shapes(mode):
     allowed tokens than the list holds."""
     for c in (_open(gc.make_cfg2(rows=8, V=200, n_hist=10, n_bias=4)), _open(gc.make_cfg2(rows=8, V=5003, n_hist=300, n_bias=24)),
               _open(gc.make_cfg3(rows=8, V=40000, n_hist=256)), _open(gc.make_cfg5(rows=8, V=32768, n_hist=400, n_bias=30))):
-        res, _ = run_case(c, 1, kept_cap=512, expect_near=0.2, mode=mode)
+        res, _ = run_case(c, 1, kept_cap=512, mode=mode)
         print(c["name"], res)
     c = _open(gc.make_tile(rows=6, V=8192, n_hist=64))
     for r in range(6):
         off = np.ones(8192, bool)
         off[np.random.default_rng(r).choice(8192, 100 + 40 * r, replace=False)] = False
         c["logits"][r][off] = -np.inf
-    res, _ = run_case(c, 1, kept_cap=512, expect_near=0.2, mode=mode)
+    res, _ = run_case(c, 1, kept_cap=512, mode=mode)
     print(res)
 
 
@@ -128,14 +129,14 @@ def test_race_draw_on_the_tile_shape_rows(mode):
     for c in (gc.make_tile(rows=6, V=151936, n_hist=2048), gc.make_cfg3(rows=6, V=40000, n_hist=256),
               gc.make_cfg5(rows=6, V=32768, n_hist=400, n_bias=30), gc.make_cfg2(rows=6, V=5003, n_hist=300, n_bias=24)):
         c["race"] = np.ones(6, np.int32)
-        res, _ = run_case(c, 1, kept_cap=64, expect_near=0.2, mode=mode)
+        res, _ = run_case(c, 1, kept_cap=64, max_differ=1 if c["name"] == "cfg3" else 0, mode=mode)
         print(c["name"], res)
 
 
 @pytest.mark.parametrize("mode", MODES)
 def test_bf16_rows(mode):
     c = gc.make_cfg3(rows=6, V=40000, n_hist=256)
-    res, _ = run_case(c, 1, expect_near=0.2, mode=mode)
+    res, _ = run_case(c, 1, max_differ=1, mode=mode)
     print(res)
 
 
@@ -283,6 +284,7 @@ def test_cfg1_shape(mode):
 @pytest.mark.parametrize("mode", MODES)
 def test_cfg2_full_size(mode):
     res, _ = run_case(gc.make_cfg2(), 1, mode=mode)
+    assert res["exact"] == 64, res
     print(res)
 
 
@@ -290,13 +292,15 @@ def test_cfg2_full_size(mode):
 def test_north_star_tile_full_size(mode):
     c = gc.make_tile()
     res, _ = run_case(c, 1, rows=range(256), kept_cap=c["V"], mode=mode)  # every row of the batch
+    assert res["exact"] == 256, res
     print(res)
 
 
 @pytest.mark.parametrize("mode", MODES)
 def test_cfg3_full_size(mode):
     c = gc.make_cfg3()
-    res, _ = run_case(c, 1, rows=range(256), expect_near=0.2, mode=mode)  # every row of the batch
+    res, _ = run_case(c, 1, rows=range(256), max_differ=1, mode=mode)  # every row of the batch
+    assert res["exact"] >= 255, res
     print(res)
 
 
@@ -330,11 +334,11 @@ def test_random_shapes_filters_and_masks_both_kernels():
     settings, temperatures and -inf masking, every case through WS_MODE_EXACT and WS_MODE_AUTO with either RNG: every
     row must give the oracle's token, kept set and probabilities (or be reported as a boundary case by the oracle)."""
     rng = np.random.default_rng(20240611)
-    seed0 = gc.DATA_SEED
+    seed0 = gc.workloads.DATA_SEED
     tot = dict(rows=0, exact=0)
     try:
         for case in range(16):
-            gc.DATA_SEED = int(rng.integers(1, 1 << 30))
+            gc.workloads.DATA_SEED = int(rng.integers(1, 1 << 30))
             kind = rng.choice(["cfg2", "cfg3", "cfg5", "tile"])
             V = int(rng.choice([1000, 4096, 8008, 32000, 50257, 65536, 100003, 163840, 200000]))
             rows = int(rng.integers(1, 6))
@@ -359,10 +363,10 @@ def test_random_shapes_filters_and_masks_both_kernels():
                     off = rng.random(V) < rng.choice([0.5, 0.9, 0.99])
                     c["logits"][r][off] = 0xFF80 if c["dtype"] == "bf16" else -np.inf
             for mode in MODES:
-                res, _ = run_case(c, int(rng.integers(0, 2)), kept_cap=min(V, 4096), expect_near=0.5, mode=mode)
+                res, _ = run_case(c, int(rng.integers(0, 2)), kept_cap=min(V, 4096), mode=mode)
                 tot["rows"] += res["rows"]
                 tot["exact"] += res["exact"]
     finally:
-        gc.DATA_SEED = seed0
+        gc.workloads.DATA_SEED = seed0
     print(tot)
-    assert tot["exact"] >= 0.9 * tot["rows"], tot
+    assert tot["exact"] == tot["rows"], tot

@@ -12,7 +12,8 @@
 namespace ws {
 
 constexpr uint32_t kSpecMaxSteps = 4096;  // 256-element steps of a row: vocab <= 1048576
-constexpr uint32_t kSpecNear = 4u;  // WS_FLAG_NEAR_DRAW
+constexpr uint32_t kSpecNear = 4u;      // WS_FLAG_NEAR_DRAW
+constexpr uint32_t kSpecBadDraft = 32u; // WS_FLAG_BAD_PARAM: a draft id outside [0, vocab); that draft is rejected
 
 struct SpecArgs {
     const float* p;
@@ -40,34 +41,43 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     int32_t* out = A.out_tokens + static_cast<size_t>(s) * P;
     const uint64_t seed = A.seed[s], step0 = A.step0[s];
 
-    if (P - 1u <= 64u) {
-        // accept chain, every draft at once: lane j of wave 0 fetches p_j(d_j), q_j(d_j) and tests its draft (one trip to
-        // memory instead of one per draft); the chain stops at the first lane that rejects
+    if (P - 1u < 64u) {
+        // accept chain, every draft at once (up to 63 drafts, so that wave 0 has a lane past the last one): lane j fetches
+        // p_j(d_j), q_j(d_j) and tests its draft (one trip to memory instead of one per draft); the chain stops at the
+        // first lane that rejects
         if (t < 64u) {
             const bool has = t + 1u < P;
             int32_t d = 0;
-            bool ok = false, near = false;
+            bool ok = false, near = false, bad = false;
             if (has) {
                 d = dr[t];
-                const double pj = p[static_cast<size_t>(t) * V + d], qj = q[static_cast<size_t>(t) * V + d];
-                const double lhs = batch_uniform(A.rng, seed, s, step0 + t, 0) * qj;
-                near = fabs(lhs - pj) < A.tol * pj;
-                ok = lhs < pj;
+                bad = d < 0 || static_cast<uint32_t>(d) >= V;
+                if (!bad) {
+                    const double pj = p[static_cast<size_t>(t) * V + d], qj = q[static_cast<size_t>(t) * V + d];
+                    const double lhs = batch_uniform(A.rng, seed, s, step0 + t, 0) * qj;
+                    near = fabs(lhs - pj) < A.tol * pj;
+                    ok = lhs < pj;
+                }
             }
-            const uint64_t rejects = __ballot(!ok);  // lanes past the last draft reject: there is always one
+            const uint64_t rejects = __ballot(!ok);  // lanes past the last draft reject: with at most 63 drafts there is always one
             const uint32_t j = static_cast<uint32_t>(__ffsll(static_cast<long long>(rejects)) - 1);
             const uint64_t tested = j >= 63u ? ~0ull : (2ull << j) - 1ull;  // drafts 0..j were looked at (j = P - 1: none there)
             const uint64_t nears = __ballot(near) & tested;
+            const uint64_t bads = __ballot(bad) & tested;
             if (t < j) out[t] = d;
             if (t == 0) {
                 s_u[0] = j;
-                s_u[1] = nears ? kSpecNear : 0u;
+                s_u[1] = (nears ? kSpecNear : 0u) | (bads ? kSpecBadDraft : 0u);
             }
         }
     } else if (t == 0) {  // accept chain, draft by draft
         uint32_t j = 0, fl = 0;
         for (; j + 1 < P; ++j) {
             const int32_t d = dr[j];
+            if (d < 0 || static_cast<uint32_t>(d) >= V) {
+                fl |= kSpecBadDraft;
+                break;
+            }
             const double pj = p[static_cast<size_t>(j) * V + d], qj = q[static_cast<size_t>(j) * V + d];
             const double lhs = batch_uniform(A.rng, seed, s, step0 + j, 0) * qj;
             if (fabs(lhs - pj) < A.tol * pj) fl |= kSpecNear;

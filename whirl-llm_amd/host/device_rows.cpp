@@ -128,6 +128,11 @@ void DeviceRows::setAdjust(const RowAdjust& a) {
     ready_.clear();  // rows filtered under the old penalties are of no use any more
 }
 
+void DeviceRows::newCycle() {
+    ready_.clear();
+    adjusted_row_ = kNoRow;
+}
+
 // Parameters of `n` rows that share sampler `s` and the current penalties, and the penalty lists once per row, go to
 // the device (the lists are replicated because a batch addresses them through one ascending offset array).
 void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
@@ -272,15 +277,18 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     if (gr >= rows_) throw DeviceError("prepareRow", WS_E_INVALID, "prepareRow: row out of range");
     s.row = gr;
     adjusted_row_ = kNoRow;
-    const Ready* q = nullptr;
+    Ready* q = nullptr;
     const bool same = ready_key_.inv_t == s.inv_t && ready_key_.top_k == s.top_k && ready_key_.top_p == s.top_p && ready_key_.min_p == s.min_p;
     if (same)
-        for (const Ready& c : ready_)
+        for (Ready& c : ready_)
             if (c.gr == gr) q = &c;
     if (!q) {
         filterOnDevice(s, gr, 1);
         q = &ready_[0];
     }
+    // A filtered row serves one prepareRow: the model rewrites the logits buffer every step, and a row kept beyond its
+    // use would hand last step's candidates to the next cycle's call for the same row.
+    q->gr = kNoRow;
     last_flags_ = q->flags;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
     const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
