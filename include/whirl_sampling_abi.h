@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define WS_ABI_VERSION 1
+#define WS_ABI_VERSION 2
 
 enum {
     WS_OK = 0,
@@ -126,10 +126,23 @@ enum {
     WS_FLAG_ALL_MASKED = 1u << 3,  /* every logit of the row is -inf / NaN: token = -1 */
     WS_FLAG_OVERFLOW = 1u << 4,    /* more tied / clustered candidates at a cut than the kernel resolves: token = -1 */
     WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
-    WS_FLAG_OPEN = 1u << 6         /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
+    WS_FLAG_OPEN = 1u << 6,        /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order
                                       (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
+    WS_FLAG_APPROX_ENTROPY = 1u << 7 /* `entropy` counts the kept tokens outside the gathered bins at the middle of their
+                                      histogram bin (each within 1/128 of its place: the entropy is within 1/128 absolute,
+                                      usually far closer) instead of one by one; rows whose kept set a
+                                      top-k bounds are always exact */
 };
+
+/* What a caller does with the WS_FLAG_NEAR_* bits: nothing has to be done. A row that carries one still has the
+ * token, kept count and probability the kernel computed - they are the kernel's best answer and the same on every run.
+ * The bit only says that the deciding comparison (cumulative mass against top-p, a probability against the min-p floor,
+ * the uniform against a CDF step) came out within `tol` relative of the other way, so a sampler that sums in another
+ * order or precision - the reference's host sampler sums in double, candidate by candidate - may land on the neighbouring
+ * candidate. Both answers are draws from distributions that differ by less than `tol`; a serving engine uses the token as
+ * it is. A test harness that compares with another implementation counts such rows instead of failing on them. Rows
+ * without the bit agree with the reference's sampler exactly. */
 
 /* One batch of rows. Everything per row is a device array of `rows` entries (SoA); a NULL array means the stated
  * default for every row. The engine fills these from what it already keeps per slot: Sampler fields
@@ -185,6 +198,18 @@ typedef struct ws_batch {
                                src/sampling/sampler.cpp:80-106: argmin of E(token) / p(token) over the kept set, E keyed by
                                (seed, step, token); an open row races over its 256 candidates when the uniform falls on
                                their mass, else walks the rest of the row) instead of the inverse CDF (NULL: none) */
+    /* ---- since ABI version 2 */
+    const uint32_t* hist_len;   /* per row: ids in the row's history, which then is hist[hist_off[r] .. hist_off[r] + hist_len[r])
+                                   and hist_off needs `rows` entries only (NULL: hist_off[r + 1] - hist_off[r]). Rows may share
+                                   and overlap their windows: the verify rows of a sequence read its device history
+                                   (ws_history) at growing lengths. */
+    const int32_t* query;       /* per row: a token whose probability is asked for, < 0 = none (NULL: none) */
+    double* query_prob;         /* out (may be NULL): probability of `query` under the row's filtered distribution, as
+                                   probOf gives it (src/sampling/sampler.cpp:108-116): its renormalised share when it is in
+                                   the kept set, 0 when it is not; on an open row its share of the whole row */
+    double* entropy;            /* out (may be NULL): -sum p ln p over the kept set (renormalised p; an open row: over its
+                                   256 candidates with their shares of the whole row), what the typical acceptance rule
+                                   compares with (src/sampling/acceptor.cpp:77-84). See WS_FLAG_APPROX_ENTROPY. */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
@@ -216,19 +241,61 @@ typedef struct ws_adjust {
 
 int ws_adjust_rows(void* stream, const ws_adjust* a);
 
-/* Draft acceptance on the device for the plain sampling rule. Stands in for the host loop Acceptor::sample
- * (src/sampling/acceptor.cpp:63-100, rule "sample": no race, no typical acceptance), which samples output index
- * n_gen + acc from verify row acc and accepts while the token equals the draft. Each output index draws from its own
- * counter (src/sampling/acceptor.h:10-12), so the caller samples all verify rows of all sequences in one
- * ws_sample_batch launch - row of position j of a sequence: step = n_gen + j, seed and filters of the sequence - and
- * this call turns the tokens into counts, with no host round trip in between. Per sequence s, control area
- * c = ctl_all + area[s] (layout above): nd = c[WS_CTL_ND] clamped to 0..15, drafts c[WS_CTL_DRAFTS .. + nd).
- *   acc = number of leading positions j < nd whose token equals draft j; chosen = token of position acc;
- *   c[WS_CTL_ROWS + j] = token of position j for j <= acc (the words the greedy path fills with row argmaxes,
- *   src/model/qwen35/forward/mtp_verify.cpp:226); n_accepted[s] = acc; chosen[s].
- *   status[s] = WS_ACCEPT_HOST when a position up to the stop has no usable token (token < 0): the host then runs
- *   Acceptor::sample for that sequence. */
-enum { WS_ACCEPT_OK = 0, WS_ACCEPT_HOST = 1 };
+/* A sequence's token history on the device (not in the reference, which keeps Slot::cache_tokens on the host,
+ * src/server/engine_slot.h:38-65, and appends to it after every cycle, src/server/engine_decode.cpp:548-549). Slot i owns
+ * tokens[i * cap .. (i + 1) * cap): the first len[i] entries are the tokens the model holds, entry len[i] is the token
+ * that goes in next (`next`; the caller writes it when the slot starts, the accept kernels write it afterwards), behind it
+ * ws_history_stage places the drafts of the running cycle. The accept kernels append what a cycle kept - next, the accepted
+ * drafts - set the chosen token as the new next and advance n_gen, so the penalties (ws_batch.hist) and the repeat guard
+ * of the next cycle read it in place: no per-cycle upload. n_slots * cap must stay below 2^32. */
+typedef struct ws_history {
+    int32_t* tokens;      /* device [n_slots][cap] */
+    uint32_t* len;        /* device [n_slots] */
+    uint64_t* n_gen;      /* device [n_slots] (may be NULL): output tokens produced so far (Slot::n_gen) */
+    const uint32_t* slot; /* device [n_seq]: slot of each sequence of the call */
+    uint32_t cap;
+} ws_history;
+
+/* Before the verify rows of a cycle are sampled. Per sequence s with control area c (nd = c[WS_CTL_ND] clamped to 0..15):
+ * the drafts c[WS_CTL_DRAFTS .. + nd) go behind the slot's `next`, and for its rows row0[s] + j, j = 0..nd:
+ *   hist_off[row] = slot * cap, hist_len[row] = len + 1 + j   (the text, next, the drafts before position j),
+ *   query[row] = draft j, -1 at j = nd;  step[row] = n_gen + j
+ * which are the ws_batch arrays of the same names. status[s] = WS_ACCEPT_HISTORY_FULL (and hist_len 0) when the slot has
+ * no room for the cycle. */
+typedef struct ws_history_stage_args {
+    ws_history hist;
+    const int32_t* ctl_all;
+    const int32_t* area;  /* device [n_seq] */
+    const uint32_t* row0; /* device [n_seq] */
+    uint32_t n_seq;
+    uint32_t* hist_off;   /* out, device [rows] */
+    uint32_t* hist_len;   /* out, device [rows] */
+    int32_t* query;       /* out, device [rows] (may be NULL) */
+    uint64_t* step;       /* out, device [rows] (may be NULL; needs hist.n_gen) */
+    uint32_t* status;     /* out, device [n_seq] */
+} ws_history_stage_args;
+int ws_history_stage(void* stream, const ws_history_stage_args* a);
+
+/* Draft acceptance on the device for the sampled rules. Stands in for the host loop Acceptor::sample
+ * (src/sampling/acceptor.cpp:63-100), which samples output index n_gen + acc from verify row acc and accepts while the
+ * token equals the draft (rules "sample" and, with ws_batch.race, "specsample"); with `typical` set it first accepts a
+ * draft whose probability under the row's filtered distribution is at least min(eps, delta * exp(-entropy))
+ * (include/whirl/relax_accept.h:94-96) unless keeping it would close a repeated 6-gram of the sequence's text (:72-92,
+ * guard as the engine builds it, src/spec/spec_rules.h:77-83; it needs the device history) - rule "relaxacc_typical".
+ * Each output index draws from its own counter (src/sampling/acceptor.h:10-12), so the caller samples all verify rows of
+ * all sequences in one ws_sample_batch launch - row of position j of a sequence: step = n_gen + j, query = draft j, seed
+ * and filters of the sequence - and this call turns the results into counts, with no host round trip in between. Per
+ * sequence s, control area c = ctl_all + area[s] (layout above): nd = c[WS_CTL_ND] clamped to 0..15, drafts
+ * c[WS_CTL_DRAFTS .. + nd).
+ *   acc = number of leading positions j < nd that were accepted; chosen = token drawn at position acc;
+ *   c[WS_CTL_ROWS + j] = token kept at position j for j <= acc (the words the greedy path fills with row argmaxes,
+ *   src/model/qwen35/forward/mtp_verify.cpp:226); n_accepted[s] = acc; chosen[s]; relaxed[s] += drafts the typical rule kept.
+ *   status[s]: WS_ACCEPT_HOST when a position up to the stop has no usable token (token < 0): the host then runs
+ *   Acceptor::sample for that sequence; WS_ACCEPT_NEAR_TYPICAL when a typical test on an entropy that carries
+ *   WS_FLAG_APPROX_ENTROPY came out within 2 % of its threshold; WS_ACCEPT_HISTORY_FULL (with WS_ACCEPT_HOST) when the
+ *   slot's history has no room for what was accepted.
+ * With a history, next and the accepted drafts are appended to the slot, chosen becomes its next and n_gen advances. */
+enum { WS_ACCEPT_OK = 0, WS_ACCEPT_HOST = 1, WS_ACCEPT_NEAR_TYPICAL = 2, WS_ACCEPT_HISTORY_FULL = 4 };
 typedef struct ws_accept {
     const int32_t* token;  /* device [rows]: ws_batch.token of the launch that sampled the verify rows */
     const uint32_t* flags; /* device [rows]: ws_batch.flags of that launch */
@@ -238,10 +305,46 @@ typedef struct ws_accept {
     uint32_t n_seq;
     int32_t* n_accepted;   /* out, device [n_seq] */
     int32_t* chosen;       /* out, device [n_seq] */
-    uint32_t* status;      /* out, device [n_seq]: WS_ACCEPT_* */
+    uint32_t* status;      /* out, device [n_seq]: WS_ACCEPT_* bits */
+    /* ---- since ABI version 2 (all zero: the plain rule, no history) */
+    int32_t typical;            /* non-zero: rule relaxacc_typical */
+    const double* query_prob;   /* device [rows]: ws_batch.query_prob of the launch (queries = the drafts) */
+    const double* entropy;      /* device [rows]: ws_batch.entropy of the launch */
+    float eps, delta;           /* relax::Params (include/whirl/relax_accept.h:44-51) */
+    uint32_t* relaxed;          /* device [n_seq] (may be NULL), incremented */
+    ws_history hist;            /* tokens NULL: no device history (then no repeat guard either) */
 } ws_accept;
 
 int ws_accept_sampled(void* stream, const ws_accept* a);
+
+/* Acceptor::greedy on the device (src/sampling/acceptor.cpp:30-61). Per sequence: c[WS_CTL_ROWS + j] holds the argmax of
+ * verify row j (argmax_rows_to), the drafts are kept while they equal it; with `relax` a draft that differs is still kept
+ * when it is among the row's relax_k largest logits - fewer than relax_k candidates before it in (logit desc, id asc)
+ * order - with exp(logit - max) >= alpha (include/whirl/relax_accept.h:55-70) and does not close a repeated 6-gram.
+ * The rows' largest logits come from ws_topk_rows(K = k, inv_t = 1) in its [ids | vals | stats] layout
+ * (src/sampling/acceptor.h:42-48): row of position j of sequence s = row0[s] + j. chosen = the argmax at the stop.
+ * relaxed[s] += drafts kept by the relaxed rule, relax_gap[s] += their distance below the row maximum. */
+typedef struct ws_accept_greedy_args {
+    int32_t* ctl_all;
+    const int32_t* area;  /* device [n_seq] */
+    const uint32_t* row0; /* device [n_seq] */
+    uint32_t n_seq;
+    int32_t relax;
+    const int32_t* relax_ids;  /* device [max_rows * k] */
+    const float* relax_vals;   /* device [max_rows * k] */
+    const float* relax_stats;  /* device [max_rows * 2] */
+    uint32_t k;                /* entries per row in the tables */
+    uint32_t relax_k;          /* relax::Params::topk() */
+    float alpha;
+    int32_t* n_accepted;       /* out, device [n_seq] */
+    int32_t* chosen;           /* out, device [n_seq] */
+    uint32_t* status;          /* out, device [n_seq] */
+    uint32_t* relaxed;         /* device [n_seq] (may be NULL), incremented */
+    double* relax_gap;         /* device [n_seq] (may be NULL), added to */
+    ws_history hist;           /* tokens NULL: no device history (then no repeat guard either) */
+} ws_accept_greedy_args;
+
+int ws_accept_greedy(void* stream, const ws_accept_greedy_args* a);
 
 /* Classic speculative sampling (accept u * q < p, else resample from max(p - q, 0)); no counterpart in the
  * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32

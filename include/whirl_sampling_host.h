@@ -44,8 +44,7 @@ int wsh_sample_rows(void* stream, const wsh_rows* a);
 
 /* Acceptor::sample (src/sampling/acceptor.cpp:63-100) for one sequence over device logits: verify rows row0 .. row0 + nd
  * of d_logits, drafts dr[0 .. nd), output index n_gen + accepted. With prefetch != 0 the rows are filtered by one device
- * launch (sampling::DeviceRows::prefetchRows) before the loop, otherwise one launch per visited row. Relaxed acceptance
- * and the repetition guard are off. */
+ * launch (sampling::DeviceRows::prefetchRows) before the loop, otherwise one launch per visited row. */
 typedef struct wsh_accept {
     const float* d_logits; /* device, [rows][vocab] */
     uint32_t rows, vocab;
@@ -60,6 +59,15 @@ typedef struct wsh_accept {
     int32_t prefetch;
     uint32_t acc, chosen;        /* out */
     uint32_t big_used, full_used; /* out: Sampler counters after the loop */
+    /* the "relaxacc_typical" rule (src/sampling/acceptor.cpp:77-90): typ != 0 also accepts a draft with
+     * p(draft) >= min(eps, delta * exp(-entropy)) under the row's filtered distribution, unless keeping it would end the
+     * text (hist, next, drafts so far) in a 6-gram it already holds (include/whirl/relax_accept.h:72-92) */
+    int32_t typ;
+    float eps, delta;
+    const uint32_t* hist; /* host: the sequence's text (may be NULL with n_hist 0: the guard never fires) */
+    uint32_t n_hist;
+    uint32_t next;        /* the token that goes into the model next: it comes before the drafts in the guard's text */
+    uint32_t relaxed;     /* out: drafts the typical rule kept */
 } wsh_accept;
 int wsh_accept_sample(void* stream, wsh_accept* a);
 const char* wsh_last_error(void);

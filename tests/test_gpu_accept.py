@@ -76,7 +76,7 @@ def _device_accept(seqs, spoil=None):
         ctl[s, 48] = q["nd"]
     ctl_d = t(ctl.reshape(-1).copy())
     area = t(np.arange(len(seqs), dtype=np.int32) * 64)
-    n_acc, chosen, status = m.accept_sampled(smp.token, smp.flags, t(row0[:-1].astype(np.int32)), ctl_d, area)
+    n_acc, chosen, status, _ = m.accept_sampled(smp.token, smp.flags, t(row0[:-1].astype(np.int32)), ctl_d, area)
     torch.cuda.synchronize()
     return (n_acc.cpu().numpy(), chosen.cpu().numpy(), status.cpu().numpy(), ctl_d.cpu().numpy().reshape(-1, 64),
             smp.token.cpu().numpy(), smp.flags.cpu().numpy(), row0)

@@ -20,7 +20,8 @@ DTYPE_F32, DTYPE_BF16 = 0, 1
 RNG_SPLITMIX, RNG_PHILOX = 0, 1
 MODE_AUTO, MODE_EXACT, MODE_FUSED = 0, 1, 2
 FLAG_NEAR_TOP_P, FLAG_NEAR_MIN_P, FLAG_NEAR_DRAW = 1, 2, 4
-FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN = 8, 16, 32, 64
+FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN, FLAG_APPROX_ENTROPY = 8, 16, 32, 64, 128
+ACCEPT_OK, ACCEPT_HOST, ACCEPT_NEAR_TYPICAL, ACCEPT_HISTORY_FULL = 0, 1, 2, 4
 FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
 CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
 
@@ -51,7 +52,8 @@ class Batch(C.Structure):
                 ("stats", C.c_void_p), ("margin", C.c_void_p), ("kept_ids", C.c_void_p), ("kept_logits", C.c_void_p),
                 ("kept_cap", C.c_uint32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32),
-                ("race", C.c_void_p)]
+                ("race", C.c_void_p),
+                ("hist_len", C.c_void_p), ("query", C.c_void_p), ("query_prob", C.c_void_p), ("entropy", C.c_void_p)]
 
 
 class SpecVerify(C.Structure):
@@ -69,10 +71,31 @@ class Adjust(C.Structure):
                 ("allow_stride", C.c_uint64), ("out", C.c_void_p), ("out_stride", C.c_uint64)]
 
 
+class History(C.Structure):
+    """ws_history of include/whirl_sampling_abi.h."""
+    _fields_ = [("tokens", C.c_void_p), ("len", C.c_void_p), ("n_gen", C.c_void_p), ("slot", C.c_void_p), ("cap", C.c_uint32)]
+
+
 class Accept(C.Structure):
     """ws_accept of include/whirl_sampling_abi.h."""
     _fields_ = [("token", C.c_void_p), ("flags", C.c_void_p), ("row0", C.c_void_p), ("ctl_all", C.c_void_p), ("area", C.c_void_p),
-                ("n_seq", C.c_uint32), ("n_accepted", C.c_void_p), ("chosen", C.c_void_p), ("status", C.c_void_p)]
+                ("n_seq", C.c_uint32), ("n_accepted", C.c_void_p), ("chosen", C.c_void_p), ("status", C.c_void_p),
+                ("typical", C.c_int32), ("query_prob", C.c_void_p), ("entropy", C.c_void_p), ("eps", C.c_float), ("delta", C.c_float),
+                ("relaxed", C.c_void_p), ("hist", History)]
+
+
+class AcceptGreedy(C.Structure):
+    """ws_accept_greedy_args of include/whirl_sampling_abi.h."""
+    _fields_ = [("ctl_all", C.c_void_p), ("area", C.c_void_p), ("row0", C.c_void_p), ("n_seq", C.c_uint32), ("relax", C.c_int32),
+                ("relax_ids", C.c_void_p), ("relax_vals", C.c_void_p), ("relax_stats", C.c_void_p), ("k", C.c_uint32),
+                ("relax_k", C.c_uint32), ("alpha", C.c_float), ("n_accepted", C.c_void_p), ("chosen", C.c_void_p), ("status", C.c_void_p),
+                ("relaxed", C.c_void_p), ("relax_gap", C.c_void_p), ("hist", History)]
+
+
+class HistoryStage(C.Structure):
+    """ws_history_stage_args of include/whirl_sampling_abi.h."""
+    _fields_ = [("hist", History), ("ctl_all", C.c_void_p), ("area", C.c_void_p), ("row0", C.c_void_p), ("n_seq", C.c_uint32),
+                ("hist_off", C.c_void_p), ("hist_len", C.c_void_p), ("query", C.c_void_p), ("step", C.c_void_p), ("status", C.c_void_p)]
 
 
 # every symbol include/whirl_sampling_abi.h declares: (result type, argument types)
@@ -97,6 +120,8 @@ ABI = {
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
     "ws_accept_sampled": (C.c_int, [C.c_void_p, C.POINTER(Accept)]),
+    "ws_accept_greedy": (C.c_int, [C.c_void_p, C.POINTER(AcceptGreedy)]),
+    "ws_history_stage": (C.c_int, [C.c_void_p, C.POINTER(HistoryStage)]),
     "ws_spec_verify_workspace": (C.c_uint64, [C.POINTER(SpecVerify)]),
     "ws_spec_verify_classic": (C.c_int, [C.c_void_p, C.POINTER(SpecVerify)]),
 }
@@ -237,10 +262,38 @@ def adjust_rows(logits, hist=None, hist_off=None, rep=None, pres=None, freq=None
     return out
 
 
-def accept_sampled(token, flags, row0, ctl_all, area):
+class DeviceHistory:
+    """The sequences' token histories on the device (ws_history): tokens int32 [n_slots, cap], len int32 [n_slots], n_gen
+    int64 [n_slots]. Slot i's text is tokens[i, :len[i]], tokens[i, len[i]] is the token that goes in next."""
+
+    def __init__(self, n_slots, cap, device="cuda:0"):
+        self.tokens = torch.zeros((n_slots, cap), dtype=torch.int32, device=device)
+        self.len = torch.zeros(n_slots, dtype=torch.int32, device=device)
+        self.n_gen = torch.zeros(n_slots, dtype=torch.int64, device=device)
+        self.cap = cap
+
+    def ref(self, slot):
+        """ws_history for the sequences whose slots are `slot` (int32 device tensor)."""
+        return History(tokens=_p(self.tokens), len=_p(self.len), n_gen=_p(self.n_gen), slot=_p(slot), cap=self.cap)
+
+
+def history_stage(hist, slot, ctl_all, area, row0, hist_off, hist_len, query=None, step=None):
+    """Drafts of the cycle behind every sequence's text, and the rows' history windows / queries / output indices for the
+    batched sampler (ws_history_stage). Returns status int32 [n_seq]."""
+    n_seq = row0.numel()
+    status = torch.empty(n_seq, dtype=torch.int32, device=row0.device)
+    a = HistoryStage(hist=hist.ref(slot), ctl_all=_p(ctl_all), area=_p(area), row0=_p(row0), n_seq=n_seq, hist_off=_p(hist_off),
+                     hist_len=_p(hist_len), query=_p(query), step=_p(step), status=_p(status))
+    check(lib().ws_history_stage(_stream(), C.byref(a)), "ws_history_stage")
+    return status
+
+
+def accept_sampled(token, flags, row0, ctl_all, area, typical=None, hist=None, slot=None):
     """Accepted draft count and chosen token per sequence from the sampled tokens of its verify rows (ws_accept_sampled).
     token int32 [rows], flags uint32-as-int32 [rows], row0 int32 [n_seq], ctl_all int32 control areas, area int32 [n_seq]
-    word offsets; all device tensors. Returns (n_accepted, chosen, status) int32 device tensors; ctl_all is updated."""
+    word offsets; all device tensors. typical: dict(query_prob, entropy, eps, delta) for the relaxacc_typical rule.
+    hist / slot: a DeviceHistory and the sequences' slots. Returns (n_accepted, chosen, status, relaxed) int32 device
+    tensors; ctl_all (and the history) is updated."""
     for name, v in (("token", token), ("flags", flags), ("row0", row0), ("ctl_all", ctl_all), ("area", area)):
         if not v.is_cuda or v.dtype != torch.int32 or not v.is_contiguous():
             raise WsError(f"{name}: contiguous int32 device tensor")
@@ -248,10 +301,39 @@ def accept_sampled(token, flags, row0, ctl_all, area):
     n_acc = torch.empty(n_seq, dtype=torch.int32, device=token.device)
     chosen = torch.empty(n_seq, dtype=torch.int32, device=token.device)
     status = torch.empty(n_seq, dtype=torch.int32, device=token.device)
+    relaxed = torch.zeros(n_seq, dtype=torch.int32, device=token.device)
     a = Accept(token=_p(token), flags=_p(flags), row0=_p(row0), ctl_all=_p(ctl_all), area=_p(area), n_seq=n_seq,
-               n_accepted=_p(n_acc), chosen=_p(chosen), status=_p(status))
+               n_accepted=_p(n_acc), chosen=_p(chosen), status=_p(status), relaxed=_p(relaxed))
+    if typical is not None:
+        a.typical = 1
+        a.query_prob, a.entropy = _p(typical["query_prob"]), _p(typical["entropy"])
+        a.eps, a.delta = typical["eps"], typical["delta"]
+    if hist is not None:
+        a.hist = hist.ref(slot)
     check(lib().ws_accept_sampled(_stream(), C.byref(a)), "ws_accept_sampled")
-    return n_acc, chosen, status
+    return n_acc, chosen, status, relaxed
+
+
+def accept_greedy(ctl_all, area, row0, relax=None, hist=None, slot=None):
+    """Acceptor::greedy on the device (ws_accept_greedy). relax: dict(ids, vals, stats, k, relax_k, alpha) with the rows'
+    largest logits as ws_topk_rows wrote them. Returns (n_accepted, chosen, status, relaxed, relax_gap)."""
+    n_seq = row0.numel()
+    dev = row0.device
+    n_acc = torch.empty(n_seq, dtype=torch.int32, device=dev)
+    chosen = torch.empty(n_seq, dtype=torch.int32, device=dev)
+    status = torch.empty(n_seq, dtype=torch.int32, device=dev)
+    relaxed = torch.zeros(n_seq, dtype=torch.int32, device=dev)
+    gap = torch.zeros(n_seq, dtype=torch.float64, device=dev)
+    a = AcceptGreedy(ctl_all=_p(ctl_all), area=_p(area), row0=_p(row0), n_seq=n_seq, n_accepted=_p(n_acc), chosen=_p(chosen),
+                     status=_p(status), relaxed=_p(relaxed), relax_gap=_p(gap))
+    if relax is not None:
+        a.relax = 1
+        a.relax_ids, a.relax_vals, a.relax_stats = _p(relax["ids"]), _p(relax["vals"]), _p(relax["stats"])
+        a.k, a.relax_k, a.alpha = relax["k"], relax["relax_k"], relax["alpha"]
+    if hist is not None:
+        a.hist = hist.ref(slot)
+    check(lib().ws_accept_greedy(_stream(), C.byref(a)), "ws_accept_greedy")
+    return n_acc, chosen, status, relaxed, gap
 
 
 class BatchSampler:
@@ -260,7 +342,8 @@ class BatchSampler:
 
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
-                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None):
+                 max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None,
+                 hist_len=None, query=None, want_entropy=False):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -269,7 +352,7 @@ class BatchSampler:
         rows, V = logits.shape
         self.keep = dict(logits=logits, inv_t=inv_t, seed=seed, step=step, top_k=top_k, top_p=top_p, min_p=min_p,
                          hist=hist, hist_off=hist_off, rep=rep, pres=pres, freq=freq, bias_ids=bias_ids,
-                         bias_vals=bias_vals, bias_off=bias_off, allow=allow, race=race)
+                         bias_vals=bias_vals, bias_off=bias_off, allow=allow, race=race, hist_len=hist_len, query=query)
         self.token = torch.empty(rows, dtype=torch.int32, device=dev)
         self.prob = torch.empty(rows, dtype=torch.float32, device=dev)
         self.n_kept = torch.empty(rows, dtype=torch.int32, device=dev)
@@ -293,6 +376,10 @@ class BatchSampler:
         b.tol = tol
         b.mode = mode
         b.race = _p(race)
+        b.hist_len, b.query = _p(hist_len), _p(query)
+        self.query_prob = torch.zeros(rows, dtype=torch.float64, device=dev) if query is not None else None
+        self.entropy = torch.zeros(rows, dtype=torch.float64, device=dev) if want_entropy else None
+        b.query_prob, b.entropy = _p(self.query_prob), _p(self.entropy)
         need = lib().ws_sample_batch_workspace(C.byref(b))
         self.workspace = torch.empty(max(int(need), 16), dtype=torch.uint8, device=dev)
         b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()
@@ -336,7 +423,8 @@ class HostAccept(C.Structure):
     _fields_ = [("d_logits", C.c_void_p), ("rows", C.c_uint32), ("vocab", C.c_uint32), ("inv_t", C.c_float), ("top_k", C.c_uint32),
                 ("top_p", C.c_double), ("min_p", C.c_double), ("seed", C.c_uint64), ("race", C.c_int32), ("dr", C.c_void_p),
                 ("nd", C.c_uint32), ("row0", C.c_uint32), ("n_gen", C.c_uint64), ("prefetch", C.c_int32), ("acc", C.c_uint32),
-                ("chosen", C.c_uint32), ("big_used", C.c_uint32), ("full_used", C.c_uint32)]
+                ("chosen", C.c_uint32), ("big_used", C.c_uint32), ("full_used", C.c_uint32), ("typ", C.c_int32), ("eps", C.c_float),
+                ("delta", C.c_float), ("hist", C.c_void_p), ("n_hist", C.c_uint32), ("next", C.c_uint32), ("relaxed", C.c_uint32)]
 
 
 HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]),
@@ -392,16 +480,23 @@ def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p
     return out
 
 
-def host_accept_sample(logits, dr, nd, row0, n_gen, temp, top_k, top_p, min_p, seed, race=False, prefetch=True):
-    """Acceptor::sample of the C++ host API for one sequence over device logits (wsh_accept_sample). Returns
-    (accepted, chosen, big_used, full_used)."""
+def host_accept_sample(logits, dr, nd, row0, n_gen, temp, top_k, top_p, min_p, seed, race=False, prefetch=True, typical=None):
+    """Acceptor::sample of the C++ host API for one sequence over device logits (wsh_accept_sample). typical:
+    dict(eps, delta, hist, next) for the relaxacc_typical rule. Returns (accepted, chosen, big_used, full_used), with
+    `typical` also the number of drafts that rule kept."""
     import numpy as np
     _dev_f32(logits)
     dr = np.ascontiguousarray(dr, dtype=np.uint32)
     a = HostAccept(d_logits=_p(logits), rows=logits.shape[0], vocab=logits.shape[1], inv_t=float(np.float32(1.0 / temp)), top_k=top_k,
                    top_p=top_p, min_p=min_p, seed=seed, race=int(race), dr=dr.ctypes.data_as(C.c_void_p), nd=nd, row0=row0,
                    n_gen=n_gen, prefetch=int(prefetch))
+    if typical is not None:
+        hist = np.ascontiguousarray(typical.get("hist", np.zeros(0, np.uint32)), dtype=np.uint32)
+        a.typ, a.eps, a.delta, a.next = 1, typical["eps"], typical["delta"], typical.get("next", 0)
+        a.hist, a.n_hist = hist.ctypes.data_as(C.c_void_p), hist.size
     rc = host_lib().wsh_accept_sample(_stream(), C.byref(a))
     if rc != 0:
         raise WsError(f"wsh_accept_sample: {host_lib().wsh_last_error().decode()} ({rc})")
+    if typical is not None:
+        return a.acc, a.chosen, a.big_used, a.full_used, a.relaxed
     return a.acc, a.chosen, a.big_used, a.full_used

@@ -238,6 +238,10 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.lds_tie = p.lds_tie;
     a.two_sweep = b->mode == WS_MODE_AUTO ? 1 : 0;
     a.race = b->race;
+    a.hist_len = b->hist ? b->hist_len : nullptr;
+    a.query = b->query;
+    a.query_prob = b->query_prob;
+    a.entropy = b->entropy;
     if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);
     static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
     if (!attr_set) {
@@ -284,10 +288,16 @@ int ws_adjust_rows(void* stream, const ws_adjust* b) {
     return done();
 }
 
+namespace {
+ws::HistoryRef history_ref(const ws_history& h) { return ws::HistoryRef{h.tokens, h.len, h.n_gen, h.slot, h.cap}; }
+bool history_ok(const ws_history& h) { return !h.tokens || (h.len && h.slot && h.cap >= 2u); }
+}  // namespace
+
 int ws_accept_sampled(void* stream, const ws_accept* b) {
     if (!b || !b->token || !b->flags || !b->row0 || !b->ctl_all || !b->area || !b->n_accepted || !b->chosen || !b->status)
         return WS_E_INVALID;
-    if (b->n_seq == 0) return WS_E_INVALID;
+    if (b->n_seq == 0 || !history_ok(b->hist)) return WS_E_INVALID;
+    if (b->typical && (!b->query_prob || !b->entropy)) return WS_E_INVALID;
     ws::AcceptArgs a{};
     a.token = b->token;
     a.flags = b->flags;
@@ -299,7 +309,61 @@ int ws_accept_sampled(void* stream, const ws_accept* b) {
     a.n_accepted = b->n_accepted;
     a.chosen = b->chosen;
     a.status = b->status;
-    hipLaunchKernelGGL(ws::accept_sampled_kernel, dim3((b->n_seq + 63u) / 64u), dim3(64), 0, S(stream), a);
+    a.query_prob = b->query_prob;
+    a.entropy = b->entropy;
+    a.typical = b->typical;
+    a.eps = b->eps;
+    a.delta = b->delta;
+    a.approx_mask = WS_FLAG_APPROX_ENTROPY;
+    a.relaxed = b->relaxed;
+    a.hist = history_ref(b->hist);
+    hipLaunchKernelGGL(ws::accept_sampled_kernel, dim3(b->n_seq), dim3(64), 0, S(stream), a);
+    return done();
+}
+
+int ws_accept_greedy(void* stream, const ws_accept_greedy_args* b) {
+    if (!b || !b->ctl_all || !b->area || !b->row0 || !b->n_accepted || !b->chosen || !b->status || b->n_seq == 0) return WS_E_INVALID;
+    if (!history_ok(b->hist)) return WS_E_INVALID;
+    if (b->relax && (!b->relax_ids || !b->relax_vals || !b->relax_stats || b->k == 0 || b->relax_k == 0)) return WS_E_INVALID;
+    ws::AcceptGreedyArgs a{};
+    a.ctl_all = b->ctl_all;
+    a.area = b->area;
+    a.row0 = b->row0;
+    a.n_seq = b->n_seq;
+    a.relax = b->relax;
+    a.relax_ids = b->relax_ids;
+    a.relax_vals = b->relax_vals;
+    a.relax_stats = b->relax_stats;
+    a.k = b->k;
+    a.relax_k = b->relax_k;
+    a.alpha = b->alpha;
+    a.n_accepted = b->n_accepted;
+    a.chosen = b->chosen;
+    a.status = b->status;
+    a.relaxed = b->relaxed;
+    a.relax_gap = b->relax_gap;
+    a.hist = history_ref(b->hist);
+    hipLaunchKernelGGL(ws::accept_greedy_kernel, dim3(b->n_seq), dim3(64), 0, S(stream), a);
+    return done();
+}
+
+int ws_history_stage(void* stream, const ws_history_stage_args* b) {
+    if (!b || !b->hist.tokens || !history_ok(b->hist) || !b->ctl_all || !b->area || !b->row0 || !b->hist_off || !b->hist_len || !b->status ||
+        b->n_seq == 0)
+        return WS_E_INVALID;
+    if (b->step && !b->hist.n_gen) return WS_E_INVALID;
+    ws::StageArgs a{};
+    a.hist = history_ref(b->hist);
+    a.ctl_all = b->ctl_all;
+    a.area = b->area;
+    a.row0 = b->row0;
+    a.n_seq = b->n_seq;
+    a.hist_off = b->hist_off;
+    a.hist_len = b->hist_len;
+    a.query = b->query;
+    a.step = b->step;
+    a.status = b->status;
+    hipLaunchKernelGGL(ws::history_stage_kernel, dim3((b->n_seq + 63u) / 64u), dim3(64), 0, S(stream), a);
     return done();
 }
 

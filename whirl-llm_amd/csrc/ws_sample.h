@@ -43,7 +43,7 @@ constexpr float kG0 = 16776924.0f, kG1 = -130126.3125f;
 
 // flag bits (WS_FLAG_* of the C ABI)
 constexpr uint32_t kOpenList = 256u;  // candidates of the engine's short list (k_small, src/server/engine_sampling.h:20)
-constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u;
+constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u, kApproxEntropy = 128u;
 
 struct BatchArgs {
     const void* logits;
@@ -85,6 +85,10 @@ struct BatchArgs {
     int two_sweep;     // rows the single sweep cannot take: histogram against a provisional bound in the first sweep (else: exact mode)
     const int32_t* race;  // per row, non-zero: exponential-race draw
     uint32_t lds_cnt;  // byte offset of the per-rank tables {history count | bias entries, index of the first bias entry}: 8 * patch_cap bytes
+    const uint32_t* hist_len;  // per row or nullptr: ids of the row's history (else hist_off[row + 1] - hist_off[row])
+    const int32_t* query;      // per row or nullptr: a token whose probability is asked for (< 0: none)
+    double* query_prob;        // out per row or nullptr
+    double* entropy;           // out per row or nullptr: entropy of the kept set
 };
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
@@ -605,7 +609,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     rv.pv = pv;
 
     // ------------------------------------------------------------------ phase 0: penalties and bias
-    const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? A.hist_off[row + 1] - h0 : 0u;
+    const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? (A.hist_len ? A.hist_len[row] : A.hist_off[row + 1] - h0) : 0u;
     const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
     uint32_t n_touched = 0;  // distinct tokens the history and the bias list touch
     float m_adj = -INFINITY;  // largest adjusted logit among them
@@ -1055,6 +1059,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 A.stats[2 * row + 1] = 0.f;
             }
             if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
+            if (A.query_prob) A.query_prob[row] = 0.0;
+            if (A.entropy) A.entropy[row] = 0.0;
         }
         return;
     }
@@ -1298,6 +1304,22 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double m1base = has_r1 ? pm[r1lo] : 0.0;
     const uint32_t n_list = n_r0 + n_r1;
     if (n_list > kCap || n_list == 0) flags |= kOverflow;
+    // Entropy of the kept set (asked for by the typical acceptance rule): -sum p ln p = ln Zk + sum e a / Zk with
+    // e = exp(-a), a = (max - x) * inv_t. The gathered candidates give their terms exactly further down; the bins that
+    // are kept whole - before range 0, and between the ranges - give theirs here from the scanned masses, every token
+    // of a bin counted at the middle of the bin (a to +-1/128): h_before / h_between.
+    double h_before = 0.0, h_between = 0.0;
+    if (A.entropy && !(flags & kOverflow)) {  // uniform
+        double s0 = 0.0, s1 = 0.0;
+        for (int b = static_cast<int>(t); b < kTail; b += WS_BLOCK) {
+            const double dm = pm[b + 1] - pm[b];
+            const double a_mid = (static_cast<double>(b) + 0.5) * (1.0 / 64.0) - lift;
+            if (b < r0lo) s0 += dm * a_mid;
+            else if (has_r1 && b > r0hi && b < r1lo) s1 += dm * a_mid;
+        }
+        h_before = block_sum(s0, red_d);
+        h_between = block_sum(s1, red_d);
+    }
     if (t == 0) s_cnt = s_u[4] = s_u[5] = 0;
     __syncthreads();  // the last reads of pm / pc are done: their LDS is the key buffer and the candidate list from here
 
@@ -1312,6 +1334,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 A.stats[2 * row + 1] = static_cast<float>(Z);
             }
             if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
+            if (A.query_prob) A.query_prob[row] = 0.0;
+            if (A.entropy) A.entropy[row] = 0.0;
         }
         return;
     }
@@ -1323,7 +1347,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     int32_t token = -1;
     double ptok = 0;
     uint64_t kept_key = 0ull;
+    double Zk_out = 0.0;  // mass of the kept set (the row's float normaliser on an open row)
     bool finished = false;
+    bool finished_lean = false;
     // ------------------------------------------------------------------ pass 3: gather, sort, exact masses
     {
         const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = static_cast<uint32_t>(r0hi - r0lo);
@@ -1467,7 +1493,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     struct LeanResult {
                         int32_t token;
                         uint32_t n3, overflow, ok;
-                        double ptok, mg_top_p, mg_min_p, mg_draw;
+                        double ptok, mg_top_p, mg_min_p, mg_draw, Zk;
                         unsigned long long kept_key;
                     };
                     __shared__ LeanResult s_res;
@@ -1624,6 +1650,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                             kept_key = 0ull;
                         }
                     }
+                    Zk_out = Zk;
                     // ---- the draw (src/sampling/sampler.cpp:118-131)
                     if (!lean_failed) {
                         const double target = batch_uniform(A.rng, seed, row, step, 0) * Zk;
@@ -1642,7 +1669,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                             }
                         }
                     }
-                    if (lane == 0u) s_res = LeanResult{token, n3, flags & kOverflow, lean_failed ? 0u : 1u, ptok, mg_top_p, mg_min_p, mg_draw, kept_key};
+                    if (lane == 0u) s_res = LeanResult{token, n3, flags & kOverflow, lean_failed ? 0u : 1u, ptok, mg_top_p, mg_min_p, mg_draw, Zk_out, kept_key};
                     }  // wave 0
                     __syncthreads();  // the answers are in place, and the bucket tables are done with
                     if (s_res.ok) {
@@ -1654,7 +1681,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         mg_min_p = s_res.mg_min_p;
                         mg_draw = s_res.mg_draw;
                         kept_key = s_res.kept_key;
-                        finished = true;
+                        Zk_out = s_res.Zk;
+                        finished = finished_lean = true;
                     } else {
                         mg_top_p = mg_min_p = mg_draw = 1.0;
                         n3 = n1;
@@ -1727,6 +1755,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 A.stats[2 * row + 1] = static_cast<float>(Z);
             }
             if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
+            if (A.query_prob) A.query_prob[row] = 0.0;
+            if (A.entropy) A.entropy[row] = 0.0;
         }
         return;
     }
@@ -2493,12 +2523,63 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     }
     if (race && open_row) mg_draw = fmin(mg_draw, fabs(target - inc_of(i_last)) / Zk);  // the list-or-rest decision
+    Zk_out = Zk;
     }  // the sort-based finish
     // zero-mass tail candidates a top-k kept (no top-p / min-p cut them away again)
     const uint32_t tail_extra = (!use_top_p && !use_min_p && n3 == n1) ? n1_asked - n1 : 0u;
     if (mg_top_p < tol) flags |= kNearTopP;
     if (mg_min_p < tol) flags |= kNearMinP;
     if (mg_draw < tol) flags |= kNearDraw;
+
+    // ------------------------------------------------------------------ optional: the kept set's entropy
+    if (A.entropy) {  // uniform
+        // terms of the gathered candidates that are kept: exact
+        double se = 0.0, sm = 0.0;
+        auto term = [&](uint64_t key) {
+            if (key < kept_key || (key >> 32) == 0ull) return;
+            const float x = unkey32(static_cast<uint32_t>(key >> 32));
+            const double a = static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t);
+            const double e = exp(-a);
+            if (e > 0.0) {
+                se += e * a;
+                sm += e;
+            }
+        };
+        __syncthreads();
+        if (finished_lean) {  // the keys lie in the buckets' places
+            const uint32_t* cnt_of = reinterpret_cast<const uint32_t*>(s_pool + 128);
+            const uint32_t shift = A.lds_tie ? 5u : 4u;
+            for (uint32_t slot = t; slot < (128u << shift); slot += WS_BLOCK)
+                if ((slot & ((1u << shift) - 1u)) < cnt_of[slot >> shift]) term(reinterpret_cast<const uint64_t*>(lds)[slot]);
+        } else {
+            const uint32_t n_sorted = open_row ? min(n3, n_list) : n_list;
+            for (uint32_t i = t; i < n_sorted; i += WS_BLOCK) term(keys[i]);
+        }
+        const double s_list = block_sum(se, red_d), m_list = block_sum(sm, red_d);
+        double h = 0.0;
+        if (token >= 0 && Zk_out > 0.0) {
+            if (open_row) {  // the listed candidates, each with its share of the whole row (not renormalised)
+                h = (s_list + log(Zk_out) * m_list) / Zk_out;
+            } else {
+                const bool past_r0 = has_r1 && n3 >= c1base;  // the cut lies in range 1 or at its edge: the bins between are kept too
+                const double s_bins = h_before + (past_r0 ? h_between : 0.0);
+                if (s_bins != 0.0) flags |= kApproxEntropy;
+                h = log(Zk_out) + (s_bins + s_list) / Zk_out;
+            }
+        }
+        if (t == 0) A.entropy[row] = h;
+    }
+    if (A.query_prob && t == 0) {
+        // probability of one named token under the filtered distribution (probOf, src/sampling/sampler.cpp:108-116)
+        const int32_t q = A.query ? A.query[row] : -1;
+        double pq = 0.0;
+        if (q >= 0 && static_cast<uint32_t>(q) < V && token >= 0 && Zk_out > 0.0) {
+            const float xq = adjusted_logit(rv, static_cast<uint32_t>(q));
+            const bool kept = open_row || key64(xq, static_cast<uint32_t>(q)) >= kept_key;
+            if (kept && xq > -INFINITY) pq = exp(-(static_cast<double>(__fsub_rn(m, xq)) * static_cast<double>(inv_t))) / Zk_out;
+        }
+        A.query_prob[row] = pq;
+    }
 
     WS_MARK(7);
 #ifdef WS_PHASE_TIMERS

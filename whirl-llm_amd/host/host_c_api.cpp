@@ -87,15 +87,27 @@ int wsh_accept_sample(void* stream, wsh_accept* a) {
         s.race = a->race != 0;
         s.row_base = a->row0;
         if (a->prefetch) src.prefetchRows(s, 0, a->nd + 1);
-        const whirl::relax::Params no_relax{};
-        const ws::Acceptor acceptor(no_relax);
+        whirl::relax::Params relax{};
+        if (a->typ) {
+            relax.on = true;
+            relax.eps = a->eps;
+            relax.delta = a->delta;
+        }
+        const ws::Acceptor acceptor(relax);
         std::uint32_t relaxed = 0;
         ws::Drafts drafts;
         drafts.dr = std::span<const std::uint32_t>(a->dr, a->nd);
         drafts.nd = a->nd;
         drafts.row0 = a->row0;
-        const ws::Accepted r = acceptor.sample(src, s, drafts, false, static_cast<std::uint32_t>(a->n_gen),
-                                               [](std::uint32_t) { return false; }, relaxed);
+        // the engine's guard (tests/sampling/sampling_unit.inc:103-108): the text, then next, then the drafts up to and with position r
+        const std::span<const std::uint32_t> text(a->hist, a->hist ? a->n_hist : 0u);
+        auto repeats = [&](std::uint32_t upto) {
+            std::vector<std::uint32_t> tail{a->next};
+            for (std::uint32_t j = 0; j <= upto && j < a->nd; ++j) tail.push_back(a->dr[j]);
+            return whirl::relax::extendsRepeat(text, tail);
+        };
+        const ws::Accepted r = acceptor.sample(src, s, drafts, a->typ != 0, static_cast<std::uint32_t>(a->n_gen), repeats, relaxed);
+        a->relaxed = relaxed;
         a->acc = r.acc;
         a->chosen = r.chosen;
         a->big_used = s.big_used;
