@@ -124,7 +124,10 @@ enum {
     WS_FLAG_NEAR_DRAW = 1u << 2,   /* the uniform was within `tol` (probability units) of a CDF step; race draw: the two smallest
                                       keys are within `tol` (relative) of each other */
     WS_FLAG_ALL_MASKED = 1u << 3,  /* every logit of the row is -inf / NaN: token = -1 */
-    WS_FLAG_OVERFLOW = 1u << 4,    /* more tied / clustered candidates at a cut than the kernel resolves: token = -1 */
+    WS_FLAG_OVERFLOW = 1u << 4,    /* kept for callers of ABI 1, no longer set: a row whose cuts or draw fall among more
+                                      candidates than the kernel's list of 4096 holds (a top-k above 4096, thousands of
+                                      equal logits, a very flat row) is answered by an exact path inside the same launch -
+                                      same results, some hundreds of microseconds for such a row */
     WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
     WS_FLAG_OPEN = 1u << 6,        /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order

@@ -117,6 +117,7 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) { return ~wave_min_
 __device__ __forceinline__ float wave_sum(float v) { return last_lane(wave_incl_scan(v)); }
 __device__ __forceinline__ double wave_sum(double v) { return last_lane(wave_incl_scan(v)); }
 __device__ __forceinline__ uint32_t wave_sum(uint32_t v) { return last_lane(wave_incl_scan(v)); }
+__device__ __forceinline__ uint64_t wave_sum(uint64_t v) { return last_lane(wave_incl_scan(v)); }
 
 // greedy pick: the larger value, on equal values the lower index (kernels/shared/block_argmax.h:16)
 struct Best {

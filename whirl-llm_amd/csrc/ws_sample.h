@@ -536,6 +536,359 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
     }
 }
 
+// ---- the exact path. Rows whose candidate ranges hold more than the list - a top-k beyond its capacity, thousands of
+// candidates with one logit, a flat row whose draw bins alone overflow it - are answered here without any list. Every
+// token's mass is taken in fixed point (units of 2^-44 of the largest), so sums are integers and the same whatever the
+// order; candidates are ordered by their 64-bit key (logit, then id), and each question - the key at a rank, the first
+// key at which the running mass reaches a value - is a radix walk over that key, twelve bits a level, one pass over the
+// row per level with a 4096-entry histogram of counts and masses in LDS. A few dozen passes over a row that sits in L2:
+// hundreds of microseconds, for rows that otherwise had no answer. The decisions are the rules of the main path (the
+// cuts of src/sampling/sampler.cpp:15-78, the walk of :118-146, the race of :80-106). A function of its own, not
+// inlined, so that its registers and code do not weigh on the kernel's sweep.
+struct ExactIn {
+    const void* base;
+    const uint32_t* allow;
+    uint32_t V;
+    int dtype;
+    uint32_t touched_at;  // LDS offset of the touched bitmap, prefix and values; ~0 when no token is touched
+    float m, inv_t;
+    uint32_t top_k, n1_asked;
+    double top_p, min_p, u;
+    uint64_t rbase;       // race hash base of the row
+    uint32_t mode;        // 1 prefix (top-k below the vocabulary), 2 open row, 4 top-p, 8 min-p, 16 race
+};
+struct ExactOut {
+    int32_t token;
+    uint32_t n3, rest;    // rest: an open row's walk left the listed candidates (list_mass, target say where)
+    uint64_t kept_key;
+    double Zk, ptok, mg_top_p, mg_min_p, mg_draw, list_mass, target;
+};
+
+__device__ __noinline__ ExactOut exact_row(const ExactIn in) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ unsigned long long x_w[6];
+    __shared__ unsigned long long x_red_q[WS_WAVES];
+    __shared__ double x_red_d[WS_WAVES];
+    __shared__ uint32_t x_red_u[WS_WAVES];
+    __shared__ uint32_t x_first;
+    const uint32_t t = threadIdx.x, V = in.V;
+    const float m = in.m, inv_t = in.inv_t;
+    const bool prefix_mode = in.mode & 1u, open_row = in.mode & 2u, use_top_p = in.mode & 4u, use_min_p = in.mode & 8u, race = in.mode & 16u;
+    RowView rv;
+    rv.base = in.base;
+    rv.V = V;
+    rv.dtype = in.dtype;
+    rv.vec = false;
+    rv.allow = in.allow;
+    const uint32_t nW = (V + 31u) >> 5;
+    rv.touched = in.touched_at != 0xffffffffu ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) : nullptr;
+    rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u);
+    rv.pv = reinterpret_cast<const float*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    constexpr double kFx = 17592186044416.0;  // 2^44
+    uint64_t* hm = reinterpret_cast<uint64_t*>(lds);          // masses per digit
+    uint32_t* hc = reinterpret_cast<uint32_t*>(lds + 32768);  // counts per digit
+    uint64_t* red_w = reinterpret_cast<uint64_t*>(x_red_q);
+    ExactOut out{};
+    out.mg_top_p = out.mg_min_p = out.mg_draw = 1.0;
+
+    auto each_token = [&](auto&& f) {  // every token with its adjusted logit, four loads in flight per thread
+        for (uint32_t i0 = 0; i0 < V; i0 += 4u * WS_BLOCK) {
+            float xr[4];
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) xr[q] = raw_logit(rv, min(i0 + q * WS_BLOCK + t, V - 1u));
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) {
+                const uint32_t i = i0 + q * WS_BLOCK + t;
+                if (i < V) f(i, is_touched(rv, i) ? rv.pv[rank_of(rv, i)] : (is_allowed(rv, i) ? xr[q] : -INFINITY));
+            }
+        }
+    };
+    auto e_of = [&](float x) { return exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t))); };
+    auto fx_of = [&](float x) -> uint64_t {
+        const double e = e_of(x);
+        return e > 0.0 ? static_cast<uint64_t>(__double2ll_rn(e * kFx)) : 0ull;
+    };
+    auto id_of = [](uint64_t key) { return static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(key)); };
+    auto x_of = [](uint64_t key) { return unkey32(static_cast<uint32_t>(key >> 32)); };
+    // The first key, in descending order, at which the running total - counts (by_mass false) or masses - reaches
+    // `want`; before_c / before_m: what ranks before it. found false: the whole row stays below `want`.
+    struct Walk {
+        bool found;
+        uint64_t key, before_m;
+        uint32_t before_c;
+        uint64_t own_m;
+    };
+    auto walk = [&](bool by_mass, uint64_t want) -> Walk {
+        uint64_t prefix = 0, base_m = 0;
+        uint32_t base_c = 0;
+        int hi = 64;  // bits [hi, 64) of the key are fixed to `prefix`
+        for (;;) {
+            const int width = hi >= 12 ? 12 : hi, lo = hi - width;
+            const uint32_t nd = 1u << width;
+            for (uint32_t d = t; d < nd; d += WS_BLOCK) {
+                hm[d] = 0ull;
+                hc[d] = 0u;
+            }
+            if (t == 0) x_first = 0xffffffffu;
+            __syncthreads();
+            each_token([&](uint32_t i, float x) {
+                const uint64_t k = key64(x, i);
+                if (hi == 64 || (k >> (hi & 63)) == prefix) {
+                    const uint32_t d = static_cast<uint32_t>(k >> lo) & (nd - 1u);
+                    atomicAdd(&hc[d], 1u);
+                    const uint64_t fx = fx_of(x);
+                    if (fx) atomicAdd(reinterpret_cast<unsigned long long*>(&hm[d]), static_cast<unsigned long long>(fx));
+                }
+            });
+            __syncthreads();
+            // digits from the largest down: thread t holds places 8 t .. 8 t + 7 of that order
+            uint64_t lm[8], sm = 0;
+            uint32_t lc[8], sc = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; ++q) {
+                const uint32_t j = 8u * t + q;
+                const bool valid = j < nd;
+                const uint32_t d = valid ? nd - 1u - j : 0u;
+                lm[q] = valid ? hm[d] : 0ull;
+                lc[q] = valid ? hc[d] : 0u;
+                sm += lm[q];
+                sc += lc[q];
+            }
+            uint64_t tot_m;
+            uint32_t tot_c;
+            uint64_t rm = base_m + block_excl_scan(sm, red_w, &tot_m);
+            uint32_t rc = base_c + block_excl_scan(sc, x_red_u, &tot_c);
+            uint32_t at = 0xffffffffu, bc = 0, oc = 0;
+            uint64_t bm = 0, om = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; ++q) {
+                const bool reached = by_mass ? rm + lm[q] >= want : static_cast<uint64_t>(rc + lc[q]) >= want;
+                if (at == 0xffffffffu && lc[q] != 0u && reached) {
+                    at = 8u * t + q;
+                    bm = rm;
+                    bc = rc;
+                    om = lm[q];
+                    oc = lc[q];
+                }
+                rm += lm[q];
+                rc += lc[q];
+            }
+            if (at != 0xffffffffu) atomicMin(&x_first, at);
+            __syncthreads();
+            const uint32_t first = x_first;
+            if (first == 0xffffffffu) return Walk{false, 0ull, base_m + tot_m, base_c + tot_c, 0ull};  // at the first level only
+            if (at == first) {
+                x_w[0] = bm;
+                x_w[1] = bc;
+                x_w[2] = om;
+                x_w[3] = oc;
+            }
+            __syncthreads();
+            base_m = x_w[0];
+            base_c = static_cast<uint32_t>(x_w[1]);
+            const uint64_t own_m = x_w[2];
+            const uint32_t own_c = static_cast<uint32_t>(x_w[3]);
+            const uint64_t d = nd - 1u - first;
+            prefix = hi == 64 ? d : ((prefix << width) | d);
+            hi = lo;
+            if (hi == 0) return Walk{true, prefix, base_m, base_c, own_m};
+            if (own_c == 1u) {  // one key is left under the prefix: one pass finds it
+                each_token([&](uint32_t i, float x) {
+                    const uint64_t k = key64(x, i);
+                    if ((k >> hi) == prefix) x_w[4] = k;
+                });
+                __syncthreads();
+                const uint64_t key = x_w[4];
+                __syncthreads();
+                return Walk{true, key, base_m, base_c, own_m};
+            }
+        }
+    };
+    // smallest race key of the block, the candidate that is earlier in sorted order (the larger `who`) on equal keys
+    const double inf = __longlong_as_double(0x7FF0000000000000ll);
+    auto block_first = [&](double& k, uint64_t& who) {
+#pragma unroll
+        for (int o = 32; o; o >>= 1) {
+            const double ko = __shfl_xor(k, o);
+            const uint64_t wo = __shfl_xor(who, o);
+            if (ko < k || (ko == k && wo > who)) {
+                k = ko;
+                who = wo;
+            }
+        }
+        __syncthreads();
+        if (lane_id() == 0) {
+            x_red_d[wave_id()] = k;
+            x_red_q[wave_id()] = who;
+        }
+        __syncthreads();
+        k = x_red_d[0];
+        who = x_red_q[0];
+        for (uint32_t w = 1; w < WS_WAVES; ++w) {
+            const double ko = x_red_d[w];
+            const uint64_t wo = x_red_q[w];
+            if (ko < k || (ko == k && wo > who)) {
+                k = ko;
+                who = wo;
+            }
+        }
+    };
+
+    // total mass, and the first key in sorted order
+    uint64_t z_own = 0, k_own = 0;
+    each_token([&](uint32_t i, float x) {
+        z_own += fx_of(x);
+        const uint64_t k = key64(x, i);
+        k_own = k > k_own ? k : k_own;
+    });
+    const uint64_t Zfx = block_sum(z_own, red_w);
+    if (t == 0) x_w[5] = 0ull;
+    __syncthreads();
+    atomicMax(&x_w[5], static_cast<unsigned long long>(k_own));
+    __syncthreads();
+    const uint64_t k_top = x_w[5];
+    const double Zs = static_cast<double>(Zfx) / kFx, Zfs = static_cast<double>(static_cast<float>(Zs));
+    const double u = in.u;
+    uint64_t kk = 0ull, kept_fx = Zfx;  // the kept set: keys >= kk, nk of them, kept_fx their mass
+    uint32_t nk = V;
+    // the race over every token at or above a key (E = -ln(1 - U), U hashed from the row's base and the token)
+    auto race_from = [&](uint64_t from, double Zk) {
+        auto race_key = [&](uint64_t cand) {
+            const double e = e_of(x_of(cand));
+            const uint64_t h = mix64(in.rbase + (static_cast<uint64_t>(static_cast<uint32_t>(id_of(cand))) + 1ull) * 0xE7037ED1A0B428DBull);
+            const double E = -log(1.0 - unit53(h));
+            return e > 0.0 ? E * Zk / e : inf;
+        };
+        double k1 = inf, k2nd = inf;
+        uint64_t w1 = 0;
+        each_token([&](uint32_t i, float x) {
+            const uint64_t c = key64(x, i);
+            if (c < from) return;
+            const double k = race_key(c);
+            if (k < k1 || (k == k1 && c > w1)) {
+                k2nd = k1;
+                k1 = k;
+                w1 = c;
+            } else if (k < k2nd) {
+                k2nd = k;
+            }
+        });
+        double kb = k1;
+        uint64_t wb = w1;
+        block_first(kb, wb);
+        double ks = (w1 == wb && k1 == kb) ? k2nd : k1;
+        uint64_t ws_ = 0;
+        block_first(ks, ws_);
+        if (!(kb < inf)) wb = k_top;  // no candidate has a mass: the first one in sorted order
+        out.token = id_of(wb);
+        out.ptok = e_of(x_of(wb)) / Zk;
+        out.mg_draw = ks < inf ? (ks - kb) / kb : 1.0;
+    };
+    if (prefix_mode || open_row) {  // the first n1_asked candidates
+        const Walk w1 = walk(false, in.n1_asked);
+        kk = w1.key;
+        kept_fx = w1.before_m + w1.own_m;
+        nk = in.n1_asked;
+    }
+    auto draw_walk = [&](double Zk_fx) {  // inverse-CDF draw among the first nk keys; false: the walk left them
+        const double T = u * Zk_fx;
+        const Walk wd = walk(true, static_cast<uint64_t>(floor(T)) + 1ull);
+        if (!wd.found || wd.before_c >= nk) return false;
+        const double inc = static_cast<double>(wd.before_m + wd.own_m), exc = static_cast<double>(wd.before_m);
+        out.token = id_of(wd.key);
+        out.ptok = e_of(x_of(wd.key)) / (Zk_fx / kFx);
+        out.mg_draw = fmin(inc - T, wd.before_c > 0u ? T - exc : 1e300) / Zk_fx;
+        return true;
+    };
+    if (!open_row) {
+        if (use_top_p) {
+            double Xf = in.top_p * (prefix_mode ? static_cast<double>(kept_fx) : (in.top_k > 0 ? Zs : Zfs) * kFx);
+            auto cut_at = [&](double xf) { return walk(true, xf > 1.0 ? static_cast<uint64_t>(ceil(xf)) : 1ull); };
+            Walk w2 = cut_at(Xf);
+            if (!prefix_mode && in.top_k == 0 && (!w2.found || w2.before_c >= 16384u)) {  // past the engine's candidates: the complete row
+                Xf = in.top_p * static_cast<double>(Zfx);
+                w2 = cut_at(Xf);
+            }
+            if (w2.found && w2.before_c < nk) {
+                const double inc = static_cast<double>(w2.before_m + w2.own_m), exc = static_cast<double>(w2.before_m);
+                out.mg_top_p = fmin(inc - Xf, w2.before_c > 0u ? Xf - exc : Xf) / Xf;
+                nk = w2.before_c + 1u;
+                kk = w2.key;
+                kept_fx = w2.before_m + w2.own_m;
+            } else {
+                out.mg_top_p = 0.0;
+            }
+        }
+        if (use_min_p) {
+            // tokens with at least min_p of the largest mass: a prefix of the sorted order
+            const double min_p = in.min_p;
+            uint32_t c_own = 0;
+            uint64_t s_own = 0, kmin_own = ~0ull;
+            double near = 1.0;
+            each_token([&](uint32_t i, float x) {
+                const double e = e_of(x);
+                near = fmin(near, fabs(e - min_p) / min_p);
+                if (e >= min_p) {
+                    ++c_own;
+                    s_own += e > 0.0 ? static_cast<uint64_t>(__double2ll_rn(e * kFx)) : 0ull;
+                    const uint64_t k = key64(x, i);
+                    kmin_own = k < kmin_own ? k : kmin_own;
+                }
+            });
+            const uint32_t passed = block_sum(c_own, x_red_u);
+            const uint64_t s_pass = block_sum(s_own, red_w);
+            if (t == 0) {
+                x_w[0] = ~0ull;
+                x_w[1] = 0x7FF0000000000000ull;
+            }
+            __syncthreads();
+            atomicMin(&x_w[0], static_cast<unsigned long long>(kmin_own));
+            atomicMin(&x_w[1], static_cast<unsigned long long>(__double_as_longlong(near)));  // non-negative doubles order like their bits
+            __syncthreads();
+            const uint64_t k_floor = x_w[0];
+            out.mg_min_p = __longlong_as_double(static_cast<long long>(x_w[1]));
+            __syncthreads();
+            if (passed < nk) {
+                if (passed >= 1u) {
+                    nk = passed;
+                    kk = k_floor;
+                    kept_fx = s_pass;
+                } else {  // the top candidate always stays
+                    nk = 1u;
+                    kk = k_top;
+                    kept_fx = fx_of(x_of(k_top));
+                }
+            }
+        }
+        const double Zk = static_cast<double>(kept_fx) / kFx;
+        if (race) {
+            race_from(kk, Zk);
+        } else if (!draw_walk(static_cast<double>(kept_fx))) {  // the walk falls through to the last kept candidate
+            out.token = id_of(kk ? kk : k_top);
+            out.ptok = e_of(x_of(kk ? kk : k_top)) / Zk;
+            out.mg_draw = 0.0;
+        }
+        out.Zk = Zk;
+    } else {
+        // an open row: the listed candidates in sorted order over the float normaliser, then the rest in id order
+        out.list_mass = static_cast<double>(kept_fx) / kFx;
+        out.target = u * Zfs;
+        if (race && out.target < out.list_mass) {
+            race_from(kk, Zfs);
+            out.mg_draw = fmin(out.mg_draw, fabs(out.target - out.list_mass) / Zfs);
+        } else if (!draw_walk(Zfs * kFx)) {
+            out.rest = 1u;
+        } else if (race) {
+            out.mg_draw = fmin(out.mg_draw, fabs(out.target - out.list_mass) / Zfs);
+        }
+        out.Zk = Zfs;
+    }
+    out.n3 = nk;
+    out.kept_key = kk;
+    __syncthreads();
+    return out;
+}
+
 // Debug builds (-DWS_PHASE_TIMERS): thread 0 notes the shader clock at each mark in LDS (no barrier, no global store on
 // the way) and writes the times since the start of the row into kept_logits when the row is done.
 #ifdef WS_PHASE_TIMERS
@@ -1323,23 +1676,6 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (t == 0) s_cnt = s_u[4] = s_u[5] = 0;
     __syncthreads();  // the last reads of pm / pc are done: their LDS is the key buffer and the candidate list from here
 
-    if (flags & kOverflow) {
-        if (t == 0) {
-            A.token[row] = -1;
-            A.flags[row] = flags;
-            if (A.prob) A.prob[row] = 0.f;
-            if (A.n_kept) A.n_kept[row] = 0u;
-            if (A.stats) {
-                A.stats[2 * row] = m;
-                A.stats[2 * row + 1] = static_cast<float>(Z);
-            }
-            if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
-            if (A.query_prob) A.query_prob[row] = 0.0;
-            if (A.entropy) A.entropy[row] = 0.0;
-        }
-        return;
-    }
-
     WS_MARK(3);
     // what the cuts and the draw leave behind: filled by the bucket finish inside pass 3 or by the sort-based one after it
     double mg_top_p = 1.0, mg_min_p = 1.0, mg_draw = 1.0;
@@ -1351,7 +1687,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     bool finished = false;
     bool finished_lean = false;
     // ------------------------------------------------------------------ pass 3: gather, sort, exact masses
-    {
+    // (a row whose ranges hold more candidates than the list skips all of this and takes the exact path further down)
+    if (!(flags & kOverflow)) {  // uniform
         const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = static_cast<uint32_t>(r0hi - r0lo);
         const uint32_t u1 = static_cast<uint32_t>(r1lo), w1 = r1hi >= r1lo ? static_cast<uint32_t>(r1hi - r1lo) : 0u;
         const bool two = r1hi >= r1lo;
@@ -1744,24 +2081,210 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             });
     }
     __syncthreads();
-    if (flags & kOverflow) {  // uniform: more cached hits than the list holds
-        if (t == 0) {
-            A.token[row] = -1;
-            A.flags[row] = flags;
-            if (A.prob) A.prob[row] = 0.f;
-            if (A.n_kept) A.n_kept[row] = 0u;
-            if (A.stats) {
-                A.stats[2 * row] = m;
-                A.stats[2 * row + 1] = static_cast<float>(Z);
-            }
-            if (A.margin) A.margin[3 * row] = A.margin[3 * row + 1] = A.margin[3 * row + 2] = 0.0;
-            if (A.query_prob) A.query_prob[row] = 0.0;
-            if (A.entropy) A.entropy[row] = 0.0;
-        }
-        return;
-    }
     WS_MARK(4);
-    if (!finished) {  // uniform: the sort-based finish
+    // The race draw's pieces (src/sampling/sampler.cpp:80-106, src/common/spec_sample.cpp:83-87): E(token) = -ln(1 - U) with U
+    // hashed from (seed, step, token); a candidate's key is E / p.
+    const uint64_t rbase = mix64((seed ^ 0xA0761D6478BD642Full) + (step + 1ull) * 0x9E3779B97F4A7C15ull);
+    const double inf = __longlong_as_double(0x7FF0000000000000ll);
+    auto hash_of = [&](uint32_t id) { return mix64(rbase + (static_cast<uint64_t>(id) + 1ull) * 0xE7037ED1A0B428DBull); };
+    auto race_key = [&](uint64_t cand, double Zk) {  // E / p of a candidate given as (logit key, ~id); inf when it has no mass
+        const float x = unkey32(static_cast<uint32_t>(cand >> 32));
+        const double e = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
+        const double E = -log(1.0 - unit53(hash_of(0xffffffffu - static_cast<uint32_t>(cand))));
+        return e > 0.0 ? E * Zk / e : inf;
+    };
+    // smallest key of the block, the candidate that is earlier in sorted order (the larger `who`) on equal keys
+    auto block_first = [&](double& k, uint64_t& who) {
+        const uint32_t lane = static_cast<uint32_t>(lane_id());
+        const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+#pragma unroll
+        for (int o = 32; o; o >>= 1) {
+            const double ko = __shfl_xor(k, o);
+            const uint64_t wo = __shfl_xor(who, o);
+            if (ko < k || (ko == k && wo > who)) {
+                k = ko;
+                who = wo;
+            }
+        }
+        __syncthreads();
+        if (lane == 0) {
+            red_d[wv] = k;
+            red_q[wv] = who;
+        }
+        __syncthreads();
+        k = red_d[0];
+        who = red_q[0];
+        for (uint32_t w = 1; w < WS_WAVES; ++w) {
+            const double ko = red_d[w];
+            const uint64_t wo = red_q[w];
+            if (ko < k || (ko == k && wo > who)) {
+                k = ko;
+                who = wo;
+            }
+        }
+    };
+    // An open row whose uniform falls past the listed candidates (keys >= list_key, mass list_mass): the rest of the walk.
+    // Leaves token, ptok and mg_draw. Uses keys[] as scratch.
+    auto open_rest = [&](uint64_t list_key, double list_mass, double target, double Zk) {
+        bool found = false;
+        // Past the listed candidates: the sum goes on over the tokens outside the list, in id order
+        // (src/sampling/sampler.cpp:132-146). One more sweep over the row leaves the mass of every chunk of
+        // consecutive tokens (the 64 vectors one wave loads with one instruction: 256 fp32 or 512 bf16 tokens) in
+        // LDS; every wave then finds the chunk in which the sum passes the target and scans that chunk. Masses
+        // here come from the 32-bit exponential unit (1.2e-7 relative), so the running sum is good to ~1e-7 of
+        // the row's mass: inside the smallest `tol`.
+        const uint32_t lane = static_cast<uint32_t>(lane_id());
+        const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+        const double rest = target - list_mass;
+        // mass of a token outside the list: 2^((x - m) * inv_t * log2 e) with the product carried in two floats (the
+        // exponent to ~1e-7 absolute), 0 for listed tokens, for -inf and for NaN (masked, or touched in the sweep)
+        const double k2 = static_cast<double>(inv_t) * 1.4426950408889634;
+        const float kh = static_cast<float>(k2), kl = static_cast<float>(k2 - static_cast<double>(kh));
+        const float cut_x = unkey32(static_cast<uint32_t>(list_key >> 32));
+        const uint32_t cut_id = 0xffffffffu - static_cast<uint32_t>(list_key);
+        auto mass = [&](uint32_t i, float x) -> float {
+            const float d = __fsub_rn(x, m);
+            const float yh = __fmul_rn(d, kh);
+            const float yl = __fmaf_rn(d, kl, __fmaf_rn(d, kh, -yh));
+            const float n = rintf(yh);
+            const float e = ldexpf(__builtin_amdgcn_exp2f(__fadd_rn(__fsub_rn(yh, n), yl)), static_cast<int>(n));
+            const bool out = (yh > -140.f) & !(x > cut_x) & (!(x == cut_x) | (i > cut_id));  // no branches: bitwise
+            return out ? e : 0.f;
+        };
+        const uint32_t per = rv.dtype == 0 ? 4u : 8u, shift = rv.dtype == 0 ? 8u : 9u;
+        const uint32_t n_vec = rv.vec ? V / per : 0u;  // tokens below n_vec * per arrive in 128-bit vectors
+        const uint32_t n_chunks = (V >> shift) + 1u;
+        double* chunk = reinterpret_cast<double*>(keys);
+        WS_MARK(27);
+        __syncthreads();  // every wave has taken what it needs from keys[] and ps[]
+        for (uint32_t c = t; c < n_chunks; c += WS_BLOCK) chunk[c] = 0.0;
+        __syncthreads();
+        if (n_vec) {
+            float acc[2 * kWide] = {};  // per group of four tokens of a load (a bf16 vector has two), slot >> 2
+            stream_row_wide(
+                rv,
+                [&](uint32_t i, float x, int slot) {
+                    acc[slot >> 2] += mass(i, x);  // tokens after the last whole vector land here too and are never written out
+                },
+                [&](uint32_t j0, uint32_t) {
+                    if (j0 == 0xffffffffu) return;  // the tokens after the last whole vector follow below
+#pragma unroll
+                    for (int u = 0; u < kWide; ++u) {
+                        const uint32_t v0 = j0 + u * WS_BLOCK + wv * 64u;  // first vector of this wave's load
+                        const float own = per == 4u ? acc[u] : __fadd_rn(acc[2 * u], acc[2 * u + 1]);
+                        const double tot = wave_sum(static_cast<double>(own));
+                        if (lane == 0 && v0 < n_vec) chunk[v0 >> 6] = tot;
+                    }
+#pragma unroll
+                    for (int k = 0; k < 2 * kWide; ++k) acc[k] = 0.f;
+                });
+        }
+        __syncthreads();
+        WS_MARK(28);
+        // touched tokens were skipped by the sweep: their adjusted logits, by rank
+        if (n_touched) {
+            const uint32_t span = (nW + WS_BLOCK - 1) / WS_BLOCK;
+            const uint32_t w0 = t * span, w1 = min(w0 + span, nW);
+            for (uint32_t w = w0; w < w1; ++w) {
+                uint32_t bits = touched[w];
+                uint32_t r = wprefix[w];
+                while (bits) {
+                    const uint32_t i = (w << 5) + (__ffs(bits) - 1u);
+                    bits &= bits - 1u;
+                    const float e = i < n_vec * per ? mass(i, pv[r]) : 0.f;
+                    ++r;
+                    if (e != 0.f) unsafeAtomicAdd(&chunk[i >> shift], static_cast<double>(e));
+                }
+            }
+        }
+        // tokens after the last whole vector (a row that is not aligned has only such tokens): 64 per wave and round
+        for (uint32_t i0 = n_vec * per + wv * 64u; i0 < V; i0 += WS_BLOCK) {
+            const uint32_t i = i0 + lane;
+            const double tot = wave_sum(i < V ? static_cast<double>(mass(i, adjusted_logit(rv, i))) : 0.0);
+            if (lane == 0 && tot != 0.0) unsafeAtomicAdd(&chunk[i0 >> shift], tot);
+        }
+        __syncthreads();
+        WS_MARK(29);
+        // chunk in which the sum passes `rest`: lane l adds up chunks [l g, (l + 1) g), a scan over the lanes, then a
+        // walk through the group of the first lane that is past it
+        const uint32_t g = (n_chunks + 63u) >> 6;
+        double mine = 0;
+        for (uint32_t c = lane * g; c < min(n_chunks, (lane + 1u) * g); ++c) mine += chunk[c];
+        const double upto = wave_incl_scan(mine);
+        const uint64_t past = __ballot(upto > rest);
+        double before = 0;
+        uint32_t cx = n_chunks;
+        if (past) {
+            const int src = __ffsll(static_cast<unsigned long long>(past)) - 1;
+            before = __shfl(upto - mine, src);
+            for (uint32_t c = src * g; c < min(n_chunks, (src + 1u) * g); ++c) {
+                const double tc = chunk[c];
+                if (before + tc > rest) {
+                    cx = c;
+                    break;
+                }
+                before += tc;
+            }
+        }
+        if (cx < n_chunks) {
+            // every wave scans the chunk: lane l owns its l-th vector, or 4 (8) tokens of a row without vectors
+            const uint32_t lo = cx << shift;
+            float e[8], half[2] = {0.f, 0.f};  // summed as the sweep sums them: by groups of four
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; ++q) {
+                const uint32_t i = lo + per * lane + q;
+                e[q] = (q < per && i < V) ? mass(i, adjusted_logit(rv, i)) : 0.f;
+                half[q >> 2] += e[q];
+            }
+            const double own = static_cast<double>(__fadd_rn(half[0], half[1]));
+            const double incl = before + wave_incl_scan(own);
+            uint64_t over = __ballot(incl > rest);
+            const uint64_t any = __ballot(own > 0.0);
+            bool seam = false;
+            if (!over && any) {  // the chunk's total was added up in another order: its last token with a mass
+                over = 1ull << (63 - __builtin_clzll(any));
+                seam = true;
+            }
+            if (over) {
+                const int src = __ffsll(static_cast<unsigned long long>(over)) - 1;
+                double c = incl - own, in = 0, ex = 0, pe = 0;
+                int32_t tk = -1;
+#pragma unroll
+                for (uint32_t q = 0; q < 8u; ++q) {
+                    if (e[q] > 0.f && (seam || (tk < 0 && c + e[q] > rest))) {
+                        tk = static_cast<int32_t>(lo + per * lane + q);
+                        ex = c;
+                        in = c + e[q];
+                        pe = e[q];
+                    }
+                    c += e[q];
+                }
+                token = __shfl(tk, src);
+                in = __shfl(in, src);
+                ex = __shfl(ex, src);
+                ptok = __shfl(pe, src) / Zk;
+                mg_draw = seam ? 0.0 : fmin(in - rest, rest - ex) / Zk;
+                found = token >= 0;
+            }
+        }
+        WS_MARK(30);
+        if (!found) {
+            // the walk ends without passing the target (the float normaliser lies above the exact sum): the
+            // reference returns the last token it walked, the highest id outside the list
+            token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(list_key));  // every token is listed: the last of the list
+            for (uint32_t j = V; j-- > 0u;) {
+                const float x = adjusted_logit(rv, j);
+                if (!(key64(x, j) >= list_key)) {
+                    token = static_cast<int32_t>(j);
+                    break;
+                }
+            }
+            ptok = 0;
+            mg_draw = 0.0;
+            found = true;
+        }
+    };
+    if (!finished && !(flags & kOverflow)) {  // uniform: the sort-based finish
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
         float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
@@ -2201,43 +2724,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         raced = true;
         const uint32_t lane = static_cast<uint32_t>(lane_id());
         const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
-        const uint64_t rbase = mix64((seed ^ 0xA0761D6478BD642Full) + (step + 1ull) * 0x9E3779B97F4A7C15ull);
-        const double inf = __longlong_as_double(0x7FF0000000000000ll);
-        auto hash_of = [&](uint32_t id) { return mix64(rbase + (static_cast<uint64_t>(id) + 1ull) * 0xE7037ED1A0B428DBull); };
-        auto key_of = [&](uint64_t cand) {  // E / p of a candidate given as (logit key, ~id); inf when it has no mass
-            const float x = unkey32(static_cast<uint32_t>(cand >> 32));
-            const double e = exp(-(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t)));
-            const double E = -log(1.0 - unit53(hash_of(0xffffffffu - static_cast<uint32_t>(cand))));
-            return e > 0.0 ? E * Zk / e : inf;
-        };
-        // smallest key of the block, the candidate that is earlier in sorted order (the larger `who`) on equal keys
-        auto block_first = [&](double& k, uint64_t& who) {
-#pragma unroll
-            for (int o = 32; o; o >>= 1) {
-                const double ko = __shfl_xor(k, o);
-                const uint64_t wo = __shfl_xor(who, o);
-                if (ko < k || (ko == k && wo > who)) {
-                    k = ko;
-                    who = wo;
-                }
-            }
-            __syncthreads();
-            if (lane == 0) {
-                red_d[wv] = k;
-                red_q[wv] = who;
-            }
-            __syncthreads();
-            k = red_d[0];
-            who = red_q[0];
-            for (uint32_t w = 1; w < WS_WAVES; ++w) {
-                const double ko = red_d[w];
-                const uint64_t wo = red_q[w];
-                if (ko < k || (ko == k && wo > who)) {
-                    k = ko;
-                    who = wo;
-                }
-            }
-        };
+        auto key_of = [&](uint64_t cand) { return race_key(cand, Zk); };
         const uint64_t* cand = keys;
         uint32_t n_cand = n3;  // top-k and open rows: the kept set is the first n3 entries of the sorted list
         if (!prefix_mode && !open_row) {
@@ -2354,163 +2841,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         }
         if (!found && open_row) {
-            // Past the listed candidates: the sum goes on over the tokens outside the list, in id order
-            // (src/sampling/sampler.cpp:132-146). One more sweep over the row leaves the mass of every chunk of
-            // consecutive tokens (the 64 vectors one wave loads with one instruction: 256 fp32 or 512 bf16 tokens) in
-            // LDS; every wave then finds the chunk in which the sum passes the target and scans that chunk. Masses
-            // here come from the 32-bit exponential unit (1.2e-7 relative), so the running sum is good to ~1e-7 of
-            // the row's mass: inside the smallest `tol`.
-            const uint32_t lane = static_cast<uint32_t>(lane_id());
-            const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
-            const uint64_t list_key = kept_key;
-            const double rest = target - inc_of(i_last);
-            // mass of a token outside the list: 2^((x - m) * inv_t * log2 e) with the product carried in two floats (the
-            // exponent to ~1e-7 absolute), 0 for listed tokens, for -inf and for NaN (masked, or touched in the sweep)
-            const double k2 = static_cast<double>(inv_t) * 1.4426950408889634;
-            const float kh = static_cast<float>(k2), kl = static_cast<float>(k2 - static_cast<double>(kh));
-            const float cut_x = unkey32(static_cast<uint32_t>(list_key >> 32));
-            const uint32_t cut_id = 0xffffffffu - static_cast<uint32_t>(list_key);
-            auto mass = [&](uint32_t i, float x) -> float {
-                const float d = __fsub_rn(x, m);
-                const float yh = __fmul_rn(d, kh);
-                const float yl = __fmaf_rn(d, kl, __fmaf_rn(d, kh, -yh));
-                const float n = rintf(yh);
-                const float e = ldexpf(__builtin_amdgcn_exp2f(__fadd_rn(__fsub_rn(yh, n), yl)), static_cast<int>(n));
-                const bool out = (yh > -140.f) & !(x > cut_x) & (!(x == cut_x) | (i > cut_id));  // no branches: bitwise
-                return out ? e : 0.f;
-            };
-            const uint32_t per = rv.dtype == 0 ? 4u : 8u, shift = rv.dtype == 0 ? 8u : 9u;
-            const uint32_t n_vec = rv.vec ? V / per : 0u;  // tokens below n_vec * per arrive in 128-bit vectors
-            const uint32_t n_chunks = (V >> shift) + 1u;
-            double* chunk = reinterpret_cast<double*>(keys);
-            WS_MARK(27);
-            __syncthreads();  // every wave has taken what it needs from keys[] and ps[]
-            for (uint32_t c = t; c < n_chunks; c += WS_BLOCK) chunk[c] = 0.0;
-            __syncthreads();
-            if (n_vec) {
-                float acc[2 * kWide] = {};  // per group of four tokens of a load (a bf16 vector has two), slot >> 2
-                stream_row_wide(
-                    rv,
-                    [&](uint32_t i, float x, int slot) {
-                        acc[slot >> 2] += mass(i, x);  // tokens after the last whole vector land here too and are never written out
-                    },
-                    [&](uint32_t j0, uint32_t) {
-                        if (j0 == 0xffffffffu) return;  // the tokens after the last whole vector follow below
-#pragma unroll
-                        for (int u = 0; u < kWide; ++u) {
-                            const uint32_t v0 = j0 + u * WS_BLOCK + wv * 64u;  // first vector of this wave's load
-                            const float own = per == 4u ? acc[u] : __fadd_rn(acc[2 * u], acc[2 * u + 1]);
-                            const double tot = wave_sum(static_cast<double>(own));
-                            if (lane == 0 && v0 < n_vec) chunk[v0 >> 6] = tot;
-                        }
-#pragma unroll
-                        for (int k = 0; k < 2 * kWide; ++k) acc[k] = 0.f;
-                    });
-            }
-            __syncthreads();
-            WS_MARK(28);
-            // touched tokens were skipped by the sweep: their adjusted logits, by rank
-            if (n_touched) {
-                const uint32_t span = (nW + WS_BLOCK - 1) / WS_BLOCK;
-                const uint32_t w0 = t * span, w1 = min(w0 + span, nW);
-                for (uint32_t w = w0; w < w1; ++w) {
-                    uint32_t bits = touched[w];
-                    uint32_t r = wprefix[w];
-                    while (bits) {
-                        const uint32_t i = (w << 5) + (__ffs(bits) - 1u);
-                        bits &= bits - 1u;
-                        const float e = i < n_vec * per ? mass(i, pv[r]) : 0.f;
-                        ++r;
-                        if (e != 0.f) unsafeAtomicAdd(&chunk[i >> shift], static_cast<double>(e));
-                    }
-                }
-            }
-            // tokens after the last whole vector (a row that is not aligned has only such tokens): 64 per wave and round
-            for (uint32_t i0 = n_vec * per + wv * 64u; i0 < V; i0 += WS_BLOCK) {
-                const uint32_t i = i0 + lane;
-                const double tot = wave_sum(i < V ? static_cast<double>(mass(i, adjusted_logit(rv, i))) : 0.0);
-                if (lane == 0 && tot != 0.0) unsafeAtomicAdd(&chunk[i0 >> shift], tot);
-            }
-            __syncthreads();
-            WS_MARK(29);
-            // chunk in which the sum passes `rest`: lane l adds up chunks [l g, (l + 1) g), a scan over the lanes, then a
-            // walk through the group of the first lane that is past it
-            const uint32_t g = (n_chunks + 63u) >> 6;
-            double mine = 0;
-            for (uint32_t c = lane * g; c < min(n_chunks, (lane + 1u) * g); ++c) mine += chunk[c];
-            const double upto = wave_incl_scan(mine);
-            const uint64_t past = __ballot(upto > rest);
-            double before = 0;
-            uint32_t cx = n_chunks;
-            if (past) {
-                const int src = __ffsll(static_cast<unsigned long long>(past)) - 1;
-                before = __shfl(upto - mine, src);
-                for (uint32_t c = src * g; c < min(n_chunks, (src + 1u) * g); ++c) {
-                    const double tc = chunk[c];
-                    if (before + tc > rest) {
-                        cx = c;
-                        break;
-                    }
-                    before += tc;
-                }
-            }
-            if (cx < n_chunks) {
-                // every wave scans the chunk: lane l owns its l-th vector, or 4 (8) tokens of a row without vectors
-                const uint32_t lo = cx << shift;
-                float e[8], half[2] = {0.f, 0.f};  // summed as the sweep sums them: by groups of four
-#pragma unroll
-                for (uint32_t q = 0; q < 8u; ++q) {
-                    const uint32_t i = lo + per * lane + q;
-                    e[q] = (q < per && i < V) ? mass(i, adjusted_logit(rv, i)) : 0.f;
-                    half[q >> 2] += e[q];
-                }
-                const double own = static_cast<double>(__fadd_rn(half[0], half[1]));
-                const double incl = before + wave_incl_scan(own);
-                uint64_t over = __ballot(incl > rest);
-                const uint64_t any = __ballot(own > 0.0);
-                bool seam = false;
-                if (!over && any) {  // the chunk's total was added up in another order: its last token with a mass
-                    over = 1ull << (63 - __builtin_clzll(any));
-                    seam = true;
-                }
-                if (over) {
-                    const int src = __ffsll(static_cast<unsigned long long>(over)) - 1;
-                    double c = incl - own, in = 0, ex = 0, pe = 0;
-                    int32_t tk = -1;
-#pragma unroll
-                    for (uint32_t q = 0; q < 8u; ++q) {
-                        if (e[q] > 0.f && (seam || (tk < 0 && c + e[q] > rest))) {
-                            tk = static_cast<int32_t>(lo + per * lane + q);
-                            ex = c;
-                            in = c + e[q];
-                            pe = e[q];
-                        }
-                        c += e[q];
-                    }
-                    token = __shfl(tk, src);
-                    in = __shfl(in, src);
-                    ex = __shfl(ex, src);
-                    ptok = __shfl(pe, src) / Zk;
-                    mg_draw = seam ? 0.0 : fmin(in - rest, rest - ex) / Zk;
-                    found = token >= 0;
-                }
-            }
-            WS_MARK(30);
-            if (!found) {
-                // the walk ends without passing the target (the float normaliser lies above the exact sum): the
-                // reference returns the last token it walked, the highest id outside the list
-                token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(list_key));  // every token is listed: the last of the list
-                for (uint32_t j = V; j-- > 0u;) {
-                    const float x = adjusted_logit(rv, j);
-                    if (!(key64(x, j) >= list_key)) {
-                        token = static_cast<int32_t>(j);
-                        break;
-                    }
-                }
-                ptok = 0;
-                mg_draw = 0.0;
-                found = true;
-            }
+            open_rest(kept_key, inc_of(i_last), target, Zk);
+            found = true;
         }
         if (!found) {
             if (i_last < n_list) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
@@ -2525,6 +2857,57 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (race && open_row) mg_draw = fmin(mg_draw, fabs(target - inc_of(i_last)) / Zk);  // the list-or-rest decision
     Zk_out = Zk;
     }  // the sort-based finish
+
+    // ------------------------------------------------------------------ the exact path
+    // Rows the list cannot hold - a top-k beyond its capacity, thousands of candidates with one logit, a flat row whose
+    // draw bins alone overflow it - are answered by exact_row, without any list.
+    auto each_token = [&](auto&& f) {  // every token with its adjusted logit, four loads in flight per thread
+        for (uint32_t i0 = 0; i0 < V; i0 += 4u * WS_BLOCK) {
+            float xr[4];
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) xr[q] = raw_logit(rv, min(i0 + q * WS_BLOCK + t, V - 1u));
+#pragma unroll
+            for (uint32_t q = 0; q < 4u; ++q) {
+                const uint32_t i = i0 + q * WS_BLOCK + t;
+                if (i < V) f(i, is_touched(rv, i) ? rv.pv[rank_of(rv, i)] : (is_allowed(rv, i) ? xr[q] : -INFINITY));
+            }
+        }
+    };
+    bool finished_slow = false;
+    if ((flags & kOverflow) && m > -INFINITY) {  // uniform
+        flags &= ~kOverflow;
+        finished = finished_slow = true;
+        finished_lean = false;
+        ExactIn in;
+        in.base = rv.base;
+        in.allow = rv.allow;
+        in.V = V;
+        in.dtype = rv.dtype;
+        in.touched_at = rv.touched ? A.lds_ab : 0xffffffffu;
+        in.m = m;
+        in.inv_t = inv_t;
+        in.top_k = top_k;
+        in.n1_asked = n1_asked;
+        in.top_p = top_p;
+        in.min_p = min_p;
+        in.u = batch_uniform(A.rng, seed, row, step, 0);
+        in.rbase = rbase;
+        in.mode = (prefix_mode ? 1u : 0u) | (open_row ? 2u : 0u) | (use_top_p ? 4u : 0u) | (use_min_p ? 8u : 0u) | (race ? 16u : 0u);
+        __syncthreads();  // whatever used the LDS before is done with it
+        const ExactOut out = exact_row(in);
+        token = out.token;
+        ptok = out.ptok;
+        n3 = out.n3;
+        kept_key = out.kept_key;
+        Zk_out = out.Zk;
+        mg_top_p = out.mg_top_p;
+        mg_min_p = out.mg_min_p;
+        mg_draw = out.mg_draw;
+        if (out.rest) {  // an open row whose uniform falls past the listed candidates
+            open_rest(kept_key, out.list_mass, out.target, Zk_out);
+            if (race) mg_draw = fmin(mg_draw, fabs(out.target - out.list_mass) / Zk_out);
+        }
+    }
     // zero-mass tail candidates a top-k kept (no top-p / min-p cut them away again)
     const uint32_t tail_extra = (!use_top_p && !use_min_p && n3 == n1) ? n1_asked - n1 : 0u;
     if (mg_top_p < tol) flags |= kNearTopP;
@@ -2546,7 +2929,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         };
         __syncthreads();
-        if (finished_lean) {  // the keys lie in the buckets' places
+        if (finished_slow) {  // no list: every kept token of the row
+            each_token([&](uint32_t i, float x) { term(key64(x, i)); });
+        } else if (finished_lean) {  // the keys lie in the buckets' places
             const uint32_t* cnt_of = reinterpret_cast<const uint32_t*>(s_pool + 128);
             const uint32_t shift = A.lds_tie ? 5u : 4u;
             for (uint32_t slot = t; slot < (128u << shift); slot += WS_BLOCK)
@@ -2562,7 +2947,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 h = (s_list + log(Zk_out) * m_list) / Zk_out;
             } else {
                 const bool past_r0 = has_r1 && n3 >= c1base;  // the cut lies in range 1 or at its edge: the bins between are kept too
-                const double s_bins = h_before + (past_r0 ? h_between : 0.0);
+                const double s_bins = finished_slow ? 0.0 : h_before + (past_r0 ? h_between : 0.0);
                 if (s_bins != 0.0) flags |= kApproxEntropy;
                 h = log(Zk_out) + (s_bins + s_list) / Zk_out;
             }
