@@ -132,6 +132,9 @@ enum {
     WS_FLAG_OPEN = 1u << 6,        /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order
                                       (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
+    WS_FLAG_SPLIT_TIMEOUT = 1u << 8, /* a row split over several workgroups (see ws_batch.workspace) whose parts did not all
+                                      start within about a second - the launch shared the GPU with work that held its compute
+                                      units: token = -1; zero-fill the workspace before it is used again */
     WS_FLAG_APPROX_ENTROPY = 1u << 7 /* `entropy` counts the kept tokens outside the gathered bins at the middle of their
                                       histogram bin (each within 1/128 of its place: the entropy is within 1/128 absolute,
                                       usually far closer) instead of one by one; rows whose kept set a
@@ -193,7 +196,11 @@ typedef struct ws_batch {
     float* kept_logits; /* out (may be NULL): penalty-applied logits of kept_ids */
     uint32_t kept_cap;
 
-    void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes */
+    void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes, or NULL. It serves small batches: with
+                               fewer rows than the GPU has compute units a row is worked on by several workgroups, which
+                               meet in this memory. The caller zero-fills it once before its first use and leaves it
+                               alone afterwards: every launch puts back the zeros the next one needs. Two launches that overlap in time need a workspace each.
+                               Without it (or with too little of it) every row is one workgroup's. */
     uint64_t workspace_bytes;
     double tol;             /* flag tolerance, relative; values below 1e-6 (and 0) mean 1e-6, the accuracy of the mass estimates */
     int32_t mode;           /* WS_MODE_* */
@@ -213,6 +220,9 @@ typedef struct ws_batch {
     double* entropy;            /* out (may be NULL): -sum p ln p over the kept set (renormalised p; an open row: over its
                                    256 candidates with their shares of the whole row), what the typical acceptance rule
                                    compares with (src/sampling/acceptor.cpp:77-84). See WS_FLAG_APPROX_ENTROPY. */
+    uint32_t max_split;         /* most workgroups a row may be split over (a power of two up to 16, rows * parts within the
+                                   GPU's compute units, at least 16384 tokens a part): 0 = the library decides (8 or 16
+                                   parts when the batch is small enough for that, else none), 1 = never split */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

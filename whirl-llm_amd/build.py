@@ -6,13 +6,15 @@
 
 Usage: python whirl-llm_amd/build.py
 """
+import concurrent.futures
 import os
 import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "csrc", "ws_abi.hip")
-SRC_FUSED = os.path.join(HERE, "csrc", "ws_fused.hip")
+SRC_FUSED = os.path.join(HERE, "csrc", "ws_fused.hip")  # the single-sweep sampler kernel
+SRC_SPLIT = os.path.join(HERE, "csrc", "ws_split.hip")  # the same kernel for rows split over several workgroups
 # packed FP32 instructions are switched off for every device compile of this repository
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          # the fused sweep is one fully unrolled loop of ~20 batches (its bin cache must stay in registers)
@@ -38,8 +40,15 @@ def build(verbose=True):
     so = os.path.join(HERE, "libwhirl_sampling_hip.so")
     co = os.path.join(HERE, "whirl_sampling_gfx950.co")
     host = os.path.join(HERE, "libwhirl_sampling_host.so")
-    run([hipcc, *FLAGS, "-fPIC", "-shared", "-o", so, SRC, SRC_FUSED])
-    run([hipcc, *FLAGS, "--genco", "-o", co, SRC])
+    # the three translation units and the bare code object side by side (each takes a minute or two), then the link
+    objdir = os.path.join(HERE, "csrc", "obj")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.basename(src)[:-4] + ".o") for src in (SRC, SRC_FUSED, SRC_SPLIT)]
+    jobs = [[hipcc, *FLAGS, "-fPIC", "-c", "-o", obj, src] for obj, src in zip(objs, (SRC, SRC_FUSED, SRC_SPLIT))]
+    jobs.append([hipcc, *FLAGS, "--genco", "-o", co, SRC])
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(run, jobs))
+    run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", so, *objs])
     # host layer: plain C++20, no device code; -ffp-contract=off keeps the float arithmetic of the penalties unfused
     run([os.environ.get("CXX", "g++"), "-std=c++20", "-O2", "-fPIC", "-shared", "-ffp-contract=off", "-Wall", "-Wextra",
          "-D__HIP_PLATFORM_AMD__", "-I" + INCLUDE, "-I" + os.path.join(rocm, "include"), "-o", host, *HOST_SRCS,

@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstring>
 
 #include "ws_accept.h"
@@ -18,6 +20,8 @@
 namespace ws {
 // ws_fused.hip: the fused-sweep kernel, built for 512-thread workgroups
 int launch_fused(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
+// ws_split.hip: the same with rows split over several workgroups
+int launch_split(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
 }  // namespace ws
 
 namespace {
@@ -26,6 +30,12 @@ inline hipStream_t S(void* s) { return static_cast<hipStream_t>(s); }
 inline int done() { return static_cast<int>(hipGetLastError()); }
 
 constexpr uint32_t kMaxLds = 160u * 1024u;  // LDS per workgroup on gfx950
+// what the sampler kernel declares statically (reduction scratch, exponent tables, the exact path's words), rounded up
+#ifdef WS_PHASE_TIMERS
+constexpr uint32_t kStaticLds = 4096u + 512u;  // + the phase marks
+#else
+constexpr uint32_t kStaticLds = 4096u;
+#endif
 
 struct BatchPlan {
     uint32_t patch_cap;
@@ -34,9 +44,23 @@ struct BatchPlan {
     uint32_t lds_tie;
     uint32_t lds_total;
     bool fused;
-    uint64_t workspace;
+    uint32_t split_log2;  // the most parts per row that pay for this batch
+    uint64_t workspace;   // bytes for that
     int err;
 };
+
+// compute units of the current device (one workgroup of the sampler per unit)
+int compute_units() {
+    static std::atomic<int> known[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    int n = known[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = -1;
+        known[dev].store(n, std::memory_order_relaxed);
+    }
+    return n > 0 ? n : 0;
+}
 
 BatchPlan plan_batch(const ws_batch* b) {
     BatchPlan p{};
@@ -60,7 +84,7 @@ BatchPlan plan_batch(const ws_batch* b) {
     const bool vec_rows = b->vocab % 8u == 0 && (b->row_stride * esz) % 16u == 0 && reinterpret_cast<uintptr_t>(b->logits) % 16u == 0;
     const uint64_t fused_total = 65536u + maps + cap * 8u;
     // (a token's bias entries are counted in 11 bits of its rank word)
-    const bool can_fuse = vec_rows && b->vocab <= 163840u && fused_total + 4096u <= kMaxLds && (!b->bias_ids || b->max_bias <= 2047u);
+    const bool can_fuse = vec_rows && b->vocab <= 163840u && fused_total + kStaticLds <= kMaxLds && (!b->bias_ids || b->max_bias <= 2047u);
     if (b->mode == WS_MODE_FUSED && !can_fuse) return p;
     p.fused = b->mode != WS_MODE_EXACT && can_fuse;
     uint64_t ab, total;
@@ -73,21 +97,36 @@ BatchPlan plan_batch(const ws_batch* b) {
         total = ab + maps;
         p.lds_cnt = 0;
     }
-    if (total + 4096u > kMaxLds) return p;  // history + bias too long for the LDS rank tables
+    if (total + kStaticLds > kMaxLds) return p;  // history + bias too long for the LDS rank tables
     // spare room, when there is any, for a second copy of the histogram during the single sweep (odd lanes add there,
     // which halves the collisions of a wave's atomics on a crowded bin) and later for the tie bitmap of the sort
     // (vocab / 32 words + 16-bit prefixes)
     const uint64_t tie_bytes = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
     const uint64_t spare_bytes = tie_bytes > 32768u ? tie_bytes : 32768u;
     p.lds_tie = 0;
-    if (total + spare_bytes + 4096u <= kMaxLds) {
+    if (total + spare_bytes + kStaticLds <= kMaxLds) {
         p.lds_tie = static_cast<uint32_t>((total + 15u) & ~uint64_t{15});
         total = p.lds_tie + spare_bytes;
     }
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
-    p.workspace = 0;  // every intermediate lives in LDS
+    // Small batches of the single-sweep kernel: with rows to spare on the compute units a row is split over 2, 4, 8 or
+    // 16 workgroups (each at least 16384 tokens), which meet in global memory. All parts of all rows have to be running
+    // at the same time - they wait for each other - so rows * parts stays within the compute units of the device.
+    p.split_log2 = 0;
+    p.workspace = 0;
+    if (p.fused && b->max_split != 1u) {
+        const uint32_t cus = static_cast<uint32_t>(compute_units());
+        const uint32_t most = b->max_split ? b->max_split : 16u;
+        uint32_t lg = 0;
+        while (lg < 4u && (2u << lg) <= most && b->rows * (2u << lg) <= cus && b->vocab / (2u << lg) >= 16384u) ++lg;
+        // Meeting in global memory costs two round trips of some ten thousand clocks; measured on batches of 151936-token
+        // rows, eight parts and more win that back, four and fewer do not. A caller that names a number gets it.
+        if (!b->max_split && lg < 3u) lg = 0;
+        p.split_log2 = lg;
+        if (lg) p.workspace = uint64_t{b->rows} * ws::kSplitRowBytes;
+    }
     p.err = WS_OK;
     return p;
 }
@@ -198,8 +237,10 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b) {
 int ws_sample_batch(void* stream, const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     if (p.err != WS_OK) return p.err;
-    if (p.workspace && (!b->workspace || b->workspace_bytes < p.workspace)) return WS_E_WORKSPACE;
+    const bool can_split = p.workspace && b->workspace && b->workspace_bytes >= p.workspace && reinterpret_cast<uintptr_t>(b->workspace) % 8u == 0;
     ws::BatchArgs a{};
+    a.split_log2 = can_split ? p.split_log2 : 0u;
+    a.work = static_cast<unsigned char*>(b->workspace);
     a.logits = b->logits;
     a.dtype = b->dtype;
     a.rows = b->rows;
@@ -242,13 +283,17 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     a.query = b->query;
     a.query_prob = b->query_prob;
     a.entropy = b->entropy;
-    if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - 4096u);
-    static bool attr_set = false;  // raising the dynamic LDS limit is per function, once per process
-    if (!attr_set) {
+    if (p.fused && a.split_log2) return ws::launch_split(S(stream), a, b->rows << a.split_log2, p.lds_total, kMaxLds - kStaticLds);
+    if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);
+    static std::atomic<uint64_t> attr_set{0};  // the dynamic LDS limit is raised per function and device, once per process
+    int dev = 0;
+    if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_set.load(std::memory_order_acquire) & bit)) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - 4096u));
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - kStaticLds));
         if (e != hipSuccess) return static_cast<int>(e);
-        attr_set = true;
+        attr_set.fetch_or(bit, std::memory_order_release);
     }
     hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
     return done();

@@ -89,7 +89,15 @@ struct BatchArgs {
     const int32_t* query;      // per row or nullptr: a token whose probability is asked for (< 0: none)
     double* query_prob;        // out per row or nullptr
     double* entropy;           // out per row or nullptr: entropy of the kept set
+    uint32_t split_log2;       // single-sweep kernel: a row is worked on by 2^split_log2 workgroups (0: one), block = row * parts + part
+    unsigned char* work;       // split rows: kSplitRowBytes of zero-filled global memory per row, left zero-filled
 };
+
+// Global memory of a split row: the merged histogram, the merged candidate list, and four control words (parts that
+// have merged their histogram, parts that are done with the shared state, candidates listed, the row maximum as an
+// ordered integer).
+constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kSplitRowBytes = 65536u + 256u;
+constexpr uint32_t kSplitTimeout = 256u;  // flag: the parts of a row did not all turn up
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
 // replayed from LDS, where phase 0 left their adjusted logits by rank.
@@ -240,10 +248,10 @@ constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 
 
 // Provisional anchor: the larger of `floor` and the maximum of the thread block's first batch of loads, plus 8 exponent
 // units of headroom; the same registers then feed the sweep. Returns false (nothing binned) when that is not finite.
-template <int PER, bool MASKED, bool TOUCHED>
+template <int PER, bool MASKED, bool TOUCHED, bool SLICE>  // SLICE: rv is a slice of a split row, far shorter than the register cache
 __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
                                                 uint64_t* hist2, uint32_t (&cache)[kCacheRegs], float* red, uint4* stage,
-                                                uint32_t stage_cap, float& anchor, float& aq, float& m) {
+                                                uint32_t stage_cap, float& anchor, float& aq, float& m, float given_s, uint32_t rank0) {
     constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
     constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
@@ -282,13 +290,19 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
             }
         }
         s = block_max(s, red);  // its barriers also publish the zeroed histogram
+        if (given_s == given_s) s = given_s;  // a slice of a split row: the bound every part derives from the head of the row
         anchor = s + 8.f / inv_t;
         aq = anchor_product(anchor, c64);
         if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
     }
+    if (SLICE) {
+#pragma unroll
+        for (int k = 0; k < kCacheRegs; ++k) cache[k] = 0x0fff0fffu;  // registers past the slice: tail bin, never gathered
+    }
 #pragma unroll
     for (int bt = 0; bt < NB; ++bt) {
         const int slot = bt % kRing;
+        if (SLICE && static_cast<uint32_t>(bt * kBatch) * WS_BLOCK >= nv) break;  // uniform: the slice is done
         if (bt + 2 < NB) load(bt + 2, (bt + 2) % kRing);
         // The touched words of the whole batch are read before its first histogram update: LDS operations of a wave
         // complete in order, so a read placed behind the updates would make the wave wait for all of them.
@@ -331,7 +345,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
                     // when the touched ones are collected
                     const uint32_t sh = (j * PER) & 31u, tw = tws[u];
                     if ((tw >> sh) & (PER == 4 ? 15u : 255u)) {
-                        const uint32_t r = wps[u] + __popc(tw & ((1u << sh) - 1u));
+                        const uint32_t r = wps[u] + __popc(tw & ((1u << sh) - 1u)) - rank0;
                         stage[min(r, stage_cap)] = q[slot][u];  // slot stage_cap itself is a dump nobody reads
                     } else {
                         m = fmaxf(m, vm);
@@ -348,10 +362,12 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     return true;
 }
 
+template <bool SLICE>
 __device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist, uint64_t* hist2,
                                            uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap, float& anchor,
-                                           float& aq, float& m) {
-#define WS_FUSED_CALL(PER, AL, TC) fused_pass_impl<PER, AL, TC>(rv, floor_v, inv_t, c64, hist, hist2, cache, red, stage, stage_cap, anchor, aq, m)
+                                           float& aq, float& m, float given_s, uint32_t rank0) {
+#define WS_FUSED_CALL(PER, AL, TC) \
+    fused_pass_impl<PER, AL, TC, SLICE>(rv, floor_v, inv_t, c64, hist, hist2, cache, red, stage, stage_cap, anchor, aq, m, given_s, rank0)
     if (rv.dtype == 0) {
         if (rv.touched) return rv.allow ? WS_FUSED_CALL(4, true, true) : WS_FUSED_CALL(4, false, true);
         return rv.allow ? WS_FUSED_CALL(4, true, false) : WS_FUSED_CALL(4, false, false);
@@ -420,14 +436,16 @@ __device__ __forceinline__ float logit_of_bits(const RowView& rv, uint32_t bits)
 
 template <int MODE, int DTYPE>  // the row's type is a template argument: a branch on it around a load makes the compiler wait for the loads before
 __device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t a0, uint32_t a1, uint32_t a2,
-                                                uint32_t a3, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
+                                                uint32_t a3, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0,
+                                                int n_groups) {
+    // token indices count from the start of rv (a slice of a split row starts at token id0 of the row: list entries carry row indices)
     auto token_of = [&](int g, uint32_t bit) { return cache_token(DTYPE, g * 16u + 2u * (bit & 7u) + (bit >> 4), (bit >> 3) & 1u); };
     auto load_bits = [&](uint32_t i) {
         return DTYPE == 0 ? static_cast<const uint32_t*>(rv.base)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]);
     };
 #pragma unroll
     for (int g = 0; g < kCacheGroups; ++g) {
-        uint32_t h = cache_group_flags<MODE>(cache, g, a0, a1, a2, a3);
+        uint32_t h = g < n_groups ? cache_group_flags<MODE>(cache, g, a0, a1, a2, a3) : 0u;  // uniform: registers past a slice hold no token
         // every load has a register of its own that nothing else writes: a copy of a register with a load on the way
         // would have to wait for it
         hits.idx[g] = hits.idx[kCacheGroups + g] = 0xffffffffu;
@@ -448,38 +466,38 @@ __device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_
             const uint32_t i = token_of(g, static_cast<uint32_t>(__ffs(h)) - 1u);
             h &= h - 1u;
             const uint32_t slot = atomicAdd(n_list, 1u);
-            if (slot < cap) list[slot] = make_uint2(i | 0x80000000u, 0u);
+            if (slot < cap) list[slot] = make_uint2((i + id0) | 0x80000000u, 0u);
         }
     }
 }
 
 template <int DTYPE>
 __device__ __forceinline__ void scan_cache_typed(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
-                                                 uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
+                                                 uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
     const bool two = u1 <= 0x7fffu;
     auto at_least = [](uint32_t c) { return 0x80008000u - c * 0x10001u; };  // y + this: bit 15 of a half = (bin >= c)
     auto both = [](uint32_t c) { return c * 0x10001u; };
     const uint32_t n_single = (w0 + 1u) + (two ? w1 + 1u : 0u);  // bins asked for
     if (!two && u0 == 0u) {
-        scan_cache_impl<0, DTYPE>(rv, cache, at_least(w0 + 1u), 0u, 0u, 0u, hits, list, n_list, cap);
+        scan_cache_impl<0, DTYPE>(rv, cache, at_least(w0 + 1u), 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
     } else if (n_single <= 3u) {
         uint32_t c[3];
         uint32_t k = 0;
         for (uint32_t b = u0; b <= u0 + w0; ++b) c[k++] = both(b);
         if (two)
             for (uint32_t b = u1; b <= u1 + w1; ++b) c[k++] = both(b);
-        if (k == 1u) scan_cache_impl<1, DTYPE>(rv, cache, c[0], 0u, 0u, 0u, hits, list, n_list, cap);
-        else if (k == 2u) scan_cache_impl<2, DTYPE>(rv, cache, c[0], c[1], 0u, 0u, hits, list, n_list, cap);
-        else scan_cache_impl<3, DTYPE>(rv, cache, c[0], c[1], c[2], 0u, hits, list, n_list, cap);
+        if (k == 1u) scan_cache_impl<1, DTYPE>(rv, cache, c[0], 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
+        else if (k == 2u) scan_cache_impl<2, DTYPE>(rv, cache, c[0], c[1], 0u, 0u, hits, list, n_list, cap, id0, n_groups);
+        else scan_cache_impl<3, DTYPE>(rv, cache, c[0], c[1], c[2], 0u, hits, list, n_list, cap, id0, n_groups);
     } else {
         scan_cache_impl<4, DTYPE>(rv, cache, at_least(u0), at_least(u0 + w0 + 1u), at_least(two ? u1 : 0u), at_least(two ? u1 + w1 + 1u : 0u),
-                                  hits, list, n_list, cap);
+                                  hits, list, n_list, cap, id0, n_groups);
     }
 }
 __device__ __forceinline__ void scan_cache(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
-                                           uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap) {
-    if (rv.dtype == 0) scan_cache_typed<0>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap);
-    else scan_cache_typed<1>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap);
+                                           uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
+    if (rv.dtype == 0) scan_cache_typed<0>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
+    else scan_cache_typed<1>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
 }
 
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
@@ -902,7 +920,7 @@ __device__ __noinline__ ExactOut exact_row(const ExactIn in) {
     } while (0)
 #endif
 
-template <bool FUSED>
+template <bool FUSED, bool SPLIT = false>  // SPLIT: rows split over several workgroups (a build of its own: the unsplit kernel carries none of it)
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #ifdef WS_PHASE_TIMERS
     __shared__ long long ws_marks[64];
@@ -924,7 +942,10 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     uint32_t* tot_c = reinterpret_cast<uint32_t*>(s_pool + 160);
     __shared__ uint32_t s_u[8];
 
-    const uint32_t row = blockIdx.x;
+    // a row may be split over several workgroups (small batches of the single-sweep kernel): block = row * parts + part
+    const uint32_t n_parts = FUSED && SPLIT ? 1u << A.split_log2 : 1u;
+    const uint32_t row = FUSED && SPLIT ? blockIdx.x >> A.split_log2 : blockIdx.x, part = FUSED && SPLIT ? blockIdx.x & (n_parts - 1u) : 0u;
+    bool split = FUSED && SPLIT && n_parts > 1u;  // off again when this part goes on alone
     const uint32_t t = threadIdx.x;
     const uint32_t V = A.vocab;
     const uint32_t nW = (V + 31u) >> 5;
@@ -1066,6 +1087,41 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         __syncthreads();
         n_touched = n_uniq;
     }
+    // The part's slice of the row: tokens [id0, id0 + rvs.V), whole 256-token blocks; the touched tokens in it have the
+    // ranks [rank0, rank1). An unsplit row: all of it.
+    RowView rvs = rv;
+    uint32_t id0 = 0u, rank0 = 0u, rank1 = n_touched;
+    if (split) {
+        const uint32_t per_part = ((V + n_parts - 1u) / n_parts + 255u) & ~255u;
+        id0 = min(part * per_part, V);
+        rvs.V = min(per_part, V - id0);
+        rvs.base = static_cast<const unsigned char*>(rv.base) + static_cast<size_t>(id0) * esz;
+        if (rv.allow) rvs.allow = rv.allow + (id0 >> 5);
+        if (rv.touched) {
+            rvs.touched = rv.touched + (id0 >> 5);
+            rvs.wprefix = rv.wprefix + (id0 >> 5);
+            rank0 = wprefix[id0 >> 5];
+            rank1 = id0 + rvs.V < V ? wprefix[(id0 + rvs.V) >> 5] : n_touched;
+        }
+    }
+    unsigned char* work = split ? A.work + static_cast<size_t>(row) * kSplitRowBytes : nullptr;
+    uint32_t* ctrl = reinterpret_cast<uint32_t*>(work + kSplitCtrl);
+    __shared__ uint32_t s_prev;
+    // done with the row's shared memory: true for the part that says so last, which then has to clean it
+    auto leave_shared = [&]() {
+        __syncthreads();
+        if (t == 0) {
+            __threadfence();
+            s_prev = __hip_atomic_fetch_add(&ctrl[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        return s_prev == n_parts - 1u;
+    };
+    auto clean_shared = [&]() {  // zero again, for the next launch
+        uint64_t* gh = reinterpret_cast<uint64_t*>(work + kSplitHist);
+        for (uint32_t b = t; b < kBins; b += WS_BLOCK) gh[b] = 0ull;
+        if (t < 4u) ctrl[t] = 0u;
+    };
     const float* praw = reinterpret_cast<const float*>(lds + A.lds_cnt);           // raw logits of the touched tokens, by rank
     const uint32_t* pid = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt) + A.patch_cap;  // their token ids
     // Raw logit of every touched token as the sweeps see it (NaN and masked-out -> -inf), one 4-byte gather per history
@@ -1205,7 +1261,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // the sweep's histogram stands (move), takes the token out of the bin of its raw logit and puts it into the bin of the
     // adjusted one. ma / mu: the thread's largest adjusted logit, and its largest untouched, allowed logit among the
     // vectors that hold touched tokens (the sweep's running maximum leaves those vectors out).
-    auto collect_fused = [&](const uint4* stage, uint32_t stage_cap, bool move, float aq_, float c64_, float& ma, float& mu) {
+    auto collect_fused = [&](const uint4* stage, uint32_t stage_cap, bool move, float aq_, float c64_, float& ma, float& mu, uint32_t lo,
+                             uint32_t hi, uint32_t stage_rank0) {  // lo, hi: only the touched tokens in [lo, hi)
         ma = mu = -INFINITY;
         if (!n_touched) return;
         constexpr uint32_t kClaim = 0x80000000u;
@@ -1218,14 +1275,21 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const uint32_t whole_end = rv.vec ? (V & ~(per - 1u)) : 0u;  // tokens below this sit in whole 128-bit vectors
         const float tail_own = own_tail();
         auto take4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {  // four entries per thread and round, step by step side by side
+            uint32_t ahead[4];  // the ids of the round to come: requested a round early
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t j = k * WS_BLOCK + t;
+                ahead[k] = in_regs ? hid[k] : (j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu);  // kHid = 4: the first round is in registers
+            }
             for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
                 uint32_t id[4], al[4], tw[4], wp[4], rk[4], old[4];
                 uint4 vec[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const uint32_t j = j0 + k * WS_BLOCK + t;
-                    if (in_regs && j0 == 0) id[k] = hid[k];  // kHid = 4: the first round is in registers
-                    else id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
+                    id[k] = ahead[k];
+                    const uint32_t j = j0 + (4u + k) * WS_BLOCK + t;
+                    ahead[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;
+                    if (id[k] - lo >= hi - lo) id[k] = 0xffffffffu;  // another part's token (or none)
                 }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -1238,7 +1302,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
                     const uint32_t vb = i & ~(per - 1u);
-                    const uint32_t rf = wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u));  // rank of the vector's first touched token
+                    // place of the vector's first touched token in the staging room; an entry that is nobody's reads the first place
+                    // (nothing is done with it: a read of global memory would be waited for)
+                    const uint32_t rf = id[k] < V ? wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u)) - stage_rank0 : 0u;
                     rk[k] = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));                // rank_of(rv, i)
                     old[k] = id[k] < V ? atomicOr(&cnt[rk[k]], kClaim) : kClaim;
                     if (i < whole_end) {
@@ -1306,7 +1372,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // in the three-pass kernel that LDS is the histogram's, so it walks the set bits of the bitmap instead.
     auto replay_touched = [&](auto&& f) {
         if (FUSED) {
-            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) f(pid[r], pv[r]);
+            const uint32_t r_end = split ? rank1 : n_touched;
+            for (uint32_t r = (split ? rank0 : 0u) + t; r < r_end; r += WS_BLOCK) f(pid[r], pv[r]);
         } else if (n_touched) {
             const uint32_t chunk = (nW + WS_BLOCK - 1) / WS_BLOCK;
             const uint32_t w0 = t * chunk, w1 = min(w0 + chunk, nW);
@@ -1342,23 +1409,82 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         // staging room for the vectors that hold touched tokens: the LDS of the candidate masses, idle until pass 3
         uint4* stage = reinterpret_cast<uint4*>(emass);
         const uint32_t stage_cap = rv.vec ? 2047u : 0u;  // the region's last slot takes the vectors of the ranks beyond
-        if constexpr (FUSED) swept = fused_pass(rv, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m);
+        float given_s = __uint_as_float(0x7fc00000u);  // NaN: none
+        if (split) {
+            // the provisional bound has to be the same in every part: all take it from the head of the row, the loads an
+            // unsplit row starts with
+            const uint4* xv = static_cast<const uint4*>(rv.base);
+            const uint32_t nv = V >> (rv.dtype == 0 ? 2 : 3);
+            float s0 = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint4 q = xv[min(u * WS_BLOCK + t, nv - 1u)];
+                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (rv.dtype == 0) s0 = fmaxf(s0, __uint_as_float(w[e]));
+                    else s0 = fmaxf(s0, fmaxf(__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)));
+                }
+            }
+            given_s = block_max(s0, red_f);
+            if (given_s != given_s) given_s = INFINITY;  // a NaN at the head: no bound, as for an unsplit row
+        }
+        if constexpr (FUSED) swept = fused_pass<SPLIT>(rvs, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m, given_s, rank0);
         __syncthreads();
         WS_MARK(8);
+        auto all_adjusted = [&]() {  // this part goes on alone: the touched tokens of the other slices, then the largest adjusted logit
+            float ma, mu;
+            collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
+            __syncthreads();
+            float mx = -INFINITY;
+            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) mx = fmaxf(mx, pv[r]);
+            m_adj = block_max(mx, red_f);
+        };
         {
             float ma, mu;
-            collect_fused(stage, swept ? stage_cap : 0u, swept, aq, c64, ma, mu);
+            collect_fused(stage, swept ? stage_cap : 0u, swept, aq, c64, ma, mu, id0, id0 + rvs.V, rank0);
             WS_MARK(9);
             // m: over the vectors of the row that hold no touched token (allow mask applied); mu: the untouched tokens of
             // the others; ma: the adjusted tokens. The barriers of the reduction also end the moves in the histogram.
             float m_all = fmaxf(fmaxf(m, mu), ma);
             block_max2(m_all, ma, red_f, reinterpret_cast<float*>(red_u));
             m_adj = ma;
+            if (split && swept) {
+                // ---- the parts' histograms and maxima meet in global memory; every part takes the sums back
+                uint64_t* gh = reinterpret_cast<uint64_t*>(work + kSplitHist);
+                for (uint32_t b = t; b < kBins; b += WS_BLOCK) {
+                    const uint64_t h = hist[b] + (hist2 ? hist2[b] : 0ull);
+                    if (h) __hip_atomic_fetch_add(&gh[b], h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (t == 0) __hip_atomic_fetch_max(&ctrl[3], key32(m_all), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();  // every thread's additions are on their way; thread 0 publishes them (one fence for the block)
+                if (t == 0) {
+                    __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                    uint32_t spins = 0;
+                    while (__hip_atomic_load(&ctrl[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < n_parts && ++spins < (1u << 21)) __builtin_amdgcn_s_sleep(1);
+                    s_prev = spins < (1u << 21) ? 1u : 0u;
+                }
+                __syncthreads();
+                if (!s_prev) flags |= kSplitTimeout;  // uniform
+                // (the merged values are read with loads of device scope: no stale copy in this unit's caches is used)
+                m_all = unkey32(__hip_atomic_load(&ctrl[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = __hip_atomic_load(&gh[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                hist2 = nullptr;  // one copy from here
+                __syncthreads();
+            }
             if (swept) {
                 m = m_all;
                 // the sweep stands if no token beat the anchor and the anchor is not wastefully high (a masked outlier)
                 cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
             }
+        }
+        if (split && (!cached || (flags & kSplitTimeout) || !(m > -INFINITY))) {
+            // A row the sweep's bound does not fit (or that has no token at all, or whose parts did not meet): part 0 goes on
+            // alone, as for an unsplit row; the others are done.
+            if (swept && leave_shared()) clean_shared();
+            if (part != 0u) return;
+            split = false;
+            all_adjusted();
         }
         if (!cached) {
             m = -INFINITY;
@@ -1401,8 +1527,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
-    if (flags) {  // uniform over the block
-        if (t == 0) {
+    if (flags) {  // uniform over the block (and over the parts of a split row)
+        if (t == 0 && (part == 0u || !split)) {
             A.token[row] = -1;
             A.flags[row] = flags;
             if (A.prob) A.prob[row] = 0.f;
@@ -1686,6 +1812,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     double Zk_out = 0.0;  // mass of the kept set (the row's float normaliser on an open row)
     bool finished = false;
     bool finished_lean = false;
+    if (split && (flags & kOverflow)) {  // uniform over the parts (the merged histogram says so): part 0 takes the row through the exact path
+        if (leave_shared()) clean_shared();
+        if (part != 0u) return;
+        split = false;
+        float ma, mu;
+        collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
+        __syncthreads();
+    }
     // ------------------------------------------------------------------ pass 3: gather, sort, exact masses
     // (a row whose ranges hold more candidates than the list skips all of this and takes the exact path further down)
     if (!(flags & kOverflow)) {  // uniform
@@ -1734,7 +1868,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
                 {
                     CacheHits hits;
-                    scan_cache(rv, cache, u0, w0, u1r, w1, hits, list, &s_u[4], kCap);
+                    // a group of 16 registers holds 16384 consecutive tokens of the block; a slice fills only the first few
+                    const int n_groups = split ? static_cast<int>((rvs.V + 16383u) >> 14) : kCacheGroups;
+                    scan_cache(rvs, cache, u0, w0, u1r, w1, hits, list, &s_u[4], kCap, id0, n_groups);
                     WS_MARK(10);
                     // touched tokens whose adjusted logit lies in the ranges, while the last loads of the scan travel
                     replay_touched([&](uint32_t i, float x) {
@@ -1753,15 +1889,45 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 #pragma unroll
                     for (int g = 0; g < kHitSlots; ++g) {
                         if (hits.idx[g] == 0xffffffffu) continue;
-                        if (slot < kCap) list[slot] = make_uint2(hits.idx[g], hits.bits[g]);
+                        if (slot < kCap) list[slot] = make_uint2(hits.idx[g] + id0, hits.bits[g]);
                         ++slot;
                     }
                 }
                 WS_MARK(40);
                 __syncthreads();
                 WS_MARK(41);
-                const uint32_t n_hit = min(s_u[4], kCap);
+                uint32_t n_hit = min(s_u[4], kCap);
                 if (s_u[4] > kCap) flags |= kOverflow;
+                if (split) {
+                    // ---- the parts' candidates meet in global memory; the part that brings the last ones finishes the row
+                    uint2* glist = reinterpret_cast<uint2*>(work + kSplitList);
+                    __syncthreads();  // every thread has its n_hit
+                    if (t == 0) s_prev = __hip_atomic_fetch_add(&ctrl[2], s_u[4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __syncthreads();
+                    const uint32_t gbase = s_prev;
+                    for (uint32_t k = t; k < n_hit; k += WS_BLOCK)
+                        if (gbase + k < kCap) {
+                            const uint2 en = list[k];
+                            __hip_atomic_store(reinterpret_cast<uint64_t*>(&glist[gbase + k]), (static_cast<uint64_t>(en.y) << 32) | en.x, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                        }
+                    if (!leave_shared()) return;
+                    const uint32_t total = __hip_atomic_load(&ctrl[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    flags &= ~kOverflow;
+                    if (total > kCap) flags |= kOverflow;
+                    n_hit = min(total, kCap);
+                    for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
+                        const uint64_t en = __hip_atomic_load(reinterpret_cast<uint64_t*>(&glist[k]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        list[k] = make_uint2(static_cast<uint32_t>(en), static_cast<uint32_t>(en >> 32));
+                    }
+                    clean_shared();
+                    split = false;  // the row is this part's from here
+                    if (A.kept_ids || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
+                        float ma, mu;
+                        collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
+                    }
+                    __syncthreads();
+                }
                 // one entry of the list: is it kept, and its logit
                 auto entry = [&](uint2 en, bool live, uint32_t& id, float& x) {
                     id = en.x & kIdMask;
@@ -2287,7 +2453,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (!finished && !(flags & kOverflow)) {  // uniform: the sort-based finish
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
-        float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
+        float* dbg = A.kept_logits + static_cast<size_t>(row) * A.kept_cap;
         dbg[11] = static_cast<float>(n_r0);
         dbg[12] = static_cast<float>(n_r1);
         dbg[13] = static_cast<float>(r0hi - r0lo + 1);
@@ -2969,7 +3135,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     WS_MARK(7);
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
-        float* dbg = A.kept_logits + static_cast<size_t>(blockIdx.x) * A.kept_cap;
+        float* dbg = A.kept_logits + static_cast<size_t>(row) * A.kept_cap;
         for (uint32_t k = 0; k < 64u && k < A.kept_cap; ++k)
             if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
     }

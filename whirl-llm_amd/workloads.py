@@ -143,11 +143,11 @@ def upload(c, device="cuda:0"):
     return d
 
 
-def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0):
+def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0, **more):
     m = _pkg()
     return m.BatchSampler(d["logits"], d["inv_t"], d["seed"], d["step"], top_k=d["top_k"], top_p=d["top_p"], min_p=d["min_p"],
                           rng=rng_mode, hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
                           bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], max_hist=d["max_hist"],
-                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"))
+                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"), **more)
 
 
