@@ -31,7 +31,8 @@ enum {
     WS_E_INVALID = -1,     /* null pointer, zero / oversized dimension, unknown enum value */
     WS_E_WORKSPACE = -2,   /* workspace missing or smaller than ws_*_workspace() reports */
     WS_E_UNSUPPORTED = -3, /* a combination this build does not implement */
-    WS_E_NO_DEVICE = -4    /* no HIP device / the code object does not load on it */
+    WS_E_NO_DEVICE = -4,   /* no HIP device / the code object does not load on it */
+    WS_E_STATIC_LIMIT = -5 /* ws_sample_batch_static: the batch would split more rows than the library's own workspace holds */
 };
 
 /* Most rows one launch of the by-value-table kernels takes (kMaxVerifyRows, include/whirl/kernels_abi.h:359-365). */
@@ -228,6 +229,16 @@ typedef struct ws_batch {
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
 uint64_t ws_sample_batch_workspace(const ws_batch* b);
 int ws_sample_batch(void* stream, const ws_batch* b);
+/* ws_sample_batch for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it; it has no counterpart in the reference. The split rows of a small batch meet in memory that is
+ * part of the library's code object on every GPU (WS_STATIC_SPLIT_ROWS rows of it, about 2 MiB, held until the process
+ * ends) instead of b->workspace, which is ignored. Nothing is allocated or freed, here or in the kernels. A batch that
+ * would split more than WS_STATIC_SPLIT_ROWS rows (only with max_split 2 or 4: the library's own choice splits at most
+ * 32) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is looked up on the first call there (or by
+ * ws_probe): make that call before capturing a graph. All calls on one GPU share this memory: two of them that run at the
+ * same time (different streams) race; on one stream they are safe, each launch leaves the memory as the next needs it. */
+#define WS_STATIC_SPLIT_ROWS 32
+int ws_sample_batch_static(void* stream, const ws_batch* b);
 
 /* Penalised fp32 copy of logits rows: out[row][i] = the logit ws_sample_batch samples from (allow mask and NaN -> -inf,
  * bias, repetition, frequency / presence; same fields and meaning as in ws_batch). No counterpart in the reference, which

@@ -119,6 +119,7 @@ ABI = {
     "ws_dflash_topk": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
+    "ws_sample_batch_static": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
     "ws_accept_sampled": (C.c_int, [C.c_void_p, C.POINTER(Accept)]),
     "ws_accept_greedy": (C.c_int, [C.c_void_p, C.POINTER(AcceptGreedy)]),
@@ -391,6 +392,12 @@ class BatchSampler:
     def run(self, stream=None):
         s = _stream() if stream is None else C.c_void_p(stream)
         check(lib().ws_sample_batch(s, C.byref(self.desc)), "ws_sample_batch")
+        return self
+
+    def run_static(self, stream=None):
+        """The same launch over the library's own workspace (ws_sample_batch_static): nothing of this object's workspace is used."""
+        s = _stream() if stream is None else C.c_void_p(stream)
+        check(lib().ws_sample_batch_static(s, C.byref(self.desc)), "ws_sample_batch_static")
         return self
 
 

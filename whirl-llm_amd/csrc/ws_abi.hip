@@ -131,6 +131,28 @@ BatchPlan plan_batch(const ws_batch* b) {
     return p;
 }
 
+// Memory of the library's own for ws_sample_batch_static: the split rows' meeting place (kStaticRows rows of it), in every
+// GPU's copy of the code object, zero-filled when the code object is loaded and left zero-filled by every launch.
+constexpr uint32_t kStaticRows = 32;
+static __device__ __align__(256) unsigned char scratch[kStaticRows * ws::kSplitRowBytes];
+std::atomic<unsigned char*> scratch_at[64];  // per device: where its copy of `scratch` lies
+
+// the address of the current device's copy (asked for once per device; no allocation)
+int scratch_address(unsigned char** out) {
+    int dev = 0;
+    if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= 64) return WS_E_UNSUPPORTED;
+    unsigned char* at = scratch_at[dev].load(std::memory_order_acquire);
+    if (!at) {
+        void* sym = nullptr;
+        if (const hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)); e != hipSuccess) return static_cast<int>(e);
+        at = static_cast<unsigned char*>(sym);
+        scratch_at[dev].store(at, std::memory_order_release);
+    }
+    *out = at;
+    return WS_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -142,6 +164,7 @@ const char* ws_error_string(int code) {
     case WS_OK: return "ok";
     case WS_E_INVALID: return "invalid argument";
     case WS_E_WORKSPACE: return "workspace missing or too small";
+    case WS_E_STATIC_LIMIT: return "the batch would split more rows than the library's own workspace holds (32): use ws_sample_batch with a workspace, or max_split = 1";
     case WS_E_UNSUPPORTED: return "unsupported combination";
     case WS_E_NO_DEVICE: return "no usable HIP device";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
@@ -159,6 +182,8 @@ int ws_probe(void) {
         (void)hipGetLastError();
         return WS_E_NO_DEVICE;
     }
+    unsigned char* at = nullptr;  // the current device's copy of the static workspace: resolved here, outside any capture
+    if (const int e = scratch_address(&at); e != WS_OK) return e;
     return WS_OK;
 }
 
@@ -234,13 +259,13 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b) {
     return p.err == WS_OK ? p.workspace : 0;
 }
 
-int ws_sample_batch(void* stream, const ws_batch* b) {
-    const BatchPlan p = plan_batch(b);
-    if (p.err != WS_OK) return p.err;
-    const bool can_split = p.workspace && b->workspace && b->workspace_bytes >= p.workspace && reinterpret_cast<uintptr_t>(b->workspace) % 8u == 0;
+namespace {
+
+int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigned char* work, uint64_t work_bytes) {
+    const bool can_split = p.workspace && work && work_bytes >= p.workspace && reinterpret_cast<uintptr_t>(work) % 8u == 0;
     ws::BatchArgs a{};
     a.split_log2 = can_split ? p.split_log2 : 0u;
-    a.work = static_cast<unsigned char*>(b->workspace);
+    a.work = work;
     a.logits = b->logits;
     a.dtype = b->dtype;
     a.rows = b->rows;
@@ -297,6 +322,23 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
     }
     hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
     return done();
+}
+
+}  // namespace
+
+int ws_sample_batch(void* stream, const ws_batch* b) {
+    const BatchPlan p = plan_batch(b);
+    if (p.err != WS_OK) return p.err;
+    return sample_batch_on(stream, b, p, static_cast<unsigned char*>(b->workspace), b->workspace_bytes);
+}
+
+int ws_sample_batch_static(void* stream, const ws_batch* b) {
+    const BatchPlan p = plan_batch(b);
+    if (p.err != WS_OK) return p.err;
+    if (p.workspace > sizeof(scratch)) return WS_E_STATIC_LIMIT;  // more split rows than the library's own memory holds
+    unsigned char* at = nullptr;
+    if (const int e = scratch_address(&at); e != WS_OK) return e;
+    return sample_batch_on(stream, b, p, at, sizeof(scratch));
 }
 
 int ws_adjust_rows(void* stream, const ws_adjust* b) {
