@@ -47,7 +47,7 @@ def test_argmax_family(rows5):
     assert [got[10 + 3 * r] for r in range(rows)] == want and (got != -1).sum() == rows
     tok, prob = m.argmax_prob(dx[0])
     assert tok.item() == want[0]
-    assert abs(prob.item() - softmax_top(x[0])) <= 1e-4 * softmax_top(x[0]) + 1e-9
+    assert abs(prob.item() - softmax_top(x[0])) <= 2e-6 * softmax_top(x[0]) + 1e-12
 
 
 def test_argmax_odd_sizes_and_misaligned_rows():
@@ -79,7 +79,7 @@ def test_draft_pick_chain_and_rows(rows5):
     t, c, p = tok.cpu().numpy(), ctl.cpu().numpy(), prob.cpu().numpy()
     assert t[0] == 5 and t[1] == first_max(lg[1]) and t[2] == 0x7F7F7F7F and c[0] == 1 and c[1] == 1
     for r in range(2):
-        assert abs(p[r] - softmax_top(lg[r])) <= 1e-4 * softmax_top(lg[r]) + 1e-9
+        assert abs(p[r] - softmax_top(lg[r])) <= 2e-6 * softmax_top(lg[r]) + 1e-12
     ctl_all = torch.zeros(2 * m.CTL_WORDS, dtype=torch.int32, device=DEV)
     m.draft_pick_rows(dl[:2], ctl_all, [0, m.CTL_WORDS], 0, 1, 0.5)
     ca = ctl_all.cpu().numpy()
@@ -103,7 +103,7 @@ def test_draft_pick_chain_and_rows(rows5):
 
 @pytest.mark.parametrize("K", [1, 16, 40, 256, 16384])
 def test_topk_rows_against_oracle(rows5, K):
-    """Value multiset == partial sort, ids consistent with values, maximum exact, normaliser within 1e-4
+    """Value multiset == partial sort, ids consistent with values, maximum exact, normaliser within 2e-6
     (tests/kernels/test_misc.cpp:315-354); beyond that, the id SET equals the oracle's (value desc, id asc) top-K and
     entries come in ascending id order."""
     m = gpu_cases.pkg()
@@ -117,7 +117,7 @@ def test_topk_rows_against_oracle(rows5, K):
         lib.wo_topk_row(wo._ptr(np.ascontiguousarray(x[r])), x.shape[1], K, inv_t, wo._ptr(wi), wo._ptr(wv), wo._ptr(ws_))
         assert np.array_equal(ids[r], np.sort(wi))
         assert vals[r].tobytes() == x[r][ids[r]].tobytes()
-        assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1]
+        assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 2e-6 * ws_[1]
 
 
 def test_topk_rows_cold_temperature_and_crowded_stretch(rows5):
@@ -137,7 +137,7 @@ def test_topk_rows_cold_temperature_and_crowded_stretch(rows5):
             lib.wo_topk_row(wo._ptr(np.ascontiguousarray(x[r])), x.shape[1], K, np.float32(inv_t), wo._ptr(wi), wo._ptr(wv), wo._ptr(ws_))
             assert np.array_equal(ids[r], np.sort(wi)), (K, inv_t, r)
             assert vals[r].tobytes() == x[r][ids[r]].tobytes()
-            assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 1e-4 * ws_[1], (K, inv_t, r, stats[r], ws_)
+            assert stats[r, 0] == ws_[0] and abs(stats[r, 1] - ws_[1]) <= 2e-6 * ws_[1], (K, inv_t, r, stats[r], ws_)
 
 
 def test_topk_rows_seeded_sweep():

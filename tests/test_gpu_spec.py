@@ -1,7 +1,7 @@
 """GPU: speculative-sampling kernels through the C ABI against the oracle.
 
 draft_sample_rows in the idiom of the reference's kernel test (tests/kernels/test_misc.cpp:355-481): q support ids exact,
-q probabilities within 1e-4 relative of the host draft distribution, the drawn draft == the host race draw from the
+q probabilities within 1e-6 relative of the host draft distribution, the drawn draft == the host race draw from the
 written q, NaN logits never candidates. Classic accept / resample: accepted counts and every emitted token identical
 to the oracle's closed form."""
 import ctypes as C
@@ -15,6 +15,15 @@ import wo
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+
+
+Q_RTOL = 1e-6  # the bar of every probability here (the reference's own kernel test allows 1e-4); worst seen: 2.3e-7
+
+
+def _close(got, want):
+    a, b = np.array(got.p[:got.n], np.float64), np.array(want.p[:want.n], np.float64)
+    rel = np.abs(a - b) / np.maximum(b, 1e-30)
+    assert rel.size == 0 or rel.max() <= Q_RTOL, (rel.max(), a, b)
 
 
 def host_q(lib, x, inv_t, top_k, top_p, min_p):
@@ -52,14 +61,14 @@ def test_draft_sample_rows_support_probabilities_and_draw():
         got = wo.QDist()
         lib.wo_q_from_words(wo._ptr(np.ascontiguousarray(hq[b * m.Q_WORDS:(b + 1) * m.Q_WORDS])), C.byref(got))
         assert got.n == want.n and list(got.id[:got.n]) == list(want.id[:want.n])
-        np.testing.assert_allclose(np.array(got.p[:got.n]), np.array(want.p[:want.n]), rtol=1e-4, atol=1e-7)
+        _close(got, want)
         assert hc[b * 64 + 16 + r] == lib.wo_sample_race_q(C.byref(got), keys[b])
 
 
 def test_draft_sample_rows_seeded_sweep():
     """Random vocabulary sizes (down to fewer tokens than candidates), filters and temperatures, with logits rounded to
     a quarter so that many tie (ties: lowest id first, src/common/spec_sample.cpp:43-50): ids and count of q exact,
-    probabilities to 1e-4, the draw equal to the host race over the written q."""
+    probabilities to 1e-6, the draw equal to the host race over the written q."""
     m = gc.pkg()
     lib = wo.load("oracle")
     rng = np.random.default_rng(302)
@@ -85,7 +94,7 @@ def test_draft_sample_rows_seeded_sweep():
             got = wo.QDist()
             lib.wo_q_from_words(wo._ptr(np.ascontiguousarray(hq[b * m.Q_WORDS:(b + 1) * m.Q_WORDS])), C.byref(got))
             assert got.n == want.n and list(got.id[:got.n]) == list(want.id[:want.n]), (case, b, n, tks[b])
-            np.testing.assert_allclose(np.array(got.p[:got.n]), np.array(want.p[:want.n]), rtol=1e-4, atol=1e-7)
+            _close(got, want)
             assert hc[b * 64 + 16 + r] == lib.wo_sample_race_q(C.byref(got), keys[b]), (case, b)
 
 
@@ -115,7 +124,7 @@ def test_draft_sample_rows_nan_map_and_skips():
     lib.wo_q_from_words(wo._ptr(np.ascontiguousarray(hq[:m.Q_WORDS])), C.byref(got))
     assert got.n == want.n and [int(v) for v in got.id[:got.n]] == [int(vmap[i]) for i in want.id[:want.n]]
     assert all(np.isfinite(got.p[i]) for i in range(got.n)) and not set(got.id[:got.n]) & {int(vmap[i]) for i in nan_at}
-    np.testing.assert_allclose(np.array(got.p[:got.n]), np.array(want.p[:want.n]), rtol=1e-4, atol=1e-7)
+    _close(got, want)
     assert hc[16 + r] == lib.wo_sample_race_q(C.byref(got), key)
     assert hc[64 + 16 + r] == -5 and hq[m.Q_WORDS] == -1    # stopped chain: untouched
     assert hc[128 + 16 + r] == -5 and hq[2 * m.Q_WORDS] == -1  # on = 0: the greedy draft stays
