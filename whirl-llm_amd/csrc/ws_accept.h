@@ -101,6 +101,15 @@ __global__ void __launch_bounds__(64) accept_sampled_kernel(AcceptArgs A) {
     int32_t acc = 0;
     uint32_t st = 0, n_relaxed = 0;
     int32_t tok = -1;
+    if (text && n_hist + 2u + static_cast<uint32_t>(nd) > A.hist.cap) {
+        // no room for next and the drafts behind the text: the guard would read past the slot. The host takes the sequence.
+        if (threadIdx.x == 0) {
+            A.n_accepted[s] = 0;
+            A.chosen[s] = -1;
+            A.status[s] = kAcceptHistoryFull | kAcceptHost;
+        }
+        return;
+    }
     for (;;) {  // position acc: its token is the output; it is accepted when it is a draft position and equals the draft
         tok = A.token[r0 + acc];
         const uint32_t fl = A.flags[r0 + acc];
@@ -170,6 +179,14 @@ __global__ void __launch_bounds__(64) accept_greedy_kernel(AcceptGreedyArgs A) {
     int32_t acc = 0;
     uint32_t n_relaxed = 0;
     double gap = 0.0;
+    if (text && n_hist + 2u + static_cast<uint32_t>(nd) > A.hist.cap) {  // as in accept_sampled_kernel
+        if (threadIdx.x == 0) {
+            A.n_accepted[s] = 0;
+            A.chosen[s] = -1;
+            A.status[s] = kAcceptHistoryFull | kAcceptHost;
+        }
+        return;
+    }
     while (acc < nd) {
         const int32_t draft = c[16 + acc];
         if (c[acc] == draft) {

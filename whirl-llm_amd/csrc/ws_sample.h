@@ -556,7 +556,8 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
 
 // ---- the exact path. Rows whose candidate ranges hold more than the list - a top-k beyond its capacity, thousands of
 // candidates with one logit, a flat row whose draw bins alone overflow it - are answered here without any list. Every
-// token's mass is taken in fixed point (units of 2^-44 of the largest), so sums are integers and the same whatever the
+// token's mass is taken in fixed point (units of 2^-43 of the largest: a million tokens of the largest mass still add up
+// inside 64 bits), so sums are integers and the same whatever the
 // order; candidates are ordered by their 64-bit key (logit, then id), and each question - the key at a rank, the first
 // key at which the running mass reaches a value - is a radix walk over that key, twelve bits a level, one pass over the
 // row per level with a 4096-entry histogram of counts and masses in LDS. A few dozen passes over a row that sits in L2:
@@ -602,7 +603,7 @@ __device__ __noinline__ ExactOut exact_row(const ExactIn in) {
     rv.touched = in.touched_at != 0xffffffffu ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) : nullptr;
     rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u);
     rv.pv = reinterpret_cast<const float*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
-    constexpr double kFx = 17592186044416.0;  // 2^44
+    constexpr double kFx = 8796093022208.0;  // 2^43
     uint64_t* hm = reinterpret_cast<uint64_t*>(lds);          // masses per digit
     uint32_t* hc = reinterpret_cast<uint32_t*>(lds + 32768);  // counts per digit
     uint64_t* red_w = reinterpret_cast<uint64_t*>(x_red_q);
@@ -1109,11 +1110,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     __shared__ uint32_t s_prev;
     // done with the row's shared memory: true for the part that says so last, which then has to clean it
     auto leave_shared = [&]() {
+        // What this part left in the shared memory went out as device-scope atomics and stores (performed at the level all
+        // compute units see). Every wave waits until its own are acknowledged, then the barrier, then one thread counts
+        // the part in: no cache write-back is needed on the way.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (t == 0) {
-            __threadfence();
-            s_prev = __hip_atomic_fetch_add(&ctrl[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        if (t == 0) s_prev = __hip_atomic_fetch_add(&ctrl[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         return s_prev == n_parts - 1u;
     };
@@ -1452,14 +1454,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if (split && swept) {
                 // ---- the parts' histograms and maxima meet in global memory; every part takes the sums back
                 uint64_t* gh = reinterpret_cast<uint64_t*>(work + kSplitHist);
-                for (uint32_t b = t; b < kBins; b += WS_BLOCK) {
+#pragma unroll
+                for (uint32_t k = 0; k < kBins / WS_BLOCK; ++k) {
+                    const uint32_t b = k * WS_BLOCK + t;
                     const uint64_t h = hist[b] + (hist2 ? hist2[b] : 0ull);
                     if (h) __hip_atomic_fetch_add(&gh[b], h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 if (t == 0) __hip_atomic_fetch_max(&ctrl[3], key32(m_all), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();  // every thread's additions are on their way; thread 0 publishes them (one fence for the block)
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's additions are acknowledged (device-scope atomics: they are in memory)
+                __syncthreads();
                 if (t == 0) {
-                    __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     uint32_t spins = 0;
                     while (__hip_atomic_load(&ctrl[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < n_parts && ++spins < (1u << 21)) __builtin_amdgcn_s_sleep(1);
                     s_prev = spins < (1u << 21) ? 1u : 0u;
@@ -1468,7 +1473,14 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 if (!s_prev) flags |= kSplitTimeout;  // uniform
                 // (the merged values are read with loads of device scope: no stale copy in this unit's caches is used)
                 m_all = unkey32(__hip_atomic_load(&ctrl[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-                for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = __hip_atomic_load(&gh[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                {
+                    uint64_t merged[kBins / WS_BLOCK];  // all of a thread's loads on their way before the first is used
+#pragma unroll
+                    for (uint32_t k = 0; k < kBins / WS_BLOCK; ++k)
+                        merged[k] = __hip_atomic_load(&gh[k * WS_BLOCK + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (uint32_t k = 0; k < kBins / WS_BLOCK; ++k) hist[k * WS_BLOCK + t] = merged[k];
+                }
                 hist2 = nullptr;  // one copy from here
                 __syncthreads();
             }
