@@ -222,8 +222,8 @@ typedef struct ws_batch {
                                    256 candidates with their shares of the whole row), what the typical acceptance rule
                                    compares with (src/sampling/acceptor.cpp:77-84). See WS_FLAG_APPROX_ENTROPY. */
     uint32_t max_split;         /* most workgroups a row may be split over (a power of two up to 16, rows * parts within the
-                                   GPU's compute units, at least 16384 tokens a part): 0 = the library decides (8 or 16
-                                   parts when the batch is small enough for that, else none), 1 = never split */
+                                   GPU's compute units, at least 16384 tokens a part): 0 = the library decides (4, 8 or
+                                   16 parts when the batch is small enough for that, else none), 1 = never split */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
@@ -231,13 +231,14 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b);
 int ws_sample_batch(void* stream, const ws_batch* b);
 /* ws_sample_batch for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
  * harnesses that forbid it; it has no counterpart in the reference. The split rows of a small batch meet in memory that is
- * part of the library's code object on every GPU (WS_STATIC_SPLIT_ROWS rows of it, about 2 MiB, held until the process
- * ends) instead of b->workspace, which is ignored. Nothing is allocated or freed, here or in the kernels. A batch that
- * would split more than WS_STATIC_SPLIT_ROWS rows (only with max_split 2 or 4: the library's own choice splits at most
- * 32) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is looked up on the first call there (or by
- * ws_probe): make that call before capturing a graph. All calls on one GPU share this memory: two of them that run at the
- * same time (different streams) race; on one stream they are safe, each launch leaves the memory as the next needs it. */
-#define WS_STATIC_SPLIT_ROWS 32
+ * part of the library's code object on every GPU (WS_STATIC_SPLIT_ROWS rows of it, about 4 MiB, held until the process
+ * ends) instead of b->workspace, which is ignored. Nothing is allocated or freed, here or in the kernels. Every batch the
+ * library splits on its own fits (at most 64 rows are split); one that the caller's max_split would split into more rows
+ * than that (65 to 128 rows in two parts each) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is
+ * looked up on the first call there (or by ws_probe): make that call before capturing a graph. All calls on one GPU
+ * share this memory: two of them that run at the same time (different streams) race; on one stream they are safe, each
+ * launch leaves the memory as the next needs it. */
+#define WS_STATIC_SPLIT_ROWS 64
 int ws_sample_batch_static(void* stream, const ws_batch* b);
 
 /* Penalised fp32 copy of logits rows: out[row][i] = the logit ws_sample_batch samples from (allow mask and NaN -> -inf,

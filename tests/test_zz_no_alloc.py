@@ -35,7 +35,7 @@ def test_static_workspace_entry_point_matches_the_workspace_one_on_two_calls_in_
     ref, got = _both(small, 0)
     assert gc.compare_rows(small, got, range(3), 0)["exact"] == 3
     # a batch too large to split runs as ws_sample_batch does; one that would split more rows than fit is refused
-    wide = gc.make_cfg2(rows=40, V=32768, n_hist=64, n_bias=0)
+    wide = gc.make_cfg2(rows=80, V=32768, n_hist=64, n_bias=0)
     _both(wide, 1)
     d = gc.upload(wide)
     smp = gc.sampler_for(wide, d, 1, max_split=2)

@@ -121,9 +121,10 @@ BatchPlan plan_batch(const ws_batch* b) {
         const uint32_t most = b->max_split ? b->max_split : 16u;
         uint32_t lg = 0;
         while (lg < 4u && (2u << lg) <= most && b->rows * (2u << lg) <= cus && b->vocab / (2u << lg) >= 16384u) ++lg;
-        // Meeting in global memory costs two round trips of some ten thousand clocks; measured on batches of 151936-token
-        // rows, eight parts and more win that back, four and fewer do not. A caller that names a number gets it.
-        if (!b->max_split && lg < 3u) lg = 0;
+        // Meeting in global memory costs two round trips of several thousand clocks each; measured on batches of
+        // 151936-token rows, four parts and more win that back (64 rows: 49.5 against 52.9 us; 16 rows: 40 against 50),
+        // two do not. A caller that names a number gets it.
+        if (!b->max_split && lg < 2u) lg = 0;
         p.split_log2 = lg;
         if (lg) p.workspace = uint64_t{b->rows} * ws::kSplitRowBytes;
     }
@@ -133,7 +134,7 @@ BatchPlan plan_batch(const ws_batch* b) {
 
 // Memory of the library's own for ws_sample_batch_static: the split rows' meeting place (kStaticRows rows of it), in every
 // GPU's copy of the code object, zero-filled when the code object is loaded and left zero-filled by every launch.
-constexpr uint32_t kStaticRows = 32;
+constexpr uint32_t kStaticRows = 64;
 static __device__ __align__(256) unsigned char scratch[kStaticRows * ws::kSplitRowBytes];
 std::atomic<unsigned char*> scratch_at[64];  // per device: where its copy of `scratch` lies
 
@@ -164,7 +165,7 @@ const char* ws_error_string(int code) {
     case WS_OK: return "ok";
     case WS_E_INVALID: return "invalid argument";
     case WS_E_WORKSPACE: return "workspace missing or too small";
-    case WS_E_STATIC_LIMIT: return "the batch would split more rows than the library's own workspace holds (32): use ws_sample_batch with a workspace, or max_split = 1";
+    case WS_E_STATIC_LIMIT: return "the batch would split more rows than the library's own workspace holds (64): use ws_sample_batch with a workspace, or max_split = 1";
     case WS_E_UNSUPPORTED: return "unsupported combination";
     case WS_E_NO_DEVICE: return "no usable HIP device";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";

@@ -30,6 +30,9 @@
 
 namespace ws {
 
+// a uniform branch that rows rarely take: its code is laid out away from the straight path
+#define WS_RARE(x) __builtin_expect(!!(x), 0)
+#define WS_USUAL(x) __builtin_expect(!!(x), 1)
 constexpr int kBins = 4096;
 constexpr uint32_t kCap = 4096;          // candidates resolved exactly in LDS per gather
 constexpr int kPT = kBins / WS_BLOCK;    // histogram bins, and sorted candidates, owned by one thread
@@ -248,11 +251,11 @@ constexpr int kCacheRegs = 163840 / WS_BLOCK / 2;  // 80 with 1024 threads, 160 
 
 // Provisional anchor: the larger of `floor` and the maximum of the thread block's first batch of loads, plus 8 exponent
 // units of headroom; the same registers then feed the sweep. Returns false (nothing binned) when that is not finite.
-template <int PER, bool MASKED, bool TOUCHED, bool SLICE>  // SLICE: rv is a slice of a split row, far shorter than the register cache
+template <int PER, bool MASKED, bool TOUCHED, bool SLICE, int CR>  // SLICE: rv is a slice of a split row; CR: registers of the bin cache
 __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist,
-                                                uint64_t* hist2, uint32_t (&cache)[kCacheRegs], float* red, uint4* stage,
+                                                uint64_t* hist2, uint32_t (&cache)[CR], float* red, uint4* stage,
                                                 uint32_t stage_cap, float& anchor, float& aq, float& m, float given_s, uint32_t rank0) {
-    constexpr int NB = (2 * kCacheRegs) / (kBatch * PER);
+    constexpr int NB = (2 * CR) / (kBatch * PER);
     constexpr int kRing = 3;  // batches in flight: the loads of batch bt + 2 are issued before batch bt is consumed
     const uint32_t t = threadIdx.x;
     const uint32_t nv = rv.V / PER;
@@ -297,7 +300,7 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     }
     if (SLICE) {
 #pragma unroll
-        for (int k = 0; k < kCacheRegs; ++k) cache[k] = 0x0fff0fffu;  // registers past the slice: tail bin, never gathered
+        for (int k = 0; k < CR; ++k) cache[k] = 0x0fff0fffu;  // registers past the slice: tail bin, never gathered
     }
 #pragma unroll
     for (int bt = 0; bt < NB; ++bt) {
@@ -362,12 +365,12 @@ __device__ __forceinline__ bool fused_pass_impl(const RowView& rv, float floor_v
     return true;
 }
 
-template <bool SLICE>
+template <bool SLICE, int CR>
 __device__ __forceinline__ bool fused_pass(const RowView& rv, float floor_v, float inv_t, float c64, uint64_t* hist, uint64_t* hist2,
-                                           uint32_t (&cache)[kCacheRegs], float* red, uint4* stage, uint32_t stage_cap, float& anchor,
+                                           uint32_t (&cache)[CR], float* red, uint4* stage, uint32_t stage_cap, float& anchor,
                                            float& aq, float& m, float given_s, uint32_t rank0) {
 #define WS_FUSED_CALL(PER, AL, TC) \
-    fused_pass_impl<PER, AL, TC, SLICE>(rv, floor_v, inv_t, c64, hist, hist2, cache, red, stage, stage_cap, anchor, aq, m, given_s, rank0)
+    fused_pass_impl<PER, AL, TC, SLICE, CR>(rv, floor_v, inv_t, c64, hist, hist2, cache, red, stage, stage_cap, anchor, aq, m, given_s, rank0)
     if (rv.dtype == 0) {
         if (rv.touched) return rv.allow ? WS_FUSED_CALL(4, true, true) : WS_FUSED_CALL(4, false, true);
         return rv.allow ? WS_FUSED_CALL(4, true, false) : WS_FUSED_CALL(4, false, false);
@@ -397,15 +400,16 @@ __device__ __forceinline__ uint32_t cache_token(int dtype, uint32_t k, uint32_t 
 // from the register's place), so the loads travel while the scan goes on; so has its second hit in the group (a
 // handful per row). A third one and beyond goes to list[] as (token | bit 31, 0) (LDS, at most cap entries; *n_list,
 // zeroed by the caller before a barrier, counts them) and is fetched by the caller afterwards.
-constexpr int kCacheGroups = kCacheRegs / 16;
-constexpr int kHitSlots = 2 * kCacheGroups;  // two per group of registers: slots g and kCacheGroups + g
+template <int CR>
 struct CacheHits {
-    uint32_t idx[kHitSlots];   // token index, 0xffffffff = none
-    uint32_t bits[kHitSlots];  // its logit as loaded: fp32 bits, or the 16 bits of a bf16
+    static constexpr int kGroups = CR / 16;
+    static constexpr int kSlots = 2 * kGroups;  // two per group of registers: slots g and kGroups + g
+    uint32_t idx[kSlots];   // token index, 0xffffffff = none
+    uint32_t bits[kSlots];  // its logit as loaded: fp32 bits, or the 16 bits of a bf16
 };
 
-template <int MODE>  // 0: one range from bin 0; 1 / 2 / 3: so many single bins; 4: two ranges
-__device__ __forceinline__ uint32_t cache_group_flags(const uint32_t (&cache)[kCacheRegs], int g, uint32_t a0, uint32_t a1, uint32_t a2,
+template <int MODE, int CR>  // 0: one range from bin 0; 1 / 2 / 3: so many single bins; 4: two ranges
+__device__ __forceinline__ uint32_t cache_group_flags(const uint32_t (&cache)[CR], int g, uint32_t a0, uint32_t a1, uint32_t a2,
                                                       uint32_t a3) {
     uint32_t acc = 0;
 #pragma unroll
@@ -434,18 +438,19 @@ __device__ __forceinline__ float logit_of_bits(const RowView& rv, uint32_t bits)
     return fmaxf(__uint_as_float(rv.dtype == 0 ? bits : bits << 16), -INFINITY);  // NaN -> -inf
 }
 
-template <int MODE, int DTYPE>  // the row's type is a template argument: a branch on it around a load makes the compiler wait for the loads before
-__device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t a0, uint32_t a1, uint32_t a2,
-                                                uint32_t a3, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0,
+template <int MODE, int DTYPE, int CR>  // the row's type is a template argument: a branch on it around a load makes the compiler wait for the loads before
+__device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_t (&cache)[CR], uint32_t a0, uint32_t a1, uint32_t a2,
+                                                uint32_t a3, CacheHits<CR>& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0,
                                                 int n_groups) {
     // token indices count from the start of rv (a slice of a split row starts at token id0 of the row: list entries carry row indices)
     auto token_of = [&](int g, uint32_t bit) { return cache_token(DTYPE, g * 16u + 2u * (bit & 7u) + (bit >> 4), (bit >> 3) & 1u); };
     auto load_bits = [&](uint32_t i) {
         return DTYPE == 0 ? static_cast<const uint32_t*>(rv.base)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]);
     };
+    constexpr int kCacheGroups = CR / 16;
 #pragma unroll
     for (int g = 0; g < kCacheGroups; ++g) {
-        uint32_t h = g < n_groups ? cache_group_flags<MODE>(cache, g, a0, a1, a2, a3) : 0u;  // uniform: registers past a slice hold no token
+        uint32_t h = g < n_groups ? cache_group_flags<MODE, CR>(cache, g, a0, a1, a2, a3) : 0u;  // uniform: registers past a slice hold no token
         // every load has a register of its own that nothing else writes: a copy of a register with a load on the way
         // would have to wait for it
         hits.idx[g] = hits.idx[kCacheGroups + g] = 0xffffffffu;
@@ -471,33 +476,34 @@ __device__ __forceinline__ void scan_cache_impl(const RowView& rv, const uint32_
     }
 }
 
-template <int DTYPE>
-__device__ __forceinline__ void scan_cache_typed(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
-                                                 uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
+template <int DTYPE, int CR>
+__device__ __forceinline__ void scan_cache_typed(const RowView& rv, const uint32_t (&cache)[CR], uint32_t u0, uint32_t w0, uint32_t u1,
+                                                 uint32_t w1, CacheHits<CR>& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
     const bool two = u1 <= 0x7fffu;
     auto at_least = [](uint32_t c) { return 0x80008000u - c * 0x10001u; };  // y + this: bit 15 of a half = (bin >= c)
     auto both = [](uint32_t c) { return c * 0x10001u; };
     const uint32_t n_single = (w0 + 1u) + (two ? w1 + 1u : 0u);  // bins asked for
     if (!two && u0 == 0u) {
-        scan_cache_impl<0, DTYPE>(rv, cache, at_least(w0 + 1u), 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
+        scan_cache_impl<0, DTYPE, CR>(rv, cache, at_least(w0 + 1u), 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
     } else if (n_single <= 3u) {
         uint32_t c[3];
         uint32_t k = 0;
         for (uint32_t b = u0; b <= u0 + w0; ++b) c[k++] = both(b);
         if (two)
             for (uint32_t b = u1; b <= u1 + w1; ++b) c[k++] = both(b);
-        if (k == 1u) scan_cache_impl<1, DTYPE>(rv, cache, c[0], 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
-        else if (k == 2u) scan_cache_impl<2, DTYPE>(rv, cache, c[0], c[1], 0u, 0u, hits, list, n_list, cap, id0, n_groups);
-        else scan_cache_impl<3, DTYPE>(rv, cache, c[0], c[1], c[2], 0u, hits, list, n_list, cap, id0, n_groups);
+        if (k == 1u) scan_cache_impl<1, DTYPE, CR>(rv, cache, c[0], 0u, 0u, 0u, hits, list, n_list, cap, id0, n_groups);
+        else if (k == 2u) scan_cache_impl<2, DTYPE, CR>(rv, cache, c[0], c[1], 0u, 0u, hits, list, n_list, cap, id0, n_groups);
+        else scan_cache_impl<3, DTYPE, CR>(rv, cache, c[0], c[1], c[2], 0u, hits, list, n_list, cap, id0, n_groups);
     } else {
-        scan_cache_impl<4, DTYPE>(rv, cache, at_least(u0), at_least(u0 + w0 + 1u), at_least(two ? u1 : 0u), at_least(two ? u1 + w1 + 1u : 0u),
+        scan_cache_impl<4, DTYPE, CR>(rv, cache, at_least(u0), at_least(u0 + w0 + 1u), at_least(two ? u1 : 0u), at_least(two ? u1 + w1 + 1u : 0u),
                                   hits, list, n_list, cap, id0, n_groups);
     }
 }
-__device__ __forceinline__ void scan_cache(const RowView& rv, const uint32_t (&cache)[kCacheRegs], uint32_t u0, uint32_t w0, uint32_t u1,
-                                           uint32_t w1, CacheHits& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
-    if (rv.dtype == 0) scan_cache_typed<0>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
-    else scan_cache_typed<1>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
+template <int CR>
+__device__ __forceinline__ void scan_cache(const RowView& rv, const uint32_t (&cache)[CR], uint32_t u0, uint32_t w0, uint32_t u1,
+                                           uint32_t w1, CacheHits<CR>& hits, uint2* list, uint32_t* n_list, uint32_t cap, uint32_t id0, int n_groups) {
+    if (rv.dtype == 0) scan_cache_typed<0, CR>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
+    else scan_cache_typed<1, CR>(rv, cache, u0, w0, u1, w1, hits, list, n_list, cap, id0, n_groups);
 }
 
 // Smallest key whose bin is ranked before bin `bcut` (bins fall as keys rise, so the predicate is monotone):
@@ -1092,7 +1098,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // ranks [rank0, rank1). An unsplit row: all of it.
     RowView rvs = rv;
     uint32_t id0 = 0u, rank0 = 0u, rank1 = n_touched;
-    if (split) {
+    if (WS_USUAL(split)) {  // (the split kernel's usual case; compiled out of the others)
         const uint32_t per_part = ((V + n_parts - 1u) / n_parts + 255u) & ~255u;
         id0 = min(part * per_part, V);
         rvs.V = min(per_part, V - id0);
@@ -1404,7 +1410,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     float m = -INFINITY;
     bool cached = false;
     uint64_t* hist2 = FUSED && A.lds_tie ? reinterpret_cast<uint64_t*>(lds + A.lds_tie) : nullptr;  // second copy of the histogram
-    uint32_t cache[kCacheRegs];  // dead code (and no registers) in the exact instantiation
+    // the split kernel's slices are at most half a row (two parts at least): half the registers, and room for everything else
+    constexpr int kCR = SPLIT ? kCacheRegs / 2 : kCacheRegs;
+    uint32_t cache[kCR];  // dead code (and no registers) in the exact instantiation
     if (FUSED && !(flags & kBadParam)) {
         // ---------------------------------------------------------------- fused sweep: anchor, histogram, max, bins
         bool swept = false;
@@ -1412,7 +1420,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint4* stage = reinterpret_cast<uint4*>(emass);
         const uint32_t stage_cap = rv.vec ? 2047u : 0u;  // the region's last slot takes the vectors of the ranks beyond
         float given_s = __uint_as_float(0x7fc00000u);  // NaN: none
-        if (split) {
+        if (WS_USUAL(split)) {  // (the split kernel's usual case; compiled out of the others)
             // the provisional bound has to be the same in every part: all take it from the head of the row, the loads an
             // unsplit row starts with
             const uint4* xv = static_cast<const uint4*>(rv.base);
@@ -1431,7 +1439,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             given_s = block_max(s0, red_f);
             if (given_s != given_s) given_s = INFINITY;  // a NaN at the head: no bound, as for an unsplit row
         }
-        if constexpr (FUSED) swept = fused_pass<SPLIT>(rvs, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m, given_s, rank0);
+        if constexpr (FUSED) swept = fused_pass<SPLIT, kCR>(rvs, -INFINITY, inv_t, c64, hist, hist2, cache, red_f, stage, stage_cap, anchor, aq, m, given_s, rank0);
         __syncthreads();
         WS_MARK(8);
         auto all_adjusted = [&]() {  // this part goes on alone: the touched tokens of the other slices, then the largest adjusted logit
@@ -1451,7 +1459,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             float m_all = fmaxf(fmaxf(m, mu), ma);
             block_max2(m_all, ma, red_f, reinterpret_cast<float*>(red_u));
             m_adj = ma;
-            if (split && swept) {
+            if (WS_USUAL(split && swept)) {
                 // ---- the parts' histograms and maxima meet in global memory; every part takes the sums back
                 uint64_t* gh = reinterpret_cast<uint64_t*>(work + kSplitHist);
 #pragma unroll
@@ -1490,7 +1498,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
             }
         }
-        if (split && (!cached || (flags & kSplitTimeout) || !(m > -INFINITY))) {
+        if (WS_RARE(split && (!cached || (flags & kSplitTimeout) || !(m > -INFINITY)))) {
             // A row the sweep's bound does not fit (or that has no token at all, or whose parts did not meet): part 0 goes on
             // alone, as for an unsplit row; the others are done.
             if (swept && leave_shared()) clean_shared();
@@ -1498,7 +1506,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             split = false;
             all_adjusted();
         }
-        if (!cached) {
+        if (WS_RARE(!cached)) {
             m = -INFINITY;
             stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
             m = fmaxf(block_max(m, red_f), m_adj);
@@ -1531,7 +1539,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 cached = m <= anchor && (anchor - m) * c64 <= 1024.f;  // here: the histogram stands
             }
         }
-        if (!cached) {
+        if (WS_RARE(!cached)) {
             // ------------------------------------------------------------ pass 1: maximum
             m = -INFINITY;
             stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
@@ -1539,7 +1547,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
-    if (flags) {  // uniform over the block (and over the parts of a split row)
+    if (WS_RARE(flags)) {  // uniform over the block (and over the parts of a split row)
         if (t == 0 && (part == 0u || !split)) {
             A.token[row] = -1;
             A.flags[row] = flags;
@@ -1557,7 +1565,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     WS_MARK(1);
-    if (!cached) {
+    if (WS_RARE(!cached)) {
         // ---------------------------------------------------------------- pass 2: histogram of (count, mass) below the maximum
         anchor = m;
         aq = anchor_product(anchor, c64);
@@ -1800,7 +1808,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // are kept whole - before range 0, and between the ranges - give theirs here from the scanned masses, every token
     // of a bin counted at the middle of the bin (a to +-1/128): h_before / h_between.
     double h_before = 0.0, h_between = 0.0;
-    if (A.entropy && !(flags & kOverflow)) {  // uniform
+    if (WS_RARE(A.entropy && !(flags & kOverflow))) {  // uniform
         double s0 = 0.0, s1 = 0.0;
         for (int b = static_cast<int>(t); b < kTail; b += WS_BLOCK) {
             const double dm = pm[b + 1] - pm[b];
@@ -1824,7 +1832,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     double Zk_out = 0.0;  // mass of the kept set (the row's float normaliser on an open row)
     bool finished = false;
     bool finished_lean = false;
-    if (split && (flags & kOverflow)) {  // uniform over the parts (the merged histogram says so): part 0 takes the row through the exact path
+    if (WS_RARE(split && (flags & kOverflow))) {  // uniform over the parts (the merged histogram says so): part 0 takes the row through the exact path
         if (leave_shared()) clean_shared();
         if (part != 0u) return;
         split = false;
@@ -1879,9 +1887,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     s_u[6] = s_u[7] = 0u;
                 }
                 {
-                    CacheHits hits;
+                    CacheHits<kCR> hits;
                     // a group of 16 registers holds 16384 consecutive tokens of the block; a slice fills only the first few
-                    const int n_groups = split ? static_cast<int>((rvs.V + 16383u) >> 14) : kCacheGroups;
+                    const int n_groups = split ? static_cast<int>((rvs.V + 16383u) >> 14) : kCR / 16;
                     scan_cache(rvs, cache, u0, w0, u1r, w1, hits, list, &s_u[4], kCap, id0, n_groups);
                     WS_MARK(10);
                     // touched tokens whose adjusted logit lies in the ranges, while the last loads of the scan travel
@@ -1893,13 +1901,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     });
                     uint32_t mine = 0;
 #pragma unroll
-                    for (int g = 0; g < kHitSlots; ++g) mine += hits.idx[g] != 0xffffffffu ? 1u : 0u;
+                    for (int g = 0; g < CacheHits<kCR>::kSlots; ++g) mine += hits.idx[g] != 0xffffffffu ? 1u : 0u;
                     const uint32_t inc = wave_incl_scan(mine);
                     uint32_t base = 0;
                     if (lane_id() == 63 && inc) base = atomicAdd(&s_u[4], inc);
                     uint32_t slot = __shfl(base, 63) + inc - mine;
 #pragma unroll
-                    for (int g = 0; g < kHitSlots; ++g) {
+                    for (int g = 0; g < CacheHits<kCR>::kSlots; ++g) {
                         if (hits.idx[g] == 0xffffffffu) continue;
                         if (slot < kCap) list[slot] = make_uint2(hits.idx[g] + id0, hits.bits[g]);
                         ++slot;
@@ -1910,7 +1918,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 WS_MARK(41);
                 uint32_t n_hit = min(s_u[4], kCap);
                 if (s_u[4] > kCap) flags |= kOverflow;
-                if (split) {
+                if (WS_USUAL(split)) {  // (the split kernel's usual case; compiled out of the others)
                     // ---- the parts' candidates meet in global memory; the part that brings the last ones finishes the row
                     uint2* glist = reinterpret_cast<uint2*>(work + kSplitList);
                     __syncthreads();  // every thread has its n_hit
@@ -2206,7 +2214,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         kept_key = 0ull;
                     }
                 }
-                if (!finished) {  // uniform: the list goes to keys[] by range, as the sort-based finish expects it
+                if (WS_RARE(!finished)) {  // uniform: the list goes to keys[] by range, as the sort-based finish expects it
                 for (uint32_t k0 = 0; k0 < n_hit; k0 += 4u * WS_BLOCK) {
                     uint2 en[4];
                     float xs[4];
@@ -2462,7 +2470,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             found = true;
         }
     };
-    if (!finished && !(flags & kOverflow)) {  // uniform: the sort-based finish
+    if (FUSED ? WS_RARE(!finished && !(flags & kOverflow)) : !(flags & kOverflow)) {  // uniform: the sort-based finish (the only one of the kernels without a bin cache)
 #ifdef WS_PHASE_TIMERS
     if (t == 0 && A.kept_logits) {
         float* dbg = A.kept_logits + static_cast<size_t>(row) * A.kept_cap;
@@ -3052,7 +3060,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     };
     bool finished_slow = false;
-    if ((flags & kOverflow) && m > -INFINITY) {  // uniform
+    if (WS_RARE((flags & kOverflow) && m > -INFINITY)) {  // uniform
         flags &= ~kOverflow;
         finished = finished_slow = true;
         finished_lean = false;
@@ -3093,7 +3101,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if (mg_draw < tol) flags |= kNearDraw;
 
     // ------------------------------------------------------------------ optional: the kept set's entropy
-    if (A.entropy) {  // uniform
+    if (WS_RARE(A.entropy)) {  // uniform
         // terms of the gathered candidates that are kept: exact
         double se = 0.0, sm = 0.0;
         auto term = [&](uint64_t key) {
@@ -3132,7 +3140,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (t == 0) A.entropy[row] = h;
     }
-    if (A.query_prob && t == 0) {
+    if (WS_RARE(A.query_prob && t == 0)) {
         // probability of one named token under the filtered distribution (probOf, src/sampling/sampler.cpp:108-116)
         const int32_t q = A.query ? A.query[row] : -1;
         double pq = 0.0;
@@ -3169,7 +3177,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     // ------------------------------------------------------------------ optional: the kept set in ascending id order
-    if (A.kept_ids && token >= 0) {
+    if (WS_RARE(A.kept_ids && token >= 0)) {
         int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
         __syncthreads();
