@@ -133,9 +133,6 @@ enum {
     WS_FLAG_OPEN = 1u << 6,        /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order
                                       (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
-    WS_FLAG_SPLIT_TIMEOUT = 1u << 8, /* a row split over several workgroups (see ws_batch.workspace) whose parts did not all
-                                      start within about a second - the launch shared the GPU with work that held its compute
-                                      units: token = -1; zero-fill the workspace before it is used again */
     WS_FLAG_APPROX_ENTROPY = 1u << 7 /* `entropy` counts the kept tokens outside the gathered bins at the middle of their
                                       histogram bin (each within 1/128 of its place: the entropy is within 1/128 absolute,
                                       usually far closer) instead of one by one; rows whose kept set a
@@ -224,6 +221,9 @@ typedef struct ws_batch {
     uint32_t max_split;         /* most workgroups a row may be split over (a power of two up to 16, rows * parts within the
                                    GPU's compute units, at least 16384 tokens a part): 0 = the library decides (4, 8 or
                                    16 parts when the batch is small enough for that, else none), 1 = never split */
+    uint32_t split_spins;       /* split rows: how often a part looks for the others before it gives up on them (they all
+                                   have to be running at once, which a GPU shared with other work may not allow in time); the
+                                   row is then done by one workgroup - slower, same result. 0 = about a second's worth */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

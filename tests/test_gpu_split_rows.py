@@ -88,3 +88,15 @@ def test_one_row_is_split_sixteen_ways():
     smp = _run(c, 1, 0, launches=3)
     res = gc.compare_rows(c, smp, range(1), 1)
     assert res["exact"] == 1, res
+
+
+def test_parts_that_give_up_on_each_other_leave_the_row_to_one_workgroup():
+    """The bounded wait, forced from the host: with one look at the arrival counter most parts give up at once; the row is
+    then done by part 0 alone. Same tokens as ever, workspace left clean, launch after launch."""
+    c = gc.make_cfg2(rows=5, V=V, n_hist=1024, n_bias=30)
+    one = _run(c, 1, 1, launches=1)
+    smp = _run(c, 1, 0, launches=3, split_spins=1)
+    assert gc.compare_rows(c, smp, range(5), 1)["exact"] == 5
+    for name in ("token", "n_kept", "flags"):  # (the probabilities come from the histogram against the exact maximum here: last bits differ)
+        assert torch.equal(getattr(one, name), getattr(smp, name)), name
+    assert torch.allclose(one.prob, smp.prob, rtol=1e-6, atol=0)

@@ -20,7 +20,7 @@ DTYPE_F32, DTYPE_BF16 = 0, 1
 RNG_SPLITMIX, RNG_PHILOX = 0, 1
 MODE_AUTO, MODE_EXACT, MODE_FUSED = 0, 1, 2
 FLAG_NEAR_TOP_P, FLAG_NEAR_MIN_P, FLAG_NEAR_DRAW = 1, 2, 4
-FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN, FLAG_APPROX_ENTROPY, FLAG_SPLIT_TIMEOUT = 8, 16, 32, 64, 128, 256
+FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN, FLAG_APPROX_ENTROPY = 8, 16, 32, 64, 128
 ACCEPT_OK, ACCEPT_HOST, ACCEPT_NEAR_TYPICAL, ACCEPT_HISTORY_FULL = 0, 1, 2, 4
 FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
 CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
@@ -54,7 +54,7 @@ class Batch(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32),
                 ("race", C.c_void_p),
                 ("hist_len", C.c_void_p), ("query", C.c_void_p), ("query_prob", C.c_void_p), ("entropy", C.c_void_p),
-                ("max_split", C.c_uint32)]
+                ("max_split", C.c_uint32), ("split_spins", C.c_uint32)]
 
 
 class SpecVerify(C.Structure):
@@ -345,7 +345,7 @@ class BatchSampler:
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
                  max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None,
-                 hist_len=None, query=None, want_entropy=False, max_split=0):
+                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -382,7 +382,7 @@ class BatchSampler:
         self.query_prob = torch.zeros(rows, dtype=torch.float64, device=dev) if query is not None else None
         self.entropy = torch.zeros(rows, dtype=torch.float64, device=dev) if want_entropy else None
         b.query_prob, b.entropy = _p(self.query_prob), _p(self.entropy)
-        b.max_split = max_split
+        b.max_split, b.split_spins = max_split, split_spins
         need = lib().ws_sample_batch_workspace(C.byref(b))
         # zero-filled once: the parts of a split row meet here, and every launch leaves it zero-filled again
         self.workspace = torch.zeros(max(int(need), 16), dtype=torch.uint8, device=dev)

@@ -267,6 +267,7 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     ws::BatchArgs a{};
     a.split_log2 = can_split ? p.split_log2 : 0u;
     a.work = work;
+    a.split_spins = b->split_spins;
     a.logits = b->logits;
     a.dtype = b->dtype;
     a.rows = b->rows;

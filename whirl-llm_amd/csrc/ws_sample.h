@@ -94,13 +94,13 @@ struct BatchArgs {
     double* entropy;           // out per row or nullptr: entropy of the kept set
     uint32_t split_log2;       // single-sweep kernel: a row is worked on by 2^split_log2 workgroups (0: one), block = row * parts + part
     unsigned char* work;       // split rows: kSplitRowBytes of zero-filled global memory per row, left zero-filled
+    uint32_t split_spins;      // split rows: looks at the arrival counter before a part gives up on the others (0: about a second's worth)
 };
 
 // Global memory of a split row: the merged histogram, the merged candidate list, and four control words (parts that
 // have merged their histogram, parts that are done with the shared state, candidates listed, the row maximum as an
 // ordered integer).
 constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kSplitRowBytes = 65536u + 256u;
-constexpr uint32_t kSplitTimeout = 256u;  // flag: the parts of a row did not all turn up
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
 // replayed from LDS, where phase 0 left their adjusted logits by rank.
@@ -1420,6 +1420,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         uint4* stage = reinterpret_cast<uint4*>(emass);
         const uint32_t stage_cap = rv.vec ? 2047u : 0u;  // the region's last slot takes the vectors of the ranks beyond
         float given_s = __uint_as_float(0x7fc00000u);  // NaN: none
+        bool gave_up = false;  // a split row whose parts did not all arrive in time
         if (WS_USUAL(split)) {  // (the split kernel's usual case; compiled out of the others)
             // the provisional bound has to be the same in every part: all take it from the head of the row, the loads an
             // unsplit row starts with
@@ -1472,13 +1473,32 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's additions are acknowledged (device-scope atomics: they are in memory)
                 __syncthreads();
                 if (t == 0) {
-                    __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    // The wait for the other parts is bounded (they may not be running: the launch has to have the compute
+                    // units to itself for all parts to be resident at once). A part that has waited long enough gives up for
+                    // the whole row: it sets the top bit of the counter - by compare-and-swap, so that "everybody has
+                    // arrived" and "given up" exclude each other - and every part that sees the bit, now or when it arrives,
+                    // leaves the row to part 0, which does it alone. No row fails; it is only slower.
+                    constexpr uint32_t kGaveUp = 0x80000000u;
+                    const uint32_t limit = A.split_spins ? A.split_spins : 1u << 21;
+                    uint32_t v = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
                     uint32_t spins = 0;
-                    while (__hip_atomic_load(&ctrl[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < n_parts && ++spins < (1u << 21)) __builtin_amdgcn_s_sleep(1);
-                    s_prev = spins < (1u << 21) ? 1u : 0u;
+                    while (!(v & kGaveUp) && v < n_parts) {
+                        if (++spins >= limit) {
+                            uint32_t seen = v;
+                            if (__hip_atomic_compare_exchange_strong(&ctrl[0], &seen, v | kGaveUp, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                                v |= kGaveUp;
+                                break;
+                            }
+                            v = seen;  // the counter moved meanwhile: look again
+                            continue;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                        v = __hip_atomic_load(&ctrl[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    s_prev = (v & kGaveUp) ? 0u : 1u;
                 }
                 __syncthreads();
-                if (!s_prev) flags |= kSplitTimeout;  // uniform
+                gave_up = !s_prev;  // uniform
                 // (the merged values are read with loads of device scope: no stale copy in this unit's caches is used)
                 m_all = unkey32(__hip_atomic_load(&ctrl[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
                 {
@@ -1498,12 +1518,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 cached = m <= anchor && (anchor - m) * c64 <= 1024.f;
             }
         }
-        if (WS_RARE(split && (!cached || (flags & kSplitTimeout) || !(m > -INFINITY)))) {
+        if (WS_RARE(split && (!cached || gave_up || !(m > -INFINITY)))) {
             // A row the sweep's bound does not fit (or that has no token at all, or whose parts did not meet): part 0 goes on
             // alone, as for an unsplit row; the others are done.
             if (swept && leave_shared()) clean_shared();
             if (part != 0u) return;
             split = false;
+            cached = false;  // (parts that did not meet have no common histogram)
             all_adjusted();
         }
         if (WS_RARE(!cached)) {
