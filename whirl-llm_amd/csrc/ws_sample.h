@@ -160,7 +160,28 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
             const uint32_t j = j0 + u * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;
             b.q[u] = xv[jc];
-            b.na[u] = (MASKED && rv.allow) ? ~rv.allow[(jc * per) >> 5] : 0u;
+            b.na[u] = 0u;
+        }
+        if (MASKED && rv.allow) {
+            // The allow words of a wave's KB loads - 8 consecutive words per load (16 for bf16) - are fetched by one
+            // instruction, a word per lane, and handed to the lanes that need them through the LDS crossbar: one memory
+            // instruction per batch instead of one per load (a row of 262144 tokens spent a third of a masked sweep on
+            // those 4-byte loads).
+            const uint32_t lane = t & 63u, wave0 = t & ~63u;
+            const uint32_t lw = per == 4u ? 3u : 4u;  // log2 of the words per load
+            const uint32_t last_word = (V - 1u) >> 5;
+#pragma unroll
+            for (int r = 0; r < (KB * 16 + 63) / 64; ++r) {  // rounds of 64 words (one, or two for eight bf16 loads)
+                const uint32_t u_of = (static_cast<uint32_t>(r) * 64u + lane) >> lw, w_of = lane & ((1u << lw) - 1u);
+                uint32_t mine = 0u;
+                if (u_of < static_cast<uint32_t>(KB))
+                    mine = ~rv.allow[min((((j0 + u_of * WS_BLOCK + wave0) * per) >> 5) + w_of, last_word)];
+#pragma unroll
+                for (int u = 0; u < KB; ++u) {
+                    const uint32_t src = (static_cast<uint32_t>(u) << lw) + ((lane * per) >> 5);  // this lane's word among the KB << lw of the wave
+                    if ((src >> 6) == static_cast<uint32_t>(r)) b.na[u] = __shfl(mine, static_cast<int>(src & 63u));
+                }
+            }
         }
     };
     Batch cur, nxt;
@@ -2267,20 +2288,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
             }
         } else {
-            // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
-            // are re-read after the batch, from the cache lines the batch has just pulled in
-            uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
-            const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
+            // a match (a few per thousand tokens) goes to the list straight from the registers of the sweep: reading it
+            // again after the batch made every wave wait for that read - and with it for the next batch's loads, which
+            // were meant to travel meanwhile - at the end of every batch (cfg5's gather sweep: 157 K clocks per row)
             stream_row(
-                rv, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
-                [&](uint32_t j0, uint32_t i_tail) {
-                    while (hit) {
-                        const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
-                        hit &= hit - 1u;
-                        const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot >> lper) * WS_BLOCK + t) * per + (slot & (per - 1u));
-                        push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
-                    }
-                });
+                rv,
+                [&](uint32_t i, float x, int) {
+                    if (in_ranges(x)) push(i, x);  // masked and touched tokens arrive as NaN: never in a range
+                },
+                [](uint32_t, uint32_t) {});
         }
         if (!(FUSED && cached))
             replay_touched([&](uint32_t i, float x) {
