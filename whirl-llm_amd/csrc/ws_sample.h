@@ -142,7 +142,7 @@ __device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
 // before any is used, and the next batch is requested before this one is consumed. Tokens that are masked out or that
 // the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bins or ignores it, so the
 // hot loop has no branch; the touched ones are fed afterwards, by rank, with their adjusted values.
-template <bool MASKED, int KB, class F, class E>
+template <bool MASKED, bool COOP, int KB, class F, class E>  // COOP: an allow mask whose words are fetched once per wave and batch
 __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch) {
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
@@ -160,9 +160,9 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
             const uint32_t j = j0 + u * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;
             b.q[u] = xv[jc];
-            b.na[u] = 0u;
+            b.na[u] = (MASKED && !COOP && rv.allow) ? ~rv.allow[(jc * per) >> 5] : 0u;
         }
-        if (MASKED && rv.allow) {
+        if constexpr (COOP) {
             // The allow words of a wave's KB loads - 8 consecutive words per load (16 for bf16) - are fetched by one
             // instruction, a word per lane, and handed to the lanes that need them through the LDS crossbar: one memory
             // instruction per batch instead of one per load (a row of 262144 tokens spent a third of a masked sweep on
@@ -223,17 +223,20 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
     }
 }
 
-template <class F, class E>
+// COOP: take the cooperative fetch of the allow words where there is a mask (the kernels without a bin cache, whose
+// every pass is such a loop; the single-sweep kernel only falls back to these loops and keeps the plain ones)
+template <bool COOP, class F, class E>
 __device__ __forceinline__ void stream_row(const RowView& rv, F&& f, E&& end_batch) {
-    if (rv.allow || rv.touched) stream_row_impl<true, kBatch>(rv, f, end_batch);
-    else stream_row_impl<false, kBatch>(rv, f, end_batch);
+    if (COOP && rv.allow) stream_row_impl<true, true, kBatch>(rv, f, end_batch);
+    else if (rv.allow || rv.touched) stream_row_impl<true, false, kBatch>(rv, f, end_batch);
+    else stream_row_impl<false, false, kBatch>(rv, f, end_batch);
 }
 // the same with twice the loads in flight, for passes that run when the bin cache no longer holds the registers
 constexpr int kWide = 2 * kBatch;
 template <class F, class E>
 __device__ __forceinline__ void stream_row_wide(const RowView& rv, F&& f, E&& end_batch) {
-    if (rv.allow || rv.touched) stream_row_impl<true, kWide>(rv, f, end_batch);
-    else stream_row_impl<false, kWide>(rv, f, end_batch);
+    if (rv.allow || rv.touched) stream_row_impl<true, false, kWide>(rv, f, end_batch);
+    else stream_row_impl<false, false, kWide>(rv, f, end_batch);
 }
 
 // ---- bins. A token's bin coordinate is t = fma(x, -c64, aq): c64 = 64 * inv_t and aq = anchor * c64 rounded a little
@@ -1550,7 +1553,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (WS_RARE(!cached)) {
             m = -INFINITY;
-            stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+            stream_row<!FUSED>(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
             m = fmaxf(block_max(m, red_f), m_adj);
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
@@ -1569,7 +1572,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 aq = anchor_product(anchor, c64);
                 for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
                 __syncthreads();
-                stream_row(
+                stream_row<!FUSED>(
                     rv,
                     [&](uint32_t i, float x, int slot) {
                         m = fmaxf(m, x);
@@ -1584,7 +1587,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         if (WS_RARE(!cached)) {
             // ------------------------------------------------------------ pass 1: maximum
             m = -INFINITY;
-            stream_row(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
+            stream_row<!FUSED>(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
             m = fmaxf(block_max(m, red_f), m_adj);
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
@@ -1614,7 +1617,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         __syncthreads();
         for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
         __syncthreads();
-        stream_row(rv, add_to_hist, [](uint32_t, uint32_t) {});
+        stream_row<!FUSED>(rv, add_to_hist, [](uint32_t, uint32_t) {});
         replay_touched([&](uint32_t i, float x) { add_to_hist(i, x, 0); });
     }
     __syncthreads();
@@ -2288,15 +2291,20 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 }
             }
         } else {
-            // a match (a few per thousand tokens) goes to the list straight from the registers of the sweep: reading it
-            // again after the batch made every wave wait for that read - and with it for the next batch's loads, which
-            // were meant to travel meanwhile - at the end of every batch (cfg5's gather sweep: 157 K clocks per row)
-            stream_row(
-                rv,
-                [&](uint32_t i, float x, int) {
-                    if (in_ranges(x)) push(i, x);  // masked and touched tokens arrive as NaN: never in a range
-                },
-                [](uint32_t, uint32_t) {});
+            // the hot loop only records which of the thread's batch slots matched; matches (a few per thousand tokens)
+            // are re-read after the batch, from the cache lines the batch has just pulled in
+            uint32_t hit = 0;  // kBatch * 8 = 32 slots at most
+            const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
+            stream_row<!FUSED>(
+                rv, [&](uint32_t, float x, int slot) { hit |= static_cast<uint32_t>(in_ranges(x)) << slot; },
+                [&](uint32_t j0, uint32_t i_tail) {
+                    while (hit) {
+                        const uint32_t slot = static_cast<uint32_t>(__ffs(hit)) - 1u;
+                        hit &= hit - 1u;
+                        const uint32_t i = j0 == 0xffffffffu ? i_tail : (j0 + (slot >> lper) * WS_BLOCK + t) * per + (slot & (per - 1u));
+                        push(i, raw_logit(rv, i));  // a match is neither masked nor touched: its raw logit is its logit
+                    }
+                });
         }
         if (!(FUSED && cached))
             replay_touched([&](uint32_t i, float x) {
