@@ -194,11 +194,17 @@ typedef struct ws_batch {
     float* kept_logits; /* out (may be NULL): penalty-applied logits of kept_ids */
     uint32_t kept_cap;
 
-    void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes, or NULL. It serves small batches: with
-                               fewer rows than the GPU has compute units a row is worked on by several workgroups, which
-                               meet in this memory. The caller zero-fills it once before its first use and leaves it
-                               alone afterwards: every launch puts back the zeros the next one needs. Two launches that overlap in time need a workspace each.
-                               Without it (or with too little of it) every row is one workgroup's. */
+    void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes, 16-byte aligned, or NULL. It serves
+                               (a) small batches: with fewer rows than the GPU has compute units a row is worked on by
+                               several workgroups, which meet in this memory. The caller zero-fills it once before its
+                               first use and leaves it alone afterwards: every launch puts back the zeros the next one
+                               needs; (b) rows of the kernels that sweep the row twice (long or unaligned vocabularies)
+                               that have a history or a bias: the first sweep leaves the raw logits of those tokens
+                               here (8 bytes per history / bias entry) instead of gathering them one by one, and
+                               leaves the memory with arbitrary contents - zero-fill it again before a batch of
+                               another shape uses it. Two launches that overlap in time need a workspace each.
+                               Without it (or with too little of it) every row is one workgroup's and the touched
+                               tokens are gathered: slower, same results. */
     uint64_t workspace_bytes;
     double tol;             /* flag tolerance, relative; values below 1e-6 (and 0) mean 1e-6, the accuracy of the mass estimates */
     int32_t mode;           /* WS_MODE_* */
@@ -237,7 +243,7 @@ int ws_sample_batch(void* stream, const ws_batch* b);
  * than that (65 to 128 rows in two parts each) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is
  * looked up on the first call there (or by ws_probe): make that call before capturing a graph. All calls on one GPU
  * share this memory: two of them that run at the same time (different streams) race; on one stream they are safe, each
- * launch leaves the memory as the next needs it. */
+ * launch leaves the memory as the next needs it. (Only split rows use it: use (b) of b->workspace is off here.) */
 #define WS_STATIC_SPLIT_ROWS 64
 int ws_sample_batch_static(void* stream, const ws_batch* b);
 

@@ -345,7 +345,7 @@ class BatchSampler:
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
                  max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None,
-                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0):
+                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0, use_workspace=True):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -386,7 +386,8 @@ class BatchSampler:
         need = lib().ws_sample_batch_workspace(C.byref(b))
         # zero-filled once: the parts of a split row meet here, and every launch leaves it zero-filled again
         self.workspace = torch.zeros(max(int(need), 16), dtype=torch.uint8, device=dev)
-        b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()
+        if use_workspace:  # (without: no split rows, and the two-sweep kernels gather their touched tokens one by one)
+            b.workspace, b.workspace_bytes = _p(self.workspace), self.workspace.numel()
         self.desc = b
 
     def run(self, stream=None):

@@ -128,6 +128,9 @@ BatchPlan plan_batch(const ws_batch* b) {
         p.split_log2 = lg;
         if (lg) p.workspace = uint64_t{b->rows} * ws::kSplitRowBytes;
     }
+    // The kernels without a bin cache (long vocabularies, unaligned rows) take the touched tokens' raw logits from
+    // their first sweep when they have somewhere to put them: 8 bytes per history / bias entry and row.
+    if (!p.fused && cap > 0 && b->mode == WS_MODE_AUTO) p.workspace = uint64_t{b->rows} * ws::capture_row_bytes(p.patch_cap);
     p.err = WS_OK;
     return p;
 }
@@ -266,7 +269,7 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     const bool can_split = p.workspace && work && work_bytes >= p.workspace && reinterpret_cast<uintptr_t>(work) % 8u == 0;
     ws::BatchArgs a{};
     a.split_log2 = can_split ? p.split_log2 : 0u;
-    a.work = work;
+    a.work = (p.fused ? can_split : p.workspace && work && work_bytes >= p.workspace && reinterpret_cast<uintptr_t>(work) % 16u == 0) ? work : nullptr;
     a.split_spins = b->split_spins;
     a.logits = b->logits;
     a.dtype = b->dtype;
@@ -337,6 +340,7 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
 int ws_sample_batch_static(void* stream, const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     if (p.err != WS_OK) return p.err;
+    if (!p.fused) return sample_batch_on(stream, b, p, nullptr, 0);  // (nothing may be left in the split rows' memory)
     if (p.workspace > sizeof(scratch)) return WS_E_STATIC_LIMIT;  // more split rows than the library's own memory holds
     unsigned char* at = nullptr;
     if (const int e = scratch_address(&at); e != WS_OK) return e;

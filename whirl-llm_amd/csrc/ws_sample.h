@@ -101,6 +101,12 @@ struct BatchArgs {
 // have merged their histogram, parts that are done with the shared state, candidates listed, the row maximum as an
 // ordered integer).
 constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kSplitRowBytes = 65536u + 256u;
+// Workspace of one row of the three-pass kernel: per history / bias entry a word of each of phase 0's two rank
+// tables, which sit out the first sweep there. Whole memory lines, so that rows share none.
+__host__ __device__ constexpr uint64_t capture_row_bytes(uint32_t patch_cap) {
+    const uint64_t cap4 = (static_cast<uint64_t>(patch_cap) + 3u) & ~uint64_t{3};
+    return (8u * cap4 + 127u) & ~uint64_t{127};
+}
 
 // One row as the passes see it. Tokens the history or the bias list touches are skipped by the streaming loop and
 // replayed from LDS, where phase 0 left their adjusted logits by rank.
@@ -142,8 +148,11 @@ __device__ __forceinline__ float adjusted_logit(const RowView& rv, uint32_t i) {
 // before any is used, and the next batch is requested before this one is consumed. Tokens that are masked out or that
 // the history / bias touch arrive as NaN (all bits set): every consumer sends NaN to the tail bins or ignores it, so the
 // hot loop has no branch; the touched ones are fed afterwards, by rank, with their adjusted values.
-template <bool MASKED, bool COOP, int KB, class F, class E>  // COOP: an allow mask whose words are fetched once per wave and batch
-__device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch) {
+struct NoCapture {};
+// cap(rank, raw logit; -inf when masked out or NaN) for every touched token as it goes by (NoCapture: nobody asks)
+template <bool MASKED, bool COOP, int KB, class F, class E, class C = NoCapture>  // COOP: an allow mask whose words are fetched once per wave and batch
+__device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& end_batch, C&& cap = NoCapture{}) {
+    constexpr bool kCapture = !std::is_same_v<std::decay_t<C>, NoCapture>;
     const uint32_t t = threadIdx.x;
     const uint32_t V = rv.V;
     const uint32_t per = rv.dtype == 0 ? 4u : 8u;  // elements per 128-bit load
@@ -195,8 +204,29 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
             if (j >= nv) continue;
             const uint32_t i = j * per;
             const uint32_t tw = (MASKED && rv.touched) ? rv.touched[i >> 5] : 0u;
+            uint32_t wp = 0u;
+            if constexpr (kCapture) wp = rv.wprefix[i >> 5];  // (asked for with the bitmap word, not inside the branch below)
             const int32_t bw = static_cast<int32_t>((cur.na[u] | tw) >> (i & 31u));
             const uint32_t w[4] = {cur.q[u].x, cur.q[u].y, cur.q[u].z, cur.q[u].w};
+            if constexpr (kCapture && MASKED) {
+                const uint32_t tb = (tw >> (i & 31u)) & ((1u << per) - 1u);
+                if (tb) {  // (nearly every wave has a lane with such a vector: kept short, one LDS store as a rule)
+                    uint32_t rk = wp + __popc(tw & ((1u << (i & 31u)) - 1u));  // rank of the vector's first touched token
+                    const uint32_t nb = cur.na[u] >> (i & 31u);
+                    // the first one's logit out of the vector's registers, by masks (an indexed read would send the
+                    // vector through scratch memory); a second touched token in one vector is rare and read again
+                    const uint32_t e = static_cast<uint32_t>(__ffs(tb)) - 1u;
+                    const uint32_t k = rv.dtype == 0 ? e : e >> 1;
+                    uint32_t b = (cur.q[u].x & (k == 0u ? ~0u : 0u)) | (cur.q[u].y & (k == 1u ? ~0u : 0u)) |
+                                 (cur.q[u].z & (k == 2u ? ~0u : 0u)) | (cur.q[u].w & (k == 3u ? ~0u : 0u));
+                    if (rv.dtype != 0) b = (e & 1u) ? (b & 0xffff0000u) : (b << 16);
+                    cap(rk, ((nb >> e) & 1u) ? -INFINITY : fmaxf(__uint_as_float(b), -INFINITY));
+                    for (uint32_t rest = tb & (tb - 1u); rest; rest &= rest - 1u) {
+                        const uint32_t e2 = static_cast<uint32_t>(__ffs(rest)) - 1u;
+                        cap(++rk, ((nb >> e2) & 1u) ? -INFINITY : raw_logit(rv, i + e2));
+                    }
+                }
+            }
             if (rv.dtype == 0) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -218,6 +248,8 @@ __device__ __forceinline__ void stream_row_impl(const RowView& rv, F&& f, E&& en
     }
     for (uint32_t i = nv * per + t; i < V; i += WS_BLOCK) {  // unaligned row or the last few tokens: one-token batches
         const bool skip = is_touched(rv, i) || !is_allowed(rv, i);
+        if constexpr (kCapture)
+            if (is_touched(rv, i)) cap(rank_of(rv, i), is_allowed(rv, i) ? raw_logit(rv, i) : -INFINITY);
         f(i, skip ? __uint_as_float(0xffffffffu) : raw_logit(rv, i), 0);
         end_batch(0xffffffffu, i);
     }
@@ -230,6 +262,12 @@ __device__ __forceinline__ void stream_row(const RowView& rv, F&& f, E&& end_bat
     if (COOP && rv.allow) stream_row_impl<true, true, kBatch>(rv, f, end_batch);
     else if (rv.allow || rv.touched) stream_row_impl<true, false, kBatch>(rv, f, end_batch);
     else stream_row_impl<false, false, kBatch>(rv, f, end_batch);
+}
+// the same, handing the raw logits of the touched tokens to cap on the way (rows with touched tokens only)
+template <class F, class E, class C>
+__device__ __forceinline__ void stream_row_capture(const RowView& rv, F&& f, E&& end_batch, C&& cap) {
+    if (rv.allow) stream_row_impl<true, true, kBatch>(rv, f, end_batch, cap);
+    else stream_row_impl<true, false, kBatch>(rv, f, end_batch, cap);
 }
 // the same with twice the loads in flight, for passes that run when the bin cache no longer holds the registers
 constexpr int kWide = 2 * kBatch;
@@ -1161,7 +1199,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // frequency and presence, each operation rounded to float. pv[r] <- adjusted, praw[r] (the dead count slot) <- raw,
     // pid[r] (the dead bias-sum slot) <- token id. The three-pass kernel runs this before its first pass; the
     // single-sweep kernel after the sweep, when the row has just come through the caches.
-    auto gather_and_adjust = [&](const uint4* stage, uint32_t stage_cap) {
+    // (saved_*: the three-pass kernel with a workspace. Its first sweep has left the raw logits in pv and has gone
+    // over the LDS of the count table and the first-entry table, which were moved out before, the second one as a table
+    // of bias words: nothing is gathered.)
+    auto gather_and_adjust = [&](const uint4* stage, uint32_t stage_cap, const uint32_t* saved_cnt = nullptr,
+                                 const uint32_t* saved_bias = nullptr) {
         if (!n_touched) return;
         const uint32_t per = rv.dtype == 0 ? 4u : 8u, lper = rv.dtype == 0 ? 2u : 3u;
         const int32_t* hist_ids = A.hist + h0;
@@ -1238,32 +1280,63 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             }
         };
         static_assert(kHid == 4, "fetch4 takes its first round from hid");
-        fetch4(hist_ids, nh, true);
-        fetch4(bias_ids, nb, false);
+        if (!saved_cnt) {
+            fetch4(hist_ids, nh, true);
+            fetch4(bias_ids, nb, false);
+        }
         __syncthreads();
         WS_MARK(19);
         {
             float ma = -INFINITY;
-            for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
-                const uint32_t cw = cnt[r], c = cw & 0xfffffu;
-                const float raw = pv[r];
-                float x = raw;
-                if (cw >> 20) {
-                    // the bias values of this id, added one by one in listed order, starting at its first entry
-                    uint32_t j = first[r];
-                    const int32_t id = bias_ids[j];
-                    x = __fadd_rn(x, bias_vals[j]);
-                    if ((cw >> 20) > 1u)
-                        for (++j; j < nb; ++j)
-                            if (bias_ids[j] == id) x = __fadd_rn(x, bias_vals[j]);
-                }
+            auto penalise = [&](float x, uint32_t c) {
                 if (c) {
                     x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
                     x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
                 }
-                pv[r] = x;
-                cnt[r] = __float_as_uint(raw);
-                ma = fmaxf(ma, x);
+                return x;
+            };
+            // the bias values of an id, added one by one in listed order, starting at its first entry j
+            auto add_bias = [&](float x, uint32_t j, uint32_t n) {
+                const int32_t id = bias_ids[j];
+                x = __fadd_rn(x, bias_vals[j]);
+                if (n > 1u)
+                    for (++j; j < nb; ++j)
+                        if (bias_ids[j] == id) x = __fadd_rn(x, bias_vals[j]);
+                return x;
+            };
+            if (saved_cnt) {
+                for (uint32_t r0 = 0; r0 < n_touched; r0 += 4u * WS_BLOCK) {  // four ranks a thread: their reads travel together
+                    uint32_t cw[4], bw[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t r = min(r0 + k * WS_BLOCK + t, n_touched - 1u);
+                        cw[k] = saved_cnt[r];
+                        bw[k] = saved_bias[r];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t r = r0 + k * WS_BLOCK + t;
+                        if (r >= n_touched) continue;
+                        float x = pv[r];
+                        const uint32_t n = cw[k] >> 20;
+                        if (n == 1u) x = __fadd_rn(x, __uint_as_float(bw[k]));  // the one bias value itself
+                        else if (n) x = add_bias(x, bw[k], n);                   // its first entry
+                        x = penalise(x, cw[k] & 0xfffffu);
+                        pv[r] = x;
+                        ma = fmaxf(ma, x);
+                    }
+                }
+            } else {
+                for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+                    const uint32_t cw = cnt[r], c = cw & 0xfffffu;
+                    const float raw = pv[r];
+                    float x = raw;
+                    if (cw >> 20) x = add_bias(x, first[r], cw >> 20);
+                    x = penalise(x, c);
+                    pv[r] = x;
+                    cnt[r] = __float_as_uint(raw);
+                    ma = fmaxf(ma, x);
+                }
             }
             WS_MARK(20);
             block_max2(ma, mu, red_f, reinterpret_cast<float*>(red_u));  // its barriers also end the reads of first[] above
@@ -1431,6 +1504,24 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         const float tc = bin_coord(aq, c64, x, tail_f);
         atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(tc)]), bin_word(tc));
     };
+    // largest of `floor` and the untouched, allowed logits among the row's first 8 * WS_BLOCK tokens, over the block;
+    // every read is asked for before any is used
+    auto head_max = [&](float floor) {
+        float x[8];
+        uint32_t aw[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t i = min(t + k * WS_BLOCK, V - 1u);
+            x[k] = raw_logit(rv, i);
+            aw[k] = rv.allow ? rv.allow[i >> 5] : 0xffffffffu;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t i = t + k * WS_BLOCK;
+            if (i < V && ((aw[k] >> (i & 31u)) & 1u) && !is_touched(rv, i)) floor = fmaxf(floor, x[k]);
+        }
+        return block_max(floor, red_f);
+    };
     float m = -INFINITY;
     bool cached = false;
     uint64_t* hist2 = FUSED && A.lds_tie ? reinterpret_cast<uint64_t*>(lds + A.lds_tie) : nullptr;  // second copy of the histogram
@@ -1558,15 +1649,74 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     } else if (!(flags & kBadParam)) {
-        gather_and_adjust(nullptr, 0u);
-        if (A.two_sweep) {
+        bool adjusted = false;
+        if (A.two_sweep && A.work && n_touched) {
+            // ------------------------------------------------------------ with a workspace: the first sweep leaves the raw
+            // logit of every touched token in pv, by rank, as the token goes by. Gathering them from the row pulls a
+            // whole memory line per token - for a history of 8192 ids as much traffic as the sweep itself. The workspace
+            // is for the rank tables: they of phase 0 share their LDS with
+            // the histogram, so they move out first (the first-entry table as the bias value itself
+            // where an id has one bias entry, as nearly all have: one dependent read less per rank afterwards).
+            const uint32_t cap4 = (A.patch_cap + 3u) & ~3u;
+            uint32_t* gcnt = reinterpret_cast<uint32_t*>(A.work + static_cast<size_t>(row) * capture_row_bytes(A.patch_cap));
+            uint32_t* gbias = gcnt + cap4;
+            {
+                const uint32_t* cnt = reinterpret_cast<const uint32_t*>(lds + A.lds_cnt);
+                const uint32_t* first = cnt + A.patch_cap;
+                const float* bias_vals = A.bias_vals + b0;
+                for (uint32_t r0 = 0; r0 < n_touched; r0 += 4u * WS_BLOCK) {
+                    uint32_t cw[4], fw[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t r = min(r0 + k * WS_BLOCK + t, n_touched - 1u);
+                        cw[k] = cnt[r];
+                        fw[k] = first[r];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if ((cw[k] >> 20) == 1u) fw[k] = __float_as_uint(bias_vals[fw[k]]);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t r = r0 + k * WS_BLOCK + t;
+                        if (r < n_touched) {
+                            gcnt[r] = cw[k];
+                            gbias[r] = fw[k];
+                        }
+                    }
+                }
+            }
+            float s = head_max(-INFINITY);  // (its barriers also end the reads of the rank tables)
+            WS_MARK(9);
+            anchor = s + 8.f / inv_t;
+            if (anchor > -INFINITY && anchor < INFINITY) {  // uniform
+                aq = anchor_product(anchor, c64);
+                for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+                __syncthreads();
+                stream_row_capture(
+                    rv,
+                    [&](uint32_t i, float x, int slot) {
+                        m = fmaxf(m, x);
+                        add_to_hist(i, x, slot);
+                    },
+                    [](uint32_t, uint32_t) {},
+                    [&](uint32_t rank, float raw) { pv[rank] = raw; });
+                __syncthreads();
+                WS_MARK(8);
+                gather_and_adjust(nullptr, 0u, gcnt, gbias);
+                adjusted = true;
+                replay_touched([&](uint32_t i, float x) { add_to_hist(i, x, 0); });
+                m = fmaxf(block_max(m, red_f), m_adj);
+                cached = m <= anchor && (anchor - m) * c64 <= 1024.f;  // here: the histogram stands
+            } else {
+                __syncthreads();
+            }
+        }
+        if (!adjusted) gather_and_adjust(nullptr, 0u);
+        if (A.two_sweep && !adjusted) {
             // ------------------------------------------------------------ maximum and histogram in one sweep, against a
             // bound above the maximum guessed from the adjusted tokens and the head of the row (as the single-sweep
             // mode does); rows the guess does not fit fall through to the two passes below
-            float s = m_adj;
-            for (uint32_t i = t; i < min(V, 8u * WS_BLOCK); i += WS_BLOCK)
-                if (is_allowed(rv, i) && !is_touched(rv, i)) s = fmaxf(s, raw_logit(rv, i));
-            s = block_max(s, red_f);
+            float s = head_max(m_adj);
             anchor = s + 8.f / inv_t;
             if (anchor > -INFINITY && anchor < INFINITY) {  // uniform
                 aq = anchor_product(anchor, c64);
