@@ -285,6 +285,10 @@ def spec_verify_workload(steps, warmup):
     P = m._p
     v = m.SpecVerify(P(p), P(q), P(draft), n_seq, n_pos, V, P(seed), P(step0), m.RNG_PHILOX, P(out), P(nacc), P(flags), None, 0, 0.0)
     L, S = m.lib(), m._stream
+    need = int(L.ws_spec_verify_workspace(C.byref(v)))  # the workspace an engine keeps: sequences split over several workgroups
+    work = torch.zeros(max(need, 8), dtype=torch.uint8, device="cuda:0")
+    if need:
+        v.workspace, v.workspace_bytes = P(work), work.numel()
     for _ in range(warmup):
         m.check(L.ws_spec_verify_classic(S(), C.byref(v)), "ws_spec_verify_classic")
     torch.cuda.synchronize()

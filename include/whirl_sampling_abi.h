@@ -381,7 +381,12 @@ int ws_accept_greedy(void* stream, const ws_accept_greedy_args* a);
  * reference, which removed this rule (include/whirl/spec_sample.h:22-24). p, q: device [n_seq][n_pos][vocab] f32
  * probabilities (q's last position unused); draft: device [n_seq][n_pos - 1] (may be NULL when n_pos is 1). Per sequence s: u_j from
  * (seed[s], row = s, step = step0[s] + j, stream 0); the resample / bonus draw uses stream 1 and walks the vocabulary
- * in id order. out_tokens[s][0 .. n_accepted[s]] = accepted drafts then the drawn token. */
+ * in id order. out_tokens[s][0 .. n_accepted[s]] = accepted drafts then the drawn token.
+ * workspace (optional): device scratch of ws_spec_verify_workspace() bytes, 8-byte aligned, zero-filled once by the caller
+ * before its first use and left alone afterwards (every launch leaves it as the next one needs it; one launch at a
+ * time per workspace). With it, and fewer sequences than half the GPU's compute units, the one row pair a sequence has
+ * to stream is shared by 2 to 16 workgroups (32 sequences of 151936: 19 -> about 9 us); the results are the same to
+ * the last bit. ws_spec_verify_workspace() is 0 when the batch would not be split. */
 typedef struct ws_spec_verify {
     const float* p;
     const float* q;

@@ -238,3 +238,48 @@ def test_classic_verify_cfg4_shape():
     rate, near = check_spec(p, q, draft, seed, step0, 1)
     print("acceptance", rate, "near", near)
     assert 0.4 < rate < 0.8
+
+
+def _verify(p, q, draft, seed, step0, **kw):
+    m = gc.pkg()
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    r = m.spec_verify_classic(t(p), t(q), t(draft), t(seed.view(np.int64)), t(step0.view(np.int64)), rng=1, **kw)
+    torch.cuda.synchronize()
+    return [a.cpu().numpy() for a in r]
+
+
+@pytest.mark.parametrize("n_seq,V", [(1, 151936), (5, 151936), (32, 40000), (3, 40001), (100, 20000)])
+def test_classic_verify_split_over_workgroups_is_the_unsplit_result(n_seq, V):
+    """Few sequences: each one's row pair is streamed by 2 to 16 workgroups that meet in a workspace. Same accepted
+    counts, tokens and flags as one workgroup per sequence, launch after launch on one workspace (each launch leaves
+    it as the next needs it); 40001: the rows of the second sequence on are not 16-byte aligned."""
+    m = gc.pkg()
+    rng = np.random.default_rng(316 + n_seq)
+    p, q, draft, seed, step0 = spec_case(rng, n_seq, 4, V)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    v = m.SpecVerify(None, None, None, n_seq, 4, V)
+    need = int(m.lib().ws_spec_verify_workspace(C.byref(v)))
+    assert need > 0, "this shape is meant to split"
+    work = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    want = _verify(p, q, draft, seed, step0, split=False)
+    for launch in range(3):
+        got = _verify(p, q, draft, seed, step0, workspace=work)
+        for a, b in zip(got, want):
+            assert np.array_equal(a, b), (launch, a, b)
+    arrive = work.view(n_seq, -1)[:, 4096 * 8:4096 * 8 + 4]
+    assert not arrive.any().item(), "arrival counters not back at zero"
+    check_spec(p, q, draft, seed, step0, 1)  # (splits on its own) and the oracle says the same
+
+
+def test_classic_verify_split_with_an_empty_residual():
+    """p = q / 2 (unnormalised on purpose): drafts are rejected with probability 1/2 and max(p - q, 0) is zero everywhere,
+    so the token comes from p - the part that finds the total at zero streams p by itself."""
+    rng = np.random.default_rng(317)
+    _, q, draft, seed, step0 = spec_case(rng, 6, 4, 40000)
+    p = (q * np.float32(0.5)).astype(np.float32)
+    want = _verify(p, q, draft, seed, step0, split=False)
+    got = _verify(p, q, draft, seed, step0)
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b), (a, b)
+    assert (want[0] < 3).any()  # some draft was rejected
+    check_spec(p, q, draft, seed, step0, 1)

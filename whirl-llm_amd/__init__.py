@@ -402,8 +402,10 @@ class BatchSampler:
         return self
 
 
-def spec_verify_classic(p, q, draft, seed, step0, rng=RNG_PHILOX, tol=0.0):
-    """p, q: [n_seq, n_pos, V] float32 device; draft: [n_seq, n_pos - 1] int32; seed, step0: uint64-as-int64 [n_seq]."""
+def spec_verify_classic(p, q, draft, seed, step0, rng=RNG_PHILOX, tol=0.0, workspace=None, split=True):
+    """p, q: [n_seq, n_pos, V] float32 device; draft: [n_seq, n_pos - 1] int32; seed, step0: uint64-as-int64 [n_seq].
+    workspace: a zero-filled uint8 device tensor of ws_spec_verify_workspace bytes kept between calls (each call leaves
+    it as the next needs it), None: one is made for this call when the batch is small enough to split (split=False: never)."""
     n_seq, n_pos, V = p.shape
     dev = p.device
     out = torch.full((n_seq, n_pos), -1, dtype=torch.int32, device=dev)
@@ -411,6 +413,12 @@ def spec_verify_classic(p, q, draft, seed, step0, rng=RNG_PHILOX, tol=0.0):
     flags = torch.empty(n_seq, dtype=torch.int32, device=dev)
     v = SpecVerify(_p(p), _p(q), _p(draft), n_seq, n_pos, V, _p(seed), _p(step0), rng, _p(out), _p(nacc), _p(flags), None, 0,
                    tol)
+    if split:
+        if workspace is None:
+            need = int(lib().ws_spec_verify_workspace(C.byref(v)))
+            workspace = torch.zeros(need, dtype=torch.uint8, device=dev) if need else None
+        if workspace is not None:
+            v.workspace, v.workspace_bytes = _p(workspace), workspace.numel()
     check(lib().ws_spec_verify_classic(_stream(), C.byref(v)), "ws_spec_verify_classic")
     return nacc, out, flags
 

@@ -460,8 +460,8 @@ int ws_history_stage(void* stream, const ws_history_stage_args* b) {
     return done();
 }
 
-uint64_t ws_spec_verify_workspace(const ws_spec_verify* v) { return ws::spec_workspace(v); }
+uint64_t ws_spec_verify_workspace(const ws_spec_verify* v) { return ws::spec_workspace(v, compute_units()); }
 
-int ws_spec_verify_classic(void* stream, const ws_spec_verify* v) { return ws::spec_launch(S(stream), v); }
+int ws_spec_verify_classic(void* stream, const ws_spec_verify* v) { return ws::spec_launch(S(stream), v, compute_units()); }
 
 }  // extern "C"

@@ -3,7 +3,10 @@
 // The reference removed this rule (include/whirl/spec_sample.h:22-24); the result is defined by the closed form
 // in include/whirl_sampling_abi.h. One workgroup per sequence: the accept chain needs 2 gathers per draft, the
 // resample streams exactly one row pair once (per-256-element sums in id order kept in LDS, a scan over them,
-// and a re-read of the one 1 KiB step the draw lands in).
+// and a re-read of the one 1 KiB step the draw lands in). With fewer sequences than compute units and a workspace a
+// sequence is split over 2 to 16 workgroups: every part runs the accept chain (same answer everywhere), sums its share
+// of the steps and leaves the sums in the workspace; the part that arrives last collects them all and goes on as the
+// one workgroup does - the same sums added in the same order, so the same token to the last bit.
 #pragma once
 
 #include "../../include/whirl_sampling_abi.h"
@@ -27,14 +30,18 @@ struct SpecArgs {
     int32_t* n_accepted;
     uint32_t* flags;
     double tol;
+    uint32_t split_log2;  // parts per sequence, as a power of two (0: one workgroup per sequence)
+    unsigned char* work;  // split sequences: per sequence kSpecMaxSteps step sums and an arrival counter (spec_seq_bytes)
 };
+constexpr uint64_t spec_seq_bytes = kSpecMaxSteps * 8ull + 256ull;
 
 __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     __shared__ double step_sum[kSpecMaxSteps];
     __shared__ double red_d[WS_WAVES];
     __shared__ uint32_t s_u[4];
     __shared__ double s_d[4];
-    const uint32_t s = blockIdx.x, t = threadIdx.x, V = A.vocab, P = A.n_pos;
+    const uint32_t n_parts = 1u << A.split_log2;
+    const uint32_t s = blockIdx.x >> A.split_log2, part = blockIdx.x & (n_parts - 1u), t = threadIdx.x, V = A.vocab, P = A.n_pos;
     const float* p = A.p + static_cast<size_t>(s) * P * V;
     const float* q = A.q + static_cast<size_t>(s) * P * V;
     const int32_t* dr = A.draft + static_cast<size_t>(s) * (P - 1);
@@ -64,7 +71,7 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
             const uint64_t tested = j >= 63u ? ~0ull : (2ull << j) - 1ull;  // drafts 0..j were looked at (j = P - 1: none there)
             const uint64_t nears = __ballot(near) & tested;
             const uint64_t bads = __ballot(bad) & tested;
-            if (t < j) out[t] = d;
+            if (t < j && part == 0u) out[t] = d;
             if (t == 0) {
                 s_u[0] = j;
                 s_u[1] = (nears ? kSpecNear : 0u) | (bads ? kSpecBadDraft : 0u);
@@ -82,7 +89,7 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
             const double lhs = batch_uniform(A.rng, seed, s, step0 + j, 0) * qj;
             if (fabs(lhs - pj) < A.tol * pj) fl |= kSpecNear;
             if (!(lhs < pj)) break;
-            out[j] = d;
+            if (part == 0u) out[j] = d;
         }
         s_u[0] = j;
         s_u[1] = fl;
@@ -96,25 +103,30 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     const uint32_t w = wave_id(), l = lane_id();
     bool from_p = j + 1 == P;
     double total = 0;
-    for (int attempt = 0; attempt < 2; ++attempt) {
-        // weights in id order: step k covers ids [256k, 256k + 256), lane l the four ids 256k + 4l ..
+    // weights in id order: step k covers ids [256k, 256k + 256), lane l the four ids 256k + 4l ..; the steps [k_lo, k_hi)
+    auto sweep = [&](uint32_t k_lo, uint32_t k_hi) {
         const bool aligned = (reinterpret_cast<uintptr_t>(pr) & 15u) == 0 && (reinterpret_cast<uintptr_t>(qr) & 15u) == 0;
-        // whole aligned steps, kS of a wave at a time: their loads go out together (one step at a time is one trip to
-        // memory per step and wave)
-        constexpr uint32_t kS = 4;
-        const uint32_t whole = aligned ? V >> 8 : 0u;  // steps of 256 ids that lie inside the row
-        uint32_t k_next = w;
-        for (; k_next + (kS - 1u) * WS_WAVES < whole; k_next += kS * WS_WAVES) {
+        // whole aligned steps, up to kS of a wave at a time: their loads go out together (one step at a time is one trip
+        // to memory per step and wave)
+        constexpr uint32_t kS = 8;
+        const uint32_t whole = min(aligned ? V >> 8 : 0u, k_hi);  // steps of 256 ids that lie inside the row
+        uint32_t k_next = k_lo + w;
+        for (; k_next < whole; k_next += kS * WS_WAVES) {
             float4 a[kS], b[kS];
 #pragma unroll
             for (uint32_t u = 0; u < kS; ++u) {
-                const uint32_t i = ((k_next + u * WS_WAVES) << 8) + 4u * l;
-                a[u] = *reinterpret_cast<const float4*>(pr + i);
-                b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (!from_p) b[u] = *reinterpret_cast<const float4*>(qr + i);
+                const uint32_t k = k_next + u * WS_WAVES;  // (the same for the whole wave)
+                const uint32_t i = (k << 8) + 4u * l;
+                a[u] = b[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (k < whole) {
+                    a[u] = *reinterpret_cast<const float4*>(pr + i);
+                    if (!from_p) b[u] = *reinterpret_cast<const float4*>(qr + i);
+                }
             }
 #pragma unroll
             for (uint32_t u = 0; u < kS; ++u) {
+                const uint32_t k = k_next + u * WS_WAVES;
+                if (k >= whole) break;
                 const float r0 = a[u].x - b[u].x, r1 = a[u].y - b[u].y, r2 = a[u].z - b[u].z, r3 = a[u].w - b[u].w;
                 double acc = 0;
                 acc += r0 > 0.f ? static_cast<double>(r0) : 0.0;
@@ -122,10 +134,13 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
                 acc += r2 > 0.f ? static_cast<double>(r2) : 0.0;
                 acc += r3 > 0.f ? static_cast<double>(r3) : 0.0;
                 acc = wave_sum(acc);
-                if (l == 0) step_sum[k_next + u * WS_WAVES] = acc;
+                if (l == 0) step_sum[k] = acc;
             }
         }
-        for (uint32_t k = k_next; k < n_steps; k += WS_WAVES) {
+        // what is left of the wave's steps: the row's last, partial step, or every step of an unaligned row
+        uint32_t k_rest = k_lo + w;
+        if (k_rest < whole) k_rest += (whole - k_rest + WS_WAVES - 1u) / WS_WAVES * WS_WAVES;
+        for (uint32_t k = k_rest; k < k_hi; k += WS_WAVES) {
             const uint32_t i = (k << 8) + 4u * l;
             double acc = 0;
             if (i + 3 < V && aligned) {
@@ -146,6 +161,31 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
             acc = wave_sum(acc);
             if (l == 0) step_sum[k] = acc;
         }
+    };
+    const uint32_t per_part = (n_steps + n_parts - 1u) >> A.split_log2;
+    const uint32_t k_lo = min(part * per_part, n_steps), k_hi = min(k_lo + per_part, n_steps);
+    sweep(k_lo, k_hi);
+    if (n_parts > 1u) {
+        // the parts meet: sums out (stores and loads that go to the memory every compute unit sees), then the arrival
+        // counter; whoever finds all the others there already collects their sums and goes on alone
+        unsigned long long* gsum = reinterpret_cast<unsigned long long*>(A.work + static_cast<size_t>(s) * spec_seq_bytes);
+        uint32_t* arrive = reinterpret_cast<uint32_t*>(gsum + kSpecMaxSteps);
+        __syncthreads();
+        for (uint32_t k = k_lo + t; k < k_hi; k += WS_BLOCK)
+            __hip_atomic_store(&gsum[k], static_cast<unsigned long long>(__double_as_longlong(step_sum[k])), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's sums have arrived
+        __syncthreads();
+        if (t == 0) s_u[3] = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (no fence: the sums above went out as atomic stores and have been acknowledged, and are read back the same way)
+        __syncthreads();
+        if (s_u[3] != n_parts - 1u) return;
+        if (t == 0) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // as the next launch needs it
+        for (uint32_t k = t; k < n_steps; k += WS_BLOCK)
+            if (k < k_lo || k >= k_hi)
+                step_sum[k] = __longlong_as_double(static_cast<long long>(__hip_atomic_load(&gsum[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+    }
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        if (attempt == 1) sweep(0u, n_steps);  // (zero residual: the whole of p, by this workgroup alone)
         __syncthreads();
         // scan of the step sums: thread t owns steps 4t .. 4t+3
         double loc[4], lsum = 0;
@@ -234,16 +274,34 @@ __global__ void __launch_bounds__(WS_BLOCK) spec_verify_kernel(SpecArgs A) {
     }
 }
 
-inline uint64_t spec_workspace(const ws_spec_verify*) { return 0; }
+// parts per sequence that pay: the launch stays within the compute units, a part has at least 32 steps (8192 ids)
+inline uint32_t spec_split_log2(const ws_spec_verify* v, int compute_units) {
+    if (!v || v->n_seq == 0 || v->vocab == 0) return 0u;
+    const uint32_t n_steps = (v->vocab + 255u) >> 8;
+    uint32_t lg = 0;
+    while (lg < 4u && (static_cast<uint64_t>(v->n_seq) << (lg + 1u)) <= static_cast<uint64_t>(compute_units > 0 ? compute_units : 0) &&
+           (n_steps >> (lg + 1u)) >= 32u)
+        ++lg;
+    return lg;
+}
+inline uint64_t spec_workspace(const ws_spec_verify* v, int compute_units) {
+    return spec_split_log2(v, compute_units) ? static_cast<uint64_t>(v->n_seq) * spec_seq_bytes : 0ull;
+}
 
-inline int spec_launch(hipStream_t stream, const ws_spec_verify* v) {
+inline int spec_launch(hipStream_t stream, const ws_spec_verify* v, int compute_units) {
     if (!v || !v->p || !v->q || !v->seed || !v->step0 || !v->out_tokens || !v->n_accepted || !v->flags) return WS_E_INVALID;
     if (!v->draft && v->n_pos > 1) return WS_E_INVALID;  // one position: no draft to test, the token comes from p
     if (v->n_seq == 0 || v->n_pos < 1 || v->vocab == 0 || v->vocab > kSpecMaxSteps * 256u) return WS_E_INVALID;
     if (v->rng != WS_RNG_SPLITMIX && v->rng != WS_RNG_PHILOX) return WS_E_INVALID;
     SpecArgs a{v->p, v->q, v->draft, v->n_seq, v->n_pos, v->vocab, v->seed, v->step0, v->rng, v->out_tokens, v->n_accepted,
-               v->flags, v->tol > 0 ? v->tol : 1.0 / 1099511627776.0};
-    hipLaunchKernelGGL(spec_verify_kernel, dim3(v->n_seq), dim3(WS_BLOCK), 0, stream, a);
+               v->flags, v->tol > 0 ? v->tol : 1.0 / 1099511627776.0, 0u, nullptr};
+    const uint32_t lg = spec_split_log2(v, compute_units);
+    if (lg && v->workspace && v->workspace_bytes >= static_cast<uint64_t>(v->n_seq) * spec_seq_bytes &&
+        reinterpret_cast<uintptr_t>(v->workspace) % 8u == 0) {
+        a.split_log2 = lg;
+        a.work = static_cast<unsigned char*>(v->workspace);
+    }
+    hipLaunchKernelGGL(spec_verify_kernel, dim3(v->n_seq << a.split_log2), dim3(WS_BLOCK), 0, stream, a);
     return static_cast<int>(hipGetLastError());
 }
 
