@@ -94,6 +94,16 @@ int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, cons
  * atomics; here both are fixed: ties at the cut keep the lowest token ids, entries are in ascending id order.
  * Output layout as the engine's buffers expect it (src/server/engine_sampling.cpp:37-43). */
 int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows);
+/* ws_topk_rows with a workspace, for the engine's batches of 1 to 32 rows (same launch site; the reference gives every
+ * row to one workgroup, which leaves most of a large GPU idle): with K <= 512, rows of whole aligned 128-bit vectors and
+ * fewer rows than half the compute units, each row is shared by 2 to 16 workgroups that meet in the workspace. Same
+ * ids and vals, same maximum; the normaliser is summed in another order (same 2e-6 bound). workspace: device memory of
+ * ws_topk_rows_workspace() bytes (0: this shape is not split), 8-byte aligned, zero-filled once before its first use
+ * and left alone afterwards; one launch at a time per workspace. Without one, or for shapes that are not split, this
+ * is ws_topk_rows. */
+uint64_t ws_topk_rows_workspace(int n, int K, unsigned rows);
+int ws_topk_rows_ws(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows,
+                    void* workspace, uint64_t workspace_bytes);
 /* dflash_topk(x, n, ld, k, ids, vals): kernels/dflash.hip:36-77; launch site src/model/dflash.cpp:302 (the drafter's
  * candidates per draft position). ids / vals[row][0..k) = the k <= 64 largest logits of row `row` (rows ld floats apart)
  * in key order: larger value first, then smaller index; NaN counts as -inf and is written out as it stands. The

@@ -243,3 +243,74 @@ def test_adjust_rows_matches_the_oracle_bit_for_bit():
             lib.wo_apply_penalties(wo._ptr(x), c["V"], wo._ptr(allow) if allow is not None else None, wo._ptr(hist), hist.size,
                                    c["rep"][r], c["pres"][r], c["freq"][r], wo._ptr(bi), wo._ptr(bv), bi.size)
             assert got[r].tobytes() == x.tobytes(), (c["name"], r)
+
+
+def _topk_pair(x, K, inv_t, launches=2):
+    """topk_rows with every row shared by several workgroups against the one-workgroup kernel, launch after launch on
+    one workspace: ids, values and the maximum bit for bit, the normaliser to 2e-6 of a double-precision sum."""
+    m = gpu_cases.pkg()
+    rows, n = x.shape
+    work = m.topk_rows_workspace(n, K, rows)
+    assert work is not None, "this shape is meant to be split"
+    dx = torch.from_numpy(x).to(DEV)
+    want = [a.cpu().numpy() for a in m.topk_rows(dx, K, inv_t)]
+    for launch in range(launches):
+        got = [a.cpu().numpy() for a in m.topk_rows(dx, K, inv_t, workspace=work)]
+        assert np.array_equal(got[0], want[0]), (launch, K)
+        assert got[1].tobytes() == want[1].tobytes(), (launch, K)
+        assert np.array_equal(got[2][:, 0], want[2][:, 0]), (launch, K)
+        for r in range(rows):
+            xr = np.where(np.isnan(x[r]), -np.inf, x[r]).astype(np.float64)
+            if np.isfinite(xr.max()):
+                truth = np.exp((xr - xr.max()) * float(np.float32(inv_t))).sum()
+                assert abs(got[2][r, 1] - truth) <= 2e-6 * truth, (launch, K, r, got[2][r, 1], truth)
+    ctrl = work.view(rows, -1)[:, 2048 * 8:2048 * 8 + 12]
+    assert not ctrl.any().item(), "the meeting's counters are not back at zero"
+    return want
+
+
+@pytest.mark.parametrize("rows,K", [(1, 256), (8, 40), (32, 256), (5, 512), (3, 1)])
+def test_topk_rows_shared_between_workgroups(rows, K):
+    rng = np.random.default_rng(330 + rows)
+    x = (rng.standard_normal((rows, 151936)) * 2).astype(np.float32)
+    ids, vals, _ = _topk_pair(x, K, 1.0 / 0.7)
+    for r in range(rows):
+        order = np.lexsort((np.arange(x.shape[1]), -x[r].astype(np.float64)))[:K]
+        assert np.array_equal(ids[r], np.sort(order))
+
+
+def test_topk_rows_shared_rows_that_leave_the_short_list_route():
+    """Row 0: the largest logits all in one wave's stretch of one part (its list overflows: counted in full by the last
+    part); row 1: an outlier far above the head of the row, in the last part (the bound from the head does not hold);
+    row 2: quarter-rounded logits, thousands tie at the cut; row 3: 90 % -inf; row 4: NaN stretches; row 5: a constant row."""
+    rng = np.random.default_rng(331)
+    n = 151936
+    x = (rng.standard_normal((6, n)) * 2).astype(np.float32)
+    x[0, 100000:100200] = 20.0 + np.arange(200, dtype=np.float32) * 0.01
+    x[1, n - 5] += 60.0
+    x[2] = np.round(x[2] * 4) / 4
+    x[3, rng.random(n) < 0.9] = -np.inf
+    x[4, rng.random(n) < 0.3] = np.nan
+    x[5, :] = 0.25
+    for K, inv_t in ((256, 1.0), (64, 2.0), (512, 0.5)):
+        ids, vals, _ = _topk_pair(x, K, inv_t)
+        for r in range(6):
+            xr = np.where(np.isnan(x[r]), -np.inf, x[r]).astype(np.float32)
+            order = np.lexsort((np.arange(n), -xr.astype(np.float64)))[:K]
+            assert np.array_equal(ids[r], np.sort(order)), (K, r)
+
+
+def test_topk_rows_ws_falls_back_for_shapes_it_does_not_split():
+    m = gpu_cases.pkg()
+    assert m.topk_rows_workspace(151936, 16384, 4) is None   # a long list: the multi-pass route
+    assert m.topk_rows_workspace(151937, 256, 4) is None     # rows that are not whole vectors
+    assert m.topk_rows_workspace(151936, 256, 200) is None   # enough rows for every compute unit
+    assert m.topk_rows_workspace(20000, 256, 4) is None      # short rows
+    rng = np.random.default_rng(332)
+    x = (rng.standard_normal((4, 20000)) * 2).astype(np.float32)
+    dx = torch.from_numpy(x).to(DEV)
+    spare = torch.zeros(4 * 16640, dtype=torch.uint8, device=DEV)
+    a = [t.cpu().numpy() for t in m.topk_rows(dx, 256, 1.0)]
+    b = [t.cpu().numpy() for t in m.topk_rows(dx, 256, 1.0, workspace=spare)]
+    for p, q in zip(a, b):
+        assert p.tobytes() == q.tobytes()

@@ -116,6 +116,9 @@ ABI = {
                                        C.POINTER(DSampArgs), C.c_void_p, C.c_uint]),
     "ws_topk_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_uint]),
+    "ws_topk_rows_workspace": (C.c_uint64, [C.c_int, C.c_int, C.c_uint]),
+    "ws_topk_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
+                                  C.c_uint, C.c_void_p, C.c_uint64]),
     "ws_dflash_topk": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
@@ -227,15 +230,27 @@ def draft_sample_rows(x, ctl_all, area, r, args, qbuf, vmap=None):
                                      _p(qbuf), x.shape[0]), "ws_draft_sample_rows")
 
 
-def topk_rows(x, K, inv_t):
-    """x: [rows, n] -> ids int32 [rows, K] (ascending id), vals float32 [rows, K], stats float32 [rows, 2]."""
+def topk_rows(x, K, inv_t, workspace=None):
+    """x: [rows, n] -> ids int32 [rows, K] (ascending id), vals float32 [rows, K], stats float32 [rows, 2].
+    workspace: a zero-filled uint8 device tensor of ws_topk_rows_workspace bytes kept between calls - small batches then
+    share each row between several workgroups (ws_topk_rows_ws)."""
     _dev_f32(x)
     rows = x.shape[0]
     ids = torch.full((rows, K), -1, dtype=torch.int32, device=x.device)
     vals = torch.zeros((rows, K), dtype=torch.float32, device=x.device)
     stats = torch.empty((rows, 2), dtype=torch.float32, device=x.device)
-    check(lib().ws_topk_rows(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows), "ws_topk_rows")
+    if workspace is not None:
+        check(lib().ws_topk_rows_ws(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows, _p(workspace),
+                                    workspace.numel()), "ws_topk_rows_ws")
+    else:
+        check(lib().ws_topk_rows(_stream(), _p(x), x.shape[1], K, inv_t, _p(ids), _p(vals), _p(stats), rows), "ws_topk_rows")
     return ids, vals, stats
+
+
+def topk_rows_workspace(n, K, rows, device="cuda:0"):
+    """Zero-filled workspace for topk_rows on this shape, None when the shape is not split."""
+    need = int(lib().ws_topk_rows_workspace(n, K, rows))
+    return torch.zeros(need, dtype=torch.uint8, device=device) if need else None
 
 
 def dflash_topk(x, k):

@@ -252,6 +252,34 @@ int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* i
     return done();
 }
 
+namespace {
+// parts per row that pay for ws_topk_rows_ws: a short list (the route that needs no second pass), whole aligned vectors,
+// the launch within the compute units, at least 16384 tokens a part
+unsigned topk_split_log2(const float* x, int n, int K, unsigned rows) {
+    if (K > static_cast<int>(ws::kTopkCap / 4u) || (n & 3) != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0) return 0u;
+    const uint64_t cus = static_cast<uint64_t>(compute_units());
+    unsigned lg = 0;
+    while (lg < 4u && (static_cast<uint64_t>(rows) << (lg + 1u)) <= cus && (n >> (lg + 1u)) >= 16384) ++lg;
+    return lg;
+}
+}  // namespace
+
+uint64_t ws_topk_rows_workspace(int n, int K, unsigned rows) {
+    // (the row pointer's alignment is looked at when the launch comes; an aligned one is assumed here)
+    return topk_split_log2(nullptr, n, K, rows) ? uint64_t{rows} * ws::kTopkSplitRowBytes : 0ull;
+}
+
+int ws_topk_rows_ws(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows,
+                    void* workspace, uint64_t workspace_bytes) {
+    if (!x || !ids || !vals || !stats || n <= 0 || K <= 0 || rows == 0) return WS_E_INVALID;
+    const unsigned lg = topk_split_log2(x, n, K, rows);
+    if (!lg || !workspace || workspace_bytes < uint64_t{rows} * ws::kTopkSplitRowBytes || reinterpret_cast<uintptr_t>(workspace) % 8u != 0)
+        return ws_topk_rows(stream, x, n, K, inv_t, ids, vals, stats, rows);
+    hipLaunchKernelGGL(topk_rows_split, dim3(rows << lg), dim3(WS_BLOCK), 0, S(stream), x, n, K, inv_t, ids, vals, stats, lg,
+                       static_cast<unsigned char*>(workspace));
+    return done();
+}
+
 int ws_dflash_topk(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows) {
     if (!x || !ids || !vals || n <= 0 || ld < n || k <= 0 || k > 64 || rows == 0) return WS_E_INVALID;
     hipLaunchKernelGGL(dflash_topk, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, ld, k, ids, vals);

@@ -125,7 +125,8 @@ __device__ __forceinline__ uint32_t topk_bin(float v, float scale, float a32, fl
 // SUM false: only the maximum is tracked (a caller that wants no normaliser: the exponentials are a third of the pass).
 template <bool COUNT, bool SUM = true>
 __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int n, float inv_t, float scale, float a32, uint32_t* hist,
-                                                int list_bin, uint64_t* list, uint32_t* n_list, float ref, float& m, float& s) {
+                                                int list_bin, uint64_t* list, uint32_t* n_list, float ref, float& m, float& s,
+                                                uint32_t id0 = 0u) {  // id0: the token id of x[0] (a slice of a row)
     const float tail = static_cast<float>(kTopkTail + lane_id());
     const float k2 = inv_t * 1.4426950408889634f;  // exp((v - m) * inv_t) = 2^((v - m) * k2)
     const bool fixed = ref == ref;  // uniform
@@ -140,7 +141,7 @@ __device__ __forceinline__ void topk_first_pass(const float* __restrict__ x, int
         } else if (static_cast<int>(b) <= list_bin) {  // a few per thousand tokens
             atomicAdd(&hist[b], 1u);
             const uint32_t slot = atomicAdd(&n_list[wave_id()], 1u);
-            if (slot < kTopkWaveCap) list[wave_id() * kTopkWaveCap + slot] = key64(v, static_cast<uint32_t>(i));
+            if (slot < kTopkWaveCap) list[wave_id() * kTopkWaveCap + slot] = key64(v, id0 + static_cast<uint32_t>(i));
         }
     };
     // Every term is 2^(fma(v, k2, -mk)) with mk the ROUNDED product reference * k2: one instruction for the exponent,
@@ -433,8 +434,22 @@ __device__ __forceinline__ bool topk_by_counts(const float* __restrict__ x, int 
 
 // The K largest logits of one row (x, n tokens) into ids / vals in ascending id order, ties at the cut to the lowest ids;
 // stats (unless null) = {max, sum exp((x - max) * inv_t)}. Every return is taken by the whole workgroup.
+// A row shared by several workgroups (few rows, a short list: K up to kTopkCap / 4): every part takes the bound, the
+// bins and the listing threshold from the head of the row (the same for all), runs the first pass over its slice,
+// and leaves its listed tokens, its maximum and its sum (against the common reference) in the row's workspace; the part
+// that arrives last takes them all and goes on as the one workgroup does with the same list - so the same ids and
+// values; the normaliser is the sum of the parts' sums. Rows the short-list route does not take are done by part 0 alone.
+// Workspace of a row: kTopkCap keys, then 64 words: [0] parts arrived, [1] tokens listed, [2] a wave's stretch of the
+// list overflowed, [16 + 2 p], [17 + 2 p] maximum and sum of part p. Zero-filled once; every launch leaves [0..2] at zero.
+constexpr uint64_t kTopkSplitRowBytes = kTopkCap * 8ull + 256ull;
+struct TopkSplit {
+    uint32_t parts = 1u, part = 0u;
+    unsigned char* work = nullptr;  // of this row
+};
+
 template <bool SUM = true>
-__device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
+__device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats,
+                                             TopkSplit sp = TopkSplit{}) {
     __shared__ __align__(16) uint32_t hist[4096];  // also viewed as 64- and 128-bit words
     __shared__ uint64_t cand[ws::kTopkCap];
     __shared__ float red_f[WS_WAVES];
@@ -508,8 +523,78 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
     // the maximum between the two: terms up to e^(8 inv_t), which a float holds for temperatures above 1 / 8)
     const float nan = __uint_as_float(0x7fc00000u);
     const float ref = (counted && inv_t > 0.f && inv_t <= 8.f) ? bound - 8.f : nan;
-    if (counted) ws::topk_first_pass<true, SUM>(x, n, inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s);
-    else ws::topk_first_pass<false, SUM>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
+    bool split = sp.parts > 1u;
+    if (split && !(SUM && counted && list_bin >= 0 && ref == ref)) {  // (every part sees the same head: the same answer)
+        if (sp.part != 0u) return;
+        split = false;
+    }
+    if (split) {
+        __shared__ uint32_t s_meet[4];
+        const uint32_t t = threadIdx.x, w = ws::wave_id(), l = ws::lane_id();
+        const int nv_all = n >> 2, per = (nv_all + static_cast<int>(sp.parts) - 1) / static_cast<int>(sp.parts);
+        const int v0 = min(static_cast<int>(sp.part) * per, nv_all), v1 = min(v0 + per, nv_all);
+        ws::topk_first_pass<true, SUM>(x + 4 * v0, 4 * (v1 - v0), inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s,
+                                       static_cast<uint32_t>(4 * v0));
+        __syncthreads();  // the wave lists and their counters are complete
+        const float top_p = ws::block_max(m, red_f);
+        const float sum_p = ws::block_sum(s, red_f);  // against ref, like every part's
+        unsigned long long* glist = reinterpret_cast<unsigned long long*>(sp.work);
+        uint32_t* ctrl = reinterpret_cast<uint32_t*>(sp.work + ws::kTopkCap * 8ull);
+        {
+            // this wave's stretch of the list goes to the row's common list (stores and loads that every compute unit
+            // sees; acknowledged before the arrival counter is touched, so no cache write-back is needed)
+            const uint32_t mine = s_wn[w], cnt = min(mine, ws::kTopkWaveCap);
+            uint32_t base = 0;
+            if (l == 0 && cnt) base = __hip_atomic_fetch_add(&ctrl[1], cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            base = static_cast<uint32_t>(__shfl(static_cast<int>(base), 0));
+            for (uint32_t e = l; e < cnt; e += 64u)
+                if (base + e < ws::kTopkCap)
+                    __hip_atomic_store(&glist[base + e], static_cast<unsigned long long>(cand[w * ws::kTopkWaveCap + e]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            if (l == 0 && mine > ws::kTopkWaveCap) __hip_atomic_fetch_or(&ctrl[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (t == 0) {
+                __hip_atomic_store(&ctrl[16u + 2u * sp.part], __float_as_uint(top_p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&ctrl[17u + 2u * sp.part], __float_as_uint(sum_p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t == 0) s_meet[0] = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_meet[0] != sp.parts - 1u) return;
+        // the last one to arrive: everything is there
+        const uint32_t total = __hip_atomic_load(&ctrl[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t over = __hip_atomic_load(&ctrl[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float top_all = -INFINITY, sum_all = 0.f;
+        for (uint32_t p = 0; p < sp.parts; ++p) {  // (every thread, in part order: the same sum everywhere)
+            top_all = fmaxf(top_all, __uint_as_float(__hip_atomic_load(&ctrl[16u + 2u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+            sum_all += __uint_as_float(__hip_atomic_load(&ctrl[17u + 2u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        }
+        __syncthreads();  // every thread has read the counters
+        if (t < 3) __hip_atomic_store(&ctrl[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // as the next launch needs them
+        const bool whole = !over && total <= ws::kTopkCap;
+        for (int b = t; b < ws::kTopkBins; b += WS_BLOCK) hist[b] = 0u;
+        if (t < WS_WAVES) {
+            const uint32_t before = t * ws::kTopkWaveCap;
+            // the common list as one stretch after the other; an overflow shows as a stretch that is too long (the row is then counted in full)
+            s_wn[t] = whole ? (total > before ? min(total - before, ws::kTopkWaveCap) : 0u) : (t == 0 ? ws::kTopkWaveCap + 1u : 0u);
+        }
+        __syncthreads();
+        if (whole) {
+            for (uint32_t i = t; i < total; i += WS_BLOCK) {
+                const uint64_t k = __hip_atomic_load(&glist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                cand[i] = k;
+                atomicAdd(&hist[ws::topk_bin(ws::unkey32(static_cast<uint32_t>(k >> 32)), scale, a32, 4095.f)], 1u);  // the counts of the listed bins
+            }
+        }
+        m = top_all;
+        s = t == 0 ? sum_all : 0.f;
+        __syncthreads();
+    } else if (counted) {
+        ws::topk_first_pass<true, SUM>(x, n, inv_t, scale, a32, hist, list_bin, cand, s_wn, ref, m, s);
+    } else {
+        ws::topk_first_pass<false, SUM>(x, n, inv_t, scale, a32, hist, -1, cand, s_wn, nan, m, s);
+    }
     const float top = ws::block_max(m, red_f);
     if (SUM && ref == ref && !(top <= bound)) {  // uniform: the maximum beats the bound - the sum may have overflowed: once more, the other way
         m = -INFINITY;
@@ -572,6 +657,18 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     topk_rows(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats) {
     const size_t row = blockIdx.x;
     ws::topk_one_row(x + row * n, n, K, inv_t, ids + row * K, vals + row * K, stats + 2 * row);
+}
+
+// topk_rows with every row shared by 1 << split_log2 consecutive workgroups (no counterpart in the reference, whose
+// kernel gives a row to one workgroup; ws_topk_rows_ws launches it for small batches)
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    topk_rows_split(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned split_log2, unsigned char* work) {
+    const size_t row = blockIdx.x >> split_log2;
+    ws::TopkSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x & (sp.parts - 1u);
+    sp.work = work + row * ws::kTopkSplitRowBytes;
+    ws::topk_one_row(x + row * n, n, K, inv_t, ids + row * K, vals + row * K, stats + 2 * row, sp);
 }
 
 // dflash_topk(x, n, ld, k, ids, vals) of kernels/dflash.hip:36-77: the k <= 64 largest logits of each row in key order

@@ -93,6 +93,11 @@ struct DeviceRows::Dev {
     float* topk_vals = nullptr;
     float* topk_stats = nullptr;
     float* adjusted = nullptr;         // escalation: penalised copy of the row (ws_adjust_rows)
+    // The sampler's workspace: with it a batch of a few rows has each row worked on by several workgroups, and long
+    // vocabularies take the history tokens' logits from the sweep. Zero-filled when it is allocated: what it is used for
+    // depends on the vocabulary alone, which this object never changes, and the use that needs zeros puts them back.
+    unsigned char* work = nullptr;
+    std::uint64_t work_cap = 0;
     std::vector<unsigned char> h_prm, h_res;
     std::vector<std::int32_t> h_ids;
     std::vector<float> h_vals;
@@ -118,7 +123,7 @@ DeviceRows::~DeviceRows() {
     for (void* p : {static_cast<void*>(dev_->prm), static_cast<void*>(dev_->res), static_cast<void*>(dev_->kept_ids),
                     static_cast<void*>(dev_->kept_logits), static_cast<void*>(dev_->hist), static_cast<void*>(dev_->bias_ids),
                     static_cast<void*>(dev_->bias_vals), static_cast<void*>(dev_->topk_ids), static_cast<void*>(dev_->topk_vals),
-                    static_cast<void*>(dev_->topk_stats), static_cast<void*>(dev_->adjusted)})
+                    static_cast<void*>(dev_->topk_stats), static_cast<void*>(dev_->adjusted), static_cast<void*>(dev_->work)})
         if (p) (void)hipFree(p);
     delete dev_;
 }
@@ -244,6 +249,16 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
     b.kept_logits = d.kept_logits;
     b.kept_cap = cap;
     b.mode = WS_MODE_AUTO;
+    if (const std::uint64_t need = ws_sample_batch_workspace(&b); need > d.work_cap) {
+        if (d.work) (void)hipFree(d.work);
+        d.work = nullptr;
+        d.work_cap = 0;
+        checkHip(hipMalloc(reinterpret_cast<void**>(&d.work), need), "hipMalloc");
+        d.work_cap = need;
+        checkHip(hipMemsetAsync(d.work, 0, need, stream), "hipMemsetAsync");
+    }
+    b.workspace = d.work;
+    b.workspace_bytes = d.work_cap;
     check(ws_sample_batch(stream_, &b), "ws_sample_batch");
 
     d.h_res.resize(Dev::resultBytes(n));
