@@ -88,6 +88,15 @@ int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const 
  * from the filtered draft distribution q by the race (argmin E(v) / q(v)) into ctl[16 + r] and write q; rows <= 32. */
 int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
                          const ws_dsamp_args* a, int* qbuf, unsigned rows);
+/* ws_draft_sample_rows with a workspace (same launch site): the draft head's rows come one draft position after the
+ * other, a few rows at a time, so each launch leaves most of the GPU idle and its latency is paid up to 15 times a
+ * cycle; with a workspace each row is shared by 2 to 16 workgroups (as ws_topk_rows_ws, K = 32). Same candidates; the
+ * normaliser is summed in another order, so q's probabilities may differ in their last bits (the reference's own sum
+ * depends on the order of its atomics). workspace: ws_draft_sample_rows_workspace() bytes (0: not split), 8-byte
+ * aligned, zero-filled once, one launch at a time; without it this is ws_draft_sample_rows. */
+uint64_t ws_draft_sample_rows_workspace(int n, unsigned rows);
+int ws_draft_sample_rows_ws(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
+                            const ws_dsamp_args* a, int* qbuf, unsigned rows, void* workspace, uint64_t workspace_bytes);
 /* topk_rows(x, n, K, inv_t, ids, vals, stats): kernels/shared/sample_cand_topk_rows.h:11-98; launch site
  * src/model/qwen35/server_model.cpp:101-107. stats[row] = {max, sum exp((x - max) * inv_t)}, ids / vals[row][0..K) =
  * the K largest logits. The reference leaves their order and the choice among equal values at the cut to its

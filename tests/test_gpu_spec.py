@@ -283,3 +283,44 @@ def test_classic_verify_split_with_an_empty_residual():
         assert np.array_equal(a, b), (a, b)
     assert (want[0] < 3).any()  # some draft was rejected
     check_spec(p, q, draft, seed, step0, 1)
+
+
+def test_draft_sample_rows_shared_between_workgroups():
+    """The draft head's few rows with a workspace: each row is worked on by several workgroups (ws_draft_sample_rows_ws).
+    Against the host statement as above - ids and count of q exact, probabilities to 1e-6, the draw equal to the host race
+    over the written q - launch after launch on one workspace; rows switched off and chains that stopped are left alone;
+    quarter-rounded logits (ties) and a row with an outlier far above its head in one of the later parts."""
+    m = gc.pkg()
+    lib = wo.load("oracle")
+    rng = np.random.default_rng(304)
+    n, rows = 151936, 5
+    work = torch.zeros(int(m.lib().ws_draft_sample_rows_workspace(n, rows)), dtype=torch.uint8, device=DEV)
+    assert work.numel() > 0, "this shape is meant to be split"
+    for case in range(4):
+        r = int(rng.integers(0, 8))
+        x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
+        if case % 2:
+            x = np.round(x * 4) / 4
+        x[2, n - 100] += 50.0
+        tks = [int(v) for v in rng.choice([0, 1, 3, 20, 32, 40], rows)]
+        tps = [float(v) for v in rng.choice([1.0, 0.95, 0.5], rows)]
+        mps = [float(v) for v in rng.choice([0.0, 0.05, 0.3], rows)]
+        its = [float(1 / rng.uniform(0.3, 1.5)) for _ in range(rows)]
+        keys = [lib.wo_race_base(int(rng.integers(1, 1 << 40)), int(rng.integers(0, 1000))) for _ in range(rows)]
+        dx = torch.from_numpy(x).to(DEV)
+        ctl = torch.zeros(rows * 64, dtype=torch.int32, device=DEV)
+        ctl[3 * 64 + 49], ctl[3 * 64 + 48] = 1, 0  # row 3: the chain stopped before r
+        qb = torch.full((rows * m.Q_WORDS,), -7, dtype=torch.int32, device=DEV)
+        args = [dict(on=0 if b == 4 else 1, top_k=tks[b], qoff=b * m.Q_WORDS, inv_t=its[b], top_p=tps[b], min_p=mps[b], key=keys[b])
+                for b in range(rows)]
+        m.draft_sample_rows(dx, ctl, [64 * b for b in range(rows)], r, args, qb, workspace=work)
+        hc, hq = ctl.cpu().numpy(), qb.cpu().numpy()
+        for b in range(3):
+            want = host_q(lib, x[b], np.float32(its[b]), tks[b], tps[b], mps[b])
+            got = wo.QDist()
+            lib.wo_q_from_words(wo._ptr(np.ascontiguousarray(hq[b * m.Q_WORDS:(b + 1) * m.Q_WORDS])), C.byref(got))
+            assert got.n == want.n and list(got.id[:got.n]) == list(want.id[:want.n]), (case, b, tks[b])
+            _close(got, want)
+            assert hc[b * 64 + 16 + r] == lib.wo_sample_race_q(C.byref(got), keys[b]), (case, b)
+        assert (hq[3 * m.Q_WORDS:] == -7).all() and hc[3 * 64 + 16 + r] == 0 and hc[4 * 64 + 16 + r] == 0
+        assert not work.view(rows, -1)[:, 2048 * 8:2048 * 8 + 12].any().item(), "the meeting's counters are not back at zero"

@@ -116,6 +116,9 @@ ABI = {
                                        C.POINTER(DSampArgs), C.c_void_p, C.c_uint]),
     "ws_topk_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_uint]),
+    "ws_draft_sample_rows_workspace": (C.c_uint64, [C.c_int, C.c_uint]),
+    "ws_draft_sample_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_int, C.c_void_p,
+                                          C.POINTER(DSampArgs), C.c_void_p, C.c_uint, C.c_void_p, C.c_uint64]),
     "ws_topk_rows_workspace": (C.c_uint64, [C.c_int, C.c_int, C.c_uint]),
     "ws_topk_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_uint, C.c_void_p, C.c_uint64]),
@@ -216,8 +219,8 @@ def draft_pick_rows(x, ctl_all, area, r, n_min, p_min, vmap=None):
                                    x.shape[0]), "ws_draft_pick_rows")
 
 
-def draft_sample_rows(x, ctl_all, area, r, args, qbuf, vmap=None):
-    """args: list of per-row dicts (on, top_k, qoff, inv_t, top_p, min_p, key)."""
+def draft_sample_rows(x, ctl_all, area, r, args, qbuf, vmap=None, workspace=None):
+    """args: list of per-row dicts (on, top_k, qoff, inv_t, top_p, min_p, key). workspace: as for topk_rows (K = 32)."""
     _dev_f32(x)
     ri, da = RowIdx(), DSampArgs()
     for i, d in enumerate(area):
@@ -226,6 +229,10 @@ def draft_sample_rows(x, ctl_all, area, r, args, qbuf, vmap=None):
         da.on[i], da.top_k[i], da.qoff[i] = a.get("on", 1), a["top_k"], a["qoff"]
         da.inv_t[i], da.top_p[i], da.min_p[i] = a["inv_t"], a["top_p"], a["min_p"]
         da.key_lo[i], da.key_hi[i] = a["key"] & 0xFFFFFFFF, a["key"] >> 32
+    if workspace is not None:
+        check(lib().ws_draft_sample_rows_ws(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, _p(vmap), C.byref(da),
+                                            _p(qbuf), x.shape[0], _p(workspace), workspace.numel()), "ws_draft_sample_rows_ws")
+        return
     check(lib().ws_draft_sample_rows(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, _p(vmap), C.byref(da),
                                      _p(qbuf), x.shape[0]), "ws_draft_sample_rows")
 

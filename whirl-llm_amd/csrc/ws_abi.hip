@@ -246,6 +246,30 @@ int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, cons
     return done();
 }
 
+namespace {
+unsigned topk_split_log2(const float* x, int n, int K, unsigned rows);
+}
+uint64_t ws_topk_rows_workspace(int n, int K, unsigned rows);
+
+// (the draft sampler lists K <= 32 tokens: it splits like a topk_rows of 32)
+uint64_t ws_draft_sample_rows_workspace(int n, unsigned rows) { return ws_topk_rows_workspace(n, 32, rows); }
+
+int ws_draft_sample_rows_ws(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
+                            const ws_dsamp_args* a, int* qbuf, unsigned rows, void* workspace, uint64_t workspace_bytes) {
+    if (!x || !ctl_all || !area || !a || !qbuf || n <= 0 || r < 0 || r >= 16 || rows == 0 || rows > WS_MAX_TABLE_ROWS)
+        return WS_E_INVALID;
+    const unsigned lg = topk_split_log2(x, n, 32, rows);
+    if (!lg || !workspace || workspace_bytes < uint64_t{rows} * ws::kTopkSplitRowBytes || reinterpret_cast<uintptr_t>(workspace) % 8u != 0)
+        return ws_draft_sample_rows(stream, x, n, ctl_all, area, r, map, a, qbuf, rows);
+    RowIdx ar;
+    DSampArgs da;
+    std::memcpy(&ar, area, sizeof ar);
+    std::memcpy(&da, a, sizeof da);
+    hipLaunchKernelGGL(draft_sample_rows_split, dim3(rows << lg), dim3(WS_BLOCK), 0, S(stream), x, n, ctl_all, ar, r, map, da, qbuf, lg,
+                       static_cast<unsigned char*>(workspace));
+    return done();
+}
+
 int ws_topk_rows(void* stream, const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats, unsigned rows) {
     if (!x || !ids || !vals || !stats || n <= 0 || K <= 0 || rows == 0) return WS_E_INVALID;
     hipLaunchKernelGGL(topk_rows, dim3(rows), dim3(WS_BLOCK), 0, S(stream), x, n, K, inv_t, ids, vals, stats);

@@ -21,13 +21,14 @@ struct DSampArgs {
     unsigned key_hi[32];
 };
 
-extern "C" __global__ void __launch_bounds__(WS_BLOCK)
-    draft_sample_rows(const float* x, int n, int* ctl_all, RowIdx area, int r, const int* map, DSampArgs a, int* qbuf) {
+namespace ws {
+// one row (b: its place in the tables; sp: the row shared by several workgroups, as in topk_rows_split)
+__device__ __forceinline__ void draft_sample_row(const float* x, int n, int* ctl_all, const RowIdx& area, int r, const int* map,
+                                                 const DSampArgs& a, int* qbuf, int b, TopkSplit sp) {
     constexpr int QMAX = 32;
     __shared__ int s_id[QMAX];
     __shared__ float s_lg[QMAX];
     __shared__ float s_stats[2];
-    const int b = blockIdx.x;
     if (a.on[b] == 0) return;
     int* c = ctl_all + area.v[b];
     if (c[49] != 0 && c[48] <= r) return;  // chain stopped by the p-min cutoff at or before r
@@ -38,7 +39,7 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     const float inv_t = a.inv_t[b];
     // one pass over the row: {max, sum exp((x - max) * inv_t)} and the K largest logits in id order, ties at the cut to
     // the lowest ids (the short-list route of topk_rows)
-    ws::topk_one_row(x, n, K, inv_t, s_id, s_lg, s_stats);
+    if (!ws::topk_one_row(x, n, K, inv_t, s_id, s_lg, s_stats, sp)) return;  // (a part of a shared row that is not the last to arrive)
     __syncthreads();
     const float top = s_stats[0], sum = s_stats[1];
     if (threadIdx.x >= 64) return;
@@ -121,4 +122,23 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
         q[1 + lane] = id;
         q[1 + QMAX + lane] = __float_as_int(p);
     }
+}
+}  // namespace ws
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_sample_rows(const float* x, int n, int* ctl_all, RowIdx area, int r, const int* map, DSampArgs a, int* qbuf) {
+    ws::draft_sample_row(x, n, ctl_all, area, r, map, a, qbuf, static_cast<int>(blockIdx.x), ws::TopkSplit{});
+}
+
+// draft_sample_rows with every row shared by 1 << split_log2 consecutive workgroups (no counterpart in the reference;
+// ws_draft_sample_rows_ws launches it: the draft head's rows come one position after the other, a few rows at a time)
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_sample_rows_split(const float* x, int n, int* ctl_all, RowIdx area, int r, const int* map, DSampArgs a, int* qbuf,
+                            unsigned split_log2, unsigned char* work) {
+    const unsigned row = blockIdx.x >> split_log2;
+    ws::TopkSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x & (sp.parts - 1u);
+    sp.work = work + static_cast<size_t>(row) * ws::kTopkSplitRowBytes;
+    ws::draft_sample_row(x, n, ctl_all, area, r, map, a, qbuf, static_cast<int>(row), sp);
 }

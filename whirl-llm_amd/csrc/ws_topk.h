@@ -448,7 +448,7 @@ struct TopkSplit {
 };
 
 template <bool SUM = true>
-__device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats,
+__device__ __forceinline__ bool topk_one_row(const float* x, int n, int K, float inv_t, int* ids, float* vals, float* stats,
                                              TopkSplit sp = TopkSplit{}) {
     __shared__ __align__(16) uint32_t hist[4096];  // also viewed as 64- and 128-bit words
     __shared__ uint64_t cand[ws::kTopkCap];
@@ -525,7 +525,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
     const float ref = (counted && inv_t > 0.f && inv_t <= 8.f) ? bound - 8.f : nan;
     bool split = sp.parts > 1u;
     if (split && !(SUM && counted && list_bin >= 0 && ref == ref)) {  // (every part sees the same head: the same answer)
-        if (sp.part != 0u) return;
+        if (sp.part != 0u) return false;
         split = false;
     }
     if (split) {
@@ -561,7 +561,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
         __syncthreads();
         if (t == 0) s_meet[0] = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (s_meet[0] != sp.parts - 1u) return;
+        if (s_meet[0] != sp.parts - 1u) return false;
         // the last one to arrive: everything is there
         const uint32_t total = __hip_atomic_load(&ctrl[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const uint32_t over = __hip_atomic_load(&ctrl[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -608,7 +608,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
         stats[0] = top;
         stats[1] = sum;
     }
-    if (kk == 0) return;
+    if (kk == 0) return true;
     __syncthreads();  // the counts are complete
 
     int counts_left = counted && top <= bound;  // uniform
@@ -622,7 +622,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
         if (listed >= kk && fits) {  // the K largest are all on the list
             __shared__ uint32_t s_list[4];
             const int rc = ws::topk_from_list(x, cand, s_wn, list_bin, kk, scale, a32, hist, red_u, s_list, ids, vals);
-            if (rc == 0) return;
+            if (rc == 0) return true;
             __syncthreads();
             counts_left = rc == 1;
         }
@@ -638,7 +638,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
     }
     if (counts_left) {
         const ws::TopkLds L{hist, cand, red_f, red_u, s_sel, s_cnt, &s_n, &s_kmin};
-        if (ws::topk_by_counts(x, n, kk, scale, a32, L, ids, vals)) return;
+        if (ws::topk_by_counts(x, n, kk, scale, a32, L, ids, vals)) return true;
         __syncthreads();
     }
 
@@ -649,6 +649,7 @@ __device__ __forceinline__ void topk_one_row(const float* x, int n, int K, float
         ids[o] = i;
         vals[o] = v;
     });
+    return true;
 }
 
 }  // namespace ws
