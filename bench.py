@@ -237,6 +237,11 @@ def reference_kernels(steps):
         for K in (256, 16384):
             timed(f"topk_rows K={K}", rows, lambda: L.ws_topk_rows(S(), P(x), V, K, 1.25, P(ids), P(vals), P(st), rows),
                   rows * (V * 4 + K * 8 + 8))
+        # with the workspace an engine keeps: a row shared between several workgroups
+        work = torch.zeros(max(int(L.ws_topk_rows_workspace(V, 256, rows)), 8), dtype=torch.uint8, device="cuda:0")
+        timed("topk_rows_ws K=256", rows,
+              lambda: L.ws_topk_rows_ws(S(), P(x), V, 256, 1.25, P(ids), P(vals), P(st), rows, P(work), work.numel()),
+              rows * (V * 4 + 256 * 8 + 8))
     x = torch.randn(16, V, device="cuda:0") * 2  # the drafter's candidates: 16 per draft position, 16 positions
     ids = torch.empty((16, 16), dtype=torch.int32, device="cuda:0")
     vals = torch.empty((16, 16), dtype=torch.float32, device="cuda:0")
@@ -254,6 +259,16 @@ def reference_kernels(steps):
             da.key_lo[i], da.key_hi[i] = 12345 + i, 77
         timed("draft_sample_rows", rows,
               lambda: L.ws_draft_sample_rows(S(), P(x), V, P(ctl), C.byref(ri), 0, None, C.byref(da), P(qbuf), rows), rows * V * 4)
+        work = torch.zeros(max(int(L.ws_draft_sample_rows_workspace(V, rows)), 8), dtype=torch.uint8, device="cuda:0")
+        timed("draft_sample_rows_ws", rows,
+              lambda: L.ws_draft_sample_rows_ws(S(), P(x), V, P(ctl), C.byref(ri), 0, None, C.byref(da), P(qbuf), rows, P(work),
+                                                work.numel()), rows * V * 4)
+        # the greedy draft chain's pick (argmax + its probability), one row per sequence
+        work = torch.zeros(max(int(L.ws_draft_pick_workspace(V, rows)), 8), dtype=torch.uint8, device="cuda:0")
+        timed("draft_pick_rows", rows, lambda: L.ws_draft_pick_rows(S(), P(x), V, P(ctl), C.byref(ri), 0, 0, 0.0, None, rows), rows * V * 4)
+        timed("draft_pick_rows_ws", rows,
+              lambda: L.ws_draft_pick_rows_ws(S(), P(x), V, P(ctl), C.byref(ri), 0, 0, 0.0, None, rows, P(work), work.numel()),
+              rows * V * 4)
     x = torch.randn(1, V, device="cuda:0") * 2
     tok = torch.empty(1, dtype=torch.int32, device="cuda:0")
     pr = torch.empty(1, dtype=torch.float32, device="cuda:0")

@@ -84,6 +84,17 @@ int ws_draft_pick(void* stream, const float* x, int n, int* tok, float* prob, in
  * area at ctl_all + area->v[b]; rows <= 32. */
 int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min,
                        float p_min, const int* map, unsigned rows);
+/* ws_draft_pick / ws_draft_pick_rows with a workspace (same launch sites, src/model/qwen35/mtp_verify.cpp:101, 321):
+ * the greedy draft chain launches this once per draft position on one row (or one row per sequence), which leaves the
+ * GPU idle but for one compute unit per row; with a workspace a row is shared by 2 to 16 workgroups. Same token (first
+ * index on ties); the probability's sum is taken in another order (last bits). workspace: ws_draft_pick_workspace()
+ * bytes (256 per row; 0: this shape is not split), 4-byte aligned, zero-filled once, one launch at a time; without it
+ * these are ws_draft_pick / ws_draft_pick_rows. */
+uint64_t ws_draft_pick_workspace(int n, unsigned rows);
+int ws_draft_pick_ws(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
+                     const int* map, void* workspace, uint64_t workspace_bytes);
+int ws_draft_pick_rows_ws(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min,
+                          float p_min, const int* map, unsigned rows, void* workspace, uint64_t workspace_bytes);
 /* draft_sample_rows(x, n, ctl_all, area, r, map, a, qbuf): kernels/spec_sample.hip:34-205. Rows with a->on draw draft r
  * from the filtered draft distribution q by the race (argmin E(v) / q(v)) into ctl[16 + r] and write q; rows <= 32. */
 int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,

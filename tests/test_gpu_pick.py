@@ -314,3 +314,58 @@ def test_topk_rows_ws_falls_back_for_shapes_it_does_not_split():
     b = [t.cpu().numpy() for t in m.topk_rows(dx, 256, 1.0, workspace=spare)]
     for p, q in zip(a, b):
         assert p.tobytes() == q.tobytes()
+
+
+def test_draft_pick_shared_between_workgroups(rows5):
+    """The greedy draft chain with a workspace (ws_draft_pick_ws, ws_draft_pick_rows_ws): each row is read by several
+    workgroups. Same tokens as the one-workgroup kernels (first index on ties, also when the tied maxima sit in different
+    parts; last element; a misaligned row; a row of -inf and NaN), probabilities to 2e-6, the p-min chain cutoff and the
+    vocabulary map as before, launch after launch on one workspace."""
+    m = gpu_cases.pkg()
+    x, dx = rows5
+    rows, n = x.shape
+    w1 = torch.zeros(int(m.lib().ws_draft_pick_workspace(n, 1)), dtype=torch.uint8, device=DEV)
+    assert w1.numel() > 0, "this shape is meant to be split"
+    # the chain of test_draft_pick_chain_and_rows
+    rng = np.random.default_rng(102)
+    lg = rng.standard_normal((3, n)).astype(np.float32)
+    lg[0, 5] = 30.0
+    lg[1, 7] = 4.0
+    lg[2, 9] = 30.0
+    dl = torch.from_numpy(lg).to(DEV)
+    tok = torch.full((16,), 0x7F7F7F7F, dtype=torch.int32, device=DEV)
+    prob = torch.zeros(16, dtype=torch.float32, device=DEV)
+    ctl = torch.zeros(2, dtype=torch.int32, device=DEV)
+    for r in range(3):
+        m.draft_pick(dl[r], tok, prob, ctl, r, 1, 0.5, workspace=w1)
+    t, c, p = tok.cpu().numpy(), ctl.cpu().numpy(), prob.cpu().numpy()
+    assert t[0] == 5 and t[1] == first_max(lg[1]) and t[2] == 0x7F7F7F7F and c[0] == 1 and c[1] == 1
+    for r in range(2):
+        assert abs(p[r] - softmax_top(lg[r])) <= 2e-6 * softmax_top(lg[r]) + 1e-12
+    # rows: ties across parts, last element, map; twice on one workspace
+    wr = torch.zeros(int(m.lib().ws_draft_pick_workspace(n, rows)), dtype=torch.uint8, device=DEV)
+    perm = (100000 + 3 * torch.arange(n, dtype=torch.int32, device=DEV))
+    for launch in range(2):
+        ca = torch.zeros(rows * m.CTL_WORDS, dtype=torch.int32, device=DEV)
+        cb = torch.zeros(rows * m.CTL_WORDS, dtype=torch.int32, device=DEV)
+        area = [m.CTL_WORDS * r for r in range(rows)]
+        m.draft_pick_rows(dx, ca, area, 0, 0, 0.0, perm)
+        m.draft_pick_rows(dx, cb, area, 0, 0, 0.0, perm, workspace=wr)
+        a, b = ca.cpu().numpy(), cb.cpu().numpy()
+        for r in range(rows):
+            o = r * m.CTL_WORDS
+            assert b[o + 16] == a[o + 16] == 100000 + 3 * first_max(x[r]), (launch, r)
+            pa, pb = a[o + 32:o + 33].view(np.float32)[0], b[o + 32:o + 33].view(np.float32)[0]
+            assert abs(pb - softmax_top(x[r])) <= 2e-6 * softmax_top(x[r]) + 1e-12 and abs(pa - pb) <= 4e-6 * pa
+            assert list(b[o + 48:o + 50]) == list(a[o + 48:o + 50])
+    assert not wr.view(rows, -1)[:, :4].any().item() and not w1[:4].any().item(), "arrival counters not back at zero"
+    # a misaligned row of an odd length, and rows without a number in them
+    y = np.round(rng.standard_normal((2, 151937)) * 2, 1).astype(np.float32)
+    dy = torch.from_numpy(y).to(DEV)
+    z = np.full((1, 151936), -np.inf, np.float32)
+    z[0, 77777] = np.nan
+    for src, want in ((dy[1], first_max(y[1])), (torch.from_numpy(z).to(DEV)[0], 0)):
+        tok.fill_(-1)
+        ctl.zero_()
+        m.draft_pick(src, tok, prob, ctl, 0, 0, 0.0, workspace=w1)
+        assert tok.cpu()[0].item() == want

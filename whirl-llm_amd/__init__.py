@@ -116,6 +116,11 @@ ABI = {
                                        C.POINTER(DSampArgs), C.c_void_p, C.c_uint]),
     "ws_topk_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_uint]),
+    "ws_draft_pick_workspace": (C.c_uint64, [C.c_int, C.c_uint]),
+    "ws_draft_pick_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                   C.c_float, C.c_void_p, C.c_void_p, C.c_uint64]),
+    "ws_draft_pick_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_int, C.c_int,
+                                        C.c_float, C.c_void_p, C.c_uint, C.c_void_p, C.c_uint64]),
     "ws_draft_sample_rows_workspace": (C.c_uint64, [C.c_int, C.c_uint]),
     "ws_draft_sample_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(RowIdx), C.c_int, C.c_void_p,
                                           C.POINTER(DSampArgs), C.c_void_p, C.c_uint, C.c_void_p, C.c_uint64]),
@@ -204,17 +209,26 @@ def argmax_prob(x):
     return tok, prob
 
 
-def draft_pick(x, tok, prob, ctl, r, n_min, p_min, vmap=None):
+def draft_pick(x, tok, prob, ctl, r, n_min, p_min, vmap=None, workspace=None):
+    """workspace: a zero-filled uint8 device tensor of ws_draft_pick_workspace bytes kept between calls (ws_draft_pick_ws)."""
     _dev_f32(x)
+    if workspace is not None:
+        check(lib().ws_draft_pick_ws(_stream(), _p(x), x.numel(), _p(tok), _p(prob), _p(ctl), r, n_min, p_min, _p(vmap),
+                                     _p(workspace), workspace.numel()), "ws_draft_pick_ws")
+        return
     check(lib().ws_draft_pick(_stream(), _p(x), x.numel(), _p(tok), _p(prob), _p(ctl), r, n_min, p_min, _p(vmap)),
           "ws_draft_pick")
 
 
-def draft_pick_rows(x, ctl_all, area, r, n_min, p_min, vmap=None):
+def draft_pick_rows(x, ctl_all, area, r, n_min, p_min, vmap=None, workspace=None):
     _dev_f32(x)
     ri = RowIdx()
     for i, d in enumerate(area):
         ri.v[i] = d
+    if workspace is not None:
+        check(lib().ws_draft_pick_rows_ws(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, n_min, p_min, _p(vmap),
+                                          x.shape[0], _p(workspace), workspace.numel()), "ws_draft_pick_rows_ws")
+        return
     check(lib().ws_draft_pick_rows(_stream(), _p(x), x.shape[1], _p(ctl_all), C.byref(ri), r, n_min, p_min, _p(vmap),
                                    x.shape[0]), "ws_draft_pick_rows")
 

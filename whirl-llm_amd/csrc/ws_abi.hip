@@ -233,6 +233,44 @@ int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const 
     return done();
 }
 
+namespace {
+// parts per row that pay for the greedy draft picks: the launch within the compute units, at least 16384 tokens a part
+unsigned pick_split_log2(int n, unsigned rows) {
+    const uint64_t cus = static_cast<uint64_t>(compute_units());
+    unsigned lg = 0;
+    while (lg < 4u && (static_cast<uint64_t>(rows) << (lg + 1u)) <= cus && (n >> (lg + 1u)) >= 16384) ++lg;
+    return lg;
+}
+bool pick_workspace_ok(const void* w, uint64_t bytes, unsigned rows) {
+    return w && bytes >= uint64_t{rows} * ws::kPickSplitRowBytes && reinterpret_cast<uintptr_t>(w) % 4u == 0;
+}
+}  // namespace
+
+uint64_t ws_draft_pick_workspace(int n, unsigned rows) { return pick_split_log2(n, rows) ? uint64_t{rows} * ws::kPickSplitRowBytes : 0ull; }
+
+int ws_draft_pick_ws(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
+                     const int* map, void* workspace, uint64_t workspace_bytes) {
+    if (!x || !tok || !prob || !ctl || n <= 0 || r < 0) return WS_E_INVALID;
+    const unsigned lg = pick_split_log2(n, 1u);
+    if (!lg || !pick_workspace_ok(workspace, workspace_bytes, 1u)) return ws_draft_pick(stream, x, n, tok, prob, ctl, r, n_min, p_min, map);
+    hipLaunchKernelGGL(draft_pick_split, dim3(1u << lg), dim3(WS_BLOCK), 0, S(stream), x, n, tok, prob, ctl, r, n_min, p_min, map, lg,
+                       static_cast<unsigned*>(workspace));
+    return done();
+}
+
+int ws_draft_pick_rows_ws(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min, float p_min,
+                          const int* map, unsigned rows, void* workspace, uint64_t workspace_bytes) {
+    if (!x || !ctl_all || !area || n <= 0 || r < 0 || r >= 16 || rows == 0 || rows > WS_MAX_TABLE_ROWS) return WS_E_INVALID;
+    const unsigned lg = pick_split_log2(n, rows);
+    if (!lg || !pick_workspace_ok(workspace, workspace_bytes, rows))
+        return ws_draft_pick_rows(stream, x, n, ctl_all, area, r, n_min, p_min, map, rows);
+    RowIdx a;
+    std::memcpy(&a, area, sizeof a);
+    hipLaunchKernelGGL(draft_pick_rows_split, dim3(rows << lg), dim3(WS_BLOCK), 0, S(stream), x, n, ctl_all, a, r, n_min, p_min, map, lg,
+                       static_cast<unsigned*>(workspace));
+    return done();
+}
+
 int ws_draft_sample_rows(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, const int* map,
                          const ws_dsamp_args* a, int* qbuf, unsigned rows) {
     if (!x || !ctl_all || !area || !a || !qbuf || n <= 0 || r < 0 || r >= 16 || rows == 0 || rows > WS_MAX_TABLE_ROWS)

@@ -99,11 +99,70 @@ __device__ __forceinline__ RowTop row_top(const float* __restrict__ x, int n) {
     return r;
 }
 
+// A row shared by several workgroups (the draft chain's one row, or a few: one compute unit reads 600 KB no faster than
+// in ~15 us, and the launch is repeated for every draft position): every part takes a slice - maximum, its first index,
+// sum exp against its own maximum - and leaves the three words in the row's workspace; the part that arrives last
+// combines them in slice order (a strictly larger maximum takes over: first index on ties) and is the one that writes.
+// Workspace of a row: 64 words, [0] parts arrived, [16 + 3 p ..] part p's maximum, index and sum; zero-filled once,
+// every launch leaves [0] at zero.
+constexpr uint64_t kPickSplitRowBytes = 256ull;
+struct PickSplit {
+    uint32_t parts = 1u, part = 0u;
+    uint32_t* work = nullptr;  // of this row
+};
+// returns whether this workgroup is the one that holds the row's result
+template <bool WITH_SUM>
+__device__ __forceinline__ bool row_top_shared(const float* __restrict__ x, int n, PickSplit sp, RowTop& out) {
+    if (sp.parts <= 1u) {
+        out = row_top<WITH_SUM>(x, n);
+        return true;
+    }
+    __shared__ uint32_t s_prev;
+    const int per = (((n + static_cast<int>(sp.parts) - 1) / static_cast<int>(sp.parts)) + 3) & ~3;
+    const int lo = min(static_cast<int>(sp.part) * per, n), hi = min(lo + per, n);
+    RowTop mine = row_top<WITH_SUM>(x + lo, hi - lo);
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&sp.work[16u + 3u * sp.part], __float_as_uint(mine.best.v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&sp.work[17u + 3u * sp.part], static_cast<uint32_t>(mine.best.i + lo), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&sp.work[18u + 3u * sp.part], __float_as_uint(mine.sum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // acknowledged: the counter may say so
+        s_prev = __hip_atomic_fetch_add(&sp.work[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (s_prev != sp.parts - 1u) return false;
+    Best b = {-INFINITY, 0};
+    float vs[16], ss[16];
+#pragma unroll
+    for (uint32_t p = 0; p < 16u; ++p) {
+        vs[p] = -INFINITY;
+        ss[p] = 0.f;
+        if (p < sp.parts) {
+            vs[p] = __uint_as_float(__hip_atomic_load(&sp.work[16u + 3u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            const int at = static_cast<int>(__hip_atomic_load(&sp.work[17u + 3u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            ss[p] = __uint_as_float(__hip_atomic_load(&sp.work[18u + 3u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            if (vs[p] > b.v) {
+                b.v = vs[p];
+                b.i = at;
+            }
+        }
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (uint32_t p = 0; p < 16u; ++p)
+        if (vs[p] > -INFINITY) sum += ss[p] * __expf(vs[p] - b.v);
+    __syncthreads();  // every thread has read the counter's verdict
+    if (threadIdx.x == 0) __hip_atomic_store(&sp.work[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // as the next launch needs it
+    out.best = b;
+    out.sum = WITH_SUM ? sum : 0.f;
+    return true;
+}
+
 // kernels/shared/sample_pick_set_tokens.h:60-86
 __device__ __forceinline__ void draft_pick_row(const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min,
-                                               float p_min, const int* map) {
-    if (r > 0 && ctl[1] != 0) return;  // the chain stopped at an earlier draft (uniform over the block)
-    const RowTop t = row_top<true>(x, n);
+                                               float p_min, const int* map, PickSplit sp = PickSplit{}) {
+    if (r > 0 && ctl[1] != 0) return;  // the chain stopped at an earlier draft (uniform over the block, and over the parts of a row)
+    RowTop t;
+    if (!row_top_shared<true>(x, n, sp, t)) return;
     if (threadIdx.x == 0) {
         const float p = 1.f / t.sum;
         tok[r] = map ? map[t.best.i] : t.best.i;
@@ -162,4 +221,28 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     int* c = ctl_all + area.v[blockIdx.x];
     ws::draft_pick_row(x + static_cast<size_t>(blockIdx.x) * n, n, c + 16, reinterpret_cast<float*>(c + 32), c + 48, r, n_min,
                        p_min, map);
+}
+
+// draft_pick / draft_pick_rows with every row shared by 1 << split_log2 consecutive workgroups (no counterpart in the
+// reference; launched by ws_draft_pick_ws / ws_draft_pick_rows_ws)
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_pick_split(const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min, const int* map,
+                     unsigned split_log2, unsigned* work) {
+    ws::PickSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x;
+    sp.work = work;
+    ws::draft_pick_row(x, n, tok, prob, ctl, r, n_min, p_min, map, sp);
+}
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    draft_pick_rows_split(const float* x, int n, int* ctl_all, RowIdx area, int r, int n_min, float p_min, const int* map,
+                          unsigned split_log2, unsigned* work) {
+    const unsigned row = blockIdx.x >> split_log2;
+    ws::PickSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x & (sp.parts - 1u);
+    sp.work = work + static_cast<size_t>(row) * (ws::kPickSplitRowBytes / 4u);
+    int* c = ctl_all + area.v[row];
+    ws::draft_pick_row(x + static_cast<size_t>(row) * n, n, c + 16, reinterpret_cast<float*>(c + 32), c + 48, r, n_min, p_min, map, sp);
 }
