@@ -96,3 +96,23 @@ def test_a_full_size_row_with_a_long_top_k():
     c["top_p"][:] = [0.98, 1.0]
     res, smp = run_case(c, 1)
     assert res["exact"] == 2, res
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("V", [8032, 32000, 200000])
+def test_a_top_k_that_reaches_past_every_candidate_with_mass(mode, V):
+    """Logits spread over +-30 units at a temperature of 1/3: whatever lies more than 21 units under the maximum has no
+    mass the sampler can tell from zero, and top-k reaches far into it - those candidates are counted and listed in
+    the host filter's order, larger logit first and lower id among equals (src/sampling/sampler.cpp:18-21), with the
+    -inf tokens last by id. Row 0 has too few finite logits for its top-k; row 3 has a penalised history on top."""
+    c, rng = _base(4, V, n_hist=300, seed=9)
+    c["name"] = "top-k into the candidates without mass"
+    c["logits"] = (rng.standard_normal((4, V)) * 8).astype(np.float32)
+    c["logits"][0, rng.random(V) < 0.95] = -np.inf
+    c["logits"][1] = np.round(c["logits"][1])  # ties everywhere
+    c["inv_t"][:] = np.float32(3.0)
+    c["top_k"][:] = [1000, 3000, 500, 2500]
+    c["rep"][:3] = np.float32(1.0)
+    c["pres"][:3] = c["freq"][:3] = np.float32(0.0)
+    res, smp = run_case(c, 1, kept_cap=4096, mode=mode)
+    assert res["exact"] == 4, res

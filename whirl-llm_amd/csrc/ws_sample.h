@@ -632,6 +632,130 @@ __device__ __forceinline__ void sort_desc(uint64_t* keys, uint32_t P) {
 // hundreds of microseconds, for rows that otherwise had no answer. The decisions are the rules of the main path (the
 // cuts of src/sampling/sampler.cpp:15-78, the walk of :118-146, the race of :80-106). A function of its own, not
 // inlined, so that its registers and code do not weigh on the kernel's sweep.
+// A top-k that reaches past every candidate with mass (into logits whose mass is below e^-63 of the largest, and -inf)
+// keeps `want` of those as well, in the host filter's order: larger logit first, then lower id. Which ones, for the
+// dump of the kept set: the 32-bit key of the last logit taken, and how many of the tokens with exactly that logit
+// (the lowest ids). A radix select over the row, 12 + 12 + 8 bits; a function of its own: rare, and not worth a register
+// of the kernel. Zero-mass candidate: not above `kept_key` and in the tail bins. LDS offset 0, 16 KB, is free by then.
+struct TailIn {
+    const void* base;
+    const uint32_t* allow;
+    uint32_t V;
+    int dtype;
+    uint32_t touched_at;  // LDS offset of the touched bitmap, prefix and values; ~0 when no token is touched
+    float aq, c64;
+    uint64_t kept_key;
+    uint32_t want;
+};
+struct TailCut {
+    uint32_t key, n_equal;
+};
+__device__ __noinline__ TailCut tail_cut(const TailIn in) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t t_red[WS_WAVES];
+    __shared__ uint32_t t_sel[2];
+    const uint32_t t = threadIdx.x, V = in.V;
+    RowView rv;
+    rv.base = in.base;
+    rv.V = V;
+    rv.dtype = in.dtype;
+    rv.vec = false;
+    rv.allow = in.allow;
+    const uint32_t nW = (V + 31u) >> 5;
+    rv.touched = in.touched_at != 0xffffffffu ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) : nullptr;
+    rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u);
+    rv.pv = reinterpret_cast<const float*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    uint32_t* cnt = reinterpret_cast<uint32_t*>(lds);  // 4096 digit counts
+    constexpr uint32_t kPer = 4096u / WS_BLOCK;        // digits per thread, largest digits first
+    uint32_t prefix = 0u, fixed = 0u, need = in.want;
+    for (int level = 0; level < 3; ++level) {
+        const uint32_t shift = level == 0 ? 20u : (level == 1 ? 8u : 0u), digits = level == 2 ? 256u : 4096u;
+        __syncthreads();
+        for (uint32_t d = t; d < 4096u; d += WS_BLOCK) cnt[d] = 0u;
+        __syncthreads();
+        for (uint32_t i = t; i < V; i += WS_BLOCK) {
+            const float x = adjusted_logit(rv, i);
+            if (key64(x, i) >= in.kept_key || bin_of(in.aq, in.c64, x) < static_cast<uint32_t>(kTail)) continue;
+            const uint32_t k = key32(x);
+            if ((k & fixed) == prefix) atomicAdd(&cnt[(k >> shift) & (digits - 1u)], 1u);
+        }
+        __syncthreads();
+        uint32_t c[kPer], tot = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < kPer; ++j) {
+            c[j] = cnt[4095u - (kPer * t + j)];  // (digits a short level does not use hold no count)
+            tot += c[j];
+        }
+        uint32_t all;
+        uint32_t above = block_excl_scan(tot, t_red, &all);
+        if (t == 0) t_sel[0] = 0u, t_sel[1] = need;  // (nothing found: fewer candidates than asked for - all of them)
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < kPer; ++j) {
+            if (above < need && above + c[j] >= need) {
+                t_sel[0] = 4095u - (kPer * t + j);
+                t_sel[1] = need - above;
+            }
+            above += c[j];
+        }
+        __syncthreads();
+        prefix |= t_sel[0] << shift;
+        fixed |= (digits - 1u) << shift;
+        need = t_sel[1];
+    }
+    return TailCut{prefix, need};
+}
+
+// The kept set of a row in ascending id order (the optional dump): every token whose key is at or above `kept_key`, and
+// `want` zero-mass candidates (tail_cut). A function of its own, like the exact path: it runs for callers that ask for
+// the dump only, and the kernel keeps its registers for what every row needs.
+__device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float* klg, uint32_t kept_cap) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t d_red[WS_WAVES];
+    const uint32_t t = threadIdx.x, V = in.V;
+    RowView rv;
+    rv.base = in.base;
+    rv.V = V;
+    rv.dtype = in.dtype;
+    rv.vec = false;
+    rv.allow = in.allow;
+    const uint32_t nW = (V + 31u) >> 5;
+    rv.touched = in.touched_at != 0xffffffffu ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) : nullptr;
+    rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u);
+    rv.pv = reinterpret_cast<const float*>(lds + (in.touched_at != 0xffffffffu ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    TailCut cut{0u, 0u};
+    if (in.want) cut = tail_cut(in);  // uniform
+    __syncthreads();
+    uint32_t base = 0, tail_base = 0;
+    // id order needs consecutive ids per tile: tiles of WS_BLOCK consecutive tokens, one per thread
+    for (uint32_t i0 = 0; i0 < V; i0 += WS_BLOCK) {
+        const uint32_t i = i0 + t;
+        float x = -INFINITY;
+        uint32_t keep = 0, tl = 0;
+        if (i < V) {
+            x = adjusted_logit(rv, i);
+            keep = key64(x, i) >= in.kept_key;
+            if (in.want && !keep && bin_of(in.aq, in.c64, x) >= static_cast<uint32_t>(kTail)) {
+                // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes;
+                // among those with exactly that logit the lowest ids
+                keep = key32(x) > cut.key;
+                tl = key32(x) == cut.key;
+            }
+        }
+        uint32_t tot;
+        const uint32_t before = block_excl_scan(keep | (tl << 16), d_red, &tot);
+        const uint32_t tl_before = tail_base + (before >> 16);
+        if (tl && tl_before < cut.n_equal) keep = 1;
+        const uint32_t o = base + (before & 0xffffu) + min(tl_before, cut.n_equal);
+        if (keep && o < kept_cap) {
+            kid[o] = static_cast<int32_t>(i);
+            if (klg) klg[o] = x;
+        }
+        base += tot & 0xffffu;
+        tail_base += tot >> 16;
+    }
+}
+
 struct ExactIn {
     const void* base;
     const uint32_t* allow;
@@ -3373,31 +3497,51 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 
     // ------------------------------------------------------------------ optional: the kept set in ascending id order
     if (WS_RARE(A.kept_ids && token >= 0)) {
+        TailIn in;
+        in.base = rv.base;
+        in.allow = rv.allow;
+        in.V = V;
+        in.dtype = rv.dtype;
+        in.touched_at = rv.touched ? A.lds_ab : 0xffffffffu;
+        in.aq = aq;
+        in.c64 = c64;
+        in.kept_key = kept_key;
+        in.want = tail_extra;
+        __syncthreads();
         int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
-        __syncthreads();
-        uint32_t base = 0, tail_base = 0;
-        // id order needs consecutive ids per tile: tiles of 1024 consecutive tokens, one per thread
-        for (uint32_t i0 = 0; i0 < V; i0 += WS_BLOCK) {
-            const uint32_t i = i0 + t;
-            float x = -INFINITY;
-            uint32_t keep = 0, tl = 0;
-            if (i < V) {
-                x = adjusted_logit(rv, i);
-                keep = key64(x, i) >= kept_key;
-                tl = tail_extra && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail);  // among zero-mass candidates the lowest ids
+        if constexpr (FUSED) {
+            dump_kept_set(in, kid, klg, A.kept_cap);
+        } else {
+            // (the kernels without a bin cache keep the loop in line: as a call it doubles their spilled registers)
+            TailCut cut{0u, 0u};
+            if (tail_extra) cut = tail_cut(in);  // uniform
+            __syncthreads();
+            uint32_t base = 0, tail_base = 0;
+            for (uint32_t i0 = 0; i0 < V; i0 += WS_BLOCK) {
+                const uint32_t i = i0 + t;
+                float x = -INFINITY;
+                uint32_t keep = 0, tl = 0;
+                if (i < V) {
+                    x = adjusted_logit(rv, i);
+                    keep = key64(x, i) >= kept_key;
+                    if (tail_extra && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
+                        keep = key32(x) > cut.key;
+                        tl = key32(x) == cut.key;
+                    }
+                }
+                uint32_t tot;
+                const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
+                const uint32_t tl_before = tail_base + (before >> 16);
+                if (tl && tl_before < cut.n_equal) keep = 1;
+                const uint32_t o = base + (before & 0xffffu) + min(tl_before, cut.n_equal);
+                if (keep && o < A.kept_cap) {
+                    kid[o] = static_cast<int32_t>(i);
+                    if (klg) klg[o] = x;
+                }
+                base += tot & 0xffffu;
+                tail_base += tot >> 16;
             }
-            uint32_t tot;
-            const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
-            const uint32_t tl_before = tail_base + (before >> 16);
-            if (tl && tl_before < tail_extra) keep = 1;
-            const uint32_t o = base + (before & 0xffffu) + min(tl_before, tail_extra);
-            if (keep && o < A.kept_cap) {
-                kid[o] = static_cast<int32_t>(i);
-                if (klg) klg[o] = x;
-            }
-            base += tot & 0xffffu;
-            tail_base += tot >> 16;
         }
     }
 }
