@@ -160,7 +160,8 @@ enum {
                                       equal logits, a very flat row) is answered by an exact path inside the same launch -
                                       same results, some hundreds of microseconds for such a row */
     WS_FLAG_BAD_PARAM = 1u << 5,   /* history / bias longer than max_hist / max_bias, inv_t <= 0: token = -1 */
-    WS_FLAG_OPEN = 1u << 6,        /* no filter active (Sampler::closed false): drawn as the reference draws an open row, from
+    WS_FLAG_OPEN = 1u << 6,        /* no filter active - top_k 0, top_p 1, min_p 0 (Sampler::closed false; a top_k of the vocabulary
+                                      size or beyond does close the set, src/sampling/sampler.cpp:35-42) -: drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order
                                       (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
     WS_FLAG_APPROX_ENTROPY = 1u << 7 /* `entropy` counts the kept tokens outside the gathered bins at the middle of their

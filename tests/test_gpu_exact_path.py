@@ -116,3 +116,24 @@ def test_a_top_k_that_reaches_past_every_candidate_with_mass(mode, V):
     c["pres"][:3] = c["freq"][:3] = np.float32(0.0)
     res, smp = run_case(c, 1, kept_cap=4096, mode=mode)
     assert res["exact"] == 4, res
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("V", [1000, 32000, 200000])
+def test_a_top_k_of_the_vocabulary_size_or_beyond_closes_the_row(mode, V):
+    """top-k >= vocab with no other filter is not an open row: the reference's filter closes the set at the complete row
+    (src/sampling/sampler.cpp:35-42, 33-34), keeps every token and draws over the whole row in sorted order - not from
+    256 candidates and then in id order, as it draws a row without any filter (row 3, for contrast: flagged open)."""
+    c, rng = _base(6, V, n_hist=100, seed=10)
+    c["name"] = "top-k >= vocab"
+    c["top_k"][:] = [V, V + 5, 1000000, 0, V, V]
+    c["top_p"][4] = 0.9
+    c["min_p"][5] = 0.01
+    c["inv_t"][:] = (1.0 / rng.uniform(0.5, 1.5, 6)).astype(np.float32)
+    d = gc.upload(c)
+    smp = gc.sampler_for(c, d, 1, kept_cap=min(V, 4096), mode=mode).run()
+    res = gc.compare_rows(c, smp, [0, 1, 2, 4, 5], 1, check_kept=V <= 4096)
+    assert res["exact"] == 5, res
+    fl = smp.flags.cpu().numpy()
+    assert not (fl[[0, 1, 2, 4, 5]] & gc.pkg().FLAG_OPEN).any() and (fl[3] & gc.pkg().FLAG_OPEN)
+    assert smp.n_kept.cpu().numpy()[:3].tolist() == [V, V, V]

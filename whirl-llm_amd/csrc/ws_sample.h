@@ -2029,7 +2029,9 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     // No filter at all: an open row. The reference draws it from the engine's short candidate list in sorted order
     // first (k_small, src/server/engine_sampling.h:20), probabilities over the float normaliser, and past that list
     // from the rest of the vocabulary in id order (src/sampling/sampler.cpp:118-146). The list is gathered like a top-k.
-    const bool open_row = !use_top_p && !use_min_p && !prefix_mode;
+    // (A top-k of the vocabulary's size or beyond is a filter all the same: it closes the set at the complete row,
+    // src/sampling/sampler.cpp:35-42, and the draw then goes over the whole row in sorted order.)
+    const bool open_row = !use_top_p && !use_min_p && top_k == 0u;
     if (open_row) {
         flags |= kOpen;
         n1 = min(kOpenList, V);
