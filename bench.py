@@ -246,6 +246,9 @@ def reference_kernels(steps):
     ids = torch.empty((16, 16), dtype=torch.int32, device="cuda:0")
     vals = torch.empty((16, 16), dtype=torch.float32, device="cuda:0")
     timed("dflash_topk k=16", 16, lambda: L.ws_dflash_topk(S(), P(x), V, V, 16, P(ids), P(vals), 16), 16 * (V * 4 + 16 * 8))
+    work = torch.zeros(max(int(L.ws_dflash_topk_workspace(V, V, 16)), 8), dtype=torch.uint8, device="cuda:0")
+    timed("dflash_topk_ws k=16", 16, lambda: L.ws_dflash_topk_ws(S(), P(x), V, V, 16, P(ids), P(vals), 16, P(work), work.numel()),
+          16 * (V * 4 + 16 * 8))
     # the drafter's sampled pick (the "specsample" rule): q over the 32 largest logits + race draw, one row per sequence
     for rows in (1, 8):
         x = torch.randn(rows, V, device="cuda:0") * 2
@@ -273,6 +276,8 @@ def reference_kernels(steps):
     tok = torch.empty(1, dtype=torch.int32, device="cuda:0")
     pr = torch.empty(1, dtype=torch.float32, device="cuda:0")
     timed("argmax_prob", 1, lambda: L.ws_argmax_prob(S(), P(x), V, P(tok), P(pr)), V * 4)
+    work = torch.zeros(max(int(L.ws_draft_pick_workspace(V, 1)), 8), dtype=torch.uint8, device="cuda:0")
+    timed("argmax_prob_ws", 1, lambda: L.ws_argmax_prob_ws(S(), P(x), V, P(tok), P(pr), P(work), work.numel()), V * 4)
     return out
 
 

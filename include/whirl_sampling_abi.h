@@ -91,6 +91,8 @@ int ws_draft_pick_rows(void* stream, const float* x, int n, int* ctl_all, const 
  * bytes (256 per row; 0: this shape is not split), 4-byte aligned, zero-filled once, one launch at a time; without it
  * these are ws_draft_pick / ws_draft_pick_rows. */
 uint64_t ws_draft_pick_workspace(int n, unsigned rows);
+/* ws_argmax_prob with such a workspace (ws_draft_pick_workspace(n, 1) bytes): the one row read by several workgroups. */
+int ws_argmax_prob_ws(void* stream, const float* x, int n, int* out_tok, float* out_prob, void* workspace, uint64_t workspace_bytes);
 int ws_draft_pick_ws(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
                      const int* map, void* workspace, uint64_t workspace_bytes);
 int ws_draft_pick_rows_ws(void* stream, const float* x, int n, int* ctl_all, const ws_row_idx* area, int r, int n_min,
@@ -129,6 +131,12 @@ int ws_topk_rows_ws(void* stream, const float* x, int n, int K, float inv_t, int
  * in key order: larger value first, then smaller index; NaN counts as -inf and is written out as it stands. The
  * reference finds them in k passes over the row; here the row is read once. */
 int ws_dflash_topk(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows);
+/* ws_dflash_topk with a workspace, as ws_topk_rows_ws (same launch site): the drafter's 16 rows per draft position shared
+ * between workgroups; rows ld floats apart split only when ld is a multiple of 4. Same ids and values.
+ * ws_dflash_topk_workspace() bytes, 0 when the shape is not split; zero-filled once, one launch at a time. */
+uint64_t ws_dflash_topk_workspace(int n, int ld, unsigned rows);
+int ws_dflash_topk_ws(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows, void* workspace,
+                      uint64_t workspace_bytes);
 
 /* ---- (2) batched fused sampler ---------------------------------------------------------------------------- */
 

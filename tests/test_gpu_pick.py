@@ -369,3 +369,35 @@ def test_draft_pick_shared_between_workgroups(rows5):
         ctl.zero_()
         m.draft_pick(src, tok, prob, ctl, 0, 0, 0.0, workspace=w1)
         assert tok.cpu()[0].item() == want
+
+
+@pytest.mark.parametrize("k", [1, 16, 64])
+def test_dflash_topk_and_argmax_prob_shared_between_workgroups(k, rows5):
+    """ws_dflash_topk_ws on the cases of test_dflash_topk_key_order (ids and values exact against the oracle's k rounds and
+    the one-workgroup kernel, twice on one workspace; rows with a stride that is no multiple of 4 are not split), and
+    ws_argmax_prob_ws on a row with two equal maxima."""
+    from test_oracle_batch import dflash_case
+    m = gpu_cases.pkg()
+    lib = wo.load("oracle")
+    for n, ld in ((248320, 248320), (50000, 50004), (50000, 50003)):
+        x = np.zeros((4, ld), np.float32)
+        x[:, :n] = dflash_case(n)
+        dx = torch.from_numpy(x).to(DEV)[:, :n]
+        need = int(m.lib().ws_dflash_topk_workspace(n, ld, 4))
+        assert (need > 0) == (ld % 4 == 0)
+        work = torch.zeros(max(need, 8), dtype=torch.uint8, device=DEV)
+        want = [a.cpu().numpy() for a in m.dflash_topk(dx, k)]
+        for launch in range(2):
+            got = [a.cpu().numpy() for a in m.dflash_topk(dx, k, workspace=work)]
+            assert np.array_equal(got[0], want[0]) and got[1].tobytes() == want[1].tobytes(), (n, ld, launch)
+        for r in range(4):
+            wi, wv = np.zeros(k, np.int32), np.zeros(k, np.float32)
+            lib.wo_dflash_topk_row(wo._ptr(np.ascontiguousarray(x[r, :n])), n, k, wo._ptr(wi), wo._ptr(wv))
+            assert np.array_equal(want[0][r], wi) and want[1][r].tobytes() == wv.tobytes(), (n, r)
+    x, dx = rows5
+    w1 = torch.zeros(int(m.lib().ws_draft_pick_workspace(x.shape[1], 1)), dtype=torch.uint8, device=DEV)
+    for r in (0, 1, 2):
+        for launch in range(2):
+            tok, prob = m.argmax_prob(dx[r], workspace=w1)
+            assert tok.item() == first_max(x[r])
+            assert abs(prob.item() - softmax_top(x[r])) <= 2e-6 * softmax_top(x[r]) + 1e-12

@@ -128,6 +128,10 @@ ABI = {
     "ws_topk_rows_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_uint, C.c_void_p, C.c_uint64]),
     "ws_dflash_topk": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint]),
+    "ws_dflash_topk_workspace": (C.c_uint64, [C.c_int, C.c_int, C.c_uint]),
+    "ws_dflash_topk_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_uint, C.c_void_p,
+                                    C.c_uint64]),
+    "ws_argmax_prob_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_sample_batch_static": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
@@ -201,11 +205,15 @@ def argmax_rows_to(x, out, dst):
     return out
 
 
-def argmax_prob(x):
+def argmax_prob(x, workspace=None):
     _dev_f32(x)
     tok = torch.empty(1, dtype=torch.int32, device=x.device)
     prob = torch.empty(1, dtype=torch.float32, device=x.device)
-    check(lib().ws_argmax_prob(_stream(), _p(x), x.numel(), _p(tok), _p(prob)), "ws_argmax_prob")
+    if workspace is not None:
+        check(lib().ws_argmax_prob_ws(_stream(), _p(x), x.numel(), _p(tok), _p(prob), _p(workspace), workspace.numel()),
+              "ws_argmax_prob_ws")
+    else:
+        check(lib().ws_argmax_prob(_stream(), _p(x), x.numel(), _p(tok), _p(prob)), "ws_argmax_prob")
     return tok, prob
 
 
@@ -274,14 +282,18 @@ def topk_rows_workspace(n, K, rows, device="cuda:0"):
     return torch.zeros(need, dtype=torch.uint8, device=device) if need else None
 
 
-def dflash_topk(x, k):
+def dflash_topk(x, k, workspace=None):
     """x: [rows, n] float32, rows any stride -> ids int32 [rows, k], vals float32 [rows, k] in key order (value desc, id asc)."""
     if not x.is_cuda or x.dim() != 2 or x.dtype != torch.float32 or x.stride(1) != 1:
         raise WsError("x: [rows, n] float32 device tensor with unit inner stride")
     rows, n = x.shape
     ids = torch.full((rows, k), -1, dtype=torch.int32, device=x.device)
     vals = torch.zeros((rows, k), dtype=torch.float32, device=x.device)
-    check(lib().ws_dflash_topk(_stream(), _p(x), n, x.stride(0), k, _p(ids), _p(vals), rows), "ws_dflash_topk")
+    if workspace is not None:
+        check(lib().ws_dflash_topk_ws(_stream(), _p(x), n, x.stride(0), k, _p(ids), _p(vals), rows, _p(workspace),
+                                      workspace.numel()), "ws_dflash_topk_ws")
+    else:
+        check(lib().ws_dflash_topk(_stream(), _p(x), n, x.stride(0), k, _p(ids), _p(vals), rows), "ws_dflash_topk")
     return ids, vals
 
 

@@ -217,6 +217,8 @@ int ws_argmax_prob(void* stream, const float* x, int n, int* out_tok, float* out
     return done();
 }
 
+int ws_argmax_prob_ws(void* stream, const float* x, int n, int* out_tok, float* out_prob, void* workspace, uint64_t workspace_bytes);
+
 int ws_draft_pick(void* stream, const float* x, int n, int* tok, float* prob, int* ctl, int r, int n_min, float p_min,
                   const int* map) {
     if (!x || !tok || !prob || !ctl || n <= 0 || r < 0) return WS_E_INVALID;
@@ -245,6 +247,15 @@ bool pick_workspace_ok(const void* w, uint64_t bytes, unsigned rows) {
     return w && bytes >= uint64_t{rows} * ws::kPickSplitRowBytes && reinterpret_cast<uintptr_t>(w) % 4u == 0;
 }
 }  // namespace
+
+int ws_argmax_prob_ws(void* stream, const float* x, int n, int* out_tok, float* out_prob, void* workspace, uint64_t workspace_bytes) {
+    if (!x || !out_tok || !out_prob || n <= 0) return WS_E_INVALID;
+    const unsigned lg = pick_split_log2(n, 1u);
+    if (!lg || !pick_workspace_ok(workspace, workspace_bytes, 1u)) return ws_argmax_prob(stream, x, n, out_tok, out_prob);
+    hipLaunchKernelGGL(argmax_prob_split, dim3(1u << lg), dim3(WS_BLOCK), 0, S(stream), x, n, out_tok, out_prob, lg,
+                       static_cast<unsigned*>(workspace));
+    return done();
+}
 
 uint64_t ws_draft_pick_workspace(int n, unsigned rows) { return pick_split_log2(n, rows) ? uint64_t{rows} * ws::kPickSplitRowBytes : 0ull; }
 
@@ -338,6 +349,21 @@ int ws_topk_rows_ws(void* stream, const float* x, int n, int K, float inv_t, int
     if (!lg || !workspace || workspace_bytes < uint64_t{rows} * ws::kTopkSplitRowBytes || reinterpret_cast<uintptr_t>(workspace) % 8u != 0)
         return ws_topk_rows(stream, x, n, K, inv_t, ids, vals, stats, rows);
     hipLaunchKernelGGL(topk_rows_split, dim3(rows << lg), dim3(WS_BLOCK), 0, S(stream), x, n, K, inv_t, ids, vals, stats, lg,
+                       static_cast<unsigned char*>(workspace));
+    return done();
+}
+
+uint64_t ws_dflash_topk_workspace(int n, int ld, unsigned rows) {
+    return (ld & 3) == 0 && topk_split_log2(nullptr, n, 64, rows) ? uint64_t{rows} * ws::kTopkSplitRowBytes : 0ull;
+}
+
+int ws_dflash_topk_ws(void* stream, const float* x, int n, int ld, int k, int* ids, float* vals, unsigned rows, void* workspace,
+                      uint64_t workspace_bytes) {
+    if (!x || !ids || !vals || n <= 0 || ld < n || k <= 0 || k > 64 || rows == 0) return WS_E_INVALID;
+    const unsigned lg = (ld & 3) == 0 ? topk_split_log2(x, n, k, rows) : 0u;  // (rows ld floats apart: whole vectors when ld is)
+    if (!lg || !workspace || workspace_bytes < uint64_t{rows} * ws::kTopkSplitRowBytes || reinterpret_cast<uintptr_t>(workspace) % 8u != 0)
+        return ws_dflash_topk(stream, x, n, ld, k, ids, vals, rows);
+    hipLaunchKernelGGL(dflash_topk_split, dim3(rows << lg), dim3(WS_BLOCK), 0, S(stream), x, n, ld, k, ids, vals, lg,
                        static_cast<unsigned char*>(workspace));
     return done();
 }

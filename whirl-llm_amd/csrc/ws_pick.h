@@ -246,3 +246,18 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
     int* c = ctl_all + area.v[row];
     ws::draft_pick_row(x + static_cast<size_t>(row) * n, n, c + 16, reinterpret_cast<float*>(c + 32), c + 48, r, n_min, p_min, map, sp);
 }
+
+// argmax_prob with the row shared by 1 << split_log2 workgroups (ws_argmax_prob_ws)
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    argmax_prob_split(const float* x, int n, int* out_tok, float* out_prob, unsigned split_log2, unsigned* work) {
+    ws::PickSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x;
+    sp.work = work;
+    ws::RowTop t;
+    if (!ws::row_top_shared<true>(x, n, sp, t)) return;
+    if (threadIdx.x == 0) {
+        out_tok[0] = t.best.i;
+        out_prob[0] = 1.f / t.sum;
+    }
+}

@@ -524,7 +524,7 @@ __device__ __forceinline__ bool topk_one_row(const float* x, int n, int K, float
     const float nan = __uint_as_float(0x7fc00000u);
     const float ref = (counted && inv_t > 0.f && inv_t <= 8.f) ? bound - 8.f : nan;
     bool split = sp.parts > 1u;
-    if (split && !(SUM && counted && list_bin >= 0 && ref == ref)) {  // (every part sees the same head: the same answer)
+    if (split && !(counted && list_bin >= 0 && (!SUM || ref == ref))) {  // (every part sees the same head: the same answer)
         if (sp.part != 0u) return false;
         split = false;
     }
@@ -676,17 +676,15 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK)
 // (larger value first, then smaller index; NaN counts as -inf and is written out as it stands), rows ld floats apart.
 // The reference takes k passes over the row, one winner each; here the row is read once by the select above and the
 // k winners are put in order by one wave.
-extern "C" __global__ void __launch_bounds__(WS_BLOCK) dflash_topk(const float* x, int n, int ld, int k, int* ids, float* vals) {
-    const size_t row = blockIdx.x;
-    ids += row * k;
-    vals += row * k;
-    ws::topk_one_row<false>(x + row * ld, n, k, 1.f, ids, vals, nullptr);  // no normaliser asked for
+namespace ws {
+__device__ __forceinline__ void dflash_topk_row(const float* x, int n, int k, int* ids, float* vals, TopkSplit sp) {
+    if (!ws::topk_one_row<false>(x, n, k, 1.f, ids, vals, nullptr, sp)) return;  // no normaliser asked for (false: a part of a shared row that is not the last to arrive)
     __syncthreads();  // the winners are in ids / vals, in id order
     const int kk = k < n ? k : n;
     if (threadIdx.x >= 64) return;
     const int lane = threadIdx.x;
     const int id = lane < kk ? ids[lane] : 0x7fffffff;
-    const float raw = lane < kk ? x[row * ld + id] : -INFINITY;  // as it stands in the row: a NaN is written out as NaN
+    const float raw = lane < kk ? x[id] : -INFINITY;  // as it stands in the row: a NaN is written out as NaN
     const float v = fmaxf(raw, -INFINITY);  // NaN -> -inf
     int rank = 0;
     for (int j = 0; j < kk; ++j) {
@@ -702,4 +700,21 @@ extern "C" __global__ void __launch_bounds__(WS_BLOCK) dflash_topk(const float* 
         ids[o] = 0x7fffffff;
         vals[o] = -INFINITY;
     }
+}
+}  // namespace ws
+
+extern "C" __global__ void __launch_bounds__(WS_BLOCK) dflash_topk(const float* x, int n, int ld, int k, int* ids, float* vals) {
+    const size_t row = blockIdx.x;
+    ws::dflash_topk_row(x + row * ld, n, k, ids + row * k, vals + row * k, ws::TopkSplit{});
+}
+
+// dflash_topk with every row shared by 1 << split_log2 consecutive workgroups (ws_dflash_topk_ws)
+extern "C" __global__ void __launch_bounds__(WS_BLOCK)
+    dflash_topk_split(const float* x, int n, int ld, int k, int* ids, float* vals, unsigned split_log2, unsigned char* work) {
+    const size_t row = blockIdx.x >> split_log2;
+    ws::TopkSplit sp;
+    sp.parts = 1u << split_log2;
+    sp.part = blockIdx.x & (sp.parts - 1u);
+    sp.work = work + row * ws::kTopkSplitRowBytes;
+    ws::dflash_topk_row(x + row * ld, n, k, ids + row * k, vals + row * k, sp);
 }
