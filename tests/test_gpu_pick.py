@@ -219,13 +219,16 @@ def test_dflash_topk_rejects_long_lists():
 
 def test_adjust_rows_matches_the_oracle_bit_for_bit():
     """ws_adjust_rows: the penalised copy of a row equals the oracle's wo_apply_penalties on every token, with mask, bias
-    (repeated ids included), history counts, fp32 and bf16 input, through the rank tables and through the list scan."""
+    (repeated ids included), history counts, fp32 and bf16 input, through the rank tables and through the list scan,
+    rows held by one workgroup and rows shared by up to sixteen."""
     gc = gpu_cases
     m = gc.pkg()
     lib = wo.load("oracle")
     cases = [gc.make_cfg2(rows=5, V=32000, n_hist=700, n_bias=40), gc.make_cfg5(rows=3, V=16384, n_hist=300, n_bias=25),
              gc.make_cfg3(rows=3, V=24000, n_hist=200),
-             gc.make_cfg2(rows=2, V=1000000, n_hist=300, n_bias=20)]  # a bitmap of this vocabulary does not fit the LDS: the list-scan route
+             gc.make_cfg2(rows=2, V=1000000, n_hist=300, n_bias=20),  # a bitmap of this vocabulary does not fit the LDS: the list-scan route
+             gc.make_cfg2(rows=1, V=151936, n_hist=2048, n_bias=300),  # one row shared by sixteen workgroups
+             gc.make_cfg2(rows=3, V=50001, n_hist=500, n_bias=30)]  # rows off the 16-byte grid, a last slice that ends inside a word
     cases[0]["bias_ids"][:, 3] = cases[0]["bias_ids"][:, 0]
     cases[0]["bias_ids"][:, 9] = cases[0]["bias_ids"][:, 0]
     for c in cases:

@@ -493,7 +493,11 @@ int ws_adjust_rows(void* stream, const ws_adjust* b) {
         if (e != hipSuccess) return static_cast<int>(e);
         adjust_attr_set = true;
     }
-    hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows), dim3(WS_BLOCK), ws::kAdjustLds, S(stream), a);
+    // a small batch shares a row between workgroups (slices of at least 8192 tokens, one workgroup per compute unit)
+    uint32_t parts = 1;
+    while (parts < 16u && static_cast<uint64_t>(b->rows) * (parts * 2u) <= compute_units() && b->vocab / (parts * 2u) >= 8192u) parts *= 2u;
+    a.parts = parts;
+    hipLaunchKernelGGL(ws::adjust_rows_kernel, dim3(b->rows * parts), dim3(WS_BLOCK), ws::kAdjustLds, S(stream), a);
     return done();
 }
 

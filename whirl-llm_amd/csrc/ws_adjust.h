@@ -1,7 +1,9 @@
 // adjust_rows: a penalised fp32 copy of logits rows, for callers that want the adjusted logits themselves (a top-k of
 // them, a full-row download). Same order of operations as the batched sampler: NaN and masked-out -> -inf, bias values
 // of an id added one by one in listed order, repetition (x > 0 ? x / rep : x * rep), then x -= freq * count + pres,
-// every operation rounded to float. One workgroup per row; the row is copied once, then the touched tokens are patched.
+// every operation rounded to float. A row is copied once, then the touched tokens are patched; a small batch shares a
+// row between several workgroups, each of which copies and patches its own slice of whole 32-token words (every one of
+// them builds the rank tables of the whole row: a rank counts all the ids before it), so they need no meeting.
 // The usual way, as in the batched sampler: an LDS bitmap of the ids the lists name, a popcount prefix per word (rank of
 // an id = perfect hash), per rank the history count and the index of the first bias entry by LDS atomics, then one
 // thread per touched token. Lists too long for the rank tables (LDS left after the bitmap / 8 bytes per entry) are
@@ -32,15 +34,49 @@ struct AdjustArgs {
     float* out;
     uint64_t out_stride;
     uint32_t lds_bytes;
+    uint32_t parts;  // workgroups per row
 };
 
 __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
-    const uint32_t row = blockIdx.x, t = threadIdx.x, V = A.vocab;
+    const uint32_t row = blockIdx.x / A.parts, part = blockIdx.x % A.parts, t = threadIdx.x, V = A.vocab;
+    const uint32_t nW = (V + 31u) >> 5;
+    const uint32_t wpp = (nW + A.parts - 1u) / A.parts;  // bitmap words per slice
+    const uint32_t wlo = min(part * wpp, nW), whi = min(wlo + wpp, nW);
+    const uint32_t lo = wlo << 5, hi = min(whi << 5, V);
     const size_t esz = A.dtype == 0 ? 4 : 2;
     const unsigned char* base = static_cast<const unsigned char*>(A.logits) + static_cast<size_t>(row) * A.row_stride * esz;
     const uint32_t* allow = A.allow ? A.allow + static_cast<size_t>(row) * A.allow_stride : nullptr;
     float* out = A.out + static_cast<size_t>(row) * A.out_stride;
-    for (uint32_t i = t; i < V; i += WS_BLOCK) {
+    // fp32 rows whose input and output are 16-byte aligned go by 128-bit vectors, four in flight per thread
+    uint32_t done_to = lo;
+    if (A.dtype == 0 && ((reinterpret_cast<uintptr_t>(base) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+        const uint32_t nv = hi >> 2;
+        const float4* __restrict__ xv = reinterpret_cast<const float4*>(base);
+        float4* __restrict__ ov = reinterpret_cast<float4*>(out);
+        for (uint32_t j0 = lo >> 2; j0 < nv; j0 += 4u * WS_BLOCK) {
+            float4 q[4];
+            uint32_t aw[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; ++u) {
+                const uint32_t j = min(j0 + u * WS_BLOCK + t, nv - 1u);  // a slice holds at least one vector when the loop runs
+                q[u] = xv[j];
+                aw[u] = allow ? allow[j >> 3] >> ((j & 7u) << 2) : 0xfu;
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 4u; ++u) {
+                const uint32_t j = j0 + u * WS_BLOCK + t;
+                if (j >= nv) continue;
+                float4 o;
+                o.x = (aw[u] & 1u) ? fmaxf(q[u].x, -INFINITY) : -INFINITY;  // NaN -> -inf
+                o.y = (aw[u] & 2u) ? fmaxf(q[u].y, -INFINITY) : -INFINITY;
+                o.z = (aw[u] & 4u) ? fmaxf(q[u].z, -INFINITY) : -INFINITY;
+                o.w = (aw[u] & 8u) ? fmaxf(q[u].w, -INFINITY) : -INFINITY;
+                ov[j] = o;
+            }
+        }
+        done_to = max(lo, nv << 2);
+    }
+    for (uint32_t i = done_to + t; i < hi; i += WS_BLOCK) {
         float x = A.dtype == 0 ? reinterpret_cast<const float*>(base)[i] : bf16_to_f32(reinterpret_cast<const uint16_t*>(base)[i]);
         x = fmaxf(x, -INFINITY);  // NaN -> -inf
         if (allow && !((allow[i >> 5] >> (i & 31u)) & 1u)) x = -INFINITY;
@@ -57,7 +93,6 @@ __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
     __shared__ uint32_t red_u[WS_WAVES];
     const uint32_t n_all = nb + nh;
     if (n_all == 0) return;
-    const uint32_t nW = (V + 31u) >> 5;
     const uint32_t tab_off = (nW * 6u + 15u) & ~15u;  // bitmap words, 16-bit prefixes, then the rank tables
     if (tab_off < A.lds_bytes && n_all <= (A.lds_bytes - tab_off) / 8u && n_all <= 65535u) {  // uniform
         uint32_t* touched = reinterpret_cast<uint32_t*>(lds);
@@ -104,6 +139,10 @@ __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
         uint32_t r = run0;
         for (uint32_t w = w0; w < w1; ++w) {
             uint32_t bits = touched[w];
+            if (w < wlo || w >= whi) {  // another workgroup's slice
+                r += __popc(bits);
+                continue;
+            }
             while (bits) {
                 const uint32_t id = (w << 5) + static_cast<uint32_t>(__ffs(bits)) - 1u;
                 bits &= bits - 1u;
@@ -137,7 +176,7 @@ __global__ void __launch_bounds__(WS_BLOCK) adjust_rows_kernel(AdjustArgs A) {
     // entry e of the concatenation (bias list, then history) owns its id when no earlier entry names it
     for (uint32_t e = t; e < n_all; e += WS_BLOCK) {
         const int32_t id = id_at(e);
-        if (id < 0 || static_cast<uint32_t>(id) >= V) continue;
+        if (id < 0 || static_cast<uint32_t>(id) < lo || static_cast<uint32_t>(id) >= hi) continue;
         bool owner = true;
         for (uint32_t k = 0; k < e && owner; ++k) owner = id_at(k) != id;
         if (!owner) continue;
