@@ -24,7 +24,7 @@ struct DeviceError : std::runtime_error {
     int code;
 };
 
-// optional per-row penalties and bias, all host arrays (copied to the device per call)
+// optional per-row penalties and bias, all host arrays (copied per call to pinned memory that the device reads in place)
 struct RowAdjust {
     const std::int32_t* history = nullptr;  // token ids seen so far
     std::uint32_t n_history = 0;
@@ -80,7 +80,6 @@ private:
     void* stream_;
     RowAdjust adj_;
     Dev* dev_;
-    std::vector<float> row_host_;
     std::vector<std::uint8_t> marks_;
     std::uint32_t last_flags_ = 0;
     std::vector<Ready> ready_;

@@ -706,13 +706,106 @@ __device__ __noinline__ TailCut tail_cut(const TailIn in) {
     return TailCut{prefix, need};
 }
 
+// Tokens of a row picked by keep(i, logit) - bit 0: kept outright, bit 1: kept while fewer than n_equal tokens with this
+// bit came before it - written out in ascending token id. Every wave takes a stretch of consecutive 256-token tiles, four
+// consecutive tokens per lane and tile (one 128-bit load of fp32, 64 bits of bf16): a first pass counts what the stretch
+// keeps, the waves' counts are scanned once, and a second pass, fed from the cache, ranks and writes. Kept tokens are few,
+// so the second pass does its lane scan only for the tiles that hold one; the workgroup meets at two barriers in all.
+template <class KEEP>
+__device__ __forceinline__ void write_in_id_order(const RowView& rv, uint32_t n_equal, int32_t* kid, float* klg, uint32_t kept_cap, KEEP&& keep) {
+    __shared__ uint32_t w_cnt[2 * WS_WAVES];
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6, V = rv.V;
+    const uint32_t tiles = (V + 255u) >> 8, per_wave = (tiles + WS_WAVES - 1u) / WS_WAVES;
+    const uint32_t lo = min(wave * per_wave, tiles) << 8, hi = min(min((wave + 1u) * per_wave, tiles) << 8, V);
+    const bool wide = (reinterpret_cast<uintptr_t>(rv.base) & (rv.dtype == 0 ? 15u : 7u)) == 0;
+    // flags of tokens i .. i + 3 (bits 0-3: kept outright, bits 4-7: kept while ties last) and their logits
+    auto look = [&](uint32_t i, float (&x)[4]) -> uint32_t {
+        if (i >= hi) return 0u;
+        if (wide && i + 4u <= V) {
+            if (rv.dtype == 0) {
+                const float4 q = *reinterpret_cast<const float4*>(static_cast<const float*>(rv.base) + i);
+                x[0] = q.x, x[1] = q.y, x[2] = q.z, x[3] = q.w;
+            } else {
+                const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(rv.base) + i);
+                x[0] = bf16_to_f32(static_cast<uint16_t>(q.x)), x[1] = bf16_to_f32(static_cast<uint16_t>(q.x >> 16));
+                x[2] = bf16_to_f32(static_cast<uint16_t>(q.y)), x[3] = bf16_to_f32(static_cast<uint16_t>(q.y >> 16));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = fmaxf(x[e], -INFINITY);  // NaN -> -inf
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = i + e < V ? raw_logit(rv, i + e) : -INFINITY;
+        }
+        // masked-out tokens and those the lists touch (four tokens from a multiple of four share a bitmap word)
+        const uint32_t tb = rv.touched ? (rv.touched[i >> 5] >> (i & 31u)) & 0xfu : 0u;
+        const uint32_t ab = rv.allow ? (rv.allow[i >> 5] >> (i & 31u)) & 0xfu : 0xfu;
+        if (tb | (ab ^ 0xfu)) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (i + e < V) x[e] = adjusted_logit(rv, i + e);
+        }
+        uint32_t f = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t k = i + e < V ? keep(i + e, x[e]) : 0u;
+            f |= ((k & 1u) << e) | ((k >> 1) << (4 + e));
+        }
+        return f;
+    };
+    uint32_t nk = 0, nt = 0;
+#pragma unroll 4
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
+        float x[4];
+        const uint32_t f = look(i0 + 4u * lane, x);
+        nk += __popc(f & 0xfu);
+        nt += __popc(f >> 4);
+    }
+    nk = wave_sum(nk);
+    nt = wave_sum(nt);
+    __syncthreads();  // (w_cnt may still be read by an earlier call)
+    if (lane == 0) {
+        w_cnt[wave] = nk;
+        w_cnt[WS_WAVES + wave] = nt;
+    }
+    __syncthreads();
+    uint32_t base = 0, tail_base = 0;
+    for (uint32_t w = 0; w < wave; ++w) {
+        base += w_cnt[w];
+        tail_base += w_cnt[WS_WAVES + w];
+    }
+    if (!(nk | nt)) return;  // nothing kept in this wave's stretch (uniform over the wave; no barrier follows)
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
+        float x[4];
+        const uint32_t i = i0 + 4u * lane;
+        const uint32_t f = look(i, x);
+        if (!__ballot(f != 0u)) continue;
+        const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
+        const uint32_t inc = wave_incl_scan(mine);
+        uint32_t kb = base + ((inc - mine) & 0xffffu), tb = tail_base + ((inc - mine) >> 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bool tie = (f >> (4 + e)) & 1u;
+            const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
+            const uint32_t o = kb + min(tb, n_equal);
+            if (k && o < kept_cap) {
+                kid[o] = static_cast<int32_t>(i + e);
+                if (klg) klg[o] = x[e];
+            }
+            kb += (f >> e) & 1u;
+            tb += tie ? 1u : 0u;
+        }
+        const uint32_t tot = last_lane(inc);
+        base += tot & 0xffffu;
+        tail_base += tot >> 16;
+    }
+}
+
 // The kept set of a row in ascending id order (the optional dump): every token whose key is at or above `kept_key`, and
 // `want` zero-mass candidates (tail_cut). A function of its own, like the exact path: it runs for callers that ask for
 // the dump only, and the kernel keeps its registers for what every row needs.
 __device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float* klg, uint32_t kept_cap) {
     extern __shared__ __align__(16) unsigned char lds[];
-    __shared__ uint32_t d_red[WS_WAVES];
-    const uint32_t t = threadIdx.x, V = in.V;
+    const uint32_t V = in.V;
     RowView rv;
     rv.base = in.base;
     rv.V = V;
@@ -726,34 +819,19 @@ __device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float*
     TailCut cut{0u, 0u};
     if (in.want) cut = tail_cut(in);  // uniform
     __syncthreads();
-    uint32_t base = 0, tail_base = 0;
-    // id order needs consecutive ids per tile: tiles of WS_BLOCK consecutive tokens, one per thread
-    for (uint32_t i0 = 0; i0 < V; i0 += WS_BLOCK) {
-        const uint32_t i = i0 + t;
-        float x = -INFINITY;
-        uint32_t keep = 0, tl = 0;
-        if (i < V) {
-            x = adjusted_logit(rv, i);
-            keep = key64(x, i) >= in.kept_key;
-            if (in.want && !keep && bin_of(in.aq, in.c64, x) >= static_cast<uint32_t>(kTail)) {
-                // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes;
-                // among those with exactly that logit the lowest ids
-                keep = key32(x) > cut.key;
-                tl = key32(x) == cut.key;
-            }
+    const uint64_t kept_key = in.kept_key;
+    const bool want = in.want != 0u;
+    const float aq = in.aq, c64 = in.c64;
+    write_in_id_order(rv, cut.n_equal, kid, klg, kept_cap, [&](uint32_t i, float x) -> uint32_t {
+        uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
+        if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
+            // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes; among those
+            // with exactly that logit the lowest ids
+            keep = key32(x) > cut.key ? 1u : 0u;
+            if (key32(x) == cut.key) keep = 2u;
         }
-        uint32_t tot;
-        const uint32_t before = block_excl_scan(keep | (tl << 16), d_red, &tot);
-        const uint32_t tl_before = tail_base + (before >> 16);
-        if (tl && tl_before < cut.n_equal) keep = 1;
-        const uint32_t o = base + (before & 0xffffu) + min(tl_before, cut.n_equal);
-        if (keep && o < kept_cap) {
-            kid[o] = static_cast<int32_t>(i);
-            if (klg) klg[o] = x;
-        }
-        base += tot & 0xffffu;
-        tail_base += tot >> 16;
-    }
+        return keep;
+    });
 }
 
 struct ExactIn {
@@ -3519,31 +3597,15 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             TailCut cut{0u, 0u};
             if (tail_extra) cut = tail_cut(in);  // uniform
             __syncthreads();
-            uint32_t base = 0, tail_base = 0;
-            for (uint32_t i0 = 0; i0 < V; i0 += WS_BLOCK) {
-                const uint32_t i = i0 + t;
-                float x = -INFINITY;
-                uint32_t keep = 0, tl = 0;
-                if (i < V) {
-                    x = adjusted_logit(rv, i);
-                    keep = key64(x, i) >= kept_key;
-                    if (tail_extra && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
-                        keep = key32(x) > cut.key;
-                        tl = key32(x) == cut.key;
-                    }
+            const bool want = tail_extra != 0u;
+            write_in_id_order(rv, cut.n_equal, kid, klg, A.kept_cap, [&](uint32_t i, float x) -> uint32_t {
+                uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
+                if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
+                    keep = key32(x) > cut.key ? 1u : 0u;
+                    if (key32(x) == cut.key) keep = 2u;
                 }
-                uint32_t tot;
-                const uint32_t before = block_excl_scan(keep | (tl << 16), red_u, &tot);
-                const uint32_t tl_before = tail_base + (before >> 16);
-                if (tl && tl_before < cut.n_equal) keep = 1;
-                const uint32_t o = base + (before & 0xffffu) + min(tl_before, cut.n_equal);
-                if (keep && o < A.kept_cap) {
-                    kid[o] = static_cast<int32_t>(i);
-                    if (klg) klg[o] = x;
-                }
-                base += tot & 0xffffu;
-                tail_base += tot >> 16;
-            }
+                return keep;
+            });
         }
     }
 }

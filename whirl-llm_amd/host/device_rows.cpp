@@ -1,7 +1,12 @@
 // sampling::DeviceRows: a RowSource whose rows are sampled on the GPU through the C ABI (whirl_sampling_abi.h).
-// One prepareRow = one launch of ws_sample_batch on that row with the kept-set dump on, one small download, and a
-// sort of the kept candidates on the host; prefetchRows does the launch and the download for several rows at once.
+// One prepareRow = one launch of ws_sample_batch on that row with the kept-set dump on, one wait for the stream, and
+// a sort of the kept candidates on the host; prefetchRows does the launch for several rows at once.
 // No vocabulary-sized work happens here unless the device flags the row.
+// Parameters, penalty lists, results and kept sets live in pinned host memory that the device addresses directly
+// (hipHostMalloc): the host writes the few hundred bytes a row needs, the kernel reads them over the bus, writes what
+// it kept straight back, and no copy command sits before or after the launch - a decode step is one launch and one
+// stream wait. Everything here waits for the stream before it returns, so the host never rewrites a block that a
+// launch still reads.
 #include "sampling/device_rows.h"
 
 #include "whirl_sampling_abi.h"
@@ -80,7 +85,7 @@ struct DeviceRows::Dev {
         return v;
     }
     std::uint32_t row_cap = 0;     // rows the blocks below are sized for
-    std::uint32_t rows_now = 0;    // rows of the parameter block that is on the device
+    // pinned host memory, read and written by the kernels in place
     unsigned char* prm = nullptr;
     unsigned char* res = nullptr;
     std::int32_t* kept_ids = nullptr;  // [row_cap][cap]
@@ -92,15 +97,14 @@ struct DeviceRows::Dev {
     std::int32_t* topk_ids = nullptr;  // escalation: ids | vals | stats of one row, kBig candidates
     float* topk_vals = nullptr;
     float* topk_stats = nullptr;
+    float* row_host = nullptr;         // loadFullRow's buffer: a pinned target makes the download one DMA transfer
+    // device memory
     float* adjusted = nullptr;         // escalation: penalised copy of the row (ws_adjust_rows)
     // The sampler's workspace: with it a batch of a few rows has each row worked on by several workgroups, and long
     // vocabularies take the history tokens' logits from the sweep. Zero-filled when it is allocated: what it is used for
     // depends on the vocabulary alone, which this object never changes, and the use that needs zeros puts them back.
     unsigned char* work = nullptr;
     std::uint64_t work_cap = 0;
-    std::vector<unsigned char> h_prm, h_res;
-    std::vector<std::int32_t> h_ids;
-    std::vector<float> h_vals;
 };
 
 // one row the device has filtered already, waiting on the host for its prepareRow
@@ -115,15 +119,15 @@ struct DeviceRows::Ready {
 DeviceRows::DeviceRows(const float* d_logits, std::uint32_t rows, std::uint32_t n_vocab, void* stream)
     : logits_(d_logits), rows_(rows), vocab_(n_vocab), stream_(stream), dev_(new Dev), marks_(n_vocab, 0) {
     check(ws_probe(), "ws_probe");
-    dev_->h_ids.resize(kBig);
-    dev_->h_vals.resize(kBig);
 }
 
 DeviceRows::~DeviceRows() {
     for (void* p : {static_cast<void*>(dev_->prm), static_cast<void*>(dev_->res), static_cast<void*>(dev_->kept_ids),
                     static_cast<void*>(dev_->kept_logits), static_cast<void*>(dev_->hist), static_cast<void*>(dev_->bias_ids),
                     static_cast<void*>(dev_->bias_vals), static_cast<void*>(dev_->topk_ids), static_cast<void*>(dev_->topk_vals),
-                    static_cast<void*>(dev_->topk_stats), static_cast<void*>(dev_->adjusted), static_cast<void*>(dev_->work)})
+                    static_cast<void*>(dev_->topk_stats), static_cast<void*>(dev_->row_host)})
+        if (p) (void)hipHostFree(p);
+    for (void* p : {static_cast<void*>(dev_->adjusted), static_cast<void*>(dev_->work)})
         if (p) (void)hipFree(p);
     delete dev_;
 }
@@ -138,49 +142,60 @@ void DeviceRows::newCycle() {
     adjusted_row_ = kNoRow;
 }
 
-// Parameters of `n` rows that share sampler `s` and the current penalties, and the penalty lists once per row, go to
-// the device (the lists are replicated because a batch addresses them through one ascending offset array).
+namespace {
+template <class T>
+void pinned(T** p, std::size_t bytes) {
+    checkHip(hipHostMalloc(reinterpret_cast<void**>(p), bytes, hipHostMallocDefault), "hipHostMalloc");
+}
+}  // namespace
+
+// Parameters of `n` rows that share sampler `s` and the current penalties, and the penalty lists once per row, written
+// where the device reads them (the lists are replicated because a batch addresses them through one ascending offset
+// array). The stream is idle when this runs.
 void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
-    auto stream = static_cast<hipStream_t>(stream_);
     Dev& d = *dev_;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
     if (n > d.row_cap) {
         for (void* p : {static_cast<void*>(d.prm), static_cast<void*>(d.res), static_cast<void*>(d.kept_ids), static_cast<void*>(d.kept_logits)})
-            if (p) (void)hipFree(p);
+            if (p) (void)hipHostFree(p);
         d.prm = d.res = nullptr;
         d.kept_ids = nullptr;
         d.kept_logits = nullptr;
+        d.row_cap = 0;
+        pinned(&d.prm, Dev::paramBytes(n));
+        pinned(&d.res, Dev::resultBytes(n));
+        pinned(&d.kept_ids, std::size_t{n} * cap * sizeof(std::int32_t));
+        pinned(&d.kept_logits, std::size_t{n} * cap * sizeof(float));
         d.row_cap = n;
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.prm), Dev::paramBytes(n)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.res), Dev::resultBytes(n)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.kept_ids), std::size_t{n} * cap * sizeof(std::int32_t)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.kept_logits), std::size_t{n} * cap * sizeof(float)), "hipMalloc");
     }
     const std::size_t nh = adj_.n_history, nb = adj_.n_bias;
     if (nh * n > d.hist_cap) {
-        if (d.hist) (void)hipFree(d.hist);
+        if (d.hist) (void)hipHostFree(d.hist);
         d.hist = nullptr;
-        d.hist_cap = std::max(nh * n, 2 * d.hist_cap);
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.hist), d.hist_cap * sizeof(std::int32_t)), "hipMalloc");
+        const std::size_t want = std::max(nh * n, 2 * d.hist_cap);
+        d.hist_cap = 0;
+        pinned(&d.hist, want * sizeof(std::int32_t));
+        d.hist_cap = want;
     }
     if (nb * n > d.bias_cap) {
-        if (d.bias_ids) (void)hipFree(d.bias_ids);
-        if (d.bias_vals) (void)hipFree(d.bias_vals);
+        if (d.bias_ids) (void)hipHostFree(d.bias_ids);
+        if (d.bias_vals) (void)hipHostFree(d.bias_vals);
         d.bias_ids = nullptr;
         d.bias_vals = nullptr;
-        d.bias_cap = std::max(nb * n, 2 * d.bias_cap);
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.bias_ids), d.bias_cap * sizeof(std::int32_t)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.bias_vals), d.bias_cap * sizeof(float)), "hipMalloc");
+        const std::size_t want = std::max(nb * n, 2 * d.bias_cap);
+        d.bias_cap = 0;
+        pinned(&d.bias_ids, want * sizeof(std::int32_t));
+        pinned(&d.bias_vals, want * sizeof(float));
+        d.bias_cap = want;
     }
     for (std::uint32_t r = 0; r < n; ++r) {
-        if (nh) checkHip(hipMemcpyAsync(d.hist + r * nh, adj_.history, nh * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+        if (nh) std::memcpy(d.hist + r * nh, adj_.history, nh * sizeof(std::int32_t));
         if (nb) {
-            checkHip(hipMemcpyAsync(d.bias_ids + r * nb, adj_.bias_ids, nb * sizeof(std::int32_t), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-            checkHip(hipMemcpyAsync(d.bias_vals + r * nb, adj_.bias_vals, nb * sizeof(float), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
+            std::memcpy(d.bias_ids + r * nb, adj_.bias_ids, nb * sizeof(std::int32_t));
+            std::memcpy(d.bias_vals + r * nb, adj_.bias_vals, nb * sizeof(float));
         }
     }
-    d.h_prm.assign(Dev::paramBytes(n), 0);
-    const Dev::ParamView h = Dev::view(d.h_prm.data(), n);
+    const Dev::ParamView h = Dev::view(d.prm, n);
     for (std::uint32_t r = 0; r < n; ++r) {
         h.top_p[r] = s.top_p;
         h.min_p[r] = s.min_p;
@@ -196,9 +211,6 @@ void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
         h.hist_off[r] = static_cast<std::uint32_t>(r * nh);
         h.bias_off[r] = static_cast<std::uint32_t>(r * nb);
     }
-    // the pageable staging buffer is read before the call returns, so it may be rewritten by the next call
-    checkHip(hipMemcpyAsync(d.prm, d.h_prm.data(), d.h_prm.size(), hipMemcpyHostToDevice, stream), "hipMemcpyAsync");
-    d.rows_now = n;
 }
 
 // One launch of the fused sampler over rows [gr0, gr0 + n), all with sampler `s` and the current penalties; what it
@@ -261,10 +273,8 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
     b.workspace_bytes = d.work_cap;
     check(ws_sample_batch(stream_, &b), "ws_sample_batch");
 
-    d.h_res.resize(Dev::resultBytes(n));
-    checkHip(hipMemcpyAsync(d.h_res.data(), d.res, d.h_res.size(), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-    checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-    const Dev::ResultView h = Dev::view_res(d.h_res.data(), n);
+    checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");  // results and kept sets are in host memory now
+    const Dev::ResultView& h = o;
     ready_.clear();
     ready_.resize(n);
     const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
@@ -276,12 +286,9 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
         q.m = h.stats[2 * r];
         q.sum = h.stats[2 * r + 1];
         if ((q.flags & unresolved) || q.n_kept > cap) continue;  // such a row is escalated when it is asked for
-        q.ids.resize(q.n_kept);
-        q.logits.resize(q.n_kept);
-        checkHip(hipMemcpyAsync(q.ids.data(), d.kept_ids + std::size_t{r} * cap, q.n_kept * sizeof(std::int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-        checkHip(hipMemcpyAsync(q.logits.data(), d.kept_logits + std::size_t{r} * cap, q.n_kept * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+        q.ids.assign(d.kept_ids + std::size_t{r} * cap, d.kept_ids + std::size_t{r} * cap + q.n_kept);
+        q.logits.assign(d.kept_logits + std::size_t{r} * cap, d.kept_logits + std::size_t{r} * cap + q.n_kept);
     }
-    checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     ready_key_ = {s.inv_t, s.top_k, s.top_p, s.min_p};
 }
 
@@ -339,7 +346,7 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
     const float* src = logits_ + static_cast<std::size_t>(gr) * vocab_;
     if (adj_.n_history || adj_.n_bias) {
         if (!d.adjusted) checkHip(hipMalloc(reinterpret_cast<void**>(&d.adjusted), vocab_ * sizeof(float)), "hipMalloc");
-        uploadInputs(s, 1);  // the row may come from an earlier batch: its lists and parameters go up again
+        uploadInputs(s, 1);  // the row may come from an earlier batch: its lists and parameters are written again
         const Dev::ParamView p = Dev::view(d.prm, 1);
         ws_adjust a{};
         a.logits = src;
@@ -366,28 +373,24 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
         adjusted_row_ = gr;
     }
     if (!d.topk_ids) {
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_ids), kBig * sizeof(std::int32_t)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_vals), kBig * sizeof(float)), "hipMalloc");
-        checkHip(hipMalloc(reinterpret_cast<void**>(&d.topk_stats), 2 * sizeof(float)), "hipMalloc");
+        pinned(&d.topk_ids, kBig * sizeof(std::int32_t));
+        pinned(&d.topk_vals, kBig * sizeof(float));
+        pinned(&d.topk_stats, 2 * sizeof(float));
     }
     Cand* c = s.cands->data();
     bool first = true;
     for (std::uint32_t k : {std::min(kSmall, vocab_), std::min(kBig, vocab_)}) {
         check(ws_topk_rows(stream_, src, static_cast<int>(vocab_), static_cast<int>(k), s.inv_t, d.topk_ids, d.topk_vals, d.topk_stats, 1),
               "ws_topk_rows");
-        float stats[2];
-        checkHip(hipMemcpyAsync(d.h_ids.data(), d.topk_ids, k * sizeof(std::int32_t), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-        checkHip(hipMemcpyAsync(d.h_vals.data(), d.topk_vals, k * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-        checkHip(hipMemcpyAsync(stats, d.topk_stats, sizeof stats, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
-        checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+        checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");  // the kernel wrote the list into host memory
         if (first) {  // the row's maximum and normaliser, once (the second call recomputes the same values)
-            s.m = stats[0];
-            s.sum = stats[1];
+            s.m = d.topk_stats[0];
+            s.sum = d.topk_stats[1];
         } else {
             s.big_used += 1;
         }
         first = false;
-        for (std::uint32_t j = 0; j < k; ++j) c[j] = {static_cast<std::uint32_t>(d.h_ids[j]), d.h_vals[j], 0.0};
+        for (std::uint32_t j = 0; j < k; ++j) c[j] = {static_cast<std::uint32_t>(d.topk_ids[j]), d.topk_vals[j], 0.0};
         if (filterCands(s, k, false)) return;
     }
     s.full_used += 1;
@@ -398,12 +401,12 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
 
 const float* DeviceRows::loadFullRow(std::uint32_t gr) {
     if (gr >= rows_) throw DeviceError("loadFullRow", WS_E_INVALID, "loadFullRow: row out of range");
-    row_host_.resize(vocab_);
+    if (!dev_->row_host) pinned(&dev_->row_host, vocab_ * sizeof(float));
     auto stream = static_cast<hipStream_t>(stream_);
     const float* src = gr == adjusted_row_ ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
-    checkHip(hipMemcpyAsync(row_host_.data(), src, vocab_ * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
+    checkHip(hipMemcpyAsync(dev_->row_host, src, vocab_ * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-    return row_host_.data();
+    return dev_->row_host;
 }
 
 float DeviceRows::logitAt(std::uint32_t gr, std::uint32_t t) {
