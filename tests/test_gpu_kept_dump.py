@@ -1,0 +1,78 @@
+"""GPU: the optional kept-set dump of ws_sample_batch (kept_ids / kept_logits) over each of its routes, against the oracle's
+kept candidates (ids as a set in ascending order, penalty-applied logits bit for bit; gpu_cases.compare_rows):
+- a top-k row takes its kept set from the gathered candidates (bucket finish, and the sort-based finish of tie-heavy rows),
+  on rows held by one workgroup and on rows shared by several;
+- every other row is read once more by its workgroup (one pass, the waves' finds lined up in LDS), or twice when a wave
+  finds more than its share of the LDS holds or when a top-k reaches into the zero-mass tail (ties by token id)."""
+import numpy as np
+import pytest
+
+import gpu_cases as gc
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(c, kept_cap, rows=None, **more):
+    d = gc.upload(c)
+    smp = gc.sampler_for(c, d, 1, kept_cap=kept_cap, **more).run()
+    rows = range(c["rows"]) if rows is None else rows
+    res = gc.compare_rows(c, smp, rows, 1)
+    nk = smp.n_kept.cpu().numpy()
+    return res, nk
+
+
+@pytest.mark.parametrize("rows", [1, 3, 40])
+def test_top_k_rows_dump_from_their_candidates(rows):
+    """Top-k 20 / 50 with and without top-p and min-p, penalties and bias: one row alone (shared by eight workgroups), three
+    rows, forty rows (one workgroup each)."""
+    c = gc.make_cfg2(rows=rows, n_hist=1024, n_bias=100)
+    c["top_k"][:] = np.where(np.arange(rows) % 2 == 0, 20, 50)
+    c["top_p"][rows // 2:] = 1.0
+    c["min_p"][::3] = 0.0
+    res, nk = _check(c, 256)
+    assert res["exact"] >= rows - 1 and nk.max() <= 50
+
+
+def test_top_k_rows_with_an_allow_mask():
+    c = gc.make_cfg5(rows=4, V=151936, n_hist=2048, n_bias=100)
+    c["top_k"][:] = [40, 200, 1000, 3000]  # the last two are beyond the candidates ranked by id: the pass over the row
+    res, nk = _check(c, 4096)
+    assert res["exact"] >= 3
+
+
+def test_tie_heavy_bf16_top_k_rows():
+    """Coarse bf16 logits put hundreds of equal logits at the cut: the sort-based finish, whose first n sorted keys are
+    the kept set."""
+    c = gc.make_cfg3(rows=6)
+    c["top_k"][:] = [50, 300, 900, 50, 300, 900]
+    c["top_p"][3:] = 1.0
+    res, nk = _check(c, 1024)
+    assert res["exact"] >= 5
+
+
+def test_top_p_rows_one_pass_and_two():
+    """Top-p alone keeps thousands of tokens (one pass, lined up in LDS); on a flat row it keeps most of the row, more than
+    the LDS lines hold (two passes)."""
+    c = gc.make_tile(rows=3, V=151936, n_hist=512)
+    res, nk = _check(c, 16384)
+    assert res["exact"] >= 2 and nk.min() > 1000
+    rng = np.random.default_rng(5)
+    f = gc.make_tile(rows=2, V=40000, n_hist=128)
+    f["logits"] = (rng.standard_normal((2, 40000)) * 0.05).astype(np.float32)
+    f["top_p"][:] = 0.9
+    res, nk = _check(f, 40000)
+    assert res["exact"] == 2 and nk.min() > 30000
+
+
+def test_top_k_into_the_zero_mass_tail():
+    """A top-k larger than the number of tokens with any mass keeps zero-mass candidates too - those with the largest
+    logits, the lowest ids among equals: nearly everything is masked out here, so the ties are the masked tokens."""
+    c = gc.make_cfg2(rows=2, V=32000, n_hist=64, n_bias=0)
+    rng = np.random.default_rng(9)
+    allow = rng.random((2, 32000)) < 0.003
+    c["allow"] = np.ascontiguousarray(np.packbits(allow, axis=1, bitorder="little").view(np.uint32))
+    c["top_k"][:] = 500
+    c["top_p"][:] = 1.0
+    c["min_p"][:] = 0.0
+    res, nk = _check(c, 1024)
+    assert res["exact"] == 2 and (nk == 500).all()

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #ifndef WS_BLOCK
 #define WS_BLOCK 1024  // threads per workgroup; the fused sweep is compiled with 512 (256 registers per thread)
 #endif

@@ -707,62 +707,132 @@ __device__ __noinline__ TailCut tail_cut(const TailIn in) {
 }
 
 // Tokens of a row picked by keep(i, logit) - bit 0: kept outright, bit 1: kept while fewer than n_equal tokens with this
-// bit came before it - written out in ascending token id. Every wave takes a stretch of consecutive 256-token tiles, four
-// consecutive tokens per lane and tile (one 128-bit load of fp32, 64 bits of bf16): a first pass counts what the stretch
-// keeps, the waves' counts are scanned once, and a second pass, fed from the cache, ranks and writes. Kept tokens are few,
-// so the second pass does its lane scan only for the tiles that hold one; the workgroup meets at two barriers in all.
+// bit came before it (only with `ties`) - written out in ascending token id; keep is asked only about logits at or above
+// `floor` (one comparison settles nearly every token). Every wave takes a stretch of consecutive 256-token tiles, four
+// consecutive tokens per lane and tile (one 128-bit load of fp32, 64 bits of bf16), sixteen tiles on their way at a
+// time: one workgroup reads the row alone here, from other dies' caches or from memory, and only many loads in flight
+// hide that distance. What a wave keeps it lines up, in order, in its share of `room` (LDS, 64 KB, idle by now); the
+// waves' counts are scanned once and every wave copies its line to its place in the output: one pass over the row, two
+// barriers. A wave that keeps more than its share holds (or a row with ties) sends the workgroup through two plain
+// passes instead - count, then rank and write.
 template <class KEEP>
-__device__ __forceinline__ void write_in_id_order(const RowView& rv, uint32_t n_equal, int32_t* kid, float* klg, uint32_t kept_cap, KEEP&& keep) {
+__device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, uint32_t n_equal, float floor, int32_t* kid, float* klg,
+                                                  uint32_t kept_cap, uint64_t* room, KEEP&& keep) {
     __shared__ uint32_t w_cnt[2 * WS_WAVES];
+    constexpr uint32_t kShare = 8192u / WS_WAVES;  // entries of `room` per wave
+    constexpr uint32_t kAhead = 16u;
     const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6, V = rv.V;
     const uint32_t tiles = (V + 255u) >> 8, per_wave = (tiles + WS_WAVES - 1u) / WS_WAVES;
     const uint32_t lo = min(wave * per_wave, tiles) << 8, hi = min(min((wave + 1u) * per_wave, tiles) << 8, V);
-    const bool wide = (reinterpret_cast<uintptr_t>(rv.base) & (rv.dtype == 0 ? 15u : 7u)) == 0;
-    // flags of tokens i .. i + 3 (bits 0-3: kept outright, bits 4-7: kept while ties last) and their logits
-    auto look = [&](uint32_t i, float (&x)[4]) -> uint32_t {
-        if (i >= hi) return 0u;
-        if (wide && i + 4u <= V) {
-            if (rv.dtype == 0) {
-                const float4 q = *reinterpret_cast<const float4*>(static_cast<const float*>(rv.base) + i);
-                x[0] = q.x, x[1] = q.y, x[2] = q.z, x[3] = q.w;
-            } else {
-                const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(rv.base) + i);
-                x[0] = bf16_to_f32(static_cast<uint16_t>(q.x)), x[1] = bf16_to_f32(static_cast<uint16_t>(q.x >> 16));
-                x[2] = bf16_to_f32(static_cast<uint16_t>(q.y)), x[3] = bf16_to_f32(static_cast<uint16_t>(q.y >> 16));
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] = fmaxf(x[e], -INFINITY);  // NaN -> -inf
+    const uint32_t lo_safe = lo < V ? lo : 0u;
+    // whole: every quad of the stretch lies inside the row and is read by one aligned vector load
+    const bool whole = (reinterpret_cast<uintptr_t>(rv.base) & (rv.dtype == 0 ? 15u : 7u)) == 0 && (hi & 3u) == 0;
+    // raw bits of tokens i .. i + 3 as floats (bf16 widened); a lane past the stretch re-reads the stretch's first tokens
+    // and is ignored
+    auto fetch = [&](uint32_t i, auto whole_) -> uint4 {
+        if (i >= hi) i = lo_safe;
+        if constexpr (decltype(whole_)::value) {
+            if (rv.dtype == 0) return *reinterpret_cast<const uint4*>(static_cast<const float*>(rv.base) + i);
+            const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(rv.base) + i);
+            return make_uint4(q.x << 16, q.x & 0xffff0000u, q.y << 16, q.y & 0xffff0000u);
         } else {
+            uint32_t w[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] = i + e < V ? raw_logit(rv, i + e) : -INFINITY;
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t j = min(i + e, V - 1u);
+                w[e] = rv.dtype == 0 ? static_cast<const uint32_t*>(rv.base)[j] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[j]) << 16;
+            }
+            return make_uint4(w[0], w[1], w[2], w[3]);
         }
+    };
+    // flags of tokens i .. i + 3 (bits 0-3: kept outright, bits 4-7: kept while ties last) and their logits
+    auto judge = [&](uint32_t i, const uint4 raw, float (&x)[4]) -> uint32_t {
+        x[0] = fmaxf(__uint_as_float(raw.x), -INFINITY), x[1] = fmaxf(__uint_as_float(raw.y), -INFINITY);  // NaN -> -inf
+        x[2] = fmaxf(__uint_as_float(raw.z), -INFINITY), x[3] = fmaxf(__uint_as_float(raw.w), -INFINITY);
+        const uint32_t live = i >= hi ? 0u : (i + 4u <= V ? 0xfu : (1u << (V - i)) - 1u);  // tokens of the quad inside the stretch
         // masked-out tokens and those the lists touch (four tokens from a multiple of four share a bitmap word)
-        const uint32_t tb = rv.touched ? (rv.touched[i >> 5] >> (i & 31u)) & 0xfu : 0u;
-        const uint32_t ab = rv.allow ? (rv.allow[i >> 5] >> (i & 31u)) & 0xfu : 0xfu;
-        if (tb | (ab ^ 0xfu)) {
+        const uint32_t iw = min(i, V - 1u);
+        const uint32_t tb = rv.touched ? (rv.touched[iw >> 5] >> (iw & 31u)) & live : 0u;
+        const uint32_t ab = rv.allow ? (rv.allow[iw >> 5] >> (iw & 31u)) | ~live : 0xfu;
+        if (tb | (~ab & 0xfu)) {  // (no second look at memory: an untouched, allowed token keeps what was loaded)
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (i + e < V) x[e] = adjusted_logit(rv, i + e);
+            for (int e = 0; e < 4; ++e) {
+                if ((tb >> e) & 1u) x[e] = rv.pv[rank_of(rv, i + e)];
+                else if (!((ab >> e) & 1u)) x[e] = -INFINITY;
+            }
         }
+        const uint32_t c = ((x[0] >= floor ? 1u : 0u) | (x[1] >= floor ? 2u : 0u) | (x[2] >= floor ? 4u : 0u) | (x[3] >= floor ? 8u : 0u)) & live;
         uint32_t f = 0;
+        if (c) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t k = i + e < V ? keep(i + e, x[e]) : 0u;
-            f |= ((k & 1u) << e) | ((k >> 1) << (4 + e));
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t k = (c >> e) & 1u ? keep(i + e, x[e]) : 0u;
+                f |= ((k & 1u) << e) | ((k >> 1) << (4 + e));
+            }
         }
         return f;
     };
+    if (!ties) {  // uniform
+        uint64_t* line = room + wave * kShare;
+        uint32_t wc = 0;
+        auto sweep = [&](auto whole_) {
+            for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead) {
+                uint4 raw[kAhead];
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, whole_);
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) {
+                    float x[4];
+                    const uint32_t i = i0 + 256u * u + 4u * lane;
+                    const uint32_t f = judge(i, raw[u], x) & 0xfu;
+                    if (!__ballot(f != 0u)) continue;
+                    const uint32_t mine = __popc(f);
+                    const uint32_t inc = wave_incl_scan(mine);
+                    uint32_t o = wc + inc - mine;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (!((f >> e) & 1u)) continue;
+                        if (o < kShare) line[o] = (static_cast<uint64_t>(i + e) << 32) | __float_as_uint(x[e]);
+                        ++o;
+                    }
+                    wc += last_lane(inc);
+                }
+            }
+        };
+        if (whole) sweep(std::true_type{});
+        else sweep(std::false_type{});
+        __syncthreads();  // (w_cnt may still be read by an earlier call)
+        if (lane == 0) w_cnt[wave] = wc;
+        __syncthreads();
+        uint32_t base = 0;
+        bool fits = true;
+        for (uint32_t w = 0; w < WS_WAVES; ++w) {
+            const uint32_t c = w_cnt[w];
+            if (w < wave) base += c;
+            fits = fits && c <= kShare;
+        }
+        if (fits) {  // uniform over the workgroup
+            for (uint32_t j = lane; j < wc; j += 64u) {
+                const uint64_t en = line[j];
+                if (base + j < kept_cap) {
+                    kid[base + j] = static_cast<int32_t>(en >> 32);
+                    if (klg) klg[base + j] = __uint_as_float(static_cast<uint32_t>(en));
+                }
+            }
+            return;
+        }
+    }
+    // ---- two passes, a tile at a time (rare)
     uint32_t nk = 0, nt = 0;
-#pragma unroll 4
     for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
         float x[4];
-        const uint32_t f = look(i0 + 4u * lane, x);
+        const uint32_t f = judge(i0 + 4u * lane, fetch(i0 + 4u * lane, std::false_type{}), x);
         nk += __popc(f & 0xfu);
         nt += __popc(f >> 4);
     }
     nk = wave_sum(nk);
     nt = wave_sum(nt);
-    __syncthreads();  // (w_cnt may still be read by an earlier call)
+    __syncthreads();  // (w_cnt may still be read: the attempt above, an earlier call)
     if (lane == 0) {
         w_cnt[wave] = nk;
         w_cnt[WS_WAVES + wave] = nt;
@@ -777,7 +847,7 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, uint32_t n_
     for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
         float x[4];
         const uint32_t i = i0 + 4u * lane;
-        const uint32_t f = look(i, x);
+        const uint32_t f = judge(i, fetch(i, std::false_type{}), x);
         if (!__ballot(f != 0u)) continue;
         const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
         const uint32_t inc = wave_incl_scan(mine);
@@ -822,7 +892,9 @@ __device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float*
     const uint64_t kept_key = in.kept_key;
     const bool want = in.want != 0u;
     const float aq = in.aq, c64 = in.c64;
-    write_in_id_order(rv, cut.n_equal, kid, klg, kept_cap, [&](uint32_t i, float x) -> uint32_t {
+    // a logit below the last kept one is not kept (floats order as their keys do)
+    const float x_last = (kept_key >> 32) ? unkey32(static_cast<uint32_t>(kept_key >> 32)) : -INFINITY;
+    write_in_id_order(rv, want, cut.n_equal, want ? -INFINITY : x_last, kid, klg, kept_cap, reinterpret_cast<uint64_t*>(lds), [&](uint32_t i, float x) -> uint32_t {
         uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
         if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
             // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes; among those
@@ -2202,6 +2274,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double m1base = has_r1 ? pm[r1lo] : 0.0;
     const uint32_t n_list = n_r0 + n_r1;
     if (n_list > kCap || n_list == 0) flags |= kOverflow;
+    // The kept-set dump of a top-k row needs no pass over the row: range 0 starts at the top of the row there, so every
+    // kept token is among the gathered candidates (and no zero-mass candidate is kept beyond them).
+    constexpr uint32_t kDumpListed = 1024u;  // candidates ranked by id against each other
+    const bool dump_listed = FUSED && A.kept_ids && prefix_mode && n1 == n1_asked && !race && !(flags & kOverflow) && n_r0 <= kDumpListed;
+    bool dumped = false;       // the dump is done
+    bool tables_whole = true;  // pv[] holds the adjusted logit of every touched token of the row (a split row: of this part's slice only)
     // Entropy of the kept set (asked for by the typical acceptance rule): -sum p ln p = ln Zk + sum e a / Zk with
     // e = exp(-a), a = (max - x) * inv_t. The gathered candidates give their terms exactly further down; the bins that
     // are kept whole - before range 0, and between the ranges - give theirs here from the scanned masses, every token
@@ -2341,9 +2419,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     }
                     clean_shared();
                     split = false;  // the row is this part's from here
-                    if (A.kept_ids || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
+                    if ((A.kept_ids && !dump_listed) || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
                         float ma, mu;
                         collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
+                    } else {
+                        tables_whole = false;
                     }
                     __syncthreads();
                 }
@@ -2605,6 +2685,40 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         kept_key = s_res.kept_key;
                         Zk_out = s_res.Zk;
                         finished = finished_lean = true;
+                        if (dump_listed && token >= 0) {  // uniform
+                            // the kept candidates, (id, logit) in one word, to the room of the buckets' masses (done with), then every
+                            // one counts the ids below its own: that is its place in the output
+                            uint64_t* sel = reinterpret_cast<uint64_t*>(lb_e);
+                            if (t == 0) s_u[7] = 0u;
+                            __syncthreads();
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                if (static_cast<uint32_t>(q) * WS_BLOCK >= n_hit) continue;  // uniform
+                                const uint32_t k = q * WS_BLOCK + t;
+                                const uint2 en = k < n_hit ? list[k] : make_uint2(0u, 0u);
+                                uint32_t id;
+                                float x;
+                                const bool on = entry(en, k < n_hit, id, x);
+                                if (on && key64(x, id) >= kept_key) {
+                                    const uint32_t slot = atomicAdd(&s_u[7], 1u);
+                                    if (slot < kDumpListed) sel[slot] = (static_cast<uint64_t>(id) << 32) | __float_as_uint(x);
+                                }
+                            }
+                            __syncthreads();
+                            const uint32_t nk = min(s_u[7], kDumpListed);
+                            int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
+                            float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
+                            for (uint32_t j = t; j < nk; j += WS_BLOCK) {
+                                const uint64_t mine = sel[j];
+                                uint32_t before = 0;
+                                for (uint32_t l = 0; l < nk; ++l) before += sel[l] < mine ? 1u : 0u;
+                                if (before < A.kept_cap) {
+                                    kid[before] = static_cast<int32_t>(mine >> 32);
+                                    if (klg) klg[before] = __uint_as_float(static_cast<uint32_t>(mine));
+                                }
+                            }
+                            dumped = true;
+                        }
                     } else {
                         mg_top_p = mg_min_p = mg_draw = 1.0;
                         n3 = n1;
@@ -3459,7 +3573,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     };
     bool finished_slow = false;
-    if (WS_RARE((flags & kOverflow) && m > -INFINITY)) {  // uniform
+    if (WS_RARE((flags & kOverflow) && !tables_whole)) token = -1;  // (a split row that ran over after its parts had left: reported unresolved)
+    if (WS_RARE((flags & kOverflow) && m > -INFINITY && tables_whole)) {  // uniform
         flags &= ~kOverflow;
         finished = finished_slow = true;
         finished_lean = false;
@@ -3559,6 +3674,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
     }
 #endif
+    // the sort-based finish of a top-k row leaves the kept candidates as the first n3 sorted keys
+    const bool dump_sorted = dump_listed && !dumped && !finished_slow && !finished_lean && token >= 0 && n3 <= kDumpListed;
+    if (WS_RARE(A.kept_ids && token >= 0 && !dumped && !dump_sorted && !tables_whole)) {  // (no way to the kept set: reported unresolved)
+        flags |= kOverflow;
+        token = -1;
+    }
     if (t == 0) {
         A.token[row] = token;
         A.flags[row] = flags;
@@ -3576,7 +3697,23 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     // ------------------------------------------------------------------ optional: the kept set in ascending id order
-    if (WS_RARE(A.kept_ids && token >= 0)) {
+    if (WS_RARE(dump_sorted)) {  // uniform: into id order by counting
+        __syncthreads();
+        int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
+        float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
+        for (uint32_t j = t; j < n3; j += WS_BLOCK) {
+            const uint64_t mine = keys[j];
+            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(mine);
+            uint32_t before = 0;
+            for (uint32_t l = 0; l < n3; ++l) before += (0xffffffffu - static_cast<uint32_t>(keys[l])) < id ? 1u : 0u;
+            if (before < A.kept_cap) {
+                kid[before] = static_cast<int32_t>(id);
+                if (klg) klg[before] = unkey32(static_cast<uint32_t>(mine >> 32));
+            }
+        }
+        dumped = true;
+    }
+    if (WS_RARE(A.kept_ids && token >= 0 && !dumped && tables_whole)) {
         TailIn in;
         in.base = rv.base;
         in.allow = rv.allow;
@@ -3590,23 +3727,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         __syncthreads();
         int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
-        if constexpr (FUSED) {
-            dump_kept_set(in, kid, klg, A.kept_cap);
-        } else {
-            // (the kernels without a bin cache keep the loop in line: as a call it doubles their spilled registers)
-            TailCut cut{0u, 0u};
-            if (tail_extra) cut = tail_cut(in);  // uniform
-            __syncthreads();
-            const bool want = tail_extra != 0u;
-            write_in_id_order(rv, cut.n_equal, kid, klg, A.kept_cap, [&](uint32_t i, float x) -> uint32_t {
-                uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
-                if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
-                    keep = key32(x) > cut.key ? 1u : 0u;
-                    if (key32(x) == cut.key) keep = 2u;
-                }
-                return keep;
-            });
-        }
+        dump_kept_set(in, kid, klg, A.kept_cap);
     }
 }
 
