@@ -329,6 +329,21 @@ def spec_verify_workload(steps, warmup):
             "device_near_flags": int((flags.cpu().numpy() != 0).sum())}
 
 
+def host_decode_step(steps):
+    """Wall clock of the C++ host API's decode step on configs[0] (one row of 151936 fp32 logits on the device, top-k 40,
+    top-p 0.95, 256-id history with repetition 1.1): sampling::DeviceRows::newCycle + prepareRow + sampling::sampleRow,
+    one object serving every step, as the engine's decode loop calls it."""
+    from __graft_entry__ import load_package
+    m = load_package()
+    w = workloads()
+    c = w.make_cfg1()
+    d = w.upload(c)
+    _, us, n_kept, _ = m.host_decode_steps(d["logits"][0], c["inv_t"][0], int(c["seed"][0]), 0, steps, warmup=20, top_k=int(c["top_k"][0]),
+                                           top_p=float(c["top_p"][0]), hist=c["hist"][0], rep=float(c["rep"][0]))
+    return {"workload": "host_api_decode_step (cfg1 through sampling::DeviceRows + sampleRow)", "us_per_token": us, "tokens_per_s": 1e6 / us,
+            "steps": steps, "n_kept": int(n_kept), "clock": "host wall clock, launch + stream wait + host filter included"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -377,6 +392,7 @@ def main():
                 _, r = run_workload(w, 20 if w == "cfg5" else max(20, a.steps // 4), 5, n_chk)
                 also.append(r)
         also.append(spec_verify_workload(max(20, a.steps // 4), 5))
+        also.append(host_decode_step(max(50, a.steps)))
     cpu = None if a.no_cpu else cpu_baseline(c)
     ab = main_res["algorithmic_MB"] * 1e6
     traffic, traffic_source = traffic_for(a.workload, a.mode)

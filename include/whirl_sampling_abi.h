@@ -232,7 +232,7 @@ typedef struct ws_batch {
     int32_t* kept_ids;  /* out (may be NULL): [rows][kept_cap] kept token ids in ascending id order (the first n_kept, or
                            the first kept_cap of them). Free for a top-k row of up to about a thousand candidates (they
                            are among what the kernel gathered anyway); any other row is read once more by its workgroup,
-                           about 60 us on a row of 151936 that has the GPU to itself, hidden among other rows in a batch.
+                           about 60 us for a row of 151936 on the compute unit that holds it.
                            Parameters and outputs may live in pinned host memory (hipHostMalloc): the kernels then read
                            and write them in place and a synchronous caller needs no copy at all. */
     float* kept_logits; /* out (may be NULL): penalty-applied logits of kept_ids */

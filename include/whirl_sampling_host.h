@@ -70,6 +70,29 @@ typedef struct wsh_accept {
     uint32_t relaxed;     /* out: drafts the typical rule kept */
 } wsh_accept;
 int wsh_accept_sample(void* stream, wsh_accept* a);
+
+/* The engine's decode loop on one row, step after step over one sampling::DeviceRows (newCycle, prepareRow, sampleRow with
+ * pos_idx = pos0 + step), as a serving loop holds it for the life of a logits buffer: `steps` tokens into token[] after
+ * `warmup` untimed ones, and the wall-clock time of the timed steps. The logits stay as they are (a model would rewrite
+ * them between steps); the history, when given, is the same at every step. */
+typedef struct wsh_steps {
+    const float* d_logits; /* device, [vocab] */
+    uint32_t vocab;
+    float inv_t;
+    uint32_t top_k;  /* 0: off */
+    double top_p;    /* 1: off */
+    double min_p;    /* 0: off */
+    uint64_t seed, pos0;
+    const int32_t* hist; /* host, may be NULL */
+    uint32_t n_hist;
+    float rep, pres, freq;
+    uint32_t steps, warmup;
+    int32_t* token;       /* out: steps tokens (may be NULL) */
+    double us_per_step;   /* out */
+    uint32_t n_kept;      /* out: Sampler::n of the last step */
+    uint32_t flags;       /* out: WS_FLAG_* of the last step */
+} wsh_steps;
+int wsh_decode_steps(void* stream, wsh_steps* a);
 const char* wsh_last_error(void);
 
 #ifdef __cplusplus

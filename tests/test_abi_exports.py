@@ -45,7 +45,8 @@ def test_host_side_argument_checks():
     b.logits, b.inv_t, b.seed, b.step, b.token, b.flags = one, one, one, one, one, one
     b.rows, b.vocab, b.row_stride = 4, 151936, 151936
     b.hist, b.hist_off, b.max_hist = one, one, 4096
-    assert lib.ws_sample_batch_workspace(C.byref(b)) == 0  # every intermediate of this build lives in LDS
+    b.max_split = 1  # (on a machine with a GPU a batch this small would share its rows between workgroups, through a workspace)
+    assert lib.ws_sample_batch_workspace(C.byref(b)) == 0  # every intermediate of an unsplit single-sweep row lives in LDS
     b.max_hist = 60000
     assert lib.ws_sample_batch(None, C.byref(b)) == -3  # rank tables would not fit the LDS
     b.vocab = 1 << 20

@@ -70,3 +70,27 @@ def test_host_rows_open_row_with_penalties_uses_the_penalised_copy():
     near, out = _run(c, range(4))
     assert near == 0
     assert all(out["flags"] & m.FLAG_OPEN) and not any(out["closed"])
+
+
+def test_decode_steps_over_one_device_rows_object():
+    """wsh_decode_steps: one sampling::DeviceRows serving step after step (newCycle, prepareRow, sampleRow) gives, at
+    every output index, the token the oracle draws for that index - a top-k row (kept set taken from the gathered
+    candidates), with and without a history, and a top-p-only row (kept set read from the row)."""
+    m = gc.pkg()
+    c = gc.make_cfg1()
+    d = gc.upload(c)
+    for top_k, top_p, hist in ((40, 0.95, None), (40, 0.95, c["hist"][0]), (0, 0.9, c["hist"][0])):
+        cc = dict(c)
+        cc["top_k"] = np.array([top_k], np.uint32)
+        cc["top_p"] = np.array([top_p])
+        cc["hist"] = None if hist is None else c["hist"]
+        if hist is None:
+            cc["rep"] = np.ones(1, np.float32)
+        tok, us, n_kept, flags = m.host_decode_steps(d["logits"][0], c["inv_t"][0], int(c["seed"][0]), 100, 12, warmup=2, top_k=top_k,
+                                                     top_p=top_p, hist=hist, rep=float(cc["rep"][0]))
+        assert us > 0 and n_kept >= 1 and not flags & (m.FLAG_OVERFLOW | m.FLAG_OPEN)
+        for i in range(12):
+            cc["step"] = np.array([100 + i], np.uint64)
+            o, _, _ = gc.oracle_row(cc, 0, 0)
+            if tok[i] != o.token:
+                assert min(o.margin, o.margin_top_p, o.margin_min_p) < 1e-6, (top_k, top_p, i, tok[i], o.token)

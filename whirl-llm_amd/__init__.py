@@ -494,8 +494,17 @@ class HostAccept(C.Structure):
                 ("delta", C.c_float), ("hist", C.c_void_p), ("n_hist", C.c_uint32), ("next", C.c_uint32), ("relaxed", C.c_uint32)]
 
 
+class HostSteps(C.Structure):
+    """wsh_steps of include/whirl_sampling_host.h."""
+    _fields_ = [("d_logits", C.c_void_p), ("vocab", C.c_uint32), ("inv_t", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_double),
+                ("min_p", C.c_double), ("seed", C.c_uint64), ("pos0", C.c_uint64), ("hist", C.c_void_p), ("n_hist", C.c_uint32),
+                ("rep", C.c_float), ("pres", C.c_float), ("freq", C.c_float), ("steps", C.c_uint32), ("warmup", C.c_uint32),
+                ("token", C.c_void_p), ("us_per_step", C.c_double), ("n_kept", C.c_uint32), ("flags", C.c_uint32)]
+
+
 HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]),
-            "wsh_accept_sample": (C.c_int, [C.c_void_p, C.POINTER(HostAccept)]), "wsh_last_error": (C.c_char_p, [])}
+            "wsh_accept_sample": (C.c_int, [C.c_void_p, C.POINTER(HostAccept)]),
+            "wsh_decode_steps": (C.c_int, [C.c_void_p, C.POINTER(HostSteps)]), "wsh_last_error": (C.c_char_p, [])}
 _host_lib = None
 
 
@@ -545,6 +554,25 @@ def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p
     if rc != 0:
         raise WsError(f"wsh_sample_rows: {host_lib().wsh_last_error().decode()} ({rc})")
     return out
+
+
+def host_decode_steps(row, inv_t, seed, pos0, steps, warmup=0, top_k=0, top_p=1.0, min_p=0.0, hist=None, rep=1.0, pres=0.0, freq=0.0):
+    """`steps` tokens from one row of device logits through one sampling::DeviceRows, the way a serving loop holds it
+    (wsh_decode_steps: newCycle, prepareRow, sampleRow with pos_idx = pos0 + step). Returns (tokens, microseconds of wall
+    clock per step, n_kept and flags of the last step)."""
+    import numpy as np
+    _dev_f32(row)
+    if row.dim() != 1:
+        raise WsError("host_decode_steps: one row of logits")
+    tok = np.zeros(max(steps, 1), np.int32)
+    h = None if hist is None else np.ascontiguousarray(hist, dtype=np.int32)
+    a = HostSteps(d_logits=_p(row), vocab=row.shape[0], inv_t=float(np.float32(inv_t)), top_k=top_k, top_p=top_p, min_p=min_p, seed=seed,
+                  pos0=pos0, hist=None if h is None else h.ctypes.data_as(C.c_void_p), n_hist=0 if h is None else h.size, rep=rep,
+                  pres=pres, freq=freq, steps=steps, warmup=warmup, token=tok.ctypes.data_as(C.c_void_p))
+    rc = host_lib().wsh_decode_steps(_stream(), C.byref(a))
+    if rc != 0:
+        raise WsError(f"wsh_decode_steps: {host_lib().wsh_last_error().decode()} ({rc})")
+    return tok[:steps], a.us_per_step, a.n_kept, a.flags
 
 
 def host_accept_sample(logits, dr, nd, row0, n_gen, temp, top_k, top_p, min_p, seed, race=False, prefetch=True, typical=None):

@@ -7,6 +7,7 @@
 #include "whirl_sampling_abi.h"
 #include "whirl_sampling_host.h"
 
+#include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <exception>
@@ -112,6 +113,51 @@ int wsh_accept_sample(void* stream, wsh_accept* a) {
         a->chosen = r.chosen;
         a->big_used = s.big_used;
         a->full_used = s.full_used;
+        return 0;
+    } catch (const ws::DeviceError& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return e.code ? e.code : -1;
+    } catch (const std::exception& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return -1;
+    }
+}
+
+int wsh_decode_steps(void* stream, wsh_steps* a) {
+    g_err[0] = 0;
+    try {
+        ws::DeviceRows src(a->d_logits, 1, a->vocab, stream);
+        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+        ws::Sampler s;
+        s.inv_t = a->inv_t;
+        s.temp = 1.0 / s.inv_t;
+        s.top_k = a->top_k;
+        s.top_p = a->top_p;
+        s.min_p = a->min_p;
+        s.seed = a->seed;
+        s.cands = &scratch;
+        ws::RowAdjust adj;
+        if (a->hist && a->n_hist) {
+            adj.history = a->hist;
+            adj.n_history = a->n_hist;
+            adj.repetition = a->rep;
+            adj.presence = a->pres;
+            adj.frequency = a->freq;
+        }
+        src.setAdjust(adj);
+        std::chrono::steady_clock::time_point t0;
+        for (uint32_t i = 0; i < a->warmup + a->steps; ++i) {
+            if (i == a->warmup) t0 = std::chrono::steady_clock::now();
+            s.pos_idx = a->pos0 + (i >= a->warmup ? i - a->warmup : 0);
+            src.newCycle();
+            src.prepareRow(s, 0);
+            const uint32_t t = ws::sampleRow(src, s, std::nullopt, 0);
+            if (i >= a->warmup && a->token) a->token[i - a->warmup] = static_cast<int32_t>(t);
+        }
+        const auto t1 = std::chrono::steady_clock::now();
+        a->us_per_step = a->steps ? std::chrono::duration<double, std::micro>(t1 - t0).count() / a->steps : 0.0;
+        a->n_kept = static_cast<uint32_t>(s.n);
+        a->flags = src.lastFlags();
         return 0;
     } catch (const ws::DeviceError& e) {
         snprintf(g_err, sizeof g_err, "%s", e.what());
