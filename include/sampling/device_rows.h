@@ -67,6 +67,8 @@ public:
 private:
     void escalate(Sampler& s, std::uint32_t gr);
     void uploadInputs(const Sampler& s, std::uint32_t n);
+    void uploadLists(std::uint32_t n);
+    void ensureAdjusted(std::uint32_t gr);
     void filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32_t n);
     struct Dev;    // device scratch
     struct Ready;  // a row filtered on the device, held for its prepareRow

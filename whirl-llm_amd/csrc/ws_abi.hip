@@ -22,6 +22,9 @@ namespace ws {
 int launch_fused(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
 // ws_split.hip: the same with rows split over several workgroups
 int launch_split(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
+// ws_fused_kept.hip, ws_split_kept.hip: the builds of the two that can write the kept-set dump
+int launch_fused_kept(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
+int launch_split_kept(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
 }  // namespace ws
 
 namespace {
@@ -429,8 +432,9 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     a.query = b->query;
     a.query_prob = b->query_prob;
     a.entropy = b->entropy;
-    if (p.fused && a.split_log2) return ws::launch_split(S(stream), a, b->rows << a.split_log2, p.lds_total, kMaxLds - kStaticLds);
-    if (p.fused) return ws::launch_fused(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);
+    if (p.fused && a.split_log2)
+        return (a.kept_ids ? ws::launch_split_kept : ws::launch_split)(S(stream), a, b->rows << a.split_log2, p.lds_total, kMaxLds - kStaticLds);
+    if (p.fused) return (a.kept_ids ? ws::launch_fused_kept : ws::launch_fused)(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);
     static std::atomic<uint64_t> attr_set{0};  // the dynamic LDS limit is raised per function and device, once per process
     int dev = 0;
     if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);

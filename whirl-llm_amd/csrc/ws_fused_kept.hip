@@ -1,0 +1,4 @@
+// ws_fused.hip once more, as the build that can write the kept-set dump (ws_batch.kept_ids).
+#define WS_KEPT_BUILD true
+#define WS_LAUNCH launch_fused_kept
+#include "ws_fused.hip"

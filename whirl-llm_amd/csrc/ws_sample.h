@@ -870,6 +870,72 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
     }
 }
 
+// Entries of the single-sweep kernel's candidate list: (token | flags, logit bits).
+constexpr uint32_t kListNeedsLoad = 0x80000000u, kListAdjusted = 0x40000000u, kListIdMask = 0x3fffffffu;
+
+// The kept-set dump of a row whose kept tokens are all among n (id << 32 | logit bits) words in LDS: every one counts
+// the ids below its own, which is its place in the output. Functions of their own, like the other dumps: they run for
+// callers that ask for the dump only, and the kernel keeps its registers for what every row needs. (LDS arrays come as
+// byte offsets into the kernel's dynamic LDS, so that their reads compile as LDS reads.)
+__device__ __noinline__ void dump_by_counting(uint32_t sel_at, uint32_t n, int32_t* kid, float* klg, uint32_t kept_cap) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const uint64_t* sel = reinterpret_cast<const uint64_t*>(lds + sel_at);
+    for (uint32_t j = threadIdx.x; j < n; j += WS_BLOCK) {
+        const uint64_t mine = sel[j];
+        uint32_t before = 0;
+        for (uint32_t l = 0; l < n; ++l) before += sel[l] < mine ? 1u : 0u;
+        if (before < kept_cap) {
+            kid[before] = static_cast<int32_t>(mine >> 32);
+            if (klg) klg[before] = __uint_as_float(static_cast<uint32_t>(mine));
+        }
+    }
+}
+// ... from the first n sorted keys (logit key << 32 | ~id) of the sort-based finish
+__device__ __noinline__ void dump_sorted_keys(uint32_t keys_at, uint32_t n, int32_t* kid, float* klg, uint32_t kept_cap) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const uint64_t* keys = reinterpret_cast<const uint64_t*>(lds + keys_at);
+    for (uint32_t j = threadIdx.x; j < n; j += WS_BLOCK) {
+        const uint64_t mine = keys[j];
+        const uint32_t id = 0xffffffffu - static_cast<uint32_t>(mine);
+        uint32_t before = 0;
+        for (uint32_t l = 0; l < n; ++l) before += (0xffffffffu - static_cast<uint32_t>(keys[l])) < id ? 1u : 0u;
+        if (before < kept_cap) {
+            kid[before] = static_cast<int32_t>(id);
+            if (klg) klg[before] = unkey32(static_cast<uint32_t>(mine >> 32));
+        }
+    }
+}
+// ... from the candidate list after the bucket finish: the entries at or above the last kept key go to `sel` first
+// touched_at: LDS offset of the touched bitmap, ~0 when no token is touched.
+__device__ __noinline__ void dump_listed_candidates(const void* base, int dtype, uint32_t touched_at, uint32_t list_at, uint32_t n_hit,
+                                                    uint64_t kept_key, uint32_t sel_at, uint32_t sel_cap, int32_t* kid, float* klg,
+                                                    uint32_t kept_cap) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t n_sel;
+    uint32_t* counter = &n_sel;
+    const uint2* list = reinterpret_cast<const uint2*>(lds + list_at);
+    uint64_t* sel = reinterpret_cast<uint64_t*>(lds + sel_at);
+    const uint32_t* touched = touched_at != 0xffffffffu ? reinterpret_cast<const uint32_t*>(lds + touched_at) : nullptr;
+    if (threadIdx.x == 0) *counter = 0u;
+    __syncthreads();
+    for (uint32_t k = threadIdx.x; k < n_hit; k += WS_BLOCK) {
+        const uint2 en = list[k];
+        const uint32_t id = en.x & kListIdMask;
+        const bool adjusted = en.x & kListAdjusted;
+        if (!adjusted && touched && ((touched[id >> 5] >> (id & 31u)) & 1u)) continue;  // fed with its adjusted logit by another entry
+        float x;
+        if (adjusted) x = __uint_as_float(en.y);
+        else if (en.x & kListNeedsLoad) x = fmaxf(dtype == 0 ? static_cast<const float*>(base)[id] : bf16_to_f32(static_cast<const uint16_t*>(base)[id]), -INFINITY);
+        else x = fmaxf(__uint_as_float(dtype == 0 ? en.y : en.y << 16), -INFINITY);
+        if (key64(x, id) >= kept_key) {
+            const uint32_t slot = atomicAdd(counter, 1u);
+            if (slot < sel_cap) sel[slot] = (static_cast<uint64_t>(id) << 32) | __float_as_uint(x);
+        }
+    }
+    __syncthreads();
+    dump_by_counting(sel_at, min(*counter, sel_cap), kid, klg, kept_cap);
+}
+
 // The kept set of a row in ascending id order (the optional dump): every token whose key is at or above `kept_key`, and
 // `want` zero-mass candidates (tail_cut). A function of its own, like the exact path: it runs for callers that ask for
 // the dump only, and the kernel keeps its registers for what every row needs.
@@ -1263,8 +1329,12 @@ __device__ __noinline__ ExactOut exact_row(const ExactIn in) {
     } while (0)
 #endif
 
-template <bool FUSED, bool SPLIT = false>  // SPLIT: rows split over several workgroups (a build of its own: the unsplit kernel carries none of it)
+// SPLIT: rows split over several workgroups (a build of its own: the unsplit kernel carries none of it). KEPT: the build
+// that can write the kept-set dump; launches without kept_ids take the single-sweep builds that cannot, which keeps the
+// dump's flags and calls out of their register allocation (with them the tile cost 1-2 % more).
+template <bool FUSED, bool SPLIT = false, bool KEPT = true>
 __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
+    int32_t* const kept_ids = KEPT ? A.kept_ids : nullptr;
 #ifdef WS_PHASE_TIMERS
     __shared__ long long ws_marks[64];
     const long long ws_t0 = clock64();
@@ -2274,12 +2344,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     const double m1base = has_r1 ? pm[r1lo] : 0.0;
     const uint32_t n_list = n_r0 + n_r1;
     if (n_list > kCap || n_list == 0) flags |= kOverflow;
-    // The kept-set dump of a top-k row needs no pass over the row: range 0 starts at the top of the row there, so every
-    // kept token is among the gathered candidates (and no zero-mass candidate is kept beyond them).
+    // The kept-set dump of a top-k row (and of an open row's list) needs no pass over the row: range 0 starts at the top
+    // of the row there, so every kept token is among the gathered candidates (and no zero-mass candidate is kept beyond them).
     constexpr uint32_t kDumpListed = 1024u;  // candidates ranked by id against each other
-    const bool dump_listed = FUSED && A.kept_ids && prefix_mode && n1 == n1_asked && !race && !(flags & kOverflow) && n_r0 <= kDumpListed;
+    const bool dump_listed =
+        FUSED && kept_ids && (prefix_mode || open_row) && n1 == n1_asked && !race && !(flags & kOverflow) && n_r0 <= kDumpListed;
     bool dumped = false;       // the dump is done
-    bool tables_whole = true;  // pv[] holds the adjusted logit of every touched token of the row (a split row: of this part's slice only)
+    uint32_t listed_n = 0;     // entries of the candidate list after a bucket finish
+    // kPartialTables in `flags` (inside the kernel only): pv[] holds the adjusted logits of this part's slice alone - the
+    // finisher of a split row that did not collect the other slices' (a bit of a word that is live anyway, not a
+    // register of its own)
+    constexpr uint32_t kPartialTables = 0x80000000u;
     // Entropy of the kept set (asked for by the typical acceptance rule): -sum p ln p = ln Zk + sum e a / Zk with
     // e = exp(-a), a = (max - x) * inv_t. The gathered candidates give their terms exactly further down; the bins that
     // are kept whole - before range 0, and between the ranges - give theirs here from the scanned masses, every token
@@ -2341,7 +2416,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                 // then line their hits up in list[] as (token, logit bits) pairs, a third hit and beyond as the token alone
                 // (kNeedsLoad), and the list is taken from there one entry per thread. A hit that is a touched token
                 // (cached with the bin of its raw logit) is dropped and fed by replay_touched.
-                constexpr uint32_t kNeedsLoad = 0x80000000u, kAdjusted = 0x40000000u, kIdMask = 0x3fffffffu;
+                constexpr uint32_t kNeedsLoad = kListNeedsLoad, kAdjusted = kListAdjusted, kIdMask = kListIdMask;
                 uint2* list = reinterpret_cast<uint2*>(emass);  // kCap entries
                 // tables of the bucket finish below: per bucket a count and a fixed-point mass (the LDS of the histogram
                 // scan's side arrays, idle by now) and places for keys and their masses: 32 per bucket where the spare LDS
@@ -2419,11 +2494,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     }
                     clean_shared();
                     split = false;  // the row is this part's from here
-                    if ((A.kept_ids && !dump_listed) || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
+                    if ((kept_ids && !dump_listed) || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
                         float ma, mu;
                         collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
                     } else {
-                        tables_whole = false;
+                        flags |= kPartialTables;
                     }
                     __syncthreads();
                 }
@@ -2685,40 +2760,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                         kept_key = s_res.kept_key;
                         Zk_out = s_res.Zk;
                         finished = finished_lean = true;
-                        if (dump_listed && token >= 0) {  // uniform
-                            // the kept candidates, (id, logit) in one word, to the room of the buckets' masses (done with), then every
-                            // one counts the ids below its own: that is its place in the output
-                            uint64_t* sel = reinterpret_cast<uint64_t*>(lb_e);
-                            if (t == 0) s_u[7] = 0u;
-                            __syncthreads();
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) {
-                                if (static_cast<uint32_t>(q) * WS_BLOCK >= n_hit) continue;  // uniform
-                                const uint32_t k = q * WS_BLOCK + t;
-                                const uint2 en = k < n_hit ? list[k] : make_uint2(0u, 0u);
-                                uint32_t id;
-                                float x;
-                                const bool on = entry(en, k < n_hit, id, x);
-                                if (on && key64(x, id) >= kept_key) {
-                                    const uint32_t slot = atomicAdd(&s_u[7], 1u);
-                                    if (slot < kDumpListed) sel[slot] = (static_cast<uint64_t>(id) << 32) | __float_as_uint(x);
-                                }
-                            }
-                            __syncthreads();
-                            const uint32_t nk = min(s_u[7], kDumpListed);
-                            int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
-                            float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
-                            for (uint32_t j = t; j < nk; j += WS_BLOCK) {
-                                const uint64_t mine = sel[j];
-                                uint32_t before = 0;
-                                for (uint32_t l = 0; l < nk; ++l) before += sel[l] < mine ? 1u : 0u;
-                                if (before < A.kept_cap) {
-                                    kid[before] = static_cast<int32_t>(mine >> 32);
-                                    if (klg) klg[before] = __uint_as_float(static_cast<uint32_t>(mine));
-                                }
-                            }
-                            dumped = true;
-                        }
+                        listed_n = n_hit;  // (the list stays as it is to the end of the kernel: the dump may want it)
                     } else {
                         mg_top_p = mg_min_p = mg_draw = 1.0;
                         n3 = n1;
@@ -3409,6 +3451,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         Zk = Z;
         kept_key = 0ull;
     }
+    if (WS_RARE(dump_listed && n3 <= kDumpListed && n3 <= n_list)) {  // uniform
+        // the kept set of a top-k row or an open row's list: the first n3 sorted keys; into id order by counting, now,
+        // while the keys lie untouched (the draw below may use their room)
+        dump_sorted_keys(0u /* keys */, n3, kept_ids + static_cast<size_t>(row) * A.kept_cap,
+                         A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr, A.kept_cap);
+        dumped = true;
+    }
 
     // ------------------------------------------------------------------ draw
     const double u = batch_uniform(A.rng, seed, row, step, 0);
@@ -3573,11 +3622,12 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         }
     };
     bool finished_slow = false;
-    if (WS_RARE((flags & kOverflow) && !tables_whole)) token = -1;  // (a split row that ran over after its parts had left: reported unresolved)
-    if (WS_RARE((flags & kOverflow) && m > -INFINITY && tables_whole)) {  // uniform
+    if (WS_RARE((flags & (kOverflow | kPartialTables)) == (kOverflow | kPartialTables))) token = -1;  // (a split row that ran over after its parts had left: reported unresolved)
+    if (WS_RARE((flags & (kOverflow | kPartialTables)) == kOverflow && m > -INFINITY)) {  // uniform
         flags &= ~kOverflow;
         finished = finished_slow = true;
         finished_lean = false;
+        dumped = false;  // (whatever an earlier finish wrote is written again from this one's result)
         ExactIn in;
         in.base = rv.base;
         in.allow = rv.allow;
@@ -3674,15 +3724,13 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
     }
 #endif
-    // the sort-based finish of a top-k row leaves the kept candidates as the first n3 sorted keys
-    const bool dump_sorted = dump_listed && !dumped && !finished_slow && !finished_lean && token >= 0 && n3 <= kDumpListed;
-    if (WS_RARE(A.kept_ids && token >= 0 && !dumped && !dump_sorted && !tables_whole)) {  // (no way to the kept set: reported unresolved)
+    if (WS_RARE(kept_ids && token >= 0 && !dumped && (flags & kPartialTables) && !(dump_listed && finished_lean))) {  // (no way to the kept set: reported unresolved)
         flags |= kOverflow;
         token = -1;
     }
     if (t == 0) {
         A.token[row] = token;
-        A.flags[row] = flags;
+        A.flags[row] = flags & ~kPartialTables;
         if (A.prob) A.prob[row] = static_cast<float>(ptok);
         if (A.n_kept) A.n_kept[row] = n3 + tail_extra;
         if (A.stats) {
@@ -3697,23 +3745,16 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     }
 
     // ------------------------------------------------------------------ optional: the kept set in ascending id order
-    if (WS_RARE(dump_sorted)) {  // uniform: into id order by counting
+    if (WS_RARE(dump_listed && finished_lean && !dumped && token >= 0)) {  // uniform
+        // after the bucket finish: the kept candidates go from the list to the room of the buckets' masses (done with)
         __syncthreads();
-        int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
-        float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
-        for (uint32_t j = t; j < n3; j += WS_BLOCK) {
-            const uint64_t mine = keys[j];
-            const uint32_t id = 0xffffffffu - static_cast<uint32_t>(mine);
-            uint32_t before = 0;
-            for (uint32_t l = 0; l < n3; ++l) before += (0xffffffffu - static_cast<uint32_t>(keys[l])) < id ? 1u : 0u;
-            if (before < A.kept_cap) {
-                kid[before] = static_cast<int32_t>(id);
-                if (klg) klg[before] = unkey32(static_cast<uint32_t>(mine >> 32));
-            }
-        }
+        if constexpr (FUSED)
+            dump_listed_candidates(rv.base, rv.dtype, rv.touched ? A.lds_ab : 0xffffffffu, 32768u /* list */, listed_n, kept_key,
+                                   A.lds_tie ? A.lds_tie : 16384u /* lb_e */, kDumpListed, kept_ids + static_cast<size_t>(row) * A.kept_cap,
+                                   A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr, A.kept_cap);
         dumped = true;
     }
-    if (WS_RARE(A.kept_ids && token >= 0 && !dumped && tables_whole)) {
+    if (WS_RARE(kept_ids && token >= 0 && !dumped && !(flags & kPartialTables))) {
         TailIn in;
         in.base = rv.base;
         in.allow = rv.allow;
@@ -3725,7 +3766,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         in.kept_key = kept_key;
         in.want = tail_extra;
         __syncthreads();
-        int32_t* kid = A.kept_ids + static_cast<size_t>(row) * A.kept_cap;
+        int32_t* kid = kept_ids + static_cast<size_t>(row) * A.kept_cap;
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
         dump_kept_set(in, kid, klg, A.kept_cap);
     }

@@ -1,0 +1,4 @@
+// ws_split.hip once more, as the build that can write the kept-set dump (ws_batch.kept_ids).
+#define WS_KEPT_BUILD true
+#define WS_LAUNCH launch_split_kept
+#include "ws_split.hip"

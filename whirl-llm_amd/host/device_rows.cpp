@@ -135,6 +135,7 @@ DeviceRows::~DeviceRows() {
 void DeviceRows::setAdjust(const RowAdjust& a) {
     adj_ = a;
     ready_.clear();  // rows filtered under the old penalties are of no use any more
+    adjusted_row_ = kNoRow;
 }
 
 void DeviceRows::newCycle() {
@@ -153,6 +154,20 @@ void pinned(T** p, std::size_t bytes) {
 // where the device reads them (the lists are replicated because a batch addresses them through one ascending offset
 // array). The stream is idle when this runs.
 void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
+    uploadLists(n);
+    const Dev::ParamView h = Dev::view(dev_->prm, n);
+    for (std::uint32_t r = 0; r < n; ++r) {
+        h.top_p[r] = s.top_p;
+        h.min_p[r] = s.min_p;
+        h.seed[r] = s.seed;
+        h.step[r] = s.pos_idx;  // the draw is made on the host; the device's own is not looked at
+        h.inv_t[r] = s.inv_t;
+        h.top_k[r] = s.top_k;
+    }
+}
+
+// the part of the inputs that does not depend on the sampler: the penalty lists, their offsets and the penalties
+void DeviceRows::uploadLists(std::uint32_t n) {
     Dev& d = *dev_;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
     if (n > d.row_cap) {
@@ -197,15 +212,9 @@ void DeviceRows::uploadInputs(const Sampler& s, std::uint32_t n) {
     }
     const Dev::ParamView h = Dev::view(d.prm, n);
     for (std::uint32_t r = 0; r < n; ++r) {
-        h.top_p[r] = s.top_p;
-        h.min_p[r] = s.min_p;
-        h.seed[r] = s.seed;
-        h.step[r] = s.pos_idx;  // the draw is made on the host; the device's own is not looked at
-        h.inv_t[r] = s.inv_t;
         h.rep[r] = adj_.repetition;
         h.pres[r] = adj_.presence;
         h.freq[r] = adj_.frequency;
-        h.top_k[r] = s.top_k;
     }
     for (std::uint32_t r = 0; r <= n; ++r) {
         h.hist_off[r] = static_cast<std::uint32_t>(r * nh);
@@ -277,7 +286,7 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
     const Dev::ResultView& h = o;
     ready_.clear();
     ready_.resize(n);
-    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
+    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
     for (std::uint32_t r = 0; r < n; ++r) {
         Ready& q = ready_[r];
         q.gr = gr0 + r;
@@ -286,6 +295,7 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
         q.m = h.stats[2 * r];
         q.sum = h.stats[2 * r + 1];
         if ((q.flags & unresolved) || q.n_kept > cap) continue;  // such a row is escalated when it is asked for
+        // (an open row's list - the engine's short candidate list - comes back like a kept set)
         q.ids.assign(d.kept_ids + std::size_t{r} * cap, d.kept_ids + std::size_t{r} * cap + q.n_kept);
         q.logits.assign(d.kept_logits + std::size_t{r} * cap, d.kept_logits + std::size_t{r} * cap + q.n_kept);
     }
@@ -313,7 +323,7 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     q->gr = kNoRow;
     last_flags_ = q->flags;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
-    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_OPEN | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
+    const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
     if ((q->flags & unresolved) || q->n_kept > cap) {
         escalate(s, gr);
         return;
@@ -322,6 +332,17 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     s.m = q->m;
     s.sum = q->sum;
     Cand* c = s.cands->data();
+    if (q->flags & WS_FLAG_OPEN) {
+        // No filter at all: the device's list is the engine's short candidate list (the 256 largest logits, lowest ids among
+        // equals), the first step of the reference's route (src/server/engine_sampling.cpp:51-66) without a launch of its
+        // own. The rest of the row is fetched if and when the draw walks past the list (loadFullRow).
+        if (n == std::min(kSmall, vocab_)) {
+            for (std::uint32_t i = 0; i < n; ++i) c[i] = {static_cast<std::uint32_t>(q->ids[i]), q->logits[i], 0.0};
+            if (filterCands(s, n, false)) return;
+        }
+        escalate(s, gr);
+        return;
+    }
     for (std::uint32_t i = 0; i < n; ++i) c[i] = {static_cast<std::uint32_t>(q->ids[i]), q->logits[i], 0.0};
     std::sort(c, c + n, [](const Cand& a, const Cand& b2) { return a.logit != b2.logit ? a.logit > b2.logit : a.id < b2.id; });
     // probabilities as the host filter leaves them: exp((double)(float)(l - m) * inv_t) / sum, renormalised over the kept set
@@ -337,6 +358,38 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     if (n > kBig) s.full_used += 1;
 }
 
+// The penalised copy of row gr on the device (ws_adjust_rows), written once per prepared row and only when something
+// asks for it: an escalation, or a draw that walks past the candidates. The stream is idle when this runs.
+void DeviceRows::ensureAdjusted(std::uint32_t gr) {
+    if (adjusted_row_ == gr) return;
+    Dev& d = *dev_;
+    if (!d.adjusted) checkHip(hipMalloc(reinterpret_cast<void**>(&d.adjusted), vocab_ * sizeof(float)), "hipMalloc");
+    uploadLists(1);  // the row may come from an earlier batch: its lists are written again
+    const Dev::ParamView p = Dev::view(d.prm, 1);
+    ws_adjust a{};
+    a.logits = logits_ + static_cast<std::size_t>(gr) * vocab_;
+    a.dtype = WS_DTYPE_F32;
+    a.rows = 1;
+    a.vocab = vocab_;
+    a.row_stride = vocab_;
+    if (adj_.n_history) {
+        a.hist = d.hist;
+        a.hist_off = p.hist_off;
+        a.rep = p.rep;
+        a.pres = p.pres;
+        a.freq = p.freq;
+    }
+    if (adj_.n_bias) {
+        a.bias_ids = d.bias_ids;
+        a.bias_vals = d.bias_vals;
+        a.bias_off = p.bias_off;
+    }
+    a.out = d.adjusted;
+    a.out_stride = vocab_;
+    check(ws_adjust_rows(stream_, &a), "ws_adjust_rows");
+    adjusted_row_ = gr;
+}
+
 // The reference's way for a row the device did not resolve (src/server/engine_sampling.cpp:51-84): the device's top 256
 // of the row through filterCands, then its top 16384, then the whole row. With penalties or a bias list in force the
 // device first writes a penalised copy of the row (ws_adjust_rows), and every later step reads that copy.
@@ -345,32 +398,8 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
     Dev& d = *dev_;
     const float* src = logits_ + static_cast<std::size_t>(gr) * vocab_;
     if (adj_.n_history || adj_.n_bias) {
-        if (!d.adjusted) checkHip(hipMalloc(reinterpret_cast<void**>(&d.adjusted), vocab_ * sizeof(float)), "hipMalloc");
-        uploadInputs(s, 1);  // the row may come from an earlier batch: its lists and parameters are written again
-        const Dev::ParamView p = Dev::view(d.prm, 1);
-        ws_adjust a{};
-        a.logits = src;
-        a.dtype = WS_DTYPE_F32;
-        a.rows = 1;
-        a.vocab = vocab_;
-        a.row_stride = vocab_;
-        if (adj_.n_history) {
-            a.hist = d.hist;
-            a.hist_off = p.hist_off;
-            a.rep = p.rep;
-            a.pres = p.pres;
-            a.freq = p.freq;
-        }
-        if (adj_.n_bias) {
-            a.bias_ids = d.bias_ids;
-            a.bias_vals = d.bias_vals;
-            a.bias_off = p.bias_off;
-        }
-        a.out = d.adjusted;
-        a.out_stride = vocab_;
-        check(ws_adjust_rows(stream_, &a), "ws_adjust_rows");
+        ensureAdjusted(gr);
         src = d.adjusted;
-        adjusted_row_ = gr;
     }
     if (!d.topk_ids) {
         pinned(&d.topk_ids, kBig * sizeof(std::int32_t));
@@ -403,7 +432,9 @@ const float* DeviceRows::loadFullRow(std::uint32_t gr) {
     if (gr >= rows_) throw DeviceError("loadFullRow", WS_E_INVALID, "loadFullRow: row out of range");
     if (!dev_->row_host) pinned(&dev_->row_host, vocab_ * sizeof(float));
     auto stream = static_cast<hipStream_t>(stream_);
-    const float* src = gr == adjusted_row_ ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
+    const bool penalised = adj_.n_history || adj_.n_bias;
+    if (penalised) ensureAdjusted(gr);
+    const float* src = penalised ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
     checkHip(hipMemcpyAsync(dev_->row_host, src, vocab_ * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     return dev_->row_host;
@@ -413,7 +444,9 @@ float DeviceRows::logitAt(std::uint32_t gr, std::uint32_t t) {
     if (gr >= rows_ || t >= vocab_) throw DeviceError("logitAt", WS_E_INVALID, "logitAt: out of range");
     float v = 0;
     auto stream = static_cast<hipStream_t>(stream_);
-    const float* src = gr == adjusted_row_ ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
+    const bool penalised = adj_.n_history || adj_.n_bias;
+    if (penalised) ensureAdjusted(gr);
+    const float* src = penalised ? dev_->adjusted : logits_ + static_cast<std::size_t>(gr) * vocab_;
     checkHip(hipMemcpyAsync(&v, src + t, sizeof v, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync");
     checkHip(hipStreamSynchronize(stream), "hipStreamSynchronize");
     return v;
