@@ -2,6 +2,8 @@
 kept candidates (ids as a set in ascending order, penalty-applied logits bit for bit; gpu_cases.compare_rows):
 - a top-k row takes its kept set from the gathered candidates (bucket finish, and the sort-based finish of tie-heavy rows),
   on rows held by one workgroup and on rows shared by several;
+- a row without a top-k that is shared by several workgroups has every part stage what the kept set can hold of its
+  slice, and the part that finishes the row picks the kept tokens out;
 - every other row is read once more by its workgroup (one pass, the waves' finds lined up in LDS), or twice when a wave
   finds more than its share of the LDS holds or when a top-k reaches into the zero-mass tail (ties by token id)."""
 import numpy as np
@@ -76,3 +78,34 @@ def test_top_k_into_the_zero_mass_tail():
     c["min_p"][:] = 0.0
     res, nk = _check(c, 1024)
     assert res["exact"] == 2 and (nk == 500).all()
+
+
+@pytest.mark.parametrize("rows", [1, 5, 20])
+def test_shared_rows_without_a_top_k_stage_their_slices(rows):
+    """Top-p / min-p rows of a small batch (8 or 4 workgroups a row): kept sets of a few to a few thousand tokens equal the
+    oracle's, launch after launch on one workspace, whose counters every launch leaves at zero; the same rows with
+    max_split = 1 (one workgroup a row, which reads the row again) give the same dump."""
+    import torch
+    c = gc.make_cfg2(rows=rows, n_hist=1024, n_bias=100)
+    c["top_k"][:] = 0
+    c["top_p"][:] = np.where(np.arange(rows) % 3 == 0, 0.5, np.where(np.arange(rows) % 3 == 1, 0.95, 1.0))
+    c["min_p"][:] = np.where(np.arange(rows) % 3 == 2, 0.001, 0.0)
+    d = gc.upload(c)
+    smp = gc.sampler_for(c, d, 1, kept_cap=16384)
+    one = gc.sampler_for(c, d, 1, kept_cap=16384, max_split=1).run()
+    torch.cuda.synchronize()
+    want_ids, want_lg, want_n = one.kept_ids.cpu().numpy(), one.kept_logits.cpu().numpy(), one.n_kept.cpu().numpy()
+    for launch in range(3):
+        smp.kept_ids.fill_(-1)
+        smp.run()
+        res = gc.compare_rows(c, smp, range(rows), 1)
+        assert res["exact"] >= rows - 1, (launch, res)
+        nk = smp.n_kept.cpu().numpy()
+        assert np.array_equal(nk, want_n), launch
+        ids, lg = smp.kept_ids.cpu().numpy(), smp.kept_logits.cpu().numpy()
+        for r in range(rows):
+            n = min(int(nk[r]), 16384)
+            assert np.array_equal(ids[r, :n], want_ids[r, :n]) and lg[r, :n].tobytes() == want_lg[r, :n].tobytes(), (launch, r)
+        ctrl = smp.workspace.view(rows, -1)[:, 65536:65536 + 256]
+        assert not ctrl.any().item(), "the rows' control words are not back at zero"
+    assert rows == 1 or nk.max() > 1000

@@ -21,9 +21,10 @@ def _run(c, rng_mode, max_split, launches=2, kept_cap=None, **more):
         smp.token.fill_(-7)
         smp.run()
     torch.cuda.synchronize()
-    if smp.workspace.numel() >= c["rows"] * 65792:  # per row: merged histogram, candidate list (scratch), control words
-        w = smp.workspace[:c["rows"] * 65792].view(c["rows"], 65792)
-        assert not w[:, :32768].any().item() and not w[:, 65536:].any().item(), "histogram / control words not zero after the launch"
+    stride = smp.workspace.numel() // c["rows"]
+    if stride >= 65792:  # per row: merged histogram, candidate list (scratch), control words; with a kept-set dump a staging area (scratch) after them
+        w = smp.workspace.view(c["rows"], stride)
+        assert not w[:, :32768].any().item() and not w[:, 65536:65792].any().item(), "histogram / control words not zero after the launch"
     return smp
 
 

@@ -48,6 +48,7 @@ struct BatchPlan {
     uint32_t lds_total;
     bool fused;
     uint32_t split_log2;  // the most parts per row that pay for this batch
+    uint64_t workspace_min;  // split rows: the least that lets them split (no staging areas), 0 when nothing is split
     uint64_t workspace;   // bytes for that
     int err;
 };
@@ -129,7 +130,10 @@ BatchPlan plan_batch(const ws_batch* b) {
         // two do not. A caller that names a number gets it.
         if (!b->max_split && lg < 2u) lg = 0;
         p.split_log2 = lg;
-        if (lg) p.workspace = uint64_t{b->rows} * ws::kSplitRowBytes;
+        // (with a kept-set dump the rows also get a staging area; a caller whose memory holds only the rows' meeting
+        // places - the library's own, ws_sample_batch_static - goes without)
+        if (lg) p.workspace_min = uint64_t{b->rows} * ws::kSplitRowBytes;
+        if (lg) p.workspace = uint64_t{b->rows} * (b->kept_ids ? ws::kSplitRowBytesKept : ws::kSplitRowBytes);
     }
     // The kernels without a bin cache (long vocabularies, unaligned rows) take the touched tokens' raw logits from
     // their first sweep when they have somewhere to put them: 8 bytes per history / bias entry and row.
@@ -385,9 +389,12 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b) {
 namespace {
 
 int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigned char* work, uint64_t work_bytes) {
-    const bool can_split = p.workspace && work && work_bytes >= p.workspace && reinterpret_cast<uintptr_t>(work) % 8u == 0;
+    const bool can_split = p.workspace_min && work && work_bytes >= p.workspace_min && reinterpret_cast<uintptr_t>(work) % 8u == 0;
+    const bool staged = can_split && work_bytes >= p.workspace && p.workspace > p.workspace_min;
     ws::BatchArgs a{};
     a.split_log2 = can_split ? p.split_log2 : 0u;
+    a.split_row_bytes = staged ? ws::kSplitRowBytesKept : ws::kSplitRowBytes;
+    a.stage_cap = staged ? ws::kSplitStageCap : 0u;
     a.work = (p.fused ? can_split : p.workspace && work && work_bytes >= p.workspace && reinterpret_cast<uintptr_t>(work) % 16u == 0) ? work : nullptr;
     a.split_spins = b->split_spins;
     a.logits = b->logits;
@@ -461,7 +468,7 @@ int ws_sample_batch_static(void* stream, const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     if (p.err != WS_OK) return p.err;
     if (!p.fused) return sample_batch_on(stream, b, p, nullptr, 0);  // (nothing may be left in the split rows' memory)
-    if (p.workspace > sizeof(scratch)) return WS_E_STATIC_LIMIT;  // more split rows than the library's own memory holds
+    if (p.workspace_min > sizeof(scratch)) return WS_E_STATIC_LIMIT;  // more split rows than the library's own memory holds
     unsigned char* at = nullptr;
     if (const int e = scratch_address(&at); e != WS_OK) return e;
     return sample_batch_on(stream, b, p, at, sizeof(scratch));

@@ -93,14 +93,20 @@ struct BatchArgs {
     double* query_prob;        // out per row or nullptr
     double* entropy;           // out per row or nullptr: entropy of the kept set
     uint32_t split_log2;       // single-sweep kernel: a row is worked on by 2^split_log2 workgroups (0: one), block = row * parts + part
-    unsigned char* work;       // split rows: kSplitRowBytes of zero-filled global memory per row, left zero-filled
+    unsigned char* work;       // split rows: split_row_bytes of zero-filled global memory per row, left zero-filled
     uint32_t split_spins;      // split rows: looks at the arrival counter before a part gives up on the others (0: about a second's worth)
+    uint32_t split_row_bytes;  // kSplitRowBytes, or kSplitRowBytesKept when the rows have a staging area
+    uint32_t stage_cap;        // entries of a row's staging area (kSplitStageCap), 0: none
 };
 
 // Global memory of a split row: the merged histogram, the merged candidate list, and four control words (parts that
 // have merged their histogram, parts that are done with the shared state, candidates listed, the row maximum as an
 // ordered integer).
 constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kSplitRowBytes = 65536u + 256u;
+// With a kept-set dump asked for, a row also has a staging area: the parts leave what the kept set can hold of their
+// slices there, in id order, and the part that finishes the row picks the kept tokens out - no workgroup reads the whole
+// row again. Control words 4 (entries staged), 8 + part (where the part's entries start) and 24 + part (how many).
+constexpr uint32_t kSplitStage = kSplitRowBytes, kSplitStageCap = 8192u, kSplitRowBytesKept = kSplitStage + kSplitStageCap * 8u;
 // Workspace of one row of the three-pass kernel: per history / bias entry a word of each of phase 0's two rank
 // tables, which sit out the first sweep there. Whole memory lines, so that rows share none.
 __host__ __device__ constexpr uint64_t capture_row_bytes(uint32_t patch_cap) {
@@ -714,10 +720,12 @@ __device__ __noinline__ TailCut tail_cut(const TailIn in) {
 // hide that distance. What a wave keeps it lines up, in order, in its share of `room` (LDS, 64 KB, idle by now); the
 // waves' counts are scanned once and every wave copies its line to its place in the output: one pass over the row, two
 // barriers. A wave that keeps more than its share holds (or a row with ties) sends the workgroup through two plain
-// passes instead - count, then rank and write.
-template <class KEEP>
-__device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, uint32_t n_equal, float floor, int32_t* kid, float* klg,
-                                                  uint32_t kept_cap, uint64_t* room, KEEP&& keep) {
+// passes instead - count, then rank and write. Where the output goes is the caller's: reserve(n), called by every
+// thread once the number of finds is known, returns the place of the first (it may hold barriers); emit(place, i, logit)
+// writes one find.
+template <class KEEP, class RESERVE, class EMIT>
+__device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, uint32_t n_equal, float floor, uint64_t* room, KEEP&& keep,
+                                                  RESERVE&& reserve, EMIT&& emit) {
     __shared__ uint32_t w_cnt[2 * WS_WAVES];
     constexpr uint32_t kShare = 8192u / WS_WAVES;  // entries of `room` per wave
     constexpr uint32_t kAhead = 16u;
@@ -804,20 +812,19 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
         __syncthreads();  // (w_cnt may still be read by an earlier call)
         if (lane == 0) w_cnt[wave] = wc;
         __syncthreads();
-        uint32_t base = 0;
+        uint32_t base = 0, all = 0;
         bool fits = true;
         for (uint32_t w = 0; w < WS_WAVES; ++w) {
             const uint32_t c = w_cnt[w];
             if (w < wave) base += c;
+            all += c;
             fits = fits && c <= kShare;
         }
         if (fits) {  // uniform over the workgroup
+            base += reserve(all);
             for (uint32_t j = lane; j < wc; j += 64u) {
                 const uint64_t en = line[j];
-                if (base + j < kept_cap) {
-                    kid[base + j] = static_cast<int32_t>(en >> 32);
-                    if (klg) klg[base + j] = __uint_as_float(static_cast<uint32_t>(en));
-                }
+                emit(base + j, static_cast<uint32_t>(en >> 32), __uint_as_float(static_cast<uint32_t>(en)));
             }
             return;
         }
@@ -838,11 +845,16 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
         w_cnt[WS_WAVES + wave] = nt;
     }
     __syncthreads();
-    uint32_t base = 0, tail_base = 0;
-    for (uint32_t w = 0; w < wave; ++w) {
-        base += w_cnt[w];
-        tail_base += w_cnt[WS_WAVES + w];
+    uint32_t base = 0, tail_base = 0, all_k = 0, all_t = 0;
+    for (uint32_t w = 0; w < WS_WAVES; ++w) {
+        if (w < wave) {
+            base += w_cnt[w];
+            tail_base += w_cnt[WS_WAVES + w];
+        }
+        all_k += w_cnt[w];
+        all_t += w_cnt[WS_WAVES + w];
     }
+    base += reserve(all_k + min(all_t, n_equal));
     if (!(nk | nt)) return;  // nothing kept in this wave's stretch (uniform over the wave; no barrier follows)
     for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
         float x[4];
@@ -857,10 +869,7 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
             const bool tie = (f >> (4 + e)) & 1u;
             const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
             const uint32_t o = kb + min(tb, n_equal);
-            if (k && o < kept_cap) {
-                kid[o] = static_cast<int32_t>(i + e);
-                if (klg) klg[o] = x[e];
-            }
+            if (k) emit(o, i + e, x[e]);
             kb += (f >> e) & 1u;
             tb += tie ? 1u : 0u;
         }
@@ -960,16 +969,106 @@ __device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float*
     const float aq = in.aq, c64 = in.c64;
     // a logit below the last kept one is not kept (floats order as their keys do)
     const float x_last = (kept_key >> 32) ? unkey32(static_cast<uint32_t>(kept_key >> 32)) : -INFINITY;
-    write_in_id_order(rv, want, cut.n_equal, want ? -INFINITY : x_last, kid, klg, kept_cap, reinterpret_cast<uint64_t*>(lds), [&](uint32_t i, float x) -> uint32_t {
-        uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
-        if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
-            // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes; among those
-            // with exactly that logit the lowest ids
-            keep = key32(x) > cut.key ? 1u : 0u;
-            if (key32(x) == cut.key) keep = 2u;
+    write_in_id_order(
+        rv, want, cut.n_equal, want ? -INFINITY : x_last, reinterpret_cast<uint64_t*>(lds),
+        [&](uint32_t i, float x) -> uint32_t {
+            uint32_t keep = key64(x, i) >= kept_key ? 1u : 0u;
+            if (want && !keep && bin_of(aq, c64, x) >= static_cast<uint32_t>(kTail)) {
+                // a zero-mass candidate: kept when its logit is above the last one a top-k of this size takes; among those
+                // with exactly that logit the lowest ids
+                keep = key32(x) > cut.key ? 1u : 0u;
+                if (key32(x) == cut.key) keep = 2u;
+            }
+            return keep;
+        },
+        [](uint32_t) { return 0u; },
+        [&](uint32_t o, uint32_t i, float x) {
+            if (o < kept_cap) {
+                kid[o] = static_cast<int32_t>(i);
+                if (klg) klg[o] = x;
+            }
+        });
+}
+
+// ---- split rows whose kept set is not among the candidates (top-p / min-p without a top-k)
+struct StageIn {
+    const void* base;       // the part's slice of the row
+    const uint32_t* allow;  // the slice's words of the allow bitmap, or nullptr
+    uint32_t V, id0;        // tokens of the slice, its first token
+    uint32_t row_V;         // tokens of the row (it lays out the touched tables)
+    int dtype;
+    uint32_t touched_at;    // LDS offset of the touched bitmap, prefix and values; ~0 when no token is touched
+    float aq, c64;
+    uint32_t last_bin;      // every kept token lies in a bin up to this one
+    uint32_t part, cap;     // this part; entries of the staging area
+};
+// Every token of the slice in a bin up to last_bin goes to the row's staging area as (id << 32 | logit bits), in id order:
+// the histogram counted them, so all parts together fit the area. Device-scope stores, like everything parts exchange.
+__device__ __noinline__ void stage_kept_superset(const StageIn in, uint64_t* stage, uint32_t* ctrl) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t s_at;
+    RowView rv;
+    rv.base = in.base;
+    rv.V = in.V;
+    rv.dtype = in.dtype;
+    rv.vec = false;
+    rv.allow = in.allow;
+    const uint32_t nW = (in.row_V + 31u) >> 5, w0 = in.id0 >> 5;
+    const bool any = in.touched_at != 0xffffffffu;
+    rv.touched = any ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) + w0 : nullptr;
+    rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (any ? in.touched_at : 0u) + nW * 4u) + w0;
+    rv.pv = reinterpret_cast<const float*>(lds + (any ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    const float aq = in.aq, c64 = in.c64;
+    const uint32_t last_bin = in.last_bin, id0 = in.id0, cap = in.cap, part = in.part;
+    __syncthreads();  // whatever used the first 64 KB of LDS before is done with it
+    write_in_id_order(
+        rv, false, 0u, -INFINITY, reinterpret_cast<uint64_t*>(lds),
+        [&](uint32_t, float x) -> uint32_t { return bin_of(aq, c64, x) <= last_bin ? 1u : 0u; },
+        [&](uint32_t n) {
+            if (threadIdx.x == 0) {
+                const uint32_t at = __hip_atomic_fetch_add(&ctrl[4], n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&ctrl[8u + part], at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&ctrl[24u + part], n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                s_at = at;
+            }
+            __syncthreads();
+            return s_at;
+        },
+        [&](uint32_t o, uint32_t i, float x) {
+            if (o < cap)
+                __hip_atomic_store(&stage[o], (static_cast<uint64_t>(id0 + i) << 32) | __float_as_uint(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        });
+}
+// The finisher's side: the staged entries at or above the last kept key, part after part (ids ascend inside a part and
+// from part to part). False when the area did not hold everything.
+__device__ __noinline__ bool dump_staged(const uint64_t* stage, uint32_t* ctrl, uint32_t n_parts, uint32_t cap, uint64_t kept_key, int32_t* kid,
+                                         float* klg, uint32_t kept_cap) {
+    __shared__ uint32_t d_red[WS_WAVES];
+    if (__hip_atomic_load(&ctrl[4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > cap) return false;  // uniform
+    uint32_t out = 0;
+    for (uint32_t p = 0; p < n_parts; ++p) {
+        const uint32_t at = __hip_atomic_load(&ctrl[8u + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t n = __hip_atomic_load(&ctrl[24u + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t j0 = 0; j0 < n; j0 += WS_BLOCK) {
+            const uint32_t j = j0 + threadIdx.x;
+            uint32_t keep = 0, id = 0;
+            float x = 0.f;
+            if (j < n) {
+                const uint64_t en = __hip_atomic_load(&stage[at + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                id = static_cast<uint32_t>(en >> 32);
+                x = __uint_as_float(static_cast<uint32_t>(en));
+                keep = key64(x, id) >= kept_key ? 1u : 0u;
+            }
+            uint32_t tot;
+            const uint32_t before = block_excl_scan(keep, d_red, &tot);
+            if (keep && out + before < kept_cap) {
+                kid[out + before] = static_cast<int32_t>(id);
+                if (klg) klg[out + before] = x;
+            }
+            out += tot;
         }
-        return keep;
-    });
+    }
+    return true;
 }
 
 struct ExactIn {
@@ -1517,7 +1616,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             rank1 = id0 + rvs.V < V ? wprefix[(id0 + rvs.V) >> 5] : n_touched;
         }
     }
-    unsigned char* work = split ? A.work + static_cast<size_t>(row) * kSplitRowBytes : nullptr;
+    unsigned char* work = split ? A.work + static_cast<size_t>(row) * A.split_row_bytes : nullptr;
     uint32_t* ctrl = reinterpret_cast<uint32_t*>(work + kSplitCtrl);
     __shared__ uint32_t s_prev;
     // done with the row's shared memory: true for the part that says so last, which then has to clean it
@@ -2349,6 +2448,17 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     constexpr uint32_t kDumpListed = 1024u;  // candidates ranked by id against each other
     const bool dump_listed =
         FUSED && kept_ids && (prefix_mode || open_row) && n1 == n1_asked && !race && !(flags & kOverflow) && n_r0 <= kDumpListed;
+    // A split row whose kept set is not among its candidates (top-p / min-p without a top-k): the parts stage what the
+    // kept set can hold of their slices - every token in a bin up to the lowest gathered one; the histogram knows how
+    // many - and the finisher picks the kept ones out. stage_last: that bin, ~0 when the row goes another way.
+    uint32_t stage_last = 0xffffffffu;
+    constexpr uint32_t kStaged = 0x40000000u;  // in `flags`, inside the kernel: the parts have staged their slices
+    if constexpr (SPLIT && KEPT) {
+        if (kept_ids && A.stage_cap && split && !prefix_mode && !open_row && !race && !(flags & kOverflow)) {  // (a top-k row is either listed or keeps zero-mass candidates)
+            const int last = max(r0hi, has_r1 ? r1hi : -1);
+            if (last >= 0 && last < kTail && pc[last + 1] <= A.stage_cap) stage_last = static_cast<uint32_t>(last);
+        }
+    }
     bool dumped = false;       // the dump is done
     uint32_t listed_n = 0;     // entries of the candidate list after a bucket finish
     // kPartialTables in `flags` (inside the kernel only): pv[] holds the adjusted logits of this part's slice alone - the
@@ -2483,6 +2593,25 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                             __hip_atomic_store(reinterpret_cast<uint64_t*>(&glist[gbase + k]), (static_cast<uint64_t>(en.y) << 32) | en.x, __ATOMIC_RELAXED,
                                                __HIP_MEMORY_SCOPE_AGENT);
                         }
+                    if constexpr (SPLIT && KEPT) {
+                        if (stage_last != 0xffffffffu) {  // uniform over the parts
+                            StageIn in;
+                            in.base = rvs.base;
+                            in.allow = rvs.allow;
+                            in.V = rvs.V;
+                            in.id0 = id0;
+                            in.row_V = V;
+                            in.dtype = rv.dtype;
+                            in.touched_at = rv.touched ? A.lds_ab : 0xffffffffu;
+                            in.aq = aq;
+                            in.c64 = c64;
+                            in.last_bin = stage_last;
+                            in.part = part;
+                            in.cap = A.stage_cap;
+                            stage_kept_superset(in, reinterpret_cast<uint64_t*>(work + kSplitStage), ctrl);
+                            flags |= kStaged;
+                        }
+                    }
                     if (!leave_shared()) return;
                     const uint32_t total = __hip_atomic_load(&ctrl[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     flags &= ~kOverflow;
@@ -2494,7 +2623,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     }
                     clean_shared();
                     split = false;  // the row is this part's from here
-                    if ((kept_ids && !dump_listed) || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
+                    if ((kept_ids && !dump_listed && !(flags & kStaged)) || A.query_prob || race || open_row || (flags & kOverflow)) {  // they look at any token of the row
                         float ma, mu;
                         collect_fused(nullptr, 0u, false, aq, c64, ma, mu, 0u, V, 0u);
                     } else {
@@ -3724,13 +3853,25 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
             if ((k < 11u || k > 14u) && ws_marks[k]) dbg[k] = static_cast<float>(ws_marks[k] - ws_t0);
     }
 #endif
+    if constexpr (SPLIT && KEPT) {
+        if (flags & kStaged) {  // uniform: this is the part that finishes the row
+            __syncthreads();
+            if (token >= 0 && !dumped && !finished_slow && kept_key != 0ull &&
+                dump_staged(reinterpret_cast<const uint64_t*>(work + kSplitStage), ctrl, n_parts, A.stage_cap, kept_key,
+                            kept_ids + static_cast<size_t>(row) * A.kept_cap,
+                            A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr, A.kept_cap))
+                dumped = true;
+            __syncthreads();
+            if (t < 33u) ctrl[t == 0u ? 4u : 7u + t] = 0u;  // words 4 and 8 .. 39, zero again for the next launch
+        }
+    }
     if (WS_RARE(kept_ids && token >= 0 && !dumped && (flags & kPartialTables) && !(dump_listed && finished_lean))) {  // (no way to the kept set: reported unresolved)
         flags |= kOverflow;
         token = -1;
     }
     if (t == 0) {
         A.token[row] = token;
-        A.flags[row] = flags & ~kPartialTables;
+        A.flags[row] = flags & ~(kPartialTables | kStaged);
         if (A.prob) A.prob[row] = static_cast<float>(ptok);
         if (A.n_kept) A.n_kept[row] = n3 + tail_extra;
         if (A.stats) {
