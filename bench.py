@@ -31,8 +31,8 @@ MODE = 0
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, sha256[:16] of whirl-llm_amd/csrc/ws_sample.h at the time)
-    ("tile", "auto"): (168794956, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "297b1988ace82537"),
-    ("tile", "exact"): (539607086, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "297b1988ace82537"),
+    ("tile", "auto"): (168797996, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "41d642cc7fe04d4a"),
+    ("tile", "exact"): (539606657, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "41d642cc7fe04d4a"),
 }
 
 

@@ -231,8 +231,10 @@ typedef struct ws_batch {
     double* margin;     /* out (may be NULL): [rows][3] distance of the top-p cut, min-p floor and draw to flipping */
     int32_t* kept_ids;  /* out (may be NULL): [rows][kept_cap] kept token ids in ascending id order (the first n_kept, or
                            the first kept_cap of them). Free for a top-k row of up to about a thousand candidates (they
-                           are among what the kernel gathered anyway); any other row is read once more by its workgroup,
-                           about 60 us for a row of 151936 on the compute unit that holds it.
+                           are among what the kernel gathered anyway). A row without a top-k that is shared by several
+                           workgroups (see workspace) has its parts stage their slices' share, about 15 us a launch; any
+                           other row is read once more by its workgroup, about 60 us for a row of 151936 on the compute
+                           unit that holds it.
                            Parameters and outputs may live in pinned host memory (hipHostMalloc): the kernels then read
                            and write them in place and a synchronous caller needs no copy at all. */
     float* kept_logits; /* out (may be NULL): penalty-applied logits of kept_ids */
@@ -242,7 +244,9 @@ typedef struct ws_batch {
                                (a) small batches: with fewer rows than the GPU has compute units a row is worked on by
                                several workgroups, which meet in this memory. The caller zero-fills it once before its
                                first use and leaves it alone afterwards: every launch puts back the zeros the next one
-                               needs; (b) rows of the kernels that sweep the row twice (long or unaligned vocabularies)
+                               needs (with kept_ids set the size asked for includes a staging area per row; memory that
+                               holds only the rows' meeting places, 65792 bytes a row, still lets them be shared);
+                               (b) rows of the kernels that sweep the row twice (long or unaligned vocabularies)
                                that have a history or a bias: the first sweep leaves the raw logits of those tokens
                                here (8 bytes per history / bias entry) instead of gathering them one by one, and
                                leaves the memory with arbitrary contents - zero-fill it again before a batch of
@@ -287,7 +291,8 @@ int ws_sample_batch(void* stream, const ws_batch* b);
  * than that (65 to 128 rows in two parts each) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is
  * looked up on the first call there (or by ws_probe): make that call before capturing a graph. All calls on one GPU
  * share this memory: two of them that run at the same time (different streams) race; on one stream they are safe, each
- * launch leaves the memory as the next needs it. (Only split rows use it: use (b) of b->workspace is off here.) */
+ * launch leaves the memory as the next needs it. (Only split rows use it: use (b) of b->workspace is off here, and so
+ * are the staging areas of the kept-set dump - a shared row without a top-k is read again by the workgroup that finishes it.) */
 #define WS_STATIC_SPLIT_ROWS 64
 int ws_sample_batch_static(void* stream, const ws_batch* b);
 
