@@ -26,13 +26,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MODE = 0
+KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # HBM bytes per launch of ws::sample_batch_kernel: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter
 # reads for a 256 MiB device copy; measured for one build of the kernel and only reported for that build (the digest
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, sha256[:16] of whirl-llm_amd/csrc/ws_sample.h at the time)
-    ("tile", "auto"): (168797996, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "41d642cc7fe04d4a"),
-    ("tile", "exact"): (539606657, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "41d642cc7fe04d4a"),
+    ("tile", "auto"): (168794330, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "43782f5d5df852b3"),
+    ("tile", "exact"): (539596577, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "43782f5d5df852b3"),
 }
 
 
@@ -80,7 +81,7 @@ def time_gpu(c, steps, warmup, rng_mode=1):
     import torch
     gc = workloads()
     d = gc.upload(c)
-    smp = gc.sampler_for(c, d, rng_mode, mode=MODE)
+    smp = gc.sampler_for(c, d, rng_mode, mode=MODE, kept_cap=KEPT_CAP)
     for _ in range(warmup):
         smp.run()
     torch.cuda.synchronize()
@@ -354,6 +355,9 @@ def main():
     ap.add_argument("--no-also", action="store_true")
     ap.add_argument("--check-rows", type=int, default=8)
     ap.add_argument("--mode", default="auto", choices=["auto", "exact", "fused"], help="ws_batch.mode for every workload")
+    ap.add_argument("--kept-cap", type=int, default=0,
+                    help="also ask for the kept-set dump (ws_batch.kept_ids / kept_logits, this many entries a row), as the C++ host API "
+                         "does: the launches then take the builds of the kernels that can write it")
     ap.add_argument("--reference-kernels", action="store_true",
                     help="time the replacements of the reference's own kernels (greedy picks, topk_rows) instead and print "
                          "their launch times as one JSON line")
@@ -380,8 +384,9 @@ def main():
     if a.reference_kernels:
         print(json.dumps({"reference_kernels": reference_kernels(max(20, a.steps // 4)), "data": "synthetic"}))
         return
-    global MODE
+    global MODE, KEPT_CAP
     MODE = {"auto": 0, "exact": 1, "fused": 2}[a.mode]
+    KEPT_CAP = a.kept_cap
     check = 0 if a.no_cpu else a.check_rows
     c, main_res = run_workload(a.workload, a.steps, a.warmup, check)
     also = []
@@ -404,7 +409,7 @@ def main():
         "config": {"workload": a.workload, "rows": c["rows"], "vocab": c["V"], "logits": c["dtype"],
                    "history_ids_per_row": 0 if c["hist"] is None else int(c["hist"].shape[1]),
                    "filters": "see whirl-llm_amd/workloads.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
-                   "sweep_mode": a.mode},
+                   "sweep_mode": a.mode, "kept_cap": a.kept_cap},
         "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "ws::sample_batch_kernel", "kernel_source_digest": kernel_digest(),

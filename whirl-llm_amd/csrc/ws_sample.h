@@ -829,13 +829,20 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
             return;
         }
     }
-    // ---- two passes, a tile at a time (rare)
+    // ---- two passes, eight tiles on their way at a time (kept sets of many thousands, rows with ties)
+    constexpr uint32_t kAhead2 = 8u;
     uint32_t nk = 0, nt = 0;
-    for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
-        float x[4];
-        const uint32_t f = judge(i0 + 4u * lane, fetch(i0 + 4u * lane, std::false_type{}), x);
-        nk += __popc(f & 0xfu);
-        nt += __popc(f >> 4);
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
+        uint4 raw[kAhead2];
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, std::false_type{});
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead2; ++u) {
+            float x[4];
+            const uint32_t f = judge(i0 + 256u * u + 4u * lane, raw[u], x);
+            nk += __popc(f & 0xfu);
+            nt += __popc(f >> 4);
+        }
     }
     nk = wave_sum(nk);
     nt = wave_sum(nt);
@@ -856,26 +863,32 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
     }
     base += reserve(all_k + min(all_t, n_equal));
     if (!(nk | nt)) return;  // nothing kept in this wave's stretch (uniform over the wave; no barrier follows)
-    for (uint32_t i0 = lo; i0 < hi; i0 += 256u) {
-        float x[4];
-        const uint32_t i = i0 + 4u * lane;
-        const uint32_t f = judge(i, fetch(i, std::false_type{}), x);
-        if (!__ballot(f != 0u)) continue;
-        const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
-        const uint32_t inc = wave_incl_scan(mine);
-        uint32_t kb = base + ((inc - mine) & 0xffffu), tb = tail_base + ((inc - mine) >> 16);
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
+        uint4 raw[kAhead2];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const bool tie = (f >> (4 + e)) & 1u;
-            const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
-            const uint32_t o = kb + min(tb, n_equal);
-            if (k) emit(o, i + e, x[e]);
-            kb += (f >> e) & 1u;
-            tb += tie ? 1u : 0u;
+        for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, std::false_type{});
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead2; ++u) {
+            float x[4];
+            const uint32_t i = i0 + 256u * u + 4u * lane;
+            const uint32_t f = judge(i, raw[u], x);
+            if (!__ballot(f != 0u)) continue;
+            const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
+            const uint32_t inc = wave_incl_scan(mine);
+            uint32_t kb = base + ((inc - mine) & 0xffffu), tb = tail_base + ((inc - mine) >> 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bool tie = (f >> (4 + e)) & 1u;
+                const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
+                const uint32_t o = kb + min(tb, n_equal);
+                if (k) emit(o, i + e, x[e]);
+                kb += (f >> e) & 1u;
+                tb += tie ? 1u : 0u;
+            }
+            const uint32_t tot = last_lane(inc);
+            base += tot & 0xffffu;
+            tail_base += tot >> 16;
         }
-        const uint32_t tot = last_lane(inc);
-        base += tot & 0xffffu;
-        tail_base += tot >> 16;
     }
 }
 
