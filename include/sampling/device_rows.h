@@ -61,6 +61,10 @@ public:
     float logitAt(std::uint32_t gr, std::uint32_t t) override;
     std::uint32_t nVocab() const override { return vocab_; }
     std::uint8_t* inCands() override { return marks_.data(); }
+    // The device drew a token when it filtered the row (same uniform, same walk: candidates in sorted order, then the
+    // rest of the row in id order). It stands for the host's walk when the sampler still is as it was at prepareRow and the
+    // device did not flag the draw as close to a boundary.
+    bool drawnToken(const Sampler& s, std::uint32_t& token) override;
 
     std::uint32_t lastFlags() const { return last_flags_; }  // WS_FLAG_* of the last prepared row
 
@@ -84,6 +88,9 @@ private:
     Dev* dev_;
     std::vector<std::uint8_t> marks_;
     std::uint32_t last_flags_ = 0;
+    std::int32_t last_token_ = -1;      // the device's own draw for the last prepared row, -1: none
+    std::uint32_t last_row_ = 0xffffffffu;
+    std::uint64_t last_pos_ = 0, last_seed_ = 0;
     std::vector<Ready> ready_;
     ReadyKey ready_key_;
     static constexpr std::uint32_t kNoRow = 0xffffffffu;

@@ -79,16 +79,21 @@ def test_decode_steps_over_one_device_rows_object():
     m = gc.pkg()
     c = gc.make_cfg1()
     d = gc.upload(c)
-    for top_k, top_p, hist in ((40, 0.95, None), (40, 0.95, c["hist"][0]), (0, 0.9, c["hist"][0])):
+    # (the last two: no filter at all - at temperature 2 most draws walk past the 256 listed candidates, and the device's
+    # own walk of the row stands in for the host's)
+    for top_k, top_p, hist, inv_t in ((40, 0.95, None, None), (40, 0.95, c["hist"][0], None), (0, 0.9, c["hist"][0], None),
+                                      (0, 1.0, c["hist"][0], None), (0, 1.0, c["hist"][0], 0.5)):
         cc = dict(c)
+        if inv_t is not None:
+            cc["inv_t"] = np.array([inv_t], np.float32)
         cc["top_k"] = np.array([top_k], np.uint32)
         cc["top_p"] = np.array([top_p])
         cc["hist"] = None if hist is None else c["hist"]
         if hist is None:
             cc["rep"] = np.ones(1, np.float32)
-        tok, us, n_kept, flags = m.host_decode_steps(d["logits"][0], c["inv_t"][0], int(c["seed"][0]), 100, 12, warmup=2, top_k=top_k,
+        tok, us, n_kept, flags = m.host_decode_steps(d["logits"][0], cc["inv_t"][0], int(c["seed"][0]), 100, 12, warmup=2, top_k=top_k,
                                                      top_p=top_p, hist=hist, rep=float(cc["rep"][0]))
-        assert us > 0 and n_kept >= 1 and not flags & (m.FLAG_OVERFLOW | m.FLAG_OPEN)
+        assert us > 0 and n_kept >= 1 and not flags & m.FLAG_OVERFLOW and bool(flags & m.FLAG_OPEN) == (top_k == 0 and top_p == 1.0)
         for i in range(12):
             cc["step"] = np.array([100 + i], np.uint64)
             o, _, _ = gc.oracle_row(cc, 0, 0)

@@ -112,6 +112,8 @@ struct DeviceRows::Ready {
     std::uint32_t gr;
     std::uint32_t n_kept, flags;
     float m, sum;
+    std::int32_t token;            // the device's own draw, made with seed and pos
+    std::uint64_t seed, pos;
     std::vector<std::int32_t> ids;
     std::vector<float> logits;
 };
@@ -136,11 +138,13 @@ void DeviceRows::setAdjust(const RowAdjust& a) {
     adj_ = a;
     ready_.clear();  // rows filtered under the old penalties are of no use any more
     adjusted_row_ = kNoRow;
+    last_token_ = -1;
 }
 
 void DeviceRows::newCycle() {
     ready_.clear();
     adjusted_row_ = kNoRow;
+    last_token_ = -1;
 }
 
 namespace {
@@ -294,6 +298,9 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
         q.flags = h.flags[r];
         q.m = h.stats[2 * r];
         q.sum = h.stats[2 * r + 1];
+        q.token = h.token[r];
+        q.seed = s.seed;
+        q.pos = s.pos_idx;
         if ((q.flags & unresolved) || q.n_kept > cap) continue;  // such a row is escalated when it is asked for
         // (an open row's list - the engine's short candidate list - comes back like a kept set)
         q.ids.assign(d.kept_ids + std::size_t{r} * cap, d.kept_ids + std::size_t{r} * cap + q.n_kept);
@@ -322,6 +329,10 @@ void DeviceRows::prepareRow(Sampler& s, std::uint32_t r) {
     // use would hand last step's candidates to the next cycle's call for the same row.
     q->gr = kNoRow;
     last_flags_ = q->flags;
+    last_token_ = s.race ? -1 : q->token;  // (the device was not asked for the race draw)
+    last_row_ = gr;
+    last_seed_ = q->seed;
+    last_pos_ = q->pos;
     const std::uint32_t cap = std::min(kKeptCap, vocab_);
     const std::uint32_t unresolved = WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
     if ((q->flags & unresolved) || q->n_kept > cap) {
@@ -426,6 +437,13 @@ void DeviceRows::escalate(Sampler& s, std::uint32_t gr) {
     const float* x = loadFullRow(gr);
     for (std::uint32_t j = 0; j < vocab_; ++j) c[j] = {j, x[j], 0.0};
     filterCands(s, vocab_, true);
+}
+
+bool DeviceRows::drawnToken(const Sampler& s, std::uint32_t& token) {
+    const std::uint32_t doubtful = WS_FLAG_NEAR_TOP_P | WS_FLAG_NEAR_MIN_P | WS_FLAG_NEAR_DRAW | WS_FLAG_OVERFLOW | WS_FLAG_BAD_PARAM | WS_FLAG_ALL_MASKED;
+    if (last_token_ < 0 || s.race || s.row != last_row_ || s.seed != last_seed_ || s.pos_idx != last_pos_ || (last_flags_ & doubtful)) return false;
+    token = static_cast<std::uint32_t>(last_token_);
+    return true;
 }
 
 const float* DeviceRows::loadFullRow(std::uint32_t gr) {
