@@ -243,9 +243,10 @@ typedef struct ws_batch {
     void* workspace;        /* device scratch, ws_sample_batch_workspace() bytes, 16-byte aligned, or NULL. It serves
                                (a) small batches: with fewer rows than the GPU has compute units a row is worked on by
                                several workgroups, which meet in this memory. The caller zero-fills it once before its
-                               first use and leaves it alone afterwards: every launch puts back the zeros the next one
-                               needs (with kept_ids set the size asked for includes a staging area per row; memory that
-                               holds only the rows' meeting places, 65792 bytes a row, still lets them be shared);
+                               first use and leaves it alone afterwards: every launch leaves all of it zero-filled again,
+                               so batches of any shape may follow each other on it (with kept_ids set the size asked for
+                               includes a staging area per row; memory that holds only the rows' meeting places, 65792
+                               bytes a row, still lets them be shared);
                                (b) rows of the kernels that sweep the row twice (long or unaligned vocabularies)
                                that have a history or a bias: the first sweep leaves the raw logits of those tokens
                                here (8 bytes per history / bias entry) instead of gathering them one by one, and

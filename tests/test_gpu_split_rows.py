@@ -22,9 +22,9 @@ def _run(c, rng_mode, max_split, launches=2, kept_cap=None, **more):
         smp.run()
     torch.cuda.synchronize()
     stride = smp.workspace.numel() // c["rows"]
-    if stride >= 65792:  # per row: merged histogram, candidate list (scratch), control words; with a kept-set dump a staging area (scratch) after them
+    if stride >= 65792:  # per row: merged histogram, candidate list, control words; with a kept-set dump a staging area after them
         w = smp.workspace.view(c["rows"], stride)
-        assert not w[:, :32768].any().item() and not w[:, 65536:65792].any().item(), "histogram / control words not zero after the launch"
+        assert not w.any().item(), "the workspace is not zero after the launch"
     return smp
 
 

@@ -1053,11 +1053,13 @@ __device__ __noinline__ void stage_kept_superset(const StageIn in, uint64_t* sta
         });
 }
 // The finisher's side: the staged entries at or above the last kept key, part after part (ids ascend inside a part and
-// from part to part). False when the area did not hold everything.
-__device__ __noinline__ bool dump_staged(const uint64_t* stage, uint32_t* ctrl, uint32_t n_parts, uint32_t cap, uint64_t kept_key, int32_t* kid,
-                                         float* klg, uint32_t kept_cap) {
+// from part to part), when `write`; false when nothing was written or the area did not hold everything. Every entry is
+// set back to zero on the way, written or not: a launch leaves the whole workspace zero-filled, whatever layout the next
+// one lays over it.
+__device__ __noinline__ bool dump_staged(uint64_t* stage, uint32_t* ctrl, uint32_t n_parts, uint32_t cap, bool write, uint64_t kept_key,
+                                         int32_t* kid, float* klg, uint32_t kept_cap) {
     __shared__ uint32_t d_red[WS_WAVES];
-    if (__hip_atomic_load(&ctrl[4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > cap) return false;  // uniform
+    if (__hip_atomic_load(&ctrl[4], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > cap) write = false;  // uniform
     uint32_t out = 0;
     for (uint32_t p = 0; p < n_parts; ++p) {
         const uint32_t at = __hip_atomic_load(&ctrl[8u + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1066,11 +1068,12 @@ __device__ __noinline__ bool dump_staged(const uint64_t* stage, uint32_t* ctrl, 
             const uint32_t j = j0 + threadIdx.x;
             uint32_t keep = 0, id = 0;
             float x = 0.f;
-            if (j < n) {
+            if (j < n && at + j < cap) {
                 const uint64_t en = __hip_atomic_load(&stage[at + j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                stage[at + j] = 0ull;
                 id = static_cast<uint32_t>(en >> 32);
                 x = __uint_as_float(static_cast<uint32_t>(en));
-                keep = key64(x, id) >= kept_key ? 1u : 0u;
+                keep = write && key64(x, id) >= kept_key ? 1u : 0u;
             }
             uint32_t tot;
             const uint32_t before = block_excl_scan(keep, d_red, &tot);
@@ -1081,7 +1084,7 @@ __device__ __noinline__ bool dump_staged(const uint64_t* stage, uint32_t* ctrl, 
             out += tot;
         }
     }
-    return true;
+    return write;
 }
 
 struct ExactIn {
@@ -2633,6 +2636,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
                     for (uint32_t k = t; k < n_hit; k += WS_BLOCK) {
                         const uint64_t en = __hip_atomic_load(reinterpret_cast<uint64_t*>(&glist[k]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         list[k] = make_uint2(static_cast<uint32_t>(en), static_cast<uint32_t>(en >> 32));
+                        reinterpret_cast<uint64_t*>(glist)[k] = 0ull;  // (the whole workspace is zero again after a launch, whatever rows the next lays over it)
                     }
                     clean_shared();
                     split = false;  // the row is this part's from here
@@ -3869,9 +3873,8 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
     if constexpr (SPLIT && KEPT) {
         if (flags & kStaged) {  // uniform: this is the part that finishes the row
             __syncthreads();
-            if (token >= 0 && !dumped && !finished_slow && kept_key != 0ull &&
-                dump_staged(reinterpret_cast<const uint64_t*>(work + kSplitStage), ctrl, n_parts, A.stage_cap, kept_key,
-                            kept_ids + static_cast<size_t>(row) * A.kept_cap,
+            if (dump_staged(reinterpret_cast<uint64_t*>(work + kSplitStage), ctrl, n_parts, A.stage_cap,
+                            token >= 0 && !dumped && !finished_slow && kept_key != 0ull, kept_key, kept_ids + static_cast<size_t>(row) * A.kept_cap,
                             A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr, A.kept_cap))
                 dumped = true;
             __syncthreads();
