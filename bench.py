@@ -32,8 +32,8 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, sha256[:16] of whirl-llm_amd/csrc/ws_sample.h at the time)
-    ("tile", "auto"): (168794330, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "43782f5d5df852b3"),
-    ("tile", "exact"): (539596577, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "43782f5d5df852b3"),
+    ("tile", "auto"): (168795725, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
+    ("tile", "exact"): (539588491, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
 }
 
 
