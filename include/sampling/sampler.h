@@ -72,7 +72,7 @@ public:
     virtual std::uint32_t nVocab() const = 0;
     // n_vocab bytes of scratch for marking candidates during a tail walk.
     virtual std::uint8_t* inCands() = 0;
-    XX: a source that has already made the
+    // Not in the reference's interface (src/sampling/sampler.h:60-73), and optional: a source that has already made the
     // inverse-CDF draw of the prepared row for exactly this sampler state (same row, seed and pos_idx, nothing excluded)
     // hands the token over, and sampleRow then need not walk the rest of an open row on the host. The token must be the
     // one the walk would find.
