@@ -331,18 +331,25 @@ def spec_verify_workload(steps, warmup):
 
 
 def host_decode_step(steps):
-    """Wall clock of the C++ host API's decode step on configs[0] (one row of 151936 fp32 logits on the device, top-k 40,
-    top-p 0.95, 256-id history with repetition 1.1): sampling::DeviceRows::newCycle + prepareRow + sampling::sampleRow,
-    one object serving every step, as the engine's decode loop calls it."""
+    """Wall clock of the C++ host API's decode step on configs[0]'s row (151936 fp32 logits on the device, temperature 0.8,
+    256-id history with repetition 1.1): sampling::DeviceRows::newCycle + prepareRow + sampling::sampleRow, one object serving
+    every step, as the engine's decode loop calls it - with configs[0]'s own filters (top-k 40 + top-p 0.95), with top-p 0.9
+    alone and without any filter."""
     from __graft_entry__ import load_package
     m = load_package()
     w = workloads()
     c = w.make_cfg1()
     d = w.upload(c)
-    _, us, n_kept, _ = m.host_decode_steps(d["logits"][0], c["inv_t"][0], int(c["seed"][0]), 0, steps, warmup=20, top_k=int(c["top_k"][0]),
-                                           top_p=float(c["top_p"][0]), hist=c["hist"][0], rep=float(c["rep"][0]))
-    return {"workload": "host_api_decode_step (cfg1 through sampling::DeviceRows + sampleRow)", "us_per_token": us, "tokens_per_s": 1e6 / us,
-            "steps": steps, "n_kept": int(n_kept), "clock": "host wall clock, launch + stream wait + host filter included"}
+    out = {"workload": "host_api_decode_step (cfg1's row through sampling::DeviceRows + sampleRow)", "steps": steps,
+           "clock": "host wall clock, launch + stream wait + host filter included"}
+    for name, top_k, top_p in (("us_per_token", int(c["top_k"][0]), float(c["top_p"][0])), ("us_per_token_top_p_only", 0, 0.9),
+                               ("us_per_token_no_filter", 0, 1.0)):
+        _, us, n_kept, _ = m.host_decode_steps(d["logits"][0], c["inv_t"][0], int(c["seed"][0]), 0, steps, warmup=20, top_k=top_k, top_p=top_p,
+                                               hist=c["hist"][0], rep=float(c["rep"][0]))
+        out[name] = us
+        out[name.replace("us_per_token", "n_kept")] = int(n_kept)
+    out["tokens_per_s"] = 1e6 / out["us_per_token"]
+    return out
 
 
 def main():
