@@ -273,10 +273,10 @@ typedef struct ws_batch {
     double* entropy;            /* out (may be NULL): -sum p ln p over the kept set (renormalised p; an open row: over its
                                    256 candidates with their shares of the whole row), what the typical acceptance rule
                                    compares with (src/sampling/acceptor.cpp:77-84). See WS_FLAG_APPROX_ENTROPY. */
-    uint32_t max_split;         /* most workgroups a row may be split over (a power of two, rows * parts within the GPU's
-                                   compute units, at least 16384 tokens a part - which makes it 8 at most for the rows the
-                                   single-sweep kernel takes): 0 = the library decides (4 or 8 parts when the batch is small
-                                   enough for that, else none), 1 = never split */
+    uint32_t max_split;         /* most workgroups a row may be split over (a power of two up to 16, rows * parts within the
+                                   GPU's compute units, at least 16384 tokens a part - 8192 for 16 parts): 0 = the library
+                                   decides (4, 8 or 16 parts when the batch is small enough for that, else none), 1 = never
+                                   split */
     uint32_t split_spins;       /* split rows: how often a part looks for the others before it gives up on them (they all
                                    have to be running at once, which a GPU shared with other work may not allow in time); the
                                    row is then done by one workgroup - slower, same result. 0 = about a second's worth */

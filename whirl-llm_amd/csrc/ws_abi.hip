@@ -116,7 +116,7 @@ BatchPlan plan_batch(const ws_batch* b) {
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
     // Small batches of the single-sweep kernel: with rows to spare on the compute units a row is split over 2, 4, 8 or
-    // 16 workgroups (each at least 16384 tokens), which meet in global memory. All parts of all rows have to be running
+    // 16 workgroups (each at least 16384 tokens; 8192 for the step from 8 to 16, which a lone 151936-token row still wins: 29.2 -> 28.0 us), which meet in global memory. All parts of all rows have to be running
     // at the same time - they wait for each other - so rows * parts stays within the compute units of the device.
     p.split_log2 = 0;
     p.workspace = 0;
@@ -124,7 +124,7 @@ BatchPlan plan_batch(const ws_batch* b) {
         const uint32_t cus = static_cast<uint32_t>(compute_units());
         const uint32_t most = b->max_split ? b->max_split : 16u;
         uint32_t lg = 0;
-        while (lg < 4u && (2u << lg) <= most && b->rows * (2u << lg) <= cus && b->vocab / (2u << lg) >= 16384u) ++lg;
+        while (lg < 4u && (2u << lg) <= most && b->rows * (2u << lg) <= cus && b->vocab / (2u << lg) >= (lg == 3u ? 8192u : 16384u)) ++lg;
         // Meeting in global memory costs two round trips of several thousand clocks each; measured on batches of
         // 151936-token rows, four parts and more win that back (64 rows: 49.5 against 52.9 us; 16 rows: 40 against 50),
         // two do not. A caller that names a number gets it.
