@@ -10,7 +10,9 @@ presence / frequency penalties over a 2048-id history per row, temperature in [0
 off, so every row needs a full-vocabulary mass select), seeded Philox draws. One JSON line goes to stdout.
 
 roofline.achieved = algorithmic bytes per launch / average launch duration, measured with HIP events recorded on the
-stream the kernel is launched on. Algorithmic bytes = rows * vocab * sizeof(logit) + 4 bytes per history id + 8 bytes
+stream the kernel is launched on, over launches that each read another copy of the logits (the copies together larger
+than the 256 MiB memory-side cache, so the rows come from HBM); roofline.achieved_warm is the same over launches that
+all read one resident copy. Algorithmic bytes = rows * vocab * sizeof(logit) + 4 bytes per history id + 8 bytes
 per bias entry + allow-mask bitmap + 16 bytes of output per row.
 cpu_baseline = the reference's own sampler (oracle/_ref, compiled from the reference sources in the build container)
 or, where that library is absent, the oracle's restatement of it, one thread, on the first rows of the same batch.
@@ -77,24 +79,51 @@ def algorithmic_bytes(c):
     return b
 
 
+INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache: a buffer re-read every launch can be served from it
+
+
+def rotation_for(nbytes):
+    """Distinct copies of a workload's logits to rotate through so that no launch finds its rows in the memory-side
+    cache: the copies together hold at least 2.5 times the cache (one copy when a single launch already streams more)."""
+    if nbytes >= 2 * INFINITY_CACHE_BYTES:
+        return 1
+    return max(2, -(-int(2.5 * INFINITY_CACHE_BYTES) // nbytes))
+
+
 def time_gpu(c, steps, warmup, rng_mode=1):
+    """Times `steps` launches twice: `cold` - each launch reads another copy of the logits, the copies together larger than
+    the memory-side cache, so the row bytes come from HBM - and `warm` - every launch on the one resident copy. Returns
+    (sampler, wall ms per step cold, kernel ms per step cold, kernel ms per step warm, copies)."""
     import torch
     gc = workloads()
     d = gc.upload(c)
     smp = gc.sampler_for(c, d, rng_mode, mode=MODE, kept_cap=KEPT_CAP)
-    for _ in range(warmup):
-        smp.run()
+    base = d["logits"]
+    n_rot = rotation_for(base.numel() * base.element_size())
+    copies = [base] + [base.clone() for _ in range(n_rot - 1)]
+    ptrs = [t.data_ptr() for t in copies]
+
+    def timed(rotate):
+        for k in range(warmup):
+            smp.desc.logits = ptrs[k % n_rot] if rotate else ptrs[0]
+            smp.run()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ev0.record()
+        for k in range(steps):
+            smp.desc.logits = ptrs[k % n_rot] if rotate else ptrs[0]
+            smp.run()
+        ev1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+    _, warm_ms = timed(False)
+    wall_ms, kern_ms = timed(True)
+    smp.desc.logits = ptrs[0]
+    smp.run()  # the outputs the parity leg reads belong to the first copy's launch (all copies hold the same logits)
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(steps):
-        smp.run()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    kern_ms = ev0.elapsed_time(ev1) / steps
-    return smp, wall_ms, kern_ms
+    return smp, wall_ms, kern_ms, warm_ms, n_rot
 
 
 def device_report(smp):
@@ -194,11 +223,13 @@ def run_workload(name, steps, warmup, check_rows):
     gc = workloads()
     make = dict(tile=gc.make_tile, cfg1=gc.make_cfg1, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
     c = make()
-    smp, wall_ms, kern_ms = time_gpu(c, steps, warmup)
+    smp, wall_ms, kern_ms, warm_ms, n_rot = time_gpu(c, steps, warmup)
     par = parity_sample(c, smp, check_rows) if check_rows else device_report(smp)
     ab = algorithmic_bytes(c)
     return c, dict(workload=name, rows=c["rows"], vocab=c["V"], dtype=c["dtype"], ms_per_step=wall_ms, kernel_ms=kern_ms,
+                   kernel_ms_warm=warm_ms, logits_copies_rotated=n_rot,
                    rows_per_s=c["rows"] / (wall_ms * 1e-3), algorithmic_MB=ab / 1e6, achieved_GBs=ab / (kern_ms * 1e-3) / 1e9,
+                   achieved_GBs_warm=ab / (warm_ms * 1e-3) / 1e9,
                    frac_of_hbm_peak=ab / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, parity=par)
 
 
@@ -230,6 +261,15 @@ def reference_kernels(steps):
         x = torch.randn(rows, V, device="cuda:0") * 2
         o = torch.empty(rows, dtype=torch.int32, device="cuda:0")
         timed("argmax_rows", rows, lambda: L.ws_argmax_rows(S(), P(x), V, P(o), rows), rows * V * 4)
+        if rows == 256:  # the same with each launch on another copy of the rows (beyond the memory-side cache): HBM reads
+            xs = [x] + [x.clone() for _ in range(rotation_for(x.numel() * 4) - 1)]
+            turn = [0]
+
+            def cold():
+                turn[0] = (turn[0] + 1) % len(xs)
+                L.ws_argmax_rows(S(), P(xs[turn[0]]), V, P(o), rows)
+            timed("argmax_rows (cold: rotating copies)", rows, cold, rows * V * 4)
+            del xs
         if rows > 32:
             continue
         ids = torch.empty((rows, 16384), dtype=torch.int32, device="cuda:0")
@@ -418,7 +458,11 @@ def main():
                    "filters": "see whirl-llm_amd/workloads.py make_" + a.workload, "rng": "philox4x32-10", "sigma": 2,
                    "sweep_mode": a.mode, "kept_cap": a.kept_cap},
         "roofline": {"bound": "hbm", "achieved": ab / (main_res["kernel_ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": main_res["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
+                     "frac": main_res["frac_of_hbm_peak"], "achieved_warm": main_res["achieved_GBs_warm"],
+                     "frac_warm": main_res["achieved_GBs_warm"] / HBM_PEAK_GBS, "kernel_ms_warm": main_res["kernel_ms_warm"],
+                     "cold": f"each launch reads another of {main_res['logits_copies_rotated']} copies of the logits (together "
+                             "beyond the 256 MiB memory-side cache); *_warm: every launch on one resident copy",
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "ws::sample_batch_kernel", "kernel_source_digest": kernel_digest(),
                      "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},
         "cpu_baseline": cpu,
