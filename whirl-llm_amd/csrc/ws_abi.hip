@@ -6,6 +6,7 @@
 
 #include <atomic>
 
+#include <cstdlib>
 #include <cstring>
 
 #include "ws_accept.h"
@@ -25,6 +26,9 @@ int launch_split(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsign
 // ws_fused_kept.hip, ws_split_kept.hip: the builds of the two that can write the kept-set dump
 int launch_fused_kept(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
 int launch_split_kept(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
+// ws_lean.hip: the lean single-sweep kernel (1024 threads a row) for batches of unsplit fp32 rows
+int launch_lean(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
+int prepare_lean(unsigned lds_limit);
 }  // namespace ws
 
 namespace {
@@ -39,6 +43,12 @@ constexpr uint32_t kStaticLds = 4096u + 512u;  // + the phase marks
 #else
 constexpr uint32_t kStaticLds = 4096u;
 #endif
+// the lean kernel's own tables and those of the three-pass code it calls
+#ifdef WS_PHASE_TIMERS
+constexpr uint32_t kStaticLean = 9216u + 512u + 1536u;
+#else
+constexpr uint32_t kStaticLean = 9216u + 512u;
+#endif
 
 struct BatchPlan {
     uint32_t patch_cap;
@@ -47,6 +57,10 @@ struct BatchPlan {
     uint32_t lds_tie;
     uint32_t lds_total;
     bool fused;
+    bool lean;            // the lean kernel can take the batch when its rows are not split (fp32, no optional outputs)
+    uint32_t lean_tie;    // its second histogram copy (0: none), its dynamic LDS, and the spare LDS of the three-pass code it calls
+    uint32_t lean_total;
+    uint32_t lean_fb_tie;
     uint32_t split_log2;  // the most parts per row that pay for this batch
     uint64_t workspace_min;  // split rows: the least that lets them split (no staging areas), 0 when nothing is split
     uint64_t workspace;   // bytes for that
@@ -115,6 +129,27 @@ BatchPlan plan_batch(const ws_batch* b) {
     p.patch_cap = static_cast<uint32_t>(cap ? cap : 1);
     p.lds_ab = static_cast<uint32_t>(ab);
     p.lds_total = static_cast<uint32_t>(total);
+    // The lean kernel shares the single-sweep layout (its static LDS is larger, so the second histogram copy fits less
+    // often); the three-pass code it hands rows back to lays its tables over the same allocation.
+#ifdef WS_PHASE_TIMERS
+    const bool wants_entropy = false;  // (debug builds: `entropy` takes the lean kernel's phase marks, 16 doubles a row)
+#else
+    const bool wants_entropy = b->entropy != nullptr;
+#endif
+    static const bool lean_on = std::getenv("WS_LEAN") != nullptr;  // (while the lean kernel is being brought up)
+    p.lean = lean_on && p.fused && b->mode == WS_MODE_AUTO && b->dtype == WS_DTYPE_F32 && !b->kept_ids && !b->query_prob && !wants_entropy && !b->race &&
+             fused_total + kStaticLean <= kMaxLds;
+    if (p.lean) {
+        uint64_t lt = fused_total;
+        p.lean_tie = 0;
+        if (lt + 32768u + kStaticLean <= kMaxLds) {
+            p.lean_tie = static_cast<uint32_t>((lt + 15u) & ~uint64_t{15});
+            lt = p.lean_tie + 32768u;
+        }
+        p.lean_total = static_cast<uint32_t>(lt);
+        const uint64_t three = 65536u + maps;
+        p.lean_fb_tie = three + spare_bytes <= lt ? static_cast<uint32_t>((three + 15u) & ~uint64_t{15}) : 0u;
+    }
     // Small batches of the single-sweep kernel: with rows to spare on the compute units a row is split over 2, 4, 8 or
     // 16 workgroups (each at least 16384 tokens; 8192 for the step from 8 to 16, which a lone 151936-token row still wins: 29.2 -> 28.0 us), which meet in global memory. All parts of all rows have to be running
     // at the same time - they wait for each other - so rows * parts stays within the compute units of the device.
@@ -441,6 +476,11 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     a.entropy = b->entropy;
     if (p.fused && a.split_log2)
         return (a.kept_ids ? ws::launch_split_kept : ws::launch_split)(S(stream), a, b->rows << a.split_log2, p.lds_total, kMaxLds - kStaticLds);
+    if (p.lean) {
+        a.lds_tie = p.lean_tie;
+        a.fb_lds_tie = p.lean_fb_tie;
+        return ws::launch_lean(S(stream), a, b->rows, p.lean_total, kMaxLds - kStaticLean);
+    }
     if (p.fused) return (a.kept_ids ? ws::launch_fused_kept : ws::launch_fused)(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);
     static std::atomic<uint64_t> attr_set{0};  // the dynamic LDS limit is raised per function and device, once per process
     int dev = 0;

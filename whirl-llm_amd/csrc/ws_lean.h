@@ -1,0 +1,1050 @@
+// The lean single-sweep sampler for gfx950: one workgroup of 1024 threads (sixteen wave64s, four per SIMD) per row,
+// for batches with at least one row per compute unit. It answers the rows most requests are made of - fp32 logits in
+// whole 128-bit vectors, a closed filter without a top-k (top-p and / or min-p), the inverse-CDF draw - and hands every
+// other row (and every row on which one of its own checks fails) to the three-pass code of ws_sample.h inside the same
+// launch. Results are those of ws_sample.h's single-sweep kernel: the same bins, the same histogram words, the same
+// decision rules (src/sampling/sampler.cpp:15-78, :118-131) and margins.
+//
+// What is different from that kernel, and why:
+//   * every token's bin is remembered as its low 8 bits, four tokens per register (40 registers instead of 160): a scan
+//     for the tokens of a few bins tests four tokens with three instructions per bin; a token of another bin with the same
+//     low bits is found as well and dropped when its logit has been read again. The registers this frees let the first
+//     two batches of the row travel while phase 0 builds its tables, and four waves per SIMD hide the tail's latencies.
+//   * the histogram is scanned four consecutive bins per thread, the cuts' and the draw's bins are found by all threads
+//     at once (every thread tests the bins it has just scanned), and the candidates' exact order is settled by all of
+//     them at once as well: a candidate adds its fixed-point mass to one of 64 buckets per range, finds its rank and its
+//     running mass among the few members of its bucket, and tests the cut and the draw on itself.
+#pragma once
+
+#include "ws_sample.h"
+
+#ifndef WS_EXP_ORDER
+#define WS_EXP_ORDER 0
+#endif
+
+namespace ws {
+
+constexpr int kLeanRegs = 40;   // bin-cache registers per thread: 160 tokens, rows of up to 163840 tokens
+constexpr int kLeanBatch = 2;   // 128-bit loads per thread and batch
+constexpr uint32_t kLeanPlaces = 32u, kLeanBuckets = 128u, kLeanMaxRange = 800u;
+constexpr uint32_t kRouteHandedBack = 0x100u;  // WS_FLAG_ROUTE_THREE_PASS
+
+#ifdef WS_PHASE_TIMERS
+#define WSL_MARK(k)                                                \
+    do {                                                           \
+        if (threadIdx.x == 0) S.marks[(k)] = clock64() - wsl_t0;   \
+    } while (0)
+#else
+#define WSL_MARK(k) \
+    do {            \
+    } while (0)
+#endif
+
+// bit 7 of every byte of y that equals the byte c4 repeats (and, possibly, of a byte above such a byte: a token found that
+// way is dropped when its logit has been read again)
+__device__ __forceinline__ uint32_t bytes_equal(uint32_t y, uint32_t c4) {
+    const uint32_t x = y ^ c4;
+    return (x - 0x01010101u) & ~x;
+}
+
+template <int NT>
+__device__ __forceinline__ uint32_t lean_flags(uint32_t y, const uint32_t (&c4)[4]) {
+    uint32_t f = bytes_equal(y, c4[0]);
+    if (NT > 1) f |= bytes_equal(y, c4[1]);
+    if (NT > 2) f |= bytes_equal(y, c4[2]);
+    if (NT > 3) f |= bytes_equal(y, c4[3]);
+    return f;
+}
+
+// What a thread's scan of its bin cache found: per group of 8 registers (32 tokens) the first two tokens whose cached byte
+// equals one of the bytes asked for, with their logits requested right there (the loads travel while the scan goes on).
+constexpr int kLeanGroups = kLeanRegs / 8;
+struct LeanHits {
+    uint32_t idx[2 * kLeanGroups];   // token index, 0xffffffff = none
+    uint32_t bits[2 * kLeanGroups];  // its logit as loaded
+};
+
+// A third token of a group and beyond goes to list[] as (token | kListNeedsLoad, 0), one LDS atomic each (rare). With
+// TO_LIST every find goes there (a second round of bytes). n_full: cache registers that hold a vector of the row in every
+// thread; register n_full holds one in threads below rem.
+template <int NT, bool TO_LIST>
+__device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const uint32_t* __restrict__ xg, uint32_t n_full,
+                                          uint32_t rem, LeanHits& H, uint2* list, uint32_t* n_list, uint32_t cap) {
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (int g = 0; g < kLeanGroups; ++g) {
+        uint32_t acc = 0;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const uint32_t c = static_cast<uint32_t>(g * 8 + r);
+            if (c > n_full) continue;  // uniform: a register past the row
+            uint32_t mask = 0x01010101u << r;
+            if (c == n_full && t >= rem) mask = 0u;
+            acc = ((lean_flags<NT>(cache[c], c4) >> (7 - r)) & mask) | acc;  // bit 8 e + r: token e of register r
+        }
+        auto token_of = [&](uint32_t bit) { return ((static_cast<uint32_t>(g * 8 + (bit & 7u)) * WS_BLOCK + t) << 2) + (bit >> 3); };
+        if (!TO_LIST) {
+            H.idx[g] = H.idx[kLeanGroups + g] = 0xffffffffu;
+            H.bits[g] = H.bits[kLeanGroups + g] = 0u;
+            if (acc) {
+                const uint32_t i = token_of(static_cast<uint32_t>(__ffs(acc)) - 1u);
+                acc &= acc - 1u;
+                H.idx[g] = i;
+                H.bits[g] = xg[i];
+            }
+            if (acc) {
+                const uint32_t i = token_of(static_cast<uint32_t>(__ffs(acc)) - 1u);
+                acc &= acc - 1u;
+                H.idx[kLeanGroups + g] = i;
+                H.bits[kLeanGroups + g] = xg[i];
+            }
+        }
+        while (acc) {
+            const uint32_t i = token_of(static_cast<uint32_t>(__ffs(acc)) - 1u);
+            acc &= acc - 1u;
+            const uint32_t slot = atomicAdd(n_list, 1u);
+            if (slot < cap) list[slot] = make_uint2(i | kListNeedsLoad, 0u);
+        }
+    }
+}
+
+// exp(-a) for 0 <= a < 63 from the tables exp(-b / 64) (s_exp: kExpHi, then kExpLo) and a polynomial on the remaining
+// [0, 1/64): a few units in the last place, a fifth of the instructions of the library's exp
+__device__ __forceinline__ double exp_neg(double a, const double* s_exp) {
+    const double t64 = a * 64.0;
+    if (!(t64 >= 0.0 && t64 < 4032.0)) return exp(-a);
+    const uint32_t n = static_cast<uint32_t>(t64);
+    const double r = a - static_cast<double>(n) * (1.0 / 64.0);
+    double p = 1.0 / 720.0;
+    p = fma(p, -r, 1.0 / 120.0);
+    p = fma(p, -r, 1.0 / 24.0);
+    p = fma(p, -r, 1.0 / 6.0);
+    p = fma(p, -r, 0.5);
+    p = fma(p, -r, 1.0);
+    p = fma(p, -r, 1.0);
+    return s_exp[n >> 6] * s_exp[64u + (n & 63u)] * p;
+}
+
+// what wave 0 works out from the scanned histogram for everybody
+struct LeanSel {
+    double X, Z, m0base, m1base, scale0, scale1, inv0, inv1;
+    int r0lo, r0hi, r1lo, r1hi;
+    uint32_t c0base, n_r0, c1base, n_r1;
+    uint32_t topp_in_list, minp_in_list, ok, pad;
+};
+
+// the lean path's static LDS, declared once by the kernel
+struct LeanShared {
+    double s_exp[128];  // kExpHi, kExpLo
+    double pm64[64];    // pm[64 i + 64]
+    double red_d[WS_WAVES];
+    double s_d[8];
+    LeanSel sel;
+    unsigned long long s_q[6];
+    unsigned long long b_mass[kLeanBuckets], b_fpre[kLeanBuckets];
+    uint32_t b_cnt[kLeanBuckets], b_cpre[kLeanBuckets];
+    uint32_t pc64[64];  // pc[64 i + 64]
+    uint32_t s_w[16];
+    uint32_t red_u[WS_WAVES];
+    float red_f[WS_WAVES];
+#ifdef WS_PHASE_TIMERS
+    long long marks[16];
+#endif
+};
+
+// One row. Returns false when the row is left to the three-pass code (nothing has been written for it then).
+template <bool MASKED>
+__device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row, LeanShared& S) {
+#ifdef WS_PHASE_TIMERS
+    const long long wsl_t0 = clock64();  // debug builds: the marks go to LDS, and at the end to `entropy`, 16 doubles a row
+    if (threadIdx.x < 16) S.marks[threadIdx.x] = 0;
+#endif
+    extern __shared__ __align__(16) unsigned char lds[];
+    float* red_f = S.red_f;
+    uint32_t* red_u = S.red_u;
+    double* red_d = S.red_d;
+    double* s_exp = S.s_exp;
+    double* pm64 = S.pm64;
+    uint32_t* pc64 = S.pc64;
+    uint32_t* s_w = S.s_w;
+    unsigned long long* s_q = S.s_q;
+    double* s_d = S.s_d;
+    uint32_t* b_cnt = S.b_cnt;
+    uint32_t* b_cpre = S.b_cpre;
+    unsigned long long* b_mass = S.b_mass;
+    unsigned long long* b_fpre = S.b_fpre;
+
+    const uint32_t t = threadIdx.x, lane = t & 63u;
+    const uint32_t wv = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(t >> 6)));
+    const uint32_t V = A.vocab;
+    const uint32_t nW = (V + 31u) >> 5;
+
+    RowView rv;
+    rv.V = V;
+    rv.dtype = 0;
+    rv.base = static_cast<const unsigned char*>(A.logits) + static_cast<size_t>(row) * A.row_stride * 4u;
+    rv.vec = true;
+    rv.allow = MASKED ? A.allow + static_cast<size_t>(row) * A.allow_stride : nullptr;
+    rv.touched = nullptr;
+    const uint32_t nv = V >> 2;
+    const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
+    // Batches 0 .. kPre - 1 have registers of their own and are all asked for before phase 0 - the bin cache is not live
+    // yet, so there is room - which puts a third of the row on its way while the tables are built; from batch kPre on
+    // the first three of those slots are a ring, two batches in flight while one is consumed.
+    constexpr int kPre = 6, kRing = 3;
+    uint4 q[kPre][kLeanBatch];
+    uint32_t na[kPre][kLeanBatch];
+    auto load = [&](int bt, int slot) {
+#pragma unroll
+        for (int u = 0; u < kLeanBatch; ++u) {
+            const uint32_t j = (bt * kLeanBatch + u) * WS_BLOCK + t;
+            const uint32_t jc = j < nv ? j : nv - 1u;
+            q[slot][u] = xv[jc];
+            na[slot][u] = MASKED ? rv.allow[(jc * 4u) >> 5] : 0xffffffffu;  // (complemented where it is used: nothing waits for the load here)
+        }
+    };
+
+#if WS_EXP_ORDER == 2
+    load(0, 0);
+    load(1, 1);
+#endif
+    uint64_t* hist = reinterpret_cast<uint64_t*>(lds);
+    uint4* stage = reinterpret_cast<uint4*>(lds + 32768);
+    uint32_t* touched = reinterpret_cast<uint32_t*>(lds + A.lds_ab);
+    uint16_t* wprefix = reinterpret_cast<uint16_t*>(lds + A.lds_ab + nW * 4u);
+    float* pv = reinterpret_cast<float*>(lds + A.lds_ab + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    uint32_t* cnt = reinterpret_cast<uint32_t*>(lds + A.lds_cnt);
+    uint32_t* first = cnt + A.patch_cap;
+    uint64_t* hist2 = A.lds_tie ? reinterpret_cast<uint64_t*>(lds + A.lds_tie) : nullptr;
+    rv.wprefix = wprefix;
+    rv.pv = pv;
+
+    const float inv_t = A.inv_t[row];
+    const uint32_t top_k = A.top_k ? A.top_k[row] : 0u;
+    const double top_p = A.top_p ? A.top_p[row] : 1.0;
+    const double min_p = A.min_p ? A.min_p[row] : 0.0;
+    const double tol = A.tol;
+    const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
+    const bool race = A.race != nullptr && A.race[row] != 0;
+    const bool use_top_p = top_p < 1.0, use_min_p = min_p > 0.0;
+    const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? (A.hist_len ? A.hist_len[row] : A.hist_off[row + 1] - h0) : 0u;
+    const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
+    // rows this code does not take: a top-k, no filter at all, the race draw, parameters the three-pass code reports
+    if (top_k != 0u || !(use_top_p || use_min_p) || race || !(inv_t > 0.f) || nh + nb > A.patch_cap) return false;
+
+    const int32_t* hist_ids = A.hist + h0;
+    const int32_t* bias_ids = A.bias_ids + b0;
+    const float* bias_vals = A.bias_vals + b0;
+    constexpr int kHid = 4;
+    uint32_t hid[kHid];
+#pragma unroll
+    for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
+    const uint32_t bid = t < nb ? static_cast<uint32_t>(bias_ids[t]) : 0xffffffffu;  // the first bias ids
+    const double exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);
+    // The row's first kPre batches are asked for behind the history ids, not before them: with every compute unit streaming,
+    // a request waits for all that is queued before it - microseconds - and phase 0 cannot start without the ids.
+    // (unconditional, addresses clamped to the row: a load behind a branch makes the compiler wait for every load before it)
+    // Every wave's ids are on their way before any wave asks for the row: the compute unit serves its waves' requests in
+    // the order they were made, and phase 0 needs all sixteen waves' ids. (A bare barrier: it waits for no memory.)
+#if WS_EXP_ORDER == 1
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the ids are here before the row is asked for
+#else
+    __builtin_amdgcn_s_barrier();
+#endif
+#pragma unroll
+    for (int bt = WS_EXP_ORDER == 2 ? 2 : 0; bt < kPre; ++bt) load(bt, bt);
+    if (wv == WS_WAVES - 1u) {  // one wave draws the row's uniform for everybody
+        const double u_ = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
+        if (lane == 0u) s_d[6] = u_;
+    }
+    WSL_MARK(0);
+
+    // ------------------------------------------------------------------ phase 0 (ws_sample.h): bitmap of the touched ids,
+    // popcount prefix per word (rank of a touched id), per-rank history count and bias entries
+    for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+    if (hist2)
+        for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
+    if (t < 128) s_exp[t] = exp_tab;
+    uint32_t n_touched = 0;
+    if (nh + nb > 0) {
+        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
+        for (uint32_t r = t; r < nh + nb; r += WS_BLOCK) {  // (at most nh + nb distinct ids)
+            cnt[r] = 0u;
+            first[r] = 0xffffffffu;
+        }
+        WSL_MARK(11);
+        __syncthreads();
+        WSL_MARK(12);
+#pragma unroll
+        for (int k = 0; k < kHid; ++k)
+            if (hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
+        for (uint32_t j = t + kHid * WS_BLOCK; j < nh; j += WS_BLOCK) {
+            const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
+            if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
+        }
+        if (bid < V) atomicOr(&touched[bid >> 5], 1u << (bid & 31u));
+        for (uint32_t j = t + WS_BLOCK; j < nb; j += WS_BLOCK) {
+            const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
+            if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
+        }
+        __syncthreads();
+        WSL_MARK(13);
+        constexpr uint32_t kChunk = 5;  // 163840 / 32 / 1024 words per thread
+        const uint32_t w0 = t * kChunk;
+        uint32_t wd[kChunk], local = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < kChunk; ++k) wd[k] = touched[min(w0 + k, nW - 1u)];
+#pragma unroll
+        for (uint32_t k = 0; k < kChunk; ++k) {
+            if (w0 + k >= nW) wd[k] = 0u;
+            local += __popc(wd[k]);
+        }
+        uint32_t n_uniq;
+        uint32_t run = block_excl_scan(local, red_u, &n_uniq);
+#pragma unroll
+        for (uint32_t k = 0; k < kChunk; ++k) {
+            if (w0 + k < nW) wprefix[w0 + k] = static_cast<uint16_t>(run);
+            run += __popc(wd[k]);
+        }
+        __syncthreads();
+        WSL_MARK(14);
+        rv.touched = touched;
+        const bool ids_now = nb == 0;  // without a bias list the second table takes the token id of each rank right away
+#pragma unroll
+        for (int k = 0; k < kHid; ++k)
+            if (hid[k] < V) {
+                const uint32_t r = rank_of(rv, hid[k]);
+                atomicAdd(&cnt[r], 1u);
+                if (ids_now) first[r] = hid[k];
+            }
+        for (uint32_t j = t + kHid * WS_BLOCK; j < nh; j += WS_BLOCK) {
+            const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
+            if (id < V) {
+                const uint32_t r = rank_of(rv, id);
+                atomicAdd(&cnt[r], 1u);
+                if (ids_now) first[r] = id;
+            }
+        }
+        for (uint32_t j = t; j < nb; j += WS_BLOCK) {
+            const uint32_t id = j == t ? bid : static_cast<uint32_t>(bias_ids[j]);
+            if (id < V) {
+                const uint32_t r = rank_of(rv, id);
+                atomicMin(&first[r], j);
+                atomicAdd(&cnt[r], 1u << 20);
+            }
+        }
+        n_touched = n_uniq;
+    }
+    WSL_MARK(1);
+
+    // ------------------------------------------------------------------ the anchor: the head of the row + 8 exponent units
+    const float c64 = inv_t * 64.f;
+    float anchor, aq;
+    {
+        float s = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < kLeanBatch; ++u) {
+            s = fmaxf(s, fmaxf(fmaxf(__uint_as_float(q[0][u].x), __uint_as_float(q[0][u].y)),
+                               fmaxf(__uint_as_float(q[0][u].z), __uint_as_float(q[0][u].w))));
+        }
+        s = block_max(s, red_f);  // its barriers also publish phase 0's tables and the zeroed histogram
+        anchor = s + 8.f / inv_t;
+        aq = anchor_product(anchor, c64);
+        if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
+    }
+
+    // ------------------------------------------------------------------ the sweep
+    uint32_t cache[kLeanRegs];
+    float m = -INFINITY;
+    {
+        constexpr int NB = kLeanRegs / kLeanBatch;
+        const float tail_f = own_tail();
+        uint64_t* myhist = (hist2 && (t & 1u)) ? hist2 : hist;
+        const bool any_touched = n_touched != 0u;  // uniform
+        const uint32_t stage_cap = 2047u;
+        const uint32_t n_full = nv / WS_BLOCK;  // vector rounds that are inside the row for every thread
+        // the bitmap words of a batch are read a batch ahead, before the batch in between adds to the histogram: LDS
+        // operations of a wave finish in order, and a read asked for behind the additions would wait for all of them
+        uint32_t tws[2][kLeanBatch], wps[2][kLeanBatch];
+        auto read_words = [&](int bt) {
+#pragma unroll
+            for (int u = 0; u < kLeanBatch; ++u) {
+                const uint32_t word = (((bt * kLeanBatch + u) * WS_BLOCK + t) * 4u) >> 5;  // (past the row: a word past the bitmap, inside the block's LDS)
+                tws[bt & 1][u] = any_touched ? touched[word] : 0u;
+                wps[bt & 1][u] = any_touched ? wprefix[word] : 0u;
+            }
+        };
+        read_words(0);
+#pragma unroll
+        for (int bt = 0; bt < NB; ++bt) {
+            const int slot = bt < kPre ? bt : bt % kRing;
+            if (static_cast<uint32_t>(bt * kLeanBatch) * WS_BLOCK >= nv) {  // uniform: the row is done
+#pragma unroll
+                for (int c = bt * kLeanBatch; c < kLeanRegs; ++c) cache[c] = 0u;
+                break;
+            }
+            if (bt + 1 < NB) read_words(bt + 1);
+#pragma unroll
+            for (int u = 0; u < kLeanBatch; ++u) {
+                const uint32_t j = (bt * kLeanBatch + u) * WS_BLOCK + t;
+                const int c = bt * kLeanBatch + u;
+                uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
+                uint32_t tw = tws[bt & 1][u], nal = MASKED ? ~na[slot][u] : 0u;
+                if (static_cast<uint32_t>(c) >= n_full && j >= nv) {  // (only the row's last round has lanes past it) NaN: the tail bins, nobody's candidate
+                    w[0] = w[1] = w[2] = w[3] = 0xffffffffu;
+                    tw = 0u;
+                }
+                const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * 4u) & 31u)) : 0;
+                uint32_t bins[4];
+                float vm = -INFINITY;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t bits = w[e];
+                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
+                    const float x = __uint_as_float(bits);
+                    vm = fmaxf(vm, x);
+                    const float tc = bin_coord(aq, c64, x, tail_f);
+                    bins[e] = static_cast<uint32_t>(tc);
+#ifndef WS_EXP_NOATOMIC
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&myhist[bins[e]]), bin_word(tc));
+#else
+                    m = fmaxf(m, __uint_as_float(static_cast<uint32_t>(bin_word(tc))));
+#endif
+                }
+                const uint32_t lo2 = __builtin_amdgcn_perm(bins[1], bins[0], 0x0c0c0400u);
+                cache[c] = __builtin_amdgcn_perm(bins[3], bins[2], 0x04000c0cu) | lo2;
+                const uint32_t sh = (j * 4u) & 31u;
+                const bool touched_vec = ((tw >> sh) & 15u) != 0u;
+                m = fmaxf(m, touched_vec ? -INFINITY : vm);  // (a vector with a touched token is looked at when that token is collected)
+                if (touched_vec) {
+                    const uint32_t r = wps[bt & 1][u] + __popc(tw & ((1u << sh) - 1u));
+                    stage[min(r, stage_cap)] = q[slot][u];
+                }
+            }
+            // the slot is free: the first three take batches kPre .. kPre + 2 right away, later ones the batch three ahead
+            constexpr int kNone = 1 << 20;
+            const int next = bt < kRing ? bt + kPre : (bt >= kPre ? bt + kRing : kNone);
+#ifndef WS_EXP_NOLOAD
+            if (next < NB) load(next, next % kRing);
+#endif
+        }
+    }
+    __syncthreads();
+    WSL_MARK(2);
+
+    // ------------------------------------------------------------------ the touched tokens (collect_fused of ws_sample.h):
+    // every history / bias entry claims its token's rank; the owner adjusts the token's logit and moves the token from the
+    // bin of its raw logit to the bin of the adjusted one
+    float ma = -INFINITY, mu = -INFINITY;
+    if (n_touched) {
+        constexpr uint32_t kClaim = 0x80000000u;
+        const uint32_t whole_end = V & ~3u;
+        const float tail_own = own_tail();
+        const uint32_t stage_cap = 2047u;
+        auto take4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {
+            for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
+                uint32_t id[4], al[4], tw[4], wp[4], rk[4], old[4];
+                uint4 vec[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t j = j0 + k * WS_BLOCK + t;
+                    id[k] = (in_regs && j0 == 0u) ? hid[k] : (j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu);
+                    if (id[k] >= V) id[k] = 0xffffffffu;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    al[k] = MASKED ? rv.allow[i >> 5] : 0xffffffffu;
+                    tw[k] = touched[i >> 5];
+                    wp[k] = wprefix[i >> 5];
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t i = id[k] < V ? id[k] : 0u;
+                    const uint32_t vb = i & ~3u;
+                    const uint32_t rf = id[k] < V ? wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u)) : 0u;
+                    rk[k] = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));
+                    old[k] = id[k] < V ? atomicOr(&cnt[rk[k]], kClaim) : kClaim;
+                    if (i < whole_end) {
+                        if (rf < stage_cap) vec[k] = stage[rf];
+                        else vec[k] = xv[i >> 2];
+                    } else {
+                        const uint32_t b = static_cast<const uint32_t*>(rv.base)[i];
+                        vec[k] = make_uint4(b, b, b, b);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (old[k] & kClaim) continue;
+                    const uint32_t i = id[k];
+                    const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
+                    const bool whole = i < whole_end;
+                    const uint32_t bits = whole ? w[i & 3u] : w[0];
+                    const float raw = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits), -INFINITY) : -INFINITY;
+                    if (whole) {
+                        const uint32_t free_bits = (al[k] & ~tw[k]) >> (i & 28u);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float(w[e]));
+                    }
+                    const uint32_t cw = old[k], c = cw & 0xfffffu, n_bias = (cw >> 20) & 0x7ffu;
+                    float x = raw;
+                    if (n_bias) {
+                        uint32_t j = first[rk[k]];
+                        x = __fadd_rn(x, bias_vals[j]);
+                        if (n_bias > 1u)
+                            for (++j; j < nb; ++j)
+                                if (static_cast<uint32_t>(bias_ids[j]) == i) x = __fadd_rn(x, bias_vals[j]);
+                    }
+                    if (c) {
+                        x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
+                        x = __fsub_rn(x, __fadd_rn(__fmul_rn(freq, static_cast<float>(c)), pres));
+                    }
+                    pv[rk[k]] = x;
+                    first[rk[k]] = i;  // the token id of the rank from here on
+                    ma = fmaxf(ma, x);
+                    const float t0 = bin_coord(aq, c64, raw, tail_own), t1 = bin_coord(aq, c64, x, tail_own);
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
+                }
+            }
+        };
+        take4(hist_ids, nh, true);
+        take4(bias_ids, nb, false);
+    }
+    WSL_MARK(3);
+    {
+        float m_all = fmaxf(fmaxf(m, mu), ma);
+        m = block_max(m_all, red_f);  // its barriers also end the moves in the histogram
+    }
+    if (!(m <= anchor && (anchor - m) * c64 <= 1024.f)) return false;  // (also a row without any token: m = -inf)
+
+    // ------------------------------------------------------------------ scan of the histogram: four consecutive bins a thread
+    const double lift = static_cast<double>(aq) * (1.0 / 64.0) - static_cast<double>(m) * static_cast<double>(inv_t);  // >= 0
+    if (wv == 0u) {  // one wave: the factor that takes masses from the anchor to the maximum
+        const double tm = exp(lift);
+        if (lane == 0u) s_d[7] = tm;
+    }
+    double* pm = reinterpret_cast<double*>(lds);                   // pm[b]: mass ranked before bin b; 4097 entries
+    uint32_t* pc = reinterpret_cast<uint32_t*>(lds + 32768 + 16);  // pc[b]: tokens ranked before bin b; 4097 entries
+    {
+        const uint32_t bb = 4u * t;
+        uint64_t h[4];
+        {
+            const ulonglong2 h01 = *reinterpret_cast<const ulonglong2*>(&hist[bb]), h23 = *reinterpret_cast<const ulonglong2*>(&hist[bb + 2u]);
+            h[0] = h01.x, h[1] = h01.y, h[2] = h23.x, h[3] = h23.y;
+            if (hist2) {
+                const ulonglong2 g01 = *reinterpret_cast<const ulonglong2*>(&hist2[bb]), g23 = *reinterpret_cast<const ulonglong2*>(&hist2[bb + 2u]);
+                h[0] += g01.x, h[1] += g01.y, h[2] += g23.x, h[3] += g23.y;
+            }
+        }
+        const double eh = s_exp[bb >> 6];
+        uint32_t c4b[4];
+        double ms[4];
+        uint32_t lc = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t b = bb + k;
+            c4b[k] = b < static_cast<uint32_t>(kTail) ? static_cast<uint32_t>(h[k] >> kCountShift) : 0u;  // (the tail's words are not looked at one by one)
+            const double fix = static_cast<double>(h[k] & ((1ull << kCountShift) - 1ull)) * kFixInv;
+            ms[k] = c4b[k] ? eh * s_exp[64 + (b & 63u)] * (static_cast<double>(c4b[k]) - fix) : 0.0;
+            lc += c4b[k];
+        }
+        const uint32_t ic = wave_incl_scan(lc);
+        __syncthreads();  // every read of the histogram is done: the prefixes go over it; the factor is in place
+        const double to_max = s_d[7];
+        double lm = 0.0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ms[k] *= to_max;
+            lm += ms[k];
+        }
+        const double im = wave_incl_scan(lm);
+        const double up = __shfl_up(im, 1);
+        if (lane == 63u) {
+            red_u[wv] = ic;
+            red_d[wv] = im;
+        }
+        __syncthreads();
+        uint32_t base_c = 0;
+        double base_m = 0.0, all_m = 0.0;
+#pragma unroll
+        for (uint32_t w = 0; w < WS_WAVES; ++w) {
+            const uint32_t sc = red_u[w];
+            const double sm = red_d[w];
+            if (w < wv) {
+                base_c += sc;
+                base_m += sm;
+            }
+            all_m += sm;
+        }
+        uint32_t rc = base_c + ic - lc;
+        double rm = base_m + (lane ? up : 0.0);
+        uint32_t ce[4];
+        double me[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ce[k] = rc;
+            me[k] = rm;
+            rc += c4b[k];
+            rm += ms[k];
+        }
+        *reinterpret_cast<uint4*>(&pc[bb]) = make_uint4(ce[0], ce[1], ce[2], ce[3]);  // (pc is 16 bytes into its region: aligned)
+        *reinterpret_cast<double2*>(&pm[bb]) = make_double2(me[0], me[1]);
+        *reinterpret_cast<double2*>(&pm[bb + 2u]) = make_double2(me[2], me[3]);
+        if ((t & 15u) == 15u) {
+            pc64[t >> 4] = t == WS_BLOCK - 1u ? V : rc;
+            pm64[t >> 4] = t == WS_BLOCK - 1u ? all_m : rm;
+        }
+        if (t == WS_BLOCK - 1u) {
+            pc[kBins] = V;  // every token of the row is in some bin: the tail holds what the others do not
+            pm[kBins] = all_m;
+        }
+    }
+    __syncthreads();
+    WSL_MARK(4);
+
+    // ------------------------------------------------------------------ select (the rules of ws_sample.h): the bins the cut
+    // and the draw can fall in, by wave 0 for everybody
+    if (wv == 0u) {
+        const double to_max = s_d[7];
+        const double Z = pm[kBins];
+        const double Zf = static_cast<double>(static_cast<float>(Z));  // Sampler::sum is a float (src/sampling/sampler.h:38)
+        auto first_bin = [&](auto&& reached_end, auto&& reached) {
+            const uint64_t coarse = __ballot(reached_end(static_cast<int>(lane)));
+            if (!coarse) return static_cast<int>(kBins);
+            const int base = 64 * (__ffsll(static_cast<unsigned long long>(coarse)) - 1);
+            const uint64_t fine = __ballot(reached(base + static_cast<int>(lane)));
+            return base + (__ffsll(static_cast<unsigned long long>(fine)) - 1);
+        };
+        auto find_mass = [&](double X, bool strict) {
+            if (!strict && !(X > 0.0)) return -1;
+            int b = strict ? first_bin([&](int i) { return pm64[i] > X; }, [&](int k) { return pm[k + 1] > X; })
+                           : first_bin([&](int i) { return pm64[i] >= X; }, [&](int k) { return pm[k + 1] >= X; });
+            while (b < kBins && pc[b + 1] == pc[b]) ++b;
+            return b < kBins ? b : -1;
+        };
+        int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
+        bool minp_in_list = false, topp_in_list = false;
+        double X = 0;
+        const double u = s_d[6];
+        int b2 = -1, lo3 = kBins, hi3 = -1;
+        if (use_top_p) {
+            X = top_p * Zf;
+            b2 = find_mass(X, false);
+            if (b2 >= 0 && pc[b2] >= 16384u) {
+                X = top_p * Z;
+                b2 = find_mass(X, false);
+            }
+            if (b2 < 0) b2 = kTail;
+        }
+        if (use_min_p) {
+            const double astar = (-log(min_p) + lift) * 64.0;
+            const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
+            lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
+            hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
+        }
+        if (use_top_p && (!use_min_p || b2 < lo3)) {
+            r1lo = r1hi = b2;
+            topp_in_list = true;
+        } else if (use_min_p && (!use_top_p || hi3 < b2)) {
+            r1lo = lo3;
+            r1hi = hi3;
+            minp_in_list = true;
+        } else if (use_top_p && use_min_p) {
+            r1lo = min(b2, lo3);
+            r1hi = max(b2, hi3);
+            minp_in_list = topp_in_list = true;
+        }
+        double zlo, zhi;
+        if (r1hi >= r1lo) {
+            zlo = pm[r1lo];
+            zhi = pm[r1hi + 1];
+            if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);
+        } else {
+            zlo = zhi = Z;
+        }
+        int b4lo = find_mass(u * zlo * (1.0 - 1e-9), true), b4hi = find_mass(u * zhi * (1.0 + 1e-9), true);
+        if (b4lo < 0) b4lo = 0;
+        if (b4hi < 0) b4hi = (r1hi >= r1lo) ? r1hi : kTail - 1;
+        if (b4hi < b4lo) b4hi = b4lo;
+        if (r1hi >= r1lo && b4hi >= r1lo - 1) {
+            r0lo = min(b4lo, r1lo);
+            r0hi = max(b4hi, r1hi);
+            r1lo = 0;
+            r1hi = -1;
+        } else {
+            r0lo = b4lo;
+            r0hi = b4hi;
+        }
+        const bool has_r1 = r1hi >= r1lo;
+        bool ok = !(r0hi >= kTail || r1hi >= kTail);  // the tail has no mass resolution
+        const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+        ok = ok && nb0 + nb1 <= 8u;
+        LeanSel sel;
+        sel.X = X;
+        sel.Z = Z;
+        sel.r0lo = r0lo, sel.r0hi = r0hi, sel.r1lo = r1lo, sel.r1hi = r1hi;
+        sel.c0base = ok ? pc[r0lo] : 0u;
+        sel.n_r0 = ok ? pc[r0hi + 1] - sel.c0base : 0u;
+        sel.m0base = ok ? pm[r0lo] : 0.0;
+        sel.c1base = ok && has_r1 ? pc[r1lo] : 0u;
+        sel.n_r1 = ok && has_r1 ? pc[r1hi + 1] - sel.c1base : 0u;
+        sel.m1base = ok && has_r1 ? pm[r1lo] : 0.0;
+        ok = ok && sel.n_r0 + sel.n_r1 != 0u && sel.n_r0 <= kLeanMaxRange && sel.n_r1 <= kLeanMaxRange;
+        // masses of a range in units of 2^-52 of the largest mass a token of the range can have
+        auto edge_mass = [&](int b) { return s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001; };
+        const double emax0 = edge_mass(ok ? r0lo : 0), emax1 = ok && has_r1 ? edge_mass(r1lo) : 1.0;
+        sel.scale0 = 4503599627370496.0 / emax0, sel.scale1 = 4503599627370496.0 / emax1;
+        sel.inv0 = emax0 * (1.0 / 4503599627370496.0), sel.inv1 = emax1 * (1.0 / 4503599627370496.0);
+        sel.topp_in_list = topp_in_list, sel.minp_in_list = minp_in_list, sel.ok = ok, sel.pad = 0u;
+        if (lane == 0u) {
+            S.sel = sel;
+            s_w[0] = 0u;
+            s_w[5] = 0u;
+        }
+    }
+    __syncthreads();  // the last reads of pm / pc are done: their LDS is the candidate list from here
+    WSL_MARK(5);
+    if (!S.sel.ok) return false;
+    const int r0lo = S.sel.r0lo, r0hi = S.sel.r0hi, r1lo = S.sel.r1lo, r1hi = S.sel.r1hi;
+    const bool has_r1 = r1hi >= r1lo;
+    const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+    const uint32_t c0base = S.sel.c0base, n_r0 = S.sel.n_r0, c1base = S.sel.c1base, n_r1 = S.sel.n_r1;
+    const uint32_t n_list = n_r0 + n_r1;
+    const bool topp_in_list = S.sel.topp_in_list != 0u, minp_in_list = S.sel.minp_in_list != 0u;
+
+    // ------------------------------------------------------------------ the tokens of those bins
+    uint2* list = reinterpret_cast<uint2*>(lds + 32768);
+    constexpr uint32_t kListCap = 4096u;
+    const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = nb0 - 1u;
+    const uint32_t u1r = has_r1 ? static_cast<uint32_t>(r1lo) : 0xffff0000u, w1 = has_r1 ? nb1 - 1u : 0u;
+    auto in_ranges = [&](float x) {
+        const uint32_t b = bin_of(aq, c64, x);
+        return b - u0 <= w0 || b - u1r <= w1;
+    };
+    {
+        LeanHits H;
+        const uint32_t* xg = static_cast<const uint32_t*>(rv.base);
+        const uint32_t n_full = nv / WS_BLOCK, rem = nv % WS_BLOCK;
+        uint32_t bins[8];
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; ++k) bins[k] = k < nb0 ? u0 + k : (k < nb0 + nb1 ? static_cast<uint32_t>(r1lo) + (k - nb0) : u0);
+        const uint32_t nt = nb0 + nb1;
+        {
+            uint32_t c4[4];
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[k] & 0xffu) * 0x01010101u;
+            const uint32_t n = min(4u, nt);
+            if (n == 1u) lean_scan<1, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+            else lean_scan<4, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+        }
+        if (nt > 4u) {  // uniform, rare: a second round for the other bytes, every find through the list
+            uint32_t c4[4];
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[4u + k] & 0xffu) * 0x01010101u;
+            lean_scan<4, true>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+        }
+        // touched tokens whose adjusted logit lies in the ranges
+        for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
+            const float x = pv[r];
+            if (in_ranges(x)) {
+                const uint32_t slot = atomicAdd(&s_w[0], 1u);
+                if (slot < kListCap) list[slot] = make_uint2(first[r] | kListAdjusted, __float_as_uint(x));
+            }
+        }
+        uint32_t mine = 0;
+#pragma unroll
+        for (int k = 0; k < 2 * kLeanGroups; ++k) mine += H.idx[k] != 0xffffffffu ? 1u : 0u;
+        const uint32_t inc = wave_incl_scan(mine);
+        uint32_t base = 0;
+        if (lane == 63u && inc) base = atomicAdd(&s_w[0], inc);
+        uint32_t slot = __shfl(base, 63) + inc - mine;
+#pragma unroll
+        for (int k = 0; k < 2 * kLeanGroups; ++k) {
+            if (H.idx[k] == 0xffffffffu) continue;
+            if (slot < kListCap) list[slot] = make_uint2(H.idx[k], H.bits[k]);
+            ++slot;
+        }
+    }
+    __syncthreads();
+    WSL_MARK(6);
+    const uint32_t n_hit = s_w[0];
+    if (n_hit > kListCap) return false;
+
+    // ------------------------------------------------------------------ the finds that are candidates: a token of another
+    // bin with the same low bits, a masked-out token and a touched token found by its raw logit are dropped
+    uint2* cand = reinterpret_cast<uint2*>(lds);  // (token, logit bits), kLeanMaxRange * 2 entries at most
+    {
+        constexpr int kR = 4;
+        uint2 en[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t k = r * WS_BLOCK + t;
+            en[r] = k < n_hit ? list[k] : make_uint2(0xffffffffu, 0u);
+        }
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            if (static_cast<uint32_t>(r) * WS_BLOCK >= n_hit) continue;  // uniform
+            const bool live = en[r].x != 0xffffffffu;
+            const uint32_t id = live ? en[r].x & kListIdMask : 0u;
+            float x = __uint_as_float(en[r].y);
+            bool ok = live;
+            if (!(en[r].x & kListAdjusted)) {
+                if (en[r].x & kListNeedsLoad) x = __uint_as_float(static_cast<const uint32_t*>(rv.base)[id]);
+                x = fmaxf(x, -INFINITY);
+                ok = ok && (!MASKED || is_allowed(rv, id)) && !is_touched(rv, id) && in_ranges(x);
+            }
+            const uint64_t mk = __ballot(ok);
+            uint32_t base = 0;
+            if (lane == 0u && mk) base = atomicAdd(&s_w[5], static_cast<uint32_t>(__popcll(mk)));
+            const uint32_t slot = __shfl(base, 0) + static_cast<uint32_t>(__popcll(mk & ((1ull << lane) - 1ull)));
+            if (ok && slot < 2u * kLeanMaxRange) cand[slot] = make_uint2(id, __float_as_uint(x));
+        }
+    }
+    if (t < kLeanBuckets) {
+        b_cnt[t] = 0u;
+        b_mass[t] = 0ull;
+    }
+    if (t == 0) {
+        s_q[0] = ~0ull;  // smallest mass at or above the min-p floor
+        s_q[1] = 0ull;   // largest mass below it
+        s_q[2] = ~0ull;  // the cut: (rank in the row << 32) | slot
+        s_q[3] = ~0ull;  // the draw
+        s_w[1] = 0u;     // candidates at or above the floor
+        s_w[2] = 0u;     // a bucket ran out of places
+        s_w[3] = 0u;     // the last kept candidate was found
+    }
+    __syncthreads();
+    WSL_MARK(7);
+    if (s_w[5] != n_list) return false;  // the histogram and the gather disagree
+    constexpr int kRounds = 2;  // n_list <= 2 kLeanMaxRange <= 2 WS_BLOCK
+    uint32_t cid[kRounds];
+    float cx[kRounds];
+    bool con[kRounds];
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        const uint32_t k = r * WS_BLOCK + t;
+        const uint2 en = k < n_list ? cand[k] : make_uint2(0u, 0u);
+        cid[r] = en.x;
+        cx[r] = __uint_as_float(en.y);
+        con[r] = k < n_list;
+    }
+    __syncthreads();  // every thread has its candidates: the LDS takes the buckets
+    struct Place {
+        uint64_t key, fx;
+    };
+    Place* lb = reinterpret_cast<Place*>(lds);  // [bucket][place]: a candidate's key and its fixed-point mass
+    const double X = S.sel.X, Z = S.sel.Z, m0base = S.sel.m0base, m1base = S.sel.m1base;
+    const double scale0 = S.sel.scale0, scale1 = S.sel.scale1, inv0 = S.sel.inv0, inv1 = S.sel.inv1;
+    const float step0 = 64.f / static_cast<float>(nb0), step1 = has_r1 ? 64.f / static_cast<float>(nb1) : 0.f;
+    const float lo0 = static_cast<float>(r0lo), lo1 = static_cast<float>(r1lo);
+    uint32_t cbkt[kRounds];
+    uint64_t cfix[kRounds], ckey[kRounds];
+    double cem[kRounds];
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        if (static_cast<uint32_t>(r) * WS_BLOCK >= n_list) continue;  // uniform
+        const float x = cx[r];
+        const float tc = bin_coord(aq, c64, x);
+        const bool in1 = has_r1 && static_cast<uint32_t>(tc) - static_cast<uint32_t>(r1lo) < nb1;
+        const float rel = fmaxf(__fmul_rn(__fsub_rn(tc, in1 ? lo1 : lo0), in1 ? step1 : step0), 0.f);
+        cbkt[r] = (in1 ? 64u : 0u) + min(63u, static_cast<uint32_t>(rel));
+        cem[r] = exp_neg(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t), s_exp);
+        cfix[r] = static_cast<uint64_t>(__double2ull_rn(cem[r] * (in1 ? scale1 : scale0)));
+        ckey[r] = key64(x, cid[r]);
+        if (con[r]) {
+            const uint32_t place = atomicAdd(&b_cnt[cbkt[r]], 1u);
+            atomicAdd(&b_mass[cbkt[r]], static_cast<unsigned long long>(cfix[r]));
+            if (place < kLeanPlaces) lb[cbkt[r] * kLeanPlaces + place] = Place{ckey[r], cfix[r]};
+            else s_w[2] = 1u;
+        }
+        if (use_min_p && minp_in_list) {  // uniform
+            const bool pass = con[r] && cem[r] >= min_p;
+            const uint64_t np = __ballot(pass);
+            if (lane == 0u && np) atomicAdd(&s_w[1], static_cast<uint32_t>(__popcll(np)));
+            if (pass) atomicMin(&s_q[0], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
+            if (con[r] && !pass) atomicMax(&s_q[1], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
+        }
+    }
+    __syncthreads();
+    WSL_MARK(8);
+    if (t < 64u) {  // wave 0: entries and masses ranked before each bucket (two buckets a lane)
+        const uint32_t bc0 = b_cnt[2u * lane], bc1 = b_cnt[2u * lane + 1u];
+        const uint64_t bf0 = b_mass[2u * lane], bf1 = b_mass[2u * lane + 1u];
+        const uint32_t cbefore = wave_incl_scan(bc0 + bc1) - (bc0 + bc1);
+        const uint64_t fbefore = wave_incl_scan(bf0 + bf1) - (bf0 + bf1);
+        b_cpre[2u * lane] = cbefore;
+        b_cpre[2u * lane + 1u] = cbefore + bc0;
+        b_fpre[2u * lane] = fbefore;
+        b_fpre[2u * lane + 1u] = fbefore + bf0;
+    }
+    __syncthreads();
+    const uint32_t got0 = b_cpre[64];
+    const uint64_t fbase1 = b_fpre[64];
+    if (s_w[2] || got0 != n_r0) return false;  // heavy ties
+    // every candidate: its rank in the row and the mass up to and with it
+    uint32_t cpos[kRounds];
+    double cin[kRounds], cex[kRounds];
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        cpos[r] = 0xffffffffu;
+        cin[r] = cex[r] = 0.0;
+        if (static_cast<uint32_t>(r) * WS_BLOCK >= n_list) continue;  // uniform
+        const uint32_t bkt = con[r] ? cbkt[r] : 0u;
+        const uint32_t n = con[r] ? b_cnt[bkt] : 0u;
+        uint32_t rank = 0;
+        uint64_t cum = 0;
+        for (uint32_t j = 0; j < n; ++j) {
+            const Place o = lb[bkt * kLeanPlaces + j];
+            rank += o.key > ckey[r] ? 1u : 0u;
+            cum += o.key >= ckey[r] ? o.fx : 0ull;
+        }
+        if (con[r]) {
+            const bool r1 = bkt >= 64u;
+            const uint64_t fb = b_fpre[bkt] - (r1 ? fbase1 : 0ull);
+            const double mb = r1 ? m1base : m0base, inv = r1 ? inv1 : inv0;
+            cin[r] = mb + static_cast<double>(fb + cum) * inv;
+            cex[r] = mb + static_cast<double>(fb + cum - cfix[r]) * inv;
+            cpos[r] = (r1 ? c1base : c0base) + (b_cpre[bkt] - (r1 ? got0 : 0u)) + rank;
+        }
+    }
+    WSL_MARK(9);
+    // ---- the cuts (src/sampling/sampler.cpp:35-74): the first candidate at which the running mass reaches X
+    const uint32_t n1 = V;
+    if (use_top_p && topp_in_list) {
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r)
+            if (cpos[r] != 0xffffffffu && cin[r] >= X && !(cex[r] >= X) && cin[r] > cex[r])
+                atomicMin(&s_q[2], (static_cast<unsigned long long>(cpos[r]) << 32) | (static_cast<uint32_t>(r) * WS_BLOCK + t));
+    }
+    __syncthreads();
+    double mg_top_p = 1.0, mg_min_p = 1.0;
+    uint32_t n2 = n1;
+    bool cut_found = false;
+    if (use_top_p && topp_in_list) {
+        const unsigned long long cq = s_q[2];
+        if (cq != ~0ull && static_cast<uint32_t>(cq >> 32) < n1) {
+            cut_found = true;
+            n2 = static_cast<uint32_t>(cq >> 32) + 1u;
+        } else {  // rounding: the cut falls just past the gathered bins
+            n2 = min(n1, has_r1 ? c1base + n_r1 : c0base + n_r0);
+            mg_top_p = 0.0;
+        }
+    }
+    uint32_t n3 = n2;
+    if (use_min_p && minp_in_list) {
+        const uint32_t passed = s_w[1];
+        double near = 1.0;
+        if (passed > 0u) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[0])) - min_p) / min_p);
+        if (passed < n_list) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[1])) - min_p) / min_p);
+        uint32_t n3p;
+        if (has_r1) n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
+        else n3p = c0base + passed;
+        n3 = min(n2, n3p);
+        if (n3 < 1u) n3 = 1u;
+        mg_min_p = near;
+    }
+    // the cut's margin, and the last kept candidate: mass of the kept set, its key, its own mass
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        if (cpos[r] == 0xffffffffu) continue;
+        if (cut_found && cpos[r] == n2 - 1u) s_d[3] = fmin(cin[r] - X, cpos[r] > 0u ? X - cex[r] : X) / X;
+        if (cpos[r] == n3 - 1u) {
+            s_d[0] = cin[r];
+            s_d[1] = cem[r];
+            s_q[4] = ckey[r];
+            s_w[3] = 1u;
+        }
+    }
+    __syncthreads();
+    if (cut_found) mg_top_p = s_d[3];
+    double Zk;
+    const bool have_last = s_w[3] != 0u;
+    if (have_last) Zk = s_d[0];
+    else if (has_r1 && n3 == c1base) Zk = m1base;  // the cut falls on the upper edge of range 1: everything in earlier bins
+    else if (n3 == c0base && n_r0) Zk = m0base;
+    else Zk = Z;
+    // ---- the draw (src/sampling/sampler.cpp:118-131): the first candidate at which the running mass passes u * Zk
+    const double target = s_d[6] * Zk;
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r)
+        if (cpos[r] != 0xffffffffu && cpos[r] < n3 && cin[r] > target && !(cex[r] > target) && cin[r] > cex[r])
+            atomicMin(&s_q[3], (static_cast<unsigned long long>(cpos[r]) << 32) | (static_cast<uint32_t>(r) * WS_BLOCK + t));
+    __syncthreads();
+    const unsigned long long dq = s_q[3];
+    if (dq == ~0ull && !have_last) return false;  // no candidate for the draw and none to fall back on
+    const uint32_t d_slot = static_cast<uint32_t>(dq), d_pos = static_cast<uint32_t>(dq >> 32);
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        if (dq != ~0ull && static_cast<uint32_t>(r) * WS_BLOCK + t == d_slot) {
+            const double mg = fmin(cin[r] - target, d_pos > 0u ? target - cex[r] : 1e300) / Zk;
+            uint32_t flags = 0;
+            if (mg_top_p < tol) flags |= kNearTopP;
+            if (mg_min_p < tol) flags |= kNearMinP;
+            if (mg < tol) flags |= kNearDraw;
+            A.token[row] = static_cast<int32_t>(cid[r]);
+            A.flags[row] = flags;
+            if (A.prob) A.prob[row] = static_cast<float>(cem[r] / Zk);
+            if (A.margin) A.margin[3 * row + 2] = mg;
+        }
+    }
+    if (t == 0) {
+        if (dq == ~0ull) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
+            uint32_t flags = kNearDraw;
+            if (mg_top_p < tol) flags |= kNearTopP;
+            if (mg_min_p < tol) flags |= kNearMinP;
+            A.token[row] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(s_q[4]));
+            A.flags[row] = flags;
+            if (A.prob) A.prob[row] = static_cast<float>(s_d[1] / Zk);
+            if (A.margin) A.margin[3 * row + 2] = 0.0;
+        }
+        if (A.n_kept) A.n_kept[row] = n3;
+        if (A.stats) {
+            A.stats[2 * row] = m;
+            A.stats[2 * row + 1] = static_cast<float>(Z);
+        }
+        if (A.margin) {
+            A.margin[3 * row] = mg_top_p;
+            A.margin[3 * row + 1] = mg_min_p;
+        }
+    }
+    WSL_MARK(10);
+#ifdef WS_PHASE_TIMERS
+    __syncthreads();
+    if (t < 16 && A.entropy) A.entropy[row * 16 + t] = static_cast<double>(S.marks[t]);
+#endif
+    return true;
+}
+
+// the three-pass code of ws_sample.h for one row, a function of its own: its registers and code stay out of the lean path
+__device__ __noinline__ void three_pass_row(const BatchArgs A, const uint32_t row) { sample_row<false, false, false>(A, row); }
+
+__global__ void __launch_bounds__(WS_BLOCK) lean_batch_kernel(BatchArgs A) {
+    __shared__ LeanShared shared;
+    const uint32_t row = blockIdx.x;
+#ifdef WS_LEAN_UNMASKED_ONLY
+    const bool done = lean_row<false>(A, row, shared);
+#else
+    const bool done = A.allow ? lean_row<true>(A, row, shared) : lean_row<false>(A, row, shared);
+#endif
+#ifndef WS_LEAN_NO_FALLBACK
+    if (done) return;
+    __syncthreads();  // whatever the lean path left in LDS is dead
+    BatchArgs B = A;
+    B.lds_ab = 65536u;
+    B.lds_cnt = 0u;
+    B.lds_tie = A.fb_lds_tie;
+    B.two_sweep = 1;
+    B.work = nullptr;
+    B.split_log2 = 0u;
+    three_pass_row(B, row);
+    if (threadIdx.x == 0) A.flags[row] |= kRouteHandedBack;
+#else
+    if (!done && threadIdx.x == 0) A.token[row] = -2;
+#endif
+}
+
+}  // namespace ws

@@ -97,6 +97,7 @@ struct BatchArgs {
     uint32_t split_spins;      // split rows: looks at the arrival counter before a part gives up on the others (0: about a second's worth)
     uint32_t split_row_bytes;  // kSplitRowBytes, or kSplitRowBytesKept when the rows have a staging area
     uint32_t stage_cap;        // entries of a row's staging area (kSplitStageCap), 0: none
+    uint32_t fb_lds_tie;       // the lean kernel: lds_tie of the three-pass code it hands rows back to
 };
 
 // Global memory of a split row: the merged histogram, the merged candidate list, and four control words (parts that
@@ -1447,8 +1448,10 @@ __device__ __noinline__ ExactOut exact_row(const ExactIn in) {
 // SPLIT: rows split over several workgroups (a build of its own: the unsplit kernel carries none of it). KEPT: the build
 // that can write the kept-set dump; launches without kept_ids take the single-sweep builds that cannot, which keeps the
 // dump's flags and calls out of their register allocation (with them the tile cost 1-2 % more).
+// One row (or one part of a split row) by the workgroup that calls it: `block` = row * parts + part. The kernels below
+// are this function; the lean kernel (ws_lean.h) calls the three-pass instantiation for the rows it hands back.
 template <bool FUSED, bool SPLIT = false, bool KEPT = true>
-__global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
+__device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t block) {
     int32_t* const kept_ids = KEPT ? A.kept_ids : nullptr;
 #ifdef WS_PHASE_TIMERS
     __shared__ long long ws_marks[64];
@@ -1472,7 +1475,7 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
 
     // a row may be split over several workgroups (small batches of the single-sweep kernel): block = row * parts + part
     const uint32_t n_parts = FUSED && SPLIT ? 1u << A.split_log2 : 1u;
-    const uint32_t row = FUSED && SPLIT ? blockIdx.x >> A.split_log2 : blockIdx.x, part = FUSED && SPLIT ? blockIdx.x & (n_parts - 1u) : 0u;
+    const uint32_t row = FUSED && SPLIT ? block >> A.split_log2 : block, part = FUSED && SPLIT ? block & (n_parts - 1u) : 0u;
     bool split = FUSED && SPLIT && n_parts > 1u;  // off again when this part goes on alone
     const uint32_t t = threadIdx.x;
     const uint32_t V = A.vocab;
@@ -3927,6 +3930,11 @@ __global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
         dump_kept_set(in, kid, klg, A.kept_cap);
     }
+}
+
+template <bool FUSED, bool SPLIT = false, bool KEPT = true>
+__global__ void __launch_bounds__(WS_BLOCK) sample_batch_kernel(BatchArgs A) {
+    sample_row<FUSED, SPLIT, KEPT>(A, blockIdx.x);
 }
 
 }  // namespace ws
