@@ -45,9 +45,9 @@ constexpr uint32_t kStaticLds = 4096u;
 #endif
 // the lean kernel's own tables and those of the three-pass code it calls
 #ifdef WS_PHASE_TIMERS
-constexpr uint32_t kStaticLean = 9216u + 512u + 1536u;
+constexpr uint32_t kStaticLean = 11776u + 768u;
 #else
-constexpr uint32_t kStaticLean = 9216u + 512u;
+constexpr uint32_t kStaticLean = 11776u;
 #endif
 
 struct BatchPlan {

@@ -18,8 +18,8 @@
 
 #include "ws_sample.h"
 
-#ifndef WS_EXP_ORDER
-#define WS_EXP_ORDER 0
+#ifndef WS_LEAN_EARLY
+#define WS_LEAN_EARLY 4  // batches binned before the history ids are looked at
 #endif
 
 namespace ws {
@@ -65,23 +65,17 @@ struct LeanHits {
 };
 
 // A third token of a group and beyond goes to list[] as (token | kListNeedsLoad, 0), one LDS atomic each (rare). With
-// TO_LIST every find goes there (a second round of bytes). n_full: cache registers that hold a vector of the row in every
-// thread; register n_full holds one in threads below rem.
+// TO_LIST every find goes there (a second round of bytes).
 template <int NT, bool TO_LIST>
-__device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const uint32_t* __restrict__ xg, uint32_t n_full,
-                                          uint32_t rem, LeanHits& H, uint2* list, uint32_t* n_list, uint32_t cap) {
+__device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const uint32_t* __restrict__ xg, LeanHits& H,
+                                          uint2* list, uint32_t* n_list, uint32_t cap) {
     const uint32_t t = threadIdx.x;
 #pragma unroll
     for (int g = 0; g < kLeanGroups; ++g) {
         uint32_t acc = 0;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const uint32_t c = static_cast<uint32_t>(g * 8 + r);
-            if (c > n_full) continue;  // uniform: a register past the row
-            uint32_t mask = 0x01010101u << r;
-            if (c == n_full && t >= rem) mask = 0u;
-            acc = ((lean_flags<NT>(cache[c], c4) >> (7 - r)) & mask) | acc;  // bit 8 e + r: token e of register r
-        }
+        for (int r = 0; r < 8; ++r)  // bit 8 e + r: token e of register r (registers past the row hold a byte nobody asks for)
+            acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & (0x01010101u << r)) | acc;
         auto token_of = [&](uint32_t bit) { return ((static_cast<uint32_t>(g * 8 + (bit & 7u)) * WS_BLOCK + t) << 2) + (bit >> 3); };
         if (!TO_LIST) {
             H.idx[g] = H.idx[kLeanGroups + g] = 0xffffffffu;
@@ -125,25 +119,21 @@ __device__ __forceinline__ double exp_neg(double a, const double* s_exp) {
     return s_exp[n >> 6] * s_exp[64u + (n & 63u)] * p;
 }
 
-// what wave 0 works out from the scanned histogram for everybody
-struct LeanSel {
-    double X, Z, m0base, m1base, scale0, scale1, inv0, inv1;
-    int r0lo, r0hi, r1lo, r1hi;
-    uint32_t c0base, n_r0, c1base, n_r1;
-    uint32_t topp_in_list, minp_in_list, ok, pad;
+// a bin as the select's searches hand it round: mass ranked before it and up to and with it, tokens before it and in it
+struct LeanBinRec {
+    double mex, min_;
+    uint32_t b, cex, c, pad;
 };
 
 // the lean path's static LDS, declared once by the kernel
 struct LeanShared {
     double s_exp[128];  // kExpHi, kExpLo
-    double pm64[64];    // pm[64 i + 64]
     double red_d[WS_WAVES];
     double s_d[8];
-    LeanSel sel;
+    LeanBinRec rec[4 * WS_WAVES + 2];  // [search][wave], then the two bins named outright
     unsigned long long s_q[6];
     unsigned long long b_mass[kLeanBuckets], b_fpre[kLeanBuckets];
     uint32_t b_cnt[kLeanBuckets], b_cpre[kLeanBuckets];
-    uint32_t pc64[64];  // pc[64 i + 64]
     uint32_t s_w[16];
     uint32_t red_u[WS_WAVES];
     float red_f[WS_WAVES];
@@ -164,8 +154,6 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     uint32_t* red_u = S.red_u;
     double* red_d = S.red_d;
     double* s_exp = S.s_exp;
-    double* pm64 = S.pm64;
-    uint32_t* pc64 = S.pc64;
     uint32_t* s_w = S.s_w;
     unsigned long long* s_q = S.s_q;
     double* s_d = S.s_d;
@@ -188,26 +176,27 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     rv.touched = nullptr;
     const uint32_t nv = V >> 2;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
-    // Batches 0 .. kPre - 1 have registers of their own and are all asked for before phase 0 - the bin cache is not live
-    // yet, so there is room - which puts a third of the row on its way while the tables are built; from batch kPre on
-    // the first three of those slots are a ring, two batches in flight while one is consumed.
-    constexpr int kPre = 6, kRing = 3;
-    uint4 q[kPre][kLeanBatch];
-    uint32_t na[kPre][kLeanBatch];
-    auto load = [&](int bt, int slot) {
+    // The row's loads run through a ring of three batches, two in flight while one is consumed (a compute unit holds about
+    // that much in flight: a wave that asks for more waits at the request). The first two batches are asked for before
+    // anything else - their address needs the kernel's arguments only - and travel while the row's parameters and then
+    // the history ids are fetched, two dependent trips to memory; the first kEarly batches are binned before those ids
+    // are looked at (what the ids touch there is put right afterwards), so that phase 0 costs its LDS work and no wait.
+    constexpr int kRing = 3, kEarly = WS_LEAN_EARLY;
+    constexpr int NB = kLeanRegs / kLeanBatch;
+    uint4 q[kRing][kLeanBatch];
+    uint32_t na[kRing][kLeanBatch];
+    auto load = [&](int bt, int slot) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < kLeanBatch; ++u) {
             const uint32_t j = (bt * kLeanBatch + u) * WS_BLOCK + t;
-            const uint32_t jc = j < nv ? j : nv - 1u;
+            const uint32_t jc = j < nv ? j : nv - 1u;  // (unconditional, clamped to the row: a load behind a branch makes the compiler wait for every load before it)
             q[slot][u] = xv[jc];
             na[slot][u] = MASKED ? rv.allow[(jc * 4u) >> 5] : 0xffffffffu;  // (complemented where it is used: nothing waits for the load here)
         }
     };
-
-#if WS_EXP_ORDER == 2
     load(0, 0);
     load(1, 1);
-#endif
+
     uint64_t* hist = reinterpret_cast<uint64_t*>(lds);
     uint4* stage = reinterpret_cast<uint4*>(lds + 32768);
     uint32_t* touched = reinterpret_cast<uint32_t*>(lds + A.lds_ab);
@@ -218,15 +207,18 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     uint64_t* hist2 = A.lds_tie ? reinterpret_cast<uint64_t*>(lds + A.lds_tie) : nullptr;
     rv.wprefix = wprefix;
     rv.pv = pv;
+    for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
+    if (hist2)
+        for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
 
     const float inv_t = A.inv_t[row];
     const uint32_t top_k = A.top_k ? A.top_k[row] : 0u;
-    const double top_p = A.top_p ? A.top_p[row] : 1.0;
-    const double min_p = A.min_p ? A.min_p[row] : 0.0;
-    const double tol = A.tol;
-    const float rep = A.rep ? A.rep[row] : 1.f, pres = A.pres ? A.pres[row] : 0.f, freq = A.freq ? A.freq[row] : 0.f;
     const bool race = A.race != nullptr && A.race[row] != 0;
-    const bool use_top_p = top_p < 1.0, use_min_p = min_p > 0.0;
+    bool use_top_p, use_min_p;
+    {
+        const double top_p0 = A.top_p ? A.top_p[row] : 1.0, min_p0 = A.min_p ? A.min_p[row] : 0.0;  // (both are read again behind the sweep)
+        use_top_p = top_p0 < 1.0, use_min_p = min_p0 > 0.0;
+    }
     const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? (A.hist_len ? A.hist_len[row] : A.hist_off[row + 1] - h0) : 0u;
     const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
     // rows this code does not take: a top-k, no filter at all, the race draw, parameters the three-pass code reports
@@ -240,41 +232,114 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 #pragma unroll
     for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
     const uint32_t bid = t < nb ? static_cast<uint32_t>(bias_ids[t]) : 0xffffffffu;  // the first bias ids
-    const double exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);
-    // The row's first kPre batches are asked for behind the history ids, not before them: with every compute unit streaming,
-    // a request waits for all that is queued before it - microseconds - and phase 0 cannot start without the ids.
-    // (unconditional, addresses clamped to the row: a load behind a branch makes the compiler wait for every load before it)
-    // Every wave's ids are on their way before any wave asks for the row: the compute unit serves its waves' requests in
-    // the order they were made, and phase 0 needs all sixteen waves' ids. (A bare barrier: it waits for no memory.)
-#if WS_EXP_ORDER == 1
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the ids are here before the row is asked for
-#else
-    __builtin_amdgcn_s_barrier();
-#endif
-#pragma unroll
-    for (int bt = WS_EXP_ORDER == 2 ? 2 : 0; bt < kPre; ++bt) load(bt, bt);
     if (wv == WS_WAVES - 1u) {  // one wave draws the row's uniform for everybody
         const double u_ = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
         if (lane == 0u) s_d[6] = u_;
     }
     WSL_MARK(0);
 
+    // ------------------------------------------------------------------ the anchor: the head of the row + 8 exponent units
+    const float c64 = inv_t * 64.f;
+    float anchor, aq;
+    {
+        float s = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < kLeanBatch; ++u) {
+            s = fmaxf(s, fmaxf(fmaxf(__uint_as_float(q[0][u].x), __uint_as_float(q[0][u].y)),
+                               fmaxf(__uint_as_float(q[0][u].z), __uint_as_float(q[0][u].w))));
+        }
+        s = block_max(s, red_f);  // its barriers also publish the zeroed histogram
+        anchor = s + 8.f / inv_t;
+        aq = anchor_product(anchor, c64);
+        if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
+    }
+
+    // ------------------------------------------------------------------ the sweep
+    uint32_t cache[kLeanRegs];
+    float m = -INFINITY;
+    float vm_early[kEarly * kLeanBatch];  // maxima of the early batches' vectors, until the bitmap says which hold a touched token
+    const float tail_f = own_tail();
+    uint64_t* myhist = (hist2 && (t & 1u)) ? hist2 : hist;
+    const uint32_t stage_cap = 2047u;
+    const uint32_t n_full = nv / WS_BLOCK;  // vector rounds that are inside the row for every thread
+    bool any_touched = false;               // uniform
+    // the bitmap words of a batch are read a batch ahead, before the batch in between adds to the histogram: LDS
+    // operations of a wave finish in order, and a read asked for behind the additions would wait for all of them
+    uint32_t tws[2][kLeanBatch], wps[2][kLeanBatch];
+    auto read_words = [&](int bt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < kLeanBatch; ++u) {
+            const uint32_t word = (((bt * kLeanBatch + u) * WS_BLOCK + t) * 4u) >> 5;  // (past the row: a word past the bitmap, inside the block's LDS)
+            tws[bt & 1][u] = any_touched ? touched[word] : 0u;
+            wps[bt & 1][u] = any_touched ? wprefix[word] : 0u;
+        }
+    };
+    // one batch: every token into the histogram, its bin's low byte into the cache; `early`: before phase 0. (A macro, not a
+    // function: the cache stays in registers only while every index into it is a constant where the loops are unrolled.)
+#define WSL_SWEEP_BATCH(bt, early)                                                                                                   \
+    {                                                                                                                                \
+        const int slot = (bt) % kRing;                                                                                               \
+        if (!(early) && (bt) + 1 < NB) read_words((bt) + 1);                                                                         \
+        _Pragma("unroll") for (int u = 0; u < kLeanBatch; ++u) {                                                                     \
+            const uint32_t j = ((bt) * kLeanBatch + u) * WS_BLOCK + t;                                                               \
+            const int c = (bt) * kLeanBatch + u;                                                                                     \
+            uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};                                                \
+            uint32_t tw = (early) ? 0u : tws[(bt) & 1][u], nal = MASKED ? ~na[slot][u] : 0u;                                         \
+            if (static_cast<uint32_t>(c) >= n_full && j >= nv) { /* (only the row's last round has lanes past it) NaN: the tail bins */ \
+                w[0] = w[1] = w[2] = w[3] = 0xffffffffu;                                                                             \
+                tw = 0u;                                                                                                             \
+            }                                                                                                                        \
+            const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * 4u) & 31u)) : 0;                                           \
+            uint32_t bins[4];                                                                                                        \
+            float vm = -INFINITY;                                                                                                    \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                                          \
+                uint32_t bits = w[e];                                                                                                \
+                if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);                                                   \
+                const float x = __uint_as_float(bits);                                                                               \
+                vm = fmaxf(vm, x);                                                                                                   \
+                const float tc = bin_coord(aq, c64, x, tail_f);                                                                      \
+                bins[e] = static_cast<uint32_t>(tc);                                                                                 \
+                WSL_HIST_ADD(bins[e], tc);                                                                                           \
+            }                                                                                                                        \
+            const uint32_t lo2 = __builtin_amdgcn_perm(bins[1], bins[0], 0x0c0c0400u);                                               \
+            uint32_t packed = __builtin_amdgcn_perm(bins[3], bins[2], 0x04000c0cu) | lo2;                                            \
+            asm volatile("" : "+v"(packed)); /* (packed here, not where the tail first looks at it: four bins would stay live) */     \
+            cache[c] = packed;                                                                                                       \
+            if (early) {                                                                                                             \
+                vm_early[c < kEarly * kLeanBatch ? c : 0] = vm;                                                                      \
+            } else {                                                                                                                 \
+                const uint32_t sh = (j * 4u) & 31u;                                                                                  \
+                const bool touched_vec = ((tw >> sh) & 15u) != 0u;                                                                   \
+                m = fmaxf(m, touched_vec ? -INFINITY : vm); /* (a vector with a touched token is looked at when that token is collected) */ \
+                if (touched_vec) {                                                                                                   \
+                    const uint32_t r = wps[(bt) & 1][u] + __popc(tw & ((1u << sh) - 1u));                                            \
+                    stage[min(r, stage_cap)] = q[slot][u];                                                                           \
+                }                                                                                                                    \
+            }                                                                                                                        \
+        }                                                                                                                            \
+    }
+#ifndef WS_EXP_NOATOMIC
+#define WSL_HIST_ADD(bin, tc) atomicAdd(reinterpret_cast<unsigned long long*>(&myhist[bin]), bin_word(tc))
+#else
+#define WSL_HIST_ADD(bin, tc) m = fmaxf(m, __uint_as_float(static_cast<uint32_t>(bin_word(tc))))
+#endif
+#ifndef WS_EXP_NOLOAD
+#define WSL_NEXT_LOAD(bt, slot) \
+    if ((bt) + kRing < NB) load((bt) + kRing, slot) /* the slot is free: the batch three ahead */
+#else
+#define WSL_NEXT_LOAD(bt, slot)
+#endif
     // ------------------------------------------------------------------ phase 0 (ws_sample.h): bitmap of the touched ids,
     // popcount prefix per word (rank of a touched id), per-rank history count and bias entries
-    for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
-    if (hist2)
-        for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
-    if (t < 128) s_exp[t] = exp_tab;
     uint32_t n_touched = 0;
+    auto phase0 = [&]() __attribute__((always_inline)) {
     if (nh + nb > 0) {
         for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
         for (uint32_t r = t; r < nh + nb; r += WS_BLOCK) {  // (at most nh + nb distinct ids)
             cnt[r] = 0u;
             first[r] = 0xffffffffu;
         }
-        WSL_MARK(11);
         __syncthreads();
-        WSL_MARK(12);
 #pragma unroll
         for (int k = 0; k < kHid; ++k)
             if (hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
@@ -288,7 +353,6 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
         }
         __syncthreads();
-        WSL_MARK(13);
         constexpr uint32_t kChunk = 5;  // 163840 / 32 / 1024 words per thread
         const uint32_t w0 = t * kChunk;
         uint32_t wd[kChunk], local = 0;
@@ -307,7 +371,6 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             run += __popc(wd[k]);
         }
         __syncthreads();
-        WSL_MARK(14);
         rv.touched = touched;
         const bool ids_now = nb == 0;  // without a bias list the second table takes the token id of each rank right away
 #pragma unroll
@@ -334,103 +397,59 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             }
         }
         n_touched = n_uniq;
+        any_touched = n_uniq != 0u;
     }
     WSL_MARK(1);
-
-    // ------------------------------------------------------------------ the anchor: the head of the row + 8 exponent units
-    const float c64 = inv_t * 64.f;
-    float anchor, aq;
-    {
-        float s = -INFINITY;
+    // the early batches' vectors: those without a touched token count for the running maximum
 #pragma unroll
-        for (int u = 0; u < kLeanBatch; ++u) {
-            s = fmaxf(s, fmaxf(fmaxf(__uint_as_float(q[0][u].x), __uint_as_float(q[0][u].y)),
-                               fmaxf(__uint_as_float(q[0][u].z), __uint_as_float(q[0][u].w))));
-        }
-        s = block_max(s, red_f);  // its barriers also publish phase 0's tables and the zeroed histogram
-        anchor = s + 8.f / inv_t;
-        aq = anchor_product(anchor, c64);
-        if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
+    for (int c = 0; c < kEarly * kLeanBatch; ++c) {
+        const uint32_t j = static_cast<uint32_t>(c) * WS_BLOCK + t;
+        const uint32_t tw = any_touched ? touched[(j * 4u) >> 5] : 0u;
+        m = fmaxf(m, ((tw >> ((j * 4u) & 31u)) & 15u) ? -INFINITY : vm_early[c]);
     }
-
-    // ------------------------------------------------------------------ the sweep
-    uint32_t cache[kLeanRegs];
-    float m = -INFINITY;
-    {
-        constexpr int NB = kLeanRegs / kLeanBatch;
-        const float tail_f = own_tail();
-        uint64_t* myhist = (hist2 && (t & 1u)) ? hist2 : hist;
-        const bool any_touched = n_touched != 0u;  // uniform
-        const uint32_t stage_cap = 2047u;
-        const uint32_t n_full = nv / WS_BLOCK;  // vector rounds that are inside the row for every thread
-        // the bitmap words of a batch are read a batch ahead, before the batch in between adds to the histogram: LDS
-        // operations of a wave finish in order, and a read asked for behind the additions would wait for all of them
-        uint32_t tws[2][kLeanBatch], wps[2][kLeanBatch];
-        auto read_words = [&](int bt) {
+    read_words(kEarly);
+    };
+    const uint32_t early_end = min(static_cast<uint32_t>(kEarly * kLeanBatch) * WS_BLOCK * 4u, V);  // tokens below this were binned before phase 0: not staged
+    load(2, 2);
+    double exp_tab = 0.0;
+    // (one unrolled loop for all batches, phase 0 inside it: the bin cache stays in registers only while every index into
+    // it is a constant once the loop is unrolled)
 #pragma unroll
-            for (int u = 0; u < kLeanBatch; ++u) {
-                const uint32_t word = (((bt * kLeanBatch + u) * WS_BLOCK + t) * 4u) >> 5;  // (past the row: a word past the bitmap, inside the block's LDS)
-                tws[bt & 1][u] = any_touched ? touched[word] : 0u;
-                wps[bt & 1][u] = any_touched ? wprefix[word] : 0u;
-            }
-        };
-        read_words(0);
-#pragma unroll
-        for (int bt = 0; bt < NB; ++bt) {
-            const int slot = bt < kPre ? bt : bt % kRing;
-            if (static_cast<uint32_t>(bt * kLeanBatch) * WS_BLOCK >= nv) {  // uniform: the row is done
-#pragma unroll
-                for (int c = bt * kLeanBatch; c < kLeanRegs; ++c) cache[c] = 0u;
-                break;
-            }
-            if (bt + 1 < NB) read_words(bt + 1);
-#pragma unroll
-            for (int u = 0; u < kLeanBatch; ++u) {
-                const uint32_t j = (bt * kLeanBatch + u) * WS_BLOCK + t;
-                const int c = bt * kLeanBatch + u;
-                uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};
-                uint32_t tw = tws[bt & 1][u], nal = MASKED ? ~na[slot][u] : 0u;
-                if (static_cast<uint32_t>(c) >= n_full && j >= nv) {  // (only the row's last round has lanes past it) NaN: the tail bins, nobody's candidate
-                    w[0] = w[1] = w[2] = w[3] = 0xffffffffu;
-                    tw = 0u;
-                }
-                const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * 4u) & 31u)) : 0;
-                uint32_t bins[4];
-                float vm = -INFINITY;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    uint32_t bits = w[e];
-                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);
-                    const float x = __uint_as_float(bits);
-                    vm = fmaxf(vm, x);
-                    const float tc = bin_coord(aq, c64, x, tail_f);
-                    bins[e] = static_cast<uint32_t>(tc);
-#ifndef WS_EXP_NOATOMIC
-                    atomicAdd(reinterpret_cast<unsigned long long*>(&myhist[bins[e]]), bin_word(tc));
-#else
-                    m = fmaxf(m, __uint_as_float(static_cast<uint32_t>(bin_word(tc))));
-#endif
-                }
-                const uint32_t lo2 = __builtin_amdgcn_perm(bins[1], bins[0], 0x0c0c0400u);
-                cache[c] = __builtin_amdgcn_perm(bins[3], bins[2], 0x04000c0cu) | lo2;
-                const uint32_t sh = (j * 4u) & 31u;
-                const bool touched_vec = ((tw >> sh) & 15u) != 0u;
-                m = fmaxf(m, touched_vec ? -INFINITY : vm);  // (a vector with a touched token is looked at when that token is collected)
-                if (touched_vec) {
-                    const uint32_t r = wps[bt & 1][u] + __popc(tw & ((1u << sh) - 1u));
-                    stage[min(r, stage_cap)] = q[slot][u];
-                }
-            }
-            // the slot is free: the first three take batches kPre .. kPre + 2 right away, later ones the batch three ahead
-            constexpr int kNone = 1 << 20;
-            const int next = bt < kRing ? bt + kPre : (bt >= kPre ? bt + kRing : kNone);
-#ifndef WS_EXP_NOLOAD
-            if (next < NB) load(next, next % kRing);
-#endif
+    for (int bt = 0; bt < NB; ++bt) {
+        if (bt == kEarly) {
+            WSL_MARK(11);
+            phase0();
         }
+        if (bt == NB - 4) exp_tab = t < 64 ? kExpHi[t] : (t < 128 ? kExpLo[t - 64] : 0.0);  // the histogram scan's tables: asked for now, parked in LDS after the sweep
+        if (bt < kEarly) {
+            WSL_SWEEP_BATCH(bt, true)
+        } else if (static_cast<uint32_t>(bt * kLeanBatch) * WS_BLOCK < nv) {  // uniform
+            WSL_SWEEP_BATCH(bt, false)
+        } else {  // past the row (no way out of the loop here: with one, the cache no longer stays in registers)
+#pragma unroll
+            for (int u = 0; u < kLeanBatch; ++u) cache[bt * kLeanBatch + u] = 0u;
+        }
+        WSL_NEXT_LOAD(bt, bt % kRing);
     }
+    if (t < 128) s_exp[t] = exp_tab;
+#undef WSL_SWEEP_BATCH
+#undef WSL_HIST_ADD
+#undef WSL_NEXT_LOAD
+    if (t < 128) s_exp[t] = exp_tab;
     __syncthreads();
     WSL_MARK(2);
+    // Everything behind the sweep reads its arguments again, through a pointer the compiler cannot see through: none of
+    // them stays in a register across the sweep (they spilled there, dozens of them, and every phase paid for it).
+    // (the kernel's argument segment itself, where BatchArgs is the first and only argument: scalar loads, no copy)
+    typedef const __attribute__((address_space(4))) BatchArgs* ArgPtr;
+    ArgPtr Ap = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(Ap));
+    const double top_p = Ap->top_p ? Ap->top_p[row] : 1.0;
+    const double min_p = Ap->min_p ? Ap->min_p[row] : 0.0;
+    const float rep = Ap->rep ? Ap->rep[row] : 1.f, pres = Ap->pres ? Ap->pres[row] : 0.f, freq = Ap->freq ? Ap->freq[row] : 0.f;
+    const int32_t* hist_ids2 = Ap->hist + h0;
+    const int32_t* bias_ids2 = Ap->bias_ids + b0;
+    const float* bias_vals2 = Ap->bias_vals + b0;
 
     // ------------------------------------------------------------------ the touched tokens (collect_fused of ws_sample.h):
     // every history / bias entry claims its token's rank; the owner adjusts the token's logit and moves the token from the
@@ -448,7 +467,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const uint32_t j = j0 + k * WS_BLOCK + t;
-                    id[k] = (in_regs && j0 == 0u) ? hid[k] : (j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu);
+                    id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;  // (read again: the sweep has the registers)
                     if (id[k] >= V) id[k] = 0xffffffffu;
                 }
 #pragma unroll
@@ -466,7 +485,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     rk[k] = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));
                     old[k] = id[k] < V ? atomicOr(&cnt[rk[k]], kClaim) : kClaim;
                     if (i < whole_end) {
-                        if (rf < stage_cap) vec[k] = stage[rf];
+                        if (rf < stage_cap && i >= early_end) vec[k] = stage[rf];
                         else vec[k] = xv[i >> 2];
                     } else {
                         const uint32_t b = static_cast<const uint32_t*>(rv.base)[i];
@@ -479,7 +498,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     const uint32_t i = id[k];
                     const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
                     const bool whole = i < whole_end;
-                    const uint32_t bits = whole ? w[i & 3u] : w[0];
+                    const uint32_t e_ = whole ? (i & 3u) : 0u; const uint32_t bits = e_ == 0u ? w[0] : (e_ == 1u ? w[1] : (e_ == 2u ? w[2] : w[3]));
                     const float raw = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits), -INFINITY) : -INFINITY;
                     if (whole) {
                         const uint32_t free_bits = (al[k] & ~tw[k]) >> (i & 28u);
@@ -491,10 +510,10 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     float x = raw;
                     if (n_bias) {
                         uint32_t j = first[rk[k]];
-                        x = __fadd_rn(x, bias_vals[j]);
+                        x = __fadd_rn(x, bias_vals2[j]);
                         if (n_bias > 1u)
                             for (++j; j < nb; ++j)
-                                if (static_cast<uint32_t>(bias_ids[j]) == i) x = __fadd_rn(x, bias_vals[j]);
+                                if (static_cast<uint32_t>(bias_ids2[j]) == i) x = __fadd_rn(x, bias_vals2[j]);
                     }
                     if (c) {
                         x = x > 0.f ? __fdiv_rn(x, rep) : __fmul_rn(x, rep);
@@ -509,8 +528,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 }
             }
         };
-        take4(hist_ids, nh, true);
-        take4(bias_ids, nb, false);
+        take4(hist_ids2, nh, true);
+        take4(bias_ids2, nb, false);
     }
     WSL_MARK(3);
     {
@@ -519,16 +538,18 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     }
     if (!(m <= anchor && (anchor - m) * c64 <= 1024.f)) return false;  // (also a row without any token: m = -inf)
 
-    // ------------------------------------------------------------------ scan of the histogram: four consecutive bins a thread
+    // ------------------------------------------------------------------ scan of the histogram: four consecutive bins a thread,
+    // the prefixes stay in registers
     const double lift = static_cast<double>(aq) * (1.0 / 64.0) - static_cast<double>(m) * static_cast<double>(inv_t);  // >= 0
     if (wv == 0u) {  // one wave: the factor that takes masses from the anchor to the maximum
         const double tm = exp(lift);
         if (lane == 0u) s_d[7] = tm;
     }
-    double* pm = reinterpret_cast<double*>(lds);                   // pm[b]: mass ranked before bin b; 4097 entries
-    uint32_t* pc = reinterpret_cast<uint32_t*>(lds + 32768 + 16);  // pc[b]: tokens ranked before bin b; 4097 entries
+    const uint32_t bb = 4u * t;  // this thread's bins: bb .. bb + 3
+    uint32_t c4b[4], ce[4];      // tokens in the bin, tokens ranked before it
+    double me[5];                // mass ranked before the bin; me[4]: before the next thread's first bin
+    double Z;
     {
-        const uint32_t bb = 4u * t;
         uint64_t h[4];
         {
             const ulonglong2 h01 = *reinterpret_cast<const ulonglong2*>(&hist[bb]), h23 = *reinterpret_cast<const ulonglong2*>(&hist[bb + 2u]);
@@ -538,20 +559,25 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 h[0] += g01.x, h[1] += g01.y, h[2] += g23.x, h[3] += g23.y;
             }
         }
-        const double eh = s_exp[bb >> 6];
-        uint32_t c4b[4];
         double ms[4];
         uint32_t lc = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t b = bb + k;
-            c4b[k] = b < static_cast<uint32_t>(kTail) ? static_cast<uint32_t>(h[k] >> kCountShift) : 0u;  // (the tail's words are not looked at one by one)
-            const double fix = static_cast<double>(h[k] & ((1ull << kCountShift) - 1ull)) * kFixInv;
-            ms[k] = c4b[k] ? eh * s_exp[64 + (b & 63u)] * (static_cast<double>(c4b[k]) - fix) : 0.0;
+            c4b[k] = bb + k < static_cast<uint32_t>(kTail) ? static_cast<uint32_t>(h[k] >> kCountShift) : 0u;  // (the tail's words are not looked at one by one)
+            ms[k] = 0.0;
             lc += c4b[k];
         }
+        if (__ballot(lc != 0u)) {  // uniform: a wave whose 256 bins hold no token needs no arithmetic
+            const double eh = s_exp[bb >> 6];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t fl = static_cast<uint32_t>(h[k]), fh = static_cast<uint32_t>(h[k] >> 32) & ((1u << (kCountShift - 32)) - 1u);
+                const double fix = (static_cast<double>(fh) * 4294967296.0 + static_cast<double>(fl)) * kFixInv;  // exact: below 2^44
+                ms[k] = c4b[k] ? eh * s_exp[64 + ((bb + k) & 63u)] * (static_cast<double>(c4b[k]) - fix) : 0.0;
+            }
+        }
         const uint32_t ic = wave_incl_scan(lc);
-        __syncthreads();  // every read of the histogram is done: the prefixes go over it; the factor is in place
+        __syncthreads();  // the factor is in place (and every read of the histogram is done)
         const double to_max = s_d[7];
         double lm = 0.0;
 #pragma unroll
@@ -566,22 +592,16 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             red_d[wv] = im;
         }
         __syncthreads();
-        uint32_t base_c = 0;
-        double base_m = 0.0, all_m = 0.0;
-#pragma unroll
-        for (uint32_t w = 0; w < WS_WAVES; ++w) {
-            const uint32_t sc = red_u[w];
-            const double sm = red_d[w];
-            if (w < wv) {
-                base_c += sc;
-                base_m += sm;
-            }
-            all_m += sm;
-        }
+        // the waves' totals, scanned by every wave again: lane w holds wave w's
+        const uint32_t wc = lane < WS_WAVES ? red_u[lane] : 0u;
+        const double wm = lane < WS_WAVES ? red_d[lane] : 0.0;
+        const uint32_t wci = wave_incl_scan(wc);
+        const double wmi = wave_incl_scan(wm);
+        const uint32_t base_c = wv ? lane_value(wci, wv - 1u) : 0u;
+        const double base_m = wv ? lane_value(wmi, wv - 1u) : 0.0;
+        Z = lane_value(wmi, WS_WAVES - 1u);
         uint32_t rc = base_c + ic - lc;
         double rm = base_m + (lane ? up : 0.0);
-        uint32_t ce[4];
-        double me[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             ce[k] = rc;
@@ -589,130 +609,190 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             rc += c4b[k];
             rm += ms[k];
         }
-        *reinterpret_cast<uint4*>(&pc[bb]) = make_uint4(ce[0], ce[1], ce[2], ce[3]);  // (pc is 16 bytes into its region: aligned)
-        *reinterpret_cast<double2*>(&pm[bb]) = make_double2(me[0], me[1]);
-        *reinterpret_cast<double2*>(&pm[bb + 2u]) = make_double2(me[2], me[3]);
-        if ((t & 15u) == 15u) {
-            pc64[t >> 4] = t == WS_BLOCK - 1u ? V : rc;
-            pm64[t >> 4] = t == WS_BLOCK - 1u ? all_m : rm;
-        }
-        if (t == WS_BLOCK - 1u) {
-            pc[kBins] = V;  // every token of the row is in some bin: the tail holds what the others do not
-            pm[kBins] = all_m;
-        }
+        me[4] = base_m + im;  // (what the next thread starts from, bit for bit)
+        if (t == WS_BLOCK - 1u) me[4] = Z;
     }
-    __syncthreads();
     WSL_MARK(4);
+    const double Zf = static_cast<double>(static_cast<float>(Z));  // Sampler::sum is a float (src/sampling/sampler.h:38)
 
     // ------------------------------------------------------------------ select (the rules of ws_sample.h): the bins the cut
-    // and the draw can fall in, by wave 0 for everybody
-    if (wv == 0u) {
-        const double to_max = s_d[7];
-        const double Z = pm[kBins];
-        const double Zf = static_cast<double>(static_cast<float>(Z));  // Sampler::sum is a float (src/sampling/sampler.h:38)
-        auto first_bin = [&](auto&& reached_end, auto&& reached) {
-            const uint64_t coarse = __ballot(reached_end(static_cast<int>(lane)));
-            if (!coarse) return static_cast<int>(kBins);
-            const int base = 64 * (__ffsll(static_cast<unsigned long long>(coarse)) - 1);
-            const uint64_t fine = __ballot(reached(base + static_cast<int>(lane)));
-            return base + (__ffsll(static_cast<unsigned long long>(fine)) - 1);
-        };
-        auto find_mass = [&](double X, bool strict) {
-            if (!strict && !(X > 0.0)) return -1;
-            int b = strict ? first_bin([&](int i) { return pm64[i] > X; }, [&](int k) { return pm[k + 1] > X; })
-                           : first_bin([&](int i) { return pm64[i] >= X; }, [&](int k) { return pm[k + 1] >= X; });
-            while (b < kBins && pc[b + 1] == pc[b]) ++b;
-            return b < kBins ? b : -1;
-        };
-        int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
-        bool minp_in_list = false, topp_in_list = false;
-        double X = 0;
-        const double u = s_d[6];
-        int b2 = -1, lo3 = kBins, hi3 = -1;
+    // and the draw can fall in. Every thread looks at the four bins it has just scanned; a search - the first bin with a
+    // token whose mass prefix reaches a value - is one ballot per wave, one record per wave in LDS and one barrier.
+    using BinRec = LeanBinRec;
+    BinRec* rec = S.rec;  // [search][wave]
+    // this thread's first bin with a token whose inclusive prefix satisfies the test; 4 when none does. Only one wave has
+    // such a bin that counts - the wave in whose 256 bins the prefix passes the value: the waves before it reach no such
+    // bin, the waves behind it are not the first - so the others answer without looking.
+    const double wave_lo = lane_value(me[0], 0u), wave_hi = lane_value(me[4], 63u);  // prefix before the wave's bins and behind them
+    auto first_own = [&](double Xq, bool strict) {
+        uint32_t k = 4u;
+        const bool mine = strict ? (wave_hi > Xq && !(wave_lo > Xq)) : (wave_hi >= Xq && !(wave_lo >= Xq));  // uniform
+        if (mine) {
+#pragma unroll
+            for (int j = 3; j >= 0; --j)
+                if (c4b[j] != 0u && (strict ? me[j + 1] > Xq : me[j + 1] >= Xq)) k = static_cast<uint32_t>(j);
+        }
+        return k;
+    };
+    auto publish = [&](uint32_t search, uint32_t k) {  // the wave's first such bin
+        const uint64_t any = __ballot(k < 4u);
+        if (any == 0ull) {
+            if (lane == 0u) rec[search * WS_WAVES + wv].b = 0xffffffffu;
+        } else if (lane == static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(any)) - 1)) {
+            BinRec r;
+            r.b = bb + k;
+            r.mex = k == 0u ? me[0] : (k == 1u ? me[1] : (k == 2u ? me[2] : me[3]));
+            r.min_ = k == 0u ? me[1] : (k == 1u ? me[2] : (k == 2u ? me[3] : me[4]));
+            r.cex = k == 0u ? ce[0] : (k == 1u ? ce[1] : (k == 2u ? ce[2] : ce[3]));
+            r.c = k == 0u ? c4b[0] : (k == 1u ? c4b[1] : (k == 2u ? c4b[2] : c4b[3]));
+            r.pad = 0u;
+            rec[search * WS_WAVES + wv] = r;
+        }
+    };
+    auto found = [&](uint32_t search) {  // the first wave's record that holds a bin (b = 0xffffffff: none)
+        BinRec r;
+        r.b = 0xffffffffu;
+        r.mex = r.min_ = 0.0;
+        r.cex = r.c = r.pad = 0u;
+        const uint32_t mine = lane < WS_WAVES ? rec[search * WS_WAVES + lane].b : 0xffffffffu;
+        const uint64_t any = __ballot(mine != 0xffffffffu);
+        if (any) r = rec[search * WS_WAVES + static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(any)) - 1)];
+        return r;
+    };
+    // the record of a bin named outright, by the thread that owns it (searches 4..7)
+    auto publish_bin = [&](uint32_t search, int b) {
+        if (b >= 0 && static_cast<uint32_t>(b) >> 2 == t) {
+            const uint32_t k = static_cast<uint32_t>(b) & 3u;
+            BinRec r;
+            r.b = static_cast<uint32_t>(b);
+            r.mex = k == 0u ? me[0] : (k == 1u ? me[1] : (k == 2u ? me[2] : me[3]));
+            r.min_ = k == 0u ? me[1] : (k == 1u ? me[2] : (k == 2u ? me[3] : me[4]));
+            r.cex = k == 0u ? ce[0] : (k == 1u ? ce[1] : (k == 2u ? ce[2] : ce[3]));
+            r.c = k == 0u ? c4b[0] : (k == 1u ? c4b[1] : (k == 2u ? c4b[2] : c4b[3]));
+            r.pad = 0u;
+            rec[4u * WS_WAVES + (search - 4u)] = r;
+        }
+    };
+    int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
+    bool minp_in_list = false, topp_in_list = false;
+    double X = 0;
+    const double u = s_d[6];
+    int lo3 = kBins, hi3 = -1;
+    if (use_min_p) {
+        const double astar = (-log(min_p) + lift) * 64.0;
+        const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
+        lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
+        hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
+    }
+    // round 1: the top-p cut against the float normaliser and against the exact one; the min-p bins by name
+    if (use_top_p) {
+        const double Xf = top_p * Zf, Xz = top_p * Z;
+        publish(0u, Xf > 0.0 ? first_own(Xf, false) : 4u);
+        publish(1u, Xz > 0.0 ? first_own(Xz, false) : 4u);
+    }
+    if (use_min_p) {
+        publish_bin(4u, min(lo3, kTail - 1));
+        publish_bin(5u, min(hi3, kTail - 1));
+    }
+    if (t == 0) {
+        s_w[0] = 0u;
+        s_w[5] = 0u;
+    }
+    __syncthreads();
+    double zlo = Z, zhi = Z;       // bounds of the kept mass
+    uint32_t r1c0 = 0, r1c1 = 0;   // tokens ranked before range 1, and up to and with its last bin
+    {
+        int b2 = -1;
+        BinRec cut;
+        cut.b = 0xffffffffu;
         if (use_top_p) {
             X = top_p * Zf;
-            b2 = find_mass(X, false);
-            if (b2 >= 0 && pc[b2] >= 16384u) {
+            cut = found(0u);
+            if (cut.b != 0xffffffffu && cut.cex >= 16384u) {
                 X = top_p * Z;
-                b2 = find_mass(X, false);
+                cut = found(1u);
             }
-            if (b2 < 0) b2 = kTail;
+            b2 = cut.b != 0xffffffffu ? static_cast<int>(cut.b) : kTail;
         }
-        if (use_min_p) {
-            const double astar = (-log(min_p) + lift) * 64.0;
-            const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
-            lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
-            hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
-        }
+        const BinRec flo = use_min_p ? rec[4u * WS_WAVES] : cut, fhi = use_min_p ? rec[4u * WS_WAVES + 1u] : cut;
         if (use_top_p && (!use_min_p || b2 < lo3)) {
             r1lo = r1hi = b2;
             topp_in_list = true;
+            zlo = cut.mex, zhi = cut.min_;
+            r1c0 = cut.cex, r1c1 = cut.cex + cut.c;
         } else if (use_min_p && (!use_top_p || hi3 < b2)) {
             r1lo = lo3;
             r1hi = hi3;
             minp_in_list = true;
+            zlo = flo.mex, zhi = fhi.min_;
+            r1c0 = flo.cex, r1c1 = fhi.cex + fhi.c;
         } else if (use_top_p && use_min_p) {
             r1lo = min(b2, lo3);
             r1hi = max(b2, hi3);
             minp_in_list = topp_in_list = true;
+            zlo = b2 < lo3 ? cut.mex : flo.mex;
+            zhi = b2 > hi3 ? cut.min_ : fhi.min_;
+            r1c0 = b2 < lo3 ? cut.cex : flo.cex;
+            r1c1 = b2 > hi3 ? cut.cex + cut.c : fhi.cex + fhi.c;
         }
-        double zlo, zhi;
-        if (r1hi >= r1lo) {
-            zlo = pm[r1lo];
-            zhi = pm[r1hi + 1];
-            if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);
-        } else {
-            zlo = zhi = Z;
-        }
-        int b4lo = find_mass(u * zlo * (1.0 - 1e-9), true), b4hi = find_mass(u * zhi * (1.0 + 1e-9), true);
-        if (b4lo < 0) b4lo = 0;
-        if (b4hi < 0) b4hi = (r1hi >= r1lo) ? r1hi : kTail - 1;
+    }
+    if (r1hi >= kTail) return false;  // the tail has no mass resolution (uniform: every thread has the same records)
+    const double m1lo = zlo;          // mass ranked before range 1
+    if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);  // the top token is always kept
+    // round 2: the bins the draw can land in
+    {
+        const double Tlo = u * zlo * (1.0 - 1e-9), Thi = u * zhi * (1.0 + 1e-9);
+        publish(2u, first_own(Tlo, true));
+        publish(3u, first_own(Thi, true));
+    }
+    __syncthreads();
+    uint32_t c0base, n_r0, c1base = 0, n_r1 = 0;
+    double m0base, m1base = 0.0;
+    {
+        const BinRec dlo = found(2u), dhi = found(3u);
+        int b4lo = dlo.b != 0xffffffffu ? static_cast<int>(dlo.b) : 0;
+        int b4hi = dhi.b != 0xffffffffu ? static_cast<int>(dhi.b) : ((r1hi >= r1lo) ? r1hi : kTail - 1);
         if (b4hi < b4lo) b4hi = b4lo;
-        if (r1hi >= r1lo && b4hi >= r1lo - 1) {
+        // (a bound that was not found by a search has no record: such rows are rare and go the other way)
+        if (dlo.b == 0xffffffffu || dhi.b == 0xffffffffu || static_cast<int>(dhi.b) < b4lo) return false;
+        if (r1hi >= r1lo && b4hi >= r1lo - 1) {  // adjacent or overlapping: one range
             r0lo = min(b4lo, r1lo);
             r0hi = max(b4hi, r1hi);
+            c0base = b4lo <= r1lo ? dlo.cex : r1c0;
+            m0base = b4lo <= r1lo ? dlo.mex : m1lo;
+            n_r0 = (b4hi >= r1hi ? dhi.cex + dhi.c : r1c1) - c0base;
             r1lo = 0;
             r1hi = -1;
         } else {
             r0lo = b4lo;
             r0hi = b4hi;
-        }
-        const bool has_r1 = r1hi >= r1lo;
-        bool ok = !(r0hi >= kTail || r1hi >= kTail);  // the tail has no mass resolution
-        const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
-        ok = ok && nb0 + nb1 <= 8u;
-        LeanSel sel;
-        sel.X = X;
-        sel.Z = Z;
-        sel.r0lo = r0lo, sel.r0hi = r0hi, sel.r1lo = r1lo, sel.r1hi = r1hi;
-        sel.c0base = ok ? pc[r0lo] : 0u;
-        sel.n_r0 = ok ? pc[r0hi + 1] - sel.c0base : 0u;
-        sel.m0base = ok ? pm[r0lo] : 0.0;
-        sel.c1base = ok && has_r1 ? pc[r1lo] : 0u;
-        sel.n_r1 = ok && has_r1 ? pc[r1hi + 1] - sel.c1base : 0u;
-        sel.m1base = ok && has_r1 ? pm[r1lo] : 0.0;
-        ok = ok && sel.n_r0 + sel.n_r1 != 0u && sel.n_r0 <= kLeanMaxRange && sel.n_r1 <= kLeanMaxRange;
-        // masses of a range in units of 2^-52 of the largest mass a token of the range can have
-        auto edge_mass = [&](int b) { return s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001; };
-        const double emax0 = edge_mass(ok ? r0lo : 0), emax1 = ok && has_r1 ? edge_mass(r1lo) : 1.0;
-        sel.scale0 = 4503599627370496.0 / emax0, sel.scale1 = 4503599627370496.0 / emax1;
-        sel.inv0 = emax0 * (1.0 / 4503599627370496.0), sel.inv1 = emax1 * (1.0 / 4503599627370496.0);
-        sel.topp_in_list = topp_in_list, sel.minp_in_list = minp_in_list, sel.ok = ok, sel.pad = 0u;
-        if (lane == 0u) {
-            S.sel = sel;
-            s_w[0] = 0u;
-            s_w[5] = 0u;
+            c0base = dlo.cex;
+            m0base = dlo.mex;
+            n_r0 = dhi.cex + dhi.c - c0base;
+            if (r1hi >= r1lo) {
+                c1base = r1c0;
+                n_r1 = r1c1 - r1c0;
+                m1base = m1lo;
+            }
         }
     }
-    __syncthreads();  // the last reads of pm / pc are done: their LDS is the candidate list from here
-    WSL_MARK(5);
-    if (!S.sel.ok) return false;
-    const int r0lo = S.sel.r0lo, r0hi = S.sel.r0hi, r1lo = S.sel.r1lo, r1hi = S.sel.r1hi;
     const bool has_r1 = r1hi >= r1lo;
+    if (r0hi >= kTail) return false;
     const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
-    const uint32_t c0base = S.sel.c0base, n_r0 = S.sel.n_r0, c1base = S.sel.c1base, n_r1 = S.sel.n_r1;
     const uint32_t n_list = n_r0 + n_r1;
-    const bool topp_in_list = S.sel.topp_in_list != 0u, minp_in_list = S.sel.minp_in_list != 0u;
+    if (nb0 + nb1 > 8u || n_list == 0u || n_r0 > kLeanMaxRange || n_r1 > kLeanMaxRange) return false;
+    // masses of a range in units of 2^-52 of a power of two above the largest mass a token of the range can have
+    const double to_max = s_d[7];
+    auto range_scale = [&](int b, double& scale, double& inv) {
+        const double emax = s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001;
+        const int e = static_cast<int>((static_cast<uint64_t>(__double_as_longlong(emax)) >> 52) & 0x7ffu) - 1022;  // emax < 2^e
+        scale = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 + 52 - e) << 52));
+        inv = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 - 52 + e) << 52));
+    };
+    double scale0, inv0, scale1 = 1.0, inv1 = 1.0;
+    range_scale(r0lo, scale0, inv0);
+    if (has_r1) range_scale(r1lo, scale1, inv1);
+    WSL_MARK(5);
 
     // ------------------------------------------------------------------ the tokens of those bins
     uint2* list = reinterpret_cast<uint2*>(lds + 32768);
@@ -726,26 +806,43 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     {
         LeanHits H;
         const uint32_t* xg = static_cast<const uint32_t*>(rv.base);
-        const uint32_t n_full = nv / WS_BLOCK, rem = nv % WS_BLOCK;
         uint32_t bins[8];
 #pragma unroll
         for (uint32_t k = 0; k < 8u; ++k) bins[k] = k < nb0 ? u0 + k : (k < nb0 + nb1 ? static_cast<uint32_t>(r1lo) + (k - nb0) : u0);
         const uint32_t nt = nb0 + nb1;
         {
+            // cache registers past the row (whole rounds, and the lanes past it in the row's last round) take a byte that
+            // none of the bins asked for has: the scan itself then needs no test of where the row ends
+            uint32_t filler = 0u;
+            for (uint32_t cand_b = 0u; cand_b < 9u; ++cand_b) {  // uniform: one of nine bytes differs from eight
+                bool used = false;
+#pragma unroll
+                for (uint32_t k = 0; k < 8u; ++k) used = used || (bins[k] & 0xffu) == cand_b;
+                if (!used) {
+                    filler = cand_b * 0x01010101u;
+                    break;
+                }
+            }
+            const uint32_t rem = nv % WS_BLOCK;
+#pragma unroll
+            for (int c = 0; c < kLeanRegs; ++c)
+                if (static_cast<uint32_t>(c) >= n_full && (static_cast<uint32_t>(c) > n_full || t >= rem)) cache[c] = filler;
+        }
+        {
             uint32_t c4[4];
 #pragma unroll
             for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[k] & 0xffu) * 0x01010101u;
             const uint32_t n = min(4u, nt);
-            if (n == 1u) lean_scan<1, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
-            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
-            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
-            else lean_scan<4, false>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+            if (n == 1u) lean_scan<1, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
+            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
+            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
+            else lean_scan<4, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
         }
         if (nt > 4u) {  // uniform, rare: a second round for the other bytes, every find through the list
             uint32_t c4[4];
 #pragma unroll
             for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[4u + k] & 0xffu) * 0x01010101u;
-            lean_scan<4, true>(cache, c4, xg, n_full, rem, H, list, &s_w[0], kListCap);
+            lean_scan<4, true>(cache, c4, xg, H, list, &s_w[0], kListCap);
         }
         // touched tokens whose adjusted logit lies in the ranges
         for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
@@ -772,6 +869,13 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     __syncthreads();
     WSL_MARK(6);
     const uint32_t n_hit = s_w[0];
+#ifdef WS_PHASE_TIMERS
+    if (t == 0) {
+        S.marks[12] = nb0 + nb1;
+        S.marks[13] = n_hit;
+        S.marks[14] = n_list;
+    }
+#endif
     if (n_hit > kListCap) return false;
 
     // ------------------------------------------------------------------ the finds that are candidates: a token of another
@@ -837,8 +941,6 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         uint64_t key, fx;
     };
     Place* lb = reinterpret_cast<Place*>(lds);  // [bucket][place]: a candidate's key and its fixed-point mass
-    const double X = S.sel.X, Z = S.sel.Z, m0base = S.sel.m0base, m1base = S.sel.m1base;
-    const double scale0 = S.sel.scale0, scale1 = S.sel.scale1, inv0 = S.sel.inv0, inv1 = S.sel.inv1;
     const float step0 = 64.f / static_cast<float>(nb0), step1 = has_r1 ? 64.f / static_cast<float>(nb1) : 0.f;
     const float lo0 = static_cast<float>(r0lo), lo1 = static_cast<float>(r1lo);
     uint32_t cbkt[kRounds];
@@ -982,66 +1084,74 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         if (dq != ~0ull && static_cast<uint32_t>(r) * WS_BLOCK + t == d_slot) {
             const double mg = fmin(cin[r] - target, d_pos > 0u ? target - cex[r] : 1e300) / Zk;
             uint32_t flags = 0;
+            const double tol = Ap->tol;
             if (mg_top_p < tol) flags |= kNearTopP;
             if (mg_min_p < tol) flags |= kNearMinP;
             if (mg < tol) flags |= kNearDraw;
-            A.token[row] = static_cast<int32_t>(cid[r]);
-            A.flags[row] = flags;
-            if (A.prob) A.prob[row] = static_cast<float>(cem[r] / Zk);
-            if (A.margin) A.margin[3 * row + 2] = mg;
+            Ap->token[row] = static_cast<int32_t>(cid[r]);
+            Ap->flags[row] = flags;
+            if (Ap->prob) Ap->prob[row] = static_cast<float>(cem[r] / Zk);
+            if (Ap->margin) Ap->margin[3 * row + 2] = mg;
         }
     }
     if (t == 0) {
         if (dq == ~0ull) {  // the walk falls through to the last kept candidate (src/sampling/sampler.cpp:131)
+            const double tol = Ap->tol;
             uint32_t flags = kNearDraw;
             if (mg_top_p < tol) flags |= kNearTopP;
             if (mg_min_p < tol) flags |= kNearMinP;
-            A.token[row] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(s_q[4]));
-            A.flags[row] = flags;
-            if (A.prob) A.prob[row] = static_cast<float>(s_d[1] / Zk);
-            if (A.margin) A.margin[3 * row + 2] = 0.0;
+            Ap->token[row] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(s_q[4]));
+            Ap->flags[row] = flags;
+            if (Ap->prob) Ap->prob[row] = static_cast<float>(s_d[1] / Zk);
+            if (Ap->margin) Ap->margin[3 * row + 2] = 0.0;
         }
-        if (A.n_kept) A.n_kept[row] = n3;
-        if (A.stats) {
-            A.stats[2 * row] = m;
-            A.stats[2 * row + 1] = static_cast<float>(Z);
+        if (Ap->n_kept) Ap->n_kept[row] = n3;
+        if (Ap->stats) {
+            Ap->stats[2 * row] = m;
+            Ap->stats[2 * row + 1] = static_cast<float>(Z);
         }
         if (A.margin) {
             A.margin[3 * row] = mg_top_p;
-            A.margin[3 * row + 1] = mg_min_p;
+            Ap->margin[3 * row + 1] = mg_min_p;
         }
     }
     WSL_MARK(10);
 #ifdef WS_PHASE_TIMERS
     __syncthreads();
-    if (t < 16 && A.entropy) A.entropy[row * 16 + t] = static_cast<double>(S.marks[t]);
+    if (t < 16 && Ap->entropy) Ap->entropy[row * 16 + t] = static_cast<double>(S.marks[t]);
 #endif
     return true;
 }
 
-// the three-pass code of ws_sample.h for one row, a function of its own: its registers and code stay out of the lean path
-__device__ __noinline__ void three_pass_row(const BatchArgs A, const uint32_t row) { sample_row<false, false, false>(A, row); }
-
-__global__ void __launch_bounds__(WS_BLOCK) lean_batch_kernel(BatchArgs A) {
-    __shared__ LeanShared shared;
-    const uint32_t row = blockIdx.x;
-#ifdef WS_LEAN_UNMASKED_ONLY
-    const bool done = lean_row<false>(A, row, shared);
-#else
-    const bool done = A.allow ? lean_row<true>(A, row, shared) : lean_row<false>(A, row, shared);
-#endif
-#ifndef WS_LEAN_NO_FALLBACK
-    if (done) return;
-    __syncthreads();  // whatever the lean path left in LDS is dead
-    BatchArgs B = A;
+// the three-pass code of ws_sample.h for one row, a function of its own: its registers and code stay out of the lean path.
+// It takes the kernel's argument segment and makes its own copy of the arguments with the three-pass layout of the LDS
+// (a copy made by the kernel would be made at the kernel's entry, on every row).
+typedef const __attribute__((address_space(4))) BatchArgs* LeanArgPtr;
+__device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
+    BatchArgs B;
+    __builtin_memcpy(&B, (const void*)Ap, sizeof(BatchArgs));
     B.lds_ab = 65536u;
     B.lds_cnt = 0u;
-    B.lds_tie = A.fb_lds_tie;
+    B.lds_tie = B.fb_lds_tie;
     B.two_sweep = 1;
     B.work = nullptr;
     B.split_log2 = 0u;
-    three_pass_row(B, row);
-    if (threadIdx.x == 0) A.flags[row] |= kRouteHandedBack;
+    sample_row<false, false, false>(B, row);
+    if (threadIdx.x == 0) B.flags[row] |= kRouteHandedBack;
+}
+
+// MASKED: the batch has an allow mask (a kernel of its own: one build carrying both paths spilled far more registers)
+template <bool MASKED>
+__global__ void __launch_bounds__(WS_BLOCK) lean_batch_kernel(BatchArgs A) {
+    __shared__ LeanShared shared;
+    const uint32_t row = blockIdx.x;
+    const bool done = lean_row<MASKED>(A, row, shared);
+#ifndef WS_LEAN_NO_FALLBACK
+    if (done) return;
+    __syncthreads();  // whatever the lean path left in LDS is dead
+    LeanArgPtr Ap = (LeanArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(Ap));
+    three_pass_row(Ap, row);
 #else
     if (!done && threadIdx.x == 0) A.token[row] = -2;
 #endif

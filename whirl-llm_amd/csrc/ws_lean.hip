@@ -14,9 +14,10 @@ int prepare_lean(unsigned lds_limit) {
     if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
     const uint64_t bit = 1ull << (dev & 63);
     if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&lean_batch_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 static_cast<int>(lds_limit));
-        if (e != hipSuccess) return static_cast<int>(e);
+        for (const void* f : {reinterpret_cast<const void*>(&lean_batch_kernel<false>), reinterpret_cast<const void*>(&lean_batch_kernel<true>)}) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_limit));
+            if (e != hipSuccess) return static_cast<int>(e);
+        }
         attr_set.fetch_or(bit, std::memory_order_release);
     }
     return 0;
@@ -24,7 +25,11 @@ int prepare_lean(unsigned lds_limit) {
 
 int launch_lean(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit) {
     if (const int e = prepare_lean(lds_limit); e != 0) return e;
-    hipLaunchKernelGGL(lean_batch_kernel, dim3(rows), dim3(WS_BLOCK), lds_bytes, stream, a);
+#ifndef WS_LEAN_UNMASKED_ONLY
+    if (a.allow) hipLaunchKernelGGL(lean_batch_kernel<true>, dim3(rows), dim3(WS_BLOCK), lds_bytes, stream, a);
+    else
+#endif
+        hipLaunchKernelGGL(lean_batch_kernel<false>, dim3(rows), dim3(WS_BLOCK), lds_bytes, stream, a);
     return static_cast<int>(hipGetLastError());
 }
 
