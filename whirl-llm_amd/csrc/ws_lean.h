@@ -15,6 +15,7 @@
 //     them at once as well: a candidate adds its fixed-point mass to one of 64 buckets per range, finds its rank and its
 //     running mass among the few members of its bucket, and tests the cut and the draw on itself.
 #pragma once
+#include <type_traits>
 
 #include "ws_sample.h"
 
@@ -68,14 +69,25 @@ struct LeanHits {
 // TO_LIST every find goes there (a second round of bytes).
 template <int NT, bool TO_LIST>
 __device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const uint32_t* __restrict__ xg, LeanHits& H,
-                                          uint2* list, uint32_t* n_list, uint32_t cap) {
+                                          uint2* list, uint32_t* n_list, uint32_t cap, uint32_t nv) {
     const uint32_t t = threadIdx.x;
 #pragma unroll
     for (int g = 0; g < kLeanGroups; ++g) {
+        // where the row ends (nv: its 128-bit vectors) is looked at per group, uniformly: a group past the row is skipped,
+        // the one group the end falls in masks its finds, the others need no test
         uint32_t acc = 0;
+        const uint32_t g_lo = static_cast<uint32_t>(g * 8) * WS_BLOCK;
+        if (g_lo + 8u * WS_BLOCK <= nv) {
 #pragma unroll
-        for (int r = 0; r < 8; ++r)  // bit 8 e + r: token e of register r (registers past the row hold a byte nobody asks for)
-            acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & (0x01010101u << r)) | acc;
+            for (int r = 0; r < 8; ++r)  // bit 8 e + r: token e of register r
+                acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & (0x01010101u << r)) | acc;
+        } else if (g_lo < nv) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t keep = g_lo + static_cast<uint32_t>(r) * WS_BLOCK + t < nv ? 0x01010101u << r : 0u;
+                acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & keep) | acc;
+            }
+        }
         auto token_of = [&](uint32_t bit) { return ((static_cast<uint32_t>(g * 8 + (bit & 7u)) * WS_BLOCK + t) << 2) + (bit >> 3); };
         if (!TO_LIST) {
             H.idx[g] = H.idx[kLeanGroups + g] = 0xffffffffu;
@@ -119,6 +131,31 @@ __device__ __forceinline__ double exp_neg(double a, const double* s_exp) {
     return s_exp[n >> 6] * s_exp[64u + (n & 63u)] * p;
 }
 
+// One of four values by number. The values come in as arguments, every one of them read before the choice: a chain
+// of conditional reads of an array's elements is turned into one read at a computed index, and the array into memory.
+template <typename T>
+__device__ __forceinline__ T pick4(uint32_t k, T a0, T a1, T a2, T a3) {
+    const T lo = k & 1u ? a1 : a0, hi = k & 1u ? a3 : a2;
+    return k & 2u ? hi : lo;
+}
+
+// a row's parameters as the scalar loads at the top of lean_row leave them
+struct LeanRowParams {
+    double top_p, min_p;
+    uint64_t seed, step;
+    float inv_t, rep, pres, freq;
+    uint32_t top_k, h0, nh, b0, nb;
+    bool race;
+};
+
+// what wave 0 works out from the searches' answers for everybody
+struct LeanSel {
+    double X, m0base, m1base, scale0, scale1, inv0, inv1;
+    int r0lo, r0hi, r1lo, r1hi;
+    uint32_t c0base, n_r0, c1base, n_r1;
+    uint32_t topp_in_list, minp_in_list, ok, pad;
+};
+
 // a bin as the select's searches hand it round: mass ranked before it and up to and with it, tokens before it and in it
 struct LeanBinRec {
     double mex, min_;
@@ -129,7 +166,8 @@ struct LeanBinRec {
 struct LeanShared {
     double s_exp[128];  // kExpHi, kExpLo
     double red_d[WS_WAVES];
-    double s_d[8];
+    double s_d[10];
+    LeanSel sel;
     LeanBinRec rec[4 * WS_WAVES + 2];  // [search][wave], then the two bins named outright
     unsigned long long s_q[6];
     unsigned long long b_mass[kLeanBuckets], b_fpre[kLeanBuckets];
@@ -138,7 +176,7 @@ struct LeanShared {
     uint32_t red_u[WS_WAVES];
     float red_f[WS_WAVES];
 #ifdef WS_PHASE_TIMERS
-    long long marks[16];
+    long long marks[32];
 #endif
 };
 
@@ -147,7 +185,7 @@ template <bool MASKED>
 __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row, LeanShared& S) {
 #ifdef WS_PHASE_TIMERS
     const long long wsl_t0 = clock64();  // debug builds: the marks go to LDS, and at the end to `entropy`, 16 doubles a row
-    if (threadIdx.x < 16) S.marks[threadIdx.x] = 0;
+    if (threadIdx.x < 32) S.marks[threadIdx.x] = 0;
 #endif
     extern __shared__ __align__(16) unsigned char lds[];
     float* red_f = S.red_f;
@@ -211,16 +249,66 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     if (hist2)
         for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
 
-    const float inv_t = A.inv_t[row];
-    const uint32_t top_k = A.top_k ? A.top_k[row] : 0u;
-    const bool race = A.race != nullptr && A.race[row] != 0;
-    bool use_top_p, use_min_p;
+    // The row's parameters, every one of them with one scalar load, all asked for together and waited for once. (Written
+    // as plain reads they become vector loads, each behind the test of its pointer and each waited for on its own: a
+    // dozen trips to memory one after the other, here and again behind the sweep.) An absent array is read at the
+    // kernel's argument segment instead and the value dropped.
+    LeanRowParams P;
     {
-        const double top_p0 = A.top_p ? A.top_p[row] : 1.0, min_p0 = A.min_p ? A.min_p[row] : 0.0;  // (both are read again behind the sweep)
-        use_top_p = top_p0 < 1.0, use_min_p = min_p0 > 0.0;
+        const uint64_t dummy = reinterpret_cast<uint64_t>((const __attribute__((address_space(4))) void*)__builtin_amdgcn_kernarg_segment_ptr());
+        auto at = [&](const void* base, uint64_t byte_off) { return base ? reinterpret_cast<uint64_t>(base) + byte_off : dummy; };
+        const uint64_t r4 = static_cast<uint64_t>(row) * 4u, r8 = static_cast<uint64_t>(row) * 8u;
+        const uint64_t p_inv_t = at(A.inv_t, r4), p_top_k = at(A.top_k, r4), p_race = at(A.race, r4), p_top_p = at(A.top_p, r8), p_min_p = at(A.min_p, r8);
+        // (the history's length: its own array, or else the next row's offset - which an offsets array with lengths beside it need not have)
+        const uint64_t p_hoff = at(A.hist ? A.hist_off : nullptr, r4);
+        const uint64_t p_hlen = A.hist ? (A.hist_len ? at(A.hist_len, r4) : at(A.hist_off, r4 + 4u)) : dummy;
+        const uint64_t p_boff = at(A.bias_ids ? A.bias_off : nullptr, r4), p_seed = at(A.seed, r8), p_step = at(A.step, r8);
+        const uint64_t p_rep = at(A.rep, r4), p_pres = at(A.pres, r4), p_freq = at(A.freq, r4);
+        uint32_t v_inv_t, v_top_k, v_race, v_hoff, v_hlen, v_rep, v_pres, v_freq;
+        uint64_t v_top_p, v_min_p, v_boff, v_seed, v_step;
+        asm volatile(
+            "s_load_dword %0, %13, 0x0\n\t"
+            "s_load_dword %1, %14, 0x0\n\t"
+            "s_load_dword %2, %15, 0x0\n\t"
+            "s_load_dwordx2 %3, %16, 0x0\n\t"
+            "s_load_dwordx2 %4, %17, 0x0\n\t"
+            "s_load_dword %5, %18, 0x0\n\t"
+            "s_load_dword %6, %19, 0x0\n\t"
+            "s_load_dwordx2 %7, %20, 0x0\n\t"
+            "s_load_dwordx2 %8, %21, 0x0\n\t"
+            "s_load_dwordx2 %9, %22, 0x0\n\t"
+            "s_load_dword %10, %23, 0x0\n\t"
+            "s_load_dword %11, %24, 0x0\n\t"
+            "s_load_dword %12, %25, 0x0\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&s"(v_inv_t), "=&s"(v_top_k), "=&s"(v_race), "=&s"(v_top_p), "=&s"(v_min_p), "=&s"(v_hoff), "=&s"(v_hlen), "=&s"(v_boff),
+              "=&s"(v_seed), "=&s"(v_step), "=&s"(v_rep), "=&s"(v_pres), "=&s"(v_freq)
+            : "s"(p_inv_t), "s"(p_top_k), "s"(p_race), "s"(p_top_p), "s"(p_min_p), "s"(p_hoff), "s"(p_hlen), "s"(p_boff), "s"(p_seed),
+              "s"(p_step), "s"(p_rep), "s"(p_pres), "s"(p_freq)
+            : "memory");
+        P.inv_t = __uint_as_float(v_inv_t);
+        P.top_k = A.top_k ? v_top_k : 0u;
+        P.race = A.race != nullptr && v_race != 0u;
+        P.top_p = A.top_p ? __longlong_as_double(static_cast<long long>(v_top_p)) : 1.0;
+        P.min_p = A.min_p ? __longlong_as_double(static_cast<long long>(v_min_p)) : 0.0;
+        P.h0 = A.hist ? v_hoff : 0u;
+        P.nh = A.hist ? (A.hist_len ? v_hlen : v_hlen - P.h0) : 0u;
+        P.b0 = A.bias_ids ? static_cast<uint32_t>(v_boff) : 0u;
+        P.nb = A.bias_ids ? static_cast<uint32_t>(v_boff >> 32) - P.b0 : 0u;
+        P.seed = v_seed;
+        P.step = v_step;
+        P.rep = A.rep ? __uint_as_float(v_rep) : 1.f;
+        P.pres = A.pres ? __uint_as_float(v_pres) : 0.f;
+        P.freq = A.freq ? __uint_as_float(v_freq) : 0.f;
     }
-    const uint32_t h0 = A.hist ? A.hist_off[row] : 0u, nh = A.hist ? (A.hist_len ? A.hist_len[row] : A.hist_off[row + 1] - h0) : 0u;
-    const uint32_t b0 = A.bias_ids ? A.bias_off[row] : 0u, nb = A.bias_ids ? A.bias_off[row + 1] - b0 : 0u;
+    const float inv_t = P.inv_t;
+    const uint32_t top_k = P.top_k;
+    const bool race = P.race;
+    const double top_p = P.top_p, min_p = P.min_p;
+    const bool use_top_p = top_p < 1.0, use_min_p = min_p > 0.0;
+    double neg_log_min_p = 0.0;  // wave 15 only (for the select, which has no time for a logarithm)
+    if (wv == WS_WAVES - 1u && use_min_p) neg_log_min_p = -log(min_p);
+    const uint32_t h0 = P.h0, nh = P.nh, b0 = P.b0, nb = P.nb;
     // rows this code does not take: a top-k, no filter at all, the race draw, parameters the three-pass code reports
     if (top_k != 0u || !(use_top_p || use_min_p) || race || !(inv_t > 0.f) || nh + nb > A.patch_cap) return false;
 
@@ -233,8 +321,11 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
     const uint32_t bid = t < nb ? static_cast<uint32_t>(bias_ids[t]) : 0xffffffffu;  // the first bias ids
     if (wv == WS_WAVES - 1u) {  // one wave draws the row's uniform for everybody
-        const double u_ = batch_uniform(A.rng, A.seed[row], row, A.step[row], 0);
-        if (lane == 0u) s_d[6] = u_;
+        const double u_ = batch_uniform(A.rng, P.seed, row, P.step, 0);
+        if (lane == 0u) {
+            s_d[6] = u_;
+            s_d[8] = neg_log_min_p;
+        }
     }
     WSL_MARK(0);
 
@@ -283,12 +374,16 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         _Pragma("unroll") for (int u = 0; u < kLeanBatch; ++u) {                                                                     \
             const uint32_t j = ((bt) * kLeanBatch + u) * WS_BLOCK + t;                                                               \
             const int c = (bt) * kLeanBatch + u;                                                                                     \
-            uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};                                                \
             uint32_t tw = (early) ? 0u : tws[(bt) & 1][u], nal = MASKED ? ~na[slot][u] : 0u;                                         \
-            if (static_cast<uint32_t>(c) >= n_full && j >= nv) { /* (only the row's last round has lanes past it) NaN: the tail bins */ \
-                w[0] = w[1] = w[2] = w[3] = 0xffffffffu;                                                                             \
-                tw = 0u;                                                                                                             \
+            if (static_cast<uint32_t>(c) >= n_full) { /* uniform: only the row's last round has lanes past it */                      \
+                const bool past = j >= nv;            /* NaN: the tail bins, nobody's candidate (in place: no copy of the vector) */  \
+                q[slot][u].x = past ? 0xffffffffu : q[slot][u].x;                                                                    \
+                q[slot][u].y = past ? 0xffffffffu : q[slot][u].y;                                                                    \
+                q[slot][u].z = past ? 0xffffffffu : q[slot][u].z;                                                                    \
+                q[slot][u].w = past ? 0xffffffffu : q[slot][u].w;                                                                    \
+                tw = past ? 0u : tw;                                                                                                 \
             }                                                                                                                        \
+            const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};                                          \
             const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * 4u) & 31u)) : 0;                                           \
             uint32_t bins[4];                                                                                                        \
             float vm = -INFINITY;                                                                                                    \
@@ -444,9 +539,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     typedef const __attribute__((address_space(4))) BatchArgs* ArgPtr;
     ArgPtr Ap = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile("" : "+s"(Ap));
-    const double top_p = Ap->top_p ? Ap->top_p[row] : 1.0;
-    const double min_p = Ap->min_p ? Ap->min_p[row] : 0.0;
-    const float rep = Ap->rep ? Ap->rep[row] : 1.f, pres = Ap->pres ? Ap->pres[row] : 0.f, freq = Ap->freq ? Ap->freq[row] : 0.f;
+    const float rep = P.rep, pres = P.pres, freq = P.freq;
     const int32_t* hist_ids2 = Ap->hist + h0;
     const int32_t* bias_ids2 = Ap->bias_ids + b0;
     const float* bias_vals2 = Ap->bias_vals + b0;
@@ -460,25 +553,28 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         const uint32_t whole_end = V & ~3u;
         const float tail_own = own_tail();
         const uint32_t stage_cap = 2047u;
-        auto take4 = [&](const int32_t* ids, uint32_t n, bool in_regs) {
-            for (uint32_t j0 = 0; j0 < n; j0 += 4u * WS_BLOCK) {
-                uint32_t id[4], al[4], tw[4], wp[4], rk[4], old[4];
-                uint4 vec[4];
+        // K ids a thread and pass (a pass with nothing in its later slots would still issue their instructions)
+        auto take = [&](auto kc, const int32_t* ids, uint32_t n, uint32_t j0, const uint32_t* kept_id) __attribute__((always_inline)) {
+            constexpr int K = decltype(kc)::value;
+            if (j0 + wv * 64u < n) {  // (per wave: one with no id left issues nothing, and the others have the SIMDs to themselves)
+                uint32_t id[K], al[K], tw[K], wp[K], rk[K], old[K];
+                uint4 vec[K];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
+                for (int k = 0; k < K; ++k) {
                     const uint32_t j = j0 + k * WS_BLOCK + t;
-                    id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;  // (read again: the sweep has the registers)
+                    if (K == 1 && kept_id != nullptr) id[k] = *kept_id;  // (the one id that stayed in a register through the sweep)
+                    else id[k] = j < n ? static_cast<uint32_t>(ids[j]) : 0xffffffffu;  // (read again: the sweep has the registers)
                     if (id[k] >= V) id[k] = 0xffffffffu;
                 }
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
+                for (int k = 0; k < K; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
                     al[k] = MASKED ? rv.allow[i >> 5] : 0xffffffffu;
                     tw[k] = touched[i >> 5];
                     wp[k] = wprefix[i >> 5];
                 }
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
+                for (int k = 0; k < K; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
                     const uint32_t vb = i & ~3u;
                     const uint32_t rf = id[k] < V ? wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u)) : 0u;
@@ -493,7 +589,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     }
                 }
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
+                for (int k = 0; k < K; ++k) {
                     if (old[k] & kClaim) continue;
                     const uint32_t i = id[k];
                     const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
@@ -528,8 +624,17 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 }
             }
         };
-        take4(hist_ids2, nh, true);
-        take4(bias_ids2, nb, false);
+        auto take_all = [&](const int32_t* ids, uint32_t n, const uint32_t* first_id) __attribute__((always_inline)) {
+            if (n <= WS_BLOCK) {  // (the usual case: one id a thread, and that one is at hand)
+                if (n) take(std::integral_constant<int, 1>{}, ids, n, 0u, first_id);
+                return;
+            }
+            uint32_t j0 = 0;
+            for (; j0 + WS_BLOCK < n; j0 += 4u * WS_BLOCK) take(std::integral_constant<int, 4>{}, ids, n, j0, nullptr);
+            if (j0 < n) take(std::integral_constant<int, 1>{}, ids, n, j0, nullptr);
+        };
+        take_all(hist_ids2, nh, &hid[0]);
+        take_all(bias_ids2, nb, &bid);
     }
     WSL_MARK(3);
     {
@@ -567,7 +672,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             ms[k] = 0.0;
             lc += c4b[k];
         }
-        if (__ballot(lc != 0u)) {  // uniform: a wave whose 256 bins hold no token needs no arithmetic
+        const bool wave_has = __ballot(lc != 0u) != 0ull;
+        if (wave_has) {  // uniform: a wave whose 256 bins hold no token needs no arithmetic
             const double eh = s_exp[bb >> 6];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -576,22 +682,25 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 ms[k] = c4b[k] ? eh * s_exp[64 + ((bb + k) & 63u)] * (static_cast<double>(c4b[k]) - fix) : 0.0;
             }
         }
-        const uint32_t ic = wave_incl_scan(lc);
+        const uint32_t ic = wave_has ? wave_incl_scan(lc) : 0u;
         __syncthreads();  // the factor is in place (and every read of the histogram is done)
         const double to_max = s_d[7];
-        double lm = 0.0;
+        double lm = 0.0, im = 0.0, up = 0.0;
+        if (wave_has) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            ms[k] *= to_max;
-            lm += ms[k];
+            for (int k = 0; k < 4; ++k) {
+                ms[k] *= to_max;
+                lm += ms[k];
+            }
+            im = wave_incl_scan(lm);
+            up = __shfl_up(im, 1);
         }
-        const double im = wave_incl_scan(lm);
-        const double up = __shfl_up(im, 1);
         if (lane == 63u) {
             red_u[wv] = ic;
             red_d[wv] = im;
         }
         __syncthreads();
+        WSL_MARK(16);
         // the waves' totals, scanned by every wave again: lane w holds wave w's
         const uint32_t wc = lane < WS_WAVES ? red_u[lane] : 0u;
         const double wm = lane < WS_WAVES ? red_d[lane] : 0.0;
@@ -641,10 +750,10 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         } else if (lane == static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(any)) - 1)) {
             BinRec r;
             r.b = bb + k;
-            r.mex = k == 0u ? me[0] : (k == 1u ? me[1] : (k == 2u ? me[2] : me[3]));
-            r.min_ = k == 0u ? me[1] : (k == 1u ? me[2] : (k == 2u ? me[3] : me[4]));
-            r.cex = k == 0u ? ce[0] : (k == 1u ? ce[1] : (k == 2u ? ce[2] : ce[3]));
-            r.c = k == 0u ? c4b[0] : (k == 1u ? c4b[1] : (k == 2u ? c4b[2] : c4b[3]));
+            r.mex = pick4(k, me[0], me[1], me[2], me[3]);
+            r.min_ = pick4(k, me[1], me[2], me[3], me[4]);
+            r.cex = pick4(k, ce[0], ce[1], ce[2], ce[3]);
+            r.c = pick4(k, c4b[0], c4b[1], c4b[2], c4b[3]);
             r.pad = 0u;
             rec[search * WS_WAVES + wv] = r;
         }
@@ -665,26 +774,25 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             const uint32_t k = static_cast<uint32_t>(b) & 3u;
             BinRec r;
             r.b = static_cast<uint32_t>(b);
-            r.mex = k == 0u ? me[0] : (k == 1u ? me[1] : (k == 2u ? me[2] : me[3]));
-            r.min_ = k == 0u ? me[1] : (k == 1u ? me[2] : (k == 2u ? me[3] : me[4]));
-            r.cex = k == 0u ? ce[0] : (k == 1u ? ce[1] : (k == 2u ? ce[2] : ce[3]));
-            r.c = k == 0u ? c4b[0] : (k == 1u ? c4b[1] : (k == 2u ? c4b[2] : c4b[3]));
+            r.mex = pick4(k, me[0], me[1], me[2], me[3]);
+            r.min_ = pick4(k, me[1], me[2], me[3], me[4]);
+            r.cex = pick4(k, ce[0], ce[1], ce[2], ce[3]);
+            r.c = pick4(k, c4b[0], c4b[1], c4b[2], c4b[3]);
             r.pad = 0u;
             rec[4u * WS_WAVES + (search - 4u)] = r;
         }
     };
-    int r0lo = 0, r0hi = -1, r1lo = 0, r1hi = -1;
-    bool minp_in_list = false, topp_in_list = false;
-    double X = 0;
-    const double u = s_d[6];
+    // The searches are every wave's work; what follows from their answers is worked out by wave 0 alone and handed
+    // round through LDS (sixteen waves doing the same arithmetic side by side take four times as long as one).
+    LeanSel& sel = S.sel;
+    // round 1: the top-p cut against the float normaliser and against the exact one; the min-p bins by name
     int lo3 = kBins, hi3 = -1;
     if (use_min_p) {
-        const double astar = (-log(min_p) + lift) * 64.0;
+        const double astar = (s_d[8] + lift) * 64.0;
         const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
         lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
         hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
     }
-    // round 1: the top-p cut against the float normaliser and against the exact one; the min-p bins by name
     if (use_top_p) {
         const double Xf = top_p * Zf, Xz = top_p * Z;
         publish(0u, Xf > 0.0 ? first_own(Xf, false) : 4u);
@@ -694,17 +802,19 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         publish_bin(4u, min(lo3, kTail - 1));
         publish_bin(5u, min(hi3, kTail - 1));
     }
-    if (t == 0) {
-        s_w[0] = 0u;
-        s_w[5] = 0u;
-    }
+    WSL_MARK(17);
     __syncthreads();
-    double zlo = Z, zhi = Z;       // bounds of the kept mass
-    uint32_t r1c0 = 0, r1c1 = 0;   // tokens ranked before range 1, and up to and with its last bin
-    {
+    WSL_MARK(15);
+    if (wv == 0u) {
+        int r1lo = 0, r1hi = -1;
+        bool minp_in_list = false, topp_in_list = false;
+        double X = 0, zlo = Z, zhi = Z;  // zlo, zhi: bounds of the kept mass
+        uint32_t r1c0 = 0, r1c1 = 0;     // tokens ranked before range 1, and up to and with its last bin
         int b2 = -1;
         BinRec cut;
         cut.b = 0xffffffffu;
+        cut.mex = cut.min_ = 0.0;
+        cut.cex = cut.c = cut.pad = 0u;
         if (use_top_p) {
             X = top_p * Zf;
             cut = found(0u);
@@ -735,26 +845,41 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             r1c0 = b2 < lo3 ? cut.cex : flo.cex;
             r1c1 = b2 > hi3 ? cut.cex + cut.c : fhi.cex + fhi.c;
         }
-    }
-    if (r1hi >= kTail) return false;  // the tail has no mass resolution (uniform: every thread has the same records)
-    const double m1lo = zlo;          // mass ranked before range 1
-    if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);  // the top token is always kept
-    // round 2: the bins the draw can land in
-    {
-        const double Tlo = u * zlo * (1.0 - 1e-9), Thi = u * zhi * (1.0 + 1e-9);
-        publish(2u, first_own(Tlo, true));
-        publish(3u, first_own(Thi, true));
+        const double m1lo = zlo;                           // mass ranked before range 1
+        if (r1lo == 0 && zlo < 1.0) zlo = fmin(1.0, zhi);  // the top token is always kept
+        if (lane == 0u) {
+            sel.X = X;
+            sel.m1base = m1lo;
+            sel.r1lo = r1lo, sel.r1hi = r1hi;
+            sel.c1base = r1c0, sel.n_r1 = r1c1;  // (until the second round: tokens before range 1, and up to and with it)
+            sel.topp_in_list = topp_in_list, sel.minp_in_list = minp_in_list;
+            sel.ok = r1hi < kTail;               // the tail has no mass resolution
+            const double u = s_d[6];
+            s_d[4] = u * zlo * (1.0 - 1e-9);     // round 2: the bins the draw can land in
+            s_d[5] = u * zhi * (1.0 + 1e-9);
+            s_w[0] = 0u;
+            s_w[5] = 0u;
+        }
     }
     __syncthreads();
-    uint32_t c0base, n_r0, c1base = 0, n_r1 = 0;
-    double m0base, m1base = 0.0;
-    {
+    if (!sel.ok) return false;
+    publish(2u, first_own(s_d[4], true));
+    publish(3u, first_own(s_d[5], true));
+    WSL_MARK(18);
+    __syncthreads();
+    WSL_MARK(19);
+    if (wv == 0u) {
+        int r0lo = 0, r0hi = -1, r1lo = sel.r1lo, r1hi = sel.r1hi;
+        const uint32_t r1c0 = sel.c1base, r1c1 = sel.n_r1;
+        const double m1lo = sel.m1base;
+        uint32_t c0base = 0, n_r0 = 0, c1base = 0, n_r1 = 0;
+        double m0base = 0.0, m1base = 0.0;
         const BinRec dlo = found(2u), dhi = found(3u);
-        int b4lo = dlo.b != 0xffffffffu ? static_cast<int>(dlo.b) : 0;
+        const int b4lo = dlo.b != 0xffffffffu ? static_cast<int>(dlo.b) : 0;
         int b4hi = dhi.b != 0xffffffffu ? static_cast<int>(dhi.b) : ((r1hi >= r1lo) ? r1hi : kTail - 1);
         if (b4hi < b4lo) b4hi = b4lo;
         // (a bound that was not found by a search has no record: such rows are rare and go the other way)
-        if (dlo.b == 0xffffffffu || dhi.b == 0xffffffffu || static_cast<int>(dhi.b) < b4lo) return false;
+        bool ok = !(dlo.b == 0xffffffffu || dhi.b == 0xffffffffu || static_cast<int>(dhi.b) < b4lo);
         if (r1hi >= r1lo && b4hi >= r1lo - 1) {  // adjacent or overlapping: one range
             r0lo = min(b4lo, r1lo);
             r0hi = max(b4hi, r1hi);
@@ -775,23 +900,38 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 m1base = m1lo;
             }
         }
+        const bool has_r1 = r1hi >= r1lo;
+        const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+        ok = ok && r0hi < kTail && nb0 + nb1 <= 8u && n_r0 + n_r1 != 0u && n_r0 <= kLeanMaxRange && n_r1 <= kLeanMaxRange;
+        // masses of a range in units of 2^-52 of a power of two above the largest mass a token of the range can have
+        const double to_max = s_d[7];
+        auto range_scale = [&](int b, double& scale, double& inv) {
+            const double emax = s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001;
+            const int e = static_cast<int>((static_cast<uint64_t>(__double_as_longlong(emax)) >> 52) & 0x7ffu) - 1022;  // emax < 2^e
+            scale = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 + 52 - e) << 52));
+            inv = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 - 52 + e) << 52));
+        };
+        double scale0 = 1.0, inv0 = 1.0, scale1 = 1.0, inv1 = 1.0;
+        if (ok) range_scale(r0lo, scale0, inv0);
+        if (ok && has_r1) range_scale(r1lo, scale1, inv1);
+        if (lane == 0u) {
+            sel.r0lo = r0lo, sel.r0hi = r0hi, sel.r1lo = r1lo, sel.r1hi = r1hi;
+            sel.c0base = c0base, sel.n_r0 = n_r0, sel.c1base = c1base, sel.n_r1 = n_r1;
+            sel.m0base = m0base, sel.m1base = m1base;
+            sel.scale0 = scale0, sel.inv0 = inv0, sel.scale1 = scale1, sel.inv1 = inv1;
+            sel.ok = ok;
+        }
     }
+    __syncthreads();
+    if (!sel.ok) return false;
+    const int r0lo = sel.r0lo, r0hi = sel.r0hi, r1lo = sel.r1lo, r1hi = sel.r1hi;
     const bool has_r1 = r1hi >= r1lo;
-    if (r0hi >= kTail) return false;
     const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
+    const uint32_t c0base = sel.c0base, n_r0 = sel.n_r0, c1base = sel.c1base, n_r1 = sel.n_r1;
     const uint32_t n_list = n_r0 + n_r1;
-    if (nb0 + nb1 > 8u || n_list == 0u || n_r0 > kLeanMaxRange || n_r1 > kLeanMaxRange) return false;
-    // masses of a range in units of 2^-52 of a power of two above the largest mass a token of the range can have
-    const double to_max = s_d[7];
-    auto range_scale = [&](int b, double& scale, double& inv) {
-        const double emax = s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001;
-        const int e = static_cast<int>((static_cast<uint64_t>(__double_as_longlong(emax)) >> 52) & 0x7ffu) - 1022;  // emax < 2^e
-        scale = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 + 52 - e) << 52));
-        inv = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 - 52 + e) << 52));
-    };
-    double scale0, inv0, scale1 = 1.0, inv1 = 1.0;
-    range_scale(r0lo, scale0, inv0);
-    if (has_r1) range_scale(r1lo, scale1, inv1);
+    const bool topp_in_list = sel.topp_in_list != 0u, minp_in_list = sel.minp_in_list != 0u;
+    const double X = sel.X, m0base = sel.m0base, m1base = sel.m1base;
+    const double scale0 = sel.scale0, inv0 = sel.inv0, scale1 = sel.scale1, inv1 = sel.inv1;
     WSL_MARK(5);
 
     // ------------------------------------------------------------------ the tokens of those bins
@@ -811,39 +951,22 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         for (uint32_t k = 0; k < 8u; ++k) bins[k] = k < nb0 ? u0 + k : (k < nb0 + nb1 ? static_cast<uint32_t>(r1lo) + (k - nb0) : u0);
         const uint32_t nt = nb0 + nb1;
         {
-            // cache registers past the row (whole rounds, and the lanes past it in the row's last round) take a byte that
-            // none of the bins asked for has: the scan itself then needs no test of where the row ends
-            uint32_t filler = 0u;
-            for (uint32_t cand_b = 0u; cand_b < 9u; ++cand_b) {  // uniform: one of nine bytes differs from eight
-                bool used = false;
-#pragma unroll
-                for (uint32_t k = 0; k < 8u; ++k) used = used || (bins[k] & 0xffu) == cand_b;
-                if (!used) {
-                    filler = cand_b * 0x01010101u;
-                    break;
-                }
-            }
-            const uint32_t rem = nv % WS_BLOCK;
-#pragma unroll
-            for (int c = 0; c < kLeanRegs; ++c)
-                if (static_cast<uint32_t>(c) >= n_full && (static_cast<uint32_t>(c) > n_full || t >= rem)) cache[c] = filler;
-        }
-        {
             uint32_t c4[4];
 #pragma unroll
             for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[k] & 0xffu) * 0x01010101u;
             const uint32_t n = min(4u, nt);
-            if (n == 1u) lean_scan<1, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
-            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
-            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
-            else lean_scan<4, false>(cache, c4, xg, H, list, &s_w[0], kListCap);
+            if (n == 1u) lean_scan<1, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else lean_scan<4, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
         }
         if (nt > 4u) {  // uniform, rare: a second round for the other bytes, every find through the list
             uint32_t c4[4];
 #pragma unroll
             for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[4u + k] & 0xffu) * 0x01010101u;
-            lean_scan<4, true>(cache, c4, xg, H, list, &s_w[0], kListCap);
+            lean_scan<4, true>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
         }
+        WSL_MARK(20);
         // touched tokens whose adjusted logit lies in the ranges
         for (uint32_t r = t; r < n_touched; r += WS_BLOCK) {
             const float x = pv[r];
@@ -852,6 +975,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 if (slot < kListCap) list[slot] = make_uint2(first[r] | kListAdjusted, __float_as_uint(x));
             }
         }
+        WSL_MARK(21);
         uint32_t mine = 0;
 #pragma unroll
         for (int k = 0; k < 2 * kLeanGroups; ++k) mine += H.idx[k] != 0xffffffffu ? 1u : 0u;
@@ -866,6 +990,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             ++slot;
         }
     }
+    WSL_MARK(22);
     __syncthreads();
     WSL_MARK(6);
     const uint32_t n_hit = s_w[0];
@@ -891,7 +1016,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
-            if (static_cast<uint32_t>(r) * WS_BLOCK >= n_hit) continue;  // uniform
+            if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u >= n_hit) continue;  // per wave
             const bool live = en[r].x != 0xffffffffu;
             const uint32_t id = live ? en[r].x & kListIdMask : 0u;
             float x = __uint_as_float(en[r].y);
@@ -948,7 +1073,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     double cem[kRounds];
 #pragma unroll
     for (int r = 0; r < kRounds; ++r) {
-        if (static_cast<uint32_t>(r) * WS_BLOCK >= n_list) continue;  // uniform
+        if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u >= n_list) continue;  // per wave
         const float x = cx[r];
         const float tc = bin_coord(aq, c64, x);
         const bool in1 = has_r1 && static_cast<uint32_t>(tc) - static_cast<uint32_t>(r1lo) < nb1;
@@ -994,7 +1119,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     for (int r = 0; r < kRounds; ++r) {
         cpos[r] = 0xffffffffu;
         cin[r] = cex[r] = 0.0;
-        if (static_cast<uint32_t>(r) * WS_BLOCK >= n_list) continue;  // uniform
+        if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u >= n_list) continue;  // per wave
         const uint32_t bkt = con[r] ? cbkt[r] : 0u;
         const uint32_t n = con[r] ? b_cnt[bkt] : 0u;
         uint32_t rank = 0;
@@ -1118,7 +1243,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     WSL_MARK(10);
 #ifdef WS_PHASE_TIMERS
     __syncthreads();
-    if (t < 16 && Ap->entropy) Ap->entropy[row * 16 + t] = static_cast<double>(S.marks[t]);
+    if (t < 32 && Ap->entropy) Ap->entropy[row * 32 + t] = static_cast<double>(S.marks[t]);
 #endif
     return true;
 }
