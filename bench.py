@@ -33,7 +33,7 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # reads for a 256 MiB device copy; measured for one build of the kernel and only reported for that build (the digest
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
-    # (workload, mode): (bytes per launch, profiles/ file, sha256[:16] of whirl-llm_amd/csrc/ws_sample.h at the time)
+    # (workload, mode): (bytes per launch, profiles/ file, kernel_digest() at the time)
     ("tile", "auto"): (168795725, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
     ("tile", "exact"): (539588491, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
 }
@@ -55,9 +55,13 @@ def checker():
 
 
 def kernel_digest():
+    """sha256[:16] over the sources of the two sampler kernels (ws_sample.h, then ws_lean.h)."""
     import hashlib
-    with open(os.path.join(ROOT, "whirl-llm_amd", "csrc", "ws_sample.h"), "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()[:16]
+    h = hashlib.sha256()
+    for name in ("ws_sample.h", "ws_lean.h"):
+        with open(os.path.join(ROOT, "whirl-llm_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def traffic_for(workload, mode):
@@ -90,13 +94,15 @@ def rotation_for(nbytes):
     return max(2, -(-int(2.5 * INFINITY_CACHE_BYTES) // nbytes))
 
 
-def time_gpu(c, steps, warmup, rng_mode=1):
+def time_gpu(c, steps, warmup, rng_mode=1, top_k_array=False):
     """Times `steps` launches twice: `cold` - each launch reads another copy of the logits, the copies together larger than
     the memory-side cache, so the row bytes come from HBM - and `warm` - every launch on the one resident copy. Returns
     (sampler, wall ms per step cold, kernel ms per step cold, kernel ms per step warm, copies)."""
     import torch
     gc = workloads()
     d = gc.upload(c)
+    if top_k_array and d["top_k"] is None:  # a batch that hands over an array of zeros instead of leaving it out
+        d["top_k"] = torch.zeros(c["rows"], dtype=torch.int32, device="cuda:0")
     smp = gc.sampler_for(c, d, rng_mode, mode=MODE, kept_cap=KEPT_CAP)
     base = d["logits"]
     n_rot = rotation_for(base.numel() * base.element_size())
@@ -131,8 +137,12 @@ def device_report(smp):
     from __graft_entry__ import load_package
     m = load_package()
     fl = smp.flags.cpu().numpy()
-    return dict(device_near_flags=int(((fl & m.FLAG_NEAR) != 0).sum()),
-                device_failed_rows=int(((fl & (m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED)) != 0).sum()))
+    n = lambda bit: int(((fl & bit) != 0).sum())
+    # rows that left the usual way inside the launch (a launch lasts as long as its slowest row)
+    routes = dict(one_sweep_no_top_k=n(m.FLAG_ROUTE_LEAN), handed_back_to_three_pass=n(m.FLAG_ROUTE_HANDED_BACK),
+                  exact_multi_pass=n(m.FLAG_ROUTE_EXACT), read_again=n(m.FLAG_ROUTE_REDONE), split_row_done_alone=n(m.FLAG_ROUTE_SPLIT_ALONE))
+    return dict(device_near_flags=n(m.FLAG_NEAR), device_failed_rows=n(m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED),
+                routes=routes)
 
 
 def parity_sample(c, smp, n_check, rng_mode=1):
@@ -219,14 +229,16 @@ def cpu_model():
     return platform.processor() or "unknown"
 
 
-def run_workload(name, steps, warmup, check_rows):
+def run_workload(name, steps, warmup, check_rows, top_k_array=False):
     gc = workloads()
     make = dict(tile=gc.make_tile, cfg1=gc.make_cfg1, cfg2=gc.make_cfg2, cfg3=gc.make_cfg3, cfg5=gc.make_cfg5)[name]
     c = make()
-    smp, wall_ms, kern_ms, warm_ms, n_rot = time_gpu(c, steps, warmup)
+    smp, wall_ms, kern_ms, warm_ms, n_rot = time_gpu(c, steps, warmup, top_k_array=top_k_array)
     par = parity_sample(c, smp, check_rows) if check_rows else device_report(smp)
     ab = algorithmic_bytes(c)
-    return c, dict(workload=name, rows=c["rows"], vocab=c["V"], dtype=c["dtype"], ms_per_step=wall_ms, kernel_ms=kern_ms,
+    lean = par["routes"]["one_sweep_no_top_k"] + par["routes"]["handed_back_to_three_pass"] > 0
+    return c, dict(workload=name + (" (top_k: an array of zeros)" if top_k_array else ""), rows=c["rows"], vocab=c["V"], dtype=c["dtype"],
+                   kernel="ws::lean_batch_kernel" if lean else "ws::sample_batch_kernel", ms_per_step=wall_ms, kernel_ms=kern_ms,
                    kernel_ms_warm=warm_ms, logits_copies_rotated=n_rot,
                    rows_per_s=c["rows"] / (wall_ms * 1e-3), algorithmic_MB=ab / 1e6, achieved_GBs=ab / (kern_ms * 1e-3) / 1e9,
                    achieved_GBs_warm=ab / (warm_ms * 1e-3) / 1e9,
@@ -443,6 +455,9 @@ def main():
                 n_chk = 0 if a.no_cpu else (1 if w == "cfg1" else 4)
                 _, r = run_workload(w, 20 if w == "cfg5" else max(20, a.steps // 4), 5, n_chk)
                 also.append(r)
+        if a.workload == "tile" and a.mode == "auto":  # the same batch through the single-sweep kernel that takes a top-k
+            _, r = run_workload("tile", max(20, a.steps // 4), 5, 0, top_k_array=True)
+            also.append(r)
         also.append(spec_verify_workload(max(20, a.steps // 4), 5))
         also.append(host_decode_step(max(50, a.steps)))
     cpu = None if a.no_cpu else cpu_baseline(c)
@@ -463,7 +478,7 @@ def main():
                      "cold": f"each launch reads another of {main_res['logits_copies_rotated']} copies of the logits (together "
                              "beyond the 256 MiB memory-side cache); *_warm: every launch on one resident copy",
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "ws::sample_batch_kernel", "kernel_source_digest": kernel_digest(),
+                     "kernel": main_res["kernel"], "kernel_source_digest": kernel_digest(),
                      "algorithmic_bytes_per_launch": ab, "kernel_ms": main_res["kernel_ms"]},
         "cpu_baseline": cpu,
         "parity": main_res["parity"],

@@ -172,11 +172,24 @@ enum {
                                       size or beyond does close the set, src/sampling/sampler.cpp:35-42) -: drawn as the reference draws an open row, from
                                       the 256 top candidates in sorted order, then from the other tokens in id order
                                       (src/sampling/sampler.cpp:118-146); n_kept and kept_ids describe those candidates */
-    WS_FLAG_APPROX_ENTROPY = 1u << 7 /* `entropy` counts the kept tokens outside the gathered bins at the middle of their
+    WS_FLAG_APPROX_ENTROPY = 1u << 7, /* `entropy` counts the kept tokens outside the gathered bins at the middle of their
                                       histogram bin (each within 1/128 of its place: the entropy is within 1/128 absolute,
                                       usually far closer) instead of one by one; rows whose kept set a
                                       top-k bounds are always exact */
+    /* Which way the row went inside the launch when it left the usual one. Results are the same on every route; a
+     * launch lasts as long as its slowest row, so a caller that counts these bits knows why a launch was slow. */
+    WS_FLAG_ROUTE_HANDED_BACK = 1u << 8, /* the one-sweep kernel for batches without a top-k left the row to the
+                                            three-pass code (a top-k after all, a race draw, a cut among thousands of
+                                            equal logits): about twice the usual time */
+    WS_FLAG_ROUTE_EXACT = 1u << 9,       /* finished by the exact multi-pass route (see WS_FLAG_OVERFLOW): hundreds of
+                                            microseconds */
+    WS_FLAG_ROUTE_REDONE = 1u << 10,     /* the single sweep's provisional bound did not hold (a token far above the
+                                            head of the row, or a masked-out outlier): the row was read again */
+    WS_FLAG_ROUTE_SPLIT_ALONE = 1u << 11, /* a split row whose parts did not meet within split_spins looks: done by
+                                            one workgroup. A caller that sees this often sets max_split = 1 */
+    WS_FLAG_ROUTE_LEAN = 1u << 12        /* done by the one-sweep kernel for batches without a top-k (information only) */
 };
+#define WS_FLAG_ROUTE_MASK 0x1f00u
 
 /* What a caller does with the WS_FLAG_NEAR_* bits: nothing has to be done. A row that carries one still has the
  * token, kept count and probability the kernel computed - they are the kernel's best answer and the same on every run.
@@ -279,7 +292,9 @@ typedef struct ws_batch {
                                    split */
     uint32_t split_spins;       /* split rows: how often a part looks for the others before it gives up on them (they all
                                    have to be running at once, which a GPU shared with other work may not allow in time); the
-                                   row is then done by one workgroup - slower, same result. 0 = about a second's worth */
+                                   row is then done by one workgroup - slower, same result, WS_FLAG_ROUTE_SPLIT_ALONE. A look takes
+                                   about a microsecond; 0 = 512 looks (going on alone costs some sixty microseconds,
+                                   so a longer wait gains nothing) */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

@@ -98,6 +98,10 @@ def test_parts_that_give_up_on_each_other_leave_the_row_to_one_workgroup():
     one = _run(c, 1, 1, launches=1)
     smp = _run(c, 1, 0, launches=3, split_spins=1)
     assert gc.compare_rows(c, smp, range(5), 1)["exact"] == 5
-    for name in ("token", "n_kept", "flags"):  # (the probabilities come from the histogram against the exact maximum here: last bits differ)
+    for name in ("token", "n_kept"):  # (the probabilities come from the histogram against the exact maximum here: last bits differ)
         assert torch.equal(getattr(one, name), getattr(smp, name)), name
+    m = gc.pkg()
+    assert torch.equal(one.flags & ~m.FLAG_ROUTE_MASK, smp.flags & ~m.FLAG_ROUTE_MASK)
+    # (which rows' parts miss each other depends on when they start: the bit is there for some launches' rows, never for an unsplit one)
+    assert not ((one.flags & m.FLAG_ROUTE_SPLIT_ALONE) != 0).any()
     assert torch.allclose(one.prob, smp.prob, rtol=1e-6, atol=0)

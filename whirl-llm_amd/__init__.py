@@ -23,6 +23,9 @@ FLAG_NEAR_TOP_P, FLAG_NEAR_MIN_P, FLAG_NEAR_DRAW = 1, 2, 4
 FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN, FLAG_APPROX_ENTROPY = 8, 16, 32, 64, 128
 ACCEPT_OK, ACCEPT_HOST, ACCEPT_NEAR_TYPICAL, ACCEPT_HISTORY_FULL = 0, 1, 2, 4
 FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
+# which way a row went inside the launch (WS_FLAG_ROUTE_*)
+FLAG_ROUTE_HANDED_BACK, FLAG_ROUTE_EXACT, FLAG_ROUTE_REDONE, FLAG_ROUTE_SPLIT_ALONE, FLAG_ROUTE_LEAN = 0x100, 0x200, 0x400, 0x800, 0x1000
+FLAG_ROUTE_MASK = 0x1f00
 CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
 
 

@@ -6,7 +6,6 @@
 
 #include <atomic>
 
-#include <cstdlib>
 #include <cstring>
 
 #include "ws_accept.h"
@@ -136,8 +135,9 @@ BatchPlan plan_batch(const ws_batch* b) {
 #else
     const bool wants_entropy = b->entropy != nullptr;
 #endif
-    static const bool lean_on = std::getenv("WS_LEAN") != nullptr;  // (while the lean kernel is being brought up)
-    p.lean = lean_on && p.fused && b->mode == WS_MODE_AUTO && b->dtype == WS_DTYPE_F32 && !b->kept_ids && !b->query_prob && !wants_entropy && !b->race &&
+    // Its rows are those without a top-k, and a batch says so by leaving `top_k` out: a row with one would be handed
+    // back to the three-pass code inside the launch, at twice the time of the kernel that takes a top-k in its stride.
+    p.lean = p.fused && b->mode == WS_MODE_AUTO && b->dtype == WS_DTYPE_F32 && !b->top_k && !b->kept_ids && !b->query_prob && !wants_entropy && !b->race &&
              fused_total + kStaticLean <= kMaxLds;
     if (p.lean) {
         uint64_t lt = fused_total;

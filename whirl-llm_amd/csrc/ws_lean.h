@@ -28,7 +28,7 @@ namespace ws {
 constexpr int kLeanRegs = 40;   // bin-cache registers per thread: 160 tokens, rows of up to 163840 tokens
 constexpr int kLeanBatch = 2;   // 128-bit loads per thread and batch
 constexpr uint32_t kLeanPlaces = 32u, kLeanBuckets = 128u, kLeanMaxRange = 800u;
-constexpr uint32_t kRouteHandedBack = 0x100u;  // WS_FLAG_ROUTE_THREE_PASS
+  // WS_FLAG_ROUTE_THREE_PASS
 
 #ifdef WS_PHASE_TIMERS
 #define WSL_MARK(k)                                                \
@@ -321,7 +321,11 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     for (int k = 0; k < kHid; ++k) hid[k] = t + k * WS_BLOCK < nh ? static_cast<uint32_t>(hist_ids[t + k * WS_BLOCK]) : 0xffffffffu;
     const uint32_t bid = t < nb ? static_cast<uint32_t>(bias_ids[t]) : 0xffffffffu;  // the first bias ids
     if (wv == WS_WAVES - 1u) {  // one wave draws the row's uniform for everybody
-        const double u_ = batch_uniform(A.rng, P.seed, row, P.step, 0);
+        // (the seed by way of a vector register: as scalar arithmetic the generator's rounds are moved out of this
+        // branch, and sixteen waves work them out)
+        uint32_t seed_lo = static_cast<uint32_t>(P.seed);
+        asm volatile("" : "+v"(seed_lo));
+        const double u_ = batch_uniform(A.rng, (P.seed & 0xffffffff00000000ull) | seed_lo, row, P.step, 0);
         if (lane == 0u) {
             s_d[6] = u_;
             s_d[8] = neg_log_min_p;
@@ -437,7 +441,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < kHid; ++k)
-            if (hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
+            if (static_cast<uint32_t>(k) * WS_BLOCK < nh && hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));
         for (uint32_t j = t + kHid * WS_BLOCK; j < nh; j += WS_BLOCK) {
             const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
@@ -470,7 +474,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         const bool ids_now = nb == 0;  // without a bias list the second table takes the token id of each rank right away
 #pragma unroll
         for (int k = 0; k < kHid; ++k)
-            if (hid[k] < V) {
+            if (static_cast<uint32_t>(k) * WS_BLOCK < nh && hid[k] < V) {
                 const uint32_t r = rank_of(rv, hid[k]);
                 atomicAdd(&cnt[r], 1u);
                 if (ids_now) first[r] = hid[k];
@@ -630,8 +634,9 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 return;
             }
             uint32_t j0 = 0;
-            for (; j0 + WS_BLOCK < n; j0 += 4u * WS_BLOCK) take(std::integral_constant<int, 4>{}, ids, n, j0, nullptr);
-            if (j0 < n) take(std::integral_constant<int, 1>{}, ids, n, j0, nullptr);
+            for (; j0 + 2u * WS_BLOCK < n; j0 += 4u * WS_BLOCK) take(std::integral_constant<int, 4>{}, ids, n, j0, nullptr);
+            if (j0 + WS_BLOCK < n) take(std::integral_constant<int, 2>{}, ids, n, j0, nullptr);
+            else if (j0 < n) take(std::integral_constant<int, 1>{}, ids, n, j0, nullptr);
         };
         take_all(hist_ids2, nh, &hid[0]);
         take_all(bias_ids2, nb, &bid);
@@ -1214,7 +1219,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             if (mg_min_p < tol) flags |= kNearMinP;
             if (mg < tol) flags |= kNearDraw;
             Ap->token[row] = static_cast<int32_t>(cid[r]);
-            Ap->flags[row] = flags;
+            Ap->flags[row] = flags | kRouteLean;
             if (Ap->prob) Ap->prob[row] = static_cast<float>(cem[r] / Zk);
             if (Ap->margin) Ap->margin[3 * row + 2] = mg;
         }
@@ -1226,7 +1231,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             if (mg_top_p < tol) flags |= kNearTopP;
             if (mg_min_p < tol) flags |= kNearMinP;
             Ap->token[row] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(s_q[4]));
-            Ap->flags[row] = flags;
+            Ap->flags[row] = flags | kRouteLean;
             if (Ap->prob) Ap->prob[row] = static_cast<float>(s_d[1] / Zk);
             if (Ap->margin) Ap->margin[3 * row + 2] = 0.0;
         }
@@ -1262,6 +1267,7 @@ __device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
     B.work = nullptr;
     B.split_log2 = 0u;
     sample_row<false, false, false>(B, row);
+    __syncthreads();  // (the row's flags are written by whichever thread finished it)
     if (threadIdx.x == 0) B.flags[row] |= kRouteHandedBack;
 }
 

@@ -47,6 +47,8 @@ constexpr float kG0 = 16776924.0f, kG1 = -130126.3125f;
 // flag bits (WS_FLAG_* of the C ABI)
 constexpr uint32_t kOpenList = 256u;  // candidates of the engine's short list (k_small, src/server/engine_sampling.h:20)
 constexpr uint32_t kNearTopP = 1u, kNearMinP = 2u, kNearDraw = 4u, kAllMasked = 8u, kOverflow = 16u, kBadParam = 32u, kOpen = 64u, kApproxEntropy = 128u;
+// which way a row went when it left the usual one (WS_FLAG_ROUTE_*): counted by callers that want to know how often
+constexpr uint32_t kRouteHandedBack = 0x100u, kRouteExact = 0x200u, kRouteRedone = 0x400u, kRouteSplitAlone = 0x800u, kRouteLean = 0x1000u;
 
 struct BatchArgs {
     const void* logits;
@@ -2056,7 +2058,8 @@ __device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t bl
                     // arrived" and "given up" exclude each other - and every part that sees the bit, now or when it arrives,
                     // leaves the row to part 0, which does it alone. No row fails; it is only slower.
                     constexpr uint32_t kGaveUp = 0x80000000u;
-                    const uint32_t limit = A.split_spins ? A.split_spins : 1u << 21;
+                    // (a look takes about a microsecond; going on alone costs some sixty: waiting much longer than that gains nothing)
+                    const uint32_t limit = A.split_spins ? A.split_spins : 512u;
                     uint32_t v = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
                     uint32_t spins = 0;
                     while (!(v & kGaveUp) && v < n_parts) {
@@ -2100,11 +2103,13 @@ __device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t bl
             // alone, as for an unsplit row; the others are done.
             if (swept && leave_shared()) clean_shared();
             if (part != 0u) return;
+            if (gave_up) flags |= kRouteSplitAlone;
             split = false;
             cached = false;  // (parts that did not meet have no common histogram)
             all_adjusted();
         }
         if (WS_RARE(!cached)) {
+            flags |= kRouteRedone;
             m = -INFINITY;
             stream_row<!FUSED>(rv, [&](uint32_t, float x, int) { m = fmaxf(m, x); }, [](uint32_t, uint32_t) {});
             m = fmaxf(block_max(m, red_f), m_adj);
@@ -2204,7 +2209,7 @@ __device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t bl
         }
         if (!(m > -INFINITY)) flags |= kAllMasked;
     }
-    if (WS_RARE(flags)) {  // uniform over the block (and over the parts of a split row)
+    if (WS_RARE(flags & (kAllMasked | kBadParam))) {  // uniform over the block (and over the parts of a split row)
         if (t == 0 && (part == 0u || !split)) {
             A.token[row] = -1;
             A.flags[row] = flags;
@@ -3774,6 +3779,7 @@ __device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t bl
     if (WS_RARE((flags & (kOverflow | kPartialTables)) == (kOverflow | kPartialTables))) token = -1;  // (a split row that ran over after its parts had left: reported unresolved)
     if (WS_RARE((flags & (kOverflow | kPartialTables)) == kOverflow && m > -INFINITY)) {  // uniform
         flags &= ~kOverflow;
+        flags |= kRouteExact;
         finished = finished_slow = true;
         finished_lean = false;
         dumped = false;  // (whatever an earlier finish wrote is written again from this one's result)

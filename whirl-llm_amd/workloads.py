@@ -117,7 +117,8 @@ def upload(c, device="cuda:0"):
     else:
         d["logits"] = torch.from_numpy(c["logits"]).to(device)
     d["inv_t"] = torch.from_numpy(c["inv_t"]).to(device)
-    d["top_k"] = torch.from_numpy(c["top_k"].view(np.int32)).to(device)
+    # (a batch without any top-k says so by leaving the array out: ws_batch.top_k = NULL)
+    d["top_k"] = torch.from_numpy(c["top_k"].view(np.int32)).to(device) if c["top_k"].any() else None
     d["top_p"] = torch.from_numpy(np.ascontiguousarray(c["top_p"], np.float64)).to(device)
     d["min_p"] = torch.from_numpy(np.ascontiguousarray(c["min_p"], np.float64)).to(device)
     d["seed"] = torch.from_numpy(c["seed"].view(np.int64)).to(device)
