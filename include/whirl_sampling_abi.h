@@ -299,6 +299,17 @@ typedef struct ws_batch {
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
 uint64_t ws_sample_batch_workspace(const ws_batch* b);
+
+/* What a launch of this batch shape does with the workspace (host-only computation; no counterpart in the reference,
+ * whose sampler has no workspace). A caller that keeps one buffer across batches of different shapes - history lengths
+ * that grow, say - has to know: after a WS_WORK_TABLES launch the buffer holds leftovers, and a WS_WORK_MEETING launch
+ * needs zeros. */
+enum {
+    WS_WORK_NONE = 0,    /* not touched */
+    WS_WORK_MEETING = 1, /* the meeting place of split rows: zero-filled on entry, left zero-filled */
+    WS_WORK_TABLES = 2   /* rank tables of the kernels that sweep a row twice: contents on entry do not matter, leftovers stay */
+};
+int ws_sample_batch_workspace_use(const ws_batch* b);
 int ws_sample_batch(void* stream, const ws_batch* b);
 /* ws_sample_batch for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
  * harnesses that forbid it; it has no counterpart in the reference. The split rows of a small batch meet in memory that is

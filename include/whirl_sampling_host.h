@@ -42,6 +42,14 @@ typedef struct wsh_rows {
 /* 0 = ok, otherwise the code of the failing call (hipError_t > 0, WS_E_* < 0); text from wsh_last_error(). Synchronous. */
 int wsh_sample_rows(void* stream, const wsh_rows* a);
 
+/* For tests of the adapter's failure path (the reference tests its own adapter over a backend that fails on demand,
+ * tests/iso/server.sample_buffers/sample_buffers_tests.cpp:28-80): on one sampling::DeviceRows over d_logits, filter
+ * every row ahead with row 0's sampler, ask for a row past the buffer (codes[0] = what the exception carried), ask for
+ * a row with a 70000-id history, which the device library refuses (codes[1]), then copy d_next over d_logits as a
+ * model's next step would, newCycle(), and go on as wsh_sample_rows does. The tokens have to be those of d_next's rows:
+ * nothing filtered before the failures may answer. */
+int wsh_failures_then_rows(void* stream, const wsh_rows* a, const float* d_next, int32_t codes[2]);
+
 /* Acceptor::sample (src/sampling/acceptor.cpp:63-100) for one sequence over device logits: verify rows row0 .. row0 + nd
  * of d_logits, drafts dr[0 .. nd), output index n_gen + accepted. With prefetch != 0 the rows are filtered by one device
  * launch (sampling::DeviceRows::prefetchRows) before the loop, otherwise one launch per visited row. */

@@ -64,3 +64,25 @@ def test_rows_whose_bound_from_the_head_does_not_hold():
     c["logits"][3, c["hist"][3, 7]] = np.float32(np.nan)
     res = gc.compare_rows(c, _both(c), range(4), 1)
     assert res["exact"] == 4, res
+
+
+def test_what_a_launch_does_with_the_workspace_is_reported():
+    """ws_sample_batch_workspace_use: the meeting place of split rows (zeros in, zeros out) for a lone row with a short
+    history, the rank tables (leftovers stay) once the history is too long for the single sweep, nothing for a batch
+    that fills the device. A caller that keeps one buffer clears it between the second kind and the first."""
+    m = gc.pkg()
+    uses = []
+    for rows, n_hist in ((1, 300), (1, 8192), (256, 300)):
+        c = gc.make_cfg2(rows=rows, V=151936, n_hist=n_hist, n_bias=0) if rows == 1 else gc.make_tile(rows=rows, n_hist=n_hist)
+        d = gc.upload(c)
+        smp = gc.sampler_for(c, d, 1, kept_cap=256)
+        use = m.lib().ws_sample_batch_workspace_use(smp.desc)
+        uses.append(use)
+        if use == m.WORK_NONE:
+            assert m.lib().ws_sample_batch_workspace(smp.desc) == 0
+            continue
+        smp.run()
+        torch.cuda.synchronize()
+        left = bool(smp.workspace.any().item())
+        assert left == (use == m.WORK_TABLES), (rows, n_hist, use, left)
+    assert uses == [m.WORK_MEETING, m.WORK_TABLES, m.WORK_NONE], uses

@@ -10,16 +10,24 @@ import gpu_cases as gc
 pytestmark = pytest.mark.gpu
 
 
-def _run(c, rows):
+def _run(c, rows, logits=None, **more):
+    """c["hist"]: an array [rows, n] or a list of per-row arrays of different lengths."""
     m = gc.pkg()
-    d = gc.upload(c)
-    nh = c["hist"].shape[1] if c["hist"] is not None else 0
+    if logits is None:
+        cu = dict(c)
+        if isinstance(c["hist"], list):
+            cu["hist"] = None  # (the device layouts of the fused entry are not used here)
+        logits = gc.upload(cu)["logits"]
     nb = c["bias_ids"].shape[1] if c["bias_ids"] is not None else 0
     R = c["rows"]
+    hist = hist_off = None
+    if c["hist"] is not None and len(c["hist"][0]) + len(c["hist"][-1]) > 0:
+        hist = np.concatenate([np.asarray(h, np.int32) for h in c["hist"]])
+        hist_off = np.concatenate([[0], np.cumsum([len(h) for h in c["hist"]])]).astype(np.uint32)
     out = m.host_sample_rows(
-        d["logits"], c["inv_t"], c["seed"], c["step"], top_k=c["top_k"], top_p=c["top_p"], min_p=c["min_p"],
-        hist=c["hist"], hist_off=np.arange(R + 1, dtype=np.uint32) * nh if nh else None, rep=c["rep"], pres=c["pres"], freq=c["freq"],
-        bias_ids=c["bias_ids"], bias_vals=c["bias_vals"], bias_off=np.arange(R + 1, dtype=np.uint32) * nb if nb else None)
+        logits, c["inv_t"], c["seed"], c["step"], top_k=c["top_k"], top_p=c["top_p"], min_p=c["min_p"],
+        hist=hist, hist_off=hist_off, rep=c["rep"], pres=c["pres"], freq=c["freq"],
+        bias_ids=c["bias_ids"], bias_vals=c["bias_vals"], bias_off=np.arange(R + 1, dtype=np.uint32) * nb if nb else None, **more)
     near = 0
     for r in rows:
         o, kept, _ = gc.oracle_row(c, r, 0)  # rng 0: the reference's uniform(seed, pos_idx)
@@ -99,3 +107,32 @@ def test_decode_steps_over_one_device_rows_object():
             o, _, _ = gc.oracle_row(cc, 0, 0)
             if tok[i] != o.token:
                 assert min(o.margin, o.margin_top_p, o.margin_min_p) < 1e-6, (top_k, top_p, i, tok[i], o.token)
+
+
+def test_history_length_changes_on_one_device_rows_object():
+    """One DeviceRows, three rows of 151936 tokens in a row: a 300-id history (a lone row is split over sixteen
+    workgroups that meet in the workspace), then 8192 ids (too long for the single sweep: the workspace takes that
+    kernel's rank tables), then 300 again - the meeting place has to be clean again."""
+    c = gc.make_cfg2(rows=3, V=151936, n_hist=8192, n_bias=0)
+    c["top_k"][:] = [0, 40, 0]
+    c["hist"] = [c["hist"][0][:300], c["hist"][1], c["hist"][2][:300]]
+    near, out = _run(c, range(3))
+    assert near == 0, out
+
+
+def test_device_rows_is_usable_after_failed_calls_and_holds_nothing_stale():
+    """A row out of range and a launch the device library refuses, each reported by an exception; then the logits are
+    rewritten, newCycle(), and every row is sampled: the answers are those of the new logits, although every row of
+    the old ones had been filtered ahead with the very same sampler settings."""
+    m = gc.pkg()
+    c = gc.make_cfg2(rows=4, V=32000, n_hist=0, n_bias=0)
+    for k in ("inv_t", "top_k", "top_p", "min_p"):
+        c[k][:] = c[k][0]
+    c["top_k"][:] = 50
+    first = gc.upload(c)["logits"]
+    c["logits"] = np.ascontiguousarray(c["logits"][:, ::-1]).copy()  # the next step's logits
+    nxt = gc.upload(c)["logits"]
+    near, out = _run(c, range(4), logits=first, failures_then=nxt)
+    assert near == 0
+    assert out["failure_codes"] == (m.E_INVALID, m.E_UNSUPPORTED), out["failure_codes"]
+    assert torch.equal(first, nxt)

@@ -29,6 +29,10 @@ FLAG_ROUTE_MASK = 0x1f00
 CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
 
 
+E_INVALID, E_WORKSPACE, E_UNSUPPORTED, E_NO_DEVICE, E_STATIC_LIMIT = -1, -2, -3, -4, -5  # WS_E_*
+WORK_NONE, WORK_MEETING, WORK_TABLES = 0, 1, 2  # ws_sample_batch_workspace_use
+
+
 class WsError(RuntimeError):
     pass
 
@@ -136,6 +140,7 @@ ABI = {
                                     C.c_uint64]),
     "ws_argmax_prob_ws": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]),
     "ws_sample_batch_workspace": (C.c_uint64, [C.POINTER(Batch)]),
+    "ws_sample_batch_workspace_use": (C.c_int, [C.POINTER(Batch)]),
     "ws_sample_batch": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_sample_batch_static": (C.c_int, [C.c_void_p, C.POINTER(Batch)]),
     "ws_adjust_rows": (C.c_int, [C.c_void_p, C.POINTER(Adjust)]),
@@ -506,6 +511,7 @@ class HostSteps(C.Structure):
 
 
 HOST_ABI = {"wsh_sample_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows)]),
+            "wsh_failures_then_rows": (C.c_int, [C.c_void_p, C.POINTER(HostRows), C.c_void_p, C.POINTER(C.c_int32 * 2)]),
             "wsh_accept_sample": (C.c_int, [C.c_void_p, C.POINTER(HostAccept)]),
             "wsh_decode_steps": (C.c_int, [C.c_void_p, C.POINTER(HostSteps)]), "wsh_last_error": (C.c_char_p, [])}
 _host_lib = None
@@ -528,7 +534,7 @@ def host_lib():
 
 
 def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p=None, hist=None, hist_off=None, rep=None, pres=None,
-                     freq=None, bias_ids=None, bias_vals=None, bias_off=None, race=False):
+                     freq=None, bias_ids=None, bias_vals=None, bias_off=None, race=False, failures_then=None):
     """One token per row through the C++ host API (sampling::DeviceRows + sampling::sampleRow). logits: [rows, vocab]
     float32 device tensor; everything else numpy arrays on the host. Returns a dict of numpy arrays
     (token, prob, n_kept, flags, closed)."""
@@ -553,7 +559,14 @@ def host_sample_rows(logits, inv_t, seed, pos_idx, top_k=None, top_p=None, min_p
                  bias_off=h(bias_off, np.uint32), race=int(race), token=out["token"].ctypes.data_as(C.c_void_p),
                  prob=out["prob"].ctypes.data_as(C.c_void_p), n_kept=out["n_kept"].ctypes.data_as(C.c_void_p),
                  flags=out["flags"].ctypes.data_as(C.c_void_p), closed=out["closed"].ctypes.data_as(C.c_void_p))
-    rc = host_lib().wsh_sample_rows(_stream(), C.byref(a))
+    if failures_then is not None:  # wsh_failures_then_rows: `logits` is overwritten with this tensor after two failed calls
+        _dev_f32(failures_then)
+        assert failures_then.shape == logits.shape
+        codes = (C.c_int32 * 2)()
+        rc = host_lib().wsh_failures_then_rows(_stream(), C.byref(a), _p(failures_then), C.byref(codes))
+        out["failure_codes"] = (int(codes[0]), int(codes[1]))
+    else:
+        rc = host_lib().wsh_sample_rows(_stream(), C.byref(a))
     if rc != 0:
         raise WsError(f"wsh_sample_rows: {host_lib().wsh_last_error().decode()} ({rc})")
     return out

@@ -421,6 +421,12 @@ uint64_t ws_sample_batch_workspace(const ws_batch* b) {
     return p.err == WS_OK ? p.workspace : 0;
 }
 
+int ws_sample_batch_workspace_use(const ws_batch* b) {
+    const BatchPlan p = plan_batch(b);
+    if (p.err != WS_OK || p.workspace == 0) return WS_WORK_NONE;
+    return p.split_log2 ? WS_WORK_MEETING : WS_WORK_TABLES;
+}
+
 namespace {
 
 int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigned char* work, uint64_t work_bytes) {

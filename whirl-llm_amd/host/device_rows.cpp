@@ -100,11 +100,15 @@ struct DeviceRows::Dev {
     float* row_host = nullptr;         // loadFullRow's buffer: a pinned target makes the download one DMA transfer
     // device memory
     float* adjusted = nullptr;         // escalation: penalised copy of the row (ws_adjust_rows)
-    // The sampler's workspace: with it a batch of a few rows has each row worked on by several workgroups, and long
-    // vocabularies take the history tokens' logits from the sweep. Zero-filled when it is allocated: what it is used for
-    // depends on the vocabulary alone, which this object never changes, and the use that needs zeros puts them back.
+    // The sampler's workspace: with it a batch of a few rows has each row worked on by several workgroups, and rows the
+    // single sweep cannot take get the history tokens' logits from their first sweep. Which of the two a launch does
+    // depends on the vocabulary and on how long the history and bias lists are (ws_sample_batch_workspace_use), so it
+    // changes while this object lives: the first use needs zeros and puts them back, the second leaves its tables
+    // behind. `work_dirty` says that the last launch was of the second kind; the next one of the first kind clears
+    // the buffer on the stream before it runs.
     unsigned char* work = nullptr;
     std::uint64_t work_cap = 0;
+    bool work_dirty = false;
 };
 
 // one row the device has filtered already, waiting on the host for its prepareRow
@@ -280,7 +284,14 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
         d.work_cap = 0;
         checkHip(hipMalloc(reinterpret_cast<void**>(&d.work), need), "hipMalloc");
         d.work_cap = need;
-        checkHip(hipMemsetAsync(d.work, 0, need, stream), "hipMemsetAsync");
+        d.work_dirty = true;  // (fresh memory: whatever it holds)
+    }
+    const int use = ws_sample_batch_workspace_use(&b);
+    if (use == WS_WORK_MEETING && d.work_dirty) {
+        checkHip(hipMemsetAsync(d.work, 0, d.work_cap, stream), "hipMemsetAsync");
+        d.work_dirty = false;
+    } else if (use == WS_WORK_TABLES) {
+        d.work_dirty = true;
     }
     b.workspace = d.work;
     b.workspace_bytes = d.work_cap;

@@ -7,11 +7,14 @@
 #include "whirl_sampling_abi.h"
 #include "whirl_sampling_host.h"
 
+#include <hip/hip_runtime.h>
+
 #include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <exception>
 #include <span>
+#include <stdexcept>
 #include <vector>
 
 namespace ws = whirl::sampling;
@@ -23,22 +26,27 @@ extern "C" {
 
 const char* wsh_last_error(void) { return g_err; }
 
-int wsh_sample_rows(void* stream, const wsh_rows* a) {
-    g_err[0] = 0;
-    try {
-        ws::DeviceRows src(a->d_logits, a->rows, a->vocab, stream);
-        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+}  // extern "C"
+
+namespace {
+ws::Sampler samplerOf(const wsh_rows* a, uint32_t r, std::vector<ws::Cand>* scratch) {
+    ws::Sampler s;
+    s.inv_t = a->inv_t[r];
+    s.temp = 1.0 / s.inv_t;
+    s.top_k = a->top_k ? a->top_k[r] : 0;
+    s.top_p = a->top_p ? a->top_p[r] : 1.0;
+    s.min_p = a->min_p ? a->min_p[r] : 0.0;
+    s.seed = a->seed[r];
+    s.pos_idx = a->pos_idx[r];
+    s.cands = scratch;
+    s.race = a->race != 0;
+    return s;
+}
+
+// one token per row of `a` over `src`, row after row: setAdjust, prepareRow, sampleRow
+void sampleEveryRow(ws::DeviceRows& src, const wsh_rows* a, std::vector<ws::Cand>& scratch) {
         for (uint32_t r = 0; r < a->rows; ++r) {
-            ws::Sampler s;
-            s.inv_t = a->inv_t[r];
-            s.temp = 1.0 / s.inv_t;
-            s.top_k = a->top_k ? a->top_k[r] : 0;
-            s.top_p = a->top_p ? a->top_p[r] : 1.0;
-            s.min_p = a->min_p ? a->min_p[r] : 0.0;
-            s.seed = a->seed[r];
-            s.pos_idx = a->pos_idx[r];
-            s.cands = &scratch;
-            s.race = a->race != 0;
+            ws::Sampler s = samplerOf(a, r, &scratch);
             ws::RowAdjust adj;
             if (a->hist) {
                 adj.history = a->hist + a->hist_off[r];
@@ -62,6 +70,61 @@ int wsh_sample_rows(void* stream, const wsh_rows* a) {
             if (a->flags) a->flags[r] = src.lastFlags();
             if (a->closed) a->closed[r] = s.closed;
         }
+}
+}  // namespace
+
+extern "C" {
+
+int wsh_sample_rows(void* stream, const wsh_rows* a) {
+    g_err[0] = 0;
+    try {
+        ws::DeviceRows src(a->d_logits, a->rows, a->vocab, stream);
+        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+        sampleEveryRow(src, a, scratch);
+        return 0;
+    } catch (const ws::DeviceError& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return e.code ? e.code : -1;
+    } catch (const std::exception& e) {
+        snprintf(g_err, sizeof g_err, "%s", e.what());
+        return -1;
+    }
+}
+
+int wsh_failures_then_rows(void* stream, const wsh_rows* a, const float* d_next, int32_t codes[2]) {
+    g_err[0] = 0;
+    codes[0] = codes[1] = 0;
+    try {
+        ws::DeviceRows src(a->d_logits, a->rows, a->vocab, stream);
+        std::vector<ws::Cand> scratch(a->vocab > 16384u ? a->vocab : 16384u);
+        // every row filtered with row 0's sampler and no penalties: results of the buffer's first contents, held on the host
+        ws::Sampler s0 = samplerOf(a, 0, &scratch);
+        src.setAdjust(ws::RowAdjust{});
+        src.prefetchRows(s0, 0, a->rows);
+        try {  // a row past the buffer
+            src.prepareRow(s0, a->rows);
+        } catch (const ws::DeviceError& e) {
+            codes[0] = e.code;
+        }
+        try {  // a history longer than the device's rank tables take: the launch itself is refused
+            std::vector<std::int32_t> long_hist(70000, 1);
+            ws::RowAdjust adj;
+            adj.history = long_hist.data();
+            adj.n_history = static_cast<std::uint32_t>(long_hist.size());
+            adj.repetition = 1.3f;
+            src.setAdjust(adj);
+            ws::Sampler s1 = samplerOf(a, 0, &scratch);
+            s1.top_p = 0.123;  // (nothing held on the host answers this one)
+            src.prepareRow(s1, 0);
+        } catch (const ws::DeviceError& e) {
+            codes[1] = e.code;
+        }
+        // the model writes the next step's logits; the caller starts the next cycle
+        if (hipMemcpyAsync(const_cast<float*>(a->d_logits), d_next, sizeof(float) * a->rows * static_cast<std::size_t>(a->vocab),
+                           hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)) != hipSuccess)
+            throw std::runtime_error("hipMemcpyAsync");
+        src.newCycle();
+        sampleEveryRow(src, a, scratch);
         return 0;
     } catch (const ws::DeviceError& e) {
         snprintf(g_err, sizeof g_err, "%s", e.what());
