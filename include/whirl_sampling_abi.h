@@ -62,7 +62,11 @@ enum { WS_Q_MAX = 32, WS_Q_WORDS = 72, WS_Q_OFF_IDS = 1, WS_Q_OFF_P = 33 };
 
 int ws_abi_version(void);
 const char* ws_error_string(int code);
-/* Loads nothing and launches nothing: 0 when a gfx950 device is present and the kernels of this library can run. */
+/* Launches nothing: 0 when a gfx950 device is present and the kernels of this library can run. On the current device
+ * it also does, once, what a first launch there would otherwise do: it looks up the address of the library's own
+ * workspace (ws_sample_batch_static) and raises the dynamic LDS limit of every kernel that needs more than the default.
+ * Call it once per device before capturing any of the entry points into a HIP graph: under capture they then only
+ * launch kernels. */
 int ws_probe(void);
 
 /* ---- (1) reference kernels ------------------------------------------------------------------------------- */
@@ -319,8 +323,9 @@ int ws_sample_batch(void* stream, const ws_batch* b);
  * than that (65 to 128 rows in two parts each) is refused with WS_E_STATIC_LIMIT. The memory's address on a device is
  * looked up on the first call there (or by ws_probe): make that call before capturing a graph. All calls on one GPU
  * share this memory: two of them that run at the same time (different streams) race; on one stream they are safe, each
- * launch leaves the memory as the next needs it. (Only split rows use it: use (b) of b->workspace is off here, and so
- * are the staging areas of the kept-set dump - a shared row without a top-k is read again by the workgroup that finishes it.) */
+ * launch leaves the memory as the next needs it. (Only split rows use it: use (b) of b->workspace is off here. The
+ * staging areas of the kept-set dump are taken from the same memory while they fit beside the rows' meeting places -
+ * batches of up to 32 rows; from 33 rows on a shared row without a top-k is read again by the workgroup that finishes it.) */
 #define WS_STATIC_SPLIT_ROWS 64
 int ws_sample_batch_static(void* stream, const ws_batch* b);
 

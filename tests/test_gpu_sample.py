@@ -275,9 +275,11 @@ def test_bias_values_of_one_id_are_added_one_by_one(mode):
     print(res)
 
 
+@pytest.mark.parametrize("rng_mode", [1, 0])  # configs[0] names a Philox-seeded draw; the reference's own uniform as well
 @pytest.mark.parametrize("mode", MODES)
-def test_cfg1_shape(mode):
-    res, _ = run_case(gc.make_cfg1(), 0, mode=mode)
+def test_cfg1_shape(mode, rng_mode):
+    res, _ = run_case(gc.make_cfg1(), rng_mode, mode=mode)
+    assert res["exact"] == 1, res
     print(res)
 
 

@@ -41,3 +41,13 @@ def test_static_workspace_entry_point_matches_the_workspace_one_on_two_calls_in_
     smp = gc.sampler_for(wide, d, 1, max_split=2)
     with pytest.raises(m.WsError, match="own workspace"):
         smp.run_static()
+
+
+def test_static_entry_point_with_a_kept_set_dump_and_no_room_for_staging():
+    """40 rows split four ways with kept_ids set: beside 40 meeting places the library's own memory has no room for the
+    staging areas, so the workgroup that finishes a row reads it again for the dump. Same outputs as with a workspace
+    that has the staging areas, and the oracle's."""
+    c = gc.make_cfg2(rows=40, V=65536, n_hist=512, n_bias=20)
+    c["top_k"][::2] = 0  # (rows without a top-k are the ones whose dump needs the row again)
+    ref, got = _both(c, 1)
+    assert gc.compare_rows(c, got, range(0, 40, 3), 1)["differ"] == 0

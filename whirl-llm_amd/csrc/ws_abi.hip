@@ -15,6 +15,7 @@
 #include "ws_pick.h"
 #include "ws_sample.h"
 #include "ws_spec.h"
+#include "ws_lds_limit.h"
 #include "ws_topk.h"
 
 namespace ws {
@@ -27,6 +28,11 @@ int launch_fused_kept(hipStream_t stream, const BatchArgs& a, unsigned rows, uns
 int launch_split_kept(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
 // ws_lean.hip: the lean single-sweep kernel (1024 threads a row) for batches of unsplit fp32 rows
 int launch_lean(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
+// each of them raises its kernels' dynamic LDS limit on the current device (once; the launchers call them too)
+int prepare_fused(unsigned lds_limit);
+int prepare_split(unsigned lds_limit);
+int prepare_fused_kept(unsigned lds_limit);
+int prepare_split_kept(unsigned lds_limit);
 int prepare_lean(unsigned lds_limit);
 }  // namespace ws
 
@@ -199,6 +205,26 @@ int scratch_address(unsigned char** out) {
     return WS_OK;
 }
 
+// the kernels launched from this file whose dynamic LDS goes beyond the default limit
+int prepare_three_pass() {
+    static std::atomic<uint64_t> done{0};
+    return ws::raise_lds_limit(done, {reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>)}, kMaxLds - kStaticLds);
+}
+int prepare_adjust() {
+    static std::atomic<uint64_t> done{0};
+    return ws::raise_lds_limit(done, {reinterpret_cast<const void*>(&ws::adjust_rows_kernel)}, ws::kAdjustLds);
+}
+// everything a launch would otherwise set on its first call on this device: ws_probe does it ahead, outside any capture
+int prepare_all() {
+    if (const int e = prepare_three_pass(); e != 0) return e;
+    if (const int e = prepare_adjust(); e != 0) return e;
+    if (const int e = ws::prepare_fused(kMaxLds - kStaticLds); e != 0) return e;
+    if (const int e = ws::prepare_split(kMaxLds - kStaticLds); e != 0) return e;
+    if (const int e = ws::prepare_fused_kept(kMaxLds - kStaticLds); e != 0) return e;
+    if (const int e = ws::prepare_split_kept(kMaxLds - kStaticLds); e != 0) return e;
+    return ws::prepare_lean(kMaxLds - kStaticLean);
+}
+
 }  // namespace
 
 extern "C" {
@@ -230,7 +256,7 @@ int ws_probe(void) {
     }
     unsigned char* at = nullptr;  // the current device's copy of the static workspace: resolved here, outside any capture
     if (const int e = scratch_address(&at); e != WS_OK) return e;
-    return WS_OK;
+    return prepare_all();
 }
 
 int ws_argmax(void* stream, const float* x, int n, int* out, int* ids, int* pos, int advance) {
@@ -488,16 +514,7 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
         return ws::launch_lean(S(stream), a, b->rows, p.lean_total, kMaxLds - kStaticLean);
     }
     if (p.fused) return (a.kept_ids ? ws::launch_fused_kept : ws::launch_fused)(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);
-    static std::atomic<uint64_t> attr_set{0};  // the dynamic LDS limit is raised per function and device, once per process
-    int dev = 0;
-    if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::sample_batch_kernel<false>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds - kStaticLds));
-        if (e != hipSuccess) return static_cast<int>(e);
-        attr_set.fetch_or(bit, std::memory_order_release);
-    }
+    if (const int e = prepare_three_pass(); e != 0) return e;
     hipLaunchKernelGGL(ws::sample_batch_kernel<false>, dim3(b->rows), dim3(WS_BLOCK), p.lds_total, S(stream), a);
     return done();
 }
@@ -543,13 +560,7 @@ int ws_adjust_rows(void* stream, const ws_adjust* b) {
     a.out = b->out;
     a.out_stride = b->out_stride;
     a.lds_bytes = ws::kAdjustLds;
-    static bool adjust_attr_set = false;  // raising the dynamic LDS limit is per function, once per process
-    if (!adjust_attr_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&ws::adjust_rows_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(ws::kAdjustLds));
-        if (e != hipSuccess) return static_cast<int>(e);
-        adjust_attr_set = true;
-    }
+    if (const int e = prepare_adjust(); e != 0) return e;
     // a small batch shares a row between workgroups (slices of at least 8192 tokens, one workgroup per compute unit)
     uint32_t parts = 1;
     while (parts < 16u && static_cast<uint64_t>(b->rows) * (parts * 2u) <= compute_units() && b->vocab / (parts * 2u) >= 8192u) parts *= 2u;
