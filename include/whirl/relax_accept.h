@@ -6,6 +6,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <span>
+#include <vector>
 
 namespace whirl::relax {
 
@@ -19,35 +20,37 @@ struct Params {
 };
 
 // ids / logits: a row's largest logits in any order (at least p.topk() of them); m: the row maximum. The draft passes
-// when fewer than topk() candidates come before it in (logit descending, id ascending) order and
-// exp(logit(draft) - m) >= alpha.
+// when it is among them, exp(logit(draft) - m) >= alpha, and fewer than topk() candidates come before it in
+// (logit descending, id ascending) order.
 inline bool acceptGreedy(const Params& p, std::span<const std::int32_t> ids, std::span<const float> logits, float m,
                          std::uint32_t draft) {
     const std::size_t n = std::min(ids.size(), logits.size());
-    std::size_t at = n;
-    for (std::size_t i = 0; i < n && at == n; ++i)
-        if (static_cast<std::uint32_t>(ids[i]) == draft) at = i;
-    if (at == n) return false;
-    std::uint32_t ahead = 0;
-    for (std::size_t i = 0; i < n; ++i)
-        if (i != at && (logits[i] > logits[at] || (logits[i] == logits[at] && static_cast<std::uint32_t>(ids[i]) < draft))) ++ahead;
-    if (ahead >= p.topk()) return false;
-    return std::exp(static_cast<double>(logits[at]) - static_cast<double>(m)) >= static_cast<double>(p.alpha);
+    const auto listed = ids.first(n);
+    const auto hit = std::find(listed.begin(), listed.end(), static_cast<std::int32_t>(draft));
+    if (hit == listed.end()) return false;
+    const float x = logits[static_cast<std::size_t>(hit - listed.begin())];
+    if (!(std::exp(static_cast<double>(x) - static_cast<double>(m)) >= static_cast<double>(p.alpha))) return false;
+    // the rank by counting down: every candidate that sorts before (x, draft) uses up one of the topk() places
+    std::uint32_t places = p.topk();
+    for (std::size_t i = 0; i < n; ++i) {
+        const bool before = logits[i] > x || (logits[i] == x && static_cast<std::uint32_t>(ids[i]) < draft);
+        if (before && --places == 0) return false;
+    }
+    return true;
 }
 
 // Would the text formed by the last `window` tokens of hist followed by tail end in an n-gram it already contains?
+// The text is laid out once and its last n tokens are searched for in everything before its last token (an earlier
+// occurrence may overlap the final one).
 inline bool extendsRepeat(std::span<const std::uint32_t> hist, std::span<const std::uint32_t> tail, std::size_t n = 6,
                           std::size_t window = 4096) {
-    const std::size_t from_hist = std::min(hist.size(), window), total = from_hist + tail.size();
-    if (total < n + 1) return false;
-    const std::size_t skip = hist.size() - from_hist;
-    auto at = [&](std::size_t i) { return i < from_hist ? hist[skip + i] : tail[i - from_hist]; };
-    for (std::size_t start = 0; start + n < total; ++start) {
-        std::size_t same = 0;
-        while (same < n && at(start + same) == at(total - n + same)) ++same;
-        if (same == n) return true;
-    }
-    return false;
+    const std::span<const std::uint32_t> recent = hist.last(std::min(hist.size(), window));
+    if (recent.size() + tail.size() < n + 1) return false;
+    thread_local std::vector<std::uint32_t> text;
+    text.assign(recent.begin(), recent.end());
+    text.insert(text.end(), tail.begin(), tail.end());
+    const auto needle = text.end() - static_cast<std::ptrdiff_t>(n);
+    return std::search(text.begin(), text.end() - 1, needle, text.end()) != text.end() - 1;
 }
 
 // Typical acceptance: h is the entropy of the filtered distribution.
