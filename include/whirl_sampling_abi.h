@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define WS_ABI_VERSION 2
+#define WS_ABI_VERSION 3
 
 enum {
     WS_OK = 0,
@@ -191,9 +191,10 @@ enum {
                                             head of the row, or a masked-out outlier): the row was read again */
     WS_FLAG_ROUTE_SPLIT_ALONE = 1u << 11, /* a split row whose parts did not meet within split_spins looks: done by
                                             one workgroup. A caller that sees this often sets max_split = 1 */
-    WS_FLAG_ROUTE_LEAN = 1u << 12        /* done by the one-sweep kernel for batches without a top-k (information only) */
+    WS_FLAG_ROUTE_LEAN = 1u << 12,       /* done by the one-sweep kernel for batches without a top-k (information only) */
+    WS_FLAG_ROUTE_SHORT = 1u << 13       /* done by the short-list kernel for batches with a bounded top-k (information only) */
 };
-#define WS_FLAG_ROUTE_MASK 0x1f00u
+#define WS_FLAG_ROUTE_MASK 0x3f00u
 
 /* What a caller does with the WS_FLAG_NEAR_* bits: nothing has to be done. A row that carries one still has the
  * token, kept count and probability the kernel computed - they are the kernel's best answer and the same on every run.
@@ -299,6 +300,13 @@ typedef struct ws_batch {
                                    row is then done by one workgroup - slower, same result, WS_FLAG_ROUTE_SPLIT_ALONE. A look takes
                                    about a microsecond; 0 = 512 looks (going on alone costs some sixty microseconds,
                                    so a longer wait gains nothing) */
+    uint32_t top_k_max;         /* 0: nothing is known about the rows' top_k. Otherwise the caller's word that every row has a
+                                   top_k of at least 1 and at most this (up to 1024): such batches - the reference's
+                                   usual sampler settings, top-k 40 - take the short-list kernel, which keeps only the
+                                   tokens that can be among a row's top_k largest instead of a histogram of all of them
+                                   (fp32 and bf16, any vocabulary whose bitmap fits the LDS, kept-set dump included;
+                                   not with `race`, `query_prob` or `entropy`). A row that breaks the word is still
+                                   answered correctly, by the three-pass code inside the launch (WS_FLAG_ROUTE_HANDED_BACK) */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

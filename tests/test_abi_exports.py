@@ -18,7 +18,7 @@ def test_every_declared_symbol_is_exported():
     lib = m.lib()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ws_abi_version() == 2
+    assert lib.ws_abi_version() == 3
     assert lib.ws_error_string(0) == b"ok" and b"workspace" in lib.ws_error_string(-2)
 
 

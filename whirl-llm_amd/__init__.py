@@ -24,8 +24,8 @@ FLAG_ALL_MASKED, FLAG_OVERFLOW, FLAG_BAD_PARAM, FLAG_OPEN, FLAG_APPROX_ENTROPY =
 ACCEPT_OK, ACCEPT_HOST, ACCEPT_NEAR_TYPICAL, ACCEPT_HISTORY_FULL = 0, 1, 2, 4
 FLAG_NEAR = FLAG_NEAR_TOP_P | FLAG_NEAR_MIN_P | FLAG_NEAR_DRAW
 # which way a row went inside the launch (WS_FLAG_ROUTE_*)
-FLAG_ROUTE_HANDED_BACK, FLAG_ROUTE_EXACT, FLAG_ROUTE_REDONE, FLAG_ROUTE_SPLIT_ALONE, FLAG_ROUTE_LEAN = 0x100, 0x200, 0x400, 0x800, 0x1000
-FLAG_ROUTE_MASK = 0x1f00
+FLAG_ROUTE_HANDED_BACK, FLAG_ROUTE_EXACT, FLAG_ROUTE_REDONE, FLAG_ROUTE_SPLIT_ALONE, FLAG_ROUTE_LEAN, FLAG_ROUTE_SHORT = 0x100, 0x200, 0x400, 0x800, 0x1000, 0x2000
+FLAG_ROUTE_MASK = 0x3f00
 CTL_WORDS, Q_WORDS, Q_MAX = 64, 72, 32
 
 
@@ -61,7 +61,7 @@ class Batch(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32),
                 ("race", C.c_void_p),
                 ("hist_len", C.c_void_p), ("query", C.c_void_p), ("query_prob", C.c_void_p), ("entropy", C.c_void_p),
-                ("max_split", C.c_uint32), ("split_spins", C.c_uint32)]
+                ("max_split", C.c_uint32), ("split_spins", C.c_uint32), ("top_k_max", C.c_uint32)]
 
 
 class SpecVerify(C.Structure):
@@ -401,7 +401,7 @@ class BatchSampler:
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
                  max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None,
-                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0, use_workspace=True):
+                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0, use_workspace=True, top_k_max=0):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -439,6 +439,7 @@ class BatchSampler:
         self.entropy = torch.zeros(rows, dtype=torch.float64, device=dev) if want_entropy else None
         b.query_prob, b.entropy = _p(self.query_prob), _p(self.entropy)
         b.max_split, b.split_spins = max_split, split_spins
+        b.top_k_max = top_k_max
         need = lib().ws_sample_batch_workspace(C.byref(b))
         # zero-filled once: the parts of a split row meet here, and every launch leaves it zero-filled again
         self.workspace = torch.zeros(max(int(need), 16), dtype=torch.uint8, device=dev)

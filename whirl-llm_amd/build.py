@@ -16,6 +16,7 @@ SRC = os.path.join(HERE, "csrc", "ws_abi.hip")
 SRC_FUSED = os.path.join(HERE, "csrc", "ws_fused.hip")  # the single-sweep sampler kernel
 SRC_SPLIT = os.path.join(HERE, "csrc", "ws_split.hip")  # the same kernel for rows split over several workgroups
 SRC_KEPT = [os.path.join(HERE, "csrc", f) for f in ("ws_fused_kept.hip", "ws_split_kept.hip")]  # both once more, with the kept-set dump
+SRC_SHORT = os.path.join(HERE, "csrc", "ws_short.hip")  # the short-list kernel for batches whose rows all have a bounded top-k
 SRC_LEAN = os.path.join(HERE, "csrc", "ws_lean.hip")  # the lean single-sweep kernel for batches of unsplit rows
 # packed FP32 instructions are switched off for every device compile of this repository
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -45,11 +46,11 @@ def build(verbose=True):
     # the five translation units and the bare code object side by side (each takes a minute or two), then the link
     objdir = os.path.join(HERE, "csrc", "obj")
     os.makedirs(objdir, exist_ok=True)
-    srcs = (SRC, SRC_FUSED, SRC_SPLIT, *SRC_KEPT, SRC_LEAN)
+    srcs = (SRC, SRC_FUSED, SRC_SPLIT, *SRC_KEPT, SRC_LEAN, SRC_SHORT)
     objs = [os.path.join(objdir, os.path.basename(src)[:-4] + ".o") for src in srcs]
     jobs = [[hipcc, *FLAGS, "-fPIC", "-c", "-o", obj, src] for obj, src in zip(objs, srcs)]
     jobs.append([hipcc, *FLAGS, "--genco", "-o", co, SRC])
-    with concurrent.futures.ThreadPoolExecutor(max_workers=7) as pool:
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
         list(pool.map(run, jobs))
     run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", so, *objs])
     # host layer: plain C++20, no device code; -ffp-contract=off keeps the float arithmetic of the penalties unfused

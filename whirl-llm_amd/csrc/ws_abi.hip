@@ -34,6 +34,9 @@ int prepare_split(unsigned lds_limit);
 int prepare_fused_kept(unsigned lds_limit);
 int prepare_split_kept(unsigned lds_limit);
 int prepare_lean(unsigned lds_limit);
+// ws_short.hip: the short-list kernel for batches whose rows all have a bounded top-k
+int launch_short(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
+int prepare_short(unsigned lds_limit);
 }  // namespace ws
 
 namespace {
@@ -48,6 +51,8 @@ constexpr uint32_t kStaticLds = 4096u + 512u;  // + the phase marks
 #else
 constexpr uint32_t kStaticLds = 4096u;
 #endif
+// the short-list kernel's own words and those of both builds of the three-pass code it calls (7664 bytes)
+constexpr uint32_t kStaticShort = 8192u;
 // the lean kernel's own tables and those of the three-pass code it calls
 #ifdef WS_PHASE_TIMERS
 constexpr uint32_t kStaticLean = 11776u + 768u;
@@ -66,6 +71,8 @@ struct BatchPlan {
     uint32_t lean_tie;    // its second histogram copy (0: none), its dynamic LDS, and the spare LDS of the three-pass code it calls
     uint32_t lean_total;
     uint32_t lean_fb_tie;
+    bool shortlist;       // the short-list kernel takes the batch: every row has a top-k of at most top_k_max (the caller's word)
+    uint32_t short_ab, short_cnt, short_total, short_fb_tie;  // its LDS: bitmap at short_ab, rank words at short_cnt
     uint32_t split_log2;  // the most parts per row that pay for this batch
     uint64_t workspace_min;  // split rows: the least that lets them split (no staging areas), 0 when nothing is split
     uint64_t workspace;   // bytes for that
@@ -156,6 +163,44 @@ BatchPlan plan_batch(const ws_batch* b) {
         const uint64_t three = 65536u + maps;
         p.lean_fb_tie = three + spare_bytes <= lt ? static_cast<uint32_t>((three + 15u) & ~uint64_t{15}) : 0u;
     }
+    // The short-list kernel: its own layout (32 KiB of list, the bitmap with 16-bit prefixes, a word and a 16-bit index
+    // per history / bias entry), and under it room for the three-pass layout of the rows it hands back.
+    p.shortlist = b->top_k && b->top_k_max >= 1u && b->top_k_max <= 1024u && b->mode == WS_MODE_AUTO && vec_rows && !b->race && !b->query_prob &&
+                  !b->entropy && (!b->bias_ids || b->max_bias <= 2047u);
+    if (p.shortlist) {
+        const uint64_t maps_s = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
+        const uint64_t tabs_s = ((cap * 4u + 15u) & ~uint64_t{15}) + ((cap * 2u + 15u) & ~uint64_t{15});
+        const uint64_t own = 32768u + maps_s + tabs_s;
+        const uint64_t three = (cap * 8u > 65536u ? ((cap * 8u + 15u) & ~uint64_t{15}) : 65536u) + maps;
+        uint64_t st = own > three ? own : three;
+        if (st + kStaticShort > kMaxLds) {
+            p.shortlist = false;
+        } else {
+            p.short_ab = 32768u;
+            p.short_cnt = static_cast<uint32_t>(32768u + maps_s);
+            p.short_fb_tie = 0;
+            if (three + spare_bytes + kStaticShort <= kMaxLds) {
+                p.short_fb_tie = static_cast<uint32_t>((three + 15u) & ~uint64_t{15});
+                if (p.short_fb_tie + spare_bytes > st) st = p.short_fb_tie + spare_bytes;
+            }
+            p.short_total = static_cast<uint32_t>(st);
+        }
+    }
+    if (p.shortlist) {  // few rows: a row is shared by up to 16 workgroups of at least 8192 tokens each; nobody waits, so there is no bound on rows * parts but usefulness
+        p.lean = false;
+        p.split_log2 = 0;
+        p.workspace = p.workspace_min = 0;
+        if (b->max_split != 1u) {
+            const uint32_t cus = static_cast<uint32_t>(compute_units());
+            const uint32_t most = b->max_split ? b->max_split : 16u;
+            uint32_t lg = 0;
+            while (lg < 4u && (2u << lg) <= most && b->rows * (2u << lg) <= cus && b->vocab / (2u << lg) >= 8192u) ++lg;
+            p.split_log2 = lg;
+            if (lg) p.workspace = p.workspace_min = uint64_t{b->rows} * ws::kShortSplitRowBytes;
+        }
+        p.err = WS_OK;
+        return p;
+    }
     // Small batches of the single-sweep kernel: with rows to spare on the compute units a row is split over 2, 4, 8 or
     // 16 workgroups (each at least 16384 tokens; 8192 for the step from 8 to 16, which a lone 151936-token row still wins: 29.2 -> 28.0 us), which meet in global memory. All parts of all rows have to be running
     // at the same time - they wait for each other - so rows * parts stays within the compute units of the device.
@@ -222,7 +267,8 @@ int prepare_all() {
     if (const int e = ws::prepare_split(kMaxLds - kStaticLds); e != 0) return e;
     if (const int e = ws::prepare_fused_kept(kMaxLds - kStaticLds); e != 0) return e;
     if (const int e = ws::prepare_split_kept(kMaxLds - kStaticLds); e != 0) return e;
-    return ws::prepare_lean(kMaxLds - kStaticLean);
+    if (const int e = ws::prepare_lean(kMaxLds - kStaticLean); e != 0) return e;
+    return ws::prepare_short(kMaxLds - kStaticShort);
 }
 
 }  // namespace
@@ -506,6 +552,13 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     a.query = b->query;
     a.query_prob = b->query_prob;
     a.entropy = b->entropy;
+    if (p.shortlist) {
+        a.lds_ab = p.short_ab;
+        a.lds_cnt = p.short_cnt;
+        a.fb_lds_tie = p.short_fb_tie;
+        a.work = a.split_log2 ? work : nullptr;
+        return ws::launch_short(S(stream), a, b->rows << a.split_log2, p.short_total, kMaxLds - kStaticShort);
+    }
     if (p.fused && a.split_log2)
         return (a.kept_ids ? ws::launch_split_kept : ws::launch_split)(S(stream), a, b->rows << a.split_log2, p.lds_total, kMaxLds - kStaticLds);
     if (p.lean) {
@@ -530,7 +583,7 @@ int ws_sample_batch(void* stream, const ws_batch* b) {
 int ws_sample_batch_static(void* stream, const ws_batch* b) {
     const BatchPlan p = plan_batch(b);
     if (p.err != WS_OK) return p.err;
-    if (!p.fused) return sample_batch_on(stream, b, p, nullptr, 0);  // (nothing may be left in the split rows' memory)
+    if (!p.fused && !p.shortlist) return sample_batch_on(stream, b, p, nullptr, 0);  // (nothing may be left in the split rows' memory)
     if (p.workspace_min > sizeof(scratch)) return WS_E_STATIC_LIMIT;  // more split rows than the library's own memory holds
     unsigned char* at = nullptr;
     if (const int e = scratch_address(&at); e != WS_OK) return e;

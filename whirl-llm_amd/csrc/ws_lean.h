@@ -1257,6 +1257,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 // It takes the kernel's argument segment and makes its own copy of the arguments with the three-pass layout of the LDS
 // (a copy made by the kernel would be made at the kernel's entry, on every row).
 typedef const __attribute__((address_space(4))) BatchArgs* LeanArgPtr;
+template <bool KEPT>  // (KEPT: the build that can write the kept-set dump)
 __device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
     BatchArgs B;
     __builtin_memcpy(&B, (const void*)Ap, sizeof(BatchArgs));
@@ -1266,7 +1267,7 @@ __device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
     B.two_sweep = 1;
     B.work = nullptr;
     B.split_log2 = 0u;
-    sample_row<false, false, false>(B, row);
+    sample_row<false, false, KEPT>(B, row);
     __syncthreads();  // (the row's flags are written by whichever thread finished it)
     if (threadIdx.x == 0) B.flags[row] |= kRouteHandedBack;
 }
@@ -1282,7 +1283,7 @@ __global__ void __launch_bounds__(WS_BLOCK) lean_batch_kernel(BatchArgs A) {
     __syncthreads();  // whatever the lean path left in LDS is dead
     LeanArgPtr Ap = (LeanArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile("" : "+s"(Ap));
-    three_pass_row(Ap, row);
+    three_pass_row<false>(Ap, row);
 #else
     if (!done && threadIdx.x == 0) A.token[row] = -2;
 #endif

@@ -110,6 +110,12 @@ constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kS
 // slices there, in id order, and the part that finishes the row picks the kept tokens out - no workgroup reads the whole
 // row again. Control words 4 (entries staged), 8 + part (where the part's entries start) and 24 + part (how many).
 constexpr uint32_t kSplitStage = kSplitRowBytes, kSplitStageCap = 8192u, kSplitRowBytesKept = kSplitStage + kSplitStageCap * 8u;
+// The short-list kernel (ws_short.h). Global memory of a row shared by several workgroups (zero-filled once, left
+// zero-filled): kShortCap keys - the tokens a row lists, all parts together -, then 64 + 4 * 16 words: [0] parts arrived,
+// [1] keys listed, [2] a part could not list its slice; from word 64 on, four words a part: maximum (as an order key),
+// threshold (order key), and the part's sum as a double against its maximum.
+constexpr uint32_t kShortCap = 4096u;
+constexpr uint32_t kShortSplitCtrl = kShortCap * 8u, kShortSplitRowBytes = kShortSplitCtrl + 4u * (64u + 4u * 16u);
 // Workspace of one row of the three-pass kernel: per history / bias entry a word of each of phase 0's two rank
 // tables, which sit out the first sweep there. Whole memory lines, so that rows share none.
 __host__ __device__ constexpr uint64_t capture_row_bytes(uint32_t patch_cap) {

@@ -278,6 +278,8 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
     b.kept_logits = d.kept_logits;
     b.kept_cap = cap;
     b.mode = WS_MODE_AUTO;
+    // every row of the launch has the sampler's top-k: a bounded one takes the short-list kernel
+    b.top_k_max = (s.top_k >= 1 && s.top_k <= 1024) ? static_cast<std::uint32_t>(s.top_k) : 0u;
     if (const std::uint64_t need = ws_sample_batch_workspace(&b); need > d.work_cap) {
         if (d.work) (void)hipFree(d.work);
         d.work = nullptr;

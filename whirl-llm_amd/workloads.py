@@ -140,6 +140,8 @@ def upload(c, device="cuda:0"):
         d["max_bias"] = n
     if c["allow"] is not None:
         d["allow"] = torch.from_numpy(c["allow"].view(np.int32)).to(device)
+    # every row has a top-k of at most 1024: the batch says so (ws_batch.top_k_max)
+    d["top_k_max"] = int(c["top_k"].max()) if c["top_k"].min() >= 1 and c["top_k"].max() <= 1024 else 0
     d["race"] = torch.from_numpy(np.ascontiguousarray(c["race"], np.int32)).to(device) if c.get("race") is not None else None
     return d
 
@@ -149,6 +151,7 @@ def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0, **more):
     return m.BatchSampler(d["logits"], d["inv_t"], d["seed"], d["step"], top_k=d["top_k"], top_p=d["top_p"], min_p=d["min_p"],
                           rng=rng_mode, hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
                           bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], max_hist=d["max_hist"],
-                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"), **more)
+                          max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"),
+                          **{"top_k_max": d.get("top_k_max", 0), **more})
 
 
