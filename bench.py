@@ -139,7 +139,7 @@ def device_report(smp):
     fl = smp.flags.cpu().numpy()
     n = lambda bit: int(((fl & bit) != 0).sum())
     # rows that left the usual way inside the launch (a launch lasts as long as its slowest row)
-    routes = dict(one_sweep_no_top_k=n(m.FLAG_ROUTE_LEAN), handed_back_to_three_pass=n(m.FLAG_ROUTE_HANDED_BACK),
+    routes = dict(one_sweep_no_top_k=n(m.FLAG_ROUTE_LEAN), short_list_top_k=n(m.FLAG_ROUTE_SHORT), handed_back_to_three_pass=n(m.FLAG_ROUTE_HANDED_BACK),
                   exact_multi_pass=n(m.FLAG_ROUTE_EXACT), read_again=n(m.FLAG_ROUTE_REDONE), split_row_done_alone=n(m.FLAG_ROUTE_SPLIT_ALONE))
     return dict(device_near_flags=n(m.FLAG_NEAR), device_failed_rows=n(m.FLAG_OVERFLOW | m.FLAG_BAD_PARAM | m.FLAG_ALL_MASKED),
                 routes=routes)
@@ -236,9 +236,10 @@ def run_workload(name, steps, warmup, check_rows, top_k_array=False):
     smp, wall_ms, kern_ms, warm_ms, n_rot = time_gpu(c, steps, warmup, top_k_array=top_k_array)
     par = parity_sample(c, smp, check_rows) if check_rows else device_report(smp)
     ab = algorithmic_bytes(c)
-    lean = par["routes"]["one_sweep_no_top_k"] + par["routes"]["handed_back_to_three_pass"] > 0
+    lean = par["routes"]["one_sweep_no_top_k"] > 0
+    short = par["routes"]["short_list_top_k"] > 0
     return c, dict(workload=name + (" (top_k: an array of zeros)" if top_k_array else ""), rows=c["rows"], vocab=c["V"], dtype=c["dtype"],
-                   kernel="ws::lean_batch_kernel" if lean else "ws::sample_batch_kernel", ms_per_step=wall_ms, kernel_ms=kern_ms,
+                   kernel="ws::lean_batch_kernel" if lean else ("ws::short_batch_kernel" if short else "ws::sample_batch_kernel"), ms_per_step=wall_ms, kernel_ms=kern_ms,
                    kernel_ms_warm=warm_ms, logits_copies_rotated=n_rot,
                    rows_per_s=c["rows"] / (wall_ms * 1e-3), algorithmic_MB=ab / 1e6, achieved_GBs=ab / (kern_ms * 1e-3) / 1e9,
                    achieved_GBs_warm=ab / (warm_ms * 1e-3) / 1e9,

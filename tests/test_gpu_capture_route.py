@@ -16,7 +16,7 @@ def _both(c, kept_cap=2048, launches=2):
     d = gc.upload(c)
     out = []
     for use in (True, False):
-        smp = gc.sampler_for(c, d, 1, kept_cap=kept_cap, use_workspace=use)
+        smp = gc.sampler_for(c, d, 1, kept_cap=kept_cap, use_workspace=use, top_k_max=0)  # (top_k_max 0: not the short-list kernel, whose rows need no tables)
         for _ in range(launches):  # the second launch finds the workspace as the first left it
             smp.token.fill_(-7)
             smp.run()
@@ -75,7 +75,7 @@ def test_what_a_launch_does_with_the_workspace_is_reported():
     for rows, n_hist in ((1, 300), (1, 8192), (256, 300)):
         c = gc.make_cfg2(rows=rows, V=151936, n_hist=n_hist, n_bias=0) if rows == 1 else gc.make_tile(rows=rows, n_hist=n_hist)
         d = gc.upload(c)
-        smp = gc.sampler_for(c, d, 1, kept_cap=256)
+        smp = gc.sampler_for(c, d, 1, kept_cap=256, top_k_max=0)
         use = m.lib().ws_sample_batch_workspace_use(smp.desc)
         uses.append(use)
         if use == m.WORK_NONE:

@@ -72,7 +72,7 @@ struct BatchPlan {
     uint32_t lean_total;
     uint32_t lean_fb_tie;
     bool shortlist;       // the short-list kernel takes the batch: every row has a top-k of at most top_k_max (the caller's word)
-    uint32_t short_ab, short_cnt, short_total, short_fb_tie;  // its LDS: bitmap at short_ab, rank words at short_cnt
+    uint32_t short_ab, short_cnt, short_total, short_fb_tie, short_fb_ab;  // its LDS: bitmap at short_ab, rank words at short_cnt
     uint32_t split_log2;  // the most parts per row that pay for this batch
     uint64_t workspace_min;  // split rows: the least that lets them split (no staging areas), 0 when nothing is split
     uint64_t workspace;   // bytes for that
@@ -179,6 +179,7 @@ BatchPlan plan_batch(const ws_batch* b) {
             p.short_ab = 32768u;
             p.short_cnt = static_cast<uint32_t>(32768u + maps_s);
             p.short_fb_tie = 0;
+            p.short_fb_ab = static_cast<uint32_t>(three - maps);
             if (three + spare_bytes + kStaticShort <= kMaxLds) {
                 p.short_fb_tie = static_cast<uint32_t>((three + 15u) & ~uint64_t{15});
                 if (p.short_fb_tie + spare_bytes > st) st = p.short_fb_tie + spare_bytes;
@@ -556,6 +557,7 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
         a.lds_ab = p.short_ab;
         a.lds_cnt = p.short_cnt;
         a.fb_lds_tie = p.short_fb_tie;
+        a.fb_lds_ab = p.short_fb_ab;
         a.work = a.split_log2 ? work : nullptr;
         return ws::launch_short(S(stream), a, b->rows << a.split_log2, p.short_total, kMaxLds - kStaticShort);
     }
@@ -564,6 +566,7 @@ int sample_batch_on(void* stream, const ws_batch* b, const BatchPlan& p, unsigne
     if (p.lean) {
         a.lds_tie = p.lean_tie;
         a.fb_lds_tie = p.lean_fb_tie;
+        a.fb_lds_ab = 65536u;
         return ws::launch_lean(S(stream), a, b->rows, p.lean_total, kMaxLds - kStaticLean);
     }
     if (p.fused) return (a.kept_ids ? ws::launch_fused_kept : ws::launch_fused)(S(stream), a, b->rows, p.lds_total, kMaxLds - kStaticLds);

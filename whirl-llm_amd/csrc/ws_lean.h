@@ -1261,7 +1261,7 @@ template <bool KEPT>  // (KEPT: the build that can write the kept-set dump)
 __device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
     BatchArgs B;
     __builtin_memcpy(&B, (const void*)Ap, sizeof(BatchArgs));
-    B.lds_ab = 65536u;
+    B.lds_ab = B.fb_lds_ab;
     B.lds_cnt = 0u;
     B.lds_tie = B.fb_lds_tie;
     B.two_sweep = 1;

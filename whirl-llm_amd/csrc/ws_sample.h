@@ -99,7 +99,8 @@ struct BatchArgs {
     uint32_t split_spins;      // split rows: looks at the arrival counter before a part gives up on the others (0: about a second's worth)
     uint32_t split_row_bytes;  // kSplitRowBytes, or kSplitRowBytesKept when the rows have a staging area
     uint32_t stage_cap;        // entries of a row's staging area (kSplitStageCap), 0: none
-    uint32_t fb_lds_tie;       // the lean kernel: lds_tie of the three-pass code it hands rows back to
+    uint32_t fb_lds_tie;       // the lean and the short-list kernel: lds_tie and lds_ab of the three-pass code they hand rows back to
+    uint32_t fb_lds_ab;
 };
 
 // Global memory of a split row: the merged histogram, the merged candidate list, and four control words (parts that
@@ -111,11 +112,11 @@ constexpr uint32_t kSplitHist = 0u, kSplitList = 32768u, kSplitCtrl = 65536u, kS
 // row again. Control words 4 (entries staged), 8 + part (where the part's entries start) and 24 + part (how many).
 constexpr uint32_t kSplitStage = kSplitRowBytes, kSplitStageCap = 8192u, kSplitRowBytesKept = kSplitStage + kSplitStageCap * 8u;
 // The short-list kernel (ws_short.h). Global memory of a row shared by several workgroups (zero-filled once, left
-// zero-filled): kShortCap keys - the tokens a row lists, all parts together -, then 64 + 4 * 16 words: [0] parts arrived,
-// [1] keys listed, [2] a part could not list its slice; from word 64 on, four words a part: maximum (as an order key),
-// threshold (order key), and the part's sum as a double against its maximum.
+// zero-filled): kShortCap keys - the tokens a row lists, a stretch of kShortCap / parts for each part -, then 64 + 8 * 16
+// words: [0] parts arrived; from word 64 on, eight words a part: maximum (as an order key), threshold (order key), the
+// part's sum as a double against its maximum, and how many keys it listed (all bits set: it could not list its slice).
 constexpr uint32_t kShortCap = 4096u;
-constexpr uint32_t kShortSplitCtrl = kShortCap * 8u, kShortSplitRowBytes = kShortSplitCtrl + 4u * (64u + 4u * 16u);
+constexpr uint32_t kShortSplitCtrl = kShortCap * 8u, kShortSplitRowBytes = kShortSplitCtrl + 4u * (64u + 8u * 16u);
 // Workspace of one row of the three-pass kernel: per history / bias entry a word of each of phase 0's two rank
 // tables, which sit out the first sweep there. Whole memory lines, so that rows share none.
 __host__ __device__ constexpr uint64_t capture_row_bytes(uint32_t patch_cap) {

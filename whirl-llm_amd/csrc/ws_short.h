@@ -21,11 +21,22 @@
 namespace ws {
 
 constexpr uint32_t kShortMaxK = 1024u;  // largest top-k: one candidate a thread in the finish
-constexpr uint32_t kShortHead = 8u;     // head of a slice: vectors a thread (the threshold is fitted to these tokens)
+constexpr uint32_t kShortHead = 8u;     // head of a slice: vectors a thread asked for before anything else
+constexpr uint32_t kShortSample = 8u;   // of those, the vectors a thread whose tokens the threshold is fitted to (32768 tokens of fp32)
 constexpr uint32_t kRouteShort = 0x2000u;
 
 
+#ifdef WS_SHORT_TIMERS
+#define WSS_MARK(k) \
+    if (threadIdx.x == 0) S.marks[k] = static_cast<float>(clock64() - wss_t0)
+#else
+#define WSS_MARK(k)
+#endif
+
 struct ShortShared {
+#ifdef WS_SHORT_TIMERS
+    float marks[16];
+#endif
     double red_d[WS_WAVES];
     double s_d[8];
     unsigned long long s_q[4];
@@ -43,6 +54,9 @@ struct ShortShared {
 template <int DT, bool MASKED>
 __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row, const uint32_t part, const uint32_t n_parts, ShortShared& S,
                                           bool& finisher) {
+#ifdef WS_SHORT_TIMERS
+    const long long wss_t0 = clock64();
+#endif
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr uint32_t TPV = DT == 0 ? 4u : 8u;  // tokens in a 128-bit vector
     const uint32_t t = threadIdx.x, lane = t & 63u;
@@ -67,11 +81,16 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     const uint32_t tok0 = j0 * TPV, tok1 = j1 * TPV;
 
     // the head of the slice is asked for before anything else
+    // (every load of the row is unconditional, its index clamped to the slice, and brings the vector's word of the allow
+    // mask with it: a load behind a branch makes the compiler wait for every load before it)
     uint4 hq[kShortHead];
+    uint32_t hna[kShortHead];
 #pragma unroll
     for (uint32_t k = 0; k < kShortHead; ++k) {
         const uint32_t j = j0 + k * WS_BLOCK + t;
-        hq[k] = xv[j < j1 ? j : (j1 > j0 ? j1 - 1u : 0u)];
+        const uint32_t jc = j < j1 ? j : (j1 > j0 ? j1 - 1u : 0u);
+        hq[k] = xv[jc];
+        hna[k] = MASKED ? allow[(jc * TPV) >> 5] : 0xffffffffu;
     }
     for (uint32_t b = t; b < 4096u; b += WS_BLOCK) head_cnt[b] = 0u;
 
@@ -121,6 +140,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         P.pres = A.pres ? __uint_as_float(v_pres) : 0.f;
         P.freq = A.freq ? __uint_as_float(v_freq) : 0.f;
     }
+    WSS_MARK(0);  // parameters in
     const float inv_t = P.inv_t;
     const uint32_t top_k = P.top_k, nh = P.nh, nb = P.nb;
     const double top_p = P.top_p, min_p = P.min_p;
@@ -133,40 +153,55 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 
     // ---- the bitmap of the touched tokens, their ranks, per-rank history counts and bias entries (phase 0 of ws_sample.h)
     uint32_t n_touched = 0;
+    constexpr uint32_t kIds = 4u;  // ids a thread keeps in registers: the first 4096 of the history, the first 1024 bias entries
+    uint32_t hid[kIds], bid = 0xffffffffu;
     if (!not_mine && nh + nb > 0u) {
+#pragma unroll
+        for (uint32_t k = 0; k < kIds; ++k) hid[k] = k * WS_BLOCK + t < nh ? static_cast<uint32_t>(hist_ids[k * WS_BLOCK + t]) : 0xffffffffu;
+        if (t < nb) bid = static_cast<uint32_t>(bias_ids[t]);
         for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
         for (uint32_t r = t; r < nh + nb; r += WS_BLOCK) {
             cnt[r] = 0u;
             first[r] = 0xffffu;
         }
         __syncthreads();
-        for (uint32_t j = t; j < nh; j += WS_BLOCK) {
-            const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
+        auto mark = [&](uint32_t id) {
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
-        }
-        for (uint32_t j = t; j < nb; j += WS_BLOCK) {
-            const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
-            if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
+        };
+#pragma unroll
+        for (uint32_t k = 0; k < kIds; ++k)
+            if (k * WS_BLOCK < nh) mark(hid[k]);
+        for (uint32_t j = kIds * WS_BLOCK + t; j < nh; j += WS_BLOCK) mark(static_cast<uint32_t>(hist_ids[j]));
+        mark(bid);
+        for (uint32_t j = WS_BLOCK + t; j < nb; j += WS_BLOCK) mark(static_cast<uint32_t>(bias_ids[j]));
+        __syncthreads();
+        // popcount prefixes: five consecutive words a thread and round (one round up to 163840 tokens)
+        constexpr uint32_t kChunk = 5u;
+        uint32_t run_total = 0;
+        for (uint32_t w0 = 0; w0 < nW; w0 += kChunk * WS_BLOCK) {
+            const uint32_t wb = w0 + t * kChunk;
+            uint32_t wd[kChunk], local = 0;
+#pragma unroll
+            for (uint32_t k = 0; k < kChunk; ++k) {
+                wd[k] = wb + k < nW ? touched[wb + k] : 0u;
+                local += __popc(wd[k]);
+            }
+            uint32_t total;
+            uint32_t run = run_total + block_excl_scan(local, S.red_u, &total);
+#pragma unroll
+            for (uint32_t k = 0; k < kChunk; ++k) {
+                if (wb + k < nW) wprefix[wb + k] = static_cast<uint16_t>(run);
+                run += __popc(wd[k]);
+            }
+            run_total += total;
         }
         __syncthreads();
-        uint32_t run_total = 0;
-        for (uint32_t w0 = 0; w0 < nW; w0 += WS_BLOCK) {  // (a vocabulary of up to 32768 * 32 tokens: a few rounds)
-            const uint32_t w = w0 + t;
-            const uint32_t wd = w < nW ? touched[w] : 0u;
-            uint32_t total;
-            const uint32_t before = block_excl_scan(static_cast<uint32_t>(__popc(wd)), S.red_u, &total);
-            if (w < nW) wprefix[w] = static_cast<uint16_t>(run_total + before);
-            run_total += total;
-            __syncthreads();
-        }
         n_touched = run_total;
         auto rank = [&](uint32_t id) { return static_cast<uint32_t>(wprefix[id >> 5]) + __popc(touched[id >> 5] & ((1u << (id & 31u)) - 1u)); };
-        for (uint32_t j = t; j < nh; j += WS_BLOCK) {
-            const uint32_t id = static_cast<uint32_t>(hist_ids[j]);
+        auto count = [&](uint32_t id) {
             if (id < V) atomicAdd(&cnt[rank(id)], 1u);
-        }
-        for (uint32_t j = t; j < nb; j += WS_BLOCK) {
-            const uint32_t id = static_cast<uint32_t>(bias_ids[j]);
+        };
+        auto bias_entry = [&](uint32_t id, uint32_t j) {
             if (id < V) {
                 const uint32_t r = rank(id);
                 atomicAdd(&cnt[r], 1u << 20);
@@ -175,21 +210,28 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 const uint32_t sh = (r & 1u) * 16u;
                 uint32_t seen = *w32;
                 while (((seen >> sh) & 0xffffu) > j) {
-                    const uint32_t want = (seen & ~(0xffffu << sh)) | (j << sh);
-                    const uint32_t got = atomicCAS(w32, seen, want);
+                    const uint32_t want_w = (seen & ~(0xffffu << sh)) | (j << sh);
+                    const uint32_t got = atomicCAS(w32, seen, want_w);
                     if (got == seen) break;
                     seen = got;
                 }
             }
-        }
+        };
+#pragma unroll
+        for (uint32_t k = 0; k < kIds; ++k)
+            if (k * WS_BLOCK < nh) count(hid[k]);
+        for (uint32_t j = kIds * WS_BLOCK + t; j < nh; j += WS_BLOCK) count(static_cast<uint32_t>(hist_ids[j]));
+        bias_entry(bid, t);
+        for (uint32_t j = WS_BLOCK + t; j < nb; j += WS_BLOCK) bias_entry(static_cast<uint32_t>(bias_ids[j]), j);
         __syncthreads();
     }
 
+    WSS_MARK(1);  // bitmap done
     // one vector: its tokens as floats, masked-out / touched / NaN ones as -inf
-    auto unpack = [&](const uint4& q, uint32_t j, float (&x)[TPV]) {
+    auto unpack = [&](const uint4& q, uint32_t na, uint32_t j, float (&x)[TPV]) {
         const uint32_t i0 = j * TPV;
         uint32_t invalid = 0u;  // bit e: token e does not count here
-        if (MASKED) invalid = ~(allow[i0 >> 5] >> (i0 & 31u));
+        if (MASKED) invalid = ~(na >> (i0 & 31u));
         if (n_touched) invalid |= touched[i0 >> 5] >> (i0 & 31u);
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
@@ -200,16 +242,33 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         }
     };
 
+    // the first two batches behind the head are asked for now: they travel while the threshold is worked out
+    constexpr uint32_t KB = 4;  // vectors a thread and batch, two batches in flight
+    uint4 qa[KB], qb[KB];
+    uint32_t naa[KB], nab[KB];
+    const uint32_t jb = j0 + kShortHead * WS_BLOCK;
+    auto load = [&](uint4 (&q)[KB], uint32_t (&na)[KB], uint32_t jbase) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t k = 0; k < KB; ++k) {
+            const uint32_t j = jbase + k * WS_BLOCK + t;
+            const uint32_t jc = j < j1 ? j : (j1 > j0 ? j1 - 1u : 0u);
+            q[k] = xv[jc];
+            na[k] = MASKED ? allow[(jc * TPV) >> 5] : 0xffffffffu;
+        }
+    };
+    load(qa, naa, jb);
+    load(qb, nab, jb + KB * WS_BLOCK);
+
     // ---- the threshold: the head's logits counted in 4096 bins of 1/64 e-fold below the head's maximum
     float ref = -INFINITY;
-    const uint32_t n_head_vec = min(j1 - j0, kShortHead * WS_BLOCK);
+    const uint32_t n_head_vec = min(j1 - j0, kShortSample * WS_BLOCK);
     {
         float x[TPV];
 #pragma unroll
-        for (uint32_t k = 0; k < kShortHead; ++k) {
+        for (uint32_t k = 0; k < kShortSample; ++k) {
             const uint32_t j = j0 + k * WS_BLOCK + t;
             if (j < j1) {
-                unpack(hq[k], j, x);
+                unpack(hq[k], hna[k], j, x);
 #pragma unroll
                 for (uint32_t e = 0; e < TPV; ++e) ref = fmaxf(ref, x[e]);
             }
@@ -218,45 +277,59 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     }
     const float c64 = inv_t * 64.f;
     float thr = -INFINITY;  // tokens above it are listed
-    const uint32_t want = (3u * top_k + 64u + n_parts - 1u) / n_parts + 32u;  // tokens this part aims to list
+    // tokens this part aims to list (a shared row's part has room for kShortCap / n_parts of them)
+    // (The count above a threshold fitted to a sample of the slice scatters like the square root of the sample's rank:
+    // half of top_k on top, 150 at least. When the sample is the whole slice - a row shared by many - the count is
+    // exact up to a bin's tokens, and what matters is that no part holds more of the row's top_k than it lists: twice
+    // its share and a dozen.)
     const uint32_t n_slice = tok1 - tok0, n_head = n_head_vec * TPV;
+    const uint32_t want = n_head >= n_slice ? 2u * ((top_k + n_parts - 1u) / n_parts) + 12u
+                                            : (top_k + max(top_k >> 1, 150u) + n_parts - 1u) / n_parts + 16u;
     bool list_all = n_head >= n_slice && want >= n_slice;
     if (!not_mine && ref > -INFINITY && !list_all) {
-        float x[TPV];
-#pragma unroll
-        for (uint32_t k = 0; k < kShortHead; ++k) {
-            const uint32_t j = j0 + k * WS_BLOCK + t;
-            if (j < j1) {
-                unpack(hq[k], j, x);
-#pragma unroll
-                for (uint32_t e = 0; e < TPV; ++e) {
-                    const float d = fminf(__fmul_rn(__fsub_rn(ref, x[e]), c64), 4095.f);  // (-inf, and anything 64 e-folds down: the last bin)
-                    atomicAdd(&head_cnt[static_cast<uint32_t>(d)], 1u);
-                }
-            }
-        }
-        __syncthreads();
         // rank in the head that about `want` tokens of the slice lie above
         const uint64_t r_star64 = (static_cast<uint64_t>(n_head) * want + n_slice - 1u) / n_slice;
         const uint32_t r_star = static_cast<uint32_t>(r_star64 < 4u ? 4u : r_star64);
-        const uint4 c4 = *reinterpret_cast<const uint4*>(&head_cnt[4u * t]);
-        const uint32_t mine = c4.x + c4.y + c4.z + c4.w;
-        uint32_t total;
-        const uint32_t before = block_excl_scan(mine, S.red_u, &total);
-        if (t == 0) S.s_w[0] = 0xffffffffu;
-        __syncthreads();
-        if (before < r_star && before + mine >= r_star) {  // the bin in which the head's r_star-th largest lies
-            uint32_t run = before, b = 4u * t;
-            const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
+        // The bins near the top are all that matters (the r_star-th largest of the head is one of its largest per cent
+        // or so): first only the tokens within 8 e-folds of the head's maximum are counted - an LDS atomic each, and a
+        // sixth of the tokens -, the others only when those turn out to be fewer than r_star.
+        constexpr float kNear = 512.f;
+        uint32_t b_star = 0xffffffffu;
+        for (int round = 0; round < 2; ++round) {  // uniform
+            float x[TPV];
 #pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) {
-                if (run < r_star && run + c[k] >= r_star) b = 4u * t + k;
-                run += c[k];
+            for (uint32_t k = 0; k < kShortSample; ++k) {
+                const uint32_t j = j0 + k * WS_BLOCK + t;
+                if (j < j1) {
+                    unpack(hq[k], hna[k], j, x);
+#pragma unroll
+                    for (uint32_t e = 0; e < TPV; ++e) {
+                        const float d = fminf(__fmul_rn(__fsub_rn(ref, x[e]), c64), 4095.f);  // (-inf, and anything 64 e-folds down: the last bin)
+                        if (round == 0 ? d < kNear : d >= kNear) atomicAdd(&head_cnt[static_cast<uint32_t>(d)], 1u);
+                    }
+                }
             }
-            S.s_w[0] = b;
+            __syncthreads();
+            const uint4 c4 = *reinterpret_cast<const uint4*>(&head_cnt[4u * t]);
+            const uint32_t mine = c4.x + c4.y + c4.z + c4.w;
+            uint32_t total;
+            const uint32_t before = block_excl_scan(mine, S.red_u, &total);
+            if (t == 0) S.s_w[0] = 0xffffffffu;
+            __syncthreads();
+            if (before < r_star && before + mine >= r_star) {  // the bin in which the head's r_star-th largest lies
+                uint32_t run = before, b = 4u * t;
+                const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    if (run < r_star && run + c[k] >= r_star) b = 4u * t + k;
+                    run += c[k];
+                }
+                S.s_w[0] = b;
+            }
+            __syncthreads();
+            b_star = S.s_w[0];
+            if (b_star != 0xffffffffu) break;
         }
-        __syncthreads();
-        const uint32_t b_star = S.s_w[0];
         if (b_star >= 4095u) list_all = true;  // (fewer than r_star tokens above the last bin: everything is listed)
         else thr = __fsub_rn(ref, __fdiv_rn(static_cast<float>(b_star + 1u), c64));
         __syncthreads();
@@ -268,32 +341,27 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     }
     __syncthreads();
 
+    WSS_MARK(2);  // threshold known
     // ---- the sweep: maximum, sum of exp against `ref`, tokens above the threshold to the list
     const float k2 = inv_t * 1.44269504088896340736f;
     const float k2lo = static_cast<float>(static_cast<double>(inv_t) * 1.44269504088896340736 - static_cast<double>(k2));
     float m = -INFINITY, s = 0.f;
-    auto push = [&](float x, uint32_t id, bool yes) {  // wave-aggregated
-        const uint64_t mk = __ballot(yes);
-        if (mk) {
-            uint32_t b = 0;
-            if (lane == static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(mk)) - 1)) b = atomicAdd(&S.s_w[1], static_cast<uint32_t>(__popcll(mk)));
-            b = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(__shfl(static_cast<int>(b), __ffsll(static_cast<unsigned long long>(mk)) - 1))));
-            const uint32_t slot = b + static_cast<uint32_t>(__popcll(mk & ((1ull << lane) - 1ull)));
-            if (yes) {
-                if (slot < kShortCap) list[slot] = key64(x, id);
-                else S.s_w[2] = 1u;
-            }
+    auto push = [&](float x, uint32_t id, bool yes) {  // (one LDS atomic a listed token: they are few)
+        if (yes) {
+            const uint32_t slot = atomicAdd(&S.s_w[1], 1u);
+            if (slot < kShortCap) list[slot] = key64(x, id);
+            else S.s_w[2] = 1u;
         }
     };
-    auto take = [&](const uint4& q, uint32_t j) {
+    auto take = [&](const uint4& q, uint32_t na, uint32_t j) {
         float x[TPV];
-        unpack(q, j, x);
+        unpack(q, na, j, x);
         float vm = -INFINITY;
 #pragma unroll
         for (uint32_t e = 0; e < TPV; ++e) {
             vm = fmaxf(vm, x[e]);
             const float a = fmaxf(__fsub_rn(x[e], ref), -1e30f);
-            s += exp2f(fmaf(a, k2lo, a * k2));
+            s += __builtin_amdgcn_exp2f(fmaf(a, k2lo, a * k2));  // (v_exp_f32: arguments below -126 give 0, which is what they are worth)
         }
         m = fmaxf(m, vm);
         if (__ballot(vm > thr)) {  // uniform: a vector with a token for the list (a few per thousand)
@@ -305,63 +373,68 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 #pragma unroll
         for (uint32_t k = 0; k < kShortHead; ++k) {
             const uint32_t j = j0 + k * WS_BLOCK + t;
-            if (j < j1) take(hq[k], j);
+            if (j < j1) take(hq[k], hna[k], j);
         }
-        constexpr uint32_t KB = 4;  // vectors a thread and batch, two batches in flight
-        uint4 qa[KB], qb[KB];
-        const uint32_t jb = j0 + kShortHead * WS_BLOCK;
-        auto load = [&](uint4 (&q)[KB], uint32_t jbase) {
+        auto eat = [&](const uint4 (&q)[KB], const uint32_t (&na)[KB], uint32_t jbase) __attribute__((always_inline)) {
 #pragma unroll
             for (uint32_t k = 0; k < KB; ++k) {
                 const uint32_t j = jbase + k * WS_BLOCK + t;
-                q[k] = xv[j < j1 ? j : j1 - 1u];
-            }
-        };
-        auto eat = [&](const uint4 (&q)[KB], uint32_t jbase) {
-#pragma unroll
-            for (uint32_t k = 0; k < KB; ++k) {
-                const uint32_t j = jbase + k * WS_BLOCK + t;
-                if (j < j1) take(q[k], j);
+                if (j < j1) take(q[k], na[k], j);
             }
         };
         if (jb < j1) {
-            load(qa, jb);
             for (uint32_t jc = jb; jc < j1; jc += 2u * KB * WS_BLOCK) {
-                if (jc + KB * WS_BLOCK < j1) load(qb, jc + KB * WS_BLOCK);
-                eat(qa, jc);
-                if (jc + 2u * KB * WS_BLOCK < j1) load(qa, jc + 2u * KB * WS_BLOCK);
-                if (jc + KB * WS_BLOCK < j1) eat(qb, jc + KB * WS_BLOCK);
+                eat(qa, naa, jc);
+                load(qa, naa, jc + 2u * KB * WS_BLOCK);
+                eat(qb, nab, jc + KB * WS_BLOCK);
+                load(qb, nab, jc + 3u * KB * WS_BLOCK);
             }
         }
     }
 
+    WSS_MARK(3);  // sweep done
     // ---- the touched tokens of the slice: adjusted logit (bias entries in list order, then repetition, then frequency /
     // presence, as ws_sample.h applies them), into the maximum, the sum and - above the threshold - the list
-    double s_adj = 0.0;  // their share of the sum, against `ref`
     if (!not_mine && n_touched) {
         constexpr uint32_t kClaim = 0x80000000u;
         auto rank = [&](uint32_t id) { return static_cast<uint32_t>(wprefix[id >> 5]) + __popc(touched[id >> 5] & ((1u << (id & 31u)) - 1u)); };
-        auto one = [&](uint32_t id) {
-            const bool mine = id < V && id >= tok0 && id < tok1;
-            float x = -INFINITY;
-            bool have = false;
-            if (mine) {
-                const uint32_t r = rank(id);
-                const uint32_t old = atomicOr(&cnt[r], kClaim);
-                if (!(old & kClaim)) {
-                    have = true;
-                    const bool allowed = !MASKED || ((allow[id >> 5] >> (id & 31u)) & 1u);
-                    const float raw = allowed ? fmaxf(DT == 0 ? reinterpret_cast<const float*>(base)[id]
-                                                              : bf16_to_f32(reinterpret_cast<const uint16_t*>(base)[id]), -INFINITY)
-                                              : -INFINITY;
-                    const uint32_t c = old & 0xfffffu, n_bias = (old >> 20) & 0x7ffu;
-                    x = raw;
+        // up to four ids a thread at a time: the claims first, then the claimed tokens' logits all asked for together,
+        // then the arithmetic (n_live: ids left in this round, so that empty slots issue nothing)
+        auto some = [&](const uint32_t (&id)[4], uint32_t n_live) {
+            uint32_t old[4], r[4];
+            float raw[4];
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                old[k] = kClaim;
+                r[k] = 0u;
+                if (k * WS_BLOCK < n_live && id[k] < V && id[k] >= tok0 && id[k] < tok1) {
+                    r[k] = rank(id[k]);
+                    old[k] = atomicOr(&cnt[r[k]], kClaim);
+                }
+            }
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                raw[k] = -INFINITY;
+                if (k * WS_BLOCK < n_live && !(old[k] & kClaim)) {
+                    const bool allowed = !MASKED || ((allow[id[k] >> 5] >> (id[k] & 31u)) & 1u);
+                    if (allowed)
+                        raw[k] = DT == 0 ? reinterpret_cast<const float*>(base)[id[k]] : bf16_to_f32(reinterpret_cast<const uint16_t*>(base)[id[k]]);
+                }
+            }
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                if (k * WS_BLOCK >= n_live) continue;  // uniform
+                const bool have = !(old[k] & kClaim);
+                float x = -INFINITY;
+                if (have) {
+                    const uint32_t c = old[k] & 0xfffffu, n_bias = (old[k] >> 20) & 0x7ffu;
+                    x = fmaxf(raw[k], -INFINITY);
                     if (n_bias) {
-                        uint32_t j = first[r];
+                        uint32_t j = first[r[k]];
                         x = __fadd_rn(x, bias_vals[j]);
                         if (n_bias > 1u)
                             for (++j; j < nb; ++j)
-                                if (static_cast<uint32_t>(bias_ids[j]) == id) x = __fadd_rn(x, bias_vals[j]);
+                                if (static_cast<uint32_t>(bias_ids[j]) == id[k]) x = __fadd_rn(x, bias_vals[j]);
                     }
                     if (c) {
                         x = x > 0.f ? __fdiv_rn(x, P.rep) : __fmul_rn(x, P.rep);
@@ -369,17 +442,32 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                     }
                     x = fmaxf(x, -INFINITY);
                     m = fmaxf(m, x);
-                    if (x > -INFINITY) s_adj += exp(static_cast<double>(__fsub_rn(x, ref)) * static_cast<double>(inv_t));
+                    const float a_ = fmaxf(__fsub_rn(x, ref), -1e30f);
+                    s += __builtin_amdgcn_exp2f(fmaf(a_, k2lo, a_ * k2));
                 }
+                push(x, id[k], have && x > thr);
             }
-            push(x, id, have && x > thr);
         };
-        for (uint32_t j0_ = 0; j0_ < nh; j0_ += WS_BLOCK) one(j0_ + t < nh ? static_cast<uint32_t>(hist_ids[j0_ + t]) : 0xffffffffu);
-        for (uint32_t j0_ = 0; j0_ < nb; j0_ += WS_BLOCK) one(j0_ + t < nb ? static_cast<uint32_t>(bias_ids[j0_ + t]) : 0xffffffffu);
+        uint32_t id4[4];
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; ++k) id4[k] = hid[k];
+        if (nh) some(id4, nh);
+        for (uint32_t jr = kIds * WS_BLOCK; jr < nh; jr += 4u * WS_BLOCK) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) id4[k] = jr + k * WS_BLOCK + t < nh ? static_cast<uint32_t>(hist_ids[jr + k * WS_BLOCK + t]) : 0xffffffffu;
+            some(id4, nh - jr);
+        }
+        for (uint32_t jr = 0; jr < nb; jr += 4u * WS_BLOCK) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k)
+                id4[k] = (jr == 0u && k == 0u) ? bid : (jr + k * WS_BLOCK + t < nb ? static_cast<uint32_t>(bias_ids[jr + k * WS_BLOCK + t]) : 0xffffffffu);
+            some(id4, nb - jr);
+        }
     }
+    WSS_MARK(4);  // touched tokens in
     __syncthreads();
     m = block_max(m, S.red_f);
-    double z = block_sum(static_cast<double>(s) + s_adj, S.red_d);  // against `ref`
+    double z = block_sum(static_cast<double>(s), S.red_d);  // against `ref`
     uint32_t n_list = S.s_w[1];
     bool bad = not_mine || S.s_w[2] != 0u || n_list > kShortCap || !(ref > -INFINITY) || !(m > -INFINITY) || !(__fsub_rn(m, ref) * inv_t < 80.f);
     float thr_max = thr;
@@ -389,71 +477,114 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         unsigned char* work = A.work + static_cast<size_t>(row) * kShortSplitRowBytes;
         uint64_t* glist = reinterpret_cast<uint64_t*>(work);
         uint32_t* ctrl = reinterpret_cast<uint32_t*>(work + kShortSplitCtrl);
+        const uint32_t region = kShortCap / n_parts;  // every part has its own stretch of the list: nothing to reserve
+        if (n_list > region) bad = true;
         if (t == 0) {
-            uint32_t b = 0;
-            if (!bad) b = __hip_atomic_fetch_add(&ctrl[1], n_list, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (bad || b + n_list > kShortCap) __hip_atomic_fetch_or(&ctrl[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            S.s_w[3] = b;
-            S.s_w[4] = (!bad && b + n_list <= kShortCap) ? 1u : 0u;
-            uint32_t* mine = ctrl + 64u + 4u * part;
+            uint32_t* mine = ctrl + 64u + 8u * part;
             __hip_atomic_store(&mine[0], key32(m > -INFINITY ? m : -INFINITY), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(&mine[1], key32(thr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             // the sum against the part's own maximum (against `ref` it may not be a number when the slice holds no token)
             const double zm = m > -INFINITY ? z * exp(static_cast<double>(__fsub_rn(ref, m)) * static_cast<double>(inv_t)) : 0.0;
             __hip_atomic_store(reinterpret_cast<unsigned long long*>(&mine[2]), static_cast<unsigned long long>(__double_as_longlong(zm)),
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&mine[4], bad ? 0xffffffffu : n_list, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __syncthreads();
-        if (S.s_w[4]) {
-            const uint32_t b = S.s_w[3];
+        if (!bad)
             for (uint32_t k = t; k < n_list; k += WS_BLOCK)
-                __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[b + k]), static_cast<unsigned long long>(list[k]), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        }
+                __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[part * region + k]), static_cast<unsigned long long>(list[k]),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's stores have been acknowledged
         __syncthreads();
         if (t == 0) S.s_w[5] = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (S.s_w[5] != n_parts - 1u) return true;  // not the last: done
         finisher = true;
-        // the last part: everybody's results (device-scope loads: no stale copy from this unit's caches)
-        n_list = __hip_atomic_load(&ctrl[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bad = __hip_atomic_load(&ctrl[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u || n_list > kShortCap;
-        float mm = -INFINITY, tt = -INFINITY;
-        for (uint32_t p = 0; p < n_parts; ++p) {
-            mm = fmaxf(mm, unkey32(__hip_atomic_load(&ctrl[64u + 4u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
-            tt = fmaxf(tt, unkey32(__hip_atomic_load(&ctrl[65u + 4u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+        // the last part: everybody's results (device-scope loads: no stale copy from this unit's caches). Lane p of every
+        // wave reads part p's words - all loads on their way at once - and the wave reduces them.
+        float mp = -INFINITY, tp = -INFINITY;
+        double zp = 0.0;
+        uint32_t np = 0u;
+        if (lane < n_parts) {
+            mp = unkey32(__hip_atomic_load(&ctrl[64u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            tp = unkey32(__hip_atomic_load(&ctrl[65u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            zp = __longlong_as_double(static_cast<long long>(
+                __hip_atomic_load(reinterpret_cast<unsigned long long*>(&ctrl[66u + 8u * lane]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+            np = __hip_atomic_load(&ctrl[68u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        double zz = 0.0;
-        for (uint32_t p = 0; p < n_parts; ++p) {
-            const float mp = unkey32(__hip_atomic_load(&ctrl[64u + 4u * p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            const double zp = __longlong_as_double(static_cast<long long>(
-                __hip_atomic_load(reinterpret_cast<unsigned long long*>(&ctrl[66u + 4u * p]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
-            if (mp > -INFINITY) zz += zp * exp(static_cast<double>(__fsub_rn(mp, mm)) * static_cast<double>(inv_t));
+        const float mm = wave_max(mp), tt = wave_max(tp);
+        const double zz = wave_sum(mp > -INFINITY ? zp * exp(static_cast<double>(__fsub_rn(mp, mm)) * static_cast<double>(inv_t)) : 0.0);
+        bad = __ballot(np == 0xffffffffu) != 0ull;
+        const uint32_t np_ok = np == 0xffffffffu ? 0u : np;
+        const uint32_t off = wave_incl_scan(np_ok) - np_ok;  // where part p's keys go in the merged list
+        n_list = wave_sum(np_ok);
+        __syncthreads();  // (everybody is done with its own list)
+        if (wv == 0u && lane < n_parts) {
+            S.red_u[lane] = np_ok;
+            S.s_w[lane & 15u] = off;
         }
+        __syncthreads();
         m = mm;
         thr_max = tt;
-        z = zz;    // against the row's maximum from here on
+        z = zz;  // against the row's maximum from here on
         ref = mm;
-        if (!(m > -INFINITY)) bad = true;
-        __syncthreads();  // (everybody is done with its own list)
-        if (!bad)
-            for (uint32_t k = t; k < n_list; k += WS_BLOCK)
-                list[k] = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[k]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the workspace as the next launch needs it
-        for (uint32_t k = t; k < min(n_list, kShortCap); k += WS_BLOCK)
-            __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[k]), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (t < 64u + 4u * n_parts) __hip_atomic_store(&ctrl[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!(m > -INFINITY) || n_list > kShortCap) bad = true;
+        {
+            constexpr uint32_t kSlots = kShortCap / WS_BLOCK;
+            uint64_t got[kSlots];
+#pragma unroll
+            for (uint32_t i = 0; i < kSlots; ++i) {
+                const uint32_t slot = i * WS_BLOCK + t, p = slot / region, k = slot - p * region;
+                const bool live = k < S.red_u[p];
+                got[i] = live ? __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[slot]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+            }
+#pragma unroll
+            for (uint32_t i = 0; i < kSlots; ++i) {
+                const uint32_t slot = i * WS_BLOCK + t, p = slot / region, k = slot - p * region;
+                if (k < S.red_u[p]) {
+                    if (!bad) list[S.s_w[p] + k] = got[i];
+                    // the workspace as the next launch needs it
+                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[slot]), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        if (t < 64u + 8u * n_parts) __hip_atomic_store(&ctrl[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
     }
+    WSS_MARK(5);  // parts met
     if (bad || n_list < top_k) return false;
 
     // ---- the candidates in order
-    uint32_t P2 = 64u;
-    while (P2 < n_list) P2 <<= 1;
-    for (uint32_t k = n_list + t; k < P2; k += WS_BLOCK) list[k] = 0ull;
-    __syncthreads();
-    sort_desc(list, P2);
+    if (n_list <= WS_BLOCK) {
+        // up to a key a thread: its place is the number of keys above it (all different: the id is part of the key).
+        // Every thread reads the same key at a time, eight reads on their way together; the keys in order go to the
+        // upper half of the list's LDS and back.
+        __syncthreads();
+        const uint64_t mine = t < n_list ? list[t] : 0ull;
+        uint32_t above = 0;
+        const uint32_t n8 = n_list & ~7u;
+        if (wv * 64u < n_list) {  // (per wave: one without a key issues nothing)
+            for (uint32_t i = 0; i < n8; i += 8u) {
+                uint64_t o[8];
+#pragma unroll
+                for (uint32_t k = 0; k < 8u; ++k) o[k] = list[i + k];
+#pragma unroll
+                for (uint32_t k = 0; k < 8u; ++k) above += o[k] > mine ? 1u : 0u;
+            }
+            for (uint32_t i = n8; i < n_list; ++i) above += list[i] > mine ? 1u : 0u;
+        }
+        uint64_t* sorted = list + 2048;
+        if (t < n_list) sorted[above] = mine;
+        __syncthreads();
+        if (t < n_list) list[t] = sorted[t];
+        __syncthreads();
+    } else {
+        uint32_t P2 = 2048u;
+        while (P2 < n_list) P2 <<= 1;
+        for (uint32_t k = n_list + t; k < P2; k += WS_BLOCK) list[k] = 0ull;
+        __syncthreads();
+        sort_desc(list, P2);
+    }
+    WSS_MARK(6);  // sorted
     // the k-th largest has to lie above every threshold (below one, a part may have left out tokens that rank before it)
     const uint64_t key_k = list[top_k - 1u];
     const float x_k = unkey32(static_cast<uint32_t>(key_k >> 32));
@@ -465,76 +596,122 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     const uint64_t key = has ? list[t] : 0ull;
     const float x = has ? unkey32(static_cast<uint32_t>(key >> 32)) : -INFINITY;
     const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key);
-    const double e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;
-    double Zk1;
-    const double cex = block_excl_scan(e, S.red_d, &Zk1);  // mass ranked before this candidate; Zk1: of all top_k
-    const double cin = cex + e;
-    const double u = batch_uniform(A.rng, P.seed, row, P.step, 0);
-    if (t == 0) {
-        S.s_q[0] = ~0ull;  // the top-p cut: first position whose running mass reaches X
-        S.s_q[1] = ~0ull;  // the draw
-        S.s_w[6] = 0u;     // candidates at or above the min-p floor
-        S.s_d[0] = 1.0;    // margins: top-p, min-p (two neighbours)
-        S.s_d[1] = 1.0;
-        S.s_d[2] = 1.0;
-    }
-    __syncthreads();
-    const double X = top_p * Zk1;
-    if (use_top_p && has && cin >= X && !(cex >= X)) atomicMin(&S.s_q[0], static_cast<unsigned long long>(t));
-    if (use_min_p) {
-        const uint64_t np = __ballot(has && e >= min_p);
-        if (lane == 0u && np) atomicAdd(&S.s_w[6], static_cast<uint32_t>(__popcll(np)));
-    }
-    __syncthreads();
-    uint32_t n2 = top_k;
-    double mg_top_p = 1.0, mg_min_p = 1.0;
-    if (use_top_p) {
-        const unsigned long long cq = S.s_q[0];
-        if (cq != ~0ull) n2 = static_cast<uint32_t>(cq) + 1u;
-        else mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
-        if (has && t == n2 - 1u && cq != ~0ull) S.s_d[0] = fmin(cin - X, t > 0u ? X - cex : X) / X;
-    }
-    uint32_t n3 = n2;
-    if (use_min_p) {
-        const uint32_t passed = S.s_w[6];  // (a prefix of the order: masses do not rise along it)
-        n3 = min(n2, passed);
-        if (n3 < 1u) n3 = 1u;
-        if (has && passed > 0u && t == passed - 1u) S.s_d[1] = fabs(e - min_p) / min_p;
-        if (has && t == passed && passed < top_k) S.s_d[2] = fabs(e - min_p) / min_p;
-    }
-    if (has && t == n3 - 1u) S.s_d[3] = cin;  // mass of the kept set
-    __syncthreads();
-    if (use_top_p && mg_top_p != 0.0) mg_top_p = S.s_d[0];
-    if (use_min_p) mg_min_p = fmin(S.s_d[1], S.s_d[2]);
-    const double Zk = S.s_d[3];
-    const double target = u * Zk;
-    if (has && t < n3 && cin > target && !(cex > target)) atomicMin(&S.s_q[1], static_cast<unsigned long long>(t));
-    __syncthreads();
-    const unsigned long long dq = S.s_q[1];
-    const uint32_t d_pos = dq != ~0ull ? static_cast<uint32_t>(dq) : n3 - 1u;  // (src/sampling/sampler.cpp:131: the walk falls through to the last kept)
     typedef const __attribute__((address_space(4))) BatchArgs* ArgPtr;
     ArgPtr Ap = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
-    if (has && t == d_pos) {
-        const double mg = dq != ~0ull ? fmin(cin - target, t > 0u ? target - cex : 1e300) / Zk : 0.0;
+    const double u = batch_uniform(A.rng, P.seed, row, P.step, 0);
+    uint32_t n3;
+    auto write_out = [&](double e_, double cin_, double cex_, double Zk_, double target_, bool drawn, double mg_top_p_, double mg_min_p_, uint32_t pos) {
+        const double mg = drawn ? fmin(cin_ - target_, pos > 0u ? target_ - cex_ : 1e300) / Zk_ : 0.0;
         const double tol = Ap->tol;
         uint32_t flags = kRouteShort;
-        if (mg_top_p < tol) flags |= kNearTopP;
-        if (mg_min_p < tol) flags |= kNearMinP;
+        if (mg_top_p_ < tol) flags |= kNearTopP;
+        if (mg_min_p_ < tol) flags |= kNearMinP;
         if (mg < tol) flags |= kNearDraw;
         Ap->token[row] = static_cast<int32_t>(id);
         Ap->flags[row] = flags;
-        if (Ap->prob) Ap->prob[row] = static_cast<float>(e / Zk);
+        if (Ap->prob) Ap->prob[row] = static_cast<float>(e_ / Zk_);
         if (Ap->n_kept) Ap->n_kept[row] = n3;
         if (Ap->stats) {
             Ap->stats[2 * row] = m;
             Ap->stats[2 * row + 1] = static_cast<float>(z * exp(static_cast<double>(__fsub_rn(ref, m)) * static_cast<double>(inv_t)));
         }
         if (Ap->margin) {
-            Ap->margin[3 * row] = mg_top_p;
-            Ap->margin[3 * row + 1] = mg_min_p;
+            Ap->margin[3 * row] = mg_top_p_;
+            Ap->margin[3 * row + 1] = mg_min_p_;
             Ap->margin[3 * row + 2] = mg;
         }
+    };
+    if (top_k <= 64u) {
+        // the usual case, a top-k of a few dozen: one wave, a candidate a lane, no barrier and no atomic
+        if (wv == 0u) {
+            const double e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;
+            const double cin = wave_incl_scan(e);
+            const double up = __shfl_up(cin, 1);
+            const double cex = lane ? up : 0.0;
+            const double Zk1 = lane_value(cin, top_k - 1u);
+            const double X = top_p * Zk1;
+            uint32_t n2 = top_k;
+            double mg_top_p = 1.0, mg_min_p = 1.0;
+            if (use_top_p) {
+                const uint64_t cm = __ballot(has && cin >= X && !(cex >= X));
+                if (cm) {
+                    const uint32_t jc = static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(cm)) - 1);
+                    n2 = jc + 1u;
+                    const double ci = lane_value(cin, jc), ce = lane_value(cex, jc);
+                    mg_top_p = fmin(ci - X, jc > 0u ? X - ce : X) / X;
+                } else {
+                    mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
+                }
+            }
+            n3 = n2;
+            if (use_min_p) {
+                const uint32_t passed = static_cast<uint32_t>(__popcll(__ballot(has && e >= min_p)));  // (a prefix of the order: masses do not rise along it)
+                n3 = min(n2, passed);
+                if (n3 < 1u) n3 = 1u;
+                const double near = fabs(e - min_p) / min_p;
+                if (passed > 0u) mg_min_p = fmin(mg_min_p, lane_value(near, passed - 1u));
+                if (passed < top_k) mg_min_p = fmin(mg_min_p, lane_value(near, passed));
+            }
+            const double Zk = lane_value(cin, n3 - 1u);
+            const double target = u * Zk;
+            const uint64_t dm = __ballot(has && lane < n3 && cin > target && !(cex > target));
+            const uint32_t d_pos = dm ? static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(dm)) - 1) : n3 - 1u;  // (src/sampling/sampler.cpp:131: the walk falls through to the last kept)
+            if (lane == d_pos) write_out(e, cin, cex, Zk, target, dm != 0ull, mg_top_p, mg_min_p, d_pos);
+            if (lane == 0u) S.s_w[7] = n3;
+        }
+        __syncthreads();
+        n3 = S.s_w[7];
+    } else {
+        double e = 0.0;
+        if (wv * 64u < top_k) e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;  // (per wave: the exponential is a hundred instructions)
+        double Zk1;
+        const double cex = block_excl_scan(e, S.red_d, &Zk1);  // mass ranked before this candidate; Zk1: of all top_k
+        const double cin = cex + e;
+        if (t == 0) {
+            S.s_q[0] = ~0ull;  // the top-p cut: first position whose running mass reaches X
+            S.s_q[1] = ~0ull;  // the draw
+            S.s_w[6] = 0u;     // candidates at or above the min-p floor
+            S.s_d[0] = 1.0;    // margins: top-p, min-p (two neighbours)
+            S.s_d[1] = 1.0;
+            S.s_d[2] = 1.0;
+        }
+        __syncthreads();
+        const double X = top_p * Zk1;
+        if (use_top_p && has && cin >= X && !(cex >= X)) atomicMin(&S.s_q[0], static_cast<unsigned long long>(t));
+        if (use_min_p) {
+            const uint64_t np = __ballot(has && e >= min_p);
+            if (lane == 0u && np) atomicAdd(&S.s_w[6], static_cast<uint32_t>(__popcll(np)));
+        }
+        __syncthreads();
+        uint32_t n2 = top_k;
+        double mg_top_p = 1.0, mg_min_p = 1.0;
+        if (use_top_p) {
+            const unsigned long long cq = S.s_q[0];
+            if (cq != ~0ull) n2 = static_cast<uint32_t>(cq) + 1u;
+            else mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
+            if (has && t == n2 - 1u && cq != ~0ull) S.s_d[0] = fmin(cin - X, t > 0u ? X - cex : X) / X;
+        }
+        n3 = n2;
+        if (use_min_p) {
+            const uint32_t passed = S.s_w[6];  // (a prefix of the order: masses do not rise along it)
+            n3 = min(n2, passed);
+            if (n3 < 1u) n3 = 1u;
+            if (has && passed > 0u && t == passed - 1u) S.s_d[1] = fabs(e - min_p) / min_p;
+            if (has && t == passed && passed < top_k) S.s_d[2] = fabs(e - min_p) / min_p;
+        }
+        if (has && t == n3 - 1u) S.s_d[3] = cin;  // mass of the kept set
+        __syncthreads();
+        if (use_top_p && mg_top_p != 0.0) mg_top_p = S.s_d[0];
+        if (use_min_p) mg_min_p = fmin(S.s_d[1], S.s_d[2]);
+        const double Zk = S.s_d[3];
+        const double target = u * Zk;
+        if (has && t < n3 && cin > target && !(cex > target)) atomicMin(&S.s_q[1], static_cast<unsigned long long>(t));
+        __syncthreads();
+        const unsigned long long dq = S.s_q[1];
+        const uint32_t d_pos = dq != ~0ull ? static_cast<uint32_t>(dq) : n3 - 1u;  // (src/sampling/sampler.cpp:131: the walk falls through to the last kept)
+        if (has && t == d_pos) write_out(e, cin, cex, Zk, target, dq != ~0ull, mg_top_p, mg_min_p, d_pos);
     }
+    WSS_MARK(7);  // drawn
     // ---- the kept set in ascending id order (the first kept_cap of it): each kept candidate counts the kept ids below its own
     if (Ap->kept_ids) {
         uint32_t* kid = reinterpret_cast<uint32_t*>(lds + 32768u - 4096u);  // (behind the sorted keys the finish uses: top_k <= 1024 of 4096 places)
@@ -550,6 +727,11 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             }
         }
     }
+#ifdef WS_SHORT_TIMERS
+    WSS_MARK(8);
+    __syncthreads();
+    if (t < 16 && Ap->kept_logits) Ap->kept_logits[static_cast<size_t>(row) * Ap->kept_cap + 100u + t] = t == 15 ? static_cast<float>(n_list) : S.marks[t];
+#endif
     return true;
 }
 
