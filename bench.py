@@ -55,10 +55,10 @@ def checker():
 
 
 def kernel_digest():
-    """sha256[:16] over the sources of the two sampler kernels (ws_sample.h, then ws_lean.h)."""
+    """sha256[:16] over the sources of the sampler kernels (ws_sample.h, ws_lean.h, ws_short.h, in this order)."""
     import hashlib
     h = hashlib.sha256()
-    for name in ("ws_sample.h", "ws_lean.h"):
+    for name in ("ws_sample.h", "ws_lean.h", "ws_short.h"):
         with open(os.path.join(ROOT, "whirl-llm_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]

@@ -115,5 +115,14 @@ def smoke():
     x = d["logits"]
     am = pkg().argmax_rows(x).cpu().numpy()
     assert np.array_equal(am, np.argmax(c["logits"], axis=1)), "argmax_rows"
+    # the same rows with a top-k on every one (the short-list kernel) and with none at all (the one-sweep kernel)
+    m = pkg()
+    for top_k, route in ((40, m.FLAG_ROUTE_SHORT), (0, m.FLAG_ROUTE_LEAN)):
+        c["top_k"][:] = top_k
+        d = upload(c)
+        smp = sampler_for(c, d, 1, kept_cap=256 if top_k else 0, max_split=1).run()
+        r2 = compare_rows(c, smp, range(8), 1, check_kept=bool(top_k))
+        fl = smp.flags.cpu().numpy()
+        assert r2["exact"] + r2["differ"] == 8 and np.all((fl & (route | m.FLAG_ROUTE_HANDED_BACK)) != 0), (top_k, r2, fl)
     print("smoke ok:", res)
     return res

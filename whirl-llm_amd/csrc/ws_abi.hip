@@ -51,8 +51,8 @@ constexpr uint32_t kStaticLds = 4096u + 512u;  // + the phase marks
 #else
 constexpr uint32_t kStaticLds = 4096u;
 #endif
-// the short-list kernel's own words and those of both builds of the three-pass code it calls (7664 bytes)
-constexpr uint32_t kStaticShort = 8192u;
+// the short-list kernel's own words and those of both builds of the three-pass code it calls (8.2 KiB)
+constexpr uint32_t kStaticShort = 9216u;
 // the lean kernel's own tables and those of the three-pass code it calls
 #ifdef WS_PHASE_TIMERS
 constexpr uint32_t kStaticLean = 11776u + 768u;

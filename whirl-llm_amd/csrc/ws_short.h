@@ -43,7 +43,59 @@ struct ShortShared {
     uint32_t s_w[16];
     uint32_t red_u[WS_WAVES];
     float red_f[WS_WAVES];
+    uint32_t bcnt[64], bstart[64];  // the bucket sort's counts and starts
 };
+
+// Sorts the n (<= kShortCap) different 64-bit keys keys[0 .. n) in LDS into descending order. bucket_of(key) in [0, 64)
+// must not rise along that order (equal for keys it cannot tell apart): a key's place is the start of its bucket plus
+// the number of larger keys among the bucket's members, which it reads after all keys have been laid out bucket by
+// bucket - a few dozen reads a key where a full comparison sort takes dozens of barriers. Every thread calls it.
+template <class B>
+__device__ __forceinline__ void bucket_sort_desc(uint64_t* keys, uint32_t n, ShortShared& S, B&& bucket_of) {
+    constexpr uint32_t K = kShortCap / WS_BLOCK;
+    const uint32_t t = threadIdx.x;
+    uint64_t key[K];
+    uint32_t bk[K], pos[K];
+    if (t < 64u) S.bcnt[t] = 0u;
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k) key[k] = k * WS_BLOCK + t < n ? keys[k * WS_BLOCK + t] : 0ull;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) {
+            bk[k] = min(63u, bucket_of(key[k]));
+            pos[k] = atomicAdd(&S.bcnt[bk[k]], 1u);
+        }
+    __syncthreads();
+    if (t < 64u) {
+        const uint32_t c = S.bcnt[t];
+        S.bstart[t] = wave_incl_scan(c) - c;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) keys[S.bstart[bk[k]] + pos[k]] = key[k];
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) {
+            const uint32_t b0 = S.bstart[bk[k]], c = S.bcnt[bk[k]];
+            uint32_t above = 0;
+            for (uint32_t i = 0; i < c; i += 4u) {  // four reads on their way together
+                uint64_t o[4];
+#pragma unroll
+                for (uint32_t q = 0; q < 4u; ++q) o[q] = keys[b0 + min(i + q, c - 1u)];
+#pragma unroll
+                for (uint32_t q = 0; q < 4u; ++q) above += (i + q < c && o[q] > key[k]) ? 1u : 0u;
+            }
+            pos[k] = b0 + above;
+        }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) keys[pos[k]] = key[k];
+    __syncthreads();
+}
 
 // LDS of a row: [0, 32 KiB) the list (before the sweep: the head's bin counts), then at lds_ab the bitmap of the touched
 // tokens, its 16-bit popcount prefixes, and at lds_cnt the per-rank words {history count | bias entries << 20 | claimed}
@@ -281,9 +333,9 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     // (The count above a threshold fitted to a sample of the slice scatters like the square root of the sample's rank:
     // half of top_k on top, 150 at least. When the sample is the whole slice - a row shared by many - the count is
     // exact up to a bin's tokens, and what matters is that no part holds more of the row's top_k than it lists: twice
-    // its share and a dozen.)
+    // its share and six.)
     const uint32_t n_slice = tok1 - tok0, n_head = n_head_vec * TPV;
-    const uint32_t want = n_head >= n_slice ? 2u * ((top_k + n_parts - 1u) / n_parts) + 12u
+    const uint32_t want = n_head >= n_slice ? 2u * ((top_k + n_parts - 1u) / n_parts) + 6u
                                             : (top_k + max(top_k >> 1, 150u) + n_parts - 1u) / n_parts + 16u;
     bool list_all = n_head >= n_slice && want >= n_slice;
     if (!not_mine && ref > -INFINITY && !list_all) {
@@ -511,6 +563,12 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 __hip_atomic_load(reinterpret_cast<unsigned long long*>(&ctrl[66u + 8u * lane]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
             np = __hip_atomic_load(&ctrl[68u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        // (the keys are asked for right away, every place of every stretch: which of them count is known when the parts' words are in)
+        constexpr uint32_t kSlots = kShortCap / WS_BLOCK;
+        uint64_t got[kSlots];
+#pragma unroll
+        for (uint32_t i = 0; i < kSlots; ++i)
+            got[i] = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[i * WS_BLOCK + t]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const float mm = wave_max(mp), tt = wave_max(tp);
         const double zz = wave_sum(mp > -INFINITY ? zp * exp(static_cast<double>(__fsub_rn(mp, mm)) * static_cast<double>(inv_t)) : 0.0);
         bad = __ballot(np == 0xffffffffu) != 0ull;
@@ -529,14 +587,6 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         ref = mm;
         if (!(m > -INFINITY) || n_list > kShortCap) bad = true;
         {
-            constexpr uint32_t kSlots = kShortCap / WS_BLOCK;
-            uint64_t got[kSlots];
-#pragma unroll
-            for (uint32_t i = 0; i < kSlots; ++i) {
-                const uint32_t slot = i * WS_BLOCK + t, p = slot / region, k = slot - p * region;
-                const bool live = k < S.red_u[p];
-                got[i] = live ? __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[slot]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
-            }
 #pragma unroll
             for (uint32_t i = 0; i < kSlots; ++i) {
                 const uint32_t slot = i * WS_BLOCK + t, p = slot / region, k = slot - p * region;
@@ -554,35 +604,17 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     if (bad || n_list < top_k) return false;
 
     // ---- the candidates in order
-    if (n_list <= WS_BLOCK) {
-        // up to a key a thread: its place is the number of keys above it (all different: the id is part of the key).
-        // Every thread reads the same key at a time, eight reads on their way together; the keys in order go to the
-        // upper half of the list's LDS and back.
-        __syncthreads();
-        const uint64_t mine = t < n_list ? list[t] : 0ull;
-        uint32_t above = 0;
-        const uint32_t n8 = n_list & ~7u;
-        if (wv * 64u < n_list) {  // (per wave: one without a key issues nothing)
-            for (uint32_t i = 0; i < n8; i += 8u) {
-                uint64_t o[8];
-#pragma unroll
-                for (uint32_t k = 0; k < 8u; ++k) o[k] = list[i + k];
-#pragma unroll
-                for (uint32_t k = 0; k < 8u; ++k) above += o[k] > mine ? 1u : 0u;
-            }
-            for (uint32_t i = n8; i < n_list; ++i) above += list[i] > mine ? 1u : 0u;
-        }
-        uint64_t* sorted = list + 2048;
-        if (t < n_list) sorted[above] = mine;
-        __syncthreads();
-        if (t < n_list) list[t] = sorted[t];
-        __syncthreads();
-    } else {
-        uint32_t P2 = 2048u;
-        while (P2 < n_list) P2 <<= 1;
-        for (uint32_t k = n_list + t; k < P2; k += WS_BLOCK) list[k] = 0ull;
-        __syncthreads();
-        sort_desc(list, P2);
+    {
+        // buckets by how far below the maximum a logit lies, on the scale of the lowest listed one
+        float dloc = 0.f;
+        for (uint32_t k = t; k < n_list; k += WS_BLOCK)
+            dloc = fmaxf(dloc, fminf(__fmul_rn(__fsub_rn(m, unkey32(static_cast<uint32_t>(list[k] >> 32))), c64), 4095.f));
+        const float dmax = block_max(dloc, S.red_f);
+        const float scale = 64.f / (dmax + 1.f);
+        bucket_sort_desc(list, n_list, S, [&](uint64_t key_) {
+            const float d = fminf(__fmul_rn(__fsub_rn(m, unkey32(static_cast<uint32_t>(key_ >> 32))), c64), 4095.f);
+            return static_cast<uint32_t>(d * scale);
+        });
     }
     WSS_MARK(6);  // sorted
     // the k-th largest has to lie above every threshold (below one, a part may have left out tokens that rank before it)
@@ -712,19 +744,17 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         if (has && t == d_pos) write_out(e, cin, cex, Zk, target, dq != ~0ull, mg_top_p, mg_min_p, d_pos);
     }
     WSS_MARK(7);  // drawn
-    // ---- the kept set in ascending id order (the first kept_cap of it): each kept candidate counts the kept ids below its own
+    // ---- the kept set in ascending id order (the first kept_cap of it): the same sort on (inverted id, logit) pairs
     if (Ap->kept_ids) {
-        uint32_t* kid = reinterpret_cast<uint32_t*>(lds + 32768u - 4096u);  // (behind the sorted keys the finish uses: top_k <= 1024 of 4096 places)
         __syncthreads();
-        if (t < n3) kid[t] = id;
+        if (t < n3) list[t] = (static_cast<uint64_t>(0xffffffffu - id) << 32) | __float_as_uint(x);
         __syncthreads();
-        if (t < n3) {
-            uint32_t below = 0;
-            for (uint32_t k = 0; k < n3; ++k) below += kid[k] < id ? 1u : 0u;
-            if (below < Ap->kept_cap) {
-                Ap->kept_ids[static_cast<size_t>(row) * Ap->kept_cap + below] = static_cast<int32_t>(id);
-                if (Ap->kept_logits) Ap->kept_logits[static_cast<size_t>(row) * Ap->kept_cap + below] = x;
-            }
+        const uint32_t per_bucket = (V + 63u) / 64u;
+        bucket_sort_desc(list, n3, S, [&](uint64_t key_) { return (0xffffffffu - static_cast<uint32_t>(key_ >> 32)) / per_bucket; });
+        if (t < n3 && t < Ap->kept_cap) {
+            const uint64_t e_ = list[t];
+            Ap->kept_ids[static_cast<size_t>(row) * Ap->kept_cap + t] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(e_ >> 32));
+            if (Ap->kept_logits) Ap->kept_logits[static_cast<size_t>(row) * Ap->kept_cap + t] = __uint_as_float(static_cast<uint32_t>(e_));
         }
     }
 #ifdef WS_SHORT_TIMERS
