@@ -34,8 +34,11 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, kernel_digest() at the time)
-    ("tile", "auto"): (168795725, "sample_batch_kernel_fused_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
-    ("tile", "exact"): (539588491, "sample_batch_kernel_exact_tile_256x151936_f32.txt", "c00ebfd1c548d685"),
+    ("tile", "auto"): (208133989, "lean_batch_kernel_tile_256x151936_f32.txt", "aa667877dd7a52b8"),
+    ("cfg1", "auto"): (1210463, "short_batch_kernel_cfg1_1x151936_f32.txt", "aa667877dd7a52b8"),
+    ("cfg2", "auto"): (67019122, "sample_batch_kernel_split_cfg2_64x151936_f32.txt", "aa667877dd7a52b8"),
+    ("cfg3", "auto"): (112547811, "sample_batch_kernel_fused_cfg3_256x151936_bf16.txt", "aa667877dd7a52b8"),
+    ("cfg5", "auto"): (1397804769, "short_batch_kernel_cfg5_1024x262144_f32.txt", "aa667877dd7a52b8"),
 }
 
 
