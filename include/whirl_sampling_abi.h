@@ -301,12 +301,18 @@ typedef struct ws_batch {
                                    about a microsecond; 0 = 512 looks (going on alone costs some sixty microseconds,
                                    so a longer wait gains nothing) */
     uint32_t top_k_max;         /* 0: nothing is known about the rows' top_k. Otherwise the caller's word that every row has a
-                                   top_k of at least 1 and at most this (up to 1024): such batches - the reference's
+                                   top_k of at least 1 and at most this (up to 1024; with min_p_min: every row that has one): such batches - the reference's
                                    usual sampler settings, top-k 40 - take the short-list kernel, which keeps only the
                                    tokens that can be among a row's top_k largest instead of a histogram of all of them
                                    (fp32 and bf16, any vocabulary whose bitmap fits the LDS, kept-set dump included;
                                    not with `race`, `query_prob` or `entropy`). A row that breaks the word is still
                                    answered correctly, by the three-pass code inside the launch (WS_FLAG_ROUTE_HANDED_BACK) */
+    double min_p_min;           /* 0: nothing is known about the rows without a top_k. Otherwise the caller's word that
+                                   every row whose top_k is 0 has a min_p of at least this (a min-p floor bounds the kept
+                                   set as a top-k does: what passes lies within -ln(min_p) / inv_t of the row's maximum).
+                                   With it - alone, or together with top_k_max for the rows that do have a top_k - the
+                                   batch takes the short-list kernel. Useful from about 1e-3 upwards: a row whose floor
+                                   lets more than 1024 tokens through is handed back like one that breaks the word */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */

@@ -28,7 +28,13 @@ def _workloads():
 workloads = _w = _workloads()
 f32_to_bf16_bits, bf16_bits_to_f32, row_f32 = _w.f32_to_bf16_bits, _w.bf16_bits_to_f32, _w.row_f32
 make_cfg1, make_cfg2, make_cfg3, make_tile, make_cfg5 = _w.make_cfg1, _w.make_cfg2, _w.make_cfg3, _w.make_tile, _w.make_cfg5
-upload, sampler_for = _w.upload, _w.sampler_for
+sampler_for = _w.sampler_for
+
+
+def upload(c, device="cuda:0", hints=False, min_p_hint=False):
+    """workloads.upload; in the tests a batch says nothing about its rows unless the test asks for it (hints=True:
+    the lean and the short-list kernel's own tests, the smoke run), so that every kernel keeps the cases written for it."""
+    return _w.upload(c, device, hints=hints, min_p_hint=min_p_hint)
 
 
 def oracle_row(c, r, rng_mode, lib=None):
@@ -119,7 +125,8 @@ def smoke():
     m = pkg()
     for top_k, route in ((40, m.FLAG_ROUTE_SHORT), (0, m.FLAG_ROUTE_LEAN)):
         c["top_k"][:] = top_k
-        d = upload(c)
+        c["min_p"][:] = 0.0  # (without a top-k a min-p would make it a short-list batch as well)
+        d = upload(c, hints=True)
         smp = sampler_for(c, d, 1, kept_cap=256 if top_k else 0, max_split=1).run()
         r2 = compare_rows(c, smp, range(8), 1, check_kept=bool(top_k))
         fl = smp.flags.cpu().numpy()

@@ -23,8 +23,9 @@ def run_lean(c, rng_mode, rows=None, max_differ=0, handed_back=0, **more):
     """One launch without a kept-set dump; the rows against the oracle; the route census."""
     m = gc.pkg()
     assert not c["top_k"].any()
-    d = gc.upload(c)
+    d = gc.upload(c, hints=True)
     assert d["top_k"] is None
+    d["min_p_min"] = 0.0  # (a batch that says its rows have a min-p goes to the short-list kernel: not this test's)
     smp = gc.sampler_for(c, d, rng_mode, max_split=1, **more).run()
     rows = range(c["rows"]) if rows is None else rows
     res = gc.compare_rows(c, smp, rows, rng_mode, check_kept=False)
@@ -116,7 +117,7 @@ def test_same_answers_as_the_kernel_that_takes_a_top_k():
     counts and maxima, probabilities within 1e-6."""
     m = gc.pkg()
     c = _no_top_k(gc.make_tile(rows=160))
-    d = gc.upload(c)
+    d = gc.upload(c, hints=True)
     a = gc.sampler_for(c, d, 1, max_split=1).run()
     d["top_k"] = torch.zeros(c["rows"], dtype=torch.int32, device="cuda:0")
     b = gc.sampler_for(c, d, 1, max_split=1).run()

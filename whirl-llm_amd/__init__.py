@@ -61,7 +61,7 @@ class Batch(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("tol", C.c_double), ("mode", C.c_int32),
                 ("race", C.c_void_p),
                 ("hist_len", C.c_void_p), ("query", C.c_void_p), ("query_prob", C.c_void_p), ("entropy", C.c_void_p),
-                ("max_split", C.c_uint32), ("split_spins", C.c_uint32), ("top_k_max", C.c_uint32)]
+                ("max_split", C.c_uint32), ("split_spins", C.c_uint32), ("top_k_max", C.c_uint32), ("min_p_min", C.c_double)]
 
 
 class SpecVerify(C.Structure):
@@ -401,7 +401,7 @@ class BatchSampler:
     def __init__(self, logits, inv_t, seed, step, top_k=None, top_p=None, min_p=None, rng=RNG_PHILOX, hist=None,
                  hist_off=None, rep=None, pres=None, freq=None, bias_ids=None, bias_vals=None, bias_off=None,
                  max_hist=0, max_bias=0, allow=None, kept_cap=0, tol=0.0, want_margin=True, mode=MODE_AUTO, race=None,
-                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0, use_workspace=True, top_k_max=0):
+                 hist_len=None, query=None, want_entropy=False, max_split=0, split_spins=0, use_workspace=True, top_k_max=0, min_p_min=0.0):
         if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
             raise WsError("logits: [rows, vocab] device tensor with unit inner stride")
         if logits.dtype not in (torch.float32, torch.bfloat16):
@@ -440,6 +440,7 @@ class BatchSampler:
         b.query_prob, b.entropy = _p(self.query_prob), _p(self.entropy)
         b.max_split, b.split_spins = max_split, split_spins
         b.top_k_max = top_k_max
+        b.min_p_min = min_p_min
         need = lib().ws_sample_batch_workspace(C.byref(b))
         # zero-filled once: the parts of a split row meet here, and every launch leaves it zero-filled again
         self.workspace = torch.zeros(max(int(need), 16), dtype=torch.uint8, device=dev)

@@ -165,8 +165,10 @@ BatchPlan plan_batch(const ws_batch* b) {
     }
     // The short-list kernel: its own layout (32 KiB of list, the bitmap with 16-bit prefixes, a word and a 16-bit index
     // per history / bias entry), and under it room for the three-pass layout of the rows it hands back.
-    p.shortlist = b->top_k && b->top_k_max >= 1u && b->top_k_max <= 1024u && b->mode == WS_MODE_AUTO && vec_rows && !b->race && !b->query_prob &&
-                  !b->entropy && (!b->bias_ids || b->max_bias <= 2047u);
+    const bool word_k = b->top_k && b->top_k_max >= 1u && b->top_k_max <= 1024u;  // every row with a top-k: at most top_k_max
+    const bool word_p = b->min_p && b->min_p_min > 0.0;                            // every row without: a min-p
+    p.shortlist = (b->top_k ? (word_k || word_p) : word_p) && (!b->top_k || b->top_k_max <= 1024u) && b->mode == WS_MODE_AUTO && vec_rows && !b->race &&
+                  !b->query_prob && !b->entropy && (!b->bias_ids || b->max_bias <= 2047u);
     if (p.shortlist) {
         const uint64_t maps_s = uint64_t{nW} * 4u + ((uint64_t{nW} * 2u + 15u) & ~uint64_t{15});
         const uint64_t tabs_s = ((cap * 4u + 15u) & ~uint64_t{15}) + ((cap * 2u + 15u) & ~uint64_t{15});

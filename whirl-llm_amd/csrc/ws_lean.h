@@ -790,7 +790,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     // The searches are every wave's work; what follows from their answers is worked out by wave 0 alone and handed
     // round through LDS (sixteen waves doing the same arithmetic side by side take four times as long as one).
     LeanSel& sel = S.sel;
-    // round 1: the top-p cut against the float normaliser and against the exact one; the min-p bins by name
+    // first search: the top-p cut against the float normaliser and against the exact one; the min-p bins by name
     int lo3 = kBins, hi3 = -1;
     if (use_min_p) {
         const double astar = (s_d[8] + lift) * 64.0;
@@ -860,7 +860,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             sel.topp_in_list = topp_in_list, sel.minp_in_list = minp_in_list;
             sel.ok = r1hi < kTail;               // the tail has no mass resolution
             const double u = s_d[6];
-            s_d[4] = u * zlo * (1.0 - 1e-9);     // round 2: the bins the draw can land in
+            s_d[4] = u * zlo * (1.0 - 1e-9);     // second search: the bins the draw can land in
             s_d[5] = u * zhi * (1.0 + 1e-9);
             s_w[0] = 0u;
             s_w[5] = 0u;

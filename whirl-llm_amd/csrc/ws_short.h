@@ -1,4 +1,5 @@
-// The short-list sampler: rows that all carry a top-k of at most kShortMaxK (the caller says so: ws_batch.top_k_max).
+// The short-list sampler: rows that carry a top-k of at most kShortMaxK, or no top-k but a min-p (the caller says so:
+// ws_batch.top_k_max, ws_batch.min_p_min).
 //
 // What src/sampling/sampler.cpp:15-78 keeps of such a row is decided among its top_k largest logits alone, so the row
 // needs no histogram of every token. One sweep at the speed of the loads:
@@ -14,7 +15,12 @@
 // maximum and sum in the row's workspace; the part that arrives last - a ticket, nobody waits - takes them all and
 // finishes the row. The top_k largest of the merged list are the row's when the k-th of them lies above every part's
 // threshold (each part listed everything above its own); a row for which that fails, whose list runs over, or that has
-// no top-k after all, is handed to the three-pass code of ws_sample.h inside the same launch (WS_FLAG_ROUTE_HANDED_BACK).
+// neither a top-k nor a min-p after all, is handed to the three-pass code of ws_sample.h inside the same launch
+// (WS_FLAG_ROUTE_HANDED_BACK).
+// A row without a top-k but with a min-p: what the floor min_p * p(max) lets through lies within -ln(min_p) / inv_t of the
+// row's maximum, so the threshold needs no fitting - the head's maximum (never above the row's) minus that distance and
+// a little more; the candidates are the whole list, the top-p cut compares with the row's normaliser (the sweep's sum,
+// rounded to float as Sampler::sum is), and a cut that falls behind the list leaves the min-p floor to decide.
 #pragma once
 #include "ws_lean.h"
 
@@ -46,40 +52,46 @@ struct ShortShared {
     uint32_t bcnt[64], bstart[64];  // the bucket sort's counts and starts
 };
 
-// Sorts the n (<= kShortCap) different 64-bit keys keys[0 .. n) in LDS into descending order. bucket_of(key) in [0, 64)
-// must not rise along that order (equal for keys it cannot tell apart): a key's place is the start of its bucket plus
+// Sorts the n (<= kShortCap) different 64-bit keys keys[0 .. n) in LDS into descending order. bucket_of(key) in [0, nb)
+// (nb: 64 or 256; bcnt, bstart: nb words of LDS each) must not rise along that order (equal for keys it cannot tell apart): a key's place is the start of its bucket plus
 // the number of larger keys among the bucket's members, which it reads after all keys have been laid out bucket by
 // bucket - a few dozen reads a key where a full comparison sort takes dozens of barriers. Every thread calls it.
 template <class B>
-__device__ __forceinline__ void bucket_sort_desc(uint64_t* keys, uint32_t n, ShortShared& S, B&& bucket_of) {
+__device__ __forceinline__ void bucket_sort_desc(uint64_t* keys, uint32_t n, uint32_t* bcnt, uint32_t* bstart, uint32_t nb, B&& bucket_of) {
     constexpr uint32_t K = kShortCap / WS_BLOCK;
     const uint32_t t = threadIdx.x;
     uint64_t key[K];
     uint32_t bk[K], pos[K];
-    if (t < 64u) S.bcnt[t] = 0u;
 #pragma unroll
     for (uint32_t k = 0; k < K; ++k) key[k] = k * WS_BLOCK + t < n ? keys[k * WS_BLOCK + t] : 0ull;
+    if (t < nb) bcnt[t] = 0u;
     __syncthreads();
 #pragma unroll
     for (uint32_t k = 0; k < K; ++k)
         if (k * WS_BLOCK + t < n) {
-            bk[k] = min(63u, bucket_of(key[k]));
-            pos[k] = atomicAdd(&S.bcnt[bk[k]], 1u);
+            bk[k] = min(nb - 1u, bucket_of(key[k]));
+            pos[k] = atomicAdd(&bcnt[bk[k]], 1u);
         }
     __syncthreads();
-    if (t < 64u) {
-        const uint32_t c = S.bcnt[t];
-        S.bstart[t] = wave_incl_scan(c) - c;
+    if (t < 64u) {  // one wave: nb / 64 consecutive counts a lane
+        const uint32_t per = nb >> 6;
+        uint32_t c = 0;
+        for (uint32_t i = 0; i < per; ++i) c += bcnt[t * per + i];
+        uint32_t run = wave_incl_scan(c) - c;
+        for (uint32_t i = 0; i < per; ++i) {
+            bstart[t * per + i] = run;
+            run += bcnt[t * per + i];
+        }
     }
     __syncthreads();
 #pragma unroll
     for (uint32_t k = 0; k < K; ++k)
-        if (k * WS_BLOCK + t < n) keys[S.bstart[bk[k]] + pos[k]] = key[k];
+        if (k * WS_BLOCK + t < n) keys[bstart[bk[k]] + pos[k]] = key[k];
     __syncthreads();
 #pragma unroll
     for (uint32_t k = 0; k < K; ++k)
         if (k * WS_BLOCK + t < n) {
-            const uint32_t b0 = S.bstart[bk[k]], c = S.bcnt[bk[k]];
+            const uint32_t b0 = bstart[bk[k]], c = bcnt[bk[k]];
             uint32_t above = 0;
             for (uint32_t i = 0; i < c; i += 4u) {  // four reads on their way together
                 uint64_t o[4];
@@ -198,7 +210,9 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     const double top_p = P.top_p, min_p = P.min_p;
     const bool use_top_p = top_p < 1.0, use_min_p = min_p > 0.0;
     // rows this code does not take (uniform over all parts of a row: every part leaves, the finisher hands the row back)
-    const bool not_mine = top_k == 0u || top_k > kShortMaxK || top_k > V || !(inv_t > 0.f) || nh + nb > A.patch_cap;
+    const bool by_k = top_k >= 1u && top_k <= kShortMaxK && top_k <= V;  // the top_k largest decide
+    const bool by_p = top_k == 0u && min_p > 0.0 && min_p <= 1.0;      // no top-k: what the min-p floor lets through decides
+    const bool not_mine = !(by_k || by_p) || !(inv_t > 0.f) || nh + nb > A.patch_cap;
     const int32_t* hist_ids = A.hist + P.h0;
     const int32_t* bias_ids = A.bias_ids + P.b0;
     const float* bias_vals = A.bias_vals + P.b0;
@@ -337,8 +351,9 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     const uint32_t n_slice = tok1 - tok0, n_head = n_head_vec * TPV;
     const uint32_t want = n_head >= n_slice ? 2u * ((top_k + n_parts - 1u) / n_parts) + 6u
                                             : (top_k + max(top_k >> 1, 150u) + n_parts - 1u) / n_parts + 16u;
-    bool list_all = n_head >= n_slice && want >= n_slice;
-    if (!not_mine && ref > -INFINITY && !list_all) {
+    bool list_all = by_k && n_head >= n_slice && want >= n_slice;
+    if (by_p && ref > -INFINITY) thr = __fadd_rn(ref, __fdiv_rn(static_cast<float>(log(min_p)) - 0.02f, inv_t));  // (0.02 e-folds below the floor: roundings)
+    if (!not_mine && by_k && ref > -INFINITY && !list_all) {
         // rank in the head that about `want` tokens of the slice lie above
         const uint64_t r_star64 = (static_cast<uint64_t>(n_head) * want + n_slice - 1u) / n_slice;
         const uint32_t r_star = static_cast<uint32_t>(r_star64 < 4u ? 4u : r_star64);
@@ -601,7 +616,8 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         __syncthreads();
     }
     WSS_MARK(5);  // parts met
-    if (bad || n_list < top_k) return false;
+    const uint32_t n_cand = by_k ? top_k : n_list;  // candidates the rules look at
+    if (bad || n_list < n_cand || n_cand == 0u || n_cand > kShortCap) return false;
 
     // ---- the candidates in order
     {
@@ -610,21 +626,30 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         for (uint32_t k = t; k < n_list; k += WS_BLOCK)
             dloc = fmaxf(dloc, fminf(__fmul_rn(__fsub_rn(m, unkey32(static_cast<uint32_t>(list[k] >> 32))), c64), 4095.f));
         const float dmax = block_max(dloc, S.red_f);
-        const float scale = 64.f / (dmax + 1.f);
-        bucket_sort_desc(list, n_list, S, [&](uint64_t key_) {
+        // (256 buckets, their counters behind the keys, while the list leaves that room; else 64 in the static words)
+        const bool wide = n_list <= kShortCap - 512u;
+        const uint32_t nbk = wide ? 256u : 64u;
+        uint32_t* bc = wide ? reinterpret_cast<uint32_t*>(list + (kShortCap - 512u)) : S.bcnt;
+        uint32_t* bs = wide ? bc + 256 : S.bstart;
+        const float scale = static_cast<float>(nbk) / (dmax + 1.f);
+        bucket_sort_desc(list, n_list, bc, bs, nbk, [&](uint64_t key_) {
             const float d = fminf(__fmul_rn(__fsub_rn(m, unkey32(static_cast<uint32_t>(key_ >> 32))), c64), 4095.f);
             return static_cast<uint32_t>(d * scale);
         });
     }
     WSS_MARK(6);  // sorted
     // the k-th largest has to lie above every threshold (below one, a part may have left out tokens that rank before it)
-    const uint64_t key_k = list[top_k - 1u];
+    // (a min-p row's thresholds lie below its floor by construction: every part's is its head's maximum less the distance)
+    const uint64_t key_k = list[n_cand - 1u];
     const float x_k = unkey32(static_cast<uint32_t>(key_k >> 32));
-    if (!(x_k > thr_max) || !(x_k > -INFINITY)) return false;
+    if ((by_k && !(x_k > thr_max)) || !(x_k > -INFINITY)) return false;
+    // what the top-p cut compares with: the mass of the top_k candidates (src/sampling/sampler.cpp:45-48, a closed set),
+    // or the row's normaliser as a float (Sampler::sum) when there is no top-k
+    const double z_row = static_cast<double>(static_cast<float>(z * exp(static_cast<double>(__fsub_rn(ref, m)) * static_cast<double>(inv_t))));
 
     // ---- the rules (src/sampling/sampler.cpp:31-74) on the top_k candidates, one a thread: masses against the maximum,
     // running sums in sorted order
-    const bool has = t < top_k;
+    const bool has = t < n_cand;
     const uint64_t key = has ? list[t] : 0ull;
     const float x = has ? unkey32(static_cast<uint32_t>(key >> 32)) : -INFINITY;
     const uint32_t id = 0xffffffffu - static_cast<uint32_t>(key);
@@ -632,14 +657,14 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     ArgPtr Ap = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
     const double u = batch_uniform(A.rng, P.seed, row, P.step, 0);
     uint32_t n3;
-    auto write_out = [&](double e_, double cin_, double cex_, double Zk_, double target_, bool drawn, double mg_top_p_, double mg_min_p_, uint32_t pos) {
+    auto write_out = [&](uint32_t id_, double e_, double cin_, double cex_, double Zk_, double target_, bool drawn, double mg_top_p_, double mg_min_p_, uint32_t pos) {
         const double mg = drawn ? fmin(cin_ - target_, pos > 0u ? target_ - cex_ : 1e300) / Zk_ : 0.0;
         const double tol = Ap->tol;
         uint32_t flags = kRouteShort;
         if (mg_top_p_ < tol) flags |= kNearTopP;
         if (mg_min_p_ < tol) flags |= kNearMinP;
         if (mg < tol) flags |= kNearDraw;
-        Ap->token[row] = static_cast<int32_t>(id);
+        Ap->token[row] = static_cast<int32_t>(id_);
         Ap->flags[row] = flags;
         if (Ap->prob) Ap->prob[row] = static_cast<float>(e_ / Zk_);
         if (Ap->n_kept) Ap->n_kept[row] = n3;
@@ -653,16 +678,100 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             Ap->margin[3 * row + 2] = mg;
         }
     };
-    if (top_k <= 64u) {
+    constexpr uint32_t KC = kShortCap / WS_BLOCK;  // candidates a thread when there are more than one a thread (a wide min-p floor)
+    uint64_t wkey[KC];
+    if (n_cand > WS_BLOCK) {
+        // thread t has the candidates at places KC t .. KC t + KC - 1 of the order; the same rules
+        double e[KC], cin[KC], cex[KC], tot = 0.0;
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j) {
+            const uint32_t pos = KC * t + j;
+            wkey[j] = pos < n_cand ? list[pos] : 0ull;
+            e[j] = pos < n_cand ? exp(static_cast<double>(__fsub_rn(unkey32(static_cast<uint32_t>(wkey[j] >> 32)), m)) * static_cast<double>(inv_t)) : 0.0;
+            tot += e[j];
+        }
+        double Zk1;
+        double run = block_excl_scan(tot, S.red_d, &Zk1);
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j) {
+            cex[j] = run;
+            run += e[j];
+            cin[j] = run;
+        }
+        if (t == 0) {
+            S.s_q[0] = ~0ull;
+            S.s_q[1] = ~0ull;
+            S.s_w[6] = 0u;
+            S.s_d[0] = 1.0;
+            S.s_d[1] = 1.0;
+            S.s_d[2] = 1.0;
+        }
+        __syncthreads();
+        const double X = top_p * (by_k ? Zk1 : z_row);
+        uint32_t pass_local = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j) {
+            const uint32_t pos = KC * t + j;
+            if (use_top_p && pos < n_cand && cin[j] >= X && !(cex[j] >= X)) atomicMin(&S.s_q[0], static_cast<unsigned long long>(pos));
+            pass_local += (pos < n_cand && e[j] >= min_p) ? 1u : 0u;
+        }
+        if (use_min_p) {
+            const uint32_t wp = wave_sum(pass_local);
+            if (lane == 0u && wp) atomicAdd(&S.s_w[6], wp);
+        }
+        __syncthreads();
+        uint32_t n2 = n_cand;
+        double mg_top_p = 1.0, mg_min_p = 1.0;
+        bool cut_behind = false;
+        const unsigned long long cq = use_top_p ? S.s_q[0] : ~0ull;
+        if (use_top_p) {
+            if (cq != ~0ull) n2 = static_cast<uint32_t>(cq) + 1u;
+            else if (by_k) mg_top_p = 0.0;
+            else cut_behind = true;
+        }
+        n3 = n2;
+        const uint32_t passed = use_min_p ? S.s_w[6] : 0u;
+        if (use_min_p) {
+            n3 = min(n2, passed);
+            if (n3 < 1u) n3 = 1u;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j) {
+            const uint32_t pos = KC * t + j;
+            if (pos >= n_cand) continue;
+            if (use_top_p && cq != ~0ull && pos == n2 - 1u) S.s_d[0] = fmin(cin[j] - X, pos > 0u ? X - cex[j] : X) / X;
+            if (use_min_p && passed > 0u && pos == passed - 1u) S.s_d[1] = fabs(e[j] - min_p) / min_p;
+            if (use_min_p && pos == passed && passed < n_cand) S.s_d[2] = fabs(e[j] - min_p) / min_p;
+            if (pos == n3 - 1u) S.s_d[3] = cin[j];
+        }
+        __syncthreads();
+        if (cut_behind) mg_top_p = (X - Zk1) / X;
+        else if (use_top_p && mg_top_p != 0.0) mg_top_p = S.s_d[0];
+        if (use_min_p) mg_min_p = fmin(S.s_d[1], S.s_d[2]);
+        const double Zk = S.s_d[3];
+        const double target = u * Zk;
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j) {
+            const uint32_t pos = KC * t + j;
+            if (pos < n3 && cin[j] > target && !(cex[j] > target)) atomicMin(&S.s_q[1], static_cast<unsigned long long>(pos));
+        }
+        __syncthreads();
+        const unsigned long long dq = S.s_q[1];
+        const uint32_t d_pos = dq != ~0ull ? static_cast<uint32_t>(dq) : n3 - 1u;
+#pragma unroll
+        for (uint32_t j = 0; j < KC; ++j)
+            if (KC * t + j == d_pos)
+                write_out(0xffffffffu - static_cast<uint32_t>(wkey[j]), e[j], cin[j], cex[j], Zk, target, dq != ~0ull, mg_top_p, mg_min_p, d_pos);
+    } else if (n_cand <= 64u) {
         // the usual case, a top-k of a few dozen: one wave, a candidate a lane, no barrier and no atomic
         if (wv == 0u) {
             const double e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;
             const double cin = wave_incl_scan(e);
             const double up = __shfl_up(cin, 1);
             const double cex = lane ? up : 0.0;
-            const double Zk1 = lane_value(cin, top_k - 1u);
-            const double X = top_p * Zk1;
-            uint32_t n2 = top_k;
+            const double Zk1 = lane_value(cin, n_cand - 1u);
+            const double X = top_p * (by_k ? Zk1 : z_row);
+            uint32_t n2 = n_cand;
             double mg_top_p = 1.0, mg_min_p = 1.0;
             if (use_top_p) {
                 const uint64_t cm = __ballot(has && cin >= X && !(cex >= X));
@@ -672,7 +781,8 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                     const double ci = lane_value(cin, jc), ce = lane_value(cex, jc);
                     mg_top_p = fmin(ci - X, jc > 0u ? X - ce : X) / X;
                 } else {
-                    mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
+                    // a top-k row: rounding, the running mass never reaches top_p of itself. Else: the cut lies behind the list
+                    mg_top_p = by_k ? 0.0 : (X - Zk1) / X;
                 }
             }
             n3 = n2;
@@ -682,20 +792,20 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 if (n3 < 1u) n3 = 1u;
                 const double near = fabs(e - min_p) / min_p;
                 if (passed > 0u) mg_min_p = fmin(mg_min_p, lane_value(near, passed - 1u));
-                if (passed < top_k) mg_min_p = fmin(mg_min_p, lane_value(near, passed));
+                if (passed < n_cand) mg_min_p = fmin(mg_min_p, lane_value(near, passed));
             }
             const double Zk = lane_value(cin, n3 - 1u);
             const double target = u * Zk;
             const uint64_t dm = __ballot(has && lane < n3 && cin > target && !(cex > target));
             const uint32_t d_pos = dm ? static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(dm)) - 1) : n3 - 1u;  // (src/sampling/sampler.cpp:131: the walk falls through to the last kept)
-            if (lane == d_pos) write_out(e, cin, cex, Zk, target, dm != 0ull, mg_top_p, mg_min_p, d_pos);
+            if (lane == d_pos) write_out(id, e, cin, cex, Zk, target, dm != 0ull, mg_top_p, mg_min_p, d_pos);
             if (lane == 0u) S.s_w[7] = n3;
         }
         __syncthreads();
         n3 = S.s_w[7];
     } else {
         double e = 0.0;
-        if (wv * 64u < top_k) e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;  // (per wave: the exponential is a hundred instructions)
+        if (wv * 64u < n_cand) e = has ? exp(static_cast<double>(__fsub_rn(x, m)) * static_cast<double>(inv_t)) : 0.0;  // (per wave: the exponential is a hundred instructions)
         double Zk1;
         const double cex = block_excl_scan(e, S.red_d, &Zk1);  // mass ranked before this candidate; Zk1: of all top_k
         const double cin = cex + e;
@@ -708,19 +818,21 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             S.s_d[2] = 1.0;
         }
         __syncthreads();
-        const double X = top_p * Zk1;
+        const double X = top_p * (by_k ? Zk1 : z_row);
         if (use_top_p && has && cin >= X && !(cex >= X)) atomicMin(&S.s_q[0], static_cast<unsigned long long>(t));
         if (use_min_p) {
             const uint64_t np = __ballot(has && e >= min_p);
             if (lane == 0u && np) atomicAdd(&S.s_w[6], static_cast<uint32_t>(__popcll(np)));
         }
         __syncthreads();
-        uint32_t n2 = top_k;
+        uint32_t n2 = n_cand;
         double mg_top_p = 1.0, mg_min_p = 1.0;
+        bool cut_behind = false;
         if (use_top_p) {
             const unsigned long long cq = S.s_q[0];
             if (cq != ~0ull) n2 = static_cast<uint32_t>(cq) + 1u;
-            else mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
+            else if (by_k) mg_top_p = 0.0;  // rounding: the running mass never reaches top_p of itself
+            else cut_behind = true;         // no top-k: the cut lies behind the list
             if (has && t == n2 - 1u && cq != ~0ull) S.s_d[0] = fmin(cin - X, t > 0u ? X - cex : X) / X;
         }
         n3 = n2;
@@ -729,11 +841,12 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             n3 = min(n2, passed);
             if (n3 < 1u) n3 = 1u;
             if (has && passed > 0u && t == passed - 1u) S.s_d[1] = fabs(e - min_p) / min_p;
-            if (has && t == passed && passed < top_k) S.s_d[2] = fabs(e - min_p) / min_p;
+            if (has && t == passed && passed < n_cand) S.s_d[2] = fabs(e - min_p) / min_p;
         }
         if (has && t == n3 - 1u) S.s_d[3] = cin;  // mass of the kept set
         __syncthreads();
-        if (use_top_p && mg_top_p != 0.0) mg_top_p = S.s_d[0];
+        if (cut_behind) mg_top_p = (X - Zk1) / X;
+        else if (use_top_p && mg_top_p != 0.0) mg_top_p = S.s_d[0];
         if (use_min_p) mg_min_p = fmin(S.s_d[1], S.s_d[2]);
         const double Zk = S.s_d[3];
         const double target = u * Zk;
@@ -741,20 +854,27 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         __syncthreads();
         const unsigned long long dq = S.s_q[1];
         const uint32_t d_pos = dq != ~0ull ? static_cast<uint32_t>(dq) : n3 - 1u;  // (src/sampling/sampler.cpp:131: the walk falls through to the last kept)
-        if (has && t == d_pos) write_out(e, cin, cex, Zk, target, dq != ~0ull, mg_top_p, mg_min_p, d_pos);
+        if (has && t == d_pos) write_out(id, e, cin, cex, Zk, target, dq != ~0ull, mg_top_p, mg_min_p, d_pos);
     }
     WSS_MARK(7);  // drawn
     // ---- the kept set in ascending id order (the first kept_cap of it): the same sort on (inverted id, logit) pairs
     if (Ap->kept_ids) {
         __syncthreads();
-        if (t < n3) list[t] = (static_cast<uint64_t>(0xffffffffu - id) << 32) | __float_as_uint(x);
+        if (n_cand > WS_BLOCK) {
+#pragma unroll
+            for (uint32_t j = 0; j < KC; ++j)
+                if (KC * t + j < n3)
+                    list[KC * t + j] = (static_cast<uint64_t>(static_cast<uint32_t>(wkey[j])) << 32) | static_cast<uint32_t>(__float_as_uint(unkey32(static_cast<uint32_t>(wkey[j] >> 32))));
+        } else if (t < n3) {
+            list[t] = (static_cast<uint64_t>(0xffffffffu - id) << 32) | __float_as_uint(x);
+        }
         __syncthreads();
         const uint32_t per_bucket = (V + 63u) / 64u;
-        bucket_sort_desc(list, n3, S, [&](uint64_t key_) { return (0xffffffffu - static_cast<uint32_t>(key_ >> 32)) / per_bucket; });
-        if (t < n3 && t < Ap->kept_cap) {
-            const uint64_t e_ = list[t];
-            Ap->kept_ids[static_cast<size_t>(row) * Ap->kept_cap + t] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(e_ >> 32));
-            if (Ap->kept_logits) Ap->kept_logits[static_cast<size_t>(row) * Ap->kept_cap + t] = __uint_as_float(static_cast<uint32_t>(e_));
+        bucket_sort_desc(list, n3, S.bcnt, S.bstart, 64u, [&](uint64_t key_) { return (0xffffffffu - static_cast<uint32_t>(key_ >> 32)) / per_bucket; });
+        for (uint32_t k = t; k < n3 && k < Ap->kept_cap; k += WS_BLOCK) {
+            const uint64_t e_ = list[k];
+            Ap->kept_ids[static_cast<size_t>(row) * Ap->kept_cap + k] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(e_ >> 32));
+            if (Ap->kept_logits) Ap->kept_logits[static_cast<size_t>(row) * Ap->kept_cap + k] = __uint_as_float(static_cast<uint32_t>(e_));
         }
     }
 #ifdef WS_SHORT_TIMERS

@@ -280,6 +280,7 @@ void DeviceRows::filterOnDevice(const Sampler& s, std::uint32_t gr0, std::uint32
     b.mode = WS_MODE_AUTO;
     // every row of the launch has the sampler's top-k: a bounded one takes the short-list kernel
     b.top_k_max = (s.top_k >= 1 && s.top_k <= 1024) ? static_cast<std::uint32_t>(s.top_k) : 0u;
+    b.min_p_min = (s.top_k == 0 && s.min_p >= 1e-3) ? s.min_p : 0.0;  // (no top-k, but a floor that keeps the set small)
     if (const std::uint64_t need = ws_sample_batch_workspace(&b); need > d.work_cap) {
         if (d.work) (void)hipFree(d.work);
         d.work = nullptr;

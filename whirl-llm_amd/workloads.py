@@ -107,8 +107,12 @@ def row_f32(c, r):
     return bf16_bits_to_f32(c["logits"][r]) if c["dtype"] == "bf16" else c["logits"][r].astype(np.float32)
 
 
-def upload(c, device="cuda:0"):
-    """numpy case -> dict of device tensors in the layouts ws_batch expects."""
+def upload(c, device="cuda:0", hints=True, min_p_hint=False):
+    """numpy case -> dict of device tensors in the layouts ws_batch expects. hints: say what is known about the rows
+    (top_k left out when no row has one, top_k_max), as a caller that wants the fastest kernel would; without them
+    every batch goes the way a descriptor that says nothing goes. min_p_hint: also say min_p_min, which sends rows
+    without a top-k but with a min-p to the short-list kernel (measured on configs[1]: no faster than the split
+    single-sweep kernel there, 50 against 48 us, so the workloads do not say it by default)."""
     import torch
     d = {}
     rows = c["rows"]
@@ -118,7 +122,7 @@ def upload(c, device="cuda:0"):
         d["logits"] = torch.from_numpy(c["logits"]).to(device)
     d["inv_t"] = torch.from_numpy(c["inv_t"]).to(device)
     # (a batch without any top-k says so by leaving the array out: ws_batch.top_k = NULL)
-    d["top_k"] = torch.from_numpy(c["top_k"].view(np.int32)).to(device) if c["top_k"].any() else None
+    d["top_k"] = torch.from_numpy(c["top_k"].view(np.int32)).to(device) if (c["top_k"].any() or not hints) else None
     d["top_p"] = torch.from_numpy(np.ascontiguousarray(c["top_p"], np.float64)).to(device)
     d["min_p"] = torch.from_numpy(np.ascontiguousarray(c["min_p"], np.float64)).to(device)
     d["seed"] = torch.from_numpy(c["seed"].view(np.int64)).to(device)
@@ -140,8 +144,14 @@ def upload(c, device="cuda:0"):
         d["max_bias"] = n
     if c["allow"] is not None:
         d["allow"] = torch.from_numpy(c["allow"].view(np.int32)).to(device)
-    # every row has a top-k of at most 1024: the batch says so (ws_batch.top_k_max)
-    d["top_k_max"] = int(c["top_k"].max()) if c["top_k"].min() >= 1 and c["top_k"].max() <= 1024 else 0
+    # What the batch says about its rows (ws_batch.top_k_max, ws_batch.min_p_min): every row has a top-k of at most 1024,
+    # or no top-k but a min-p of at least 1e-3. A batch with a row that has neither says nothing.
+    with_k, without = c["top_k"] >= 1, c["top_k"] == 0
+    mp = np.asarray(c["min_p"], np.float64)
+    d["top_k_max"], d["min_p_min"] = 0, 0.0
+    if hints and np.all(c["top_k"][with_k] <= 1024) and (not without.any() or (min_p_hint and np.all(mp[without] >= 1e-3))):
+        d["top_k_max"] = int(c["top_k"].max())
+        d["min_p_min"] = float(mp[without].min()) if without.any() else 0.0
     d["race"] = torch.from_numpy(np.ascontiguousarray(c["race"], np.int32)).to(device) if c.get("race") is not None else None
     return d
 
@@ -152,6 +162,6 @@ def sampler_for(c, d, rng_mode, kept_cap=0, tol=0.0, mode=0, **more):
                           rng=rng_mode, hist=d["hist"], hist_off=d["hist_off"], rep=d["rep"], pres=d["pres"], freq=d["freq"],
                           bias_ids=d["bias_ids"], bias_vals=d["bias_vals"], bias_off=d["bias_off"], max_hist=d["max_hist"],
                           max_bias=d["max_bias"], allow=d["allow"], kept_cap=kept_cap, tol=tol, mode=mode, race=d.get("race"),
-                          **{"top_k_max": d.get("top_k_max", 0), **more})
+                          **{"top_k_max": d.get("top_k_max", 0), "min_p_min": d.get("min_p_min", 0.0), **more})
 
 
