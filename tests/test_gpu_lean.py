@@ -1,5 +1,5 @@
-"""GPU: the one-sweep kernel for batches without a top-k (fp32 rows, ws_batch.top_k = NULL, no kept-set dump) through
-the C ABI against the CPU oracle on identical seeded inputs.
+"""GPU: the one-sweep kernel for batches without a top-k (fp32 and bf16 rows, ws_batch.top_k = NULL, no kept-set dump)
+through the C ABI against the CPU oracle on identical seeded inputs.
 
 Bars as in test_gpu_sample.py: token, kept count, row maximum identical, the token's probability and the normaliser
 within 1e-6 relative; a row may differ from the oracle only where the device reports WS_FLAG_NEAR_*, and every test
@@ -92,14 +92,53 @@ def test_no_history_no_bias_no_penalties():
     assert res["exact"] == 8 and res["lean"] >= 7, res
 
 
-def test_thousands_of_equal_logits_at_the_cut_are_handed_back():
-    """Logits rounded to one decimal: every cut falls among thousands of ties, more than the buckets of the finish
-    hold. Such rows go to the three-pass code inside the launch and say so; the answers are the oracle's."""
-    m = gc.pkg()
+def test_thousands_of_equal_logits_at_the_cut():
+    """Logits rounded to one decimal: every cut falls among thousands of ties, which the lower ids win
+    (src/sampling/sampler.cpp:18-21). Up to 2048 candidates a range are sorted in place; a row with more goes to the
+    three-pass code inside the launch and says so. Either way the answers are the oracle's."""
     c = _no_top_k(gc.make_cfg2(rows=8, V=151936, n_hist=500, n_bias=20))
     c["logits"] = np.round(c["logits"], 1)
-    res, smp = run_lean(c, 1, max_differ=8, handed_back=8)
-    assert res["handed_back"] >= 1, res
+    res, smp = run_lean(c, 1, max_differ=1, handed_back=8)
+    assert res["exact"] >= 7 and res["lean"] >= 1, res
+    print(res)
+
+
+def _as_bf16(c):
+    c["logits"] = gc.f32_to_bf16_bits(c["logits"])
+    c["dtype"] = "bf16"
+    return c
+
+
+def test_bf16_zipfian_rows_with_hundreds_of_ties_at_the_cut():
+    """configs[2]'s rows: bf16, -1.1 ln(rank) + noise, top-p 0.9 - some 17000 tokens kept, and the cut among the several
+    hundred that share its bf16 value."""
+    c = gc.make_cfg3(rows=64)
+    # (two of these rows have their cut within 1e-7 of a token's edge and are reported as such, by every kernel here)
+    res, _ = run_lean(c, 1, max_differ=2, handed_back=2)
+    assert res["exact"] >= 62 and res["lean"] >= 62, res
+    print(res)
+
+
+@pytest.mark.parametrize("rng_mode", [0, 1])
+def test_bf16_min_p_top_p_bias_and_long_histories(rng_mode):
+    c = _as_bf16(_no_top_k(gc.make_cfg2(rows=24)))
+    res, _ = run_lean(c, rng_mode, max_differ=1, handed_back=1)
+    assert res["exact"] >= 23 and res["lean"] >= 23, res
+    print(res)
+
+
+def test_bf16_rows_with_an_allow_mask():
+    c = _as_bf16(_no_top_k(gc.make_cfg5(rows=12, V=151936, n_hist=2048, n_bias=200)))
+    res, _ = run_lean(c, 1, max_differ=1, handed_back=1)
+    assert res["exact"] >= 11 and res["lean"] >= 11, res
+    print(res)
+
+
+@pytest.mark.parametrize("V", [8200, 65536, 100000, 163840])
+def test_bf16_other_vocabularies(V):
+    c = _as_bf16(_no_top_k(gc.make_cfg2(rows=8, V=V, n_hist=min(V // 4, 1000), n_bias=50)))
+    res, _ = run_lean(c, 1, max_differ=1, handed_back=1)
+    assert res["exact"] >= 7 and res["lean"] >= 7, res
     print(res)
 
 

@@ -26,7 +26,7 @@ int launch_split(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsign
 // ws_fused_kept.hip, ws_split_kept.hip: the builds of the two that can write the kept-set dump
 int launch_fused_kept(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
 int launch_split_kept(hipStream_t stream, const BatchArgs& a, unsigned blocks, unsigned lds_bytes, unsigned lds_limit);
-// ws_lean.hip: the lean single-sweep kernel (1024 threads a row) for batches of unsplit fp32 rows
+// ws_lean.hip: the lean single-sweep kernel (1024 threads a row) for batches of unsplit rows without a top-k
 int launch_lean(hipStream_t stream, const BatchArgs& a, unsigned rows, unsigned lds_bytes, unsigned lds_limit);
 // each of them raises its kernels' dynamic LDS limit on the current device (once; the launchers call them too)
 int prepare_fused(unsigned lds_limit);
@@ -67,7 +67,7 @@ struct BatchPlan {
     uint32_t lds_tie;
     uint32_t lds_total;
     bool fused;
-    bool lean;            // the lean kernel can take the batch when its rows are not split (fp32, no optional outputs)
+    bool lean;            // the lean kernel can take the batch when its rows are not split (no top-k, no optional outputs)
     uint32_t lean_tie;    // its second histogram copy (0: none), its dynamic LDS, and the spare LDS of the three-pass code it calls
     uint32_t lean_total;
     uint32_t lean_fb_tie;
@@ -150,7 +150,7 @@ BatchPlan plan_batch(const ws_batch* b) {
 #endif
     // Its rows are those without a top-k, and a batch says so by leaving `top_k` out: a row with one would be handed
     // back to the three-pass code inside the launch, at twice the time of the kernel that takes a top-k in its stride.
-    p.lean = p.fused && b->mode == WS_MODE_AUTO && b->dtype == WS_DTYPE_F32 && !b->top_k && !b->kept_ids && !b->query_prob && !wants_entropy && !b->race &&
+    p.lean = p.fused && b->mode == WS_MODE_AUTO && !b->top_k && !b->kept_ids && !b->query_prob && !wants_entropy && !b->race &&
              fused_total + kStaticLean <= kMaxLds;
     if (p.lean) {
         uint64_t lt = fused_total;

@@ -1,19 +1,21 @@
 // The lean single-sweep sampler for gfx950: one workgroup of 1024 threads (sixteen wave64s, four per SIMD) per row,
-// for batches with at least one row per compute unit. It answers the rows most requests are made of - fp32 logits in
-// whole 128-bit vectors, a closed filter without a top-k (top-p and / or min-p), the inverse-CDF draw - and hands every
-// other row (and every row on which one of its own checks fails) to the three-pass code of ws_sample.h inside the same
-// launch. Results are those of ws_sample.h's single-sweep kernel: the same bins, the same histogram words, the same
-// decision rules (src/sampling/sampler.cpp:15-78, :118-131) and margins.
+// for batches with at least one row per compute unit. It answers the rows most requests are made of - fp32 or bf16
+// logits in whole 128-bit vectors, a closed filter without a top-k (top-p and / or min-p), the inverse-CDF draw - and
+// hands every other row (and every row on which one of its own checks fails) to the three-pass code of ws_sample.h
+// inside the same launch. Results are those of ws_sample.h's single-sweep kernel: the same bins, the same histogram
+// words, the same decision rules (src/sampling/sampler.cpp:15-78, :118-131) and margins.
 //
 // What is different from that kernel, and why:
-//   * every token's bin is remembered as its low 8 bits, four tokens per register (40 registers instead of 160): a scan
-//     for the tokens of a few bins tests four tokens with three instructions per bin; a token of another bin with the same
-//     low bits is found as well and dropped when its logit has been read again. The registers this frees let the first
-//     two batches of the row travel while phase 0 builds its tables, and four waves per SIMD hide the tail's latencies.
+//   * every token's bin is remembered as eight of its bits, four tokens per register (40 registers instead of 160): a
+//     scan for the tokens of a few bins tests four tokens with three instructions per bin; a token of another bin with
+//     the same bits is found as well and dropped when its logit has been read again. The registers this frees let the
+//     first two batches of the row travel while phase 0 builds its tables, and four waves per SIMD hide the tail's
+//     latencies.
 //   * the histogram is scanned four consecutive bins per thread, the cuts' and the draw's bins are found by all threads
-//     at once (every thread tests the bins it has just scanned), and the candidates' exact order is settled by all of
-//     them at once as well: a candidate adds its fixed-point mass to one of 64 buckets per range, finds its rank and its
-//     running mass among the few members of its bucket, and tests the cut and the draw on itself.
+//     at once (every thread tests the bins it has just scanned), and one wave works out what follows from the answers.
+//   * the candidates - the tokens of those bins, 2048 a range at most - are put in their exact order (logit descending,
+//     id ascending) by a bucket sort of their 64-bit keys whose buckets follow the keys that are there, thousands of
+//     equal logits included; a block-wide scan of their masses in that order settles the cuts and the draw.
 #pragma once
 #include <type_traits>
 
@@ -27,15 +29,29 @@ namespace ws {
 
 constexpr int kLeanRegs = 40;   // bin-cache registers per thread: 160 tokens, rows of up to 163840 tokens
 constexpr int kLeanBatch = 2;   // 128-bit loads per thread and batch
-constexpr uint32_t kLeanPlaces = 32u, kLeanBuckets = 128u, kLeanMaxRange = 800u;
+constexpr uint32_t kLeanBuckets = 128u, kLeanMaxRange = 2048u;  // (kLeanBuckets: words of the finish's tables in LeanShared)
+// The bins the cut and the draw can fall in: sixteen at most, with eight different cache bytes at most among them (fp32
+// rows: eight bins; bf16 rows, where four neighbours share a byte: all sixteen).
+constexpr uint32_t kLeanMaxBins = 16u;
+// The first bin of this kernel's tail, 48 units of the exponent below the anchor: the last 1024 bins, one to a thread,
+// take the tokens below that and the masked-out ones. (A scan of the bin cache for a bin finds the tokens of the tail
+// bins with the same cached bits as well: spread over 1024 bins, a 256th of the tail's tokens at most. In 64 bins a
+// row with nine tokens in ten masked out had up to a sixteenth of them found with every bin it asked for.)
+constexpr int kLeanTail = 3072;
   // WS_FLAG_ROUTE_THREE_PASS
 
 #ifdef WS_PHASE_TIMERS
+#define WSL_FAIL(code)                                                                                   \
+    do {                                                                                                 \
+        if (threadIdx.x == 0 && A.entropy) A.entropy[row * 32 + 28] = (code) + 100.0 * sel_dbg(S);       \
+        return false;                                                                                    \
+    } while (0)
 #define WSL_MARK(k)                                                \
     do {                                                           \
         if (threadIdx.x == 0) S.marks[(k)] = clock64() - wsl_t0;   \
     } while (0)
 #else
+#define WSL_FAIL(code) return false
 #define WSL_MARK(k) \
     do {            \
     } while (0)
@@ -66,29 +82,38 @@ struct LeanHits {
 };
 
 // A third token of a group and beyond goes to list[] as (token | kListNeedsLoad, 0), one LDS atomic each (rare). With
-// TO_LIST every find goes there (a second round of bytes).
-template <int NT, bool TO_LIST>
-__device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const uint32_t* __restrict__ xg, LeanHits& H,
+// TO_LIST every find goes there (a second round of bytes). DT: 0 fp32 rows (a 128-bit vector is four tokens, one
+// register of the cache), 1 bf16 rows (eight tokens, two registers); nv: the row's vectors.
+template <int NT, bool TO_LIST, int DT>
+__device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], const uint32_t (&c4)[4], const void* __restrict__ xg, LeanHits& H,
                                           uint2* list, uint32_t* n_list, uint32_t cap, uint32_t nv) {
     const uint32_t t = threadIdx.x;
+    constexpr int kRegsPerVec = DT == 0 ? 1 : 2;
+    auto logit_bits = [&](uint32_t i) {
+        return DT == 0 ? static_cast<const uint32_t*>(xg)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(xg)[i]) << 16;
+    };
 #pragma unroll
     for (int g = 0; g < kLeanGroups; ++g) {
-        // where the row ends (nv: its 128-bit vectors) is looked at per group, uniformly: a group past the row is skipped,
-        // the one group the end falls in masks its finds, the others need no test
+        // where the row ends is looked at per group, uniformly: a group past the row is skipped, the one group the end
+        // falls in masks its finds, the others need no test
         uint32_t acc = 0;
-        const uint32_t g_lo = static_cast<uint32_t>(g * 8) * WS_BLOCK;
-        if (g_lo + 8u * WS_BLOCK <= nv) {
+        const uint32_t g_lo = static_cast<uint32_t>(g * 8 / kRegsPerVec) * WS_BLOCK;
+        if (g_lo + static_cast<uint32_t>(8 / kRegsPerVec) * WS_BLOCK <= nv) {
 #pragma unroll
             for (int r = 0; r < 8; ++r)  // bit 8 e + r: token e of register r
                 acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & (0x01010101u << r)) | acc;
         } else if (g_lo < nv) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                const uint32_t keep = g_lo + static_cast<uint32_t>(r) * WS_BLOCK + t < nv ? 0x01010101u << r : 0u;
+                const uint32_t keep = g_lo + static_cast<uint32_t>(r / kRegsPerVec) * WS_BLOCK + t < nv ? 0x01010101u << r : 0u;
                 acc = ((lean_flags<NT>(cache[g * 8 + r], c4) >> (7 - r)) & keep) | acc;
             }
         }
-        auto token_of = [&](uint32_t bit) { return ((static_cast<uint32_t>(g * 8 + (bit & 7u)) * WS_BLOCK + t) << 2) + (bit >> 3); };
+        auto token_of = [&](uint32_t bit) {
+            const uint32_t reg = static_cast<uint32_t>(g * 8) + (bit & 7u);
+            if (DT == 0) return ((reg * WS_BLOCK + t) << 2) + (bit >> 3);
+            return (((reg >> 1) * WS_BLOCK + t) << 3) + ((reg & 1u) << 2) + (bit >> 3);
+        };
         if (!TO_LIST) {
             H.idx[g] = H.idx[kLeanGroups + g] = 0xffffffffu;
             H.bits[g] = H.bits[kLeanGroups + g] = 0u;
@@ -96,13 +121,13 @@ __device__ __forceinline__ void lean_scan(const uint32_t (&cache)[kLeanRegs], co
                 const uint32_t i = token_of(static_cast<uint32_t>(__ffs(acc)) - 1u);
                 acc &= acc - 1u;
                 H.idx[g] = i;
-                H.bits[g] = xg[i];
+                H.bits[g] = logit_bits(i);
             }
             if (acc) {
                 const uint32_t i = token_of(static_cast<uint32_t>(__ffs(acc)) - 1u);
                 acc &= acc - 1u;
                 H.idx[kLeanGroups + g] = i;
-                H.bits[kLeanGroups + g] = xg[i];
+                H.bits[kLeanGroups + g] = logit_bits(i);
             }
         }
         while (acc) {
@@ -139,6 +164,63 @@ __device__ __forceinline__ T pick4(uint32_t k, T a0, T a1, T a2, T a3) {
     return k & 2u ? hi : lo;
 }
 
+// Sorts the n (<= kShortCap) different 64-bit keys keys[0 .. n) in LDS into descending order. bucket_of(key) in [0, nb)
+// (nb: 64 or 256; bcnt, bstart: nb words of LDS each) must not rise along that order (equal for keys it cannot tell apart): a key's place is the start of its bucket plus
+// the number of larger keys among the bucket's members, which it reads after all keys have been laid out bucket by
+// bucket - a few dozen reads a key where a full comparison sort takes dozens of barriers. Every thread calls it.
+template <class B>
+__device__ __forceinline__ void bucket_sort_desc(uint64_t* keys, uint32_t n, uint32_t* bcnt, uint32_t* bstart, uint32_t nb, B&& bucket_of) {
+    constexpr uint32_t K = kShortCap / WS_BLOCK;
+    const uint32_t t = threadIdx.x;
+    uint64_t key[K];
+    uint32_t bk[K], pos[K];
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k) key[k] = k * WS_BLOCK + t < n ? keys[k * WS_BLOCK + t] : 0ull;
+    if (t < nb) bcnt[t] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) {
+            bk[k] = min(nb - 1u, bucket_of(key[k]));
+            pos[k] = atomicAdd(&bcnt[bk[k]], 1u);
+        }
+    __syncthreads();
+    if (t < 64u) {  // one wave: nb / 64 consecutive counts a lane
+        const uint32_t per = nb >> 6;
+        uint32_t c = 0;
+        for (uint32_t i = 0; i < per; ++i) c += bcnt[t * per + i];
+        uint32_t run = wave_incl_scan(c) - c;
+        for (uint32_t i = 0; i < per; ++i) {
+            bstart[t * per + i] = run;
+            run += bcnt[t * per + i];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) keys[bstart[bk[k]] + pos[k]] = key[k];
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) {
+            const uint32_t b0 = bstart[bk[k]], c = bcnt[bk[k]];
+            uint32_t above = 0;
+            for (uint32_t i = 0; i < c; i += 4u) {  // four reads on their way together
+                uint64_t o[4];
+#pragma unroll
+                for (uint32_t q = 0; q < 4u; ++q) o[q] = keys[b0 + min(i + q, c - 1u)];
+#pragma unroll
+                for (uint32_t q = 0; q < 4u; ++q) above += (i + q < c && o[q] > key[k]) ? 1u : 0u;
+            }
+            pos[k] = b0 + above;
+        }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < K; ++k)
+        if (k * WS_BLOCK + t < n) keys[pos[k]] = key[k];
+    __syncthreads();
+}
+
 // a row's parameters as the scalar loads at the top of lean_row leave them
 struct LeanRowParams {
     double top_p, min_p;
@@ -150,10 +232,11 @@ struct LeanRowParams {
 
 // what wave 0 works out from the searches' answers for everybody
 struct LeanSel {
-    double X, m0base, m1base, scale0, scale1, inv0, inv1;
+    double X, m0base, m1base;
     int r0lo, r0hi, r1lo, r1hi;
     uint32_t c0base, n_r0, c1base, n_r1;
-    uint32_t topp_in_list, minp_in_list, ok, pad;
+    uint32_t topp_in_list, minp_in_list, ok, n_bytes;
+    alignas(16) uint32_t bytes[8];  // the different cache bytes of the ranges' bins (n_bytes of them), each repeated four times
 };
 
 // a bin as the select's searches hand it round: mass ranked before it and up to and with it, tokens before it and in it
@@ -167,11 +250,12 @@ struct LeanShared {
     double s_exp[128];  // kExpHi, kExpLo
     double red_d[WS_WAVES];
     double s_d[10];
-    LeanSel sel;
+    alignas(16) LeanSel sel;
     LeanBinRec rec[4 * WS_WAVES + 2];  // [search][wave], then the two bins named outright
     unsigned long long s_q[6];
-    unsigned long long b_mass[kLeanBuckets], b_fpre[kLeanBuckets];
-    uint32_t b_cnt[kLeanBuckets], b_cpre[kLeanBuckets];
+    alignas(16) unsigned long long b_mass[kLeanBuckets], b_fpre[kLeanBuckets];  // (read four words at a time, all of these)
+    alignas(16) uint32_t b_cnt[kLeanBuckets], b_cpre[kLeanBuckets];
+    alignas(16) uint32_t b_mid[4 * kLeanMaxBins];
     uint32_t s_w[16];
     uint32_t red_u[WS_WAVES];
     float red_f[WS_WAVES];
@@ -180,9 +264,20 @@ struct LeanShared {
 #endif
 };
 
+#ifdef WS_PHASE_TIMERS
+__device__ __forceinline__ double sel_dbg(const LeanShared& S) { return S.sel.n_r0 + 1e5 * S.sel.n_r1 + 1e10 * (S.sel.r0hi - S.sel.r0lo + 1) + 1e12 * (S.sel.r1hi - S.sel.r1lo + 1); }
+#endif
 // One row. Returns false when the row is left to the three-pass code (nothing has been written for it then).
-template <bool MASKED>
+template <bool MASKED, int DT>  // DT: 0 fp32 rows, 1 bf16 rows
 __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row, LeanShared& S) {
+    constexpr uint32_t kTok = DT == 0 ? 4u : 8u, kTokLog = DT == 0 ? 2u : 3u;  // tokens in a 128-bit vector
+    constexpr int kRegsPerVec = DT == 0 ? 1 : 2;                                // and its registers in the bin cache
+    // What the cache remembers of a token's bin: bits kCacheShift .. kCacheShift + 7. A scan for a bin also finds the
+    // tokens of the bins that share those bits and drops them afterwards. fp32 rows: the bins 256 apart, which hold some
+    // hundreds of tokens each. bf16 rows have their tokens on few values, four bins apart and more where the tokens are
+    // many, thousands to a value in the row's tail: there a bin's three neighbours (mostly empty) are found with it, and
+    // the bins that alias are 1024 apart, beyond the span of any row.
+    constexpr uint32_t kCacheShift = DT == 0 ? 0u : 2u;
 #ifdef WS_PHASE_TIMERS
     const long long wsl_t0 = clock64();  // debug builds: the marks go to LDS, and at the end to `entropy`, 16 doubles a row
     if (threadIdx.x < 32) S.marks[threadIdx.x] = 0;
@@ -207,20 +302,20 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 
     RowView rv;
     rv.V = V;
-    rv.dtype = 0;
-    rv.base = static_cast<const unsigned char*>(A.logits) + static_cast<size_t>(row) * A.row_stride * 4u;
+    rv.dtype = DT;
+    rv.base = static_cast<const unsigned char*>(A.logits) + static_cast<size_t>(row) * A.row_stride * (DT == 0 ? 4u : 2u);
     rv.vec = true;
     rv.allow = MASKED ? A.allow + static_cast<size_t>(row) * A.allow_stride : nullptr;
     rv.touched = nullptr;
-    const uint32_t nv = V >> 2;
+    const uint32_t nv = V >> kTokLog;
     const uint4* __restrict__ xv = static_cast<const uint4*>(rv.base);
     // The row's loads run through a ring of three batches, two in flight while one is consumed (a compute unit holds about
     // that much in flight: a wave that asks for more waits at the request). The first two batches are asked for before
     // anything else - their address needs the kernel's arguments only - and travel while the row's parameters and then
     // the history ids are fetched, two dependent trips to memory; the first kEarly batches are binned before those ids
     // are looked at (what the ids touch there is put right afterwards), so that phase 0 costs its LDS work and no wait.
-    constexpr int kRing = 3, kEarly = WS_LEAN_EARLY;
-    constexpr int NB = kLeanRegs / kLeanBatch;
+    constexpr int kRing = 3, kEarly = WS_LEAN_EARLY / kRegsPerVec;  // (as many tokens either way)
+    constexpr int NB = kLeanRegs / (kLeanBatch * kRegsPerVec);
     uint4 q[kRing][kLeanBatch];
     uint32_t na[kRing][kLeanBatch];
     auto load = [&](int bt, int slot) __attribute__((always_inline)) {
@@ -229,7 +324,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             const uint32_t j = (bt * kLeanBatch + u) * WS_BLOCK + t;
             const uint32_t jc = j < nv ? j : nv - 1u;  // (unconditional, clamped to the row: a load behind a branch makes the compiler wait for every load before it)
             q[slot][u] = xv[jc];
-            na[slot][u] = MASKED ? rv.allow[(jc * 4u) >> 5] : 0xffffffffu;  // (complemented where it is used: nothing waits for the load here)
+            na[slot][u] = MASKED ? rv.allow[(jc * kTok) >> 5] : 0xffffffffu;  // (complemented where it is used: nothing waits for the load here)
         }
     };
     load(0, 0);
@@ -310,7 +405,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     if (wv == WS_WAVES - 1u && use_min_p) neg_log_min_p = -log(min_p);
     const uint32_t h0 = P.h0, nh = P.nh, b0 = P.b0, nb = P.nb;
     // rows this code does not take: a top-k, no filter at all, the race draw, parameters the three-pass code reports
-    if (top_k != 0u || !(use_top_p || use_min_p) || race || !(inv_t > 0.f) || nh + nb > A.patch_cap) return false;
+    if (top_k != 0u || !(use_top_p || use_min_p) || race || !(inv_t > 0.f) || nh + nb > A.patch_cap) WSL_FAIL(1);
 
     const int32_t* hist_ids = A.hist + h0;
     const int32_t* bias_ids = A.bias_ids + b0;
@@ -340,21 +435,34 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         float s = -INFINITY;
 #pragma unroll
         for (int u = 0; u < kLeanBatch; ++u) {
-            s = fmaxf(s, fmaxf(fmaxf(__uint_as_float(q[0][u].x), __uint_as_float(q[0][u].y)),
-                               fmaxf(__uint_as_float(q[0][u].z), __uint_as_float(q[0][u].w))));
+            const uint32_t w[4] = {q[0][u].x, q[0][u].y, q[0][u].z, q[0][u].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (DT == 0) s = fmaxf(s, __uint_as_float(w[e]));
+                else s = fmaxf(s, fmaxf(__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)));
+            }
         }
         s = block_max(s, red_f);  // its barriers also publish the zeroed histogram
         anchor = s + 8.f / inv_t;
         aq = anchor_product(anchor, c64);
-        if (!(anchor > -INFINITY && anchor < INFINITY)) return false;
+        if (!(anchor > -INFINITY && anchor < INFINITY)) WSL_FAIL(2);
     }
 
     // ------------------------------------------------------------------ the sweep
     uint32_t cache[kLeanRegs];
     float m = -INFINITY;
     float vm_early[kEarly * kLeanBatch];  // maxima of the early batches' vectors, until the bitmap says which hold a touched token
-    const float tail_f = own_tail();
+    const float tail_f = static_cast<float>(kLeanTail + static_cast<int>(t));  // this thread's own tail bin
     uint64_t* myhist = (hist2 && (t & 1u)) ? hist2 : hist;
+    // Where a bin's word lies in the histogram. bf16 rows: the words of four neighbouring bins change places by bits 4
+    // and 5 of the bin. Such a row's tokens sit on few values four bins apart and more - in the tail of a long row two
+    // thirds of all tokens on some twenty - and in their natural places those words share four of the sixteen pairs of
+    // LDS banks: the additions of a wave would queue up there four times as long.
+#ifdef WS_NO_SWZ
+    auto hist_word = [&](uint32_t b) { return b; };
+#else
+    auto hist_word = [&](uint32_t b) { return DT == 0 ? b : b ^ ((b >> 4) & 3u); };
+#endif
     const uint32_t stage_cap = 2047u;
     const uint32_t n_full = nv / WS_BLOCK;  // vector rounds that are inside the row for every thread
     bool any_touched = false;               // uniform
@@ -364,7 +472,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     auto read_words = [&](int bt) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < kLeanBatch; ++u) {
-            const uint32_t word = (((bt * kLeanBatch + u) * WS_BLOCK + t) * 4u) >> 5;  // (past the row: a word past the bitmap, inside the block's LDS)
+            const uint32_t word = (((bt * kLeanBatch + u) * WS_BLOCK + t) * kTok) >> 5;  // (past the row: a word past the bitmap, inside the block's LDS)
             tws[bt & 1][u] = any_touched ? touched[word] : 0u;
             wps[bt & 1][u] = any_touched ? wprefix[word] : 0u;
         }
@@ -388,27 +496,36 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 tw = past ? 0u : tw;                                                                                                 \
             }                                                                                                                        \
             const uint32_t w[4] = {q[slot][u].x, q[slot][u].y, q[slot][u].z, q[slot][u].w};                                          \
-            const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * 4u) & 31u)) : 0;                                           \
-            uint32_t bins[4];                                                                                                        \
+            const int32_t bw = MASKED ? static_cast<int32_t>(nal >> ((j * kTok) & 31u)) : 0;                                         \
             float vm = -INFINITY;                                                                                                    \
-            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                                          \
-                uint32_t bits = w[e];                                                                                                \
-                if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - e)) >> 31);                                                   \
-                const float x = __uint_as_float(bits);                                                                               \
-                vm = fmaxf(vm, x);                                                                                                   \
-                const float tc = bin_coord(aq, c64, x, tail_f);                                                                      \
-                bins[e] = static_cast<uint32_t>(tc);                                                                                 \
-                WSL_HIST_ADD(bins[e], tc);                                                                                           \
+            _Pragma("unroll") for (int h = 0; h < kRegsPerVec; ++h) { /* four tokens, one register of the cache */                   \
+                uint32_t bins[4];                                                                                                    \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                                      \
+                    uint32_t bits = w[e];                                                                                            \
+                    if (DT != 0) bits = (e & 1) ? w[2 * h + (e >> 1)] & 0xffff0000u : w[2 * h + (e >> 1)] << 16;                     \
+                    if (MASKED) bits |= static_cast<uint32_t>((bw << (31 - (4 * h + e))) >> 31);                                     \
+                    const float x = __uint_as_float(bits);                                                                           \
+                    vm = fmaxf(vm, x);                                                                                               \
+                    const float tc = bin_coord(aq, c64, x, tail_f);                                                                  \
+                    bins[e] = static_cast<uint32_t>(tc);                                                                             \
+                    WSL_HIST_ADD(bins[e], tc);                                                                                       \
+                }                                                                                                                    \
+                uint32_t packed;                                                                                                     \
+                if (kCacheShift == 0) {                                                                                              \
+                    const uint32_t lo2 = __builtin_amdgcn_perm(bins[1], bins[0], 0x0c0c0400u);                                       \
+                    packed = __builtin_amdgcn_perm(bins[3], bins[2], 0x04000c0cu) | lo2;                                             \
+                } else { /* bits kCacheShift .. kCacheShift + 7 of each bin: two bins to a word, shifted together */                  \
+                    const uint32_t p01 = ((bins[1] << 16) | bins[0]) >> kCacheShift, p23 = ((bins[3] << 16) | bins[2]) >> kCacheShift; \
+                    packed = __builtin_amdgcn_perm(p23, p01, 0x06040200u);                                                           \
+                }                                                                                                                    \
+                asm volatile("" : "+v"(packed)); /* (packed here, not where the tail first looks at it: four bins would stay live) */ \
+                cache[c * kRegsPerVec + h] = packed;                                                                                 \
             }                                                                                                                        \
-            const uint32_t lo2 = __builtin_amdgcn_perm(bins[1], bins[0], 0x0c0c0400u);                                               \
-            uint32_t packed = __builtin_amdgcn_perm(bins[3], bins[2], 0x04000c0cu) | lo2;                                            \
-            asm volatile("" : "+v"(packed)); /* (packed here, not where the tail first looks at it: four bins would stay live) */     \
-            cache[c] = packed;                                                                                                       \
             if (early) {                                                                                                             \
                 vm_early[c < kEarly * kLeanBatch ? c : 0] = vm;                                                                      \
             } else {                                                                                                                 \
-                const uint32_t sh = (j * 4u) & 31u;                                                                                  \
-                const bool touched_vec = ((tw >> sh) & 15u) != 0u;                                                                   \
+                const uint32_t sh = (j * kTok) & 31u;                                                                                \
+                const bool touched_vec = ((tw >> sh) & ((1u << kTok) - 1u)) != 0u;                                                   \
                 m = fmaxf(m, touched_vec ? -INFINITY : vm); /* (a vector with a touched token is looked at when that token is collected) */ \
                 if (touched_vec) {                                                                                                   \
                     const uint32_t r = wps[(bt) & 1][u] + __popc(tw & ((1u << sh) - 1u));                                            \
@@ -418,7 +535,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }                                                                                                                            \
     }
 #ifndef WS_EXP_NOATOMIC
-#define WSL_HIST_ADD(bin, tc) atomicAdd(reinterpret_cast<unsigned long long*>(&myhist[bin]), bin_word(tc))
+#define WSL_HIST_ADD(bin, tc) atomicAdd(reinterpret_cast<unsigned long long*>(&myhist[hist_word(bin)]), bin_word(tc))
 #else
 #define WSL_HIST_ADD(bin, tc) m = fmaxf(m, __uint_as_float(static_cast<uint32_t>(bin_word(tc))))
 #endif
@@ -503,12 +620,12 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 #pragma unroll
     for (int c = 0; c < kEarly * kLeanBatch; ++c) {
         const uint32_t j = static_cast<uint32_t>(c) * WS_BLOCK + t;
-        const uint32_t tw = any_touched ? touched[(j * 4u) >> 5] : 0u;
-        m = fmaxf(m, ((tw >> ((j * 4u) & 31u)) & 15u) ? -INFINITY : vm_early[c]);
+        const uint32_t tw = any_touched ? touched[(j * kTok) >> 5] : 0u;
+        m = fmaxf(m, ((tw >> ((j * kTok) & 31u)) & ((1u << kTok) - 1u)) ? -INFINITY : vm_early[c]);
     }
     read_words(kEarly);
     };
-    const uint32_t early_end = min(static_cast<uint32_t>(kEarly * kLeanBatch) * WS_BLOCK * 4u, V);  // tokens below this were binned before phase 0: not staged
+    const uint32_t early_end = min(static_cast<uint32_t>(kEarly * kLeanBatch) * WS_BLOCK * kTok, V);  // tokens below this were binned before phase 0: not staged
     load(2, 2);
     double exp_tab = 0.0;
     // (one unrolled loop for all batches, phase 0 inside it: the bin cache stays in registers only while every index into
@@ -526,7 +643,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             WSL_SWEEP_BATCH(bt, false)
         } else {  // past the row (no way out of the loop here: with one, the cache no longer stays in registers)
 #pragma unroll
-            for (int u = 0; u < kLeanBatch; ++u) cache[bt * kLeanBatch + u] = 0u;
+            for (int u = 0; u < kLeanBatch * kRegsPerVec; ++u) cache[bt * kLeanBatch * kRegsPerVec + u] = 0u;
         }
         WSL_NEXT_LOAD(bt, bt % kRing);
     }
@@ -554,8 +671,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     float ma = -INFINITY, mu = -INFINITY;
     if (n_touched) {
         constexpr uint32_t kClaim = 0x80000000u;
-        const uint32_t whole_end = V & ~3u;
-        const float tail_own = own_tail();
+        const uint32_t whole_end = V & ~(kTok - 1u);
+        const float tail_own = static_cast<float>(kLeanTail + static_cast<int>(t));
         const uint32_t stage_cap = 2047u;
         // K ids a thread and pass (a pass with nothing in its later slots would still issue their instructions)
         auto take = [&](auto kc, const int32_t* ids, uint32_t n, uint32_t j0, const uint32_t* kept_id) __attribute__((always_inline)) {
@@ -580,15 +697,15 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     const uint32_t i = id[k] < V ? id[k] : 0u;
-                    const uint32_t vb = i & ~3u;
+                    const uint32_t vb = i & ~(kTok - 1u);
                     const uint32_t rf = id[k] < V ? wp[k] + __popc(tw[k] & ((1u << (vb & 31u)) - 1u)) : 0u;
                     rk[k] = wp[k] + __popc(tw[k] & ((1u << (i & 31u)) - 1u));
                     old[k] = id[k] < V ? atomicOr(&cnt[rk[k]], kClaim) : kClaim;
                     if (i < whole_end) {
                         if (rf < stage_cap && i >= early_end) vec[k] = stage[rf];
-                        else vec[k] = xv[i >> 2];
-                    } else {
-                        const uint32_t b = static_cast<const uint32_t*>(rv.base)[i];
+                        else vec[k] = xv[i >> kTokLog];
+                    } else {  // (a token past the row's whole vectors, as the first token of a vector of its own)
+                        const uint32_t b = DT == 0 ? static_cast<const uint32_t*>(rv.base)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[i]);
                         vec[k] = make_uint4(b, b, b, b);
                     }
                 }
@@ -598,13 +715,17 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     const uint32_t i = id[k];
                     const uint32_t w[4] = {vec[k].x, vec[k].y, vec[k].z, vec[k].w};
                     const bool whole = i < whole_end;
-                    const uint32_t e_ = whole ? (i & 3u) : 0u; const uint32_t bits = e_ == 0u ? w[0] : (e_ == 1u ? w[1] : (e_ == 2u ? w[2] : w[3]));
+                    const uint32_t e_ = whole ? (i & (kTok - 1u)) : 0u;
+                    uint32_t bits = pick4(DT == 0 ? e_ : e_ >> 1, w[0], w[1], w[2], w[3]);
+                    if (DT != 0) bits = (e_ & 1u) ? bits & 0xffff0000u : bits << 16;
                     const float raw = ((al[k] >> (i & 31u)) & 1u) ? fmaxf(__uint_as_float(bits), -INFINITY) : -INFINITY;
-                    if (whole) {
-                        const uint32_t free_bits = (al[k] & ~tw[k]) >> (i & 28u);
+                    if (whole) {  // the vector's tokens that nothing touches count for the maximum here
+                        const uint32_t free_bits = (al[k] & ~tw[k]) >> (i & (32u - kTok));
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float(w[e]));
+                        for (uint32_t e = 0; e < kTok; ++e) {
+                            const uint32_t b_ = DT == 0 ? w[e & 3u] : ((e & 1u) ? w[(e >> 1) & 3u] & 0xffff0000u : w[(e >> 1) & 3u] << 16);
+                            if ((free_bits >> e) & 1u) mu = fmaxf(mu, __uint_as_float(b_));
+                        }
                     }
                     const uint32_t cw = old[k], c = cw & 0xfffffu, n_bias = (cw >> 20) & 0x7ffu;
                     float x = raw;
@@ -623,8 +744,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                     first[rk[k]] = i;  // the token id of the rank from here on
                     ma = fmaxf(ma, x);
                     const float t0 = bin_coord(aq, c64, raw, tail_own), t1 = bin_coord(aq, c64, x, tail_own);
-                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t0)]), 0ull - bin_word(t0));
-                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[static_cast<uint32_t>(t1)]), bin_word(t1));
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[hist_word(static_cast<uint32_t>(t0))]), 0ull - bin_word(t0));
+                    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[hist_word(static_cast<uint32_t>(t1))]), bin_word(t1));
                 }
             }
         };
@@ -646,7 +767,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         float m_all = fmaxf(fmaxf(m, mu), ma);
         m = block_max(m_all, red_f);  // its barriers also end the moves in the histogram
     }
-    if (!(m <= anchor && (anchor - m) * c64 <= 1024.f)) return false;  // (also a row without any token: m = -inf)
+    if (!(m <= anchor && (anchor - m) * c64 <= 1024.f)) WSL_FAIL(3);  // (also a row without any token: m = -inf)
 
     // ------------------------------------------------------------------ scan of the histogram: four consecutive bins a thread,
     // the prefixes stay in registers
@@ -668,12 +789,25 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 const ulonglong2 g01 = *reinterpret_cast<const ulonglong2*>(&hist2[bb]), g23 = *reinterpret_cast<const ulonglong2*>(&hist2[bb + 2u]);
                 h[0] += g01.x, h[1] += g01.y, h[2] += g23.x, h[3] += g23.y;
             }
+#ifndef WS_NO_SWZ
+            if (DT != 0)
+#else
+            if (false)
+#endif
+            {  // (the four words are the four bins' own, in the places hist_word gives them)
+                const uint32_t sw = (bb >> 4) & 3u;
+                const uint64_t w0_ = h[0], w1_ = h[1], w2_ = h[2], w3_ = h[3];
+                h[0] = pick4(sw, w0_, w1_, w2_, w3_);
+                h[1] = pick4(1u ^ sw, w0_, w1_, w2_, w3_);
+                h[2] = pick4(2u ^ sw, w0_, w1_, w2_, w3_);
+                h[3] = pick4(3u ^ sw, w0_, w1_, w2_, w3_);
+            }
         }
         double ms[4];
         uint32_t lc = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            c4b[k] = bb + k < static_cast<uint32_t>(kTail) ? static_cast<uint32_t>(h[k] >> kCountShift) : 0u;  // (the tail's words are not looked at one by one)
+            c4b[k] = bb + k < static_cast<uint32_t>(kLeanTail) ? static_cast<uint32_t>(h[k] >> kCountShift) : 0u;  // (the tail's words are not looked at one by one)
             ms[k] = 0.0;
             lc += c4b[k];
         }
@@ -795,8 +929,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     if (use_min_p) {
         const double astar = (s_d[8] + lift) * 64.0;
         const double lo = floor(astar - 4e-3), hi = floor(astar + 4e-3);
-        lo3 = lo < 0 ? 0 : (lo > kTail ? kTail : static_cast<int>(lo));
-        hi3 = hi < 0 ? 0 : (hi > kTail ? kTail : static_cast<int>(hi));
+        lo3 = lo < 0 ? 0 : (lo > kLeanTail ? kLeanTail : static_cast<int>(lo));
+        hi3 = hi < 0 ? 0 : (hi > kLeanTail ? kLeanTail : static_cast<int>(hi));
     }
     if (use_top_p) {
         const double Xf = top_p * Zf, Xz = top_p * Z;
@@ -804,8 +938,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         publish(1u, Xz > 0.0 ? first_own(Xz, false) : 4u);
     }
     if (use_min_p) {
-        publish_bin(4u, min(lo3, kTail - 1));
-        publish_bin(5u, min(hi3, kTail - 1));
+        publish_bin(4u, min(lo3, kLeanTail - 1));
+        publish_bin(5u, min(hi3, kLeanTail - 1));
     }
     WSL_MARK(17);
     __syncthreads();
@@ -827,7 +961,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 X = top_p * Z;
                 cut = found(1u);
             }
-            b2 = cut.b != 0xffffffffu ? static_cast<int>(cut.b) : kTail;
+            b2 = cut.b != 0xffffffffu ? static_cast<int>(cut.b) : kLeanTail;
         }
         const BinRec flo = use_min_p ? rec[4u * WS_WAVES] : cut, fhi = use_min_p ? rec[4u * WS_WAVES + 1u] : cut;
         if (use_top_p && (!use_min_p || b2 < lo3)) {
@@ -858,7 +992,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             sel.r1lo = r1lo, sel.r1hi = r1hi;
             sel.c1base = r1c0, sel.n_r1 = r1c1;  // (until the second round: tokens before range 1, and up to and with it)
             sel.topp_in_list = topp_in_list, sel.minp_in_list = minp_in_list;
-            sel.ok = r1hi < kTail;               // the tail has no mass resolution
+            sel.ok = r1hi < kLeanTail;               // the tail has no mass resolution
             const double u = s_d[6];
             s_d[4] = u * zlo * (1.0 - 1e-9);     // second search: the bins the draw can land in
             s_d[5] = u * zhi * (1.0 + 1e-9);
@@ -867,7 +1001,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }
     }
     __syncthreads();
-    if (!sel.ok) return false;
+    if (!sel.ok) WSL_FAIL(4);
     publish(2u, first_own(s_d[4], true));
     publish(3u, first_own(s_d[5], true));
     WSL_MARK(18);
@@ -881,7 +1015,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         double m0base = 0.0, m1base = 0.0;
         const BinRec dlo = found(2u), dhi = found(3u);
         const int b4lo = dlo.b != 0xffffffffu ? static_cast<int>(dlo.b) : 0;
-        int b4hi = dhi.b != 0xffffffffu ? static_cast<int>(dhi.b) : ((r1hi >= r1lo) ? r1hi : kTail - 1);
+        int b4hi = dhi.b != 0xffffffffu ? static_cast<int>(dhi.b) : ((r1hi >= r1lo) ? r1hi : kLeanTail - 1);
         if (b4hi < b4lo) b4hi = b4lo;
         // (a bound that was not found by a search has no record: such rows are rare and go the other way)
         bool ok = !(dlo.b == 0xffffffffu || dhi.b == 0xffffffffu || static_cast<int>(dhi.b) < b4lo);
@@ -907,28 +1041,32 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }
         const bool has_r1 = r1hi >= r1lo;
         const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
-        ok = ok && r0hi < kTail && nb0 + nb1 <= 8u && n_r0 + n_r1 != 0u && n_r0 <= kLeanMaxRange && n_r1 <= kLeanMaxRange;
-        // masses of a range in units of 2^-52 of a power of two above the largest mass a token of the range can have
-        const double to_max = s_d[7];
-        auto range_scale = [&](int b, double& scale, double& inv) {
-            const double emax = s_exp[b >> 6] * s_exp[64 + (b & 63)] * to_max * 1.00001;
-            const int e = static_cast<int>((static_cast<uint64_t>(__double_as_longlong(emax)) >> 52) & 0x7ffu) - 1022;  // emax < 2^e
-            scale = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 + 52 - e) << 52));
-            inv = __longlong_as_double(static_cast<long long>(static_cast<uint64_t>(1023 - 52 + e) << 52));
-        };
-        double scale0 = 1.0, inv0 = 1.0, scale1 = 1.0, inv1 = 1.0;
-        if (ok) range_scale(r0lo, scale0, inv0);
-        if (ok && has_r1) range_scale(r1lo, scale1, inv1);
+        ok = ok && r0hi < kLeanTail && nb0 + nb1 <= kLeanMaxBins && n_r0 + n_r1 != 0u && n_r0 <= kLeanMaxRange && n_r1 <= kLeanMaxRange;
+        {  // the bytes to scan the cache for: lane k looks at the k-th bin of the ranges, the first of a kind is listed
+            const uint32_t my_bin = lane < nb0 ? static_cast<uint32_t>(r0lo) + lane : static_cast<uint32_t>(r1lo) + (lane - nb0);
+            const uint32_t my_byte = (my_bin >> kCacheShift) & 0xffu;
+            bool is_first = lane < nb0 + nb1 && lane < kLeanMaxBins;
+#pragma unroll
+            for (uint32_t j = 0; j + 1u < kLeanMaxBins; ++j) {
+                const uint32_t other = lane_value(my_byte, j);
+                if (j < lane && j < nb0 + nb1 && other == my_byte) is_first = false;
+            }
+            const uint64_t firsts = __ballot(is_first);
+            const uint32_t place = static_cast<uint32_t>(__popcll(firsts & ((1ull << lane) - 1ull)));
+            if (is_first && place < 8u) sel.bytes[place] = my_byte * 0x01010101u;
+            const uint32_t n_bytes = static_cast<uint32_t>(__popcll(firsts));
+            if (lane == 0u) sel.n_bytes = n_bytes;
+            ok = ok && n_bytes <= 8u;
+        }
         if (lane == 0u) {
             sel.r0lo = r0lo, sel.r0hi = r0hi, sel.r1lo = r1lo, sel.r1hi = r1hi;
             sel.c0base = c0base, sel.n_r0 = n_r0, sel.c1base = c1base, sel.n_r1 = n_r1;
             sel.m0base = m0base, sel.m1base = m1base;
-            sel.scale0 = scale0, sel.inv0 = inv0, sel.scale1 = scale1, sel.inv1 = inv1;
             sel.ok = ok;
         }
     }
     __syncthreads();
-    if (!sel.ok) return false;
+    if (!sel.ok) WSL_FAIL(5);
     const int r0lo = sel.r0lo, r0hi = sel.r0hi, r1lo = sel.r1lo, r1hi = sel.r1hi;
     const bool has_r1 = r1hi >= r1lo;
     const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
@@ -936,10 +1074,17 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     const uint32_t n_list = n_r0 + n_r1;
     const bool topp_in_list = sel.topp_in_list != 0u, minp_in_list = sel.minp_in_list != 0u;
     const double X = sel.X, m0base = sel.m0base, m1base = sel.m1base;
-    const double scale0 = sel.scale0, inv0 = sel.inv0, scale1 = sel.scale1, inv1 = sel.inv1;
     WSL_MARK(5);
 
     // ------------------------------------------------------------------ the tokens of those bins
+    // (the sort's tables, cleared here for the barrier behind the scan: smallest and largest logit key in each of the (up
+    // to sixteen) bins of the ranges, eight copies a bin - a lane adds to copy lane % 8 - and the buckets' counts)
+    if (t < kLeanBuckets) {
+        b_cnt[t] = 0xffffffffu;
+        b_cpre[t] = 0u;
+        if (t < 4u * kLeanMaxBins) S.b_mid[t] = 0xffffffffu;
+    }
+    if (t < 256u) reinterpret_cast<uint32_t*>(b_mass)[t] = 0u;
     uint2* list = reinterpret_cast<uint2*>(lds + 32768);
     constexpr uint32_t kListCap = 4096u;
     const uint32_t u0 = static_cast<uint32_t>(r0lo), w0 = nb0 - 1u;
@@ -950,26 +1095,21 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     };
     {
         LeanHits H;
-        const uint32_t* xg = static_cast<const uint32_t*>(rv.base);
-        uint32_t bins[8];
-#pragma unroll
-        for (uint32_t k = 0; k < 8u; ++k) bins[k] = k < nb0 ? u0 + k : (k < nb0 + nb1 ? static_cast<uint32_t>(r1lo) + (k - nb0) : u0);
-        const uint32_t nt = nb0 + nb1;
+        const void* xg = rv.base;
+        const uint32_t nt = sel.n_bytes;
+        const uint4 by0 = *reinterpret_cast<const uint4*>(&sel.bytes[0]);
         {
-            uint32_t c4[4];
-#pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[k] & 0xffu) * 0x01010101u;
+            const uint32_t c4[4] = {by0.x, by0.y, by0.z, by0.w};
             const uint32_t n = min(4u, nt);
-            if (n == 1u) lean_scan<1, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
-            else if (n == 2u) lean_scan<2, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
-            else if (n == 3u) lean_scan<3, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
-            else lean_scan<4, false>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            if (n == 1u) lean_scan<1, false, DT>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else if (n == 2u) lean_scan<2, false, DT>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else if (n == 3u) lean_scan<3, false, DT>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            else lean_scan<4, false, DT>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
         }
         if (nt > 4u) {  // uniform, rare: a second round for the other bytes, every find through the list
-            uint32_t c4[4];
-#pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) c4[k] = (bins[4u + k] & 0xffu) * 0x01010101u;
-            lean_scan<4, true>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
+            const uint4 by1 = *reinterpret_cast<const uint4*>(&sel.bytes[4]);
+            const uint32_t c4[4] = {by1.x, nt > 5u ? by1.y : by1.x, nt > 6u ? by1.z : by1.x, nt > 7u ? by1.w : by1.x};
+            lean_scan<4, true, DT>(cache, c4, xg, H, list, &s_w[0], kListCap, nv);
         }
         WSL_MARK(20);
         // touched tokens whose adjusted logit lies in the ranges
@@ -1006,11 +1146,26 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         S.marks[14] = n_list;
     }
 #endif
-    if (n_hit > kListCap) return false;
+    if (n_hit > kListCap) WSL_FAIL(6);
+    // The sort's buckets: 1024 of them in the last 8 KiB of the list's region when the finds (and so the sorted keys,
+    // which go there) leave them free, cleared here for the barrier behind the filter; the 256 of the static tables else.
+    const bool wide_sort = n_hit <= kListCap - 1024u;
+    uint32_t* bcnt = wide_sort ? reinterpret_cast<uint32_t*>(lds + 32768 + (kListCap - 1024u) * 8u) : reinterpret_cast<uint32_t*>(b_mass);
+    uint32_t* bstart = wide_sort ? bcnt + 1024 : reinterpret_cast<uint32_t*>(b_fpre);
+    const uint32_t n_buckets = wide_sort ? 1024u : 256u;
+    if (wide_sort) bcnt[t] = 0u;
 
     // ------------------------------------------------------------------ the finds that are candidates: a token of another
     // bin with the same low bits, a masked-out token and a touched token found by its raw logit are dropped
-    uint2* cand = reinterpret_cast<uint2*>(lds);  // (token, logit bits), kLeanMaxRange * 2 entries at most
+    uint2* cand = reinterpret_cast<uint2*>(lds);  // (token | slot << 28, logit bits), kLeanMaxRange * 2 entries at most
+    const bool r1_first = has_r1 && r1lo < r0lo;  // range 1 holds the larger logits
+    // a candidate's slot: the number of its bin among the ranges' bins in descending order of the logits
+    auto slot_of = [&](float x) {
+        const uint32_t b = static_cast<uint32_t>(bin_coord(aq, c64, x));
+        const bool in1 = has_r1 && b - static_cast<uint32_t>(r1lo) < nb1;
+        const uint32_t s_ = in1 ? (r1_first ? 0u : nb0) + (b - static_cast<uint32_t>(r1lo)) : (r1_first ? nb1 : 0u) + (b - static_cast<uint32_t>(r0lo));
+        return min(s_, kLeanMaxBins - 1u);
+    };
     {
         constexpr int kR = 4;
         uint2 en[kR];
@@ -1027,7 +1182,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             float x = __uint_as_float(en[r].y);
             bool ok = live;
             if (!(en[r].x & kListAdjusted)) {
-                if (en[r].x & kListNeedsLoad) x = __uint_as_float(static_cast<const uint32_t*>(rv.base)[id]);
+                if (en[r].x & kListNeedsLoad)
+                    x = __uint_as_float(DT == 0 ? static_cast<const uint32_t*>(rv.base)[id] : static_cast<uint32_t>(static_cast<const uint16_t*>(rv.base)[id]) << 16);
                 x = fmaxf(x, -INFINITY);
                 ok = ok && (!MASKED || is_allowed(rv, id)) && !is_touched(rv, id) && in_ranges(x);
             }
@@ -1035,12 +1191,14 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             uint32_t base = 0;
             if (lane == 0u && mk) base = atomicAdd(&s_w[5], static_cast<uint32_t>(__popcll(mk)));
             const uint32_t slot = __shfl(base, 0) + static_cast<uint32_t>(__popcll(mk & ((1ull << lane) - 1ull)));
-            if (ok && slot < 2u * kLeanMaxRange) cand[slot] = make_uint2(id, __float_as_uint(x));
+            if (ok && slot < 2u * kLeanMaxRange) {
+                const uint32_t s_ = slot_of(x), k32 = static_cast<uint32_t>(key64(x, 0u) >> 32);
+                cand[slot] = make_uint2(id | (s_ << 28), __float_as_uint(x));
+                atomicMin(&b_cnt[s_ * 8u + (lane & 7u)], k32);
+                atomicMax(&b_cpre[s_ * 8u + (lane & 7u)], k32);
+                S.b_mid[s_ * 4u + (lane & 3u)] = k32;  // (four of the bin's candidates, any: whichever stores land last)
+            }
         }
-    }
-    if (t < kLeanBuckets) {
-        b_cnt[t] = 0u;
-        b_mass[t] = 0ull;
     }
     if (t == 0) {
         s_q[0] = ~0ull;  // smallest mass at or above the min-p floor
@@ -1048,170 +1206,247 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         s_q[2] = ~0ull;  // the cut: (rank in the row << 32) | slot
         s_q[3] = ~0ull;  // the draw
         s_w[1] = 0u;     // candidates at or above the floor
-        s_w[2] = 0u;     // a bucket ran out of places
         s_w[3] = 0u;     // the last kept candidate was found
     }
     __syncthreads();
     WSL_MARK(7);
-    if (s_w[5] != n_list) return false;  // the histogram and the gather disagree
-    constexpr int kRounds = 2;  // n_list <= 2 kLeanMaxRange <= 2 WS_BLOCK
-    uint32_t cid[kRounds];
-    float cx[kRounds];
-    bool con[kRounds];
+    if (s_w[5] != n_list) WSL_FAIL(7);  // the histogram and the gather disagree
+    // ---- the candidates in order (logit descending, id ascending): their 64-bit keys sorted by buckets. A bucket is
+    // a bin of the ranges (eight at most) and, inside the bin, a 32nd of the span of the bin's logits - or, when all
+    // its candidates tie, as bf16 rows have them by the hundred, a 32nd of the vocabulary's ids: either way some dozens
+    // of keys to compare with, and no limit on ties. A key's place is the start of its bucket plus the number of larger
+    // keys among the bucket's members, which it reads once all keys lie bucket by bucket.
+    constexpr int kRounds = 2 * kLeanMaxRange / WS_BLOCK;  // the candidates at places kRounds t .. kRounds t + kRounds - 1 of the order
+    uint64_t* keys = reinterpret_cast<uint64_t*>(lds);            // bucket by bucket (over the candidates' pairs, which are in registers by then)
+    uint64_t* sorted = reinterpret_cast<uint64_t*>(lds + 32768);  // in order (over the finds' list)
+    {
+        uint32_t* kmin = b_cnt;
+        uint32_t* kmax = b_cpre;
+        uint64_t own[kRounds];
+        uint32_t sl[kRounds], bk[kRounds], pos[kRounds];
 #pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        const uint32_t k = r * WS_BLOCK + t;
-        const uint2 en = k < n_list ? cand[k] : make_uint2(0u, 0u);
-        cid[r] = en.x;
-        cx[r] = __uint_as_float(en.y);
-        con[r] = k < n_list;
-    }
-    __syncthreads();  // every thread has its candidates: the LDS takes the buckets
-    struct Place {
-        uint64_t key, fx;
-    };
-    Place* lb = reinterpret_cast<Place*>(lds);  // [bucket][place]: a candidate's key and its fixed-point mass
-    const float step0 = 64.f / static_cast<float>(nb0), step1 = has_r1 ? 64.f / static_cast<float>(nb1) : 0.f;
-    const float lo0 = static_cast<float>(r0lo), lo1 = static_cast<float>(r1lo);
-    uint32_t cbkt[kRounds];
-    uint64_t cfix[kRounds], ckey[kRounds];
-    double cem[kRounds];
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t k = r * WS_BLOCK + t;
+            const uint2 en = k < n_list ? cand[k] : make_uint2(0u, 0u);
+            own[r] = key64(__uint_as_float(en.y), en.x & 0x0fffffffu);
+            sl[r] = en.x >> 28;
+        }
+        // A bin's share of the buckets is cut in three: the logits above one of the bin's own candidates' (`mid`), by
+        // logit; the candidates with exactly that logit, by id; the logits below, by logit. Where hundreds tie, `mid`
+        // is theirs (two of four sampled candidates agree on it), and they spread over half the bin's buckets; where
+        // no two logits are the same the middle part holds one candidate and the other half of the buckets serves.
+        const uint32_t nt_ = nb0 + nb1;
+        const uint32_t nsub = n_buckets >> (nt_ <= 1u ? 0u : (nt_ <= 2u ? 1u : (nt_ <= 4u ? 2u : (nt_ <= 8u ? 3u : 4u))));  // buckets a bin
+        const uint32_t nl = nsub / 2u - 1u, nid = nsub / 2u;
+        const float ids_scale = static_cast<float>(nid) / static_cast<float>(V);
 #pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u >= n_list) continue;  // per wave
-        const float x = cx[r];
-        const float tc = bin_coord(aq, c64, x);
-        const bool in1 = has_r1 && static_cast<uint32_t>(tc) - static_cast<uint32_t>(r1lo) < nb1;
-        const float rel = fmaxf(__fmul_rn(__fsub_rn(tc, in1 ? lo1 : lo0), in1 ? step1 : step0), 0.f);
-        cbkt[r] = (in1 ? 64u : 0u) + min(63u, static_cast<uint32_t>(rel));
-        cem[r] = exp_neg(static_cast<double>(__fsub_rn(m, x)) * static_cast<double>(inv_t), s_exp);
-        cfix[r] = static_cast<uint64_t>(__double2ull_rn(cem[r] * (in1 ? scale1 : scale0)));
-        ckey[r] = key64(x, cid[r]);
-        if (con[r]) {
-            const uint32_t place = atomicAdd(&b_cnt[cbkt[r]], 1u);
-            atomicAdd(&b_mass[cbkt[r]], static_cast<unsigned long long>(cfix[r]));
-            if (place < kLeanPlaces) lb[cbkt[r] * kLeanPlaces + place] = Place{ckey[r], cfix[r]};
-            else s_w[2] = 1u;
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t k = r * WS_BLOCK + t;
+            if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u < n_list && k < n_list) {
+                const uint4 a0 = *reinterpret_cast<const uint4*>(&kmin[sl[r] * 8u]), a1 = *reinterpret_cast<const uint4*>(&kmin[sl[r] * 8u + 4u]);
+                const uint4 b0 = *reinterpret_cast<const uint4*>(&kmax[sl[r] * 8u]), b1 = *reinterpret_cast<const uint4*>(&kmax[sl[r] * 8u + 4u]);
+                // (`mid`: the logit two of the four sampled candidates share, or else the smallest of the four)
+                const uint4 sm = *reinterpret_cast<const uint4*>(&S.b_mid[sl[r] * 4u]);
+                uint32_t mid = min(min(sm.x, sm.y), min(sm.z, sm.w));
+                if (sm.z != 0xffffffffu && sm.z == sm.w) mid = sm.z;
+                if (sm.y != 0xffffffffu && (sm.y == sm.z || sm.y == sm.w)) mid = sm.y;
+                if (sm.x != 0xffffffffu && (sm.x == sm.y || sm.x == sm.z || sm.x == sm.w)) mid = sm.x;
+                const uint32_t lo = min(min(min(a0.x, a0.y), min(a0.z, a0.w)), min(min(a1.x, a1.y), min(a1.z, a1.w)));
+                const uint32_t hi = max(max(max(b0.x, b0.y), max(b0.z, b0.w)), max(max(b1.x, b1.y), max(b1.z, b1.w)));
+                const uint32_t k32 = static_cast<uint32_t>(own[r] >> 32);
+                // (none of the expressions rises along the order, whatever the rounding: conversion, product and truncation keep it)
+                const float per = static_cast<float>(nl) * __builtin_amdgcn_rcpf(static_cast<float>(hi - lo) + 1.f);
+                const uint32_t lk = min(nl - 1u, static_cast<uint32_t>(static_cast<float>(hi - k32) * per));
+                const uint32_t lm = min(nl - 1u, static_cast<uint32_t>(static_cast<float>(hi - mid) * per));
+                const uint32_t by_id = min(nid - 1u, static_cast<uint32_t>(static_cast<float>(0xffffffffu - static_cast<uint32_t>(own[r])) * ids_scale));
+                const uint32_t sub = k32 > mid ? lk : (k32 == mid ? lm + 1u + by_id : lk + 1u + nid);
+                bk[r] = sl[r] * nsub + sub;
+                pos[r] = atomicAdd(&bcnt[bk[r]], 1u);
+            }
         }
-        if (use_min_p && minp_in_list) {  // uniform
-            const bool pass = con[r] && cem[r] >= min_p;
-            const uint64_t np = __ballot(pass);
-            if (lane == 0u && np) atomicAdd(&s_w[1], static_cast<uint32_t>(__popcll(np)));
-            if (pass) atomicMin(&s_q[0], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
-            if (con[r] && !pass) atomicMax(&s_q[1], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
+        __syncthreads();
+        if (wv == 0u) {  // one wave: four or sixteen consecutive counts a lane
+            if (wide_sort) {
+                uint4 c[4];
+                uint32_t sum = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    c[i] = *reinterpret_cast<const uint4*>(&bcnt[lane * 16u + 4u * i]);
+                    sum += c[i].x + c[i].y + c[i].z + c[i].w;
+                }
+                uint32_t run = wave_incl_scan(sum) - sum;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *reinterpret_cast<uint4*>(&bstart[lane * 16u + 4u * i]) = make_uint4(run, run + c[i].x, run + c[i].x + c[i].y, run + c[i].x + c[i].y + c[i].z);
+                    run += c[i].x + c[i].y + c[i].z + c[i].w;
+                }
+            } else {
+                const uint4 c = *reinterpret_cast<const uint4*>(&bcnt[lane * 4u]);
+                const uint32_t sum = c.x + c.y + c.z + c.w;
+                const uint32_t run = wave_incl_scan(sum) - sum;
+                *reinterpret_cast<uint4*>(&bstart[lane * 4u]) = make_uint4(run, run + c.x, run + c.x + c.y, run + c.x + c.y + c.z);
+            }
         }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r)
+            if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u < n_list && r * WS_BLOCK + t < n_list) {
+                bk[r] = bstart[bk[r]] | (bcnt[bk[r]] << 16);  // (start and count of the bucket: below 65536 both)
+                keys[(bk[r] & 0xffffu) + pos[r]] = own[r];
+            }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r)
+            if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u < n_list && r * WS_BLOCK + t < n_list) {
+                const uint32_t b0 = bk[r] & 0xffffu, c = bk[r] >> 16;
+                uint32_t above = 0;
+                for (uint32_t i = 0; i < c; i += 4u) {  // four reads on their way together
+                    uint64_t o[4];
+#pragma unroll
+                    for (uint32_t q_ = 0; q_ < 4u; ++q_) o[q_] = keys[b0 + min(i + q_, c - 1u)];
+#pragma unroll
+                    for (uint32_t q_ = 0; q_ < 4u; ++q_) above += (i + q_ < c && o[q_] > own[r]) ? 1u : 0u;
+                }
+                sorted[b0 + above] = own[r];
+            }
+        __syncthreads();
     }
-    __syncthreads();
     WSL_MARK(8);
-    if (t < 64u) {  // wave 0: entries and masses ranked before each bucket (two buckets a lane)
-        const uint32_t bc0 = b_cnt[2u * lane], bc1 = b_cnt[2u * lane + 1u];
-        const uint64_t bf0 = b_mass[2u * lane], bf1 = b_mass[2u * lane + 1u];
-        const uint32_t cbefore = wave_incl_scan(bc0 + bc1) - (bc0 + bc1);
-        const uint64_t fbefore = wave_incl_scan(bf0 + bf1) - (bf0 + bf1);
-        b_cpre[2u * lane] = cbefore;
-        b_cpre[2u * lane + 1u] = cbefore + bc0;
-        b_fpre[2u * lane] = fbefore;
-        b_fpre[2u * lane + 1u] = fbefore + bf0;
+    // every candidate: its rank in the row and the mass up to and with it
+    const uint32_t nA = r1_first ? n_r1 : n_r0;  // candidates of the range with the larger logits: they come first
+    const double mA = r1_first ? m1base : m0base, mB = r1_first ? m0base : m1base;
+    const uint32_t cA = r1_first ? c1base : c0base, cB = r1_first ? c0base : c1base;
+    // Thread t takes the places kr t .. kr t + kr - 1 of the order, kr as small as the number of candidates allows
+    // (one thread's candidates are worked through one after the other). Only the waves that hold places work from
+    // here on (wave 0 always does); the others pass the barriers and issue nothing else.
+    const uint32_t kr = (n_list + WS_BLOCK - 1u) / WS_BLOCK;  // 1 .. kRounds
+    const bool act = wv * 64u * kr < n_list;
+    uint32_t cid[kRounds], cpos[kRounds];
+    uint64_t ckey[kRounds];
+    double cem[kRounds], cin[kRounds], cex[kRounds], pre[kRounds];
+    double mine_ = 0.0, inc = 0.0, total = 0.0;
+    if (act) {
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t pos = kr * t + static_cast<uint32_t>(r);
+            const bool on = static_cast<uint32_t>(r) < kr && pos < n_list;
+            ckey[r] = on ? sorted[pos] : 0ull;
+            cid[r] = 0xffffffffu - static_cast<uint32_t>(ckey[r]);
+            cem[r] = 0.0;
+            if (static_cast<uint32_t>(r) < kr && on) cem[r] = exp_neg(static_cast<double>(__fsub_rn(m, unkey32(static_cast<uint32_t>(ckey[r] >> 32)))) * static_cast<double>(inv_t), s_exp);
+            mine_ += cem[r];
+        }
+        inc = wave_incl_scan(mine_);
+    }
+    if (lane == 63u) red_d[wv] = inc;
+    __syncthreads();
+    if (act) {
+        const double wm = lane < WS_WAVES ? red_d[lane] : 0.0;
+        const double wmi = wave_incl_scan(wm);
+        total = lane_value(wmi, WS_WAVES - 1u);
+        pre[0] = (wv ? lane_value(wmi, wv - 1u) : 0.0) + (inc - mine_);
+#pragma unroll
+        for (int r = 1; r < kRounds; ++r) pre[r] = pre[r - 1] + cem[r - 1];
+#pragma unroll
+        for (int r = 0; r < kRounds; ++r)
+            if (static_cast<uint32_t>(r) < kr && kr * t + static_cast<uint32_t>(r) == nA) s_d[2] = pre[r];  // mass of the first range's candidates
     }
     __syncthreads();
-    const uint32_t got0 = b_cpre[64];
-    const uint64_t fbase1 = b_fpre[64];
-    if (s_w[2] || got0 != n_r0) return false;  // heavy ties
-    // every candidate: its rank in the row and the mass up to and with it
-    uint32_t cpos[kRounds];
-    double cin[kRounds], cex[kRounds];
-#pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        cpos[r] = 0xffffffffu;
-        cin[r] = cex[r] = 0.0;
-        if (static_cast<uint32_t>(r) * WS_BLOCK + wv * 64u >= n_list) continue;  // per wave
-        const uint32_t bkt = con[r] ? cbkt[r] : 0u;
-        const uint32_t n = con[r] ? b_cnt[bkt] : 0u;
-        uint32_t rank = 0;
-        uint64_t cum = 0;
-        for (uint32_t j = 0; j < n; ++j) {
-            const Place o = lb[bkt * kLeanPlaces + j];
-            rank += o.key > ckey[r] ? 1u : 0u;
-            cum += o.key >= ckey[r] ? o.fx : 0ull;
-        }
-        if (con[r]) {
-            const bool r1 = bkt >= 64u;
-            const uint64_t fb = b_fpre[bkt] - (r1 ? fbase1 : 0ull);
-            const double mb = r1 ? m1base : m0base, inv = r1 ? inv1 : inv0;
-            cin[r] = mb + static_cast<double>(fb + cum) * inv;
-            cex[r] = mb + static_cast<double>(fb + cum - cfix[r]) * inv;
-            cpos[r] = (r1 ? c1base : c0base) + (b_cpre[bkt] - (r1 ? got0 : 0u)) + rank;
-        }
-    }
     WSL_MARK(9);
     // ---- the cuts (src/sampling/sampler.cpp:35-74): the first candidate at which the running mass reaches X
     const uint32_t n1 = V;
-    if (use_top_p && topp_in_list) {
+    if (act) {
+        const double massA = nA < n_list ? s_d[2] : total;
 #pragma unroll
-        for (int r = 0; r < kRounds; ++r)
-            if (cpos[r] != 0xffffffffu && cin[r] >= X && !(cex[r] >= X) && cin[r] > cex[r])
+        for (int r = 0; r < kRounds; ++r) {
+            const uint32_t pos = kr * t + static_cast<uint32_t>(r);
+            cpos[r] = 0xffffffffu;
+            cin[r] = cex[r] = 0.0;
+            if (static_cast<uint32_t>(r) >= kr) continue;  // uniform
+            if (pos < n_list) {
+                const bool inA = pos < nA;
+                cex[r] = (inA ? mA : mB) + (pre[r] - (inA ? 0.0 : massA));
+                cin[r] = cex[r] + cem[r];
+                cpos[r] = (inA ? cA + pos : cB + (pos - nA));
+            }
+            if (use_min_p && minp_in_list) {  // uniform
+                const bool pass = pos < n_list && cem[r] >= min_p;
+                const uint64_t np = __ballot(pass);
+                if (lane == 0u && np) atomicAdd(&s_w[1], static_cast<uint32_t>(__popcll(np)));
+                if (pass) atomicMin(&s_q[0], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
+                if (pos < n_list && !pass) atomicMax(&s_q[1], static_cast<unsigned long long>(__double_as_longlong(cem[r])));
+            }
+            if (use_top_p && topp_in_list && cpos[r] != 0xffffffffu && cin[r] >= X && !(cex[r] >= X) && cin[r] > cex[r])
                 atomicMin(&s_q[2], (static_cast<unsigned long long>(cpos[r]) << 32) | (static_cast<uint32_t>(r) * WS_BLOCK + t));
+        }
     }
     __syncthreads();
     double mg_top_p = 1.0, mg_min_p = 1.0;
-    uint32_t n2 = n1;
+    uint32_t n2 = n1, n3 = n1;
     bool cut_found = false;
-    if (use_top_p && topp_in_list) {
-        const unsigned long long cq = s_q[2];
-        if (cq != ~0ull && static_cast<uint32_t>(cq >> 32) < n1) {
-            cut_found = true;
-            n2 = static_cast<uint32_t>(cq >> 32) + 1u;
-        } else {  // rounding: the cut falls just past the gathered bins
-            n2 = min(n1, has_r1 ? c1base + n_r1 : c0base + n_r0);
-            mg_top_p = 0.0;
+    if (act) {
+        if (use_top_p && topp_in_list) {
+            const unsigned long long cq = s_q[2];
+            if (cq != ~0ull && static_cast<uint32_t>(cq >> 32) < n1) {
+                cut_found = true;
+                n2 = static_cast<uint32_t>(cq >> 32) + 1u;
+            } else {  // rounding: the cut falls just past the gathered bins
+                n2 = min(n1, has_r1 ? c1base + n_r1 : c0base + n_r0);
+                mg_top_p = 0.0;
+            }
         }
-    }
-    uint32_t n3 = n2;
-    if (use_min_p && minp_in_list) {
-        const uint32_t passed = s_w[1];
-        double near = 1.0;
-        if (passed > 0u) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[0])) - min_p) / min_p);
-        if (passed < n_list) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[1])) - min_p) / min_p);
-        uint32_t n3p;
-        if (has_r1) n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
-        else n3p = c0base + passed;
-        n3 = min(n2, n3p);
-        if (n3 < 1u) n3 = 1u;
-        mg_min_p = near;
-    }
-    // the cut's margin, and the last kept candidate: mass of the kept set, its key, its own mass
+        n3 = n2;
+        if (use_min_p && minp_in_list) {
+            const uint32_t passed = s_w[1];
+            double near = 1.0;
+            if (passed > 0u) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[0])) - min_p) / min_p);
+            if (passed < n_list) near = fmin(near, fabs(__longlong_as_double(static_cast<long long>(s_q[1])) - min_p) / min_p);
+            uint32_t n3p;
+            if (has_r1) n3p = passed >= n_r0 ? c1base + (passed - n_r0) : c0base + passed;
+            else n3p = c0base + passed;
+            n3 = min(n2, n3p);
+            if (n3 < 1u) n3 = 1u;
+            mg_min_p = near;
+        }
+        // the cut's margin, and the last kept candidate: mass of the kept set, its key, its own mass
 #pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        if (cpos[r] == 0xffffffffu) continue;
-        if (cut_found && cpos[r] == n2 - 1u) s_d[3] = fmin(cin[r] - X, cpos[r] > 0u ? X - cex[r] : X) / X;
-        if (cpos[r] == n3 - 1u) {
-            s_d[0] = cin[r];
-            s_d[1] = cem[r];
-            s_q[4] = ckey[r];
-            s_w[3] = 1u;
+        for (int r = 0; r < kRounds; ++r) {
+            if (static_cast<uint32_t>(r) >= kr || cpos[r] == 0xffffffffu) continue;
+            if (cut_found && cpos[r] == n2 - 1u) s_d[3] = fmin(cin[r] - X, cpos[r] > 0u ? X - cex[r] : X) / X;
+            if (cpos[r] == n3 - 1u) {
+                s_d[0] = cin[r];
+                s_d[1] = cem[r];
+                s_q[4] = ckey[r];
+                s_w[3] = 1u;
+            }
         }
     }
     __syncthreads();
-    if (cut_found) mg_top_p = s_d[3];
-    double Zk;
     const bool have_last = s_w[3] != 0u;
-    if (have_last) Zk = s_d[0];
-    else if (has_r1 && n3 == c1base) Zk = m1base;  // the cut falls on the upper edge of range 1: everything in earlier bins
-    else if (n3 == c0base && n_r0) Zk = m0base;
-    else Zk = Z;
-    // ---- the draw (src/sampling/sampler.cpp:118-131): the first candidate at which the running mass passes u * Zk
-    const double target = s_d[6] * Zk;
+    double Zk = Z, target = 0.0;
+    if (act) {
+        if (cut_found) mg_top_p = s_d[3];
+        if (have_last) Zk = s_d[0];
+        else if (has_r1 && n3 == c1base) Zk = m1base;  // the cut falls on the upper edge of range 1: everything in earlier bins
+        else if (n3 == c0base && n_r0) Zk = m0base;
+        else Zk = Z;
+        // ---- the draw (src/sampling/sampler.cpp:118-131): the first candidate at which the running mass passes u * Zk
+        target = s_d[6] * Zk;
 #pragma unroll
-    for (int r = 0; r < kRounds; ++r)
-        if (cpos[r] != 0xffffffffu && cpos[r] < n3 && cin[r] > target && !(cex[r] > target) && cin[r] > cex[r])
-            atomicMin(&s_q[3], (static_cast<unsigned long long>(cpos[r]) << 32) | (static_cast<uint32_t>(r) * WS_BLOCK + t));
+        for (int r = 0; r < kRounds; ++r)
+            if (static_cast<uint32_t>(r) < kr && cpos[r] != 0xffffffffu && cpos[r] < n3 && cin[r] > target && !(cex[r] > target) && cin[r] > cex[r])
+                atomicMin(&s_q[3], (static_cast<unsigned long long>(cpos[r]) << 32) | (static_cast<uint32_t>(r) * WS_BLOCK + t));
+    }
     __syncthreads();
     const unsigned long long dq = s_q[3];
-    if (dq == ~0ull && !have_last) return false;  // no candidate for the draw and none to fall back on
+    if (dq == ~0ull && !have_last) WSL_FAIL(8);  // no candidate for the draw and none to fall back on
+#ifndef WS_PHASE_TIMERS  // (that build has a barrier at the end)
+    if (!act) return true;
+#endif
     const uint32_t d_slot = static_cast<uint32_t>(dq), d_pos = static_cast<uint32_t>(dq >> 32);
 #pragma unroll
     for (int r = 0; r < kRounds; ++r) {
-        if (dq != ~0ull && static_cast<uint32_t>(r) * WS_BLOCK + t == d_slot) {
+        if (static_cast<uint32_t>(r) < kr && dq != ~0ull && static_cast<uint32_t>(r) * WS_BLOCK + t == d_slot) {
             const double mg = fmin(cin[r] - target, d_pos > 0u ? target - cex[r] : 1e300) / Zk;
             uint32_t flags = 0;
             const double tol = Ap->tol;
@@ -1240,8 +1475,8 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             Ap->stats[2 * row] = m;
             Ap->stats[2 * row + 1] = static_cast<float>(Z);
         }
-        if (A.margin) {
-            A.margin[3 * row] = mg_top_p;
+        if (Ap->margin) {
+            Ap->margin[3 * row] = mg_top_p;
             Ap->margin[3 * row + 1] = mg_min_p;
         }
     }
@@ -1273,11 +1508,11 @@ __device__ __noinline__ void three_pass_row(LeanArgPtr Ap, const uint32_t row) {
 }
 
 // MASKED: the batch has an allow mask (a kernel of its own: one build carrying both paths spilled far more registers)
-template <bool MASKED>
+template <bool MASKED, int DT>
 __global__ void __launch_bounds__(WS_BLOCK) lean_batch_kernel(BatchArgs A) {
     __shared__ LeanShared shared;
     const uint32_t row = blockIdx.x;
-    const bool done = lean_row<MASKED>(A, row, shared);
+    const bool done = lean_row<MASKED, DT>(A, row, shared);
 #ifndef WS_LEAN_NO_FALLBACK
     if (done) return;
     __syncthreads();  // whatever the lean path left in LDS is dead

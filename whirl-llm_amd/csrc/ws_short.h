@@ -52,63 +52,6 @@ struct ShortShared {
     uint32_t bcnt[64], bstart[64];  // the bucket sort's counts and starts
 };
 
-// Sorts the n (<= kShortCap) different 64-bit keys keys[0 .. n) in LDS into descending order. bucket_of(key) in [0, nb)
-// (nb: 64 or 256; bcnt, bstart: nb words of LDS each) must not rise along that order (equal for keys it cannot tell apart): a key's place is the start of its bucket plus
-// the number of larger keys among the bucket's members, which it reads after all keys have been laid out bucket by
-// bucket - a few dozen reads a key where a full comparison sort takes dozens of barriers. Every thread calls it.
-template <class B>
-__device__ __forceinline__ void bucket_sort_desc(uint64_t* keys, uint32_t n, uint32_t* bcnt, uint32_t* bstart, uint32_t nb, B&& bucket_of) {
-    constexpr uint32_t K = kShortCap / WS_BLOCK;
-    const uint32_t t = threadIdx.x;
-    uint64_t key[K];
-    uint32_t bk[K], pos[K];
-#pragma unroll
-    for (uint32_t k = 0; k < K; ++k) key[k] = k * WS_BLOCK + t < n ? keys[k * WS_BLOCK + t] : 0ull;
-    if (t < nb) bcnt[t] = 0u;
-    __syncthreads();
-#pragma unroll
-    for (uint32_t k = 0; k < K; ++k)
-        if (k * WS_BLOCK + t < n) {
-            bk[k] = min(nb - 1u, bucket_of(key[k]));
-            pos[k] = atomicAdd(&bcnt[bk[k]], 1u);
-        }
-    __syncthreads();
-    if (t < 64u) {  // one wave: nb / 64 consecutive counts a lane
-        const uint32_t per = nb >> 6;
-        uint32_t c = 0;
-        for (uint32_t i = 0; i < per; ++i) c += bcnt[t * per + i];
-        uint32_t run = wave_incl_scan(c) - c;
-        for (uint32_t i = 0; i < per; ++i) {
-            bstart[t * per + i] = run;
-            run += bcnt[t * per + i];
-        }
-    }
-    __syncthreads();
-#pragma unroll
-    for (uint32_t k = 0; k < K; ++k)
-        if (k * WS_BLOCK + t < n) keys[bstart[bk[k]] + pos[k]] = key[k];
-    __syncthreads();
-#pragma unroll
-    for (uint32_t k = 0; k < K; ++k)
-        if (k * WS_BLOCK + t < n) {
-            const uint32_t b0 = bstart[bk[k]], c = bcnt[bk[k]];
-            uint32_t above = 0;
-            for (uint32_t i = 0; i < c; i += 4u) {  // four reads on their way together
-                uint64_t o[4];
-#pragma unroll
-                for (uint32_t q = 0; q < 4u; ++q) o[q] = keys[b0 + min(i + q, c - 1u)];
-#pragma unroll
-                for (uint32_t q = 0; q < 4u; ++q) above += (i + q < c && o[q] > key[k]) ? 1u : 0u;
-            }
-            pos[k] = b0 + above;
-        }
-    __syncthreads();
-#pragma unroll
-    for (uint32_t k = 0; k < K; ++k)
-        if (k * WS_BLOCK + t < n) keys[pos[k]] = key[k];
-    __syncthreads();
-}
-
 // LDS of a row: [0, 32 KiB) the list (before the sweep: the head's bin counts), then at lds_ab the bitmap of the touched
 // tokens, its 16-bit popcount prefixes, and at lds_cnt the per-rank words {history count | bias entries << 20 | claimed}
 // and 16-bit indices of each rank's first bias entry.
