@@ -315,7 +315,9 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 #pragma unroll
                     for (uint32_t e = 0; e < TPV; ++e) {
                         const float d = fminf(__fmul_rn(__fsub_rn(ref, x[e]), c64), 4095.f);  // (-inf, and anything 64 e-folds down: the last bin)
-                        if (round == 0 ? d < kNear : d >= kNear) atomicAdd(&head_cnt[static_cast<uint32_t>(d)], 1u);
+                        // (the last bin - masked-out tokens, nine in ten of some rows - is nobody's threshold and is
+                        // not counted: the additions of a wave to that one word would queue up sixty-four deep)
+                        if (round == 0 ? d < kNear : (d >= kNear && d < 4095.f)) atomicAdd(&head_cnt[static_cast<uint32_t>(d)], 1u);
                     }
                 }
             }
@@ -426,6 +428,8 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             for (uint32_t k = 0; k < 4u; ++k) {
                 raw[k] = -INFINITY;
                 if (k * WS_BLOCK < n_live && !(old[k] & kClaim)) {
+                    // (the logit only where the mask allows the token: nine in ten of a masked row's history ids would
+                    // fetch a sector each for nothing, half as many bytes again as the row itself)
                     const bool allowed = !MASKED || ((allow[id[k] >> 5] >> (id[k] & 31u)) & 1u);
                     if (allowed)
                         raw[k] = DT == 0 ? reinterpret_cast<const float*>(base)[id[k]] : bf16_to_f32(reinterpret_cast<const uint16_t*>(base)[id[k]]);
@@ -475,9 +479,25 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         }
     }
     WSS_MARK(4);  // touched tokens in
-    __syncthreads();
-    m = block_max(m, S.red_f);
-    double z = block_sum(static_cast<double>(s), S.red_d);  // against `ref`
+    double z;  // the sum against `ref`
+    {          // the block's maximum and sum with one barrier between them
+        const float wm_ = wave_max(m);
+        const double ws_ = wave_sum(static_cast<double>(s));
+        __syncthreads();
+        if (lane == 0u) {
+            S.red_f[wv] = wm_;
+            S.red_d[wv] = ws_;
+        }
+        __syncthreads();
+        m = S.red_f[0];
+        z = S.red_d[0];
+#pragma unroll
+        for (uint32_t w = 1; w < WS_WAVES; ++w) {
+            m = fmaxf(m, S.red_f[w]);
+            z += S.red_d[w];
+        }
+    }
+    WSS_MARK(9);
     uint32_t n_list = S.s_w[1];
     bool bad = not_mine || S.s_w[2] != 0u || n_list > kShortCap || !(ref > -INFINITY) || !(m > -INFINITY) || !(__fsub_rn(m, ref) * inv_t < 80.f);
     float thr_max = thr;
@@ -489,74 +509,119 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         uint32_t* ctrl = reinterpret_cast<uint32_t*>(work + kShortSplitCtrl);
         const uint32_t region = kShortCap / n_parts;  // every part has its own stretch of the list: nothing to reserve
         if (n_list > region) bad = true;
+        // Nothing here waits for a store to be acknowledged: a word or key that has been written is not zero (the
+        // workspace is, between launches), and the part that finishes the row reads again what it still finds zero.
         if (t == 0) {
             uint32_t* mine = ctrl + 64u + 8u * part;
             __hip_atomic_store(&mine[0], key32(m > -INFINITY ? m : -INFINITY), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(&mine[1], key32(thr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            // the sum against the part's own maximum (against `ref` it may not be a number when the slice holds no token)
-            const double zm = m > -INFINITY ? z * exp(static_cast<double>(__fsub_rn(ref, m)) * static_cast<double>(inv_t)) : 0.0;
-            __hip_atomic_store(reinterpret_cast<unsigned long long*>(&mine[2]), static_cast<unsigned long long>(__double_as_longlong(zm)),
+            // the sum as it is, against the part's `ref`, and `ref` with it (zero when the slice holds no token: against
+            // such a `ref` it may not be a number); its last bit set, so that the word is not zero
+            const double zr = m > -INFINITY ? z : 0.0;
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(&mine[2]), static_cast<unsigned long long>(__double_as_longlong(zr)) | 1ull,
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&mine[4], bad ? 0xffffffffu : n_list, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&mine[5], key32(ref), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&mine[4], bad ? 0xffffffffu : n_list + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (!bad)
             for (uint32_t k = t; k < n_list; k += WS_BLOCK)
                 __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[part * region + k]), static_cast<unsigned long long>(list[k]),
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's stores have been acknowledged
+        __syncthreads();  // every wave's stores have been issued
+        WSS_MARK(10);
+        // (The ticket orders nothing by itself and need not: every word the parts exchange is written and read by
+        // device-scope atomic accesses, which go past this unit's caches. An acquire / release ticket would write back
+        // and invalidate the caches on top of that, some thousand clocks on every part.)
+        if (t == 0) S.s_w[5] = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (t == 0) S.s_w[5] = __hip_atomic_fetch_add(&ctrl[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
+        WSS_MARK(11);
         if (S.s_w[5] != n_parts - 1u) return true;  // not the last: done
         finisher = true;
-        // the last part: everybody's results (device-scope loads: no stale copy from this unit's caches). Lane p of every
-        // wave reads part p's words - all loads on their way at once - and the wave reduces them.
-        float mp = -INFINITY, tp = -INFINITY;
-        double zp = 0.0;
-        uint32_t np = 0u;
-        if (lane < n_parts) {
-            mp = unkey32(__hip_atomic_load(&ctrl[64u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            tp = unkey32(__hip_atomic_load(&ctrl[65u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            zp = __longlong_as_double(static_cast<long long>(
-                __hip_atomic_load(reinterpret_cast<unsigned long long*>(&ctrl[66u + 8u * lane]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
-            np = __hip_atomic_load(&ctrl[68u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        // the last part: everybody's results. Lane p of the first wave reads part p's words - all loads on their way at
+        // once - and the wave reduces them. A word still zero is on its way (its store was issued before the ticket was
+        // drawn, this load after it came back): read again, a bounded number of times.
+        constexpr uint32_t kTries = 64u;
         // (the keys are asked for right away, every place of every stretch: which of them count is known when the parts' words are in)
         constexpr uint32_t kSlots = kShortCap / WS_BLOCK;
         uint64_t got[kSlots];
 #pragma unroll
         for (uint32_t i = 0; i < kSlots; ++i)
             got[i] = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[i * WS_BLOCK + t]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float mm = wave_max(mp), tt = wave_max(tp);
-        const double zz = wave_sum(mp > -INFINITY ? zp * exp(static_cast<double>(__fsub_rn(mp, mm)) * static_cast<double>(inv_t)) : 0.0);
-        bad = __ballot(np == 0xffffffffu) != 0ull;
-        const uint32_t np_ok = np == 0xffffffffu ? 0u : np;
-        const uint32_t off = wave_incl_scan(np_ok) - np_ok;  // where part p's keys go in the merged list
-        n_list = wave_sum(np_ok);
-        __syncthreads();  // (everybody is done with its own list)
-        if (wv == 0u && lane < n_parts) {
-            S.red_u[lane] = np_ok;
-            S.s_w[lane & 15u] = off;
+        if (t == 0) S.bcnt[0] = 0u;  // (a key is missing)
+        __syncthreads();             // (everybody is done with its own list)
+        if (wv == 0u) {  // (one wave: sixteen doing the same arithmetic side by side take four times as long)
+            float mp = -INFINITY, tp = -INFINITY, rp = -INFINITY;
+            double zp = 0.0;
+            uint32_t np = 0u;
+            bool late = false;
+            for (uint32_t tries = 0; tries < kTries; ++tries) {
+                uint32_t w0 = 1u, w1 = 1u, w4 = 1u, w5 = 1u;
+                unsigned long long w2 = 1ull;
+                if (lane < n_parts) {
+                    w0 = __hip_atomic_load(&ctrl[64u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    w1 = __hip_atomic_load(&ctrl[65u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    w2 = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&ctrl[66u + 8u * lane]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    w4 = __hip_atomic_load(&ctrl[68u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    w5 = __hip_atomic_load(&ctrl[69u + 8u * lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    mp = unkey32(w0);
+                    tp = unkey32(w1);
+                    zp = __longlong_as_double(static_cast<long long>(w2));
+                    np = w4 == 0xffffffffu ? w4 : w4 - 1u;
+                    rp = unkey32(w5);
+                }
+                late = __ballot(w0 == 0u || w1 == 0u || w2 == 0ull || w4 == 0u || w5 == 0u) != 0ull;
+                if (!late) break;
+            }
+            const float mm = wave_max(mp), tt = wave_max(tp);
+            const double zz = wave_sum(mp > -INFINITY ? zp * exp(static_cast<double>(__fsub_rn(rp, mm)) * static_cast<double>(inv_t)) : 0.0);
+            const bool any_bad = late || __ballot(np == 0xffffffffu) != 0ull;
+            const uint32_t np_ok = (late || np == 0xffffffffu) ? 0u : np;
+            const uint32_t off = wave_incl_scan(np_ok) - np_ok;  // where part p's keys go in the merged list
+            const uint32_t total = wave_sum(np_ok);
+            if (lane < n_parts) {
+                S.red_u[lane] = np_ok;
+                S.s_w[lane & 15u] = off;
+            }
+            if (lane == 0u) {
+                S.red_f[0] = mm;
+                S.red_f[1] = tt;
+                S.s_d[0] = zz;
+                S.bstart[0] = total;
+                S.bstart[1] = (any_bad ? 1u : 0u) | (late ? 2u : 0u);
+            }
         }
+        WSS_MARK(12);
         __syncthreads();
-        m = mm;
-        thr_max = tt;
-        z = zz;  // against the row's maximum from here on
-        ref = mm;
+        m = S.red_f[0];
+        thr_max = S.red_f[1];
+        z = S.s_d[0];  // against the row's maximum from here on
+        ref = m;
+        n_list = S.bstart[0];
+        bad = (S.bstart[1] & 1u) != 0u;
+        const bool late = (S.bstart[1] & 2u) != 0u;
         if (!(m > -INFINITY) || n_list > kShortCap) bad = true;
+        const uint32_t region_log2 = static_cast<uint32_t>(__ffs(region)) - 1u;  // (a power of two, as the number of parts is)
         {
+            bool missing = false;
 #pragma unroll
             for (uint32_t i = 0; i < kSlots; ++i) {
-                const uint32_t slot = i * WS_BLOCK + t, p = slot / region, k = slot - p * region;
+                const uint32_t slot = i * WS_BLOCK + t, p = slot >> region_log2, k = slot - (p << region_log2);
                 if (k < S.red_u[p]) {
+                    for (uint32_t tries = 0; got[i] == 0ull && tries < kTries; ++tries)  // (a key still on its way)
+                        got[i] = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&glist[slot]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (got[i] == 0ull) missing = true;
                     if (!bad) list[S.s_w[p] + k] = got[i];
                     // the workspace as the next launch needs it
                     __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[slot]), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else if (late) {  // (the parts' counts are not known: every place is cleared)
+                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(&glist[slot]), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
+            if (missing) S.bcnt[0] = 1u;
         }
         if (t < 64u + 8u * n_parts) __hip_atomic_store(&ctrl[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
+        if (S.bcnt[0] != 0u) bad = true;  // a key that never came: the row goes the other way
     }
     WSS_MARK(5);  // parts met
     const uint32_t n_cand = by_k ? top_k : n_list;  // candidates the rules look at

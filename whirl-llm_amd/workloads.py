@@ -107,12 +107,12 @@ def row_f32(c, r):
     return bf16_bits_to_f32(c["logits"][r]) if c["dtype"] == "bf16" else c["logits"][r].astype(np.float32)
 
 
-def upload(c, device="cuda:0", hints=True, min_p_hint=False):
+def upload(c, device="cuda:0", hints=True, min_p_hint=True):
     """numpy case -> dict of device tensors in the layouts ws_batch expects. hints: say what is known about the rows
     (top_k left out when no row has one, top_k_max), as a caller that wants the fastest kernel would; without them
     every batch goes the way a descriptor that says nothing goes. min_p_hint: also say min_p_min, which sends rows
-    without a top-k but with a min-p to the short-list kernel (measured on configs[1]: no faster than the split
-    single-sweep kernel there, 50 against 48 us, so the workloads do not say it by default)."""
+    without a top-k but with a min-p to the short-list kernel (measured on configs[1]: 45 against 48 us of the split
+    single-sweep kernel)."""
     import torch
     d = {}
     rows = c["rows"]
