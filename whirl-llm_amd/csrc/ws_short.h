@@ -180,9 +180,24 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 #pragma unroll
         for (uint32_t k = 0; k < kIds; ++k)
             if (k * WS_BLOCK < nh) mark(hid[k]);
-        for (uint32_t j = kIds * WS_BLOCK + t; j < nh; j += WS_BLOCK) mark(static_cast<uint32_t>(hist_ids[j]));
+        // (ids beyond those in registers: four loads on their way together, not one trip to memory each)
+        auto four = [&](const int32_t* ids, uint32_t n, uint32_t j0, uint32_t (&e)[4]) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) e[k] = j0 + k * WS_BLOCK + t < n ? static_cast<uint32_t>(ids[j0 + k * WS_BLOCK + t]) : 0xffffffffu;
+        };
+        for (uint32_t j0 = kIds * WS_BLOCK; j0 < nh; j0 += 4u * WS_BLOCK) {
+            uint32_t e[4];
+            four(hist_ids, nh, j0, e);
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) mark(e[k]);
+        }
         mark(bid);
-        for (uint32_t j = WS_BLOCK + t; j < nb; j += WS_BLOCK) mark(static_cast<uint32_t>(bias_ids[j]));
+        for (uint32_t j0 = WS_BLOCK; j0 < nb; j0 += 4u * WS_BLOCK) {
+            uint32_t e[4];
+            four(bias_ids, nb, j0, e);
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) mark(e[k]);
+        }
         __syncthreads();
         // popcount prefixes: five consecutive words a thread and round (one round up to 163840 tokens)
         constexpr uint32_t kChunk = 5u;
@@ -229,9 +244,19 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 #pragma unroll
         for (uint32_t k = 0; k < kIds; ++k)
             if (k * WS_BLOCK < nh) count(hid[k]);
-        for (uint32_t j = kIds * WS_BLOCK + t; j < nh; j += WS_BLOCK) count(static_cast<uint32_t>(hist_ids[j]));
+        for (uint32_t j0 = kIds * WS_BLOCK; j0 < nh; j0 += 4u * WS_BLOCK) {
+            uint32_t e[4];
+            four(hist_ids, nh, j0, e);
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) count(e[k]);
+        }
         bias_entry(bid, t);
-        for (uint32_t j = WS_BLOCK + t; j < nb; j += WS_BLOCK) bias_entry(static_cast<uint32_t>(bias_ids[j]), j);
+        for (uint32_t j0 = WS_BLOCK; j0 < nb; j0 += 4u * WS_BLOCK) {
+            uint32_t e[4];
+            four(bias_ids, nb, j0, e);
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) bias_entry(e[k], j0 + k * WS_BLOCK + t);
+        }
         __syncthreads();
     }
 
@@ -410,13 +435,27 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     if (!not_mine && n_touched) {
         constexpr uint32_t kClaim = 0x80000000u;
         auto rank = [&](uint32_t id) { return static_cast<uint32_t>(wprefix[id >> 5]) + __popc(touched[id >> 5] & ((1u << (id & 31u)) - 1u)); };
-        // up to four ids a thread at a time: the claims first, then the claimed tokens' logits all asked for together,
-        // then the arithmetic (n_live: ids left in this round, so that empty slots issue nothing)
-        auto some = [&](const uint32_t (&id)[4], uint32_t n_live) {
-            uint32_t old[4], r[4];
-            float raw[4];
+        // History and bias entries are one sequence here (whoever claims a token applies both kinds), up to eight
+        // entries a thread at a time: the ids not in registers asked for together, then the claims, then the claimed
+        // tokens' logits asked for together, then the arithmetic - three trips to memory a round
+        // (n_live: entries left in this round, so that empty slots issue nothing).
+        const uint32_t n_all = nh + nb;
+        auto some = [&](auto ks, uint32_t j0) {
+            constexpr uint32_t KS = decltype(ks)::value;
+            const uint32_t n_live = n_all - j0;
+            uint32_t id[KS], old[KS], r[KS];
+            float raw[KS];
 #pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) {
+            for (uint32_t k = 0; k < KS; ++k) {
+                id[k] = 0xffffffffu;
+                if (k * WS_BLOCK >= n_live) continue;  // uniform
+                const uint32_t j = j0 + k * WS_BLOCK + t;
+                if (j0 == 0u && k < kIds && (k + 1u) * WS_BLOCK <= nh) id[k] = hid[k];  // (uniform: a whole round of history ids in registers)
+                else if (j < nh) id[k] = static_cast<uint32_t>(hist_ids[j]);
+                else if (j < n_all) id[k] = static_cast<uint32_t>(bias_ids[j - nh]);
+            }
+#pragma unroll
+            for (uint32_t k = 0; k < KS; ++k) {
                 old[k] = kClaim;
                 r[k] = 0u;
                 if (k * WS_BLOCK < n_live && id[k] < V && id[k] >= tok0 && id[k] < tok1) {
@@ -425,7 +464,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 }
             }
 #pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) {
+            for (uint32_t k = 0; k < KS; ++k) {
                 raw[k] = -INFINITY;
                 if (k * WS_BLOCK < n_live && !(old[k] & kClaim)) {
                     // (the logit only where the mask allows the token: nine in ten of a masked row's history ids would
@@ -436,7 +475,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 }
             }
 #pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) {
+            for (uint32_t k = 0; k < KS; ++k) {
                 if (k * WS_BLOCK >= n_live) continue;  // uniform
                 const bool have = !(old[k] & kClaim);
                 float x = -INFINITY;
@@ -462,21 +501,10 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                 push(x, id[k], have && x > thr);
             }
         };
-        uint32_t id4[4];
-#pragma unroll
-        for (uint32_t k = 0; k < 4u; ++k) id4[k] = hid[k];
-        if (nh) some(id4, nh);
-        for (uint32_t jr = kIds * WS_BLOCK; jr < nh; jr += 4u * WS_BLOCK) {
-#pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k) id4[k] = jr + k * WS_BLOCK + t < nh ? static_cast<uint32_t>(hist_ids[jr + k * WS_BLOCK + t]) : 0xffffffffu;
-            some(id4, nh - jr);
-        }
-        for (uint32_t jr = 0; jr < nb; jr += 4u * WS_BLOCK) {
-#pragma unroll
-            for (uint32_t k = 0; k < 4u; ++k)
-                id4[k] = (jr == 0u && k == 0u) ? bid : (jr + k * WS_BLOCK + t < nb ? static_cast<uint32_t>(bias_ids[jr + k * WS_BLOCK + t]) : 0xffffffffu);
-            some(id4, nb - jr);
-        }
+        // (four entries a thread when that is all there is: the wider code costs a short list a microsecond)
+        if (n_all <= 4u * WS_BLOCK) some(std::integral_constant<uint32_t, 4u>{}, 0u);
+        else
+            for (uint32_t j0 = 0; j0 < n_all; j0 += 8u * WS_BLOCK) some(std::integral_constant<uint32_t, 8u>{}, j0);
     }
     WSS_MARK(4);  // touched tokens in
     double z;  // the sum against `ref`
