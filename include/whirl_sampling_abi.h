@@ -192,7 +192,7 @@ enum {
     WS_FLAG_ROUTE_SPLIT_ALONE = 1u << 11, /* a split row whose parts did not meet within split_spins looks: done by
                                             one workgroup. A caller that sees this often sets max_split = 1 */
     WS_FLAG_ROUTE_LEAN = 1u << 12,       /* done by the one-sweep kernel for batches without a top-k (information only) */
-    WS_FLAG_ROUTE_SHORT = 1u << 13       /* done by the short-list kernel for batches with a bounded top-k (information only) */
+    WS_FLAG_ROUTE_SHORT = 1u << 13       /* done by the short-list kernel for batches with a bounded top-k or a min-p (information only) */
 };
 #define WS_FLAG_ROUTE_MASK 0x3f00u
 
@@ -220,7 +220,8 @@ typedef struct ws_batch {
     uint64_t row_stride; /* elements between rows (>= vocab) */
 
     const float* inv_t;     /* 1 / temperature, > 0 (Sampler::inv_t) */
-    const uint32_t* top_k;  /* 0 = off (NULL: off) */
+    const uint32_t* top_k;  /* 0 = off (NULL: off - and the caller's word that no row has one: fp32 and bf16 batches
+                               without optional outputs then take the one-sweep kernel written for such rows) */
     const double* top_p;    /* 1 = off (NULL: off) */
     const double* min_p;    /* 0 = off (NULL: off) */
     const uint64_t* seed;   /* Sampler::seed */
@@ -312,7 +313,8 @@ typedef struct ws_batch {
                                    set as a top-k does: what passes lies within -ln(min_p) / inv_t of the row's maximum).
                                    With it - alone, or together with top_k_max for the rows that do have a top_k - the
                                    batch takes the short-list kernel. Useful from about 1e-3 upwards: a row whose floor
-                                   lets more than 1024 tokens through is handed back like one that breaks the word */
+                                   lets more than 4096 tokens through (a row shared by n workgroups: 4096 / n in one of its parts)
+                                   is handed back like one that breaks the word */
 } ws_batch;
 
 /* Bytes of device scratch ws_sample_batch needs for this batch shape (host-only computation). */
