@@ -343,6 +343,14 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist[b] = 0ull;
     if (hist2)
         for (uint32_t b = t; b < kBins; b += WS_BLOCK) hist2[b] = 0ull;
+    // (phase 0's tables as well, while the first loads travel: their sizes are the launch's, not the row's)
+    if (A.hist || A.bias_ids) {  // (a launch without either has no room for them)
+        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
+        for (uint32_t r = t; r < A.patch_cap; r += WS_BLOCK) {
+            cnt[r] = 0u;
+            first[r] = 0xffffffffu;
+        }
+    }
 
     // The row's parameters, every one of them with one scalar load, all asked for together and waited for once. (Written
     // as plain reads they become vector loads, each behind the test of its pointer and each waited for on its own: a
@@ -549,13 +557,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     // popcount prefix per word (rank of a touched id), per-rank history count and bias entries
     uint32_t n_touched = 0;
     auto phase0 = [&]() __attribute__((always_inline)) {
-    if (nh + nb > 0) {
-        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
-        for (uint32_t r = t; r < nh + nb; r += WS_BLOCK) {  // (at most nh + nb distinct ids)
-            cnt[r] = 0u;
-            first[r] = 0xffffffffu;
-        }
-        __syncthreads();
+    if (nh + nb > 0) {  // (the tables were cleared at the top; the anchor's barriers lie in between)
 #pragma unroll
         for (int k = 0; k < kHid; ++k)
             if (static_cast<uint32_t>(k) * WS_BLOCK < nh && hid[k] < V) atomicOr(&touched[hid[k] >> 5], 1u << (hid[k] & 31u));

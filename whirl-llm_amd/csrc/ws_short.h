@@ -100,6 +100,14 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         hna[k] = MASKED ? allow[(jc * TPV) >> 5] : 0xffffffffu;
     }
     for (uint32_t b = t; b < 4096u; b += WS_BLOCK) head_cnt[b] = 0u;
+    // (the tables of the touched tokens as well, while the parameters travel: their sizes are the launch's, not the row's)
+    if (A.hist || A.bias_ids) {
+        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
+        for (uint32_t r = t; r < A.patch_cap; r += WS_BLOCK) {
+            cnt[r] = 0u;
+            first[r] = 0xffffu;
+        }
+    }
 
     // ---- the row's parameters: scalar loads, asked for together (as in lean_row)
     LeanRowParams P;
@@ -168,12 +176,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
 #pragma unroll
         for (uint32_t k = 0; k < kIds; ++k) hid[k] = k * WS_BLOCK + t < nh ? static_cast<uint32_t>(hist_ids[k * WS_BLOCK + t]) : 0xffffffffu;
         if (t < nb) bid = static_cast<uint32_t>(bias_ids[t]);
-        for (uint32_t w = t; w < nW; w += WS_BLOCK) touched[w] = 0u;
-        for (uint32_t r = t; r < nh + nb; r += WS_BLOCK) {
-            cnt[r] = 0u;
-            first[r] = 0xffffu;
-        }
-        __syncthreads();
+        __syncthreads();  // (the tables were cleared at the top)
         auto mark = [&](uint32_t id) {
             if (id < V) atomicOr(&touched[id >> 5], 1u << (id & 31u));
         };
