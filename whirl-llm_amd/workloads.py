@@ -1,4 +1,5 @@
-"""Synthetic workloads of the sampling path: the configurations BASELINE.json lists and the north-star tile, as seeded
+"""Synthetic workloads of the sampling path: the five benchmark configurations (configs[0] .. configs[4]: a lone decode
+row, a mixed batch, bf16 Zipfian rows, classic verification, long masked rows) and the north-star tile, as seeded
 numpy arrays, their upload into the device layouts ws_batch expects, and a BatchSampler over them. Used by bench.py,
 the GPU tests and the smoke run; nothing here touches a CPU sampler."""
 import numpy as np
