@@ -659,7 +659,30 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
     if (bad || n_list < n_cand || n_cand == 0u || n_cand > kShortCap) return false;
 
     // ---- the candidates in order
-    {
+    if (n_list <= WS_BLOCK / 4u) {
+        // A short list (a lone row's top-k 40 lists some 200 keys): every key against every other, four threads a key,
+        // each counting the larger keys in a quarter of the list - two barriers, where the bucket sort takes seven.
+        const uint32_t ki = t >> 2, qr = t & 3u;
+        const uint32_t chunk = ((n_list + 7u) >> 3) << 1;  // keys a quarter, even: two keys a read
+        const uint32_t lo = qr * chunk, hi = min(lo + chunk, n_list);
+        const uint64_t own = ki < n_list ? list[ki] : 0ull;
+        uint32_t above = 0;
+        if (ki < n_list) {
+            for (uint32_t j = lo; j < hi; j += 8u) {  // four reads on their way together (one past the quarter's end stays inside the list's 32 KiB and is not counted)
+                ulonglong2 o[4];
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r) o[r] = *reinterpret_cast<const ulonglong2*>(&list[j + 2u * r]);
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r)
+                    above += ((j + 2u * r < hi && o[r].x > own) ? 1u : 0u) + ((j + 2u * r + 1u < hi && o[r].y > own) ? 1u : 0u);
+            }
+        }
+        above += __shfl_xor(above, 1);
+        above += __shfl_xor(above, 2);
+        __syncthreads();  // (every key has been read)
+        if (ki < n_list && qr == 0u) list[above] = own;  // (the keys are all different: so are their ranks)
+        __syncthreads();
+    } else {
         // buckets by how far below the maximum a logit lies, on the scale of the lowest listed one
         float dloc = 0.f;
         for (uint32_t k = t; k < n_list; k += WS_BLOCK)
