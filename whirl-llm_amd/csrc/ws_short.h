@@ -333,6 +333,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         // sixth of the tokens -, the others only when those turn out to be fewer than r_star.
         constexpr float kNear = 512.f;
         uint32_t b_star = 0xffffffffu;
+        if (t == 0) S.s_w[0] = 0xffffffffu;  // (the bin, once found; the barrier behind the counting publishes this)
         for (int round = 0; round < 2; ++round) {  // uniform
             float x[TPV];
 #pragma unroll
@@ -354,8 +355,6 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             const uint32_t mine = c4.x + c4.y + c4.z + c4.w;
             uint32_t total;
             const uint32_t before = block_excl_scan(mine, S.red_u, &total);
-            if (t == 0) S.s_w[0] = 0xffffffffu;
-            __syncthreads();
             if (before < r_star && before + mine >= r_star) {  // the bin in which the head's r_star-th largest lies
                 uint32_t run = before, b = 4u * t;
                 const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
@@ -372,14 +371,13 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
         }
         if (b_star >= 4095u) list_all = true;  // (fewer than r_star tokens above the last bin: everything is listed)
         else thr = __fsub_rn(ref, __fdiv_rn(static_cast<float>(b_star + 1u), c64));
-        __syncthreads();
     }
     if (list_all) thr = -INFINITY;
     if (t == 0) {
         S.s_w[1] = 0u;  // tokens listed
         S.s_w[2] = 0u;  // the list ran over
     }
-    __syncthreads();
+    __syncthreads();  // (the counts and the bin have been read: the list takes the counts' place)
 
     WSS_MARK(2);  // threshold known
     // ---- the sweep: maximum, sum of exp against `ref`, tokens above the threshold to the list
