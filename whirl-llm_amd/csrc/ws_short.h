@@ -63,6 +63,7 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
                                           bool& finisher) {
 #ifdef WS_SHORT_TIMERS
     const long long wss_t0 = clock64();
+    if (threadIdx.x == 0) S.marks[13] = 0.f;
 #endif
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr uint32_t TPV = DT == 0 ? 4u : 8u;  // tokens in a 128-bit vector
@@ -508,6 +509,9 @@ __device__ __forceinline__ bool short_row(const BatchArgs& A, const uint32_t row
             for (uint32_t j0 = 0; j0 < n_all; j0 += 8u * WS_BLOCK) some(std::integral_constant<uint32_t, 8u>{}, j0);
     }
     WSS_MARK(4);  // touched tokens in
+#ifdef WS_SHORT_TIMERS
+    if (lane == 0u) atomicMax(reinterpret_cast<int*>(&S.marks[13]), __float_as_int(static_cast<float>(clock64() - wss_t0)));  // the slowest wave's
+#endif
     double z;  // the sum against `ref`
     {          // the block's maximum and sum with one barrier between them
         const float wm_ = wave_max(m);
