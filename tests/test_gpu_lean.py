@@ -94,7 +94,7 @@ def test_no_history_no_bias_no_penalties():
 
 def test_thousands_of_equal_logits_at_the_cut():
     """Logits rounded to one decimal: every cut falls among thousands of ties, which the lower ids win
-    (src/sampling/sampler.cpp:18-21). Up to 2048 candidates a range are sorted in place; a row with more goes to the
+    (src/sampling/sampler.cpp:18-21). Up to 4096 candidates a row are sorted in place; a row with more goes to the
     three-pass code inside the launch and says so. Either way the answers are the oracle's."""
     c = _no_top_k(gc.make_cfg2(rows=8, V=151936, n_hist=500, n_bias=20))
     c["logits"] = np.round(c["logits"], 1)
@@ -116,6 +116,17 @@ def test_bf16_zipfian_rows_with_hundreds_of_ties_at_the_cut():
     # (two of these rows have their cut within 1e-7 of a token's edge and are reported as such, by every kernel here)
     res, _ = run_lean(c, 1, max_differ=2, handed_back=2)
     assert res["exact"] >= 62 and res["lean"] >= 62, res
+    print(res)
+
+
+def test_bf16_ties_from_hundreds_to_thousands_at_the_cut():
+    """The same rows with top-p from 0.8 to 0.985: the deeper the cut, the more tokens share its bf16 value - 500 to
+    beyond the 4096 a row that the kernel sorts in place (one, two, three and four candidates a thread, the 1024
+    buckets and the 256); the rows beyond are handed back. Every answer is the oracle's either way."""
+    c = gc.make_cfg3(rows=18)
+    c["top_p"][:] = np.repeat([0.8, 0.9, 0.93, 0.95, 0.97, 0.985], 3)
+    res, _ = run_lean(c, 0, max_differ=2, handed_back=9)
+    assert res["exact"] >= 16 and res["lean"] >= 9, res
     print(res)
 
 

@@ -13,7 +13,7 @@
 //     latencies.
 //   * the histogram is scanned four consecutive bins per thread, the cuts' and the draw's bins are found by all threads
 //     at once (every thread tests the bins it has just scanned), and one wave works out what follows from the answers.
-//   * the candidates - the tokens of those bins, 2048 a range at most - are put in their exact order (logit descending,
+//   * the candidates - the tokens of those bins, 4096 a row at most - are put in their exact order (logit descending,
 //     id ascending) by a bucket sort of their 64-bit keys whose buckets follow the keys that are there, thousands of
 //     equal logits included; a block-wide scan of their masses in that order settles the cuts and the draw.
 #pragma once
@@ -29,7 +29,8 @@ namespace ws {
 
 constexpr int kLeanRegs = 40;   // bin-cache registers per thread: 160 tokens, rows of up to 163840 tokens
 constexpr int kLeanBatch = 2;   // 128-bit loads per thread and batch
-constexpr uint32_t kLeanBuckets = 128u, kLeanMaxRange = 2048u;  // (kLeanBuckets: words of the finish's tables in LeanShared)
+constexpr uint32_t kLeanBuckets = 128u;   // words of the finish's tables in LeanShared
+constexpr uint32_t kLeanMaxList = 4096u;  // candidates of a row's ranges together: what the sort's 32 KiB hold
 // The bins the cut and the draw can fall in: sixteen at most, with eight different cache bytes at most among them (fp32
 // rows: eight bins; bf16 rows, where four neighbours share a byte: all sixteen).
 constexpr uint32_t kLeanMaxBins = 16u;
@@ -1043,7 +1044,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }
         const bool has_r1 = r1hi >= r1lo;
         const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
-        ok = ok && r0hi < kLeanTail && nb0 + nb1 <= kLeanMaxBins && n_r0 + n_r1 != 0u && n_r0 <= kLeanMaxRange && n_r1 <= kLeanMaxRange;
+        ok = ok && r0hi < kLeanTail && nb0 + nb1 <= kLeanMaxBins && n_r0 + n_r1 != 0u && n_r0 + n_r1 <= kLeanMaxList;
         {  // the bytes to scan the cache for: lane k looks at the k-th bin of the ranges, the first of a kind is listed
             const uint32_t my_bin = lane < nb0 ? static_cast<uint32_t>(r0lo) + lane : static_cast<uint32_t>(r1lo) + (lane - nb0);
             const uint32_t my_byte = (my_bin >> kCacheShift) & 0xffu;
@@ -1159,7 +1160,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
 
     // ------------------------------------------------------------------ the finds that are candidates: a token of another
     // bin with the same low bits, a masked-out token and a touched token found by its raw logit are dropped
-    uint2* cand = reinterpret_cast<uint2*>(lds);  // (token | slot << 28, logit bits), kLeanMaxRange * 2 entries at most
+    uint2* cand = reinterpret_cast<uint2*>(lds);  // (token | slot << 28, logit bits), kLeanMaxList entries at most
     const bool r1_first = has_r1 && r1lo < r0lo;  // range 1 holds the larger logits
     // a candidate's slot: the number of its bin among the ranges' bins in descending order of the logits
     auto slot_of = [&](float x) {
@@ -1193,7 +1194,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             uint32_t base = 0;
             if (lane == 0u && mk) base = atomicAdd(&s_w[5], static_cast<uint32_t>(__popcll(mk)));
             const uint32_t slot = __shfl(base, 0) + static_cast<uint32_t>(__popcll(mk & ((1ull << lane) - 1ull)));
-            if (ok && slot < 2u * kLeanMaxRange) {
+            if (ok && slot < kLeanMaxList) {
                 const uint32_t s_ = slot_of(x), k32 = static_cast<uint32_t>(key64(x, 0u) >> 32);
                 cand[slot] = make_uint2(id | (s_ << 28), __float_as_uint(x));
                 atomicMin(&b_cnt[s_ * 8u + (lane & 7u)], k32);
@@ -1218,7 +1219,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     // its candidates tie, as bf16 rows have them by the hundred, a 32nd of the vocabulary's ids: either way some dozens
     // of keys to compare with, and no limit on ties. A key's place is the start of its bucket plus the number of larger
     // keys among the bucket's members, which it reads once all keys lie bucket by bucket.
-    constexpr int kRounds = 2 * kLeanMaxRange / WS_BLOCK;  // the candidates at places kRounds t .. kRounds t + kRounds - 1 of the order
+    constexpr int kRounds = kLeanMaxList / WS_BLOCK;  // the candidates at places kRounds t .. kRounds t + kRounds - 1 of the order
     uint64_t* keys = reinterpret_cast<uint64_t*>(lds);            // bucket by bucket (over the candidates' pairs, which are in registers by then)
     uint64_t* sorted = reinterpret_cast<uint64_t*>(lds + 32768);  // in order (over the finds' list)
     {
