@@ -662,6 +662,7 @@ struct TailIn {
     float aq, c64;
     uint64_t kept_key;
     uint32_t want;
+    uint32_t n_kept;  // tokens the dump will write (0: not known)
 };
 struct TailCut {
     uint32_t key, n_equal;
@@ -735,7 +736,7 @@ __device__ __noinline__ TailCut tail_cut(const TailIn in) {
 // writes one find.
 template <class KEEP, class RESERVE, class EMIT>
 __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, uint32_t n_equal, float floor, uint64_t* room, KEEP&& keep,
-                                                  RESERVE&& reserve, EMIT&& emit) {
+                                                  RESERVE&& reserve, EMIT&& emit, uint32_t n_expect = 0u) {
     __shared__ uint32_t w_cnt[2 * WS_WAVES];
     constexpr uint32_t kShare = 8192u / WS_WAVES;  // entries of `room` per wave
     constexpr uint32_t kAhead = 16u;
@@ -790,7 +791,7 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
         }
         return f;
     };
-    if (!ties) {  // uniform
+    if (!ties && n_expect <= 8192u) {  // uniform (a kept set known to be larger than the room goes straight to the two passes)
         uint64_t* line = room + wave * kShare;
         uint32_t wc = 0;
         auto sweep = [&](auto whole_) {
@@ -842,18 +843,22 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
     // ---- two passes, eight tiles on their way at a time (kept sets of many thousands, rows with ties)
     constexpr uint32_t kAhead2 = 8u;
     uint32_t nk = 0, nt = 0;
-    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
-        uint4 raw[kAhead2];
+    auto count_pass = [&](auto whole_) {
+        for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
+            uint4 raw[kAhead2];
 #pragma unroll
-        for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, std::false_type{});
+            for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, whole_);
 #pragma unroll
-        for (uint32_t u = 0; u < kAhead2; ++u) {
-            float x[4];
-            const uint32_t f = judge(i0 + 256u * u + 4u * lane, raw[u], x);
-            nk += __popc(f & 0xfu);
-            nt += __popc(f >> 4);
+            for (uint32_t u = 0; u < kAhead2; ++u) {
+                float x[4];
+                const uint32_t f = judge(i0 + 256u * u + 4u * lane, raw[u], x);
+                nk += __popc(f & 0xfu);
+                nt += __popc(f >> 4);
+            }
         }
-    }
+    };
+    if (whole) count_pass(std::true_type{});  // (one aligned 128-bit load a quad where the stretch allows it)
+    else count_pass(std::false_type{});
     nk = wave_sum(nk);
     nt = wave_sum(nt);
     __syncthreads();  // (w_cnt may still be read: the attempt above, an earlier call)
@@ -873,33 +878,37 @@ __device__ __forceinline__ void write_in_id_order(const RowView& rv, bool ties, 
     }
     base += reserve(all_k + min(all_t, n_equal));
     if (!(nk | nt)) return;  // nothing kept in this wave's stretch (uniform over the wave; no barrier follows)
-    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
-        uint4 raw[kAhead2];
+    auto write_pass = [&](auto whole_) {
+        for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead2) {
+            uint4 raw[kAhead2];
 #pragma unroll
-        for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, std::false_type{});
+            for (uint32_t u = 0; u < kAhead2; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane, whole_);
 #pragma unroll
-        for (uint32_t u = 0; u < kAhead2; ++u) {
-            float x[4];
-            const uint32_t i = i0 + 256u * u + 4u * lane;
-            const uint32_t f = judge(i, raw[u], x);
-            if (!__ballot(f != 0u)) continue;
-            const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
-            const uint32_t inc = wave_incl_scan(mine);
-            uint32_t kb = base + ((inc - mine) & 0xffffu), tb = tail_base + ((inc - mine) >> 16);
+            for (uint32_t u = 0; u < kAhead2; ++u) {
+                float x[4];
+                const uint32_t i = i0 + 256u * u + 4u * lane;
+                const uint32_t f = judge(i, raw[u], x);
+                if (!__ballot(f != 0u)) continue;
+                const uint32_t mine = __popc(f & 0xfu) | (__popc(f >> 4) << 16);  // at most 256 of either in a tile
+                const uint32_t inc = wave_incl_scan(mine);
+                uint32_t kb = base + ((inc - mine) & 0xffffu), tb = tail_base + ((inc - mine) >> 16);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const bool tie = (f >> (4 + e)) & 1u;
-                const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
-                const uint32_t o = kb + min(tb, n_equal);
-                if (k) emit(o, i + e, x[e]);
-                kb += (f >> e) & 1u;
-                tb += tie ? 1u : 0u;
+                for (int e = 0; e < 4; ++e) {
+                    const bool tie = (f >> (4 + e)) & 1u;
+                    const bool k = ((f >> e) & 1u) || (tie && tb < n_equal);
+                    const uint32_t o = kb + min(tb, n_equal);
+                    if (k) emit(o, i + e, x[e]);
+                    kb += (f >> e) & 1u;
+                    tb += tie ? 1u : 0u;
+                }
+                const uint32_t tot = last_lane(inc);
+                base += tot & 0xffffu;
+                tail_base += tot >> 16;
             }
-            const uint32_t tot = last_lane(inc);
-            base += tot & 0xffffu;
-            tail_base += tot >> 16;
         }
-    }
+    };
+    if (whole) write_pass(std::true_type{});
+    else write_pass(std::false_type{});
 }
 
 // Entries of the single-sweep kernel's candidate list: (token | flags, logit bits).
@@ -968,6 +977,99 @@ __device__ __noinline__ void dump_listed_candidates(const void* base, int dtype,
     dump_by_counting(sel_at, min(*counter, sel_cap), kid, klg, kept_cap);
 }
 
+// The usual dump - every token whose key is at or above `kept_key`, nothing else wanted - of a row of whole, aligned
+// 128-bit vectors, in ascending id order: two passes over the wave's stretch of the row (count, then write), some
+// a hundred instructions a tile of 256 tokens each where the general code below takes 180.
+__device__ __noinline__ void dump_kept_fast(const TailIn in, int32_t* kid, float* klg, uint32_t kept_cap) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    __shared__ uint32_t w_kept[WS_WAVES];
+    const uint32_t V = in.V, nW = (V + 31u) >> 5;
+    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+    const bool any_touched = in.touched_at != 0xffffffffu;
+    RowView rv;
+    rv.base = in.base;
+    rv.V = V;
+    rv.dtype = in.dtype;
+    rv.vec = false;
+    rv.allow = in.allow;
+    rv.touched = any_touched ? reinterpret_cast<const uint32_t*>(lds + in.touched_at) : nullptr;
+    rv.wprefix = reinterpret_cast<const uint16_t*>(lds + (any_touched ? in.touched_at : 0u) + nW * 4u);
+    rv.pv = reinterpret_cast<const float*>(lds + (any_touched ? in.touched_at : 0u) + nW * 4u + ((nW * 2u + 15u) & ~15u));
+    const uint64_t kept_key = in.kept_key;
+    const uint32_t tiles = (V + 255u) >> 8, per_wave = (tiles + WS_WAVES - 1u) / WS_WAVES;
+    const uint32_t lo = min(wave * per_wave, tiles) << 8, hi = min(min((wave + 1u) * per_wave, tiles) << 8, V);
+    const bool f32 = in.dtype == 0;
+    // tokens i .. i + 3 (i a multiple of four below hi): their logits as the sampler saw them, bit e of the result: kept
+    auto fetch = [&](uint32_t i) -> uint4 {
+        if (i >= hi) i = lo < V ? lo : 0u;  // (a lane past the stretch reads the stretch's first tokens again and is ignored)
+        if (f32) return *reinterpret_cast<const uint4*>(static_cast<const float*>(in.base) + i);
+        const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(in.base) + i);
+        return make_uint4(q.x << 16, q.x & 0xffff0000u, q.y << 16, q.y & 0xffff0000u);
+    };
+    auto judge = [&](uint32_t i, const uint4 raw, float (&x)[4]) -> uint32_t {
+        if (i >= hi) return 0u;
+        x[0] = fmaxf(__uint_as_float(raw.x), -INFINITY), x[1] = fmaxf(__uint_as_float(raw.y), -INFINITY);  // NaN -> -inf
+        x[2] = fmaxf(__uint_as_float(raw.z), -INFINITY), x[3] = fmaxf(__uint_as_float(raw.w), -INFINITY);
+        const uint32_t tb = rv.touched ? (rv.touched[i >> 5] >> (i & 31u)) & 0xfu : 0u;
+        const uint32_t ab = rv.allow ? (rv.allow[i >> 5] >> (i & 31u)) & 0xfu : 0xfu;
+        if (tb | (ab ^ 0xfu)) {  // (rare: a token the lists touch has its adjusted logit in the table, a masked-out one none)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if ((tb >> e) & 1u) x[e] = rv.pv[rank_of(rv, i + e)];
+                else if (!((ab >> e) & 1u)) x[e] = -INFINITY;
+            }
+        }
+        uint32_t f = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f |= (key64(x[e], i + e) >= kept_key) ? 1u << e : 0u;  // (one 64-bit compare a token)
+        return f;
+    };
+    constexpr uint32_t kAhead = 8u;
+    uint32_t nk = 0;
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead) {
+        uint4 raw[kAhead];
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane);
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; ++u) {
+            float x[4];
+            nk += __popc(judge(i0 + 256u * u + 4u * lane, raw[u], x));
+        }
+    }
+    nk = wave_sum(nk);
+    __syncthreads();  // (whoever used the LDS words before is done)
+    if (lane == 0) w_kept[wave] = nk;
+    __syncthreads();
+    uint32_t base = 0;
+    for (uint32_t w = 0; w < wave; ++w) base += w_kept[w];
+    if (!nk) return;  // nothing kept in this wave's stretch (uniform over the wave; no barrier follows)
+    for (uint32_t i0 = lo; i0 < hi; i0 += 256u * kAhead) {
+        uint4 raw[kAhead];
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; ++u) raw[u] = fetch(i0 + 256u * u + 4u * lane);
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; ++u) {
+            float x[4];
+            const uint32_t i = i0 + 256u * u + 4u * lane;
+            const uint32_t f = judge(i, raw[u], x);
+            if (!__ballot(f != 0u)) continue;
+            const uint32_t mine = __popc(f);
+            const uint32_t inc = wave_incl_scan(mine);
+            uint32_t o = base + inc - mine;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (!((f >> e) & 1u)) continue;
+                if (o < kept_cap) {
+                    kid[o] = static_cast<int32_t>(i + e);
+                    if (klg) klg[o] = x[e];
+                }
+                ++o;
+            }
+            base += last_lane(inc);
+        }
+    }
+}
+
 // The kept set of a row in ascending id order (the optional dump): every token whose key is at or above `kept_key`, and
 // `want` zero-mass candidates (tail_cut). A function of its own, like the exact path: it runs for callers that ask for
 // the dump only, and the kernel keeps its registers for what every row needs.
@@ -1010,7 +1112,8 @@ __device__ __noinline__ void dump_kept_set(const TailIn in, int32_t* kid, float*
                 kid[o] = static_cast<int32_t>(i);
                 if (klg) klg[o] = x;
             }
-        });
+        },
+        in.n_kept);
 }
 
 // ---- split rows whose kept set is not among the candidates (top-p / min-p without a top-k)
@@ -3938,10 +4041,14 @@ __device__ __forceinline__ void sample_row(const BatchArgs& A, const uint32_t bl
         in.c64 = c64;
         in.kept_key = kept_key;
         in.want = tail_extra;
+        in.n_kept = n3 + tail_extra;
         __syncthreads();
         int32_t* kid = kept_ids + static_cast<size_t>(row) * A.kept_cap;
         float* klg = A.kept_logits ? A.kept_logits + static_cast<size_t>(row) * A.kept_cap : nullptr;
-        dump_kept_set(in, kid, klg, A.kept_cap);
+        // (rows of whole, aligned vectors with nothing but the kept set wanted: the lean dump)
+        const bool aligned_row = (reinterpret_cast<uintptr_t>(rv.base) & (rv.dtype == 0 ? 15u : 7u)) == 0 && (V & 3u) == 0;
+        if (tail_extra == 0u && aligned_row) dump_kept_fast(in, kid, klg, A.kept_cap);
+        else dump_kept_set(in, kid, klg, A.kept_cap);
     }
 }
 
