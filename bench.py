@@ -34,11 +34,11 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, kernel_digest() at the time)
-    ("tile", "auto"): (208286897, "lean_batch_kernel_tile_256x151936_f32.txt", "8e21ac30c64f86e9"),
-    ("cfg1", "auto"): (1217371, "short_batch_kernel_cfg1_1x151936_f32.txt", "8e21ac30c64f86e9"),
-    ("cfg2", "auto"): (56836656, "short_batch_kernel_cfg2_64x151936_f32.txt", "8e21ac30c64f86e9"),
-    ("cfg3", "auto"): (115289404, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "8e21ac30c64f86e9"),
-    ("cfg5", "auto"): (1363583248, "short_batch_kernel_cfg5_1024x262144_f32.txt", "8e21ac30c64f86e9"),
+    ("tile", "auto"): (208285815, "lean_batch_kernel_tile_256x151936_f32.txt", "d3748406a8578277"),
+    ("cfg1", "auto"): (1213453, "short_batch_kernel_cfg1_1x151936_f32.txt", "d3748406a8578277"),
+    ("cfg2", "auto"): (56830885, "short_batch_kernel_cfg2_64x151936_f32.txt", "d3748406a8578277"),
+    ("cfg3", "auto"): (115290219, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "d3748406a8578277"),
+    ("cfg5", "auto"): (1363218685, "short_batch_kernel_cfg5_1024x262144_f32.txt", "d3748406a8578277"),
 }
 
 
