@@ -408,6 +408,63 @@ def host_decode_step(steps):
     return out
 
 
+def route_census(rows=256, steps=10):
+    """How often rows leave their kernel's usual way, and what a launch costs when some do: batches of `rows` rows x
+    151936 tokens without a top-k (the one-sweep kernel) over logit shapes, temperatures and top-p / min-p settings
+    beyond the benchmark's own. One entry per cell: rows by route and the launch time on a resident copy."""
+    import numpy as np
+    import torch
+    w = workloads()
+    out = []
+
+    def cell(name, c):
+        d = w.upload(c)
+        smp = w.sampler_for(c, d, 1, mode=MODE)
+        for _ in range(3):
+            smp.run()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(steps):
+            smp.run()
+        ev1.record()
+        torch.cuda.synchronize()
+        rep = device_report(smp)
+        routes = {k: v for k, v in rep["routes"].items() if v}
+        out.append(dict(cell=name, rows=c["rows"], routes=routes, failed_rows=rep["device_failed_rows"], launch_us=round(ev0.elapsed_time(ev1) / steps * 1e3, 1)))
+
+    rng = np.random.default_rng(DATA_SEED_CENSUS)
+    base = w.make_tile(rows=rows)
+    V = base["V"]
+    for sigma in (1.0, 2.0, 4.0):
+        x = (rng.standard_normal((rows, V)) * sigma).astype(np.float32)
+        for temp in (0.5, 1.0, 1.5):
+            for top_p in (0.8, 0.95, 0.99, 0.999):
+                c = dict(base)
+                c.update(logits=x, inv_t=np.full(rows, 1.0 / temp, np.float32), top_p=np.full(rows, top_p), min_p=np.zeros(rows))
+                cell(f"fp32 N(0,{sigma:g}) T={temp:g} top-p={top_p:g}", c)
+    x = (rng.standard_normal((rows, V)) * 2.0).astype(np.float32)
+    for min_p in (0.2, 0.05, 0.01, 0.001):
+        c = dict(base)
+        c.update(logits=x, inv_t=np.ones(rows, np.float32), top_p=np.ones(rows), min_p=np.full(rows, min_p))
+        cell(f"fp32 N(0,2) T=1 min-p={min_p:g} (min_p_min said: short-list kernel)", c)
+    zipf = w.make_cfg3(rows=rows)
+    for top_p in (0.8, 0.9, 0.95, 0.99):
+        c = dict(zipf)
+        c.update(top_p=np.full(rows, top_p))
+        cell(f"bf16 Zipf(1.1) T=1 top-p={top_p:g}", c)
+    g16 = dict(base)
+    g16.update(logits=w.f32_to_bf16_bits(base["logits"]), dtype="bf16")
+    for top_p in (0.9, 0.99):
+        c = dict(g16)
+        c.update(top_p=np.full(rows, top_p))
+        cell(f"bf16 N(0,2) T=0.7..1 top-p={top_p:g}", c)
+    return out
+
+
+DATA_SEED_CENSUS = 20240611
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -424,6 +481,9 @@ def main():
     ap.add_argument("--reference-kernels", action="store_true",
                     help="time the replacements of the reference's own kernels (greedy picks, topk_rows) instead and print "
                          "their launch times as one JSON line")
+    ap.add_argument("--route-census", action="store_true",
+                    help="run batches without a top-k over a grid of logit shapes, temperatures and filters instead and print, "
+                         "per cell, how many rows took which way inside the launch and what the launch cost")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run 10 device copies of 256 MiB instead (known traffic: 256 MiB read + 256 MiB written per "
                          "copy) to scale rocprofv3's FETCH_SIZE / WRITE_SIZE")
@@ -450,6 +510,9 @@ def main():
     global MODE, KEPT_CAP
     MODE = {"auto": 0, "exact": 1, "fused": 2}[a.mode]
     KEPT_CAP = a.kept_cap
+    if a.route_census:
+        print(json.dumps({"route_census": route_census(), "data": "synthetic"}))
+        return
     check = 0 if a.no_cpu else a.check_rows
     c, main_res = run_workload(a.workload, a.steps, a.warmup, check)
     also = []

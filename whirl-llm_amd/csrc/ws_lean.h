@@ -34,6 +34,14 @@ constexpr uint32_t kLeanMaxList = 4096u;  // candidates of a row's ranges togeth
 // The bins the cut and the draw can fall in: sixteen at most, with eight different cache bytes at most among them (fp32
 // rows: eight bins; bf16 rows, where four neighbours share a byte: all sixteen).
 constexpr uint32_t kLeanMaxBins = 16u;
+// Bins are counted down from an anchor this many units of the exponent above the largest of the row's first tokens
+// (the row's maximum may lie up to 16 above it before the row is handed back). Eight were too few for peaked rows: with
+// logits of sigma 4 at T = 0.5 the maximum of 151936 tokens lies 4.8 units above that of the first 8192 on average, and
+// more than 8 on a quarter of the rows.
+constexpr float kLeanAbove = 12.f;
+// A range may span this many bins when few of them hold a token (the draw's range on a peaked row: two tokens fifty
+// bins apart); its bins then share the range's eight slots of the sort in order, several to a slot.
+constexpr uint32_t kLeanWide = 1024u;
 // The first bin of this kernel's tail, 48 units of the exponent below the anchor: the last 1024 bins, one to a thread,
 // take the tokens below that and the masked-out ones. (A scan of the bin cache for a bin finds the tokens of the tail
 // bins with the same cached bits as well: spread over 1024 bins, a 256th of the tail's tokens at most. In 64 bins a
@@ -452,7 +460,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
             }
         }
         s = block_max(s, red_f);  // its barriers also publish the zeroed histogram
-        anchor = s + 8.f / inv_t;
+        anchor = s + kLeanAbove / inv_t;
         aq = anchor_product(anchor, c64);
         if (!(anchor > -INFINITY && anchor < INFINITY)) WSL_FAIL(2);
     }
@@ -1044,15 +1052,43 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         }
         const bool has_r1 = r1hi >= r1lo;
         const uint32_t nb0 = static_cast<uint32_t>(r0hi - r0lo + 1), nb1 = has_r1 ? static_cast<uint32_t>(r1hi - r1lo + 1) : 0u;
-        ok = ok && r0hi < kLeanTail && nb0 + nb1 <= kLeanMaxBins && n_r0 + n_r1 != 0u && n_r0 + n_r1 <= kLeanMaxList;
+        ok = ok && r0hi < kLeanTail && nb0 <= kLeanWide && nb1 <= kLeanWide && n_r0 + n_r1 != 0u && n_r0 + n_r1 <= kLeanMaxList;
         {  // the bytes to scan the cache for: lane k looks at the k-th bin of the ranges, the first of a kind is listed
-            const uint32_t my_bin = lane < nb0 ? static_cast<uint32_t>(r0lo) + lane : static_cast<uint32_t>(r1lo) + (lane - nb0);
+            uint32_t my_bin = lane < nb0 ? static_cast<uint32_t>(r0lo) + lane : static_cast<uint32_t>(r1lo) + (lane - nb0);
+            uint32_t n_bins = nb0 + nb1;
+            if (ok && n_bins > kLeanMaxBins) {
+                // (uniform, rare) A peaked row: a handful of tokens, dozens of bins apart, where the draw may land. Only
+                // the bins that hold a token count: the lanes look them up in the histogram, 64 bins a round, and those
+                // with a token move up to the first lanes in order.
+                uint32_t found_bin = 0xffffffffu, n_found = 0;
+                for (uint32_t base = 0; base < nb0 + nb1; base += 64u) {
+                    const uint32_t k = base + lane;
+                    const uint32_t b = k < nb0 ? static_cast<uint32_t>(r0lo) + k : static_cast<uint32_t>(r1lo) + (k - nb0);
+                    uint64_t word = 0ull;
+                    if (k < nb0 + nb1) word = hist[hist_word(b)] + (hist2 ? hist2[hist_word(b)] : 0ull);
+                    const uint64_t has = __ballot((word >> kCountShift) != 0ull);
+                    // lane n_found + j takes the j-th bin of this round that holds a token
+                    const uint32_t want_j = lane - n_found;
+                    uint64_t rest = has;
+                    uint32_t src = 0xffffffffu;
+                    if (lane >= n_found && want_j < static_cast<uint32_t>(__popcll(has))) {
+                        for (uint32_t j = 0; j < want_j; ++j) rest &= rest - 1ull;
+                        src = static_cast<uint32_t>(__ffsll(static_cast<unsigned long long>(rest)) - 1);
+                    }
+                    const uint32_t b_src = __shfl(b, static_cast<int>(src & 63u));
+                    if (src != 0xffffffffu) found_bin = b_src;
+                    n_found += static_cast<uint32_t>(__popcll(has));
+                }
+                my_bin = found_bin;
+                n_bins = n_found;
+                ok = ok && n_found <= kLeanMaxBins;
+            }
             const uint32_t my_byte = (my_bin >> kCacheShift) & 0xffu;
-            bool is_first = lane < nb0 + nb1 && lane < kLeanMaxBins;
+            bool is_first = lane < n_bins && lane < kLeanMaxBins;
 #pragma unroll
             for (uint32_t j = 0; j + 1u < kLeanMaxBins; ++j) {
                 const uint32_t other = lane_value(my_byte, j);
-                if (j < lane && j < nb0 + nb1 && other == my_byte) is_first = false;
+                if (j < lane && j < n_bins && other == my_byte) is_first = false;
             }
             const uint64_t firsts = __ballot(is_first);
             const uint32_t place = static_cast<uint32_t>(__popcll(firsts & ((1ull << lane) - 1ull)));
@@ -1163,10 +1199,14 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
     uint2* cand = reinterpret_cast<uint2*>(lds);  // (token | slot << 28, logit bits), kLeanMaxList entries at most
     const bool r1_first = has_r1 && r1lo < r0lo;  // range 1 holds the larger logits
     // a candidate's slot: the number of its bin among the ranges' bins in descending order of the logits
+    // (a range of more than eight bins puts 2, 4, 8 .. neighbouring bins into one slot)
+    const uint32_t sh0 = nb0 > 8u ? 29u - static_cast<uint32_t>(__clz(static_cast<int>(nb0 - 1u))) : 0u;
+    const uint32_t sh1 = nb1 > 8u ? 29u - static_cast<uint32_t>(__clz(static_cast<int>(nb1 - 1u))) : 0u;
+    const uint32_t ns0 = ((nb0 - 1u) >> sh0) + 1u, ns1 = has_r1 ? ((nb1 - 1u) >> sh1) + 1u : 0u;  // slots of the ranges
     auto slot_of = [&](float x) {
         const uint32_t b = static_cast<uint32_t>(bin_coord(aq, c64, x));
         const bool in1 = has_r1 && b - static_cast<uint32_t>(r1lo) < nb1;
-        const uint32_t s_ = in1 ? (r1_first ? 0u : nb0) + (b - static_cast<uint32_t>(r1lo)) : (r1_first ? nb1 : 0u) + (b - static_cast<uint32_t>(r0lo));
+        const uint32_t s_ = in1 ? (r1_first ? 0u : ns0) + ((b - static_cast<uint32_t>(r1lo)) >> sh1) : (r1_first ? ns1 : 0u) + ((b - static_cast<uint32_t>(r0lo)) >> sh0);
         return min(s_, kLeanMaxBins - 1u);
     };
     {
@@ -1238,7 +1278,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         // logit; the candidates with exactly that logit, by id; the logits below, by logit. Where hundreds tie, `mid`
         // is theirs (two of four sampled candidates agree on it), and they spread over half the bin's buckets; where
         // no two logits are the same the middle part holds one candidate and the other half of the buckets serves.
-        const uint32_t nt_ = nb0 + nb1;
+        const uint32_t nt_ = ns0 + ns1;
         const uint32_t nsub = n_buckets >> (nt_ <= 1u ? 0u : (nt_ <= 2u ? 1u : (nt_ <= 4u ? 2u : (nt_ <= 8u ? 3u : 4u))));  // buckets a bin
         const uint32_t nl = nsub / 2u - 1u, nid = nsub / 2u;
         const float ids_scale = static_cast<float>(nid) / static_cast<float>(V);
@@ -1257,10 +1297,13 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
                 const uint32_t lo = min(min(min(a0.x, a0.y), min(a0.z, a0.w)), min(min(a1.x, a1.y), min(a1.z, a1.w)));
                 const uint32_t hi = max(max(max(b0.x, b0.y), max(b0.z, b0.w)), max(max(b1.x, b1.y), max(b1.z, b1.w)));
                 const uint32_t k32 = static_cast<uint32_t>(own[r] >> 32);
-                // (none of the expressions rises along the order, whatever the rounding: conversion, product and truncation keep it)
-                const float per = static_cast<float>(nl) * __builtin_amdgcn_rcpf(static_cast<float>(hi - lo) + 1.f);
-                const uint32_t lk = min(nl - 1u, static_cast<uint32_t>(static_cast<float>(hi - k32) * per));
-                const uint32_t lm = min(nl - 1u, static_cast<uint32_t>(static_cast<float>(hi - mid) * per));
+                // (Levels by the logits themselves, not by their keys: a bin that holds the logit 0 spans a billion keys,
+                // nearly all of its tokens among the topmost few million. None of the expressions rises along the order,
+                // whatever the rounding: difference, product and truncation keep it.)
+                const float x_hi = unkey32(hi), x_lo = unkey32(lo);
+                const float per = static_cast<float>(nl) * __builtin_amdgcn_rcpf(fmaxf(__fsub_rn(x_hi, x_lo), 1e-30f));
+                const uint32_t lk = min(nl - 1u, static_cast<uint32_t>(__fmul_rn(__fsub_rn(x_hi, unkey32(k32)), per)));
+                const uint32_t lm = min(nl - 1u, static_cast<uint32_t>(__fmul_rn(__fsub_rn(x_hi, unkey32(mid)), per)));
                 const uint32_t by_id = min(nid - 1u, static_cast<uint32_t>(static_cast<float>(0xffffffffu - static_cast<uint32_t>(own[r])) * ids_scale));
                 const uint32_t sub = k32 > mid ? lk : (k32 == mid ? lm + 1u + by_id : lk + 1u + nid);
                 bk[r] = sl[r] * nsub + sub;
