@@ -34,11 +34,11 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, kernel_digest() at the time)
-    ("tile", "auto"): (208285815, "lean_batch_kernel_tile_256x151936_f32.txt", "d3748406a8578277"),
-    ("cfg1", "auto"): (1213453, "short_batch_kernel_cfg1_1x151936_f32.txt", "d3748406a8578277"),
-    ("cfg2", "auto"): (56830885, "short_batch_kernel_cfg2_64x151936_f32.txt", "d3748406a8578277"),
-    ("cfg3", "auto"): (115290219, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "d3748406a8578277"),
-    ("cfg5", "auto"): (1363218685, "short_batch_kernel_cfg5_1024x262144_f32.txt", "d3748406a8578277"),
+    ("tile", "auto"): (208277100, "lean_batch_kernel_tile_256x151936_f32.txt", "b72d15f2a85ddc0f"),
+    ("cfg1", "auto"): (1213452, "short_batch_kernel_cfg1_1x151936_f32.txt", "b72d15f2a85ddc0f"),
+    ("cfg2", "auto"): (56833853, "short_batch_kernel_cfg2_64x151936_f32.txt", "b72d15f2a85ddc0f"),
+    ("cfg3", "auto"): (115283446, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "b72d15f2a85ddc0f"),
+    ("cfg5", "auto"): (1363176748, "short_batch_kernel_cfg5_1024x262144_f32.txt", "b72d15f2a85ddc0f"),
 }
 
 
