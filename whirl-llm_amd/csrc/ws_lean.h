@@ -1056,7 +1056,7 @@ __device__ __forceinline__ bool lean_row(const BatchArgs& A, const uint32_t row,
         {  // the bytes to scan the cache for: lane k looks at the k-th bin of the ranges, the first of a kind is listed
             uint32_t my_bin = lane < nb0 ? static_cast<uint32_t>(r0lo) + lane : static_cast<uint32_t>(r1lo) + (lane - nb0);
             uint32_t n_bins = nb0 + nb1;
-            if (ok && n_bins > kLeanMaxBins) {
+            if (ok && n_bins > (kCacheShift == 0u ? 8u : kLeanMaxBins)) {  // (more bins than the scan takes bytes)
                 // (uniform, rare) A peaked row: a handful of tokens, dozens of bins apart, where the draw may land. Only
                 // the bins that hold a token count: the lanes look them up in the histogram, 64 bins a round, and those
                 // with a token move up to the first lanes in order.
