@@ -76,5 +76,11 @@ def test_argmax_advance_and_static_sampler_in_one_captured_graph():
             g.replay()
             side.synchronize()
             for n in outputs:
-                assert torch.equal(getattr(smp, n), eager[k][n]), (k, n)
+                got, want = getattr(smp, n), eager[k][n]
+                if n in ("prob", "stats", "margin"):
+                    # (a shared row's normaliser is the sum of its parts' in the order they arrive: the last bit may differ
+                    # from launch to launch)
+                    assert torch.allclose(got.double(), want.double(), rtol=1e-6, atol=1e-12, equal_nan=True), (k, n)
+                else:
+                    assert torch.equal(got, want), (k, n)
             assert torch.equal(out, eager[k]["out"]) and torch.equal(ids, eager[k]["ids"]) and int(pos) == k + 1, k
