@@ -34,11 +34,11 @@ KEPT_CAP = 0  # entries a row of the kept-set dump (--kept-cap), 0: no dump
 # of the kernel sources the counters were taken with), otherwise null. File names are relative to profiles/.
 TRAFFIC = {
     # (workload, mode): (bytes per launch, profiles/ file, kernel_digest() at the time)
-    ("tile", "auto"): (208277100, "lean_batch_kernel_tile_256x151936_f32.txt", "b72d15f2a85ddc0f"),
-    ("cfg1", "auto"): (1213452, "short_batch_kernel_cfg1_1x151936_f32.txt", "b72d15f2a85ddc0f"),
-    ("cfg2", "auto"): (56833853, "short_batch_kernel_cfg2_64x151936_f32.txt", "b72d15f2a85ddc0f"),
-    ("cfg3", "auto"): (115283446, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "b72d15f2a85ddc0f"),
-    ("cfg5", "auto"): (1363176748, "short_batch_kernel_cfg5_1024x262144_f32.txt", "b72d15f2a85ddc0f"),
+    ("tile", "auto"): (208285157, "lean_batch_kernel_tile_256x151936_f32.txt", "f07604f05cff8423"),
+    ("cfg1", "auto"): (1213406, "short_batch_kernel_cfg1_1x151936_f32.txt", "f07604f05cff8423"),
+    ("cfg2", "auto"): (56857176, "short_batch_kernel_cfg2_64x151936_f32.txt", "f07604f05cff8423"),
+    ("cfg3", "auto"): (115277672, "lean_batch_kernel_cfg3_256x151936_bf16.txt", "f07604f05cff8423"),
+    ("cfg5", "auto"): (1363264388, "short_batch_kernel_cfg5_1024x262144_f32.txt", "f07604f05cff8423"),
 }
 
 
